@@ -1,0 +1,576 @@
+/*
+ * jitllm_oracle.c -- CPU restatement of jitLLM's Java CPU quantized matmul.
+ *
+ * TEST INFRASTRUCTURE ONLY: the checker for the HIP path, never a fallback for it.
+ * Built with -ffp-contract=off: Java never contracts a*b+c, so the only fused
+ * multiply-adds below are the explicit fmaf() calls that restate FloatVector.fma.
+ *
+ * J = src/main/java/org/beehive/jitllm in the reference checkout.
+ *
+ * Pinning (see tests/test_oracle_*.py):
+ *   decode (jo_get_float)      known answers of Q4_0DecodeTest, one-rounding closed forms over all
+ *                              65536 fp16 scales, agreement with the second wording
+ *                              (jo_get_float_alt) on the reference's random and adversarial blocks.
+ *   scalar dot                 strictly sequential fp32; brute force against an independent numpy
+ *                              float32 loop.
+ *   vector dot (128/256)       per-block lane values are fully determined and are compared with an
+ *                              independent numpy float32 model; the final reduceLanes(ADD)
+ *                              association is NOT specified by the JDK -- lane order 0..7 from
+ *                              zero is used here (what the JDK's own fallback does) and the result
+ *                              is held to a few ulp, not bit equality: "parity unpinned" for the
+ *                              last bits of that one addition chain only.
+ *   java.util.Random           published first outputs for seeds 0 and 42.
+ */
+#include "jitllm_oracle.h"
+
+#include <math.h>
+#include <omp.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define Q_BLOCK 32
+#define Q8_0_BYTES 34
+#define Q4_0_BYTES 18
+#define QK_K 256
+#define Q4_K_BYTES 144
+
+int jo_max_threads(void) { return omp_get_max_threads(); }
+
+/* J/format/GGMLType.java:7,13,18-20 */
+int jo_block_elems(int type) {
+    switch (type) {
+        case JO_Q4_0: return Q_BLOCK;
+        case JO_Q8_0: return Q_BLOCK;
+        case JO_Q4_K: return QK_K;
+        default: return 0;
+    }
+}
+
+int jo_block_bytes(int type) {
+    switch (type) {
+        case JO_Q4_0: return Q4_0_BYTES;
+        case JO_Q8_0: return Q8_0_BYTES;
+        case JO_Q4_K: return Q4_K_BYTES;
+        default: return 0;
+    }
+}
+
+/* ---- Float.float16ToFloat / Float.floatToFloat16 (J/tensor/standard/FloatTensor.java:71-79 call sites) */
+
+static inline float bits_to_float(uint32_t u) {
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static inline uint32_t float_to_bits(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+
+/* IEEE binary16 -> binary32, exact; subnormals widened, NaN payload kept in the top bits. */
+float jo_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    if (exp == 0) {
+        if (man == 0) return bits_to_float(sign);
+        /* subnormal: man * 2^-24, exactly representable */
+        float v = (float)man * 5.9604644775390625e-8f;
+        return bits_to_float(float_to_bits(v) | sign);
+    }
+    if (exp == 31) return bits_to_float(sign | 0x7F800000u | (man << 13));
+    return bits_to_float(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+/* binary32 -> binary16, round to nearest even (Float.floatToFloat16). */
+uint16_t jo_f32_to_f16(float value) {
+    uint32_t u = float_to_bits(value);
+    uint32_t sign = (u >> 16) & 0x8000u;
+    uint32_t abs = u & 0x7FFFFFFFu;
+    if (abs > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((abs >> 13) & 0x1FFu)); /* NaN */
+    if (abs >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u); /* >= 65520 rounds to infinity */
+    if (abs < 0x33000001u) return (uint16_t)sign;              /* <= 2^-25 rounds to zero */
+    int32_t e = (int32_t)(abs >> 23) - 127;
+    uint32_t man = (abs & 0x7FFFFFu) | 0x800000u;
+    int shift = (e < -14) ? (13 + (-14 - e)) : 13;
+    uint32_t half = man >> shift;
+    uint32_t rem = man & ((1u << shift) - 1u);
+    uint32_t mid = 1u << (shift - 1);
+    if (rem > mid || (rem == mid && (half & 1u))) half++;
+    if (e < -14) return (uint16_t)(sign | half); /* subnormal; a carry lands on the smallest normal */
+    return (uint16_t)(sign | (((uint32_t)(e + 15) << 10) + (half - 0x400u)));
+}
+
+static inline uint16_t read_u16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1] << 8)); }
+
+/* ---- element decoders ---------------------------------------------------------------------- */
+
+/* J/tensor/standard/Q8_0FloatTensor.java:52-61 */
+static inline float q8_0_get(const uint8_t *w, int64_t index) {
+    int64_t block_index = index / Q_BLOCK;
+    int64_t within = index % Q_BLOCK;
+    const uint8_t *blk = w + block_index * Q8_0_BYTES;
+    int8_t quant = (int8_t)blk[2 + within];
+    float scale = jo_f16_to_f32(read_u16(blk));
+    return (float)quant * scale;
+}
+
+/* J/tensor/standard/Q4_0FloatTensor.java:55-79 */
+static inline float q4_0_get(const uint8_t *w, int64_t index) {
+    int64_t block_index = index / Q_BLOCK;
+    const uint8_t *blk = w + block_index * Q4_0_BYTES;
+    float scale = jo_f16_to_f32(read_u16(blk));
+    int mod = (int)(index % Q_BLOCK);
+    int8_t quant;
+    if (mod < Q_BLOCK / 2) {
+        quant = (int8_t)(blk[2 + mod] & 0x0F);
+    } else {
+        quant = (int8_t)((blk[2 + mod - Q_BLOCK / 2] >> 4) & 0x0F);
+    }
+    quant = (int8_t)(quant - 8);
+    return (float)quant * scale;
+}
+
+/* J/tensor/standard/Q4_KFloatTensor.java:68-75 */
+static inline int q4_k_scale(int j, const uint8_t *s) {
+    if (j < 4) return s[j] & 63;
+    return (s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4);
+}
+
+/* J/tensor/standard/Q4_KFloatTensor.java:78-85 */
+static inline int q4_k_min(int j, const uint8_t *s) {
+    if (j < 4) return s[j + 4] & 63;
+    return (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+}
+
+/* J/tensor/standard/Q4_KFloatTensor.java:87-122 */
+static inline float q4_k_get(const uint8_t *w, int64_t index) {
+    int64_t block_index = index / QK_K;
+    int within = (int)(index % QK_K);
+    const uint8_t *blk = w + block_index * Q4_K_BYTES;
+    float d = jo_f16_to_f32(read_u16(blk));
+    float dmin = jo_f16_to_f32(read_u16(blk + 2));
+    const uint8_t *scales = blk + 4;
+    int pair = within / 64;
+    int pos = within % 64;
+    int sub, q;
+    if (pos < 32) {
+        sub = pair * 2;
+        q = blk[16 + pair * 32 + pos] & 0xF;
+    } else {
+        sub = pair * 2 + 1;
+        q = (blk[16 + pair * 32 + (pos - 32)] >> 4) & 0xF;
+    }
+    int sc = q4_k_scale(sub, scales);
+    int m = q4_k_min(sub, scales);
+    /* d * sc * q - dmin * m, left to right, every product and the difference rounded to fp32 */
+    float t = d * (float)sc;
+    t = t * (float)q;
+    float u = dmin * (float)m;
+    return t - u;
+}
+
+float jo_get_float(int type, const uint8_t *w, int64_t index) {
+    switch (type) {
+        case JO_Q8_0: return q8_0_get(w, index);
+        case JO_Q4_0: return q4_0_get(w, index);
+        case JO_Q4_K: return q4_k_get(w, index);
+        default: return NAN;
+    }
+}
+
+void jo_dequant(int type, const uint8_t *w, int64_t n, float *out) {
+    for (int64_t i = 0; i < n; i++) out[i] = jo_get_float(type, w, i);
+}
+
+/*
+ * The reference states each decode a second time, in its device kernels, and its unit tests hold
+ * the two wordings bit-equal.  Restated from those so the first wording can be checked against
+ * something that was not typed from the same lines:
+ *   Q4_0  J/backend/tornado/kernels/TransformerComputeKernelsQ4_0.java:72-79
+ *   Q4_K  J/backend/tornado/kernels/TransformerComputeKernelsQ4_K.java:77-104
+ *   Q8_0  src/test/java/.../kernels/QuantizedDeviceDecodeParityTest.java:349-358
+ */
+float jo_get_float_alt(int type, const uint8_t *w, int64_t index) {
+    if (type == JO_Q8_0) {
+        const uint8_t *blk = w + (index / 32) * Q8_0_BYTES;
+        return jo_f16_to_f32(read_u16(blk)) * (float)(int8_t)blk[2 + index % 32];
+    }
+    if (type == JO_Q4_0) {
+        const uint8_t *blk = w + (index / 32) * Q4_0_BYTES;
+        int within = (int)(index % 32);
+        float d = jo_f16_to_f32(read_u16(blk));
+        int half = within / 16;
+        int packed = blk[2 + within - half * 16];
+        int q = (half == 0) ? (packed & 0xF) : ((packed >> 4) & 0xF);
+        return d * (float)(q - 8);
+    }
+    if (type == JO_Q4_K) {
+        const uint8_t *blk = w + (index / 256) * Q4_K_BYTES;
+        int within = (int)(index % 256);
+        float d = jo_f16_to_f32(read_u16(blk));
+        float dmin = jo_f16_to_f32(read_u16(blk + 2));
+        int pair = within / 64;
+        int pos = within - pair * 64;
+        int high = pos / 32;
+        int sub = pair * 2 + high;
+        int qb = blk[16 + pair * 32 + (pos - high * 32)];
+        int q = (high == 0) ? (qb & 0xF) : ((qb >> 4) & 0xF);
+        const uint8_t *s = blk + 4;
+        int sc, m;
+        if (sub < 4) {
+            sc = s[sub] & 63;
+            m = s[sub + 4] & 63;
+        } else {
+            int low = s[sub + 4];
+            int hi = s[sub - 4];
+            sc = (low & 0xF) | ((hi >> 6) << 4);
+            m = ((low >> 4) & 0xF) | ((s[sub] >> 6) << 4);
+        }
+        float a = d * (float)sc;
+        a = a * (float)q;
+        float b = dmin * (float)m;
+        return a - b;
+    }
+    return NAN;
+}
+
+/* ---- dot products -------------------------------------------------------------------------- */
+
+/* J/tensor/standard/FloatTensor.java:110-117 */
+static float scalar_dot(int type, const uint8_t *w, int64_t this_offset, const float *x,
+                        int64_t that_offset, int64_t size) {
+    float result = 0.0f;
+    switch (type) {
+        case JO_Q8_0:
+            for (int64_t j = 0; j < size; j++) {
+                float p = q8_0_get(w, this_offset + j) * x[that_offset + j];
+                result += p;
+            }
+            break;
+        case JO_Q4_0:
+            for (int64_t j = 0; j < size; j++) {
+                float p = q4_0_get(w, this_offset + j) * x[that_offset + j];
+                result += p;
+            }
+            break;
+        case JO_Q4_K:
+            for (int64_t j = 0; j < size; j++) {
+                float p = q4_k_get(w, this_offset + j) * x[that_offset + j];
+                result += p;
+            }
+            break;
+        default:
+            return NAN;
+    }
+    return result;
+}
+
+/*
+ * FloatVector.reduceLanes(ADD).  The JDK leaves the association open; its portable fallback folds
+ * the lanes in index order starting from zero, which is what is used here.
+ */
+static inline float reduce_lanes(const float *val, int lanes) {
+    float r = 0.0f;
+    for (int l = 0; l < lanes; l++) r += val[l];
+    return r;
+}
+
+/*
+ * One block step of the vector kernels, shared by Q8_0 and Q4_0 once the 32 weights of the block
+ * are widened to float in element order wf[0..31]:
+ *   256-bit  val = fma(((s0 + s1) + s2) + s3, d, val), s_k = x[8k..8k+7] * wf[8k..8k+7]
+ *   128-bit  two such steps over elements 0..15 and 16..31 with four 4-lane slices each
+ * J/tensor/standard/Q8_0FloatTensor.java:161-216, Q4_0FloatTensor.java:120-163.
+ * For Q4_0 the element order is lo nibbles of bytes 0..15 then hi nibbles of bytes 0..15, which is
+ * exactly (lo part 0, lo part 1, hi part 0, hi part 1) at 256 bits and (lo parts 0..3), (hi parts
+ * 0..3) at 128 bits.
+ */
+static inline __attribute__((always_inline)) void
+block_step_256(const float *wf, const float *x, float d, float *val) {
+    for (int l = 0; l < 8; l++) {
+        float s0 = x[l] * wf[l];
+        float s1 = x[8 + l] * wf[8 + l];
+        float s2 = x[16 + l] * wf[16 + l];
+        float s3 = x[24 + l] * wf[24 + l];
+        float s = ((s0 + s1) + s2) + s3;
+        val[l] = fmaf(s, d, val[l]);
+    }
+}
+
+static inline __attribute__((always_inline)) void
+block_step_128(const float *wf, const float *x, float d, float *val) {
+    for (int i = 0; i < 2; i++) {
+        const float *wh = wf + 16 * i;
+        const float *xh = x + 16 * i;
+        for (int l = 0; l < 4; l++) {
+            float s0 = xh[l] * wh[l];
+            float s1 = xh[4 + l] * wh[4 + l];
+            float s2 = xh[8 + l] * wh[8 + l];
+            float s3 = xh[12 + l] * wh[12 + l];
+            float s = ((s0 + s1) + s2) + s3;
+            val[l] = fmaf(s, d, val[l]);
+        }
+    }
+}
+
+static inline __attribute__((always_inline)) void widen_q8_0(const uint8_t *blk, float *wf) {
+    for (int i = 0; i < 32; i++) wf[i] = (float)(int8_t)blk[2 + i];
+}
+
+static inline __attribute__((always_inline)) void widen_q4_0(const uint8_t *blk, float *wf) {
+    for (int i = 0; i < 16; i++) {
+        /* byte lanes: (b & 0xF) - 8 and (b >>> 4) - 8, then castShape widens the signed byte */
+        int8_t lo = (int8_t)((blk[2 + i] & 0xF) - 8);
+        int8_t hi = (int8_t)((blk[2 + i] >> 4) - 8);
+        wf[i] = (float)lo;
+        wf[16 + i] = (float)hi;
+    }
+}
+
+/* J/tensor/standard/Q8_0FloatTensor.java:142-229 and Q4_0FloatTensor.java:90-174 */
+static inline __attribute__((always_inline)) float
+vector_dot_body(int type, int bits, const uint8_t *w, int64_t this_offset, const float *x,
+           int64_t that_offset, int64_t size) {
+    const int block_bytes = (type == JO_Q8_0) ? Q8_0_BYTES : Q4_0_BYTES;
+    float result = 0.0f;
+    int64_t j = 0;
+    int64_t alignment_bound = (-this_offset) & (Q_BLOCK - 1);
+    if (alignment_bound > size) alignment_bound = size;
+    if (alignment_bound > 0) {
+        result += scalar_dot(type, w, this_offset, x, that_offset, alignment_bound);
+        j += alignment_bound;
+    }
+    float val[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int64_t block_offset = (this_offset + j) / Q_BLOCK * block_bytes;
+    int64_t upper_bound = size / Q_BLOCK * Q_BLOCK;
+    float wf[32];
+    /* the reference loop tests j < upperBound only; j + 32 <= size is added so that a misaligned
+       offset (which no matmul caller produces) cannot read past the slice */
+    for (; j < upper_bound && j + Q_BLOCK <= size; j += Q_BLOCK, block_offset += block_bytes) {
+        const uint8_t *blk = w + block_offset;
+        float d = jo_f16_to_f32(read_u16(blk));
+        if (type == JO_Q8_0) widen_q8_0(blk, wf); else widen_q4_0(blk, wf);
+        if (bits == 256) block_step_256(wf, x + that_offset + j, d, val);
+        else block_step_128(wf, x + that_offset + j, d, val);
+    }
+    result += reduce_lanes(val, bits == 256 ? 8 : 4);
+    if (j < size) {
+        result += scalar_dot(type, w, this_offset + j, x, that_offset + j, size - j);
+    }
+    return result;
+}
+
+/* The same body compiled twice: once for AVX2+FMA hosts, once for anything else. */
+__attribute__((target("avx2,fma"))) static float
+vector_dot_avx2(int type, int bits, const uint8_t *w, int64_t this_offset, const float *x,
+                int64_t that_offset, int64_t size) {
+    return vector_dot_body(type, bits, w, this_offset, x, that_offset, size);
+}
+
+static float vector_dot_generic(int type, int bits, const uint8_t *w, int64_t this_offset,
+                                const float *x, int64_t that_offset, int64_t size) {
+    return vector_dot_body(type, bits, w, this_offset, x, that_offset, size);
+}
+
+static float vector_dot(int type, int bits, const uint8_t *w, int64_t this_offset, const float *x,
+                        int64_t that_offset, int64_t size) {
+    static int have_avx2 = -1;
+    if (have_avx2 < 0) have_avx2 = __builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma");
+    return have_avx2 ? vector_dot_avx2(type, bits, w, this_offset, x, that_offset, size)
+                     : vector_dot_generic(type, bits, w, this_offset, x, that_offset, size);
+}
+
+/*
+ * Q8_0FloatTensor.dot (J/tensor/standard/Q8_0FloatTensor.java:89-99), Q4_0FloatTensor.dot
+ * (Q4_0FloatTensor.java:82-88), Q4_KFloatTensor.dot (Q4_KFloatTensor.java:124-127).  The flavour
+ * is the branch a JVM would take: vector kernels exist for 128- and 256-bit species only
+ * (FloatTensor.java:33-36); Q4_K is always scalar.
+ */
+float jo_dot(int type, int flavour, const uint8_t *w, int64_t this_offset, const float *x,
+             int64_t that_offset, int64_t size) {
+    if (type != JO_Q4_K && (flavour == JO_DOT_VEC128 || flavour == JO_DOT_VEC256)) {
+        return vector_dot(type, flavour, w, this_offset, x, that_offset, size);
+    }
+    return scalar_dot(type, w, this_offset, x, that_offset, size);
+}
+
+/* J/tensor/standard/FloatTensor.java:123-125 + J/auxiliary/Parallel.java:9-11 */
+void jo_matmul(int type, int flavour, const uint8_t *w, const float *x, float *out, int dim0,
+               int dim1, int nthreads) {
+    if (nthreads < 1) nthreads = 1;
+#pragma omp parallel for schedule(static) num_threads(nthreads)
+    for (int i = 0; i < dim0; i++) {
+        out[i] = jo_dot(type, flavour, w, (int64_t)i * dim1, x, 0, dim1);
+    }
+}
+
+/* J/tensor/standard/FloatTensor.java:127-140 + J/auxiliary/Parallel.java:13-20 */
+void jo_matmul_batch(int type, int flavour, const uint8_t *w, const float *X, float *out,
+                     int context, int dim0, int dim1, int nthreads) {
+    if (nthreads < 1) nthreads = 1;
+    int64_t total = (int64_t)dim0 * context;
+#pragma omp parallel for schedule(static) num_threads(nthreads)
+    for (int64_t ti = 0; ti < total; ti++) {
+        int idx_arr = (int)(ti / dim0);
+        int i = (int)(ti % dim0);
+        out[(int64_t)idx_arr * dim0 + i] =
+            jo_dot(type, flavour, w, (int64_t)i * dim1, X + (int64_t)idx_arr * dim1, 0, dim1);
+    }
+}
+
+/* J/inference/op/CpuOperations.java:255-260 */
+void jo_swiglu(float *gate, const float *up, int64_t n) {
+    for (int64_t i = 0; i < n; i++) {
+        float value = gate[i];
+        float act = value / (float)(1.0 + exp(-(double)value));
+        gate[i] = act * up[i];
+    }
+}
+
+/* ---- int8 activation path (the arithmetic the reference's int8 GEMM defines) -------------- */
+
+/*
+ * J/backend/tornado/kernels/Int8GemmKernels.java:96-129 (quantizeActivationsQ8Warp):
+ * d = amax / 127; q = 0 if d == 0, else round-half-away(x * (127 / amax)) clamped to +-127, with
+ * the (x / amax) * 127 form below RECIPROCAL_FINITE_AMAX = 4e-37.
+ */
+void jo_quantize_q8(const float *x, int8_t *q, float *scales, int64_t rows, int64_t k) {
+    int64_t blocks = rows * k / 32;
+    for (int64_t b = 0; b < blocks; b++) {
+        const float *xb = x + b * 32;
+        float amax = 0.0f;
+        for (int i = 0; i < 32; i++) {
+            float a = fabsf(xb[i]);
+            if (a > amax) amax = a;
+        }
+        float d = amax / 127.0f;
+        for (int i = 0; i < 32; i++) {
+            int qv = 0;
+            if (d > 0.0f) {
+                float v;
+                if (amax >= 4.0e-37f) v = xb[i] * (127.0f / amax);
+                else v = (xb[i] / amax) * 127.0f;
+                qv = (int)floorf(fabsf(v) + 0.5f);
+                if (qv > 127) qv = 127;
+                if (v < 0.0f) qv = -qv;
+            }
+            q[b * 32 + i] = (int8_t)qv;
+        }
+        scales[b] = d;
+    }
+}
+
+/*
+ * J/backend/tornado/kernels/Int8GemmKernels.java:17-23: each 32-block's dot product exact in
+ * int32; acc = fma((float)dot * dA, dW, acc) over the blocks in k order.  Weights are Q8_0 quants
+ * or Q4_0 nibbles recentred to q - 8; dW is the fp16 block scale widened to fp32.
+ */
+void jo_gemm_int8_block_scaled(int type, const int8_t *aq, const float *ascale, const uint8_t *w,
+                               float *out, int m, int n, int k, int nthreads) {
+    if (nthreads < 1) nthreads = 1;
+    const int kb = k / 32;
+    const int block_bytes = jo_block_bytes(type);
+#pragma omp parallel for schedule(static) num_threads(nthreads)
+    for (int col = 0; col < n; col++) {
+        for (int row = 0; row < m; row++) {
+            float acc = 0.0f;
+            for (int b = 0; b < kb; b++) {
+                const uint8_t *blk = w + ((int64_t)col * kb + b) * block_bytes;
+                float dw = jo_f16_to_f32(read_u16(blk));
+                const int8_t *a = aq + (int64_t)row * k + b * 32;
+                int32_t dot = 0;
+                if (type == JO_Q8_0) {
+                    for (int i = 0; i < 32; i++) dot += (int32_t)a[i] * (int8_t)blk[2 + i];
+                } else {
+                    for (int i = 0; i < 16; i++) {
+                        dot += (int32_t)a[i] * ((blk[2 + i] & 0xF) - 8);
+                        dot += (int32_t)a[16 + i] * ((blk[2 + i] >> 4) - 8);
+                    }
+                }
+                float t = (float)dot * ascale[(int64_t)row * kb + b];
+                acc = fmaf(t, dw, acc);
+            }
+            out[(int64_t)row * n + col] = acc;
+        }
+    }
+}
+
+/* ---- java.util.Random (the generator the reference's test fixtures are drawn from) --------- */
+
+#define JR_MULT 0x5DEECE66DLL
+#define JR_MASK ((1LL << 48) - 1)
+
+void jo_jrandom_init(jo_jrandom *r, int64_t seed) {
+    r->seed = (seed ^ JR_MULT) & JR_MASK;
+    r->have_next_next_gaussian = 0;
+    r->next_next_gaussian = 0.0;
+}
+
+static inline int32_t jr_next(jo_jrandom *r, int bits) {
+    r->seed = (int64_t)(((uint64_t)r->seed * (uint64_t)JR_MULT + 0xBULL) & (uint64_t)JR_MASK);
+    return (int32_t)(r->seed >> (48 - bits));
+}
+
+int32_t jo_jrandom_next_int(jo_jrandom *r) { return jr_next(r, 32); }
+
+int32_t jo_jrandom_next_int_bound(jo_jrandom *r, int32_t bound) {
+    if (bound <= 0) return 0;
+    int32_t v = jr_next(r, 31);
+    int32_t m = bound - 1;
+    if ((bound & m) == 0) return (int32_t)(((int64_t)bound * (int64_t)v) >> 31);
+    int32_t u = v;
+    /* reject while u - (u % bound) + m overflows int32 */
+    while (1) {
+        v = u % bound;
+        int64_t t = (int64_t)u - v + m;
+        if (t <= INT32_MAX) break;
+        u = jr_next(r, 31);
+    }
+    return v;
+}
+
+int jo_jrandom_next_boolean(jo_jrandom *r) { return jr_next(r, 1) != 0; }
+
+static inline double jr_next_double(jo_jrandom *r) {
+    int64_t hi = (int64_t)jr_next(r, 26) << 27;
+    int64_t lo = jr_next(r, 27);
+    return (double)(hi + lo) * 0x1.0p-53;
+}
+
+double jo_jrandom_next_gaussian(jo_jrandom *r) {
+    if (r->have_next_next_gaussian) {
+        r->have_next_next_gaussian = 0;
+        return r->next_next_gaussian;
+    }
+    double v1, v2, s;
+    do {
+        v1 = 2 * jr_next_double(r) - 1;
+        v2 = 2 * jr_next_double(r) - 1;
+        s = v1 * v1 + v2 * v2;
+    } while (s >= 1 || s == 0);
+    double multiplier = sqrt(-2 * log(s) / s);
+    r->next_next_gaussian = v2 * multiplier;
+    r->have_next_next_gaussian = 1;
+    return v1 * multiplier;
+}
+
+void jo_jrandom_next_bytes(jo_jrandom *r, uint8_t *out, int64_t n) {
+    int64_t i = 0;
+    while (i < n) {
+        int32_t rnd = jo_jrandom_next_int(r);
+        int64_t take = n - i < 4 ? n - i : 4;
+        while (take-- > 0) {
+            out[i++] = (uint8_t)rnd;
+            rnd >>= 8;
+        }
+    }
+}
+
+int32_t jo_java_string_hash(const char *s) {
+    uint32_t h = 0;
+    for (; *s; s++) h = 31u * h + (uint8_t)*s;
+    return (int32_t)h;
+}

@@ -1,0 +1,108 @@
+"""Independent numpy statements of the block formats, written from the ggml format description
+(block_q8_0 / block_q4_0 / block_q4_K and get_scale_min_k4), NOT from the oracle's C text: they
+exist so the oracle is checked against something that was not typed from the same lines.
+All arithmetic is float32, one rounding per operation, no fused multiply-add.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+F32 = np.float32
+
+
+def half_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    return np.asarray(bits, dtype=np.uint16).view(np.float16).astype(np.float32)
+
+
+def dequant_q8_0(raw: np.ndarray) -> np.ndarray:
+    b = raw.reshape(-1, 34)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    q = b[:, 2:].view(np.int8).astype(np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        return (q * d[:, None]).astype(np.float32).reshape(-1)
+
+
+def dequant_q4_0(raw: np.ndarray) -> np.ndarray:
+    b = raw.reshape(-1, 18)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    qs = b[:, 2:]
+    lo = (qs & 0x0F).astype(np.int32) - 8
+    hi = (qs >> 4).astype(np.int32) - 8
+    q = np.concatenate([lo, hi], axis=1).astype(np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        return (q * d[:, None]).astype(np.float32).reshape(-1)
+
+
+def q4_k_scales_mins(scales12: np.ndarray):
+    """get_scale_min_k4 for j = 0..7 over [..., 12] scale bytes -> two [..., 8] integer arrays."""
+    s = scales12.astype(np.int32)
+    sc = np.empty(s.shape[:-1] + (8,), dtype=np.int32)
+    mn = np.empty_like(sc)
+    for j in range(4):
+        sc[..., j] = s[..., j] & 63
+        mn[..., j] = s[..., j + 4] & 63
+    for j in range(4, 8):
+        sc[..., j] = (s[..., j + 4] & 0xF) | ((s[..., j - 4] >> 6) << 4)
+        mn[..., j] = (s[..., j + 4] >> 4) | ((s[..., j] >> 6) << 4)
+    return sc, mn
+
+
+def dequant_q4_k(raw: np.ndarray) -> np.ndarray:
+    b = raw.reshape(-1, 144)
+    nb = b.shape[0]
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    dmin = half_bits_to_f32(b[:, 2:4].copy().view(np.uint16)[:, 0])
+    sc, mn = q4_k_scales_mins(b[:, 4:16])
+    qs = b[:, 16:].reshape(nb, 4, 32)
+    out = np.empty((nb, 8, 32), dtype=np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        for j in range(8):
+            nib = (qs[:, j // 2, :] >> (4 * (j % 2))) & 0xF
+            d1 = (d * sc[:, j].astype(np.float32)).astype(np.float32)
+            m1 = (dmin * mn[:, j].astype(np.float32)).astype(np.float32)
+            t = (d1[:, None] * nib.astype(np.float32)).astype(np.float32)
+            out[:, j, :] = (t - m1[:, None]).astype(np.float32)
+    return out.reshape(-1)
+
+
+DEQUANT = {8: dequant_q8_0, 2: dequant_q4_0, 12: dequant_q4_k}
+
+
+def scalar_dot_rows(w_deq: np.ndarray, x: np.ndarray) -> np.ndarray:
+    """Strictly sequential float32 dot of every row of ``w_deq`` [d x n] with ``x`` [n]."""
+    d, n = w_deq.shape
+    acc = np.zeros(d, dtype=np.float32)
+    for j in range(n):
+        acc = (acc + (w_deq[:, j] * x[j]).astype(np.float32)).astype(np.float32)
+    return acc
+
+
+def _fma32(a: np.ndarray, b: np.ndarray, c: np.ndarray) -> np.ndarray:
+    """fma in float32 for operands whose exact a*b+c fits a double (|terms| small): the product of
+    two float32 values is exact in float64, and one float64 add then one rounding to float32
+    differs from a true fma only by double rounding, which the callers' tolerance absorbs."""
+    return (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(np.float32)
+
+
+def vector_lane_values(t: int, raw: np.ndarray, x: np.ndarray, bits: int) -> np.ndarray:
+    """Lane accumulators of the reference's vector dot for one row, before reduceLanes."""
+    if t == 8:
+        b = raw.reshape(-1, 34)
+        wf = b[:, 2:].view(np.int8).astype(np.float32)
+    else:
+        b = raw.reshape(-1, 18)
+        qs = b[:, 2:]
+        wf = np.concatenate([(qs & 0xF).astype(np.int32) - 8, (qs >> 4).astype(np.int32) - 8],
+                            axis=1).astype(np.float32)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    lanes = bits // 32
+    val = np.zeros(lanes, dtype=np.float32)
+    xb = x.reshape(-1, 32)
+    for k in range(b.shape[0]):
+        halves = [(0, 32)] if bits == 256 else [(0, 16), (16, 32)]
+        for lo, hi in halves:
+            p = (xb[k, lo:hi] * wf[k, lo:hi]).astype(np.float32).reshape(4, lanes)
+            s = ((p[0] + p[1]).astype(np.float32) + p[2]).astype(np.float32)
+            s = (s + p[3]).astype(np.float32)
+            val = _fma32(s, np.full(lanes, d[k], dtype=np.float32), val)
+    return val

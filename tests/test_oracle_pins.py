@@ -1,0 +1,297 @@
+"""Pins the CPU oracle before anything is compared with it (no GPU needed)."""
+import numpy as np
+import pytest
+
+import fixtures as FX
+import np_models as NP
+from oracle import pyoracle as O
+
+TYPES = [O.Q8_0, O.Q4_0, O.Q4_K]
+
+
+def bits(a):
+    return np.asarray(a, dtype=np.float32).view(np.uint32)
+
+
+def assert_bit_equal(a, b):
+    a, b = np.asarray(a, np.float32), np.asarray(b, np.float32)
+    nan = np.isnan(a)
+    assert np.array_equal(nan, np.isnan(b))
+    assert np.array_equal(bits(a)[~nan], bits(b)[~nan])
+
+
+# ---- java.util.Random and String.hashCode: published values -------------------------------
+
+def test_java_random_known_values():
+    assert O.JavaRandom(0).next_int() == -1155484576
+    assert O.JavaRandom(42).next_int() == -1170105035
+    assert O.JavaRandom(0).next_gaussian() == 0.8025330637390305
+    r = O.JavaRandom(42)
+    assert [r.next_int(10) for _ in range(5)] == [0, 3, 8, 4, 0]
+    assert O.java_string_hash("hello") == 99162322
+    assert O.java_string_hash("") == 0
+
+
+def _py_next(seed, nbits):
+    seed = (seed * 0x5DEECE66D + 0xB) & ((1 << 48) - 1)
+    v = seed >> (48 - nbits)
+    if v >= 1 << (nbits - 1) and nbits == 32:
+        v -= 1 << 32
+    return seed, v
+
+
+def test_java_random_next_bytes_against_pure_python():
+    seed = (20260908 ^ 0x5DEECE66D) & ((1 << 48) - 1)
+    want = []
+    while len(want) < 37:
+        seed, v = _py_next(seed, 32)
+        for _ in range(4):
+            want.append(v & 0xFF)
+            v >>= 8
+    got = O.JavaRandom(20260908).next_bytes(37)
+    assert list(got) == want[:37]
+
+
+# ---- fp16 conversions --------------------------------------------------------------------
+
+def test_f16_to_f32_all_patterns():
+    allbits = np.arange(65536, dtype=np.uint16)
+    want = allbits.view(np.float16).astype(np.float32)
+    got = np.array([O.f16_to_f32(int(b)) for b in allbits], dtype=np.float32)
+    assert_bit_equal(got, want)
+    assert O.f16_to_f32(0x4000) == 2.0
+    assert O.f16_to_f32(0x0001) == np.float32(2.0 ** -24)
+    assert O.f16_to_f32(0xFBFF) == -65504.0
+
+
+def test_f32_to_f16_round_to_nearest_even():
+    rng = np.random.default_rng(1)
+    vals = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 20000),
+        np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e9, 2.0 ** -24, 2.0 ** -25,
+                  2.0 ** -25 * 1.0001, 2.0 ** -14, 6.1e-5, np.inf, -np.inf], dtype=np.float32),
+        np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)[:0x7C00],
+    ]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([O.f32_to_f16(v) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+# ---- element decode: known answers, closed forms, second wording ---------------------------
+
+def test_q4_0_spec_known_answers():
+    """T/backend/tornado/kernels/Q4_0DecodeTest.java:95-126."""
+    raw = np.zeros(18, dtype=np.uint8)
+    raw[0], raw[1], raw[2], raw[3] = 0x00, 0x40, 0x0F, 0x80
+    for alt in (False, True):
+        assert O.get_float(O.Q4_0, raw, 0, alt) == 14.0
+        assert O.get_float(O.Q4_0, raw, 16, alt) == -16.0
+        assert O.get_float(O.Q4_0, raw, 1, alt) == -16.0
+        assert O.get_float(O.Q4_0, raw, 17, alt) == 0.0
+
+
+def test_q8_0_closed_form_all_scales_all_quants():
+    """q * d is one correctly rounded product of exact operands: any IEEE float32 multiply agrees."""
+    scales = np.arange(65536, dtype=np.uint16)
+    raw = np.zeros((65536, 8, 34), dtype=np.uint8)
+    raw[:, :, 0] = (scales & 0xFF)[:, None]
+    raw[:, :, 1] = (scales >> 8)[:, None]
+    raw[:, :, 2:] = np.arange(256, dtype=np.uint8).reshape(8, 32)[None]
+    got = O.dequant(O.Q8_0, raw.reshape(-1)).reshape(65536, 256)
+    d = scales.view(np.float16).astype(np.float64)
+    q = np.arange(256, dtype=np.uint8).view(np.int8).astype(np.float64)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = (d[:, None] * q[None, :]).astype(np.float32)
+    assert_bit_equal(got, want)
+
+
+def test_q4_0_closed_form_all_scales_all_nibbles():
+    scales = np.arange(65536, dtype=np.uint16)
+    raw = np.zeros((65536, 18), dtype=np.uint8)
+    raw[:, 0] = scales & 0xFF
+    raw[:, 1] = scales >> 8
+    # byte i: low nibble i, high nibble 15 - i -> element i has q = i, element 16 + i has q = 15 - i
+    raw[:, 2:] = (np.arange(16) | ((15 - np.arange(16)) << 4)).astype(np.uint8)[None]
+    got = O.dequant(O.Q4_0, raw.reshape(-1)).reshape(65536, 32)
+    d = scales.view(np.float16).astype(np.float64)
+    q = np.concatenate([np.arange(16), 15 - np.arange(16)]).astype(np.float64) - 8
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = (d[:, None] * q[None, :]).astype(np.float32)
+    assert_bit_equal(got, want)
+
+
+@pytest.mark.parametrize("t,seed,blocks", [(O.Q4_0, 20260908, 16), (O.Q4_K, 20260904, 8),
+                                            (O.Q8_0, 20260908, 16)])
+def test_random_bytes_decode_three_ways(t, seed, blocks):
+    """Q4_0DecodeTest.java:36-85 / Q4_KDecodeTest.java:32-75: host wording == device wording, and
+    both == the independent numpy statement of the ggml layout."""
+    raw = FX.random_bytes(seed, blocks * O.block_bytes(t))
+    main = O.dequant(t, raw)
+    assert_bit_equal(main, O.dequant_alt(t, raw))
+    assert_bit_equal(main, NP.DEQUANT[t](raw))
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_adversarial_blocks_decode_three_ways(t):
+    """QuantizedDeviceDecodeParityTest.java:98-121,191,313,349 (24 blocks, special fp16 scales)."""
+    seed = 20260908 + O.java_string_hash(FX.TYPE_NAMES[t])
+    raw = FX.adversarial_blocks(t, 24, seed)
+    main = O.dequant(t, raw)
+    assert_bit_equal(main, O.dequant_alt(t, raw))
+    assert_bit_equal(main, NP.DEQUANT[t](raw))
+
+
+def test_q4_k_scale_unpacking_round_trip():
+    """Every (scale, min) in 0..63 survives pack -> the oracle's unpack, at every sub-block."""
+    from jitllm_amd import synthetic
+    sc = np.arange(64, dtype=np.uint8)
+    for j in range(8):
+        for mval in (0, 21, 63):
+            s = np.zeros((64, 8), dtype=np.uint8)
+            m = np.zeros((64, 8), dtype=np.uint8)
+            s[:, j] = sc
+            m[:, j] = mval
+            raw = np.zeros((64, 144), dtype=np.uint8)
+            raw[:, 0:2] = np.array([0x00, 0x3C], dtype=np.uint8)  # d = 1
+            raw[:, 2:4] = np.array([0x00, 0x3C], dtype=np.uint8)  # dmin = 1
+            raw[:, 4:16] = synthetic.pack_q4_k_scales(s, m)
+            raw[:, 16:] = 0x11  # every nibble q = 1
+            out = O.dequant(O.Q4_K, raw.reshape(-1)).reshape(64, 8, 32)
+            assert np.array_equal(out[:, j, 0], sc.astype(np.float32) - mval)
+            other = [k for k in range(8) if k != j]
+            assert np.all(out[:, other, :] == 0.0)
+
+
+# ---- dot products -------------------------------------------------------------------------
+
+@pytest.mark.parametrize("t,name", [(O.Q4_0, "q4_0"), (O.Q4_K, "q4_K"), (O.Q8_0, "q8_0")])
+def test_scalar_dot_is_the_reference_tests_host_sum(t, name):
+    """NativeQuantizedKernelAccelTest.java:106-135: expected[row] = sum over col of
+    getFloat(row*N+col) * x[col], sequential float32 -- which is also FloatTensor.scalarDot."""
+    raw = FX.probe_blocks(t, FX.probe_seed(name))
+    x = FX.probe_x()
+    got = O.matmul(t, raw, x, FX.D_PROBE, FX.N_PROBE, O.DOT_SCALAR)
+    deq = NP.DEQUANT[t](raw).reshape(FX.D_PROBE, FX.N_PROBE)
+    want = NP.scalar_dot_rows(deq, x)
+    assert_bit_equal(got, want)
+
+
+@pytest.mark.parametrize("t", [O.Q8_0, O.Q4_0])
+@pytest.mark.parametrize("width", [128, 256])
+def test_vector_dot_lane_model(t, width):
+    """Per-lane accumulators are fully determined; the final lane fold is held to a few ulp of the
+    magnitude sum because the JDK leaves reduceLanes' association open."""
+    from jitllm_amd import synthetic
+    n = 2048
+    raw = synthetic.weight(t, 4, n, seed=11)
+    x = synthetic.activations(n, seed=12)
+    rb = O.block_bytes(t) * n // 32
+    for r in range(4):
+        row = raw[r * rb:(r + 1) * rb]
+        val = NP.vector_lane_values(t, row, x, width)
+        want_seq = np.float32(0)
+        for v in val:
+            want_seq = np.float32(want_seq + v)
+        got = O.dot(t, width, raw, r * n, x, 0, n)
+        mag = np.abs(NP.DEQUANT[t](row) * x).sum()
+        assert abs(float(got) - float(want_seq)) <= 4 * np.finfo(np.float32).eps * mag
+        pairwise = val.astype(np.float64).sum()
+        assert abs(float(got) - pairwise) <= 8 * np.finfo(np.float32).eps * mag
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_dot_flavours_agree_to_rounding(t):
+    from jitllm_amd import synthetic
+    n, d = 1024, 16
+    raw = synthetic.weight(t, d, n, seed=5)
+    x = synthetic.activations(n, seed=6)
+    ref = (NP.DEQUANT[t](raw).reshape(d, n).astype(np.float64) * x).sum(axis=1)
+    mag = np.abs(NP.DEQUANT[t](raw).reshape(d, n).astype(np.float64) * x).sum(axis=1)
+    for flavour in (O.DOT_SCALAR, O.DOT_VEC128, O.DOT_VEC256):
+        got = O.matmul(t, raw, x, d, n, flavour)
+        assert np.max(np.abs(got - ref) / mag) < 2e-6
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_matmul_thread_count_and_batching_are_invisible(t):
+    """FloatTensor.java:123-140: rows are independent dots, so the thread count cannot change a
+    bit, and the batched form is B single-vector calls."""
+    from jitllm_amd import synthetic
+    n, d, B = 512, 37, 5
+    raw = synthetic.weight(t, d, n, seed=7)
+    X = synthetic.activations((B, n), seed=8)
+    for flavour in (O.DOT_SCALAR, O.DOT_VEC256):
+        one = O.matmul_batch(t, raw, X, d, n, flavour, nthreads=1)
+        many = O.matmul_batch(t, raw, X, d, n, flavour, nthreads=4)
+        assert_bit_equal(one, many)
+        for b in range(B):
+            assert_bit_equal(one[b], O.matmul(t, raw, X[b], d, n, flavour, nthreads=3))
+
+
+def test_vector_dot_unaligned_head_and_tail_use_scalar():
+    from jitllm_amd import synthetic
+    raw = synthetic.weight(O.Q8_0, 1, 256, seed=3)
+    x = synthetic.activations(256, seed=4)
+    # offset 32, size 40: one vector block then an 8-element scalar tail
+    got = O.dot(O.Q8_0, O.DOT_VEC256, raw, 32, x, 32, 40)
+    val = NP.vector_lane_values(O.Q8_0, raw[34:68], x[32:64], 256)
+    head = np.float32(0)
+    for v in val:
+        head = np.float32(head + v)
+    tail = np.float32(0)
+    deq = NP.dequant_q8_0(raw)
+    for j in range(64, 72):
+        tail = np.float32(tail + np.float32(deq[j] * x[j]))
+    want = np.float32(np.float32(0) + head)
+    want = np.float32(want + tail)
+    assert abs(float(got) - float(want)) <= 1e-5 * abs(float(want)) + 1e-6
+
+
+def test_swiglu_form():
+    g = np.array([-30.0, -1.5, 0.0, 0.25, 3.0, 40.0], dtype=np.float32)
+    u = np.array([2.0, -1.0, 5.0, 4.0, 0.5, 1.0], dtype=np.float32)
+    got = O.swiglu(g, u)
+    want = (g / (1.0 + np.exp(-g.astype(np.float64))).astype(np.float32)).astype(np.float32) * u
+    assert_bit_equal(got, want.astype(np.float32))
+    assert got[2] == 0.0 and got[5] == 40.0
+
+
+# ---- int8 activation path -------------------------------------------------------------------
+
+def test_quantize_q8_definition():
+    """Int8GemmKernels.java:75-129: d = amax/127, q = round-half-away(x * (127/amax)), zero block
+    -> zero scale and zero quants."""
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((6, 64)).astype(np.float32)
+    x[1, 0:32] = 0.0
+    x[2, 32:64] *= 1e-38
+    x[3, 5] = 2.5  # amax element maps to exactly +-127
+    q, s = O.quantize_q8(x)
+    xb = x.reshape(-1, 32)
+    amax = np.abs(xb).max(axis=1)
+    assert_bit_equal(s.reshape(-1), (amax / np.float32(127.0)).astype(np.float32))
+    assert np.all(q.reshape(-1, 32)[amax == 0] == 0)
+    nz = amax >= 4e-37
+    inv = (np.float32(127.0) / amax[nz]).astype(np.float32)
+    v = (xb[nz] * inv[:, None]).astype(np.float32)
+    want = np.sign(v) * np.floor(np.abs(v) + np.float32(0.5))
+    assert np.array_equal(q.reshape(-1, 32)[nz], np.clip(want, -127, 127).astype(np.int8))
+    assert np.abs(q).max() == 127
+
+
+def test_int8_gemm_matches_fp64_product_of_the_quantised_operands():
+    """Qwen35Q8_0Int8ProjectionAccelTest.java:101-172: m=256, n=384, k=320, seeds 21/22; only the
+    fp32 accumulation separates the GEMM from the fp64 product; worst/magnitude < 1e-5."""
+    m, n, k = 256, 384, 320
+    raw = FX.int8_gemm_weights(n, k, 21)
+    a = FX.int8_gemm_activations(m, k, 22)
+    q, s = O.quantize_q8(a)
+    got = O.gemm_int8_block_scaled(O.Q8_0, q, s, raw, n)
+    b = raw.reshape(n, k // 32, 34)
+    dw = b[:, :, 0:2].copy().view(np.uint16)[:, :, 0].view(np.float16).astype(np.float64)
+    wq = b[:, :, 2:].view(np.int8).astype(np.int64)
+    dots = np.einsum("mbi,nbi->mnb", q.reshape(m, k // 32, 32).astype(np.int64), wq)
+    terms = dots.astype(np.float64) * s.astype(np.float64)[:, None, :] * dw[None, :, :]
+    worst = np.max(np.abs(got - terms.sum(axis=2)) / np.abs(terms).sum(axis=2))
+    assert worst < 1e-5
