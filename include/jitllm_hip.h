@@ -1,0 +1,179 @@
+/*
+ * jitllm_hip.h -- C ABI of libjitllm_hip.so: jitLLM's quantized weight projections on one MI355X.
+ *
+ * The library replaces, inside a forward pass, the TornadoVM tasks behind three Java seams of the
+ * reference (J = src/main/java/org/beehive/jitllm):
+ *   decode          J/backend/tornado/layers/QuantizedProjections.java        (matvec, floatMatvec,
+ *                   residualMatvec, gateUp, and the fused q|k|v kernels its layer builders call)
+ *   batched decode  J/backend/tornado/layers/QuantizedBatchProjections.java   (projection, gateUp)
+ *   batched prefill J/backend/tornado/ops/Implementation.java + Instance.java (needs/create/emit)
+ * Weights are GGUF blocks in the file's own layout (Q8_0 34 B / 32, Q4_0 18 B / 32, Q4_K 144 B /
+ * 256; J/format/GGMLType.java:7,13,18-20), uploaded once and never converted.  Activations and
+ * outputs are fp32 device buffers that the caller owns and rebinds by value, never by address.
+ *
+ * Conventions
+ *   - every entry point returns JL_OK (0) or a negative jl_status; jl_last_error() then names the
+ *     cause on the calling thread.  Nothing falls back silently: an unsupported combination is
+ *     JL_ERR_UNSUPPORTED, never a slower path computing something else.
+ *   - `n` is the row length (input features), `d` the row count (output features), as in the
+ *     reference's kernels.  A `[d x n]` weight is d rows of n / block_elems blocks, row-major.
+ *   - all work is enqueued on the context's HIP stream and is ordered on it; no entry point below
+ *     jl_weight_upload / jl_malloc allocates device memory.
+ *   - a context is used by one host thread at a time (the reference's sessions are
+ *     single-threaded: docs/architecture/memory-and-concurrency.md:101-115).
+ */
+#ifndef JITLLM_HIP_H
+#define JITLLM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JL_ABI_VERSION 1
+
+typedef enum jl_status {
+    JL_OK = 0,
+    JL_ERR_INVALID = -1,     /* bad argument: null pointer, shape that is not whole blocks, ... */
+    JL_ERR_UNSUPPORTED = -2, /* combination with no kernel (IllegalStateException "no ... kernel for") */
+    JL_ERR_HIP = -3,         /* a HIP runtime call failed; the message carries hipGetErrorString */
+    JL_ERR_OOM = -4,         /* device allocation failed (the reference's GPUL-MEM-001) */
+    JL_ERR_WORKSPACE = -5    /* caller's workspace smaller than jl_gemm_workspace_bytes asked for */
+} jl_status;
+
+/* ggml type ids as a GGUF tensor-info record carries them (GGMLType ordinals). */
+typedef enum jl_ggml_type { JL_Q4_0 = 2, JL_Q8_0 = 8, JL_Q4_K = 12 } jl_ggml_type;
+
+/* What a projection does with its result (Int8GemmKernels.java:617-621 EPILOGUE_*). */
+typedef enum jl_epilogue {
+    JL_STORE = 0,    /* out  = W.x                                                   */
+    JL_RESIDUAL = 1, /* out += W.x   (matrixVectorGenericWithResidual*, residualMatvec) */
+    JL_SWIGLU = 2    /* out  = SiLU(W1.x) * (W3.x), SiLU(g) = g / (1 + exp(-g))       */
+} jl_epilogue;
+
+/* Arithmetic of the batched GEMM (jl_gemm). */
+typedef enum jl_gemm_math {
+    JL_MATH_DEFAULT = 0, /* JL_MATH_F16 for every type                                         */
+    JL_MATH_F16 = 1,     /* weights decoded to fp16 in LDS, activations rounded to fp16, fp32  */
+                         /* accumulation on fp16 MFMA (TransformerBatchPrefillKernels gemmMMAQ8) */
+    JL_MATH_INT8 = 2     /* activations quantised per 32-block to int8, int8 MFMA, one fp32     */
+                         /* scale product per block (Int8GemmKernels.java:17-23); Q8_0 and Q4_0 */
+} jl_gemm_math;
+
+typedef struct jl_context jl_context;
+typedef struct jl_weight jl_weight;
+
+int jl_abi_version(void);
+const char *jl_last_error(void);
+
+/* ---- context: one device, one stream ------------------------------------------------------- */
+
+/* Creates a context on `device` with a stream of its own (default priority). */
+int jl_context_create(int device, jl_context **out);
+/* Same, on a stream the caller owns (a hipStream_t); the stream is borrowed, never destroyed. */
+int jl_context_create_on_stream(int device, void *hip_stream, jl_context **out);
+int jl_context_destroy(jl_context *ctx);
+/* Blocks until everything enqueued on the context's stream has finished. */
+int jl_sync(jl_context *ctx);
+void *jl_context_stream(jl_context *ctx);
+/* Compute units of the device and its name (DeviceCapability of the reference's backend SPI). */
+int jl_device_info(jl_context *ctx, int *compute_units, char *name, size_t name_bytes);
+
+/* ---- device buffers for fp32 activations (TornadoVM FloatArray of the reference) ----------- */
+
+int jl_malloc(jl_context *ctx, size_t bytes, void **device_ptr);
+int jl_free(jl_context *ctx, void *device_ptr);
+/* Stream-ordered copies; the host side has returned only after the copy completed. */
+int jl_upload(jl_context *ctx, void *device_dst, const void *host_src, size_t bytes);
+int jl_download(jl_context *ctx, void *host_dst, const void *device_src, size_t bytes);
+/* Fills `count` floats with `value` (FloatArray.init). */
+int jl_fill_f32(jl_context *ctx, float *device_dst, float value, size_t count);
+
+/* ---- weights (TornadoTensor: J/backend/tornado/tensor/TornadoTensor.java:17-101) ----------- */
+
+/*
+ * Uploads the raw blocks of a `[rows x cols]` weight as the GGUF file stores them, with no
+ * conversion (ModelLoader.loadTornadoTensorNative, J/model/loader/ModelLoader.java:246-290).
+ * `host_blocks` points at the first block, i.e. past the 16-byte array header the reference's
+ * mmapped segments carry (TornadoTensorLoader.java:42-44).
+ */
+int jl_weight_upload(jl_context *ctx, int ggml_type, const void *host_blocks, int64_t rows,
+                     int64_t cols, jl_weight **out);
+/* Wraps blocks already resident in device memory (16-byte aligned); nothing is copied or owned. */
+int jl_weight_wrap(jl_context *ctx, int ggml_type, const void *device_blocks, int64_t rows,
+                   int64_t cols, jl_weight **out);
+int jl_weight_free(jl_weight *w);
+int jl_weight_info(const jl_weight *w, int *ggml_type, int64_t *rows, int64_t *cols,
+                   int64_t *bytes);
+/* Device address of the blocks (TornadoTensor.asByteArray). */
+const void *jl_weight_blocks(const jl_weight *w);
+
+/*
+ * Decodes every element to fp32 with the host tensor's own arithmetic -- bit for bit what
+ * Q8_0FloatTensor.getFloat (Q8_0FloatTensor.java:52-61), Q4_0FloatTensor.getFloat
+ * (Q4_0FloatTensor.java:55-79) and Q4_KFloatTensor.getFloat (Q4_KFloatTensor.java:87-122) return.
+ * `out` holds rows * cols floats.  The parity probe; also dequantize*ToFP16's fp32 sibling.
+ */
+int jl_dequant_f32(jl_context *ctx, const jl_weight *w, float *out);
+
+/* ---- decode: one activation vector (QuantizedProjections.java) ----------------------------- */
+
+/*
+ * out = W.x (JL_STORE; QuantizedProjections.floatMatvec :200-254, matrixVectorGenericQ8Byte,
+ * matrixVectorGenericQ4_0, matrixVectorGenericQ4_K) or out += W.x (JL_RESIDUAL;
+ * QuantizedProjections.residualMatvec :260-379).  x holds cols floats, out rows floats.
+ */
+int jl_gemv(jl_context *ctx, const jl_weight *w, const float *x, float *out, int epilogue);
+
+/*
+ * q = Wq.x, k = Wk.x, v = Wv.x in one launch (fusedQKVMatmulQ8,
+ * TransformerComputeKernelsLayered.java:2488+; fusedQKVMatmulQ4_0; fusedQKVMatmulQ4_KNonSquare).
+ * The three weights share the type and the row length.
+ */
+int jl_gemv_qkv(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const jl_weight *wv,
+                const float *x, float *q, float *k, float *v);
+
+/*
+ * hb = SiLU(W1.x) * (W3.x) in one launch (fusedFeedForwardWithSiLUAndGLUActivationQ8_0Byte,
+ * TransformerComputeKernelsLayered.java:2453-2479; fusedFFNGateUpSiLUQ4_0; fusedFFNGateUpSiLUQ4_K;
+ * QuantizedProjections.gateUp :400-480).  Both weights share type and shape; a mixed pair is
+ * JL_ERR_UNSUPPORTED and the caller runs two jl_gemv and jl_swiglu, as the reference does.
+ */
+int jl_gemv_gate_up(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, const float *x,
+                    float *hb);
+
+/* gate[i] = SiLU(gate[i]) * up[i] (siluAndMultiply; the unfused tail of gateUp). */
+int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
+
+/* ---- batched decode and batched prefill: `batch` activation rows ---------------------------- */
+
+/*
+ * Bytes of scratch jl_gemm needs for a call of this shape (Implementation.needs,
+ * J/backend/tornado/ops/Implementation.java:31-36: sized before anything is allocated, so a
+ * memory preflight equals what the call uses).  `max_rows` is the largest `batch`, `cols` the
+ * row length, `math` a jl_gemm_math.
+ */
+size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int math);
+
+/*
+ * C[b][col_offset + j] (op)= sum_k X[b][k] * W_i[j][k] for the `count` weights laid side by
+ * side (C = A.[W0|W1|...]^T, FP16Projections / DecodedMatMul.project :93-109), over the first
+ * `active_rows` of `batch` rows; rows past active_rows are left exactly as they were
+ * (QuantizedBatchProjections.projection :76-309, matrixVectorTiledBatchQ4_0/Q4_K's activeRows).
+ *   X    [batch x cols] fp32 row-major          C  fp32, row stride `ldo` floats
+ *   epilogue JL_STORE / JL_RESIDUAL, or JL_SWIGLU with count == 2 (gate, up):
+ *            C[b][col_offset + j] = SiLU(X_b.W0_j) * (X_b.W1_j)
+ *   math     a jl_gemm_math; JL_MATH_INT8 with a Q4_K weight is JL_ERR_UNSUPPORTED
+ * This is Int8GemmKernels.gemmInt8Q8_0's contract (:651-676: epilogue, rowsHolder, ldo,
+ * colOffset) and gemmMMAQ8's, behind one call.
+ */
+int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
+            int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
+            int math, void *workspace, size_t workspace_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

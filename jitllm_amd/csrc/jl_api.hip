@@ -1,0 +1,306 @@
+// C-ABI entry points of libjitllm_hip.so: context, device buffers, weights, argument checks.
+// The kernels live in jl_dequant.hip, jl_gemv.hip and jl_gemm.hip.
+#include <stdarg.h>
+#include <string.h>
+
+#include <new>
+
+#include "jl_internal.h"
+
+static thread_local char g_error[512] = "";
+
+int jl_fail(int status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+extern "C" {
+
+int jl_abi_version(void) { return JL_ABI_VERSION; }
+
+const char *jl_last_error(void) { return g_error; }
+
+static int context_create(int device, hipStream_t borrowed, bool borrow, jl_context **out) {
+    JL_REQUIRE(out != nullptr, "jl_context_create: out is null");
+    *out = nullptr;
+    int count = 0;
+    JL_HIP(hipGetDeviceCount(&count));
+    JL_REQUIRE(device >= 0 && device < count, "jl_context_create: device %d of %d", device, count);
+    JL_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    JL_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "device %d is %s; this library carries gfx950 (MI355X) code only", device,
+                       prop.gcnArchName);
+    }
+    jl_context *ctx = new (std::nothrow) jl_context();
+    JL_REQUIRE(ctx != nullptr, "jl_context_create: host allocation failed");
+    ctx->device = device;
+    ctx->compute_units = prop.multiProcessorCount;
+    snprintf(ctx->name, sizeof ctx->name, "%s", prop.name);
+    if (borrow) {
+        ctx->stream = borrowed;
+        ctx->owns_stream = false;
+    } else {
+        hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+        if (e != hipSuccess) {
+            delete ctx;
+            return jl_fail(JL_ERR_HIP, "hipStreamCreateWithFlags failed: %s", hipGetErrorString(e));
+        }
+        ctx->owns_stream = true;
+    }
+    *out = ctx;
+    return JL_OK;
+}
+
+int jl_context_create(int device, jl_context **out) {
+    return context_create(device, nullptr, false, out);
+}
+
+int jl_context_create_on_stream(int device, void *hip_stream, jl_context **out) {
+    return context_create(device, (hipStream_t)hip_stream, true, out);
+}
+
+int jl_context_destroy(jl_context *ctx) {
+    if (!ctx) return JL_OK;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return JL_OK;
+}
+
+int jl_sync(jl_context *ctx) {
+    JL_REQUIRE(ctx != nullptr, "jl_sync: context is null");
+    JL_HIP(hipStreamSynchronize(ctx->stream));
+    return JL_OK;
+}
+
+void *jl_context_stream(jl_context *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+int jl_device_info(jl_context *ctx, int *compute_units, char *name, size_t name_bytes) {
+    JL_REQUIRE(ctx != nullptr, "jl_device_info: context is null");
+    if (compute_units) *compute_units = ctx->compute_units;
+    if (name && name_bytes) snprintf(name, name_bytes, "%s", ctx->name);
+    return JL_OK;
+}
+
+int jl_malloc(jl_context *ctx, size_t bytes, void **device_ptr) {
+    JL_REQUIRE(ctx && device_ptr, "jl_malloc: null argument");
+    *device_ptr = nullptr;
+    JL_HIP(hipSetDevice(ctx->device));
+    hipError_t e = hipMalloc(device_ptr, bytes ? bytes : 16);
+    if (e != hipSuccess) {
+        return jl_fail(JL_ERR_OOM, "device allocation of %zu bytes failed: %s", bytes,
+                       hipGetErrorString(e));
+    }
+    return JL_OK;
+}
+
+int jl_free(jl_context *ctx, void *device_ptr) {
+    JL_REQUIRE(ctx != nullptr, "jl_free: context is null");
+    if (!device_ptr) return JL_OK;
+    JL_HIP(hipStreamSynchronize(ctx->stream));
+    JL_HIP(hipFree(device_ptr));
+    return JL_OK;
+}
+
+int jl_upload(jl_context *ctx, void *device_dst, const void *host_src, size_t bytes) {
+    JL_REQUIRE(ctx && (bytes == 0 || (device_dst && host_src)), "jl_upload: null argument");
+    if (!bytes) return JL_OK;
+    JL_HIP(hipMemcpyAsync(device_dst, host_src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    JL_HIP(hipStreamSynchronize(ctx->stream));
+    return JL_OK;
+}
+
+int jl_download(jl_context *ctx, void *host_dst, const void *device_src, size_t bytes) {
+    JL_REQUIRE(ctx && (bytes == 0 || (host_dst && device_src)), "jl_download: null argument");
+    if (!bytes) return JL_OK;
+    JL_HIP(hipMemcpyAsync(host_dst, device_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    JL_HIP(hipStreamSynchronize(ctx->stream));
+    return JL_OK;
+}
+
+int jl_fill_f32(jl_context *ctx, float *device_dst, float value, size_t count) {
+    JL_REQUIRE(ctx && (count == 0 || device_dst), "jl_fill_f32: null argument");
+    if (!count) return JL_OK;
+    return jl_launch_fill(ctx, device_dst, value, count);
+}
+
+static int weight_check(const char *who, int type, int64_t rows, int64_t cols) {
+    if (jl_block_elems(type) == 0) {
+        return jl_fail(JL_ERR_UNSUPPORTED, "%s: no projection kernel for a ggml type %d weight", who,
+                       type);
+    }
+    JL_REQUIRE(rows > 0 && cols > 0, "%s: shape %lld x %lld", who, (long long)rows, (long long)cols);
+    JL_REQUIRE(cols % jl_block_elems(type) == 0,
+               "%s: row length %lld is not a whole number of %s blocks (%d)", who, (long long)cols,
+               jl_type_name(type), jl_block_elems(type));
+    JL_REQUIRE(rows <= INT32_MAX && cols <= INT32_MAX, "%s: shape exceeds 2^31", who);
+    return JL_OK;
+}
+
+int jl_weight_upload(jl_context *ctx, int ggml_type, const void *host_blocks, int64_t rows,
+                     int64_t cols, jl_weight **out) {
+    JL_REQUIRE(ctx && host_blocks && out, "jl_weight_upload: null argument");
+    *out = nullptr;
+    int st = weight_check("jl_weight_upload", ggml_type, rows, cols);
+    if (st != JL_OK) return st;
+    int64_t bytes = rows * (cols / jl_block_elems(ggml_type)) * jl_block_bytes(ggml_type);
+    void *dev = nullptr;
+    st = jl_malloc(ctx, (size_t)bytes, &dev);
+    if (st != JL_OK) return st;
+    st = jl_upload(ctx, dev, host_blocks, (size_t)bytes);
+    if (st != JL_OK) {
+        (void)hipFree(dev);
+        return st;
+    }
+    jl_weight *w = new (std::nothrow) jl_weight();
+    if (!w) {
+        (void)hipFree(dev);
+        return jl_fail(JL_ERR_INVALID, "jl_weight_upload: host allocation failed");
+    }
+    *w = jl_weight{ctx, ggml_type, rows, cols, bytes, (const uint8_t *)dev, true};
+    *out = w;
+    return JL_OK;
+}
+
+int jl_weight_wrap(jl_context *ctx, int ggml_type, const void *device_blocks, int64_t rows,
+                   int64_t cols, jl_weight **out) {
+    JL_REQUIRE(ctx && device_blocks && out, "jl_weight_wrap: null argument");
+    *out = nullptr;
+    int st = weight_check("jl_weight_wrap", ggml_type, rows, cols);
+    if (st != JL_OK) return st;
+    JL_REQUIRE(((uintptr_t)device_blocks & 15) == 0,
+               "jl_weight_wrap: blocks must be 16-byte aligned in device memory");
+    int64_t bytes = rows * (cols / jl_block_elems(ggml_type)) * jl_block_bytes(ggml_type);
+    jl_weight *w = new (std::nothrow) jl_weight();
+    JL_REQUIRE(w != nullptr, "jl_weight_wrap: host allocation failed");
+    *w = jl_weight{ctx, ggml_type, rows, cols, bytes, (const uint8_t *)device_blocks, false};
+    *out = w;
+    return JL_OK;
+}
+
+int jl_weight_free(jl_weight *w) {
+    if (!w) return JL_OK;
+    int st = JL_OK;
+    if (w->owns_blocks) st = jl_free(w->ctx, (void *)w->blocks);
+    delete w;
+    return st;
+}
+
+int jl_weight_info(const jl_weight *w, int *ggml_type, int64_t *rows, int64_t *cols,
+                   int64_t *bytes) {
+    JL_REQUIRE(w != nullptr, "jl_weight_info: weight is null");
+    if (ggml_type) *ggml_type = w->type;
+    if (rows) *rows = w->rows;
+    if (cols) *cols = w->cols;
+    if (bytes) *bytes = w->bytes;
+    return JL_OK;
+}
+
+const void *jl_weight_blocks(const jl_weight *w) { return w ? w->blocks : nullptr; }
+
+int jl_dequant_f32(jl_context *ctx, const jl_weight *w, float *out) {
+    JL_REQUIRE(ctx && w && out, "jl_dequant_f32: null argument");
+    return jl_launch_dequant(ctx, w, out);
+}
+
+int jl_gemv(jl_context *ctx, const jl_weight *w, const float *x, float *out, int epilogue) {
+    JL_REQUIRE(ctx && w && x && out, "jl_gemv: null argument");
+    JL_REQUIRE(epilogue == JL_STORE || epilogue == JL_RESIDUAL,
+               "jl_gemv: epilogue %d (JL_STORE or JL_RESIDUAL)", epilogue);
+    return jl_launch_gemv(ctx, &w, 1, &out, nullptr, x, epilogue);
+}
+
+int jl_gemv_qkv(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const jl_weight *wv,
+                const float *x, float *q, float *k, float *v) {
+    JL_REQUIRE(ctx && wq && wk && wv && x && q && k && v, "jl_gemv_qkv: null argument");
+    if (wq->type != wk->type || wq->type != wv->type) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "jl_gemv_qkv: no fused q|k|v kernel for mixed weights %s/%s/%s",
+                       jl_type_name(wq->type), jl_type_name(wk->type), jl_type_name(wv->type));
+    }
+    JL_REQUIRE(wq->cols == wk->cols && wq->cols == wv->cols,
+               "jl_gemv_qkv: row lengths differ (%lld, %lld, %lld)", (long long)wq->cols,
+               (long long)wk->cols, (long long)wv->cols);
+    const jl_weight *ws[3] = {wq, wk, wv};
+    float *outs[3] = {q, k, v};
+    return jl_launch_gemv(ctx, ws, 3, outs, nullptr, x, JL_STORE);
+}
+
+int jl_gemv_gate_up(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, const float *x,
+                    float *hb) {
+    JL_REQUIRE(ctx && w1 && w3 && x && hb, "jl_gemv_gate_up: null argument");
+    if (w1->type != w3->type) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "jl_gemv_gate_up: no fused gate/up kernel for a %s gate and a %s up weight",
+                       jl_type_name(w1->type), jl_type_name(w3->type));
+    }
+    JL_REQUIRE(w1->rows == w3->rows && w1->cols == w3->cols,
+               "jl_gemv_gate_up: gate is %lld x %lld, up is %lld x %lld", (long long)w1->rows,
+               (long long)w1->cols, (long long)w3->rows, (long long)w3->cols);
+    return jl_launch_gemv(ctx, &w1, 1, &hb, w3, x, JL_SWIGLU);
+}
+
+int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count) {
+    JL_REQUIRE(ctx && gate && up && count >= 0, "jl_swiglu: bad argument");
+    if (!count) return JL_OK;
+    return jl_launch_swiglu(ctx, gate, up, count);
+}
+
+size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int math) {
+    if (max_rows <= 0 || cols <= 0) return 0;
+    return jl_gemm_workspace_bytes_impl(max_rows, cols, math);
+}
+
+int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
+            int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
+            int math, void *workspace, size_t workspace_bytes) {
+    JL_REQUIRE(ctx && weights && X && C, "jl_gemm: null argument");
+    JL_REQUIRE(count >= 1 && count <= 8, "jl_gemm: %d weights (1..8)", count);
+    JL_REQUIRE(batch >= 1 && active_rows >= 0 && active_rows <= batch,
+               "jl_gemm: active_rows %lld of batch %lld", (long long)active_rows, (long long)batch);
+    JL_REQUIRE(epilogue == JL_STORE || epilogue == JL_RESIDUAL || epilogue == JL_SWIGLU,
+               "jl_gemm: epilogue %d", epilogue);
+    int64_t total = 0;
+    for (int i = 0; i < count; i++) {
+        JL_REQUIRE(weights[i] != nullptr, "jl_gemm: weight %d is null", i);
+        if (weights[i]->type != weights[0]->type) {
+            return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: mixed weight types %s and %s in one call",
+                           jl_type_name(weights[0]->type), jl_type_name(weights[i]->type));
+        }
+        JL_REQUIRE(weights[i]->cols == weights[0]->cols, "jl_gemm: weight %d row length %lld != %lld",
+                   i, (long long)weights[i]->cols, (long long)weights[0]->cols);
+        total += weights[i]->rows;
+    }
+    if (epilogue == JL_SWIGLU) {
+        JL_REQUIRE(count == 2 && weights[0]->rows == weights[1]->rows,
+                   "jl_gemm: JL_SWIGLU takes a gate and an up weight of equal shape");
+        total = weights[0]->rows;
+    }
+    JL_REQUIRE(col_offset >= 0 && ldo >= col_offset + total,
+               "jl_gemm: ldo %lld < col_offset %lld + %lld output columns", (long long)ldo,
+               (long long)col_offset, (long long)total);
+    if (math == JL_MATH_DEFAULT) math = JL_MATH_F16;
+    JL_REQUIRE(math == JL_MATH_F16 || math == JL_MATH_INT8, "jl_gemm: math %d", math);
+    if (math == JL_MATH_INT8 && weights[0]->type == JL_Q4_K) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "jl_gemm: no int8 kernel for a Q4_K weight (d*sc*q - dmin*m is not an int8 "
+                       "value); use JL_MATH_F16");
+    }
+    if (active_rows == 0) return JL_OK;
+    size_t need = jl_gemm_workspace_bytes_impl(batch, weights[0]->cols, math);
+    if (workspace_bytes < need || (need && !workspace)) {
+        return jl_fail(JL_ERR_WORKSPACE, "jl_gemm: workspace %zu bytes, %zu needed", workspace_bytes,
+                       need);
+    }
+    return jl_launch_gemm(ctx, weights, count, X, C, batch, active_rows, ldo, col_offset, epilogue,
+                          math, workspace, workspace_bytes);
+}
+
+}  // extern "C"

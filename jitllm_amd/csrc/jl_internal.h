@@ -1,0 +1,64 @@
+// Host-side internals shared by the translation units of libjitllm_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/jitllm_hip.h"
+
+struct jl_context {
+    int device;
+    hipStream_t stream;
+    bool owns_stream;
+    int compute_units;
+    char name[128];
+};
+
+struct jl_weight {
+    jl_context *ctx;
+    int type;
+    int64_t rows;
+    int64_t cols;
+    int64_t bytes;
+    const uint8_t *blocks;  // device address of the first block
+    bool owns_blocks;
+};
+
+// Block geometry (reference: J/format/GGMLType.java:7,13,18-20).
+static inline int jl_block_elems(int type) {
+    return type == JL_Q4_K ? 256 : (type == JL_Q8_0 || type == JL_Q4_0) ? 32 : 0;
+}
+static inline int jl_block_bytes(int type) {
+    return type == JL_Q4_K ? 144 : type == JL_Q8_0 ? 34 : type == JL_Q4_0 ? 18 : 0;
+}
+static inline const char *jl_type_name(int type) {
+    return type == JL_Q4_K ? "Q4_K" : type == JL_Q8_0 ? "Q8_0" : type == JL_Q4_0 ? "Q4_0" : "?";
+}
+
+// Records the calling thread's error message and returns `status`.
+int jl_fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define JL_HIP(call)                                                                      \
+    do {                                                                                  \
+        hipError_t e_ = (call);                                                           \
+        if (e_ != hipSuccess)                                                             \
+            return jl_fail(e_ == hipErrorOutOfMemory ? JL_ERR_OOM : JL_ERR_HIP,           \
+                           "%s failed: %s", #call, hipGetErrorString(e_));                \
+    } while (0)
+
+#define JL_REQUIRE(cond, ...)                                  \
+    do {                                                       \
+        if (!(cond)) return jl_fail(JL_ERR_INVALID, __VA_ARGS__); \
+    } while (0)
+
+// Launchers implemented per translation unit; each returns a jl_status.
+int jl_launch_dequant(jl_context *ctx, const jl_weight *w, float *out);
+int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *const *outs,
+                   const jl_weight *w_up, const float *x, int epilogue);
+int jl_launch_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
+int jl_launch_fill(jl_context *ctx, float *dst, float value, size_t count);
+int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
+                   float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
+                   int epilogue, int math, void *workspace, size_t workspace_bytes);
+size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int math);

@@ -1,0 +1,152 @@
+"""Host mirror of the reference's projection seams, issuing HIP kernels through the C ABI.
+
+``QuantizedProjections`` mirrors J/backend/tornado/layers/QuantizedProjections.java (decode, one
+activation vector) and ``QuantizedBatchProjections`` mirrors
+J/backend/tornado/layers/QuantizedBatchProjections.java (``batchSize`` activation rows), with the
+same method names, argument meaning (``n`` = row length, ``d`` = output rows) and error behaviour:
+a combination with no kernel raises, it never runs something else.  Where the reference adds a task
+to a TaskGraph, these enqueue the kernel on the context's stream; the ``graph`` / ``name`` arguments
+of the reference therefore disappear.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+from . import _lib as L
+from .ggml import GGMLType
+from .runtime import Context, DeviceBuffer, FloatArray, TornadoTensor
+
+FUSED_GATE_UP_TYPES = (GGMLType.Q8_0, GGMLType.Q4_0, GGMLType.Q4_K)
+
+
+@dataclass
+class TornadoWorkspace:
+    """The persistent activation arrays a layer's projections read and write
+    (J/backend/tornado/workspace/TornadoWorkspace.java): bound once, values move, arrays never."""
+    wrapX: FloatArray | None = None
+    wrapXb: FloatArray | None = None
+    wrapHb: FloatArray | None = None
+    wrapHb2: FloatArray | None = None
+
+
+def _check_shape(w: TornadoTensor, n: int, d: int) -> None:
+    if (w.cols, w.rows) != (n, d):
+        raise ValueError(f"weight is {w.rows}x{w.cols}, projection asked for d={d}, n={n}")
+
+
+class QuantizedProjections:
+    """Single-token projections over weights kept in the file's representations."""
+
+    def __init__(self, context: Context, ws: TornadoWorkspace):
+        self.context = context
+        self.ws = ws
+        self._lib = context._lib
+
+    def packed(self) -> bool:
+        """The packed-integer (quantised activation) decode path of the reference is not part of
+        this library: the projections read fp32 activations, as the CPU path does."""
+        return False
+
+    def matvec(self, out: FloatArray, w: TornadoTensor, n: int, d: int) -> None:
+        """``out = w . wrapXb`` (QuantizedProjections.java:140-194)."""
+        self.floatMatvec(self.ws.wrapXb, out, w, n, d)
+
+    def floatMatvec(self, x: FloatArray, out: FloatArray, w: TornadoTensor, n: int, d: int) -> None:
+        """``out = w . x`` (QuantizedProjections.java:200-254)."""
+        _check_shape(w, n, d)
+        L.check(self._lib.jl_gemv(self.context.handle, w.handle, x.ptr, out.ptr, L.JL_STORE))
+
+    def residualMatvec(self, x: FloatArray, w: TornadoTensor, n: int, d: int) -> None:
+        """``wrapX += w . x`` (QuantizedProjections.java:260-379)."""
+        _check_shape(w, n, d)
+        L.check(self._lib.jl_gemv(self.context.handle, w.handle, x.ptr, self.ws.wrapX.ptr,
+                                  L.JL_RESIDUAL))
+
+    def fusedQKV(self, x: FloatArray, q: FloatArray, k: FloatArray, v: FloatArray,
+                 wq: TornadoTensor, wk: TornadoTensor, wv: TornadoTensor) -> None:
+        """q | k | v in one launch (fusedQKVMatmulQ8 and its Q4_0 / Q4_K siblings, called directly
+        on the kernels by the reference's layer builders, LlamaQ8_0FFNLayers.java:316-329)."""
+        L.check(self._lib.jl_gemv_qkv(self.context.handle, wq.handle, wk.handle, wv.handle, x.ptr,
+                                      q.ptr, k.ptr, v.ptr))
+
+    def fusedGateUp(self, w1: TornadoTensor, w3: TornadoTensor) -> bool:
+        """QuantizedProjections.java:386-393."""
+        return w1.data_type() == w3.data_type() and w1.data_type() in FUSED_GATE_UP_TYPES
+
+    def gateUp(self, w1: TornadoTensor, w3: TornadoTensor, n: int, d: int) -> None:
+        """``wrapHb = SiLU(w1 . wrapXb) * (w3 . wrapXb)`` (QuantizedProjections.java:400-480): one
+        fused launch where both weights share a type, else two projections into ``wrapHb`` and
+        ``wrapHb2`` and an element-wise SwiGLU."""
+        _check_shape(w1, n, d)
+        _check_shape(w3, n, d)
+        if self.fusedGateUp(w1, w3):
+            L.check(self._lib.jl_gemv_gate_up(self.context.handle, w1.handle, w3.handle,
+                                              self.ws.wrapXb.ptr, self.ws.wrapHb.ptr))
+            return
+        if self.ws.wrapHb2 is None:
+            raise RuntimeError("a layer that splits gate and up needs wrapHb2 bound")
+        self.matvec(self.ws.wrapHb, w1, n, d)
+        self.matvec(self.ws.wrapHb2, w3, n, d)
+        L.check(self._lib.jl_swiglu(self.context.handle, self.ws.wrapHb.ptr, self.ws.wrapHb2.ptr, d))
+
+
+class QuantizedBatchProjections:
+    """Projections of ``batchSize`` activation rows at once (batched decode, batched prefill)."""
+
+    def __init__(self, context: Context, batchSize: int, max_cols: int, math: int = L.JL_MATH_DEFAULT):
+        self.context = context
+        self.batchSize = int(batchSize)
+        self.math = math
+        self._lib = context._lib
+        self._max_cols = int(max_cols)
+        nbytes = self._lib.jl_gemm_workspace_bytes(self.batchSize, self._max_cols, math)
+        self.workspace = DeviceBuffer(context, max(nbytes, 256))
+
+    def workspace_bytes(self) -> int:
+        return self.workspace.nbytes
+
+    def _gemm(self, weights, x: FloatArray, out: FloatArray, activeRows: int, ldo: int,
+              colOffset: int, epilogue: int) -> None:
+        n = weights[0].cols
+        if n > self._max_cols:
+            raise ValueError(f"row length {n} exceeds the {self._max_cols} the workspace was sized for")
+        arr = (C.c_void_p * len(weights))(*[w.handle for w in weights])
+        L.check(self._lib.jl_gemm(self.context.handle, arr, len(weights), x.ptr, out.ptr,
+                                  self.batchSize, activeRows, ldo, colOffset, epilogue, self.math,
+                                  self.workspace.ptr, self.workspace.nbytes))
+
+    def projection(self, x: FloatArray, out: FloatArray, w: TornadoTensor, n: int, d: int,
+                   residual: bool, activeRows: int | None = None) -> None:
+        """``out = w . x`` over the batch, or ``out += w . x`` with ``residual``
+        (QuantizedBatchProjections.java:76-309).  Rows past ``activeRows`` are left untouched."""
+        _check_shape(w, n, d)
+        rows = self.batchSize if activeRows is None else activeRows
+        self._gemm([w], x, out, rows, d, 0, L.JL_RESIDUAL if residual else L.JL_STORE)
+
+    def fusedQKV(self, x: FloatArray, out: FloatArray, wq: TornadoTensor, wk: TornadoTensor,
+                 wv: TornadoTensor, activeRows: int | None = None) -> None:
+        """``out[b] = [wq . x_b | wk . x_b | wv . x_b]``, the side-by-side layout of the
+        reference's FP16Projections (C = A . [W0|W1|W2]^T)."""
+        rows = self.batchSize if activeRows is None else activeRows
+        ldo = wq.rows + wk.rows + wv.rows
+        self._gemm([wq, wk, wv], x, out, rows, ldo, 0, L.JL_STORE)
+
+    def fusedGateUp(self, w1: TornadoTensor, w3: TornadoTensor) -> bool:
+        """QuantizedBatchProjections.java:315-321 (the tiled, non-SIMD-group answer)."""
+        return w1.data_type() == w3.data_type() and w1.data_type() in FUSED_GATE_UP_TYPES
+
+    def gateUp(self, x: FloatArray, hb: FloatArray, w1: TornadoTensor, w3: TornadoTensor, dim: int,
+               hidDim: int, activeRows: int | None = None) -> None:
+        """``hb = SiLU(w1 . x) * (w3 . x)`` over the batch (QuantizedBatchProjections.java:329-458;
+        the RMS norm the reference folds in front is not part of this path: ``x`` is already
+        normalised)."""
+        _check_shape(w1, dim, hidDim)
+        _check_shape(w3, dim, hidDim)
+        if not self.fusedGateUp(w1, w3):
+            raise L.UnsupportedProjection(
+                L.JL_ERR_UNSUPPORTED,
+                f"no fused batched gate/up kernel for a {w1.data_type().name} gate and a "
+                f"{w3.data_type().name} up weight")
+        rows = self.batchSize if activeRows is None else activeRows
+        self._gemm([w1, w3], x, hb, rows, hidDim, 0, L.JL_SWIGLU)

@@ -1,0 +1,169 @@
+"""GPU parity: batched decode and batched prefill (jl_gemm) through the C ABI."""
+import numpy as np
+import pytest
+
+import fixtures as FX
+from gpu_util import magnitude, rel_err, say
+from oracle import pyoracle as O
+
+pytestmark = pytest.mark.gpu
+
+NAMES = {O.Q8_0: "q8_0", O.Q4_0: "q4_0", O.Q4_K: "q4_K"}
+UNTOUCHED = np.float32(-12345.5)  # BatchProjectionTilingAccelTest.java:61
+F16_BOUND = 2e-3                  # fp16-MFMA path: max |d| / sum |w x|
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from jitllm_amd.runtime import Context
+    c = Context(0)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("t,what", [(O.Q4_0, "q40"), (O.Q4_K, "q4k"), (O.Q8_0, "q80")])
+def test_batch_projection_reference_fixture(ctx, t, what):
+    """BatchProjectionTilingAccelTest.java:151-215: N = 512, D = 37, widths {1,2,7,8,9,16},
+    activeRows in {1, width}; plain and residual; rows past activeRows keep -12345.5 exactly."""
+    from jitllm_amd.projections import QuantizedBatchProjections
+    raw = FX.probe_blocks(t, 20260909 + O.java_string_hash(what), both_scales=(t == O.Q4_K))
+    w = ctx.load_weight(t, raw, FX.D_PROBE, FX.N_PROBE)
+    for width in (1, 2, 7, 8, 9, 16):
+        for active in ([1] if width == 1 else [1, width]):
+            say("batch fixture", what, width, active)
+            X = FX.batch_activation(width)
+            expected = O.matmul_batch(t, raw, X[:active], FX.D_PROBE, FX.N_PROBE)
+            mag = magnitude(t, raw, X[:active], FX.D_PROBE, FX.N_PROBE)
+            proj = QuantizedBatchProjections(ctx, width, FX.N_PROBE)
+            xd = ctx.from_numpy(X)
+            for residual in (False, True):
+                out = ctx.float_array(width * FX.D_PROBE, fill=UNTOUCHED)
+                proj.projection(xd, out, w, FX.N_PROBE, FX.D_PROBE, residual, activeRows=active)
+                ctx.sync()
+                got = out.get().reshape(width, FX.D_PROBE)
+                assert np.all(got[active:] == UNTOUCHED)
+                want = expected + (UNTOUCHED if residual else np.float32(0))
+                assert rel_err(got[:active], want, mag + (12345.5 * 6e-8 if residual else 0)) < F16_BOUND
+
+
+@pytest.mark.parametrize("t,d,n,B", [
+    (O.Q4_K, 4096, 4096, 8), (O.Q4_K, 1024, 4096, 32), (O.Q4_K, 4096, 12288, 64),
+    (O.Q8_0, 2048, 2048, 64), (O.Q4_0, 1024, 4096, 33), (O.Q8_0, 200, 2048, 130),
+])
+def test_batched_projection_matches_oracle(ctx, t, d, n, B):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("batched", NAMES[t], d, n, B)
+    raw = synthetic.weight(t, d, n, seed=7000 + d)
+    X = synthetic.activations((B, n), seed=7100 + B)
+    ref = O.matmul_batch(t, raw, X, d, n, O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256)
+    w = ctx.load_weight(t, raw, d, n)
+    out = ctx.float_array(B * d, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, B, n).projection(ctx.from_numpy(X), out, w, n, d, False)
+    ctx.sync()
+    got = out.get().reshape(B, d)
+    assert np.all(got != UNTOUCHED)
+    err = rel_err(got, ref, magnitude(t, raw, X, d, n))
+    assert err < F16_BOUND, err
+    assert err < 2e-4, err  # random rounding errors: far inside the worst-case bound
+
+
+def test_batched_row_is_the_single_vector_result(ctx):
+    """FloatTensor.java:127-140: batched row b is the same dot as the single-vector call, so the
+    batched kernel's rows must agree with each other when their activations are equal."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("batched equal rows")
+    d, n, B = 512, 2048, 12
+    raw = synthetic.weight(O.Q8_0, d, n, seed=71)
+    x = synthetic.activations(n, seed=72)
+    X = np.tile(x, (B, 1))
+    out = ctx.float_array(B * d)
+    QuantizedBatchProjections(ctx, B, n).projection(ctx.from_numpy(X), out,
+                                                    ctx.load_weight(O.Q8_0, raw, d, n), n, d, False)
+    ctx.sync()
+    got = out.get().reshape(B, d)
+    assert np.all(got == got[0])
+
+
+@pytest.mark.parametrize("t,dq,dkv,n,T", [(O.Q8_0, 2048, 512, 2048, 256), (O.Q4_K, 256, 128, 1024, 70)])
+def test_prefill_fused_qkv_side_by_side(ctx, t, dq, dkv, n, T):
+    """C = A . [Wq|Wk|Wv]^T with the outputs side by side (FP16Projections / DecodedMatMul.project)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("prefill qkv", NAMES[t], dq, dkv, n, T)
+    dims = (dq, dkv, dkv)
+    raws = [synthetic.weight(t, d, n, seed=81 + i) for i, d in enumerate(dims)]
+    X = synthetic.activations((T, n), seed=85)
+    ws = [ctx.load_weight(t, r, d, n) for r, d in zip(raws, dims)]
+    ld = sum(dims)
+    out = ctx.float_array(T * ld, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n).fusedQKV(ctx.from_numpy(X), out, *ws)
+    ctx.sync()
+    got = out.get().reshape(T, ld)
+    col = 0
+    for raw, d in zip(raws, dims):
+        ref = O.matmul_batch(t, raw, X, d, n)
+        assert rel_err(got[:, col:col + d], ref, magnitude(t, raw, X, d, n)) < 2e-4
+        col += d
+
+
+@pytest.mark.parametrize("t,d,n,T", [(O.Q8_0, 1024, 2048, 96), (O.Q4_K, 200, 512, 9), (O.Q4_0, 96, 1024, 130)])
+def test_batched_gate_up(ctx, t, d, n, T):
+    """hb = SiLU(w1 . x) * (w3 . x) per row (BatchProjectionTilingAccelTest.java:409, fused gate/up)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("batched gate_up", NAMES[t], d, n, T)
+    r1 = synthetic.weight(t, d, n, seed=91)
+    r3 = synthetic.weight(t, d, n, seed=92)
+    X = synthetic.activations((T, n), seed=93)
+    g = O.matmul_batch(t, r1, X, d, n)
+    u = O.matmul_batch(t, r3, X, d, n)
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(T, d)
+    hb = ctx.float_array(T * d, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n).gateUp(ctx.from_numpy(X), hb, ctx.load_weight(t, r1, d, n),
+                                                ctx.load_weight(t, r3, d, n), n, d)
+    ctx.sync()
+    got = hb.get().reshape(T, d)
+    mg, mu = magnitude(t, r1, X, d, n), magnitude(t, r3, X, d, n)
+    bound = 2e-4 * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
+
+
+def test_huge_activation_rows_stay_finite(ctx):
+    """Rows far outside fp16's range are rescaled by a power of two, not turned into infinities."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("batched huge rows")
+    d, n, B = 128, 1024, 4
+    raw = synthetic.weight(O.Q8_0, d, n, seed=95)
+    X = synthetic.activations((B, n), seed=96)
+    X[1] *= 1e7
+    X[2] *= 1e-6
+    ref = O.matmul_batch(O.Q8_0, raw, X, d, n)
+    out = ctx.float_array(B * d)
+    QuantizedBatchProjections(ctx, B, n).projection(ctx.from_numpy(X), out,
+                                                    ctx.load_weight(O.Q8_0, raw, d, n), n, d, False)
+    ctx.sync()
+    got = out.get().reshape(B, d)
+    assert np.all(np.isfinite(got))
+    assert rel_err(got, ref, magnitude(O.Q8_0, raw, X, d, n)) < F16_BOUND
+
+
+def test_batched_errors(ctx):
+    import ctypes as C
+    from jitllm_amd import _lib as L, synthetic
+    say("batched errors")
+    lib = L.load()
+    w = ctx.load_weight(O.Q4_K, synthetic.weight(O.Q4_K, 64, 256, 1), 64, 256)
+    x, o = ctx.float_array(4 * 256, 0.0), ctx.float_array(4 * 64, 0.0)
+    arr = (C.c_void_p * 1)(w.handle)
+    ws = ctx.raw_buffer(1 << 20)
+    st = lib.jl_gemm(ctx.handle, arr, 1, x.ptr, o.ptr, 4, 4, 64, 0, L.JL_STORE, L.JL_MATH_INT8, ws.ptr, ws.nbytes)
+    assert st == L.JL_ERR_UNSUPPORTED and b"Q4_K" in lib.jl_last_error()
+    st = lib.jl_gemm(ctx.handle, arr, 1, x.ptr, o.ptr, 4, 4, 64, 0, L.JL_STORE, L.JL_MATH_F16, ws.ptr, 16)
+    assert st == L.JL_ERR_WORKSPACE
+    st = lib.jl_gemm(ctx.handle, arr, 1, x.ptr, o.ptr, 4, 5, 64, 0, L.JL_STORE, L.JL_MATH_F16, ws.ptr, ws.nbytes)
+    assert st == L.JL_ERR_INVALID
+    st = lib.jl_gemm(ctx.handle, arr, 1, x.ptr, o.ptr, 4, 4, 32, 0, L.JL_STORE, L.JL_MATH_F16, ws.ptr, ws.nbytes)
+    assert st == L.JL_ERR_INVALID and b"ldo" in lib.jl_last_error()

@@ -1,0 +1,223 @@
+"""GPU parity: element decode (bit-exact) and the decode GEMV family, through the C ABI."""
+import numpy as np
+import pytest
+
+import fixtures as FX
+from gpu_util import bits_equal, magnitude, reference_tolerance_ok, rel_err, say
+from oracle import pyoracle as O
+
+pytestmark = pytest.mark.gpu
+
+TYPES = [O.Q8_0, O.Q4_0, O.Q4_K]
+NAMES = {O.Q8_0: "q8_0", O.Q4_0: "q4_0", O.Q4_K: "q4_K"}
+POISON = np.float32(-999999.0)
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from jitllm_amd.runtime import Context
+    c = Context(0)
+    yield c
+    c.close()
+
+
+def upload(ctx, t, raw, d, n):
+    return ctx.load_weight(t, raw, d, n)
+
+
+# ---- element decode: bit-exact --------------------------------------------------------------
+
+@pytest.mark.parametrize("t,seed,blocks", [(O.Q4_0, 20260908, 16), (O.Q4_K, 20260904, 8),
+                                            (O.Q8_0, 20260908, 16)])
+def test_decode_random_bytes_bit_exact(ctx, t, seed, blocks):
+    """Q4_0DecodeTest / Q4_KDecodeTest inputs: arbitrary bytes, NaN and Inf scales included."""
+    say("decode random", NAMES[t])
+    raw = FX.random_bytes(seed, blocks * O.block_bytes(t))
+    n = O.block_elems(t)
+    w = upload(ctx, t, raw, blocks, n)
+    assert bits_equal(w.dequantize(), O.dequant(t, raw))
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_decode_adversarial_blocks_bit_exact(ctx, t):
+    """QuantizedDeviceDecodeParityTest.java:98-121: zero, subnormal, unit and extreme scales."""
+    say("decode adversarial", NAMES[t])
+    raw = FX.adversarial_blocks(t, 24, 20260908 + O.java_string_hash(FX.TYPE_NAMES[t]))
+    w = upload(ctx, t, raw, 24, O.block_elems(t))
+    assert bits_equal(w.dequantize(), O.dequant(t, raw))
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_decode_synthetic_weight_bit_exact(ctx, t):
+    from jitllm_amd import synthetic
+    say("decode synthetic", NAMES[t])
+    d, n = 96, 2048
+    raw = synthetic.weight(t, d, n, seed=101)
+    w = upload(ctx, t, raw, d, n)
+    assert bits_equal(w.dequantize(), O.dequant(t, raw))
+
+
+def test_q4_0_spec_known_answers_on_device(ctx):
+    """Q4_0DecodeTest.java:95-126."""
+    raw = np.zeros(18, dtype=np.uint8)
+    raw[0], raw[1], raw[2], raw[3] = 0x00, 0x40, 0x0F, 0x80
+    say("decode q4_0 known answers")
+    out = upload(ctx, O.Q4_0, raw, 1, 32).dequantize().reshape(-1)
+    assert (out[0], out[16], out[1], out[17]) == (14.0, -16.0, -16.0, 0.0)
+
+
+# ---- GEMV: the reference's own kernel test ----------------------------------------------------
+
+@pytest.mark.parametrize("t", TYPES)
+def test_matvec_reference_probe(ctx, t):
+    """NativeQuantizedKernelAccelTest.java:106-172: N = 512, D = 37, every row written, each within
+    max(1e-3, 1e-4 |expected|) of the host's sequential sum."""
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("matvec probe", NAMES[t])
+    raw = FX.probe_blocks(t, FX.probe_seed(NAMES[t]))
+    x = FX.probe_x()
+    expected = O.matmul(t, raw, x, FX.D_PROBE, FX.N_PROBE, O.DOT_SCALAR)
+    w = upload(ctx, t, raw, FX.D_PROBE, FX.N_PROBE)
+    xd = ctx.from_numpy(x)
+    out = ctx.float_array(FX.D_PROBE, fill=POISON)
+    proj = QuantizedProjections(ctx, TornadoWorkspace(wrapXb=xd))
+    proj.matvec(out, w, FX.N_PROBE, FX.D_PROBE)
+    ctx.sync()
+    got = out.get()
+    assert np.all(got != POISON)
+    assert np.all(reference_tolerance_ok(got, expected)), np.abs(got - expected).max()
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_residual_matvec_reference_probe(ctx, t):
+    """matrixVectorGenericWithResidual*: wrapX += w . x."""
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("residual probe", NAMES[t])
+    raw = FX.probe_blocks(t, FX.probe_seed(NAMES[t]))
+    x = FX.probe_x()
+    expected = O.matmul(t, raw, x, FX.D_PROBE, FX.N_PROBE, O.DOT_SCALAR)
+    base = np.linspace(-3, 3, FX.D_PROBE).astype(np.float32)
+    w = upload(ctx, t, raw, FX.D_PROBE, FX.N_PROBE)
+    wrap_x = ctx.from_numpy(base)
+    proj = QuantizedProjections(ctx, TornadoWorkspace(wrapX=wrap_x))
+    proj.residualMatvec(ctx.from_numpy(x), w, FX.N_PROBE, FX.D_PROBE)
+    ctx.sync()
+    assert np.all(reference_tolerance_ok(wrap_x.get(), base + expected))
+
+
+# ---- GEMV at the benchmark's shapes -----------------------------------------------------------
+
+SHAPES = [
+    (O.Q8_0, 2048, 2048), (O.Q8_0, 512, 2048), (O.Q8_0, 8192, 2048), (O.Q8_0, 2048, 8192),
+    (O.Q8_0, 1001, 2048),                      # ragged: rows not a multiple of the tile
+    (O.Q4_0, 4096, 4096), (O.Q4_0, 1024, 4096), (O.Q4_0, 2048, 14336), (O.Q4_0, 1792, 4096),
+    (O.Q4_K, 4096, 4096), (O.Q4_K, 1024, 4096), (O.Q4_K, 1536, 12288), (O.Q4_K, 3072, 4096),
+    (O.Q8_0, 300, 3072), (O.Q4_0, 300, 5120), (O.Q4_K, 130, 1536),   # S not a power of two
+    (O.Q8_0, 77, 96), (O.Q4_0, 5, 32), (O.Q4_K, 9, 256), (O.Q8_0, 3, 32768),  # catch-all kernel
+]
+
+
+@pytest.mark.parametrize("t,d,n", SHAPES)
+def test_gemv_matches_oracle(ctx, t, d, n):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("gemv", NAMES[t], d, n)
+    raw = synthetic.weight(t, d, n, seed=1000 + d + n)
+    x = synthetic.activations(n, seed=2000 + n)
+    flavour = O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256
+    ref = O.matmul(t, raw, x, d, n, flavour)
+    w = upload(ctx, t, raw, d, n)
+    out = ctx.float_array(d, fill=POISON)
+    QuantizedProjections(ctx, TornadoWorkspace()).floatMatvec(ctx.from_numpy(x), out, w, n, d)
+    ctx.sync()
+    got = out.get()
+    assert np.all(got != POISON)
+    err = rel_err(got, ref, magnitude(t, raw, x, d, n))
+    assert err < 1e-3, err
+    assert err < 2e-5, err  # fp32 arithmetic throughout: only the summation order differs
+
+
+@pytest.mark.parametrize("t,dq,dkv,n", [(O.Q8_0, 2048, 512, 2048), (O.Q4_0, 4096, 1024, 4096),
+                                         (O.Q4_K, 4096, 1024, 4096), (O.Q8_0, 100, 37, 512)])
+def test_fused_qkv(ctx, t, dq, dkv, n):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("qkv", NAMES[t], dq, dkv, n)
+    raws = [synthetic.weight(t, d, n, seed=31 + i) for i, d in enumerate((dq, dkv, dkv))]
+    x = synthetic.activations(n, seed=41)
+    ws = [upload(ctx, t, r, d, n) for r, d in zip(raws, (dq, dkv, dkv))]
+    outs = [ctx.float_array(d, fill=POISON) for d in (dq, dkv, dkv)]
+    QuantizedProjections(ctx, TornadoWorkspace()).fusedQKV(ctx.from_numpy(x), *outs, *ws)
+    ctx.sync()
+    for raw, d, out in zip(raws, (dq, dkv, dkv), outs):
+        ref = O.matmul(t, raw, x, d, n)
+        assert rel_err(out.get(), ref, magnitude(t, raw, x, d, n)) < 2e-5
+
+
+@pytest.mark.parametrize("t,d,n", [(O.Q8_0, 8192, 2048), (O.Q4_0, 14336, 4096),
+                                    (O.Q4_K, 12288, 4096), (O.Q4_K, 37, 512)])
+def test_fused_gate_up(ctx, t, d, n):
+    """hb = SiLU(w1 . x) * (w3 . x), held against the host's matVec, matVec, swiGLU sequence
+    (InferenceCore.java:127-129)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("gate_up", NAMES[t], d, n)
+    r1 = synthetic.weight(t, d, n, seed=51)
+    r3 = synthetic.weight(t, d, n, seed=52)
+    x = synthetic.activations(n, seed=53)
+    g = O.matmul(t, r1, x, d, n)
+    u = O.matmul(t, r3, x, d, n)
+    ref = O.swiglu(g, u)
+    hb = ctx.float_array(d, fill=POISON)
+    proj = QuantizedProjections(ctx, TornadoWorkspace(wrapXb=ctx.from_numpy(x), wrapHb=hb))
+    proj.gateUp(upload(ctx, t, r1, d, n), upload(ctx, t, r3, d, n), n, d)
+    ctx.sync()
+    got = hb.get()
+    # error of a product: relative errors of gate and up add; scale by the magnitudes of both
+    mg = magnitude(t, r1, x, d, n)
+    mu = magnitude(t, r3, x, d, n)
+    bound = 2e-5 * (mg * np.abs(u) + mu * np.abs(g) * 1.2 + 1e-6)
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + 1e-6)
+
+
+def test_mixed_gate_up_runs_two_projections_and_swiglu(ctx):
+    """QuantizedProjections.gateUp's unfused branch: gate and up of different types."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("gate_up mixed")
+    d, n = 512, 1024
+    r1 = synthetic.weight(O.Q4_K, d, n, seed=61)
+    r3 = synthetic.weight(O.Q8_0, d, n, seed=62)
+    x = synthetic.activations(n, seed=63)
+    ref = O.swiglu(O.matmul(O.Q4_K, r1, x, d, n), O.matmul(O.Q8_0, r3, x, d, n))
+    ws = TornadoWorkspace(wrapXb=ctx.from_numpy(x), wrapHb=ctx.float_array(d),
+                          wrapHb2=ctx.float_array(d))
+    proj = QuantizedProjections(ctx, ws)
+    w1, w3 = upload(ctx, O.Q4_K, r1, d, n), upload(ctx, O.Q8_0, r3, d, n)
+    assert not proj.fusedGateUp(w1, w3)
+    proj.gateUp(w1, w3, n, d)
+    ctx.sync()
+    assert np.allclose(ws.wrapHb.get(), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_errors_name_the_cause(ctx):
+    """No silent fallback: unsupported combinations and bad shapes raise."""
+    import ctypes as C
+    from jitllm_amd import _lib as L, synthetic
+    say("errors")
+    lib = L.load()
+    h = C.c_void_p()
+    raw = np.zeros(64, dtype=np.uint8)
+    st = lib.jl_weight_upload(ctx.handle, 14, raw.ctypes.data, 1, 32, C.byref(h))  # Q6_K: no kernel
+    assert st == L.JL_ERR_UNSUPPORTED and b"ggml type 14" in lib.jl_last_error()
+    st = lib.jl_weight_upload(ctx.handle, O.Q8_0, raw.ctypes.data, 1, 48, C.byref(h))
+    assert st == L.JL_ERR_INVALID and b"whole number" in lib.jl_last_error()
+    w8 = upload(ctx, O.Q8_0, synthetic.weight(O.Q8_0, 64, 256, 1), 64, 256)
+    w4 = upload(ctx, O.Q4_K, synthetic.weight(O.Q4_K, 64, 256, 2), 64, 256)
+    x, o = ctx.float_array(256, 0.0), ctx.float_array(64, 0.0)
+    st = lib.jl_gemv_gate_up(ctx.handle, w8.handle, w4.handle, x.ptr, o.ptr)
+    assert st == L.JL_ERR_UNSUPPORTED and b"no fused gate/up kernel" in lib.jl_last_error()
+    with pytest.raises(L.UnsupportedProjection):
+        L.check(lib.jl_gemv_qkv(ctx.handle, w8.handle, w4.handle, w8.handle, x.ptr, o.ptr, o.ptr, o.ptr))
+    assert lib.jl_gemv(ctx.handle, w8.handle, x.ptr, o.ptr, L.JL_SWIGLU) == L.JL_ERR_INVALID
+    assert lib.jl_gemv(ctx.handle, None, x.ptr, o.ptr, L.JL_STORE) == L.JL_ERR_INVALID
