@@ -1,0 +1,336 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized weight-matmul hot path on one MI355X.
+
+A step is one pass of the decode projection set of Llama-3.2-1B in Q8_0, batch 1 -- per layer the
+fused q|k|v projection, the output projection (residual), the fused gate/up SwiGLU projection and
+the down projection (residual), 16 layers, then the 2048 -> 128256 vocabulary projection: 65 kernel
+launches, 1 316 320 256 algorithmic bytes (weights in GGUF block layout + fp32 input + fp32 output,
+each once).  Inputs are resident in HBM before the timed region.  Every layer owns distinct device
+buffers, so the 1.3 GB sweep cannot live in the 256 MB memory-side cache.
+
+Prints one JSON line.  `value` is GB/s of algorithmic bytes; `roofline` is the dominant kernel
+(the fused gate/up GEMV) against the 8 TB/s HBM peak; `cpu_baseline` is the oracle's restatement of
+the reference's Java CPU matmul timed on this machine's host cores; `prefill` and `batched` carry
+the MFMA side of the metric.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+F16_MFMA_PEAK_TFLOPS = 2500.0
+INT8_MFMA_PEAK_TOPS = 5000.0
+
+# Llama-3.2-1B geometry (BASELINE.json configs[1])
+DIM, KV_DIM, HIDDEN, VOCAB, LAYERS = 2048, 512, 8192, 128256, 16
+
+
+class Hip:
+    """The few HIP runtime calls the benchmark needs for timing: events on the context's stream."""
+
+    def __init__(self):
+        self.lib = C.CDLL("libamdhip64.so")
+        self.lib.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.lib.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.lib.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.lib.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.lib.hipEventDestroy.argtypes = [C.c_void_p]
+
+    def event(self):
+        e = C.c_void_p()
+        assert self.lib.hipEventCreate(C.byref(e)) == 0
+        return e
+
+    def record(self, e, stream):
+        assert self.lib.hipEventRecord(e, stream) == 0
+
+    def elapsed_ms(self, a, b) -> float:
+        assert self.lib.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.lib.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return float(ms.value)
+
+
+def q8_bytes(rows, cols):
+    return rows * (cols // 32) * 34
+
+
+def gemv_bytes(rows, cols, block_bytes=34, block_elems=32, weights=1, outs=None):
+    """Algorithmic bytes of one launch: weights + fp32 input + fp32 output."""
+    outs = rows * weights if outs is None else outs
+    return weights * rows * (cols // block_elems) * block_bytes + 4 * cols + 4 * outs
+
+
+def build_decode_set(ctx, t):
+    """Device-resident weights and activation arrays of the projection set."""
+    from jitllm_amd import synthetic
+    host = {
+        "wq": synthetic.weight(t, DIM, DIM, 11), "wk": synthetic.weight(t, KV_DIM, DIM, 12),
+        "wv": synthetic.weight(t, KV_DIM, DIM, 13), "wo": synthetic.weight(t, DIM, DIM, 14),
+        "w1": synthetic.weight(t, HIDDEN, DIM, 15), "w3": synthetic.weight(t, HIDDEN, DIM, 16),
+        "w2": synthetic.weight(t, DIM, HIDDEN, 17),
+    }
+    shapes = {"wq": (DIM, DIM), "wk": (KV_DIM, DIM), "wv": (KV_DIM, DIM), "wo": (DIM, DIM),
+              "w1": (HIDDEN, DIM), "w3": (HIDDEN, DIM), "w2": (DIM, HIDDEN)}
+    layers = []
+    for _ in range(LAYERS):  # the same host bytes, but a device buffer of its own per layer
+        layers.append({k: ctx.load_weight(t, host[k], *shapes[k]) for k in host})
+    wcls_host = synthetic.weight(t, VOCAB, DIM, 18)
+    wcls = ctx.load_weight(t, wcls_host, VOCAB, DIM)
+    host["wcls"] = wcls_host
+    shapes["wcls"] = (VOCAB, DIM)
+    acts = {
+        "x": ctx.from_numpy(synthetic.activations(DIM, 21)),
+        "xb": ctx.from_numpy(synthetic.activations(DIM, 22)),
+        "q": ctx.float_array(DIM), "k": ctx.float_array(KV_DIM), "v": ctx.float_array(KV_DIM),
+        "hb": ctx.float_array(HIDDEN), "logits": ctx.float_array(VOCAB),
+    }
+    return layers, wcls, acts, host, shapes
+
+
+def decode_step(proj, layers, wcls, acts, hooks=None):
+    """One token's projections in the reference's decode order (LlamaQ8_0FFNLayers.java:212-525)."""
+    for i, w in enumerate(layers):
+        proj.fusedQKV(acts["xb"], acts["q"], acts["k"], acts["v"], w["wq"], w["wk"], w["wv"])
+        proj.residualMatvec(acts["xb"], w["wo"], DIM, DIM)
+        if hooks:
+            hooks[0](i)
+        proj.gateUp(w["w1"], w["w3"], DIM, HIDDEN)
+        if hooks:
+            hooks[1](i)
+        proj.residualMatvec(acts["hb"], w["w2"], HIDDEN, DIM)
+    proj.floatMatvec(acts["xb"], acts["logits"], wcls, DIM, VOCAB)
+
+
+def decode_bytes():
+    """Algorithmic bytes of a step: every one of the 7 projections of a layer counted on its own
+    (weight blocks + fp32 input + fp32 output), as the benchmark's definition does, even where one
+    launch serves several of them."""
+    per_layer = (gemv_bytes(DIM, DIM) + 2 * gemv_bytes(KV_DIM, DIM) + gemv_bytes(DIM, DIM)
+                 + 2 * gemv_bytes(HIDDEN, DIM) + gemv_bytes(DIM, HIDDEN))
+    return LAYERS * per_layer + gemv_bytes(VOCAB, DIM)
+
+
+def cpu_baseline(host, shapes, t, reps=3):
+    """The oracle (a C restatement of FloatTensor.matmul with the 256-bit vectorDot lane order,
+    rows spread over the host cores) on one layer's seven projections plus the vocabulary
+    projection -- 344 MB of the 1 316 MB set."""
+    from jitllm_amd import synthetic
+    from oracle import pyoracle as O
+    threads = O.max_threads()
+    x_dim = synthetic.activations(DIM, 31)
+    x_hid = synthetic.activations(HIDDEN, 32)
+    names = ["wq", "wk", "wv", "wo", "w1", "w3", "w2", "wcls"]
+    nbytes = sum(gemv_bytes(*shapes[k]) for k in names)
+    times = []
+    for _ in range(reps + 1):
+        t0 = time.perf_counter()
+        for k in names:
+            rows, cols = shapes[k]
+            O.matmul(int(t), host[k], x_hid if cols == HIDDEN else x_dim, rows, cols,
+                     O.DOT_VEC256, threads)
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times[1:])
+    return {"value": round(nbytes / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"one layer's 7 projections + vocabulary projection ({nbytes} B), "
+                      f"median of {reps} passes after 1 warm-up, 256-bit vectorDot order",
+            "tok_s_equiv": round(nbytes / med / decode_bytes(), 3)}
+
+
+def bench_gemm(ctx, hip, t, T, steps, warmup):
+    """Batched prefill of one Llama-3.2-1B layer (q|k|v, o, gate/up SwiGLU, down) over T tokens."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    w = {
+        "wq": ctx.load_weight(t, synthetic.weight(t, DIM, DIM, 41), DIM, DIM),
+        "wk": ctx.load_weight(t, synthetic.weight(t, KV_DIM, DIM, 42), KV_DIM, DIM),
+        "wv": ctx.load_weight(t, synthetic.weight(t, KV_DIM, DIM, 43), KV_DIM, DIM),
+        "wo": ctx.load_weight(t, synthetic.weight(t, DIM, DIM, 44), DIM, DIM),
+        "w1": ctx.load_weight(t, synthetic.weight(t, HIDDEN, DIM, 45), HIDDEN, DIM),
+        "w3": ctx.load_weight(t, synthetic.weight(t, HIDDEN, DIM, 46), HIDDEN, DIM),
+        "w2": ctx.load_weight(t, synthetic.weight(t, DIM, HIDDEN, 47), DIM, HIDDEN),
+    }
+    X = ctx.from_numpy(synthetic.activations((T, DIM), 48))
+    H = ctx.from_numpy(synthetic.activations((T, HIDDEN), 49) * np.float32(0.1))
+    qkv = ctx.float_array(T * (DIM + 2 * KV_DIM))
+    res = ctx.float_array(T * DIM, fill=0.0)
+    hb = ctx.float_array(T * HIDDEN)
+    proj = QuantizedBatchProjections(ctx, T, HIDDEN)
+
+    def layer():
+        proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
+        proj.projection(X, res, w["wo"], DIM, DIM, True)
+        proj.gateUp(X, hb, w["w1"], w["w3"], DIM, HIDDEN)
+        proj.projection(H, res, w["w2"], HIDDEN, DIM, True)
+
+    for _ in range(warmup):
+        layer()
+    ctx.sync()
+    e0, e1 = hip.event(), hip.event()
+    hip.record(e0, ctx.stream)
+    for _ in range(steps):
+        layer()
+    hip.record(e1, ctx.stream)
+    ms = hip.elapsed_ms(e0, e1) / steps
+    flops = 2.0 * T * (DIM * (DIM + 2 * KV_DIM) + DIM * DIM + 2 * DIM * HIDDEN + HIDDEN * DIM)
+    tflops = flops / (ms * 1e-3) / 1e12
+    return {"tokens": T, "ms_per_layer": round(ms, 4), "tok_s_16_layers": round(T / (ms * 1e-3 * LAYERS), 1),
+            "tflops": round(tflops, 1), "frac_f16_mfma_peak": round(tflops / F16_MFMA_PEAK_TFLOPS, 4),
+            "math": "f16 MFMA after in-LDS dequant"}
+
+
+def bench_batched_q4k(ctx, hip, B, steps, warmup):
+    """Q4_K batched decode, Qwen3-8B-like shapes (dim 4096, ffn 12288, kv 1024), B sequences."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.projections import QuantizedBatchProjections
+    t = GGMLType.Q4_K
+    dim, kv, ffn = 4096, 1024, 12288
+    w = {
+        "wq": ctx.load_weight(t, synthetic.weight(t, dim, dim, 61), dim, dim),
+        "wk": ctx.load_weight(t, synthetic.weight(t, kv, dim, 62), kv, dim),
+        "wv": ctx.load_weight(t, synthetic.weight(t, kv, dim, 63), kv, dim),
+        "wo": ctx.load_weight(t, synthetic.weight(t, dim, dim, 64), dim, dim),
+        "w1": ctx.load_weight(t, synthetic.weight(t, ffn, dim, 65), ffn, dim),
+        "w3": ctx.load_weight(t, synthetic.weight(t, ffn, dim, 66), ffn, dim),
+        "w2": ctx.load_weight(t, synthetic.weight(t, dim, ffn, 67), dim, ffn),
+    }
+    X = ctx.from_numpy(synthetic.activations((B, dim), 68))
+    H = ctx.from_numpy(synthetic.activations((B, ffn), 69) * np.float32(0.1))
+    qkv = ctx.float_array(B * (dim + 2 * kv))
+    res = ctx.float_array(B * dim, fill=0.0)
+    hb = ctx.float_array(B * ffn)
+    proj = QuantizedBatchProjections(ctx, B, ffn)
+
+    def layer():
+        proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
+        proj.projection(X, res, w["wo"], dim, dim, True)
+        proj.gateUp(X, hb, w["w1"], w["w3"], dim, ffn)
+        proj.projection(H, res, w["w2"], ffn, dim, True)
+
+    for _ in range(warmup):
+        layer()
+    ctx.sync()
+    e0, e1 = hip.event(), hip.event()
+    hip.record(e0, ctx.stream)
+    for _ in range(steps):
+        layer()
+    hip.record(e1, ctx.stream)
+    ms = hip.elapsed_ms(e0, e1) / steps
+    wbytes = sum(x.nbytes for x in w.values())
+    # fp32 activations in and out, once per projection
+    io = 4 * B * (dim + dim + 2 * kv + dim + dim + dim + ffn + ffn + dim)
+    flops = 2.0 * B * (dim * (dim + 2 * kv) + dim * dim + 2 * dim * ffn + ffn * dim)
+    gbs = (wbytes + io) / (ms * 1e-3) / 1e9
+    return {"B": B, "ms_per_layer": round(ms, 4), "GB_s": round(gbs, 1),
+            "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+            "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "bytes": wbytes + io}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the prefill / batched legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path is built and measured on a single MI355X; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    from jitllm_amd.runtime import Context
+
+    t = GGMLType.Q8_0
+    hip = Hip()
+    with Context(0) as ctx:
+        cu, name = ctx.device_info()
+        layers, wcls, acts, host, shapes = build_decode_set(ctx, t)
+        ws = TornadoWorkspace(wrapX=acts["x"], wrapXb=acts["xb"], wrapHb=acts["hb"])
+        proj = QuantizedProjections(ctx, ws)
+        total_bytes = decode_bytes()
+        assert total_bytes == 1316320256, total_bytes
+
+        for _ in range(args.warmup):
+            decode_step(proj, layers, wcls, acts)
+        ctx.sync()
+
+        # timed region: K steps, with an event pair around every launch of the dominant kernel
+        stream = ctx.stream
+        e0, e1 = hip.event(), hip.event()
+        pairs = [[(hip.event(), hip.event()) for _ in range(LAYERS)] for _ in range(args.steps)]
+        t0 = time.perf_counter()
+        hip.record(e0, stream)
+        for s in range(args.steps):
+            decode_step(proj, layers, wcls, acts,
+                        hooks=(lambda i, s=s: hip.record(pairs[s][i][0], stream),
+                               lambda i, s=s: hip.record(pairs[s][i][1], stream)))
+        hip.record(e1, stream)
+        ctx.sync()
+        wall = time.perf_counter() - t0
+        ms_step = hip.elapsed_ms(e0, e1) / args.steps
+        gate_up_ms = [hip.elapsed_ms(a, b) for step in pairs for (a, b) in step]
+        gate_up_avg = sum(gate_up_ms) / len(gate_up_ms)
+        gate_up_bytes = 2 * gemv_bytes(HIDDEN, DIM)
+
+        # the same K steps without the per-launch events, to show what they cost
+        hip.record(e0, stream)
+        for _ in range(args.steps):
+            decode_step(proj, layers, wcls, acts)
+        hip.record(e1, stream)
+        ms_step_clean = hip.elapsed_ms(e0, e1) / args.steps
+
+        ms = min(ms_step, ms_step_clean)
+        gbs = total_bytes / (ms * 1e-3) / 1e9
+        achieved = gate_up_bytes / (gate_up_avg * 1e-3) / 1e9
+        out = {
+            "metric": "Q-GEMV HBM GB/s (% of peak) + prefill tok/s (% MFMA peak), 1xMI355X",
+            "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "data": "synthetic (seeded Q8_0 blocks; one layer's host bytes uploaded into 16 distinct "
+                    "device buffers)",
+            "config": {"workload": "Q8_0 Llama-3.2-1B decode projection set, batch 1: 16 x (q|k|v, o, "
+                                   "gate/up SwiGLU, down) + vocabulary projection, 65 launches/token",
+                       "bytes_per_step": total_bytes, "device": name, "compute_units": cu},
+            "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+            "tok_s": round(1e3 / ms, 1),
+            "ms_per_step_with_events": round(ms_step, 4),
+            "ms_per_step_clean": round(ms_step_clean, 4),
+            "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
+            "roofline": {"bound": "hbm", "kernel": "jl_gemv_tiles<Q8_0, gate/up> 2 x [8192 x 2048]",
+                         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                         "bytes_per_launch": gate_up_bytes,
+                         "avg_launch_us": round(gate_up_avg * 1e3, 3),
+                         "launches_timed": len(gate_up_ms)},
+        }
+        if not args.no_extra:
+            out["prefill"] = [bench_gemm(ctx, hip, t, T, max(3, args.steps // 10), 2)
+                              for T in (512, 2048)]
+            out["batched_q4k"] = [bench_batched_q4k(ctx, hip, B, max(5, args.steps // 5), 3)
+                                  for B in (8, 32, 64)]
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_baseline(host, shapes, t)
+        else:
+            out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -27,8 +27,8 @@ constexpr int kMaxWeights = 8;
 
 // ---- activations: fp32 -> fp16 with a power-of-two row scale --------------------------------
 
-// One wave per row.  scale = 1 unless the row's largest magnitude exceeds 2^15, then the power of
-// two that brings it to at most 2^15; a16 = half(x / scale) (the division is exact).
+// One wave per row: scale = the power of two that brings the row's largest magnitude into
+// [2^11, 2^12); a16 = half(x / scale) (the division is exact).
 __global__ void __launch_bounds__(256)
 jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__restrict__ row_scale,
                int rows, int padded_rows, int k) {
@@ -49,12 +49,16 @@ jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__r
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, JL_WAVE));
+    // Every row is brought to [2^11, 2^12) at its largest magnitude: huge rows stay finite in
+    // fp16, tiny rows keep their bits out of fp16's subnormal range, and the power of two is
+    // undone exactly in the epilogue.
     float scale = 1.f, inv = 1.f;
-    if (amax > 32768.f && amax < INFINITY) {
+    if (amax > 0.f && amax < INFINITY) {
         int e;
         frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
-        scale = ldexpf(1.f, e - 15);
-        inv = ldexpf(1.f, 15 - e);
+        e = e < -100 ? -100 : e;
+        scale = ldexpf(1.f, e - 12);
+        inv = ldexpf(1.f, 12 - e);
     }
     for (int i = lane * 4; i < k; i += JL_WAVE * 4) {
         float4 v = *(const float4 *)(x + i);

@@ -147,7 +147,8 @@ def test_huge_activation_rows_stay_finite(ctx):
     ctx.sync()
     got = out.get().reshape(B, d)
     assert np.all(np.isfinite(got))
-    assert rel_err(got, ref, magnitude(O.Q8_0, raw, X, d, n)) < F16_BOUND
+    err = rel_err(got, ref, magnitude(O.Q8_0, raw, X, d, n))
+    assert err < 2e-4, err
 
 
 def test_batched_errors(ctx):
