@@ -49,20 +49,16 @@ struct GemvParams {
 };
 
 template <int TYPE> struct Traits;
-template <> struct Traits<JL_Q8_0> { static constexpr int kLoads = 5; };
-template <> struct Traits<JL_Q4_0> { static constexpr int kLoads = 3; };
-template <> struct Traits<JL_Q4_K> { static constexpr int kLoads = 3; };
+template <> struct Traits<JL_Q8_0> { static constexpr int kX4 = 4; };  // 68 B = 4 x 16 + 4
+template <> struct Traits<JL_Q4_0> { static constexpr int kX4 = 2; };  // 36 B = 2 x 16 + 4
+template <> struct Traits<JL_Q4_K> { static constexpr int kX4 = 2; };  // 144 B / 4 = 36 B
 
 __device__ __forceinline__ float ubyte(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
 __device__ __forceinline__ float sbyte(uint32_t v, int k) { return (float)(int)(int8_t)(v >> (8 * k)); }
 
 // Dot of one Q8_0 block pair (68 bytes, 4-byte aligned in LDS) with 64 activations.
 //   bytes 0..1 scale A | 2..33 quants A | 34..35 scale B | 36..67 quants B
-__device__ __forceinline__ float slice_dot_q8_0(const uint8_t *p, const float (&x)[64]) {
-    const uint32_t *dw = (const uint32_t *)p;
-    uint32_t w[17];
-#pragma unroll
-    for (int i = 0; i < 17; i++) w[i] = dw[i];
+__device__ __forceinline__ float slice_dot_q8_0(const uint32_t (&w)[17], const float (&x)[64]) {
     float dA = jl_half_bits_to_float(w[0]);
     float dB = jl_half_bits_to_float(w[8] >> 16);
     float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
@@ -86,9 +82,8 @@ __device__ __forceinline__ float slice_dot_q8_0(const uint8_t *p, const float (&
 // activations facing block A and block B, so that sum((q - 8) x) = sum(q x) - 8 sum(x).
 //   bytes 0..1 scale A | 2..17 nibbles A | 18..19 scale B | 20..35 nibbles B
 // element i < 16 of a block is the low nibble of its byte i, element 16 + i the high nibble.
-__device__ __forceinline__ float slice_dot_q4_0(const uint8_t *p, const float (&x)[64],
+__device__ __forceinline__ float slice_dot_q4_0(const uint32_t (&dw)[9], const float (&x)[64],
                                                 const float (&sx)[2]) {
-    const uint32_t *dw = (const uint32_t *)p;
     uint32_t lo[9], hi[9];
     uint32_t w0 = dw[0], w4 = dw[4];
 #pragma unroll
@@ -121,11 +116,9 @@ __device__ __forceinline__ float slice_dot_q4_0(const uint8_t *p, const float (&
 // 16 bytes (d, dmin, 12 packed scale bytes), `qs` the 32 nibble bytes of pair `pair`: low nibbles
 // are sub-block 2*pair (activations 0..31), high nibbles sub-block 2*pair+1 (activations 32..63).
 // sum(w x) = (d sc) sum(q x) - (dmin m) sum(x) per sub-block.
-__device__ __forceinline__ float slice_dot_q4_k(const uint8_t *hdr, const uint8_t *qs, int pair,
-                                                const float (&x)[64], const float (&sx)[2]) {
-    uint4 h = *(const uint4 *)hdr;
-    uint4 q0 = *(const uint4 *)qs;
-    uint4 q1 = *(const uint4 *)(qs + 16);
+__device__ __forceinline__ float slice_dot_q4_k(const uint4 &h, const uint4 &q0, const uint4 &q1,
+                                                int pair, const float (&x)[64],
+                                                const float (&sx)[2]) {
     uint32_t w[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
     float d = jl_half_bits_to_float(h.x);
     float dmin = jl_half_bits_to_float(h.x >> 16);
@@ -151,97 +144,201 @@ __device__ __forceinline__ float slice_dot_q4_k(const uint8_t *hdr, const uint8_
     return lo_term + hi_term;
 }
 
+// ---- LDS access by hand ----------------------------------------------------------------------
+//
+// The tile stages are filled by LDS-DMA loads (global_load_lds_*), which the compiler tracks only
+// coarsely: any LDS read it can see makes it wait for every outstanding vector-memory operation,
+// which would drain the prefetch pipeline each tile.  All LDS traffic of the kernel therefore goes
+// through inline assembly with explicit waits, and the workgroup barrier is the bare instruction.
+
+typedef __attribute__((address_space(1))) const void gvoid;
+typedef __attribute__((address_space(3))) void lvoid;
+
+// s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
+#define JL_WAIT_VM(N) \
+    __builtin_amdgcn_s_waitcnt(((N)&0xF) | (((N) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+__device__ __forceinline__ void wait_vm_tiles(int tiles, int per_tile) {
+    // per_tile is 3 or 5, tiles 0..2: every case is an immediate
+    int n = tiles * per_tile;
+    if (n >= 10) JL_WAIT_VM(10);
+    else if (n == 6) JL_WAIT_VM(6);
+    else if (n == 5) JL_WAIT_VM(5);
+    else if (n == 3) JL_WAIT_VM(3);
+    else JL_WAIT_VM(0);
+}
+
+__device__ __forceinline__ uint32_t lds_read_b32(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+    return v;
+}
+
+__device__ __forceinline__ void lds_write_b32(uint32_t addr, uint32_t v) {
+    asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(addr), "v"(v) : "memory");
+}
+
+__device__ __forceinline__ void lds_read_x4(uint32_t addr, uint32_t (&w)[4]) {
+    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&v"(*(uint4 *)w) : "v"(addr) : "memory");
+}
+
+// 16 activations' worth of registers (four 128-bit reads) with one wait
+__device__ __forceinline__ void lds_read_16f(uint32_t addr, float *x) {
+    float4 a, b, c, d;
+    asm volatile(
+        "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:16\n\t"
+        "ds_read_b128 %2, %4 offset:32\n\tds_read_b128 %3, %4 offset:48\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(d) : "v"(addr) : "memory");
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
+    x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+    x[8] = c.x; x[9] = c.y; x[10] = c.z; x[11] = c.w;
+    x[12] = d.x; x[13] = d.y; x[14] = d.z; x[15] = d.w;
+}
+
+// 17 consecutive dwords (one Q8_0 block pair)
+__device__ __forceinline__ void lds_read_17(uint32_t addr, uint32_t (&w)[17]) {
+    asm volatile(
+        "ds_read_b32 %0, %17\n\tds_read_b32 %1, %17 offset:4\n\tds_read_b32 %2, %17 offset:8\n\t"
+        "ds_read_b32 %3, %17 offset:12\n\tds_read_b32 %4, %17 offset:16\n\tds_read_b32 %5, %17 offset:20\n\t"
+        "ds_read_b32 %6, %17 offset:24\n\tds_read_b32 %7, %17 offset:28\n\tds_read_b32 %8, %17 offset:32\n\t"
+        "ds_read_b32 %9, %17 offset:36\n\tds_read_b32 %10, %17 offset:40\n\tds_read_b32 %11, %17 offset:44\n\t"
+        "ds_read_b32 %12, %17 offset:48\n\tds_read_b32 %13, %17 offset:52\n\tds_read_b32 %14, %17 offset:56\n\t"
+        "ds_read_b32 %15, %17 offset:60\n\tds_read_b32 %16, %17 offset:64\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3]), "=&v"(w[4]), "=&v"(w[5]), "=&v"(w[6]),
+          "=&v"(w[7]), "=&v"(w[8]), "=&v"(w[9]), "=&v"(w[10]), "=&v"(w[11]), "=&v"(w[12]),
+          "=&v"(w[13]), "=&v"(w[14]), "=&v"(w[15]), "=&v"(w[16])
+        : "v"(addr) : "memory");
+}
+
+// 9 consecutive dwords (one Q4_0 block pair)
+__device__ __forceinline__ void lds_read_9(uint32_t addr, uint32_t (&w)[9]) {
+    asm volatile(
+        "ds_read_b32 %0, %9\n\tds_read_b32 %1, %9 offset:4\n\tds_read_b32 %2, %9 offset:8\n\t"
+        "ds_read_b32 %3, %9 offset:12\n\tds_read_b32 %4, %9 offset:16\n\tds_read_b32 %5, %9 offset:20\n\t"
+        "ds_read_b32 %6, %9 offset:24\n\tds_read_b32 %7, %9 offset:28\n\tds_read_b32 %8, %9 offset:32\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3]), "=&v"(w[4]), "=&v"(w[5]), "=&v"(w[6]),
+          "=&v"(w[7]), "=&v"(w[8])
+        : "v"(addr) : "memory");
+}
+
+// a Q4_K super-block header (16 B) and the 32 nibble bytes of one pair
+__device__ __forceinline__ void lds_read_q4k(uint32_t hdr, uint32_t qs, uint4 &h, uint4 &q0, uint4 &q1) {
+    asm volatile(
+        "ds_read_b128 %0, %3\n\tds_read_b128 %1, %4\n\tds_read_b128 %2, %4 offset:16\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(h), "=&v"(q0), "=&v"(q1) : "v"(hdr), "v"(qs) : "memory");
+}
+
 template <int TYPE>
-__device__ __forceinline__ float slice_dot(const uint8_t *tile, int r, int s, int row_bytes,
-                                           const float (&x)[64], const float (&sx)[2]) {
-    const uint8_t *row = tile + r * row_bytes;
+__device__ __forceinline__ float slice_dot_lds(uint32_t stage, int r, int s, int row_bytes,
+                                               const float (&x)[64], const float (&sx)[2]) {
+    const uint32_t row = stage + (uint32_t)(r * row_bytes);
     if constexpr (TYPE == JL_Q8_0) {
-        return slice_dot_q8_0(row + s * 68, x);
+        uint32_t w[17];
+        lds_read_17(row + s * 68, w);
+        return slice_dot_q8_0(w, x);
     } else if constexpr (TYPE == JL_Q4_0) {
-        return slice_dot_q4_0(row + s * 36, x, sx);
+        uint32_t w[9];
+        lds_read_9(row + s * 36, w);
+        return slice_dot_q4_0(w, x, sx);
     } else {
-        const uint8_t *sb = row + (s >> 2) * 144;
-        return slice_dot_q4_k(sb, sb + 16 + (s & 3) * 32, s & 3, x, sx);
+        uint4 h, q0, q1;
+        uint32_t sb = row + (s >> 2) * 144;
+        lds_read_q4k(sb, sb + 16 + (s & 3) * 32, h, q0, q1);
+        return slice_dot_q4_k(h, q0, q1, s & 3, x, sx);
     }
 }
 
-// LDS map: [0, 256) cross-wave partial sums (2 parities x 2 results x up to 8 waves... 32 floats
-// used), then a region that first holds the activation vector and afterwards the tile stages.
-constexpr int kPartialBytes = 256;
+// LDS map: [0, kPartialBytes) row partial sums, two parities; then the stage ring.  The activation
+// vector is staged in the ring's last stage (or, when it is larger than a stage, in a region of
+// its own after the ring) until every thread holds its 64 activations in registers.
+constexpr int kPartialBytes = 4096;  // 2 parities x 512 floats
+constexpr int kStages = 3;
 
 template <int TYPE, bool DUAL>
 __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr int NL = Traits<TYPE>::kLoads;
-    constexpr int NW = DUAL ? 2 : 1;
+    constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
+    constexpr int L = X4 + 1;                     // plus one 4-byte load
+    constexpr int SLICE = X4 * 16 + 4;            // bytes of a tile one thread brings in
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
-    const int r = tid / p.Sp;
-    const int s = tid - r * p.Sp;
+    const int wave = tid / JL_WAVE;
+    const int lane = tid & (JL_WAVE - 1);
+    const int r = tid / p.Sp;           // row of the tile this thread works on
+    const int s = tid - r * p.Sp;       // its 64-column slice
     const bool active = (s < p.S) && (r < p.R);
-    const int tile_bytes = p.R * p.row_bytes;  // a multiple of 16 (checked on the host)
+    const int half_rows = DUAL ? p.R / 2 : p.R;       // output rows per tile
+    const int half_bytes = half_rows * p.row_bytes;   // bytes of a tile that come from one weight
     const int total_tiles = p.seg_tile_begin[p.nseg];
+    const int stage_bytes = nthreads * SLICE;
 
-    float *partial = (float *)lds;
-    uint8_t *region = lds + kPartialBytes;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
+    const uint32_t ring0 = lds0 + kPartialBytes;
+    uint8_t *ring = lds + kPartialBytes;
 
-    uint4 stg[NW][NL];
-
-    // Start the first tile's loads before anything else so they overlap the activation set-up.
-    auto issue = [&](int tile) {
+    // Brings tile `tile` into stage `st`.  Every thread issues exactly L loads, whatever the tile:
+    // lanes that have nothing to fetch re-read the segment's first bytes into their own slot, so
+    // each wave's outstanding-load count is a compile-time constant per tile.
+    auto issue = [&](int tile, int st) {
         int seg = 0;
 #pragma unroll
         for (int i = 1; i < kMaxSeg; i++)
             if (i < p.nseg && tile >= p.seg_tile_begin[i]) seg = i;
-        int local = tile - p.seg_tile_begin[seg];
-        int64_t offset = (int64_t)local * tile_bytes;
-        int64_t remain = (int64_t)p.seg_rows[seg] * p.row_bytes - offset;
-        int bytes = remain < tile_bytes ? (int)remain : tile_bytes;
+        const int local = tile - p.seg_tile_begin[seg];
+        const int64_t offset = (int64_t)local * half_bytes;
+        const int64_t remain = (int64_t)p.seg_rows[seg] * p.row_bytes - offset;
+        const int bytes = remain < half_bytes ? (int)remain : half_bytes;
         const uint8_t *base = p.w[seg] + offset;
-#pragma unroll
-        for (int k = 0; k < NL; k++) {
-            int off = (k * nthreads + tid) * 16;
-            stg[0][k] = off < bytes ? *(const uint4 *)(base + off) : make_uint4(0, 0, 0, 0);
-        }
-        if constexpr (DUAL) {
-            const uint8_t *base_up = p.w_up + offset;
-#pragma unroll
-            for (int k = 0; k < NL; k++) {
-                int off = (k * nthreads + tid) * 16;
-                stg[1][k] = off < bytes ? *(const uint4 *)(base_up + off) : make_uint4(0, 0, 0, 0);
+        const uint8_t *base_up = DUAL ? p.w_up + offset : nullptr;
+        uint8_t *dst = ring + st * stage_bytes;
+        auto source = [&](int off, int width) -> const uint8_t * {
+            if constexpr (DUAL) {
+                if (off >= half_bytes) {
+                    int o2 = off - half_bytes;
+                    return o2 + width <= bytes ? base_up + o2 : p.w[seg];
+                }
             }
-        }
-    };
-    auto commit = [&](uint8_t *buf) {
+            return off + width <= bytes ? base + off : p.w[seg];
+        };
 #pragma unroll
-        for (int w = 0; w < NW; w++) {
-#pragma unroll
-            for (int k = 0; k < NL; k++) {
-                int off = (k * nthreads + tid) * 16;
-                if (off < tile_bytes) *(uint4 *)(buf + w * tile_bytes + off) = stg[w][k];
-            }
+        for (int k = 0; k < X4; k++) {
+            const int wave_off = (k * nthreads + wave * JL_WAVE) * 16;
+            __builtin_amdgcn_global_load_lds((gvoid *)source(wave_off + lane * 16, 16),
+                                             (lvoid *)(dst + wave_off), 16, 0, 0);
         }
+        const int wave_off = X4 * nthreads * 16 + wave * JL_WAVE * 4;
+        __builtin_amdgcn_global_load_lds((gvoid *)source(wave_off + lane * 4, 4),
+                                         (lvoid *)(dst + wave_off), 4, 0, 0);
     };
 
-    int tile = blockIdx.x;
-    if (tile < total_tiles) issue(tile);
+    // my tiles: blockIdx.x, blockIdx.x + gridDim.x, ...
+    const int first = blockIdx.x;
+    const int mine = first < total_tiles ? (total_tiles - first + gridDim.x - 1) / gridDim.x : 0;
 
-    // activations: global -> LDS (coalesced) -> 64 registers per thread
-    float *xs = (float *)region;
-    for (int i = tid * 4; i < p.n; i += nthreads * 4) *(float4 *)(xs + i) = *(const float4 *)(p.x + i);
-    __syncthreads();
+    // activations first (oldest loads), then the first kStages - 1 tiles
+    const int x_bytes = (p.n * 4 + nthreads * 16 - 1) / (nthreads * 16) * (nthreads * 16);
+    const bool x_in_ring = x_bytes <= stage_bytes;
+    uint8_t *xs = x_in_ring ? ring + (kStages - 1) * stage_bytes : ring + kStages * stage_bytes;
+    const uint32_t xs0 = x_in_ring ? ring0 + (kStages - 1) * stage_bytes : ring0 + kStages * stage_bytes;
+    for (int base = 0; base < x_bytes; base += nthreads * 16) {
+        int off = base + tid * 16;
+        const uint8_t *src = (const uint8_t *)p.x + (off < p.n * 4 ? off : 0);
+        __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
+    }
+    int issued = 0;
+    for (; issued < kStages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
+    wait_vm_tiles(issued, L);
+    __builtin_amdgcn_s_barrier();
+
     float x[64];
     float sx[2] = {0.f, 0.f};
     if (active) {
 #pragma unroll
-        for (int k = 0; k < 16; k++) {
-            float4 v = *(const float4 *)(xs + s * 64 + 4 * k);
-            x[4 * k + 0] = v.x;
-            x[4 * k + 1] = v.y;
-            x[4 * k + 2] = v.z;
-            x[4 * k + 3] = v.w;
-        }
+        for (int k = 0; k < 4; k++) lds_read_16f(xs0 + (s * 64 + k * 16) * 4, &x[k * 16]);
     } else {
 #pragma unroll
         for (int k = 0; k < 64; k++) x[k] = 0.f;
@@ -253,71 +350,62 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
             sx[1] += x[32 + k];
         }
     }
-    __syncthreads();  // the activation staging area is reused by the tile stages below
 
-    const int stage_bytes = NW * tile_bytes;
-    const int waves_per_row = p.Sp > JL_WAVE ? p.Sp / JL_WAVE : 1;
-    const int wave = tid / JL_WAVE;
-    const int lane = tid & (JL_WAVE - 1);
+    const int group = p.Sp < JL_WAVE ? p.Sp : JL_WAVE;     // lanes that share a row inside a wave
+    const int parts = p.Sp > JL_WAVE ? p.Sp / JL_WAVE : 1;  // wave partials per row
 
-    // Finishes the rows of a tile whose per-wave partial sums sit in `partial` (rows wider than a
-    // wave only): thread `row * Sp` adds its row's wave partials and applies the epilogue.
-    auto write_out = [&](int t, float v0, float v1) {
-        int seg = 0;
+    // Adds up the partial sums of tile `t` left in parity `par` and writes its rows.
+    auto finish = [&](int t, int par) {
+        if (tid < half_rows) {
+            int seg = 0;
 #pragma unroll
-        for (int i = 1; i < kMaxSeg; i++)
-            if (i < p.nseg && t >= p.seg_tile_begin[i]) seg = i;
-        int row = (t - p.seg_tile_begin[seg]) * p.R + r;
-        if (row < p.seg_rows[seg]) {
-            float *o = p.out[seg] + row;
-            if (p.epilogue == JL_SWIGLU) *o = jl_swiglu_value(v0, v1);
-            else if (p.epilogue == JL_RESIDUAL) *o = *o + v0;
-            else *o = v0;
-        }
-    };
-    auto finish_wide = [&](int t, int parity) {
-        if (s == 0 && r < p.R) {
-            float v0 = 0.f, v1 = 0.f;
-            for (int k = 0; k < waves_per_row; k++) {
-                v0 += partial[(parity * 2 + 0) * 8 + r * waves_per_row + k];
-                if constexpr (DUAL) v1 += partial[(parity * 2 + 1) * 8 + r * waves_per_row + k];
+            for (int i = 1; i < kMaxSeg; i++)
+                if (i < p.nseg && t >= p.seg_tile_begin[i]) seg = i;
+            const int row = (t - p.seg_tile_begin[seg]) * half_rows + tid;
+            if (row < p.seg_rows[seg]) {
+                const uint32_t pb = lds0 + par * 2048;
+                float v0 = 0.f, v1 = 0.f;
+                for (int k = 0; k < parts; k++) {
+                    v0 += __uint_as_float(lds_read_b32(pb + (tid * parts + k) * 4));
+                    if constexpr (DUAL)
+                        v1 += __uint_as_float(lds_read_b32(pb + ((half_rows + tid) * parts + k) * 4));
+                }
+                float *o = p.out[seg] + row;
+                if constexpr (DUAL) {
+                    *o = jl_swiglu_value(v0, v1);
+                } else {
+                    // no read-modify-write through a load: a load's wait would drain the prefetch ring
+                    if (p.epilogue == JL_RESIDUAL) unsafeAtomicAdd(o, v0);
+                    else *o = v0;
+                }
             }
-            write_out(t, v0, v1);
         }
     };
 
-    int iter = 0;
-    int prev_tile = -1;
-    for (; tile < total_tiles; tile += gridDim.x, iter++) {
-        uint8_t *buf = region + (iter & 1) * stage_bytes;
-        commit(buf);
-        int next = tile + gridDim.x;
-        if (next < total_tiles) issue(next);
-        __syncthreads();
-        if (waves_per_row > 1 && prev_tile >= 0) finish_wide(prev_tile, (iter - 1) & 1);
+    for (int it = 0; it < mine; it++) {
+        const int tile = first + it * gridDim.x;
+        // tiles issued after tile `it`: up to kStages - 2 of them may stay in flight
+        wait_vm_tiles(issued - it - 1, L);
+        __builtin_amdgcn_s_barrier();
+        // the stage that tile it - 1 (or, the first time round, the activation vector) occupied
+        // is free now: every wave is past its reads
+        if (issued < mine) {
+            issue(first + issued * gridDim.x, issued % kStages);
+            issued++;
+        }
+        if (it > 0) finish(tile - gridDim.x, (it - 1) & 1);
 
-        float v0 = 0.f, v1 = 0.f;
-        if (active) {
-            v0 = slice_dot<TYPE>(buf, r, s, p.row_bytes, x, sx);
-            if constexpr (DUAL) v1 = slice_dot<TYPE>(buf + tile_bytes, r, s, p.row_bytes, x, sx);
+        float v = 0.f;
+        if (active) v = slice_dot_lds<TYPE>(ring0 + (it % kStages) * stage_bytes, r, s, p.row_bytes, x, sx);
+        v = jl_group_sum_dyn(v, group);
+        if (active && (lane & (group - 1)) == 0) {
+            const int slot = r * parts + (s / JL_WAVE);
+            lds_write_b32(lds0 + (it & 1) * 2048 + slot * 4, __float_as_uint(v));
         }
-        if (waves_per_row == 1) {
-            v0 = jl_group_sum_dyn(v0, p.Sp);
-            if constexpr (DUAL) v1 = jl_group_sum_dyn(v1, p.Sp);
-            if (s == 0 && r < p.R) write_out(tile, v0, v1);
-        } else {
-            v0 = jl_group_sum<JL_WAVE>(v0);
-            if constexpr (DUAL) v1 = jl_group_sum<JL_WAVE>(v1);
-            if (lane == 0) {
-                partial[((iter & 1) * 2 + 0) * 8 + wave] = v0;
-                if constexpr (DUAL) partial[((iter & 1) * 2 + 1) * 8 + wave] = v1;
-            }
-        }
-        prev_tile = tile;
     }
-    if (waves_per_row > 1 && prev_tile >= 0) {
-        __syncthreads();
-        finish_wide(prev_tile, (iter - 1) & 1);
+    if (mine > 0) {
+        __builtin_amdgcn_s_barrier();
+        finish(first + (mine - 1) * gridDim.x, (mine - 1) & 1);
     }
 }
 
@@ -446,22 +534,23 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
                    const jl_weight *w_up, const float *x, int epilogue) {
     const int type = w[0]->type;
     const int n = (int)w[0]->cols;
-    const int slice_bytes = type == JL_Q8_0 ? 68 : 36;
     const int row_bytes = n / jl_block_elems(type) * jl_block_bytes(type);
 
+    const bool dual = w_up != nullptr;
+    const int slice = type == JL_Q8_0 ? 68 : 36;
     bool fast = (n % 64 == 0) && (n / 64 <= 256) && (((uintptr_t)x & 15) == 0);
-    int S = n / 64, Sp = 0, R = 0;
+    int S = n / 64, Sp = 0, R = 0, half_rows = 0;
     if (fast) {
         Sp = S <= 64 ? next_pow2(S) : (S + 63) / 64 * 64;
         R = 256 / Sp;
-        if (R < 1) fast = false;
-        else if (((int64_t)R * row_bytes) % 16 != 0) fast = false;
+        half_rows = dual ? R / 2 : R;
+        if (half_rows < 1) fast = false;
+        else if (((int64_t)half_rows * row_bytes) % 16 != 0) fast = false;
     }
     for (int i = 0; fast && i < nseg; i++) {
         if (((uintptr_t)w[i]->blocks & 15) != 0) fast = false;
     }
     if (w_up && ((uintptr_t)w_up->blocks & 15) != 0) fast = false;
-    (void)slice_bytes;
 
     if (!fast) {
         for (int i = 0; i < nseg; i++) {
@@ -487,7 +576,7 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
         p.out[i] = outs[i];
         p.seg_rows[i] = (int)w[i]->rows;
         p.seg_tile_begin[i] = tiles;
-        tiles += ((int)w[i]->rows + R - 1) / R;
+        tiles += ((int)w[i]->rows + half_rows - 1) / half_rows;
     }
     p.seg_tile_begin[nseg] = tiles;
     p.w_up = w_up ? w_up->blocks : nullptr;
@@ -500,12 +589,10 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     p.epilogue = epilogue;
 
     const int threads = (R * Sp + 63) / 64 * 64;
-    const int tile_bytes = R * row_bytes;
-    const int stages = 2 * (w_up ? 2 : 1) * tile_bytes;
-    const int region = stages > n * 4 ? stages : n * 4;
-    const int lds = kPartialBytes + region;
+    const int stage_bytes = threads * slice;
+    const int x_bytes = (n * 4 + threads * 16 - 1) / (threads * 16) * (threads * 16);
+    const int lds = kPartialBytes + kStages * stage_bytes + (x_bytes <= stage_bytes ? 0 : x_bytes);
 
-    const bool dual = w_up != nullptr;
     switch (type) {
         case JL_Q8_0:
             return dual ? launch_tiles<JL_Q8_0, true>(ctx, p, threads, lds)
