@@ -24,6 +24,8 @@
 #include "jl_device.h"
 #include "jl_internal.h"
 
+#include <stdlib.h>
+
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -42,10 +44,12 @@ struct GemvParams {
     const float *x;
     int n;          // row length
     int S;          // 64-element slices per row
-    int Sp;         // S padded: next power of two when S <= 64, else next multiple of 64
+    int Sp;         // S padded to the next power of two
     int R;          // rows per tile
     int row_bytes;
     int epilogue;
+    int stages;     // depth of the LDS tile ring (2..8)
+    int debug;
 };
 
 template <int TYPE> struct Traits;
@@ -158,14 +162,20 @@ typedef __attribute__((address_space(3))) void lvoid;
 #define JL_WAIT_VM(N) \
     __builtin_amdgcn_s_waitcnt(((N)&0xF) | (((N) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
 
-__device__ __forceinline__ void wait_vm_tiles(int tiles, int per_tile) {
-    // per_tile is 3 or 5, tiles 0..2: every case is an immediate
-    int n = tiles * per_tile;
-    if (n >= 10) JL_WAIT_VM(10);
-    else if (n == 6) JL_WAIT_VM(6);
-    else if (n == 5) JL_WAIT_VM(5);
-    else if (n == 3) JL_WAIT_VM(3);
-    else JL_WAIT_VM(0);
+// Waits until at most `tiles` tiles' worth of loads (PER_TILE each) are outstanding; every case is
+// an immediate, as the instruction requires.
+template <int PER_TILE>
+__device__ __forceinline__ void wait_vm_tiles(int tiles) {
+    switch (tiles) {
+        case 0: JL_WAIT_VM(0); break;
+        case 1: JL_WAIT_VM(PER_TILE); break;
+        case 2: JL_WAIT_VM(2 * PER_TILE); break;
+        case 3: JL_WAIT_VM(3 * PER_TILE); break;
+        case 4: JL_WAIT_VM(4 * PER_TILE); break;
+        case 5: JL_WAIT_VM(5 * PER_TILE); break;
+        case 6: JL_WAIT_VM(6 * PER_TILE); break;
+        default: JL_WAIT_VM(7 * PER_TILE); break;
+    }
 }
 
 __device__ __forceinline__ uint32_t lds_read_b32(uint32_t addr) {
@@ -196,31 +206,36 @@ __device__ __forceinline__ void lds_read_16f(uint32_t addr, float *x) {
     x[12] = d.x; x[13] = d.y; x[14] = d.z; x[15] = d.w;
 }
 
-// 17 consecutive dwords (one Q8_0 block pair)
+// 17 consecutive dwords (one Q8_0 block pair): eight two-dword reads and one single
 __device__ __forceinline__ void lds_read_17(uint32_t addr, uint32_t (&w)[17]) {
+    uint2 p0, p1, p2, p3, p4, p5, p6, p7;
+    uint32_t last;
     asm volatile(
-        "ds_read_b32 %0, %17\n\tds_read_b32 %1, %17 offset:4\n\tds_read_b32 %2, %17 offset:8\n\t"
-        "ds_read_b32 %3, %17 offset:12\n\tds_read_b32 %4, %17 offset:16\n\tds_read_b32 %5, %17 offset:20\n\t"
-        "ds_read_b32 %6, %17 offset:24\n\tds_read_b32 %7, %17 offset:28\n\tds_read_b32 %8, %17 offset:32\n\t"
-        "ds_read_b32 %9, %17 offset:36\n\tds_read_b32 %10, %17 offset:40\n\tds_read_b32 %11, %17 offset:44\n\t"
-        "ds_read_b32 %12, %17 offset:48\n\tds_read_b32 %13, %17 offset:52\n\tds_read_b32 %14, %17 offset:56\n\t"
-        "ds_read_b32 %15, %17 offset:60\n\tds_read_b32 %16, %17 offset:64\n\ts_waitcnt lgkmcnt(0)"
-        : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3]), "=&v"(w[4]), "=&v"(w[5]), "=&v"(w[6]),
-          "=&v"(w[7]), "=&v"(w[8]), "=&v"(w[9]), "=&v"(w[10]), "=&v"(w[11]), "=&v"(w[12]),
-          "=&v"(w[13]), "=&v"(w[14]), "=&v"(w[15]), "=&v"(w[16])
+        "ds_read2_b32 %0, %9 offset0:0 offset1:1\n\tds_read2_b32 %1, %9 offset0:2 offset1:3\n\t"
+        "ds_read2_b32 %2, %9 offset0:4 offset1:5\n\tds_read2_b32 %3, %9 offset0:6 offset1:7\n\t"
+        "ds_read2_b32 %4, %9 offset0:8 offset1:9\n\tds_read2_b32 %5, %9 offset0:10 offset1:11\n\t"
+        "ds_read2_b32 %6, %9 offset0:12 offset1:13\n\tds_read2_b32 %7, %9 offset0:14 offset1:15\n\t"
+        "ds_read_b32 %8, %9 offset:64\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(p0), "=&v"(p1), "=&v"(p2), "=&v"(p3), "=&v"(p4), "=&v"(p5), "=&v"(p6), "=&v"(p7),
+          "=&v"(last)
         : "v"(addr) : "memory");
+    w[0] = p0.x; w[1] = p0.y; w[2] = p1.x; w[3] = p1.y; w[4] = p2.x; w[5] = p2.y; w[6] = p3.x;
+    w[7] = p3.y; w[8] = p4.x; w[9] = p4.y; w[10] = p5.x; w[11] = p5.y; w[12] = p6.x; w[13] = p6.y;
+    w[14] = p7.x; w[15] = p7.y; w[16] = last;
 }
 
 // 9 consecutive dwords (one Q4_0 block pair)
 __device__ __forceinline__ void lds_read_9(uint32_t addr, uint32_t (&w)[9]) {
+    uint2 p0, p1, p2, p3;
+    uint32_t last;
     asm volatile(
-        "ds_read_b32 %0, %9\n\tds_read_b32 %1, %9 offset:4\n\tds_read_b32 %2, %9 offset:8\n\t"
-        "ds_read_b32 %3, %9 offset:12\n\tds_read_b32 %4, %9 offset:16\n\tds_read_b32 %5, %9 offset:20\n\t"
-        "ds_read_b32 %6, %9 offset:24\n\tds_read_b32 %7, %9 offset:28\n\tds_read_b32 %8, %9 offset:32\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3]), "=&v"(w[4]), "=&v"(w[5]), "=&v"(w[6]),
-          "=&v"(w[7]), "=&v"(w[8])
+        "ds_read2_b32 %0, %5 offset0:0 offset1:1\n\tds_read2_b32 %1, %5 offset0:2 offset1:3\n\t"
+        "ds_read2_b32 %2, %5 offset0:4 offset1:5\n\tds_read2_b32 %3, %5 offset0:6 offset1:7\n\t"
+        "ds_read_b32 %4, %5 offset:32\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(p0), "=&v"(p1), "=&v"(p2), "=&v"(p3), "=&v"(last)
         : "v"(addr) : "memory");
+    w[0] = p0.x; w[1] = p0.y; w[2] = p1.x; w[3] = p1.y; w[4] = p2.x; w[5] = p2.y; w[6] = p3.x;
+    w[7] = p3.y; w[8] = last;
 }
 
 // a Q4_K super-block header (16 B) and the 32 nibble bytes of one pair
@@ -254,8 +269,15 @@ __device__ __forceinline__ float slice_dot_lds(uint32_t stage, int r, int s, int
 // LDS map: [0, kPartialBytes) row partial sums, two parities; then the stage ring.  The activation
 // vector is staged in the ring's last stage (or, when it is larger than a stage, in a region of
 // its own after the ring) until every thread holds its 64 activations in registers.
-constexpr int kPartialBytes = 4096;  // 2 parities x 512 floats
-constexpr int kStages = 3;
+constexpr int kPartialBytes = 2048;  // 2 parities x 256 floats
+
+// v + (the value two quad neighbours hold): DPP quad permutes, VALU speed, no LDS round trip
+__device__ __forceinline__ float quad_xor1(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float quad_xor2(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));
+}
 
 template <int TYPE, bool DUAL>
 __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
@@ -264,6 +286,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     constexpr int L = X4 + 1;                     // plus one 4-byte load
     constexpr int SLICE = X4 * 16 + 4;            // bytes of a tile one thread brings in
 
+    if (p.debug == 1) return;
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int wave = tid / JL_WAVE;
@@ -275,10 +298,23 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     const int half_bytes = half_rows * p.row_bytes;   // bytes of a tile that come from one weight
     const int total_tiles = p.seg_tile_begin[p.nseg];
     const int stage_bytes = nthreads * SLICE;
+    // every thread of the workgroup owns a slice and every load slot is real data
+    const bool exact = (p.S == p.Sp) && (p.R * p.Sp == nthreads);
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
     const uint32_t ring0 = lds0 + kPartialBytes;
     uint8_t *ring = lds + kPartialBytes;
+
+    // Per-thread byte offsets of its L load slots inside a tile; for a gate/up tile the slots past
+    // half_bytes read the up weight.
+    int slot_off[L];
+    bool slot_up[L];
+#pragma unroll
+    for (int k = 0; k < L; k++) {
+        int off = k < X4 ? (k * nthreads + tid) * 16 : X4 * nthreads * 16 + tid * 4;
+        slot_up[k] = DUAL && off >= half_bytes;
+        slot_off[k] = slot_up[k] ? off - half_bytes : off;
+    }
 
     // Brings tile `tile` into stage `st`.  Every thread issues exactly L loads, whatever the tile:
     // lanes that have nothing to fetch re-read the segment's first bytes into their own slot, so
@@ -293,52 +329,54 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         const int64_t remain = (int64_t)p.seg_rows[seg] * p.row_bytes - offset;
         const int bytes = remain < half_bytes ? (int)remain : half_bytes;
         const uint8_t *base = p.w[seg] + offset;
-        const uint8_t *base_up = DUAL ? p.w_up + offset : nullptr;
+        const uint8_t *base_up = DUAL ? p.w_up + offset : base;
         uint8_t *dst = ring + st * stage_bytes;
-        auto source = [&](int off, int width) -> const uint8_t * {
-            if constexpr (DUAL) {
-                if (off >= half_bytes) {
-                    int o2 = off - half_bytes;
-                    return o2 + width <= bytes ? base_up + o2 : p.w[seg];
-                }
-            }
-            return off + width <= bytes ? base + off : p.w[seg];
-        };
+        const bool whole = exact && bytes == half_bytes;  // uniform
 #pragma unroll
-        for (int k = 0; k < X4; k++) {
-            const int wave_off = (k * nthreads + wave * JL_WAVE) * 16;
-            __builtin_amdgcn_global_load_lds((gvoid *)source(wave_off + lane * 16, 16),
-                                             (lvoid *)(dst + wave_off), 16, 0, 0);
+        for (int k = 0; k < L; k++) {
+            const int width = k < X4 ? 16 : 4;
+            const int wave_off = k < X4 ? (k * nthreads + wave * JL_WAVE) * 16
+                                        : X4 * nthreads * 16 + wave * JL_WAVE * 4;
+            const uint8_t *src = (DUAL && slot_up[k] ? base_up : base) + slot_off[k];
+            if (!whole && slot_off[k] + width > bytes) src = p.w[seg];
+            if (k < X4)
+                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + wave_off), 16, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + wave_off), 4, 0, 0);
         }
-        const int wave_off = X4 * nthreads * 16 + wave * JL_WAVE * 4;
-        __builtin_amdgcn_global_load_lds((gvoid *)source(wave_off + lane * 4, 4),
-                                         (lvoid *)(dst + wave_off), 4, 0, 0);
     };
 
     // my tiles: blockIdx.x, blockIdx.x + gridDim.x, ...
     const int first = blockIdx.x;
     const int mine = first < total_tiles ? (total_tiles - first + gridDim.x - 1) / gridDim.x : 0;
 
-    // activations first (oldest loads), then the first kStages - 1 tiles
-    const int x_bytes = (p.n * 4 + nthreads * 16 - 1) / (nthreads * 16) * (nthreads * 16);
-    const bool x_in_ring = x_bytes <= stage_bytes;
-    uint8_t *xs = x_in_ring ? ring + (kStages - 1) * stage_bytes : ring + kStages * stage_bytes;
-    const uint32_t xs0 = x_in_ring ? ring0 + (kStages - 1) * stage_bytes : ring0 + kStages * stage_bytes;
+    // Activations first (oldest loads), then the first stages - 1 tiles.  In LDS a thread's 64
+    // activations take 17 sixteen-byte slots, the last one padding: slices then start 272 bytes
+    // apart and the 128-bit reads below spread over all banks (256 bytes apart they would all
+    // land on the same four).  Slot q holds floats 64 * (q / 17) + 4 * (q % 17) ... + 3.
+    const int x_slots = p.S * 17;
+    const int x_bytes = (x_slots + nthreads - 1) / nthreads * nthreads * 16;
+    const bool x_in_ring = x_bytes <= stage_bytes;  // else a region of its own after the ring
+    uint8_t *xs = x_in_ring ? ring + (p.stages - 1) * stage_bytes : ring + p.stages * stage_bytes;
+    const uint32_t xs0 = x_in_ring ? ring0 + (p.stages - 1) * stage_bytes : ring0 + p.stages * stage_bytes;
     for (int base = 0; base < x_bytes; base += nthreads * 16) {
-        int off = base + tid * 16;
-        const uint8_t *src = (const uint8_t *)p.x + (off < p.n * 4 ? off : 0);
-        __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
+        const int q = base / 16 + tid;
+        const int sl = q / 17, k = q - sl * 17;
+        const int off = (sl < p.S && k < 16) ? (sl * 64 + k * 4) * 4 : 0;
+        __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.x + off),
+                                         (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
     }
     int issued = 0;
-    for (; issued < kStages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
-    wait_vm_tiles(issued, L);
+    for (; issued < p.stages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
+    wait_vm_tiles<L>(issued);
     __builtin_amdgcn_s_barrier();
+    if (p.debug == 2) { JL_WAIT_VM(0); return; }
 
     float x[64];
     float sx[2] = {0.f, 0.f};
     if (active) {
 #pragma unroll
-        for (int k = 0; k < 4; k++) lds_read_16f(xs0 + (s * 64 + k * 16) * 4, &x[k * 16]);
+        for (int k = 0; k < 4; k++) lds_read_16f(xs0 + s * 272 + k * 64, &x[k * 16]);
     } else {
 #pragma unroll
         for (int k = 0; k < 64; k++) x[k] = 0.f;
@@ -351,25 +389,47 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         }
     }
 
-    const int group = p.Sp < JL_WAVE ? p.Sp : JL_WAVE;     // lanes that share a row inside a wave
-    const int parts = p.Sp > JL_WAVE ? p.Sp / JL_WAVE : 1;  // wave partials per row
+    // A row's Sp lane sums are folded over quads in registers, then one lane per quad leaves its
+    // partial in LDS and the row's finishing thread adds the P = Sp / 4 partials one tile later.
+    const int P = p.Sp >= 4 ? p.Sp / 4 : 1;
+    constexpr uint32_t kParity = kPartialBytes / 2;
 
-    // Adds up the partial sums of tile `t` left in parity `par` and writes its rows.
+    // Segmented sum over aligned groups of `width` lanes (a power of two): row-local DPP moves up
+    // to 16 lanes, cross-row permutes beyond.
+    auto group_sum = [&](float v, int width) {
+        if (width >= 2) v += quad_xor1(v);
+        if (width >= 4) v += quad_xor2(v);
+        if (width >= 8)
+            v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));
+        if (width >= 16)
+            v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));
+        if (width >= 32) v += __shfl_xor(v, 16, JL_WAVE);
+        if (width >= 64) v += __shfl_xor(v, 32, JL_WAVE);
+        return v;
+    };
+
+    // Finishes tile `t` from the partials of parity `par`.  The R * P partial slots are at most
+    // 64 when P >= 1 quad per row, so wave 0 takes one slot per lane, folds each row's P lanes and
+    // lets the row's first lane apply the epilogue; narrower rows (P == 1) take one thread each.
     auto finish = [&](int t, int par) {
-        if (tid < half_rows) {
+        const int slots = half_rows * P;
+        if (tid < slots) {
             int seg = 0;
 #pragma unroll
             for (int i = 1; i < kMaxSeg; i++)
                 if (i < p.nseg && t >= p.seg_tile_begin[i]) seg = i;
-            const int row = (t - p.seg_tile_begin[seg]) * half_rows + tid;
-            if (row < p.seg_rows[seg]) {
-                const uint32_t pb = lds0 + par * 2048;
-                float v0 = 0.f, v1 = 0.f;
-                for (int k = 0; k < parts; k++) {
-                    v0 += __uint_as_float(lds_read_b32(pb + (tid * parts + k) * 4));
-                    if constexpr (DUAL)
-                        v1 += __uint_as_float(lds_read_b32(pb + ((half_rows + tid) * parts + k) * 4));
-                }
+            const uint32_t pb = lds0 + par * kParity;
+            float v0 = __uint_as_float(lds_read_b32(pb + tid * 4));
+            float v1 = 0.f;
+            if constexpr (DUAL) v1 = __uint_as_float(lds_read_b32(pb + (slots + tid) * 4));
+            if (P > 1) {
+                const int width = P < JL_WAVE ? P : JL_WAVE;
+                v0 = group_sum(v0, width);
+                if constexpr (DUAL) v1 = group_sum(v1, width);
+            }
+            const int j = tid / P;  // row of the tile
+            const int row = (t - p.seg_tile_begin[seg]) * half_rows + j;
+            if (tid - j * P == 0 && row < p.seg_rows[seg]) {
                 float *o = p.out[seg] + row;
                 if constexpr (DUAL) {
                     *o = jl_swiglu_value(v0, v1);
@@ -384,23 +444,24 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
 
     for (int it = 0; it < mine; it++) {
         const int tile = first + it * gridDim.x;
-        // tiles issued after tile `it`: up to kStages - 2 of them may stay in flight
-        wait_vm_tiles(issued - it - 1, L);
+        // tiles issued after tile `it`: up to stages - 2 of them may stay in flight
+        wait_vm_tiles<L>(issued - it - 1);
         __builtin_amdgcn_s_barrier();
         // the stage that tile it - 1 (or, the first time round, the activation vector) occupied
         // is free now: every wave is past its reads
         if (issued < mine) {
-            issue(first + issued * gridDim.x, issued % kStages);
+            issue(first + issued * gridDim.x, issued % p.stages);
             issued++;
         }
         if (it > 0) finish(tile - gridDim.x, (it - 1) & 1);
 
         float v = 0.f;
-        if (active) v = slice_dot_lds<TYPE>(ring0 + (it % kStages) * stage_bytes, r, s, p.row_bytes, x, sx);
-        v = jl_group_sum_dyn(v, group);
-        if (active && (lane & (group - 1)) == 0) {
-            const int slot = r * parts + (s / JL_WAVE);
-            lds_write_b32(lds0 + (it & 1) * 2048 + slot * 4, __float_as_uint(v));
+        if (active && p.debug != 3) v = slice_dot_lds<TYPE>(ring0 + (it % p.stages) * stage_bytes, r, s, p.row_bytes, x, sx);
+        if (p.Sp >= 2) v += quad_xor1(v);
+        if (p.Sp >= 4) v += quad_xor2(v);
+        if (r < p.R && (p.Sp < 4 ? s == 0 : (s & 3) == 0)) {
+            const int slot = r * P + (s >> 2);
+            lds_write_b32(lds0 + (it & 1) * kParity + slot * 4, __float_as_uint(v));
         }
     }
     if (mine > 0) {
@@ -510,6 +571,8 @@ template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds) {
     auto fn = jl_gemv_tiles<TYPE, DUAL>;
     int per_cu = blocks_per_cu((const void *)fn, ctx->device, threads, lds);
+    static const int cap = getenv("JL_GEMV_WGS_PER_CU") ? atoi(getenv("JL_GEMV_WGS_PER_CU")) : 0;
+    if (cap > 0 && per_cu > cap) per_cu = cap;
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
     if (grid > total) grid = total;
@@ -541,7 +604,7 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     bool fast = (n % 64 == 0) && (n / 64 <= 256) && (((uintptr_t)x & 15) == 0);
     int S = n / 64, Sp = 0, R = 0, half_rows = 0;
     if (fast) {
-        Sp = S <= 64 ? next_pow2(S) : (S + 63) / 64 * 64;
+        Sp = next_pow2(S);
         R = 256 / Sp;
         half_rows = dual ? R / 2 : R;
         if (half_rows < 1) fast = false;
@@ -590,8 +653,16 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
 
     const int threads = (R * Sp + 63) / 64 * 64;
     const int stage_bytes = threads * slice;
-    const int x_bytes = (n * 4 + threads * 16 - 1) / (threads * 16) * (threads * 16);
-    const int lds = kPartialBytes + kStages * stage_bytes + (x_bytes <= stage_bytes ? 0 : x_bytes);
+    const int x_bytes = (S * 17 + threads - 1) / threads * threads * 16;  // 17 slots per slice
+    const int x_extra = x_bytes <= stage_bytes ? 0 : x_bytes;
+    // Ring depth: few tiles per workgroup want all of them in flight at once (deep ring, fewer
+    // workgroups per compute unit); long streams want many workgroups with a short ring.
+    static const int forced = getenv("JL_GEMV_STAGES") ? atoi(getenv("JL_GEMV_STAGES")) : 0;
+    int stages = forced >= 2 && forced <= 8 ? forced : 2;
+    p.stages = stages;
+    static const int dbg = getenv("JL_GEMV_DEBUG") ? atoi(getenv("JL_GEMV_DEBUG")) : 0;
+    p.debug = dbg;
+    const int lds = kPartialBytes + stages * stage_bytes + x_extra;
 
     switch (type) {
         case JL_Q8_0:
