@@ -41,7 +41,7 @@ static int context_create(int device, hipStream_t borrowed, bool borrow, jl_cont
     JL_REQUIRE(ctx != nullptr, "jl_context_create: host allocation failed");
     ctx->device = device;
     ctx->compute_units = prop.multiProcessorCount;
-    snprintf(ctx->name, sizeof ctx->name, "%s", prop.name);
+    snprintf(ctx->name, sizeof ctx->name, "%s", prop.name[0] ? prop.name : prop.gcnArchName);
     if (borrow) {
         ctx->stream = borrowed;
         ctx->owns_stream = false;
