@@ -69,61 +69,195 @@ jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__r
     if (lane == 0) row_scale[row] = scale;
 }
 
-// ---- weight slice decode: 32 consecutive elements of one row -> fp16 -------------------------
+// ---- LDS access by hand ----------------------------------------------------------------------
+// Operand tiles arrive by LDS-DMA (global_load_lds_*).  The compiler answers any LDS access it can
+// see after such a load with a full vmcnt(0) wait, which would serialise the operand ring, so every
+// LDS access of the kernel is inline assembly with its own lgkmcnt wait, the barrier is the bare
+// instruction and the vector-memory waits are placed by hand.
 
-// `blk` addresses the 32-element unit: a Q8_0 / Q4_0 block, or for Q4_K the super-block with
-// `sub` naming the 32-element sub-block.  Each value is the host decode rounded once to fp16.
+typedef __attribute__((address_space(1))) const void gvoid;
+typedef __attribute__((address_space(3))) void lvoid;
+
+#define JL_WAIT_VM(N) \
+    __builtin_amdgcn_s_waitcnt(((N)&0xF) | (((N) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+// s_waitcnt vmcnt(n) for a run-time n (the instruction takes an immediate)
+__device__ __forceinline__ void wait_vm(int n) {
+    switch (n) {
+#define C(i) case i: JL_WAIT_VM(i); break;
+        C(0) C(1) C(2) C(3) C(4) C(5) C(6) C(7) C(8) C(9) C(10) C(11) C(12) C(13) C(14) C(15)
+        C(16) C(17) C(18) C(19) C(20) C(21) C(22) C(23) C(24) C(25) C(26) C(27) C(28) C(29) C(30)
+        C(31) C(32) C(33) C(34) C(35) C(36) C(37) C(38) C(39) C(40) C(41) C(42) C(43) C(44) C(45)
+        C(46) C(47) C(48) C(49) C(50) C(51) C(52) C(53) C(54) C(55) C(56) C(57) C(58) C(59) C(60)
+        C(61) C(62)
+#undef C
+        default: JL_WAIT_VM(63); break;
+    }
+}
+
+__device__ __forceinline__ half8 lds_read_h8(uint32_t addr) {
+    half8 v;
+    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+    return v;
+}
+
+// N 128-bit fragment reads with one wait
+template <int N>
+__device__ __forceinline__ void lds_read_h8n(const uint32_t (&addr)[N], half8 (&v)[N]) {
+    static_assert(N == 2 || N == 4, "fragment batch");
+    if constexpr (N == 4) {
+        asm volatile(
+            "ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\t"
+            "ds_read_b128 %3, %7\n\ts_waitcnt lgkmcnt(0)"
+            : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
+            : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]) : "memory");
+    } else {
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(v[0]), "=&v"(v[1]) : "v"(addr[0]), "v"(addr[1]) : "memory");
+    }
+}
+
+__device__ __forceinline__ void lds_write_4xh8(uint32_t addr, const half8 (&v)[4]) {
+    asm volatile(
+        "ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:16\n\tds_write_b128 %0, %3 offset:32\n\t"
+        "ds_write_b128 %0, %4 offset:48\n\ts_waitcnt lgkmcnt(0)"
+        : : "v"(addr), "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]) : "memory");
+}
+
+__device__ __forceinline__ void lds_read_9dw(uint32_t addr, uint32_t (&w)[9]) {
+    uint2 p0, p1, p2, p3;
+    uint32_t last;
+    asm volatile(
+        "ds_read2_b32 %0, %5 offset0:0 offset1:1\n\tds_read2_b32 %1, %5 offset0:2 offset1:3\n\t"
+        "ds_read2_b32 %2, %5 offset0:4 offset1:5\n\tds_read2_b32 %3, %5 offset0:6 offset1:7\n\t"
+        "ds_read_b32 %4, %5 offset:32\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(p0), "=&v"(p1), "=&v"(p2), "=&v"(p3), "=&v"(last) : "v"(addr) : "memory");
+    w[0] = p0.x; w[1] = p0.y; w[2] = p1.x; w[3] = p1.y; w[4] = p2.x; w[5] = p2.y; w[6] = p3.x;
+    w[7] = p3.y; w[8] = last;
+}
+
+__device__ __forceinline__ void lds_read_5dw(uint32_t addr, uint32_t (&w)[5]) {
+    uint2 p0, p1;
+    uint32_t last;
+    asm volatile(
+        "ds_read2_b32 %0, %3 offset0:0 offset1:1\n\tds_read2_b32 %1, %3 offset0:2 offset1:3\n\t"
+        "ds_read_b32 %2, %3 offset:16\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(p0), "=&v"(p1), "=&v"(last) : "v"(addr) : "memory");
+    w[0] = p0.x; w[1] = p0.y; w[2] = p1.x; w[3] = p1.y; w[4] = last;
+}
+
+__device__ __forceinline__ void lds_read_3x4(uint32_t a0, uint32_t a1, uint4 &h, uint4 &q0, uint4 &q1) {
+    asm volatile(
+        "ds_read_b128 %0, %3\n\tds_read_b128 %1, %4\n\tds_read_b128 %2, %4 offset:16\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(h), "=&v"(q0), "=&v"(q1) : "v"(a0), "v"(a1) : "memory");
+}
+
+// ---- weight decode: raw block bytes -> fp16, two elements per instruction ----------------------
+//
+// A byte b in 0..255 placed under the exponent byte 0x64 is the fp16 number 1024 + b, exactly; one
+// packed subtract recentres it (1152 = 1024 + 128 for a sign-flipped int8, 1032 = 1024 + 8 for a
+// nibble), one packed multiply applies the block scale.  Both products are exact before their one
+// rounding, so the result is the host's float decode rounded once to fp16.
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ h2 bytes_to_h2(uint32_t v, uint32_t sel) {
+    // sel picks two bytes of v (selector values 4..7) and pairs each with 0x64 (selector 0)
+    return __builtin_bit_cast(h2, __builtin_amdgcn_perm(v, 0x64646464u, sel));
+}
+
+// 4 bytes (already in 0..255 "offset" form) -> 4 fp16 = (byte - bias) * d
+__device__ __forceinline__ void dword_to_h4(uint32_t v, h2 bias, h2 d, _Float16 *dst) {
+    h2 lo = (bytes_to_h2(v, 0x00050004u) - bias) * d;
+    h2 hi = (bytes_to_h2(v, 0x00070006u) - bias) * d;
+    dst[0] = lo[0];
+    dst[1] = lo[1];
+    dst[2] = hi[0];
+    dst[3] = hi[1];
+}
+
+// One thread decodes the 32 elements (row, half) of the 64-wide slice from the raw tile in LDS.
+// raw_row = LDS address of the row's raw slice (Q8_0 68 B, Q4_0 36 B; Q4_K: 32 nibble bytes, with
+// hdr = LDS address of the super-block's 16-byte header and sub = sub-block index 0..7).
 template <int TYPE>
-__device__ __forceinline__ void decode32_to_f16(const uint8_t *blk, int sub, _Float16 *dst) {
+__device__ __forceinline__ void decode_half_slice(uint32_t raw_row, uint32_t hdr, int half, int sub,
+                                                  half8 (&out)[4]) {
+    _Float16 w[32];
     if constexpr (TYPE == JL_Q8_0) {
-        // 34 bytes, 2-byte aligned: read as 17 halfwords
-        const uint16_t *h = (const uint16_t *)blk;
-        float d = jl_half_bits_to_float(h[0]);
+        // bytes 0..1 scale A | 2..33 quants A | 34..35 scale B | 36..67 quants B
+        uint32_t dw[9];
+        lds_read_9dw(raw_row + half * 32, dw);
+        uint32_t q[8];
+        _Float16 d;
+        if (half == 0) {
+            d = __builtin_bit_cast(_Float16, (unsigned short)(dw[0] & 0xFFFF));
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            uint32_t v = h[1 + i];
-            float q0 = (float)(int)(int8_t)(v & 0xFF);
-            float q1 = (float)(int)(int8_t)(v >> 8);
-            dst[2 * i] = (_Float16)__fmul_rn(q0, d);
-            dst[2 * i + 1] = (_Float16)__fmul_rn(q1, d);
+            for (int i = 0; i < 8; i++) q[i] = __builtin_amdgcn_alignbit(dw[i + 1], dw[i], 16);
+        } else {
+            d = __builtin_bit_cast(_Float16, (unsigned short)(dw[0] >> 16));
+#pragma unroll
+            for (int i = 0; i < 8; i++) q[i] = dw[i + 1];
         }
-    } else if constexpr (TYPE == JL_Q4_0) {
-        const uint16_t *h = (const uint16_t *)blk;
-        float d = jl_half_bits_to_float(h[0]);
+        const h2 bias = {(_Float16)1152.f, (_Float16)1152.f};
+        const h2 dd = {d, d};
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            uint32_t v = h[1 + i];  // bytes 2i, 2i+1
-            dst[2 * i] = (_Float16)__fmul_rn((float)((int)(v & 0xF) - 8), d);
-            dst[2 * i + 1] = (_Float16)__fmul_rn((float)((int)((v >> 8) & 0xF) - 8), d);
-            dst[16 + 2 * i] = (_Float16)__fmul_rn((float)((int)((v >> 4) & 0xF) - 8), d);
-            dst[16 + 2 * i + 1] = (_Float16)__fmul_rn((float)((int)(v >> 12) - 8), d);
+        for (int i = 0; i < 8; i++) dword_to_h4(q[i] ^ 0x80808080u, bias, dd, &w[4 * i]);
+    } else if constexpr (TYPE == JL_Q4_0) {
+        // bytes 0..1 scale A | 2..17 nibbles A | 18..19 scale B | 20..35 nibbles B
+        uint32_t dw[5];
+        lds_read_5dw(raw_row + half * 16, dw);
+        uint32_t nb[4];
+        _Float16 d;
+        if (half == 0) {
+            d = __builtin_bit_cast(_Float16, (unsigned short)(dw[0] & 0xFFFF));
+#pragma unroll
+            for (int i = 0; i < 4; i++) nb[i] = __builtin_amdgcn_alignbit(dw[i + 1], dw[i], 16);
+        } else {
+            d = __builtin_bit_cast(_Float16, (unsigned short)(dw[0] >> 16));
+#pragma unroll
+            for (int i = 0; i < 4; i++) nb[i] = dw[i + 1];
+        }
+        const h2 bias = {(_Float16)1032.f, (_Float16)1032.f};
+        const h2 dd = {d, d};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            dword_to_h4(nb[i] & 0x0F0F0F0Fu, bias, dd, &w[4 * i]);              // elements 4i..4i+3
+            dword_to_h4((nb[i] >> 4) & 0x0F0F0F0Fu, bias, dd, &w[16 + 4 * i]);  // elements 16+4i..
         }
     } else {
-        const uint32_t *hdr = (const uint32_t *)blk;
-        uint32_t h0 = hdr[0];
-        float d = jl_half_bits_to_float(h0);
-        float dmin = jl_half_bits_to_float(h0 >> 16);
+        uint4 h, q0, q1;
+        lds_read_3x4(hdr, raw_row, h, q0, q1);
+        float d = jl_half_bits_to_float(h.x);
+        float dmin = jl_half_bits_to_float(h.x >> 16);
         int sc, mn;
-        jl_q4k_scale_min(hdr[1], hdr[2], hdr[3], sub, sc, mn);
-        float ds = __fmul_rn(d, (float)sc);
-        float dm = __fmul_rn(dmin, (float)mn);
-        const uint32_t *qs = (const uint32_t *)(blk + 16 + (sub >> 1) * 32);
-        int shift = (sub & 1) * 4;
+        jl_q4k_scale_min(h.y, h.z, h.w, sub, sc, mn);
+        // (d sc) and (dmin m) rounded to fp16, then q * ds - dm in one fused fp16 operation
+        const _Float16 ds = (_Float16)(d * (float)sc);
+        const _Float16 dm = (_Float16)(dmin * (float)mn);
+        const h2 ds2 = {ds, ds}, dm2 = {dm, dm};
+        const h2 bias = {(_Float16)1024.f, (_Float16)1024.f};
+        const uint32_t qs[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        const int shift = (sub & 1) * 4;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             uint32_t v = (qs[i] >> shift) & 0x0F0F0F0Fu;
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                float q = (float)((v >> (8 * b)) & 0xFF);
-                dst[4 * i + b] = (_Float16)__fsub_rn(__fmul_rn(ds, q), dm);
-            }
+            h2 lo = (bytes_to_h2(v, 0x00050004u) - bias) * ds2 - dm2;
+            h2 hi = (bytes_to_h2(v, 0x00070006u) - bias) * ds2 - dm2;
+            w[4 * i + 0] = lo[0];
+            w[4 * i + 1] = lo[1];
+            w[4 * i + 2] = hi[0];
+            w[4 * i + 3] = hi[1];
         }
     }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) out[i][j] = w[8 * i + j];
 }
 
 struct GemmParams {
     const uint8_t *w[kMaxWeights];
-    int w_rows[kMaxWeights];
     int w_begin[kMaxWeights + 1];  // first virtual output column of each weight
     int count;
     const _Float16 *A;       // [padded_rows x k] fp16
@@ -138,146 +272,258 @@ struct GemmParams {
     int row_bytes;
 };
 
-constexpr int BM = 128, BN = 128, BK = 64;
-constexpr int LDS_STRIDE = BK + 8;  // halfs; 144-byte rows keep 16-byte fragment reads conflict-light
+constexpr int BN = 128, BK = 64;
+constexpr int W16_STRIDE = 144;                // bytes per decoded row: 64 halfs + 16 bytes of padding
+constexpr int W16_BYTES = BN * W16_STRIDE;     // 18432
+constexpr int HDR_BYTES = 256 * 16;            // one Q4_K header slot per thread
+constexpr int HDR_RING = 4;
 
-// Workgroup: 256 threads = 4 waves as 2 (M) x 2 (N); wave tile 64 x 64 = 4 x 4 MFMA blocks of
-// 16 x 16.  For JL_SWIGLU the 128 tile columns are 64 gate rows followed by the 64 up rows of the
-// same output columns, and a wave's four column blocks are {gate, gate, up, up} of its 32 outputs.
+template <int TYPE> struct Raw;
+template <> struct Raw<JL_Q8_0> { static constexpr int kRowBytes = 68, kLoads = 9; };   // 2176 dwords
+template <> struct Raw<JL_Q4_0> { static constexpr int kRowBytes = 36, kLoads = 5; };   // 1152 dwords
+template <> struct Raw<JL_Q4_K> { static constexpr int kRowBytes = 32, kLoads = 1; };   // 256 x 16 B
+
+// bytes of one raw-weight stage: every one of the 256 threads' load slots has a place of its own
 template <int TYPE>
+constexpr int raw_stage_bytes() {
+    return Raw<TYPE>::kLoads * 256 * (TYPE == JL_Q4_K ? 16 : 4);
+}
+
+template <int TYPE, int BM, int NS>
+constexpr int gemm_lds_bytes() {
+    return NS * raw_stage_bytes<TYPE>() + (TYPE == JL_Q4_K ? HDR_RING * HDR_BYTES : 0) +
+           NS * BM * 128 + 2 * W16_BYTES;
+}
+
+// Workgroup: 256 threads = 4 waves; tile BM x 128 outputs, 64 columns of K per step.
+//   BM = 128: waves 2 (M) x 2 (N), wave tile 64 x 64
+//   BM <= 64: waves 1 x 4, wave tile BM x 32
+// For JL_SWIGLU the 128 tile columns are 64 gate rows followed by the 64 up rows of the same 64
+// outputs; a wave's column blocks are arranged so that it holds gate and up of the same outputs.
+template <int TYPE, int BM, int NS>
 __global__ void __launch_bounds__(256) jl_gemm_f16(GemmParams p) {
-    __shared__ __attribute__((aligned(16))) _Float16 As[2][BM * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) _Float16 Ws[2][BN * LDS_STRIDE];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int RAWB = raw_stage_bytes<TYPE>();
+    static_assert(RAWB >= BN * Raw<TYPE>::kRowBytes, "raw stage too small");
+    static_assert(BM == 32 || BM == 64 || BM == 128, "row tile");
+    constexpr int NLW = Raw<TYPE>::kLoads;
+    constexpr int NLA = BM * 8 / 256;
+    constexpr int ABYTES = BM * 128;
+    constexpr int WM = BM == 128 ? 2 : 1;
+    constexpr int WN = 4 / WM;
+    constexpr int TM = BM / WM;       // wave tile rows
+    constexpr int TN = BN / WN;       // wave tile columns
+    constexpr int MB = TM / 16;       // 16 x 16 blocks per wave along M
+    constexpr int NB = TN / 16;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int m0 = blockIdx.y * BM;
     const bool swiglu = p.epilogue == JL_SWIGLU;
     const int cols_per_tile = swiglu ? BN / 2 : BN;
-    const int n0 = blockIdx.x * cols_per_tile;  // first virtual output column of the tile
+    const int n0 = blockIdx.x * cols_per_tile;
 
-    // --- loader roles ---
-    // weights: thread t decodes 32 elements: tile row t / 2, half (t & 1) of the 64-wide slice
-    const int wr = tid >> 1;
-    const int wh = tid & 1;
-    const uint8_t *wrow = nullptr;  // start of the source weight row, or null past the last column
-    {
-        int vcol;
-        int widx = 0;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
+    uint8_t *raw_ring = lds;
+    uint8_t *hdr_ring = lds + NS * RAWB;
+    uint8_t *a_ring = hdr_ring + (TYPE == JL_Q4_K ? HDR_RING * HDR_BYTES : 0);
+    const uint32_t raw0 = lds0;
+    const uint32_t hdr0 = lds0 + NS * RAWB;
+    const uint32_t a0 = hdr0 + (TYPE == JL_Q4_K ? HDR_RING * HDR_BYTES : 0);
+    const uint32_t w16_0 = a0 + NS * ABYTES;
+
+    // source row of tile row r (null past the last output column)
+    auto row_ptr = [&](int r) -> const uint8_t * {
+        int vcol, widx = 0;
         if (swiglu) {
-            widx = wr >= 64 ? 1 : 0;
-            vcol = n0 + (wr & 63);
-            if (vcol < p.n_total) wrow = p.w[widx] + (int64_t)vcol * p.row_bytes;
-        } else {
-            vcol = n0 + wr;
-            if (vcol < p.n_total) {
-#pragma unroll
-                for (int i = 1; i < kMaxWeights; i++)
-                    if (i < p.count && vcol >= p.w_begin[i]) widx = i;
-                wrow = p.w[widx] + (int64_t)(vcol - p.w_begin[widx]) * p.row_bytes;
-            }
+            widx = r >= 64 ? 1 : 0;
+            vcol = n0 + (r & 63);
+            return vcol < p.n_total ? p.w[widx] + (int64_t)vcol * p.row_bytes : nullptr;
         }
+        vcol = n0 + r;
+        if (vcol >= p.n_total) return nullptr;
+#pragma unroll
+        for (int i = 1; i < kMaxWeights; i++)
+            if (i < p.count && vcol >= p.w_begin[i]) widx = i;
+        return p.w[widx] + (int64_t)(vcol - p.w_begin[widx]) * p.row_bytes;
+    };
+
+    // ---- per-thread DMA sources (a slot with nothing to fetch re-reads the first weight bytes) ----
+    const uint8_t *wsrc[NLW];
+    bool wlive[NLW];
+#pragma unroll
+    for (int j = 0; j < NLW; j++) {
+        const int i = j * 256 + tid;
+        const uint8_t *rp = nullptr;
+        int within = 0;
+        if constexpr (TYPE == JL_Q4_K) {
+            rp = row_ptr(i >> 1);            // 2 sixteen-byte chunks per row
+            within = 16 + (i & 1) * 16;
+        } else {
+            constexpr int DW = Raw<TYPE>::kRowBytes / 4;
+            const int r = i / DW;
+            if (r < BN) rp = row_ptr(r);
+            within = (i - r * DW) * 4;
+        }
+        wlive[j] = rp != nullptr;
+        wsrc[j] = wlive[j] ? rp + within : p.w[0];
     }
-    // activations: thread t copies 32 halfs (64 bytes): tile row t / 2, half (t & 1)
-    const _Float16 *arow = p.A + (int64_t)(m0 + (tid >> 1)) * p.k + (tid & 1) * 32;
-
-    half8 a_stage[4];
-    _Float16 w_stage[32];
-
-    auto load = [&](int kt) {
-        const half8 *src = (const half8 *)(arow + kt * BK);
+    const uint8_t *hsrc = nullptr;  // Q4_K: this thread's header source (rows 0..127)
+    bool hlive = false;
+    if constexpr (TYPE == JL_Q4_K) {
+        const uint8_t *rp = tid < BN ? row_ptr(tid) : nullptr;
+        hlive = rp != nullptr;
+        hsrc = hlive ? rp : p.w[0];
+    }
+    const uint8_t *asrc[NLA];
 #pragma unroll
-        for (int i = 0; i < 4; i++) a_stage[i] = src[i];
-        if (wrow) {
-            if constexpr (TYPE == JL_Q4_K) {
-                int e = kt * BK + wh * 32;  // element index in the row
-                decode32_to_f16<TYPE>(wrow + (e >> 8) * 144, (e & 255) >> 5, w_stage);
-            } else {
-                constexpr int BB = TYPE == JL_Q8_0 ? 34 : 18;
-                decode32_to_f16<TYPE>(wrow + (int64_t)(kt * 2 + wh) * BB, 0, w_stage);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 32; i++) w_stage[i] = (_Float16)0;
-        }
-    };
-    auto commit = [&](int buf) {
-        half8 *ad = (half8 *)(&As[buf][(tid >> 1) * LDS_STRIDE + (tid & 1) * 32]);
-#pragma unroll
-        for (int i = 0; i < 4; i++) ad[i] = a_stage[i];
-        half8 *wd = (half8 *)(&Ws[buf][wr * LDS_STRIDE + wh * 32]);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            half8 v;
-#pragma unroll
-            for (int j = 0; j < 8; j++) v[j] = w_stage[8 * i + j];
-            wd[i] = v;
-        }
-    };
-
-    floatx4 acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    // LDS row of each of the wave's four column blocks
-    int brow[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        if (swiglu) brow[j] = (j >> 1) * 64 + wn * 32 + (j & 1) * 16;
-        else brow[j] = wn * 64 + j * 16;
+    for (int j = 0; j < NLA; j++) {
+        const int i = j * 256 + tid;
+        int r = i >> 3, c = i & 7;
+        if (r >= BM) r = 0;
+        asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + ((c ^ (r & 7)) << 4);
     }
 
     const int ksteps = p.k / BK;
-    load(0);
-    for (int kt = 0; kt < ksteps; kt++) {
-        const int buf = kt & 1;
-        commit(buf);
-        __syncthreads();
-        if (kt + 1 < ksteps) load(kt + 1);
+
+    // number of loads a thread issues for step s
+    auto loads_of = [&](int s) -> int {
+        return NLW + NLA + ((TYPE == JL_Q4_K && (s & 3) == 0) ? 1 : 0);
+    };
+    auto issue = [&](int s) {
+        const int st = s % NS;
+        uint8_t *rdst = raw_ring + st * RAWB;
+        int64_t woff;
+        if constexpr (TYPE == JL_Q4_K) woff = (int64_t)(s >> 2) * 144 + (s & 3) * 32;
+        else woff = (int64_t)s * Raw<TYPE>::kRowBytes;
 #pragma unroll
-        for (int ks = 0; ks < BK / 32; ks++) {
-            half8 a[4], b[4];
-            const int koff = ks * 32 + (lane >> 4) * 8;
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                a[i] = *(const half8 *)(&As[buf][(wm * 64 + i * 16 + (lane & 15)) * LDS_STRIDE + koff]);
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                b[j] = *(const half8 *)(&Ws[buf][(brow[j] + (lane & 15)) * LDS_STRIDE + koff]);
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < NLW; j++) {
+            const uint8_t *src = wlive[j] ? wsrc[j] + woff : wsrc[j];
+            if constexpr (TYPE == JL_Q4_K)
+                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(rdst + (j * 256 + wave * 64) * 16), 16, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(rdst + (j * 256 + wave * 64) * 4), 4, 0, 0);
         }
+        if constexpr (TYPE == JL_Q4_K) {
+            if ((s & 3) == 0) {
+                const uint8_t *src = hlive ? hsrc + (int64_t)(s >> 2) * 144 : hsrc;
+                uint8_t *hdst = hdr_ring + ((s >> 2) % HDR_RING) * HDR_BYTES;
+                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(hdst + wave * 64 * 16), 16, 0, 0);
+            }
+        }
+        uint8_t *adst = a_ring + st * ABYTES;
+#pragma unroll
+        for (int j = 0; j < NLA; j++)
+            __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)s * 128),
+                                             (lvoid *)(adst + (j * 256 + wave * 64) * 16), 16, 0, 0);
+    };
+
+    // ---- decode role: tile row tid % 128, half tid / 128 (uniform per wave) ----
+    const int drow = tid & 127;
+    const int dhalf = tid >> 7;
+    auto dequant = [&](int s) {
+        half8 v[4];
+        const uint32_t rr = raw0 + (s % NS) * RAWB + drow * Raw<TYPE>::kRowBytes;
+        const uint32_t hh = hdr0 + ((s >> 2) % HDR_RING) * HDR_BYTES + drow * 16;
+        decode_half_slice<TYPE>(rr, hh, dhalf, (s & 3) * 2 + dhalf, v);
+        lds_write_4xh8(w16_0 + (s & 1) * W16_BYTES + drow * W16_STRIDE + dhalf * 64, v);
+    };
+
+    floatx4 acc[MB][NB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int j = 0; j < NB; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // LDS row of each of the wave's column blocks
+    int brow[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        if (swiglu) brow[j] = (j / (NB / 2)) * 64 + wn * (TN / 2) + (j % (NB / 2)) * 16;
+        else brow[j] = wn * TN + j * 16;
     }
 
-    // epilogue: lane holds rows 4 * (lane / 16) + e, column lane % 16 of each 16 x 16 block
+    // fragments of both 32-column halves of a step, then the MFMAs: the reads sit ahead of the next
+    // step's decode in program order so that the matrix pipe runs under the decode's VALU work
+    half8 fa[2][MB], fb[2][NB];
+    auto load_frags = [&](int s) {
+        const uint32_t abase = a0 + (s % NS) * ABYTES;
+        const uint32_t wbase = w16_0 + (s & 1) * W16_BYTES;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+        for (int ks = 0; ks < 2; ks++) {
+            const int chunk = ks * 4 + (lane >> 4);
+            uint32_t aa[MB], ba[NB];
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                const int r = wm * TM + i * 16 + (lane & 15);
+                aa[i] = abase + r * 128 + ((chunk ^ (r & 7)) << 4);
+            }
+#pragma unroll
+            for (int j = 0; j < NB; j++) ba[j] = wbase + (brow[j] + (lane & 15)) * W16_STRIDE + chunk * 16;
+            lds_read_h8n<MB>(aa, fa[ks]);
+            lds_read_h8n<NB>(ba, fb[ks]);
+        }
+    };
+    auto do_mfma = [&]() {
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[ks][i], fb[ks][j], acc[i][j], 0, 0, 0);
+    };
+
+    // ---- pipeline ----
+    int issued = 0;
+    for (; issued < NS - 1 && issued < ksteps; issued++) issue(issued);
+    {
+        int pending = 0;
+        for (int s = 1; s < issued; s++) pending += loads_of(s);
+        wait_vm(pending);
+    }
+    __builtin_amdgcn_s_barrier();
+    dequant(0);
+
+    for (int kt = 0; kt < ksteps; kt++) {
+        // step kt + 1 must have landed; steps kt + 2 .. issued - 1 may stay in flight
+        int pending = 0;
+        for (int s = kt + 2; s < issued; s++) pending += loads_of(s);
+        wait_vm(pending);
+        __builtin_amdgcn_s_barrier();
+        if (issued < ksteps) {
+            issue(issued);
+            issued++;
+        }
+        load_frags(kt);
+        if (kt + 1 < ksteps) dequant(kt + 1);
+        do_mfma();
+    }
+
+    // ---- epilogue: lane holds rows 4 * (lane / 16) + e, column lane % 16 of each block ----
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            int m = m0 + wm * 64 + i * 16 + (lane >> 4) * 4 + e;
+            const int m = m0 + wm * TM + i * 16 + (lane >> 4) * 4 + e;
             if (m >= p.rows) continue;
-            float rs = p.row_scale[m];
+            const float rs = p.row_scale[m];
             float *crow = p.C + (int64_t)m * p.ldo + p.col_offset;
             if (swiglu) {
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    int col = n0 + wn * 32 + j * 16 + (lane & 15);
+                for (int j = 0; j < NB / 2; j++) {
+                    const int col = n0 + wn * (TN / 2) + j * 16 + (lane & 15);
                     if (col < p.n_total)
-                        crow[col] = jl_swiglu_value(acc[i][j][e] * rs, acc[i][j + 2][e] * rs);
+                        crow[col] = jl_swiglu_value(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
                 }
             } else {
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    int col = n0 + wn * 64 + j * 16 + (lane & 15);
+                for (int j = 0; j < NB; j++) {
+                    const int col = n0 + wn * TN + j * 16 + (lane & 15);
                     if (col < p.n_total) {
-                        float v = acc[i][j][e] * rs;
+                        const float v = acc[i][j][e] * rs;
                         if (p.epilogue == JL_RESIDUAL) crow[col] += v;
                         else crow[col] = v;
                     }
@@ -292,12 +538,40 @@ size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 }  // namespace
 
 size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int math) {
-    size_t padded = round_up((size_t)max_rows, BM);
+    size_t padded = round_up((size_t)max_rows, 128);
     if (math == JL_MATH_INT8) {
         return round_up(padded * (size_t)cols, 256) + round_up(padded * (size_t)(cols / 32) * 4, 256);
     }
     return round_up(padded * (size_t)cols * 2, 256) + round_up(padded * 4, 256);
 }
+
+namespace {
+
+template <int TYPE, int BM, int NS>
+int launch_gemm(jl_context *ctx, const GemmParams &p, dim3 grid) {
+    auto fn = jl_gemm_f16<TYPE, BM, NS>;
+    constexpr int lds = gemm_lds_bytes<TYPE, BM, NS>();
+    static_assert(lds <= 160 * 1024, "operand rings exceed the 160 KB of LDS");
+    static bool configured[16] = {};
+    if (ctx->device < 16 && !configured[ctx->device]) {
+        JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        configured[ctx->device] = true;
+    }
+    hipLaunchKernelGGL(fn, grid, dim3(256), lds, ctx->stream, p);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
+}
+
+template <int TYPE>
+int launch_gemm_type(jl_context *ctx, const GemmParams &p, int rows) {
+    const int cols_per_tile = p.epilogue == JL_SWIGLU ? BN / 2 : BN;
+    const unsigned ntiles = (unsigned)((p.n_total + cols_per_tile - 1) / cols_per_tile);
+    if (rows <= 32) return launch_gemm<TYPE, 32, 6>(ctx, p, dim3(ntiles, 1));
+    if (rows <= 64) return launch_gemm<TYPE, 64, 6>(ctx, p, dim3(ntiles, 1));
+    return launch_gemm<TYPE, 128, 4>(ctx, p, dim3(ntiles, (unsigned)((rows + 127) / 128)));
+}
+
+}  // namespace
 
 int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
@@ -311,12 +585,14 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     JL_REQUIRE(k % 64 == 0, "jl_gemm: row length %d is not a multiple of 64", k);
     JL_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)workspace & 255) == 0,
                "jl_gemm: X must be 16-byte and the workspace 256-byte aligned");
+    for (int i = 0; i < count; i++)
+        JL_REQUIRE(((uintptr_t)weights[i]->blocks & 15) == 0, "jl_gemm: weight %d is not 16-byte aligned", i);
     const int rows = (int)active_rows;
-    const int padded = (int)round_up((size_t)rows, BM);
+    const int padded = (int)round_up((size_t)rows, 128);
     // the workspace was sized for `batch` rows, of which `rows` <= batch are converted
     _Float16 *A = (_Float16 *)workspace;
     float *row_scale =
-        (float *)((uint8_t *)workspace + round_up(round_up((size_t)batch, BM) * (size_t)k * 2, 256));
+        (float *)((uint8_t *)workspace + round_up(round_up((size_t)batch, 128) * (size_t)k * 2, 256));
 
     hipLaunchKernelGGL(jl_rows_to_f16, dim3((padded + 3) / 4), dim3(256), 0, ctx->stream, X, A,
                        row_scale, rows, padded, k);
@@ -327,7 +603,6 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     int begin = 0;
     for (int i = 0; i < count; i++) {
         p.w[i] = weights[i]->blocks;
-        p.w_rows[i] = (int)weights[i]->rows;
         p.w_begin[i] = begin;
         begin += (int)weights[i]->rows;
     }
@@ -343,21 +618,11 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     p.epilogue = epilogue;
     p.row_bytes = k / jl_block_elems(type) * jl_block_bytes(type);
 
-    const int cols_per_tile = epilogue == JL_SWIGLU ? BN / 2 : BN;
-    dim3 grid((p.n_total + cols_per_tile - 1) / cols_per_tile, padded / BM);
     switch (type) {
-        case JL_Q8_0:
-            hipLaunchKernelGGL(jl_gemm_f16<JL_Q8_0>, grid, dim3(256), 0, ctx->stream, p);
-            break;
-        case JL_Q4_0:
-            hipLaunchKernelGGL(jl_gemm_f16<JL_Q4_0>, grid, dim3(256), 0, ctx->stream, p);
-            break;
-        case JL_Q4_K:
-            hipLaunchKernelGGL(jl_gemm_f16<JL_Q4_K>, grid, dim3(256), 0, ctx->stream, p);
-            break;
+        case JL_Q8_0: return launch_gemm_type<JL_Q8_0>(ctx, p, rows);
+        case JL_Q4_0: return launch_gemm_type<JL_Q4_0>(ctx, p, rows);
+        case JL_Q4_K: return launch_gemm_type<JL_Q4_K>(ctx, p, rows);
         default:
             return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
     }
-    JL_HIP(hipGetLastError());
-    return JL_OK;
 }
