@@ -13,6 +13,8 @@
 //     rounded once to fp16, which is what the reference's dequantize*ToFP16 kernels store;
 //   * the contraction runs on v_mfma_f32_16x16x32_f16 with fp32 accumulators;
 //   * epilogues: store, residual add, SwiGLU of a gate/up pair; rows past active_rows untouched.
+#include <stdlib.h>
+
 #include "jl_device.h"
 #include "jl_internal.h"
 
@@ -101,19 +103,35 @@ __device__ __forceinline__ half8 lds_read_h8(uint32_t addr) {
     return v;
 }
 
-// N 128-bit fragment reads with one wait
+// N 128-bit fragment reads, issued without waiting: the registers are valid only after
+// lds_wait_frags() has been given the same arrays.  Nothing may touch them in between.
 template <int N>
-__device__ __forceinline__ void lds_read_h8n(const uint32_t (&addr)[N], half8 (&v)[N]) {
+__device__ __forceinline__ void lds_issue_h8n(const uint32_t (&addr)[N], half8 (&v)[N]) {
     static_assert(N == 2 || N == 4, "fragment batch");
     if constexpr (N == 4) {
         asm volatile(
             "ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\t"
-            "ds_read_b128 %3, %7\n\ts_waitcnt lgkmcnt(0)"
+            "ds_read_b128 %3, %7"
             : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
             : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]) : "memory");
     } else {
-        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3"
                      : "=&v"(v[0]), "=&v"(v[1]) : "v"(addr[0]), "v"(addr[1]) : "memory");
+    }
+}
+
+template <int NA, int NBF>
+__device__ __forceinline__ void lds_wait_frags(half8 (&a)[NA], half8 (&b)[NBF]) {
+    if constexpr (NA == 4 && NBF == 4) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]),
+                       "+v"(b[2]), "+v"(b[3]) : : "memory");
+    } else if constexpr (NA == 4 && NBF == 2) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1])
+                     : : "memory");
+    } else {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]) : : "memory");
     }
 }
 
@@ -256,6 +274,13 @@ __device__ __forceinline__ void decode_half_slice(uint32_t raw_row, uint32_t hdr
         for (int j = 0; j < 8; j++) out[i][j] = w[8 * i + j];
 }
 
+// SiLU(g) * u in single precision: g / (1 + exp(-g)) with expf, a few ulp from the host's double
+// form and three orders of magnitude inside the fp16 path's tolerance; the double-precision exp
+// costs about 150 instructions per output, which matters at T x hidden outputs per call.
+__device__ __forceinline__ float gemm_swiglu(float g, float u) {
+    return g / (1.0f + expf(-g)) * u;
+}
+
 struct GemmParams {
     const uint8_t *w[kMaxWeights];
     int w_begin[kMaxWeights + 1];  // first virtual output column of each weight
@@ -270,13 +295,13 @@ struct GemmParams {
     int64_t col_offset;
     int epilogue;
     int row_bytes;
+    int ntiles, mtiles;      // tile grid (columns, rows)
 };
 
 constexpr int BN = 128, BK = 64;
 constexpr int W16_STRIDE = 144;                // bytes per decoded row: 64 halfs + 16 bytes of padding
 constexpr int W16_BYTES = BN * W16_STRIDE;     // 18432
 constexpr int HDR_BYTES = 256 * 16;            // one Q4_K header slot per thread
-constexpr int HDR_RING = 4;
 
 template <int TYPE> struct Raw;
 template <> struct Raw<JL_Q8_0> { static constexpr int kRowBytes = 68, kLoads = 9; };   // 2176 dwords
@@ -291,17 +316,22 @@ constexpr int raw_stage_bytes() {
 
 template <int TYPE, int BM, int NS>
 constexpr int gemm_lds_bytes() {
-    return NS * raw_stage_bytes<TYPE>() + (TYPE == JL_Q4_K ? HDR_RING * HDR_BYTES : 0) +
+    return NS * raw_stage_bytes<TYPE>() + (TYPE == JL_Q4_K ? NS * HDR_BYTES : 0) +
            NS * BM * 128 + 2 * W16_BYTES;
 }
 
-// Workgroup: 256 threads = 4 waves; tile BM x 128 outputs, 64 columns of K per step.
-//   BM = 128: waves 2 (M) x 2 (N), wave tile 64 x 64
-//   BM <= 64: waves 1 x 4, wave tile BM x 32
+// Workgroup: 512 threads = 8 waves, two per SIMD, split by role so that one role's waits are
+// covered by the other's work: waves 0-3 are *producers* (issue the LDS-DMA loads of both operands
+// and decode the raw weight slice of the next step into fp16), waves 4-7 are *consumers* (read the
+// MFMA fragments and run the matrix pipe).  One barrier per 64-column step hands a decoded slice
+// from producers to consumers and a finished stage back.  Tile BM x 128 outputs:
+//   BM = 128: consumer waves 2 (M) x 2 (N), wave tile 64 x 64
+//   BM <= 64: consumer waves 1 x 4, wave tile BM x 32
 // For JL_SWIGLU the 128 tile columns are 64 gate rows followed by the 64 up rows of the same 64
 // outputs; a wave's column blocks are arranged so that it holds gate and up of the same outputs.
 template <int TYPE, int BM, int NS>
-__global__ void __launch_bounds__(256) jl_gemm_f16(GemmParams p) {
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+jl_gemm_f16(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int RAWB = raw_stage_bytes<TYPE>();
     static_assert(RAWB >= BN * Raw<TYPE>::kRowBytes, "raw stage too small");
@@ -316,38 +346,64 @@ __global__ void __launch_bounds__(256) jl_gemm_f16(GemmParams p) {
     constexpr int MB = TM / 16;       // 16 x 16 blocks per wave along M
     constexpr int NB = TN / 16;
 
-    const int tid = threadIdx.x;
+    // the role and the wave index are the same for every lane of a wave: keep them in scalar
+    // registers so that the pipeline's bookkeeping (and the waits it selects) stays scalar code
+    const int wave8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const bool producer = wave8 < 4;
+    const int tid = threadIdx.x & 255;  // index inside the role
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = wave8 & 3;
     const int wm = wave / WN, wn = wave % WN;
-    const int m0 = blockIdx.y * BM;
     const bool swiglu = p.epilogue == JL_SWIGLU;
     const int cols_per_tile = swiglu ? BN / 2 : BN;
-    const int n0 = blockIdx.x * cols_per_tile;
+    // Tile order.  Workgroups go to the 8 XCDs round-robin by launch index, and each XCD has an L2
+    // of its own: give every XCD one contiguous run of the tile list, ordered so that the tiles it
+    // works on at any moment are a 4 (row tiles) x 8 (column tiles) patch whose operands fit that L2.
+    int mt, nt;
+    {
+        const int total = p.ntiles * p.mtiles;
+        const int per_xcd = (total + 7) / 8;
+        const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if ((blockIdx.x >> 3) >= per_xcd || logical >= total) return;
+        constexpr int GM = 4;
+        const int group = logical / (GM * p.ntiles);
+        const int rest = logical - group * (GM * p.ntiles);
+        const int rows_in_group = p.mtiles - group * GM < GM ? p.mtiles - group * GM : GM;
+        nt = rest / rows_in_group;
+        mt = group * GM + rest - nt * rows_in_group;
+    }
+    const int m0 = mt * BM;
+    const int n0 = nt * cols_per_tile;
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
     uint8_t *raw_ring = lds;
     uint8_t *hdr_ring = lds + NS * RAWB;
-    uint8_t *a_ring = hdr_ring + (TYPE == JL_Q4_K ? HDR_RING * HDR_BYTES : 0);
+    uint8_t *a_ring = hdr_ring + (TYPE == JL_Q4_K ? NS * HDR_BYTES : 0);
     const uint32_t raw0 = lds0;
     const uint32_t hdr0 = lds0 + NS * RAWB;
-    const uint32_t a0 = hdr0 + (TYPE == JL_Q4_K ? HDR_RING * HDR_BYTES : 0);
+    const uint32_t a0 = hdr0 + (TYPE == JL_Q4_K ? NS * HDR_BYTES : 0);
     const uint32_t w16_0 = a0 + NS * ABYTES;
 
-    // source row of tile row r (null past the last output column)
+    // source row of tile row r (null past the last output column); the weight table is walked with
+    // constant indices so that it stays in scalar registers
     auto row_ptr = [&](int r) -> const uint8_t * {
-        int vcol, widx = 0;
         if (swiglu) {
-            widx = r >= 64 ? 1 : 0;
-            vcol = n0 + (r & 63);
-            return vcol < p.n_total ? p.w[widx] + (int64_t)vcol * p.row_bytes : nullptr;
+            const int vcol = n0 + (r & 63);
+            const uint8_t *base = r >= 64 ? p.w[1] : p.w[0];
+            return vcol < p.n_total ? base + (int64_t)vcol * p.row_bytes : nullptr;
         }
-        vcol = n0 + r;
+        const int vcol = n0 + r;
         if (vcol >= p.n_total) return nullptr;
+        const uint8_t *base = p.w[0];
+        int first = 0;
 #pragma unroll
-        for (int i = 1; i < kMaxWeights; i++)
-            if (i < p.count && vcol >= p.w_begin[i]) widx = i;
-        return p.w[widx] + (int64_t)(vcol - p.w_begin[widx]) * p.row_bytes;
+        for (int i = 1; i < kMaxWeights; i++) {
+            if (i < p.count && vcol >= p.w_begin[i]) {
+                base = p.w[i];
+                first = p.w_begin[i];
+            }
+        }
+        return base + (int64_t)(vcol - first) * p.row_bytes;
     };
 
     // ---- per-thread DMA sources (a slot with nothing to fetch re-reads the first weight bytes) ----
@@ -383,15 +439,14 @@ __global__ void __launch_bounds__(256) jl_gemm_f16(GemmParams p) {
         const int i = j * 256 + tid;
         int r = i >> 3, c = i & 7;
         if (r >= BM) r = 0;
-        asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + ((c ^ (r & 7)) << 4);
+        asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + ((c ^ ((r >> 1) & 7)) << 4);
     }
 
     const int ksteps = p.k / BK;
 
-    // number of loads a thread issues for step s
-    auto loads_of = [&](int s) -> int {
-        return NLW + NLA + ((TYPE == JL_Q4_K && (s & 3) == 0) ? 1 : 0);
-    };
+    // loads a thread issues per step (a Q4_K super-block header is re-fetched with each of its
+    // four steps -- 16 bytes a row out of L2 -- so that the count is the same for every step)
+    constexpr int LPS = NLW + NLA + (TYPE == JL_Q4_K ? 1 : 0);
     auto issue = [&](int s) {
         const int st = s % NS;
         uint8_t *rdst = raw_ring + st * RAWB;
@@ -407,11 +462,9 @@ __global__ void __launch_bounds__(256) jl_gemm_f16(GemmParams p) {
                 __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(rdst + (j * 256 + wave * 64) * 4), 4, 0, 0);
         }
         if constexpr (TYPE == JL_Q4_K) {
-            if ((s & 3) == 0) {
-                const uint8_t *src = hlive ? hsrc + (int64_t)(s >> 2) * 144 : hsrc;
-                uint8_t *hdst = hdr_ring + ((s >> 2) % HDR_RING) * HDR_BYTES;
-                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(hdst + wave * 64 * 16), 16, 0, 0);
-            }
+            const uint8_t *src = hlive ? hsrc + (int64_t)(s >> 2) * 144 : hsrc;
+            uint8_t *hdst = hdr_ring + (s % NS) * HDR_BYTES;
+            __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(hdst + wave * 64 * 16), 16, 0, 0);
         }
         uint8_t *adst = a_ring + st * ABYTES;
 #pragma unroll
@@ -426,7 +479,7 @@ __global__ void __launch_bounds__(256) jl_gemm_f16(GemmParams p) {
     auto dequant = [&](int s) {
         half8 v[4];
         const uint32_t rr = raw0 + (s % NS) * RAWB + drow * Raw<TYPE>::kRowBytes;
-        const uint32_t hh = hdr0 + ((s >> 2) % HDR_RING) * HDR_BYTES + drow * 16;
+        const uint32_t hh = hdr0 + (s % NS) * HDR_BYTES + drow * 16;
         decode_half_slice<TYPE>(rr, hh, dhalf, (s & 3) * 2 + dhalf, v);
         lds_write_4xh8(w16_0 + (s & 1) * W16_BYTES + drow * W16_STRIDE + dhalf * 64, v);
     };
@@ -445,87 +498,120 @@ __global__ void __launch_bounds__(256) jl_gemm_f16(GemmParams p) {
         else brow[j] = wn * TN + j * 16;
     }
 
-    // fragments of both 32-column halves of a step, then the MFMAs: the reads sit ahead of the next
-    // step's decode in program order so that the matrix pipe runs under the decode's VALU work
+    // A step is two 32-column halves.  The second half's fragment reads are in flight while the
+    // first half's MFMAs run.
     half8 fa[2][MB], fb[2][NB];
-    auto load_frags = [&](int s) {
+    auto issue_frags = [&](int s, int ks) {
         const uint32_t abase = a0 + (s % NS) * ABYTES;
         const uint32_t wbase = w16_0 + (s & 1) * W16_BYTES;
+        const int chunk = ks * 4 + (lane >> 4);
+        uint32_t aa[MB], ba[NB];
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-            const int chunk = ks * 4 + (lane >> 4);
-            uint32_t aa[MB], ba[NB];
-#pragma unroll
-            for (int i = 0; i < MB; i++) {
-                const int r = wm * TM + i * 16 + (lane & 15);
-                aa[i] = abase + r * 128 + ((chunk ^ (r & 7)) << 4);
-            }
-#pragma unroll
-            for (int j = 0; j < NB; j++) ba[j] = wbase + (brow[j] + (lane & 15)) * W16_STRIDE + chunk * 16;
-            lds_read_h8n<MB>(aa, fa[ks]);
-            lds_read_h8n<NB>(ba, fb[ks]);
+        for (int i = 0; i < MB; i++) {
+            const int r = wm * TM + i * 16 + (lane & 15);
+            aa[i] = abase + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4);
         }
+#pragma unroll
+        for (int j = 0; j < NB; j++) ba[j] = wbase + (brow[j] + (lane & 15)) * W16_STRIDE + chunk * 16;
+        lds_issue_h8n<MB>(aa, fa[ks]);
+        lds_issue_h8n<NB>(ba, fb[ks]);
     };
-    auto do_mfma = [&]() {
+    auto mfma_half = [&](int ks) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++)
+        for (int i = 0; i < MB; i++)
 #pragma unroll
-            for (int i = 0; i < MB; i++)
-#pragma unroll
-                for (int j = 0; j < NB; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[ks][i], fb[ks][j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < NB; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+    };
+    auto consume = [&](int s) {
+        issue_frags(s, 0);
+        lds_wait_frags<MB, NB>(fa[0], fb[0]);
+        issue_frags(s, 1);
+        mfma_half(0);
+        lds_wait_frags<MB, NB>(fa[1], fb[1]);
+        mfma_half(1);
     };
 
     // ---- pipeline ----
+    // Step s occupies operand stage s % NS.  Producers keep NS - 1 steps of loads in flight and
+    // decode one step ahead of the consumers; the barrier at the top of iteration kt publishes the
+    // decoded slice of step kt and the landed activations of step kt, and frees what step kt - 1 used.
     int issued = 0;
-    for (; issued < NS - 1 && issued < ksteps; issued++) issue(issued);
-    {
-        int pending = 0;
-        for (int s = 1; s < issued; s++) pending += loads_of(s);
-        wait_vm(pending);
+    if (producer) {
+        for (; issued < NS - 1 && issued < ksteps; issued++) issue(issued);
+        wait_vm((issued - 1) * LPS);
     }
     __builtin_amdgcn_s_barrier();
-    dequant(0);
+    if (producer) dequant(0);
 
-    for (int kt = 0; kt < ksteps; kt++) {
-        // step kt + 1 must have landed; steps kt + 2 .. issued - 1 may stay in flight
-        int pending = 0;
-        for (int s = kt + 2; s < issued; s++) pending += loads_of(s);
-        wait_vm(pending);
+    // steady state: step kt + NS - 1 is issued in iteration kt, so when step kt + 1 is awaited
+    // exactly NS - 3 younger steps are in flight -- the wait is an immediate
+    const int steady = ksteps - (NS - 1) > 0 ? ksteps - (NS - 1) : 0;
+    int kt = 0;
+    for (; kt < steady; kt++) {
+        if (producer) JL_WAIT_VM((NS - 3) * LPS);
         __builtin_amdgcn_s_barrier();
-        if (issued < ksteps) {
-            issue(issued);
-            issued++;
+        if (producer) {
+            issue(kt + NS - 1);
+            dequant(kt + 1);
+        } else {
+            consume(kt);
         }
-        load_frags(kt);
-        if (kt + 1 < ksteps) dequant(kt + 1);
-        do_mfma();
     }
+    // drain: nothing left to issue
+    for (; kt < ksteps; kt++) {
+        if (producer) {
+            const int ahead = ksteps - (kt + 2);
+            wait_vm(ahead > 0 ? ahead * LPS : 0);
+        }
+        __builtin_amdgcn_s_barrier();
+        if (producer) {
+            if (kt + 1 < ksteps) dequant(kt + 1);
+        } else {
+            consume(kt);
+        }
+    }
+    if (producer) return;
 
-    // ---- epilogue: lane holds rows 4 * (lane / 16) + e, column lane % 16 of each block ----
+    // ---- epilogue (consumers) ----
+    // The weight fragment went in as the MFMA's row operand, so a lane holds four consecutive
+    // output columns 4 * (lane / 16) .. + 3 of activation row lane % 16 of each block: one
+    // 16-byte store per block.
 #pragma unroll
     for (int i = 0; i < MB; i++) {
+        const int m = m0 + wm * TM + i * 16 + (lane & 15);
+        if (m >= p.rows) continue;
+        const float rs = p.row_scale[m];
+        float *crow = p.C + (int64_t)m * p.ldo + p.col_offset;
+        if (swiglu) {
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int m = m0 + wm * TM + i * 16 + (lane >> 4) * 4 + e;
-            if (m >= p.rows) continue;
-            const float rs = p.row_scale[m];
-            float *crow = p.C + (int64_t)m * p.ldo + p.col_offset;
-            if (swiglu) {
+            for (int j = 0; j < NB / 2; j++) {
+                const int col = n0 + wn * (TN / 2) + j * 16 + (lane >> 4) * 4;
 #pragma unroll
-                for (int j = 0; j < NB / 2; j++) {
-                    const int col = n0 + wn * (TN / 2) + j * 16 + (lane & 15);
-                    if (col < p.n_total)
-                        crow[col] = jl_swiglu_value(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
-                }
-            } else {
+                for (int e = 0; e < 4; e++)
+                    if (col + e < p.n_total)
+                        crow[col + e] = gemm_swiglu(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
+            }
+        } else {
 #pragma unroll
-                for (int j = 0; j < NB; j++) {
-                    const int col = n0 + wn * TN + j * 16 + (lane & 15);
-                    if (col < p.n_total) {
-                        const float v = acc[i][j][e] * rs;
-                        if (p.epilogue == JL_RESIDUAL) crow[col] += v;
-                        else crow[col] = v;
+            for (int j = 0; j < NB; j++) {
+                const int col = n0 + wn * TN + j * 16 + (lane >> 4) * 4;
+                float4 v = {acc[i][j][0] * rs, acc[i][j][1] * rs, acc[i][j][2] * rs, acc[i][j][3] * rs};
+                float *dst = crow + col;
+                if (col + 3 < p.n_total && (((uintptr_t)dst) & 15) == 0) {
+                    if (p.epilogue == JL_RESIDUAL) {
+                        float4 o = *(const float4 *)dst;
+                        v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+                    }
+                    *(float4 *)dst = v;
+                } else {
+                    const float ve[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (col + e < p.n_total) {
+                            if (p.epilogue == JL_RESIDUAL) dst[e] += ve[e];
+                            else dst[e] = ve[e];
+                        }
                     }
                 }
             }
@@ -557,18 +643,22 @@ int launch_gemm(jl_context *ctx, const GemmParams &p, dim3 grid) {
         JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         configured[ctx->device] = true;
     }
-    hipLaunchKernelGGL(fn, grid, dim3(256), lds, ctx->stream, p);
+    hipLaunchKernelGGL(fn, grid, dim3(512), lds, ctx->stream, p);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
 
 template <int TYPE>
-int launch_gemm_type(jl_context *ctx, const GemmParams &p, int rows) {
+int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows) {
     const int cols_per_tile = p.epilogue == JL_SWIGLU ? BN / 2 : BN;
-    const unsigned ntiles = (unsigned)((p.n_total + cols_per_tile - 1) / cols_per_tile);
-    if (rows <= 32) return launch_gemm<TYPE, 32, 6>(ctx, p, dim3(ntiles, 1));
-    if (rows <= 64) return launch_gemm<TYPE, 64, 6>(ctx, p, dim3(ntiles, 1));
-    return launch_gemm<TYPE, 128, 4>(ctx, p, dim3(ntiles, (unsigned)((rows + 127) / 128)));
+    p.ntiles = (p.n_total + cols_per_tile - 1) / cols_per_tile;
+    const int bm = rows <= 32 ? 32 : rows <= 64 ? 64 : 128;
+    p.mtiles = (rows + bm - 1) / bm;
+    // one workgroup per tile, padded so that each of the 8 XCDs gets the same number of launch slots
+    const unsigned grid = (unsigned)((p.ntiles * p.mtiles + 7) / 8 * 8);
+    if (bm == 32) return launch_gemm<TYPE, 32, 6>(ctx, p, dim3(grid));
+    if (bm == 64) return launch_gemm<TYPE, 64, 6>(ctx, p, dim3(grid));
+    return launch_gemm<TYPE, 128, 4>(ctx, p, dim3(grid));
 }
 
 }  // namespace
