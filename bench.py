@@ -185,7 +185,7 @@ def bench_gemm(ctx, hip, t, T, steps, warmup):
     qkv = ctx.float_array(T * (DIM + 2 * KV_DIM))
     res = ctx.float_array(T * DIM, fill=0.0)
     hb = ctx.float_array(T * HIDDEN)
-    proj = QuantizedBatchProjections(ctx, T, HIDDEN)
+    proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN)
 
     def layer():
         proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
@@ -230,7 +230,7 @@ def bench_batched_q4k(ctx, hip, B, steps, warmup):
     qkv = ctx.float_array(B * (dim + 2 * kv))
     res = ctx.float_array(B * dim, fill=0.0)
     hb = ctx.float_array(B * ffn)
-    proj = QuantizedBatchProjections(ctx, B, ffn)
+    proj = QuantizedBatchProjections(ctx, B, ffn, 2 * ffn)
 
     def layer():
         proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])

@@ -150,12 +150,16 @@ int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
 /* ---- batched decode and batched prefill: `batch` activation rows ---------------------------- */
 
 /*
- * Bytes of scratch jl_gemm needs for a call of this shape (Implementation.needs,
+ * Bytes of scratch jl_gemm needs (Implementation.needs,
  * J/backend/tornado/ops/Implementation.java:31-36: sized before anything is allocated, so a
  * memory preflight equals what the call uses).  `max_rows` is the largest `batch`, `cols` the
- * row length, `math` a jl_gemm_math.
+ * largest row length, `out_cols` the largest number of output columns one call produces (a gate/up
+ * pair counts both weights' rows), `math` a jl_gemm_math.  The scratch holds the fp16 copy of the
+ * activations, one scale per row, and -- for calls of at most 64 rows, which cut K across
+ * workgroups -- the partial sums of the cuts.  A smaller workspace that still holds the first two
+ * is accepted; such calls simply do not cut K.
  */
-size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int math);
+size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols, int math);
 
 /*
  * C[b][col_offset + j] (op)= sum_k X[b][k] * W_i[j][k] for the `count` weights laid side by

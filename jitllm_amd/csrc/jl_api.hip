@@ -253,9 +253,9 @@ int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count) {
     return jl_launch_swiglu(ctx, gate, up, count);
 }
 
-size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int math) {
-    if (max_rows <= 0 || cols <= 0) return 0;
-    return jl_gemm_workspace_bytes_impl(max_rows, cols, math);
+size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols, int math) {
+    if (max_rows <= 0 || cols <= 0 || out_cols < 0) return 0;
+    return jl_gemm_workspace_bytes_impl(max_rows, cols, out_cols, math == JL_MATH_DEFAULT ? JL_MATH_F16 : math);
 }
 
 int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
@@ -294,7 +294,8 @@ int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const f
                        "value); use JL_MATH_F16");
     }
     if (active_rows == 0) return JL_OK;
-    size_t need = jl_gemm_workspace_bytes_impl(batch, weights[0]->cols, math);
+    // the activation copy and the row scales are mandatory; split-K planes are used if they fit
+    size_t need = jl_gemm_workspace_bytes_impl(batch, weights[0]->cols, 0, math);
     if (workspace_bytes < need || (need && !workspace)) {
         return jl_fail(JL_ERR_WORKSPACE, "jl_gemm: workspace %zu bytes, %zu needed", workspace_bytes,
                        need);

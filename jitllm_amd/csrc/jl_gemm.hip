@@ -296,6 +296,8 @@ struct GemmParams {
     int epilogue;
     int row_bytes;
     int ntiles, mtiles;      // tile grid (columns, rows)
+    int splits;              // K is cut into `splits` equal runs of steps, one workgroup each
+    float *partial;          // splits > 1: [splits][mtiles * BM][ntiles * 128] fp32 partial sums
 };
 
 constexpr int BN = 128, BK = 64;
@@ -363,8 +365,9 @@ jl_gemm_f16(GemmParams p) {
     {
         const int total = p.ntiles * p.mtiles;
         const int per_xcd = (total + 7) / 8;
-        const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-        if ((blockIdx.x >> 3) >= per_xcd || logical >= total) return;
+        const int bx = blockIdx.x % (per_xcd * 8);
+        const int logical = (bx & 7) * per_xcd + (bx >> 3);
+        if (logical >= total) return;
         constexpr int GM = 4;
         const int group = logical / (GM * p.ntiles);
         const int rest = logical - group * (GM * p.ntiles);
@@ -374,6 +377,7 @@ jl_gemm_f16(GemmParams p) {
     }
     const int m0 = mt * BM;
     const int n0 = nt * cols_per_tile;
+    const int split = blockIdx.x / (((p.ntiles * p.mtiles + 7) / 8) * 8);
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
     uint8_t *raw_ring = lds;
@@ -442,17 +446,19 @@ jl_gemm_f16(GemmParams p) {
         asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + ((c ^ ((r >> 1) & 7)) << 4);
     }
 
-    const int ksteps = p.k / BK;
+    const int ksteps = p.k / BK / p.splits;   // steps of this workgroup
+    const int kbase = split * ksteps;          // its first step
 
     // loads a thread issues per step (a Q4_K super-block header is re-fetched with each of its
     // four steps -- 16 bytes a row out of L2 -- so that the count is the same for every step)
     constexpr int LPS = NLW + NLA + (TYPE == JL_Q4_K ? 1 : 0);
     auto issue = [&](int s) {
         const int st = s % NS;
+        const int g = kbase + s;  // step index along the whole row
         uint8_t *rdst = raw_ring + st * RAWB;
         int64_t woff;
-        if constexpr (TYPE == JL_Q4_K) woff = (int64_t)(s >> 2) * 144 + (s & 3) * 32;
-        else woff = (int64_t)s * Raw<TYPE>::kRowBytes;
+        if constexpr (TYPE == JL_Q4_K) woff = (int64_t)(g >> 2) * 144 + (g & 3) * 32;
+        else woff = (int64_t)g * Raw<TYPE>::kRowBytes;
 #pragma unroll
         for (int j = 0; j < NLW; j++) {
             const uint8_t *src = wlive[j] ? wsrc[j] + woff : wsrc[j];
@@ -462,14 +468,14 @@ jl_gemm_f16(GemmParams p) {
                 __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(rdst + (j * 256 + wave * 64) * 4), 4, 0, 0);
         }
         if constexpr (TYPE == JL_Q4_K) {
-            const uint8_t *src = hlive ? hsrc + (int64_t)(s >> 2) * 144 : hsrc;
+            const uint8_t *src = hlive ? hsrc + (int64_t)(g >> 2) * 144 : hsrc;
             uint8_t *hdst = hdr_ring + (s % NS) * HDR_BYTES;
             __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(hdst + wave * 64 * 16), 16, 0, 0);
         }
         uint8_t *adst = a_ring + st * ABYTES;
 #pragma unroll
         for (int j = 0; j < NLA; j++)
-            __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)s * 128),
+            __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)g * 128),
                                              (lvoid *)(adst + (j * 256 + wave * 64) * 16), 16, 0, 0);
     };
 
@@ -480,7 +486,7 @@ jl_gemm_f16(GemmParams p) {
         half8 v[4];
         const uint32_t rr = raw0 + (s % NS) * RAWB + drow * Raw<TYPE>::kRowBytes;
         const uint32_t hh = hdr0 + (s % NS) * HDR_BYTES + drow * 16;
-        decode_half_slice<TYPE>(rr, hh, dhalf, (s & 3) * 2 + dhalf, v);
+        decode_half_slice<TYPE>(rr, hh, dhalf, ((kbase + s) & 3) * 2 + dhalf, v);
         lds_write_4xh8(w16_0 + (s & 1) * W16_BYTES + drow * W16_STRIDE + dhalf * 64, v);
     };
 
@@ -577,6 +583,23 @@ jl_gemm_f16(GemmParams p) {
     // The weight fragment went in as the MFMA's row operand, so a lane holds four consecutive
     // output columns 4 * (lane / 16) .. + 3 of activation row lane % 16 of each block: one
     // 16-byte store per block.
+    if (p.splits > 1) {
+        // partial sums of this run of K: plain 16-byte stores into the scratch plane of this split;
+        // jl_gemm_reduce adds the planes in order and applies the epilogue
+        const int64_t plane = (int64_t)p.mtiles * BM * p.ntiles * BN;
+        float *pp = p.partial + split * plane;
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+            const int m = m0 + wm * TM + i * 16 + (lane & 15);
+            float *prow = pp + (int64_t)m * (p.ntiles * BN) + nt * BN;
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+                const int c = brow[j] + (lane >> 4) * 4;  // column inside the 128-wide tile
+                *(float4 *)(prow + c) = float4{acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MB; i++) {
         const int m = m0 + wm * TM + i * 16 + (lane & 15);
@@ -619,16 +642,75 @@ jl_gemm_f16(GemmParams p) {
     }
 }
 
+// Sums the split-K planes in split order (so the result does not depend on scheduling) and
+// applies row scale and epilogue.  One thread per output element.
+__global__ void __launch_bounds__(256)
+jl_gemm_reduce(const float *__restrict__ partial, const float *__restrict__ row_scale,
+               float *__restrict__ C, int rows, int n_total, int ntiles, int64_t plane, int splits,
+               int64_t ldo, int64_t col_offset, int epilogue) {
+    const int col = blockIdx.x * blockDim.x + threadIdx.x;
+    const int m = blockIdx.y;
+    if (col >= n_total || m >= rows) return;
+    const int64_t width = (int64_t)ntiles * BN;
+    float *out = C + (int64_t)m * ldo + col_offset + col;
+    if (epilogue == JL_SWIGLU) {
+        // tile t holds gate columns 64 t .. 64 t + 63 in its first half and the up columns after
+        const int64_t g = (int64_t)m * width + (col >> 6) * BN + (col & 63);
+        float sg = 0.f, su = 0.f;
+        for (int z = 0; z < splits; z++) {
+            sg += partial[z * plane + g];
+            su += partial[z * plane + g + 64];
+        }
+        const float rs = row_scale[m];
+        *out = gemm_swiglu(sg * rs, su * rs);
+    } else {
+        const int64_t g = (int64_t)m * width + col;
+        float sum = 0.f;
+        for (int z = 0; z < splits; z++) sum += partial[z * plane + g];
+        sum *= row_scale[m];
+        if (epilogue == JL_RESIDUAL) *out += sum;
+        else *out = sum;
+    }
+}
+
 size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
 
-size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int math) {
-    size_t padded = round_up((size_t)max_rows, 128);
+namespace {
+
+// Split-K factor for a skinny call (at most 64 activation rows): enough workgroups to cover the
+// chip, at least 8 steps (512 columns) per split, and partial-sum traffic (written once, read once)
+// no larger than the weight bytes themselves.  A divisor of the step count.
+int choose_splits(int rows, int k, int ntiles, int row_bytes, int compute_units) {
+    if (rows > 64) return 1;
+    const int ksteps = k / BK;
+    const int padded = rows <= 32 ? 32 : 64;
+    int want = (2 * compute_units + ntiles - 1) / ntiles;
+    int by_steps = ksteps / 8;
+    int by_traffic = row_bytes / (8 * padded);
+    int s = want < by_steps ? want : by_steps;
+    if (by_traffic < s) s = by_traffic;
+    if (s < 1) s = 1;
+    while (ksteps % s) s--;
+    return s;
+}
+
+size_t a16_bytes(int64_t rows, int64_t cols) { return round_up(round_up((size_t)rows, 128) * (size_t)cols * 2, 256); }
+size_t scale_bytes(int64_t rows) { return round_up(round_up((size_t)rows, 128) * 4, 256); }
+
+}  // namespace
+
+// Workspace: fp16 activations | row scales | split-K planes.  The planes are bounded by the
+// traffic rule in choose_splits: splits * padded_rows <= row_bytes / 8, so splits * padded_rows *
+// columns * 4 <= columns * row_bytes / 2 with row_bytes <= 34 * cols / 32.
+size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_cols, int math) {
     if (math == JL_MATH_INT8) {
+        size_t padded = round_up((size_t)max_rows, 128);
         return round_up(padded * (size_t)cols, 256) + round_up(padded * (size_t)(cols / 32) * 4, 256);
     }
-    return round_up(padded * (size_t)cols * 2, 256) + round_up(padded * 4, 256);
+    size_t planes = round_up(round_up((size_t)out_cols, 128) * (size_t)cols * 17 / 32 + 64 * 128 * 4, 256);
+    return a16_bytes(max_rows, cols) + scale_bytes(max_rows) + planes;
 }
 
 namespace {
@@ -649,16 +731,29 @@ int launch_gemm(jl_context *ctx, const GemmParams &p, dim3 grid) {
 }
 
 template <int TYPE>
-int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows) {
+int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows, float *planes, size_t plane_bytes) {
     const int cols_per_tile = p.epilogue == JL_SWIGLU ? BN / 2 : BN;
     p.ntiles = (p.n_total + cols_per_tile - 1) / cols_per_tile;
     const int bm = rows <= 32 ? 32 : rows <= 64 ? 64 : 128;
     p.mtiles = (rows + bm - 1) / bm;
-    // one workgroup per tile, padded so that each of the 8 XCDs gets the same number of launch slots
-    const unsigned grid = (unsigned)((p.ntiles * p.mtiles + 7) / 8 * 8);
-    if (bm == 32) return launch_gemm<TYPE, 32, 6>(ctx, p, dim3(grid));
-    if (bm == 64) return launch_gemm<TYPE, 64, 6>(ctx, p, dim3(grid));
-    return launch_gemm<TYPE, 128, 4>(ctx, p, dim3(grid));
+    p.splits = choose_splits(rows, p.k, p.ntiles, p.row_bytes, ctx->compute_units);
+    const int64_t plane = (int64_t)p.mtiles * bm * p.ntiles * BN;
+    if (p.splits > 1 && (size_t)p.splits * plane * 4 > plane_bytes) p.splits = 1;
+    p.partial = planes;
+    // one workgroup per (tile, split); the tile count is padded to a multiple of 8 so that each XCD
+    // gets the same number of launch slots per split
+    const unsigned per_split = (unsigned)((p.ntiles * p.mtiles + 7) / 8 * 8);
+    const dim3 grid(per_split * p.splits);
+    int st;
+    if (bm == 32) st = launch_gemm<TYPE, 32, 6>(ctx, p, grid);
+    else if (bm == 64) st = launch_gemm<TYPE, 64, 6>(ctx, p, grid);
+    else st = launch_gemm<TYPE, 128, 4>(ctx, p, grid);
+    if (st != JL_OK || p.splits == 1) return st;
+    hipLaunchKernelGGL(jl_gemm_reduce, dim3((p.n_total + 255) / 256, rows), dim3(256), 0, ctx->stream,
+                       planes, p.row_scale, p.C, rows, p.n_total, p.ntiles, plane, p.splits, p.ldo,
+                       p.col_offset, p.epilogue);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
 }
 
 }  // namespace
@@ -666,7 +761,6 @@ int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows) {
 int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
                    int epilogue, int math, void *workspace, size_t workspace_bytes) {
-    (void)workspace_bytes;
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     if (math == JL_MATH_INT8) {
@@ -681,8 +775,10 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const int padded = (int)round_up((size_t)rows, 128);
     // the workspace was sized for `batch` rows, of which `rows` <= batch are converted
     _Float16 *A = (_Float16 *)workspace;
-    float *row_scale =
-        (float *)((uint8_t *)workspace + round_up(round_up((size_t)batch, 128) * (size_t)k * 2, 256));
+    float *row_scale = (float *)((uint8_t *)workspace + a16_bytes(batch, k));
+    const size_t head = a16_bytes(batch, k) + scale_bytes(batch);
+    float *planes = (float *)((uint8_t *)workspace + head);
+    const size_t plane_bytes = workspace_bytes > head ? workspace_bytes - head : 0;
 
     hipLaunchKernelGGL(jl_rows_to_f16, dim3((padded + 3) / 4), dim3(256), 0, ctx->stream, X, A,
                        row_scale, rows, padded, k);
@@ -709,9 +805,9 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     p.row_bytes = k / jl_block_elems(type) * jl_block_bytes(type);
 
     switch (type) {
-        case JL_Q8_0: return launch_gemm_type<JL_Q8_0>(ctx, p, rows);
-        case JL_Q4_0: return launch_gemm_type<JL_Q4_0>(ctx, p, rows);
-        case JL_Q4_K: return launch_gemm_type<JL_Q4_K>(ctx, p, rows);
+        case JL_Q8_0: return launch_gemm_type<JL_Q8_0>(ctx, p, rows, planes, plane_bytes);
+        case JL_Q4_0: return launch_gemm_type<JL_Q4_0>(ctx, p, rows, planes, plane_bytes);
+        case JL_Q4_K: return launch_gemm_type<JL_Q4_K>(ctx, p, rows, planes, plane_bytes);
         default:
             return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
     }

@@ -94,13 +94,17 @@ class QuantizedProjections:
 class QuantizedBatchProjections:
     """Projections of ``batchSize`` activation rows at once (batched decode, batched prefill)."""
 
-    def __init__(self, context: Context, batchSize: int, max_cols: int, math: int = L.JL_MATH_DEFAULT):
+    def __init__(self, context: Context, batchSize: int, max_cols: int, max_out_cols: int = 0,
+                 math: int = L.JL_MATH_DEFAULT):
+        """``max_cols`` is the longest row any projection reads, ``max_out_cols`` the most output
+        columns one call produces (gate + up rows for a fused gate/up); together they size the
+        workspace once, before anything runs (Implementation.needs)."""
         self.context = context
         self.batchSize = int(batchSize)
         self.math = math
         self._lib = context._lib
         self._max_cols = int(max_cols)
-        nbytes = self._lib.jl_gemm_workspace_bytes(self.batchSize, self._max_cols, math)
+        nbytes = self._lib.jl_gemm_workspace_bytes(self.batchSize, self._max_cols, int(max_out_cols), math)
         self.workspace = DeviceBuffer(context, max(nbytes, 256))
 
     def workspace_bytes(self) -> int:

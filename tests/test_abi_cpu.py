@@ -44,10 +44,14 @@ def test_argument_checks_need_no_device(lib):
     assert lib.jl_sync(None) == L.JL_ERR_INVALID
     assert b"context is null" in lib.jl_last_error()
     assert lib.jl_gemv(None, None, None, None, 0) == L.JL_ERR_INVALID
-    assert lib.jl_gemm_workspace_bytes(0, 2048, 0) == 0
-    f16 = lib.jl_gemm_workspace_bytes(512, 2048, L.JL_MATH_F16)
+    assert lib.jl_gemm_workspace_bytes(0, 2048, 2048, 0) == 0
+    f16 = lib.jl_gemm_workspace_bytes(512, 2048, 0, L.JL_MATH_F16)
     assert f16 >= 512 * 2048 * 2 + 512 * 4 and f16 % 256 == 0
-    assert lib.jl_gemm_workspace_bytes(100, 2048, L.JL_MATH_F16) >= 128 * 2048 * 2
+    assert lib.jl_gemm_workspace_bytes(100, 2048, 0, L.JL_MATH_F16) >= 128 * 2048 * 2
+    # split-K planes grow with the output width, never beyond about half the weight bytes
+    wide = lib.jl_gemm_workspace_bytes(64, 4096, 12288, L.JL_MATH_F16)
+    assert f16 < wide <= 128 * 4096 * 2 + 1024 + 12288 * 4096 * 17 // 32 + (1 << 16)
+    assert lib.jl_gemm_workspace_bytes(64, 4096, 12288, L.JL_MATH_DEFAULT) == wide
 
 
 def test_without_a_device_context_creation_fails_loudly(lib):

@@ -34,7 +34,7 @@ def test_batch_projection_reference_fixture(ctx, t, what):
             X = FX.batch_activation(width)
             expected = O.matmul_batch(t, raw, X[:active], FX.D_PROBE, FX.N_PROBE)
             mag = magnitude(t, raw, X[:active], FX.D_PROBE, FX.N_PROBE)
-            proj = QuantizedBatchProjections(ctx, width, FX.N_PROBE)
+            proj = QuantizedBatchProjections(ctx, width, FX.N_PROBE, FX.D_PROBE)
             xd = ctx.from_numpy(X)
             for residual in (False, True):
                 out = ctx.float_array(width * FX.D_PROBE, fill=UNTOUCHED)
@@ -59,7 +59,7 @@ def test_batched_projection_matches_oracle(ctx, t, d, n, B):
     ref = O.matmul_batch(t, raw, X, d, n, O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256)
     w = ctx.load_weight(t, raw, d, n)
     out = ctx.float_array(B * d, fill=UNTOUCHED)
-    QuantizedBatchProjections(ctx, B, n).projection(ctx.from_numpy(X), out, w, n, d, False)
+    QuantizedBatchProjections(ctx, B, n, d).projection(ctx.from_numpy(X), out, w, n, d, False)
     ctx.sync()
     got = out.get().reshape(B, d)
     assert np.all(got != UNTOUCHED)
@@ -79,7 +79,7 @@ def test_batched_row_is_the_single_vector_result(ctx):
     x = synthetic.activations(n, seed=72)
     X = np.tile(x, (B, 1))
     out = ctx.float_array(B * d)
-    QuantizedBatchProjections(ctx, B, n).projection(ctx.from_numpy(X), out,
+    QuantizedBatchProjections(ctx, B, n, d).projection(ctx.from_numpy(X), out,
                                                     ctx.load_weight(O.Q8_0, raw, d, n), n, d, False)
     ctx.sync()
     got = out.get().reshape(B, d)
@@ -98,7 +98,7 @@ def test_prefill_fused_qkv_side_by_side(ctx, t, dq, dkv, n, T):
     ws = [ctx.load_weight(t, r, d, n) for r, d in zip(raws, dims)]
     ld = sum(dims)
     out = ctx.float_array(T * ld, fill=UNTOUCHED)
-    QuantizedBatchProjections(ctx, T, n).fusedQKV(ctx.from_numpy(X), out, *ws)
+    QuantizedBatchProjections(ctx, T, n, ld).fusedQKV(ctx.from_numpy(X), out, *ws)
     ctx.sync()
     got = out.get().reshape(T, ld)
     col = 0
@@ -121,7 +121,7 @@ def test_batched_gate_up(ctx, t, d, n, T):
     u = O.matmul_batch(t, r3, X, d, n)
     ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(T, d)
     hb = ctx.float_array(T * d, fill=UNTOUCHED)
-    QuantizedBatchProjections(ctx, T, n).gateUp(ctx.from_numpy(X), hb, ctx.load_weight(t, r1, d, n),
+    QuantizedBatchProjections(ctx, T, n, 2 * d).gateUp(ctx.from_numpy(X), hb, ctx.load_weight(t, r1, d, n),
                                                 ctx.load_weight(t, r3, d, n), n, d)
     ctx.sync()
     got = hb.get().reshape(T, d)
@@ -142,7 +142,7 @@ def test_huge_activation_rows_stay_finite(ctx):
     X[2] *= 1e-6
     ref = O.matmul_batch(O.Q8_0, raw, X, d, n)
     out = ctx.float_array(B * d)
-    QuantizedBatchProjections(ctx, B, n).projection(ctx.from_numpy(X), out,
+    QuantizedBatchProjections(ctx, B, n, d).projection(ctx.from_numpy(X), out,
                                                     ctx.load_weight(O.Q8_0, raw, d, n), n, d, False)
     ctx.sync()
     got = out.get().reshape(B, d)
