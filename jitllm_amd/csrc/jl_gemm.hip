@@ -29,28 +29,31 @@ constexpr int kMaxWeights = 8;
 
 // ---- activations: fp32 -> fp16 with a power-of-two row scale --------------------------------
 
-// One wave per row: scale = the power of two that brings the row's largest magnitude into
-// [2^11, 2^12); a16 = half(x / scale) (the division is exact).
+// One workgroup per row: scale = the power of two that brings the row's largest magnitude into
+// [2^11, 2^12); a16 = half(x / scale) (the division is exact).  Rows past `rows` are zero-filled.
 __global__ void __launch_bounds__(256)
 jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__restrict__ row_scale,
-               int rows, int padded_rows, int k) {
-    int row = blockIdx.x * 4 + threadIdx.x / JL_WAVE;
-    int lane = threadIdx.x & (JL_WAVE - 1);
-    if (row >= padded_rows) return;
+               int rows, int k) {
+    __shared__ float wave_max[4];
+    const int row = blockIdx.x;
+    const int tid = threadIdx.x;
     _Float16 *a = A + (int64_t)row * k;
     if (row >= rows) {
-        for (int i = lane * 4; i < k; i += JL_WAVE * 4) *(half4 *)(a + i) = half4{0, 0, 0, 0};
-        if (lane == 0) row_scale[row] = 1.f;
+        for (int i = tid * 4; i < k; i += 1024) *(half4 *)(a + i) = half4{0, 0, 0, 0};
+        if (tid == 0) row_scale[row] = 1.f;
         return;
     }
     const float *x = X + (int64_t)row * k;
     float amax = 0.f;
-    for (int i = lane * 4; i < k; i += JL_WAVE * 4) {
+    for (int i = tid * 4; i < k; i += 1024) {
         float4 v = *(const float4 *)(x + i);
         amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, JL_WAVE));
+    if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
     // Every row is brought to [2^11, 2^12) at its largest magnitude: huge rows stay finite in
     // fp16, tiny rows keep their bits out of fp16's subnormal range, and the power of two is
     // undone exactly in the epilogue.
@@ -62,13 +65,13 @@ jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__r
         scale = ldexpf(1.f, e - 12);
         inv = ldexpf(1.f, 12 - e);
     }
-    for (int i = lane * 4; i < k; i += JL_WAVE * 4) {
+    for (int i = tid * 4; i < k; i += 1024) {
         float4 v = *(const float4 *)(x + i);
         half4 h = {(_Float16)(v.x * inv), (_Float16)(v.y * inv), (_Float16)(v.z * inv),
                    (_Float16)(v.w * inv)};
         *(half4 *)(a + i) = h;
     }
-    if (lane == 0) row_scale[row] = scale;
+    if (tid == 0) row_scale[row] = scale;
 }
 
 // ---- LDS access by hand ----------------------------------------------------------------------
@@ -772,7 +775,8 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     for (int i = 0; i < count; i++)
         JL_REQUIRE(((uintptr_t)weights[i]->blocks & 15) == 0, "jl_gemm: weight %d is not 16-byte aligned", i);
     const int rows = (int)active_rows;
-    const int padded = (int)round_up((size_t)rows, 128);
+    // rows are padded to the row tile the kernel will use, never beyond what the workspace holds
+    const int padded = (int)round_up((size_t)rows, rows <= 32 ? 32 : rows <= 64 ? 64 : 128);
     // the workspace was sized for `batch` rows, of which `rows` <= batch are converted
     _Float16 *A = (_Float16 *)workspace;
     float *row_scale = (float *)((uint8_t *)workspace + a16_bytes(batch, k));
@@ -780,8 +784,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     float *planes = (float *)((uint8_t *)workspace + head);
     const size_t plane_bytes = workspace_bytes > head ? workspace_bytes - head : 0;
 
-    hipLaunchKernelGGL(jl_rows_to_f16, dim3((padded + 3) / 4), dim3(256), 0, ctx->stream, X, A,
-                       row_scale, rows, padded, k);
+    hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
     JL_HIP(hipGetLastError());
 
     GemmParams p{};
