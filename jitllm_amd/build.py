@@ -6,7 +6,7 @@ import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-LIB = os.environ.get("JITLLM_HIP_LIBRARY") or os.path.join(HERE, "lib", "libjitllm_hip.so")
+LIB = os.path.join(HERE, "lib", "libjitllm_hip.so")
 
 
 def build(force: bool = True, jobs: int = 8) -> str:

@@ -24,8 +24,6 @@
 #include "jl_device.h"
 #include "jl_internal.h"
 
-#include <stdlib.h>
-
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -49,7 +47,6 @@ struct GemvParams {
     int row_bytes;
     int epilogue;
     int stages;     // depth of the LDS tile ring (2..8)
-    int debug;
 };
 
 template <int TYPE> struct Traits;
@@ -286,7 +283,6 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     constexpr int L = X4 + 1;                     // plus one 4-byte load
     constexpr int SLICE = X4 * 16 + 4;            // bytes of a tile one thread brings in
 
-    if (p.debug == 1) return;
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int wave = tid / JL_WAVE;
@@ -370,7 +366,6 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     for (; issued < p.stages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
     wait_vm_tiles<L>(issued);
     __builtin_amdgcn_s_barrier();
-    if (p.debug == 2) { JL_WAIT_VM(0); return; }
 
     float x[64];
     float sx[2] = {0.f, 0.f};
@@ -456,7 +451,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         if (it > 0) finish(tile - gridDim.x, (it - 1) & 1);
 
         float v = 0.f;
-        if (active && p.debug != 3) v = slice_dot_lds<TYPE>(ring0 + (it % p.stages) * stage_bytes, r, s, p.row_bytes, x, sx);
+        if (active) v = slice_dot_lds<TYPE>(ring0 + (it % p.stages) * stage_bytes, r, s, p.row_bytes, x, sx);
         if (p.Sp >= 2) v += quad_xor1(v);
         if (p.Sp >= 4) v += quad_xor2(v);
         if (r < p.R && (p.Sp < 4 ? s == 0 : (s & 3) == 0)) {
@@ -571,8 +566,6 @@ template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds) {
     auto fn = jl_gemv_tiles<TYPE, DUAL>;
     int per_cu = blocks_per_cu((const void *)fn, ctx->device, threads, lds);
-    static const int cap = getenv("JL_GEMV_WGS_PER_CU") ? atoi(getenv("JL_GEMV_WGS_PER_CU")) : 0;
-    if (cap > 0 && per_cu > cap) per_cu = cap;
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
     if (grid > total) grid = total;
@@ -655,13 +648,10 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     const int stage_bytes = threads * slice;
     const int x_bytes = (S * 17 + threads - 1) / threads * threads * 16;  // 17 slots per slice
     const int x_extra = x_bytes <= stage_bytes ? 0 : x_bytes;
-    // Ring depth: few tiles per workgroup want all of them in flight at once (deep ring, fewer
-    // workgroups per compute unit); long streams want many workgroups with a short ring.
-    static const int forced = getenv("JL_GEMV_STAGES") ? atoi(getenv("JL_GEMV_STAGES")) : 0;
-    int stages = forced >= 2 && forced <= 8 ? forced : 2;
+    // Ring depth 2: measured on every benchmark shape, a deeper ring at the lower occupancy its LDS
+    // footprint forces is slower than two stages with up to four workgroups per compute unit.
+    const int stages = 2;
     p.stages = stages;
-    static const int dbg = getenv("JL_GEMV_DEBUG") ? atoi(getenv("JL_GEMV_DEBUG")) : 0;
-    p.debug = dbg;
     const int lds = kPartialBytes + stages * stage_bytes + x_extra;
 
     switch (type) {
