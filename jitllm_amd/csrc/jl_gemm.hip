@@ -198,8 +198,8 @@ __device__ __forceinline__ void dword_to_h4(uint32_t v, h2 bias, h2 d, _Float16 
     dst[3] = hi[1];
 }
 
-// One thread decodes the 32 elements (row, half) of the 64-wide slice from the raw tile in LDS.
-// raw_row = LDS address of the row's raw slice (Q8_0 68 B, Q4_0 36 B; Q4_K: 32 nibble bytes, with
+// One thread decodes the 32 elements (row, half) of a 64-wide slice from the raw stage in LDS.
+// raw_row = LDS address of the slice's raw bytes (Q8_0 68 B, Q4_0 36 B; Q4_K: 32 nibble bytes, with
 // hdr = LDS address of the super-block's 16-byte header and sub = sub-block index 0..7).
 template <int TYPE>
 __device__ __forceinline__ void decode_half_slice(uint32_t raw_row, uint32_t hdr, int half, int sub,
@@ -304,25 +304,41 @@ struct GemmParams {
 };
 
 constexpr int BN = 128, BK = 64;
+constexpr int SUPER = 4;                       // 64-column steps per raw-weight stage (256 columns)
 constexpr int W16_STRIDE = 144;                // bytes per decoded row: 64 halfs + 16 bytes of padding
 constexpr int W16_BYTES = BN * W16_STRIDE;     // 18432
-constexpr int HDR_BYTES = 256 * 16;            // one Q4_K header slot per thread
 
+// Raw weight bytes of one row for 256 columns -- always a whole number of 16-byte chunks, and
+// 16-byte aligned in the file layout, which is what lets the stage be fetched with 128-bit loads:
+// Q8_0 8 blocks = 272 B, Q4_0 8 blocks = 144 B, Q4_K one super-block = 144 B.
 template <int TYPE> struct Raw;
-template <> struct Raw<JL_Q8_0> { static constexpr int kRowBytes = 68, kLoads = 9; };   // 2176 dwords
-template <> struct Raw<JL_Q4_0> { static constexpr int kRowBytes = 36, kLoads = 5; };   // 1152 dwords
-template <> struct Raw<JL_Q4_K> { static constexpr int kRowBytes = 32, kLoads = 1; };   // 256 x 16 B
+template <> struct Raw<JL_Q8_0> { static constexpr int kRowBytes = 272, kStepBytes = 68; };
+template <> struct Raw<JL_Q4_0> { static constexpr int kRowBytes = 144, kStepBytes = 36; };
+template <> struct Raw<JL_Q4_K> { static constexpr int kRowBytes = 144, kStepBytes = 32; };
 
-// bytes of one raw-weight stage: every one of the 256 threads' load slots has a place of its own
-template <int TYPE>
-constexpr int raw_stage_bytes() {
-    return Raw<TYPE>::kLoads * 256 * (TYPE == JL_Q4_K ? 16 : 4);
+// 128-bit loads per thread (256 producer threads) for one raw stage, and the stage's LDS footprint
+// (every load slot has a place of its own, including the few past the last row)
+template <int TYPE> constexpr int raw_loads() { return (BN * Raw<TYPE>::kRowBytes / 16 + 255) / 256; }
+template <int TYPE> constexpr int raw_stage_bytes() { return raw_loads<TYPE>() * 256 * 16; }
+
+// Activation stages: as many as the 160 KB of LDS leave room for (the Q8_0 raw stages are larger).
+template <int TYPE, int BM> constexpr int a_stages() {
+    return BM == 128 && TYPE == JL_Q8_0 ? 3 : 5;
 }
 
-template <int TYPE, int BM, int NS>
+// Loads that may still be in flight when step s = 4 u + q is awaited (steady state): everything
+// issued after the youngest load the step needs.  Producers issue, in iteration i (after its
+// barrier), first the next raw stage if i % 4 == 0 (RL loads) and then activation step i + AHEAD
+// (NLA loads).  Step s needs activation step s (iteration s - AHEAD) and the raw stage of step s + 1
+// (iteration 4 u - 4, or 4 u when q == 3).
+constexpr int allowed_in_flight(int q, int AHEAD, int NLA, int RL) {
+    if (q == 3 && AHEAD > 3) return NLA + 2 * NLA;  // the raw stage opened at q == 0 is the youngest need
+    return (AHEAD - 1) * NLA + ((q >= 1 && q < AHEAD) ? RL : 0);
+}
+
+template <int TYPE, int BM>
 constexpr int gemm_lds_bytes() {
-    return NS * raw_stage_bytes<TYPE>() + (TYPE == JL_Q4_K ? NS * HDR_BYTES : 0) +
-           NS * BM * 128 + 2 * W16_BYTES;
+    return 2 * raw_stage_bytes<TYPE>() + a_stages<TYPE, BM>() * BM * 128 + 2 * W16_BYTES;
 }
 
 // Workgroup: 512 threads = 8 waves, two per SIMD, split by role so that one role's waits are
@@ -334,15 +350,22 @@ constexpr int gemm_lds_bytes() {
 //   BM <= 64: consumer waves 1 x 4, wave tile BM x 32
 // For JL_SWIGLU the 128 tile columns are 64 gate rows followed by the 64 up rows of the same 64
 // outputs; a wave's column blocks are arranged so that it holds gate and up of the same outputs.
-template <int TYPE, int BM, int NS>
+//
+// Operand movement.  Raw weights: one stage = 128 rows x 256 columns, fetched with 128-bit LDS-DMA
+// loads once per four steps (two stages).  Activations: one stage = BM rows x 64 columns of fp16,
+// 16-byte chunks XOR-swizzled by row so that fragment reads are bank-conflict free, fetched every
+// step (three or four stages).  Decoded weights: two buffers of 128 x 64 fp16.
+template <int TYPE, int BM>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 jl_gemm_f16(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int RAWB = raw_stage_bytes<TYPE>();
-    static_assert(RAWB >= BN * Raw<TYPE>::kRowBytes, "raw stage too small");
-    static_assert(BM == 32 || BM == 64 || BM == 128, "row tile");
-    constexpr int NLW = Raw<TYPE>::kLoads;
-    constexpr int NLA = BM * 8 / 256;
+    constexpr int RB = Raw<TYPE>::kRowBytes;
+    constexpr int CPR = RB / 16;            // 16-byte chunks per raw row
+    constexpr int RL = raw_loads<TYPE>();   // raw loads per thread and stage
+    constexpr int NSA = a_stages<TYPE, BM>();
+    constexpr int AHEAD = NSA - 1;          // activation steps in flight ahead of the one in use
+    constexpr int NLA = BM * 8 / 256;       // activation loads per thread and step
     constexpr int ABYTES = BM * 128;
     constexpr int WM = BM == 128 ? 2 : 1;
     constexpr int WN = 4 / WM;
@@ -350,6 +373,7 @@ jl_gemm_f16(GemmParams p) {
     constexpr int TN = BN / WN;       // wave tile columns
     constexpr int MB = TM / 16;       // 16 x 16 blocks per wave along M
     constexpr int NB = TN / 16;
+    static_assert(BM == 32 || BM == 64 || BM == 128, "row tile");
 
     // the role and the wave index are the same for every lane of a wave: keep them in scalar
     // registers so that the pipeline's bookkeeping (and the waits it selects) stays scalar code
@@ -361,144 +385,158 @@ jl_gemm_f16(GemmParams p) {
     const int wm = wave / WN, wn = wave % WN;
     const bool swiglu = p.epilogue == JL_SWIGLU;
     const int cols_per_tile = swiglu ? BN / 2 : BN;
-    // Tile order.  Workgroups go to the 8 XCDs round-robin by launch index, and each XCD has an L2
-    // of its own: give every XCD one contiguous run of the tile list, ordered so that the tiles it
-    // works on at any moment are a 4 (row tiles) x 8 (column tiles) patch whose operands fit that L2.
-    int mt, nt;
-    {
-        const int total = p.ntiles * p.mtiles;
-        const int per_xcd = (total + 7) / 8;
-        const int bx = blockIdx.x % (per_xcd * 8);
-        const int logical = (bx & 7) * per_xcd + (bx >> 3);
-        if (logical >= total) return;
+    const int total_tiles = p.ntiles * p.mtiles;
+    const int per_xcd = (total_tiles + 7) / 8;
+    const int usteps = p.k / (BK * SUPER) / p.splits;  // raw stages (256 columns) per work item
+    const int ksteps = usteps * SUPER;
+
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
+    uint8_t *raw_ring = lds;
+    uint8_t *a_ring = lds + 2 * RAWB;
+    const uint32_t raw0 = lds0;
+    const uint32_t a0 = lds0 + 2 * RAWB;
+    const uint32_t w16_0 = a0 + NSA * ABYTES;
+
+    // Persistent workgroups: the launch has one workgroup per compute unit (or fewer) and each walks
+    // work items wg, wg + G, ... -- a work item is one (tile, split).  Producers run straight on
+    // into the next item's first loads while the consumers are still storing the previous tile, so
+    // the load latency at the head of a tile and the stores at its tail overlap.
+    // Item order: workgroups go to the 8 XCDs round-robin by launch index and each XCD has an L2 of
+    // its own, so XCD x takes the x-th contiguous eighth of the tile list, ordered so that the tiles
+    // its workgroups hold at any moment are a 4 (row tiles) x 8 (column tiles) patch.
+    const int xcd = blockIdx.x & 7;
+    const int slot = blockIdx.x >> 3;
+    const int slots = (gridDim.x + 7) >> 3;  // workgroups per XCD
+    const int items = per_xcd * p.splits;
+
+    // (tile row, tile column, split) of a work item; false when the item is padding
+    auto locate = [&](int item, int &mt, int &nt, int &split) -> bool {
+        split = item / per_xcd;
+        const int logical = xcd * per_xcd + (item - split * per_xcd);
+        if (logical >= total_tiles) return false;
         constexpr int GM = 4;
         const int group = logical / (GM * p.ntiles);
         const int rest = logical - group * (GM * p.ntiles);
         const int rows_in_group = p.mtiles - group * GM < GM ? p.mtiles - group * GM : GM;
         nt = rest / rows_in_group;
         mt = group * GM + rest - nt * rows_in_group;
-    }
-    const int m0 = mt * BM;
-    const int n0 = nt * cols_per_tile;
-    const int split = blockIdx.x / (((p.ntiles * p.mtiles + 7) / 8) * 8);
+        return true;
+    };
 
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
-    uint8_t *raw_ring = lds;
-    uint8_t *hdr_ring = lds + NS * RAWB;
-    uint8_t *a_ring = hdr_ring + (TYPE == JL_Q4_K ? NS * HDR_BYTES : 0);
-    const uint32_t raw0 = lds0;
-    const uint32_t hdr0 = lds0 + NS * RAWB;
-    const uint32_t a0 = hdr0 + (TYPE == JL_Q4_K ? NS * HDR_BYTES : 0);
-    const uint32_t w16_0 = a0 + NS * ABYTES;
+    // The two roles are separate loops (with the same barriers in the same order) rather than
+    // branches inside one loop: a wave only ever runs one of them, and written this way the
+    // register allocator sees that their states are never live together.
+    //
+    // Local step s = 4 u + q uses raw stage u and activation stage s.  Producers issue
+    //   at the head of an item   raw(0), A(0 .. AHEAD - 1)
+    //   iteration s              [raw(u + 1) when q == 0]  A(s + AHEAD)     -- after the barrier of s
+    // and before the barrier of s they wait until only allowed_in_flight(q) loads are outstanding.
+    // Barriers per item: one after the head loads, one per step, one at the end (every LDS read of
+    // the item is done before the next item's loads may land).
+    static_assert(AHEAD >= 2 && AHEAD <= 4, "the wait table covers 2..4 steps of look-ahead");
 
-    // source row of tile row r (null past the last output column); the weight table is walked with
-    // constant indices so that it stays in scalar registers
-    auto row_ptr = [&](int r) -> const uint8_t * {
-        if (swiglu) {
-            const int vcol = n0 + (r & 63);
-            const uint8_t *base = r >= 64 ? p.w[1] : p.w[0];
-            return vcol < p.n_total ? base + (int64_t)vcol * p.row_bytes : nullptr;
-        }
-        const int vcol = n0 + r;
-        if (vcol >= p.n_total) return nullptr;
-        const uint8_t *base = p.w[0];
-        int first = 0;
+    if (producer) {
+        const int drow = tid & 127;  // decode role: tile row tid % 128, half tid / 128
+        const int dhalf = tid >> 7;
+        for (int item = slot; item < items; item += slots) {
+            int mt, nt, split;
+            if (!locate(item, mt, nt, split)) continue;
+            const int m0 = mt * BM;
+            const int n0 = nt * cols_per_tile;
+            const int ubase = split * usteps;  // first raw stage of this item
+
+            // source row of tile row r (null past the last output column); the weight table is
+            // walked with constant indices so that it stays in scalar registers
+            auto row_ptr = [&](int r) -> const uint8_t * {
+                if (swiglu) {
+                    const int vcol = n0 + (r & 63);
+                    const uint8_t *base = r >= 64 ? p.w[1] : p.w[0];
+                    return vcol < p.n_total ? base + (int64_t)vcol * p.row_bytes : nullptr;
+                }
+                const int vcol = n0 + r;
+                if (vcol >= p.n_total) return nullptr;
+                const uint8_t *base = p.w[0];
+                int first = 0;
 #pragma unroll
-        for (int i = 1; i < kMaxWeights; i++) {
-            if (i < p.count && vcol >= p.w_begin[i]) {
-                base = p.w[i];
-                first = p.w_begin[i];
+                for (int i = 1; i < kMaxWeights; i++) {
+                    if (i < p.count && vcol >= p.w_begin[i]) {
+                        base = p.w[i];
+                        first = p.w_begin[i];
+                    }
+                }
+                return base + (int64_t)(vcol - first) * p.row_bytes;
+            };
+            // per-thread DMA sources (a slot with nothing to fetch re-reads the first weight bytes)
+            const uint8_t *wsrc[RL];
+            int wstep[RL];  // bytes a slot's source advances per raw stage: RB, or 0 for a dummy slot
+#pragma unroll
+            for (int j = 0; j < RL; j++) {
+                const int i = j * 256 + tid;
+                const int r = i / CPR;
+                const uint8_t *rp = r < BN ? row_ptr(r) : nullptr;
+                wstep[j] = rp ? RB : 0;
+                wsrc[j] = rp ? rp + (int64_t)ubase * RB + (i - r * CPR) * 16 : p.w[0];
             }
-        }
-        return base + (int64_t)(vcol - first) * p.row_bytes;
-    };
-
-    // ---- per-thread DMA sources (a slot with nothing to fetch re-reads the first weight bytes) ----
-    const uint8_t *wsrc[NLW];
-    bool wlive[NLW];
+            const uint8_t *asrc[NLA];
 #pragma unroll
-    for (int j = 0; j < NLW; j++) {
-        const int i = j * 256 + tid;
-        const uint8_t *rp = nullptr;
-        int within = 0;
-        if constexpr (TYPE == JL_Q4_K) {
-            rp = row_ptr(i >> 1);            // 2 sixteen-byte chunks per row
-            within = 16 + (i & 1) * 16;
-        } else {
-            constexpr int DW = Raw<TYPE>::kRowBytes / 4;
-            const int r = i / DW;
-            if (r < BN) rp = row_ptr(r);
-            within = (i - r * DW) * 4;
+            for (int j = 0; j < NLA; j++) {
+                const int i = j * 256 + tid;
+                const int r = i >> 3, c = i & 7;
+                asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k + (int64_t)ubase * (BK * SUPER)) +
+                          ((c ^ ((r >> 1) & 7)) << 4);
+            }
+            auto issue_raw = [&](int u) {  // raw stage u (local index) -> ring slot u & 1
+                uint8_t *dst = raw_ring + (u & 1) * RAWB;
+#pragma unroll
+                for (int j = 0; j < RL; j++)
+                    __builtin_amdgcn_global_load_lds((gvoid *)(wsrc[j] + (int64_t)u * wstep[j]),
+                                                     (lvoid *)(dst + (j * 256 + wave * 64) * 16), 16, 0, 0);
+            };
+            auto issue_a = [&](int s) {  // activation step s (local index) -> ring slot s % NSA
+                uint8_t *dst = a_ring + (s % NSA) * ABYTES;
+#pragma unroll
+                for (int j = 0; j < NLA; j++)
+                    __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)s * 128),
+                                                     (lvoid *)(dst + (j * 256 + wave * 64) * 16), 16, 0, 0);
+            };
+            auto dequant = [&](int s) {
+                half8 v[4];
+                const int u = s / SUPER, q = s % SUPER;
+                const uint32_t row = raw0 + (u & 1) * RAWB + drow * RB;
+                if constexpr (TYPE == JL_Q4_K)
+                    decode_half_slice<TYPE>(row + 16 + q * 32, row, dhalf, q * 2 + dhalf, v);
+                else
+                    decode_half_slice<TYPE>(row + q * Raw<TYPE>::kStepBytes, 0, dhalf, 0, v);
+                lds_write_4xh8(w16_0 + (s & 1) * W16_BYTES + drow * W16_STRIDE + dhalf * 64, v);
+            };
+
+            issue_raw(0);
+#pragma unroll
+            for (int a = 0; a < AHEAD; a++)
+                if (a < ksteps) issue_a(a);
+            JL_WAIT_VM(0);
+            __builtin_amdgcn_s_barrier();
+            dequant(0);
+            for (int s = 0; s < ksteps; s++) {
+                const int u = s / SUPER, q = s % SUPER;
+                const bool last = u + 1 == usteps;
+                // the wait takes an immediate: one case per position inside the raw stage
+                if (last) JL_WAIT_VM(0);
+                else if (q == 0) JL_WAIT_VM(allowed_in_flight(0, AHEAD, NLA, RL));
+                else if (q == 1) JL_WAIT_VM(allowed_in_flight(1, AHEAD, NLA, RL));
+                else if (q == 2) JL_WAIT_VM(allowed_in_flight(2, AHEAD, NLA, RL));
+                else JL_WAIT_VM(allowed_in_flight(3, AHEAD, NLA, RL));
+                __builtin_amdgcn_s_barrier();
+                if (q == 0 && !last) issue_raw(u + 1);
+                if (s + AHEAD < ksteps) issue_a(s + AHEAD);
+                if (s + 1 < ksteps) dequant(s + 1);
+            }
+            __builtin_amdgcn_s_barrier();
         }
-        wlive[j] = rp != nullptr;
-        wsrc[j] = wlive[j] ? rp + within : p.w[0];
+        return;
     }
-    const uint8_t *hsrc = nullptr;  // Q4_K: this thread's header source (rows 0..127)
-    bool hlive = false;
-    if constexpr (TYPE == JL_Q4_K) {
-        const uint8_t *rp = tid < BN ? row_ptr(tid) : nullptr;
-        hlive = rp != nullptr;
-        hsrc = hlive ? rp : p.w[0];
-    }
-    const uint8_t *asrc[NLA];
-#pragma unroll
-    for (int j = 0; j < NLA; j++) {
-        const int i = j * 256 + tid;
-        int r = i >> 3, c = i & 7;
-        if (r >= BM) r = 0;
-        asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + ((c ^ ((r >> 1) & 7)) << 4);
-    }
 
-    const int ksteps = p.k / BK / p.splits;   // steps of this workgroup
-    const int kbase = split * ksteps;          // its first step
-
-    // loads a thread issues per step (a Q4_K super-block header is re-fetched with each of its
-    // four steps -- 16 bytes a row out of L2 -- so that the count is the same for every step)
-    constexpr int LPS = NLW + NLA + (TYPE == JL_Q4_K ? 1 : 0);
-    auto issue = [&](int s) {
-        const int st = s % NS;
-        const int g = kbase + s;  // step index along the whole row
-        uint8_t *rdst = raw_ring + st * RAWB;
-        int64_t woff;
-        if constexpr (TYPE == JL_Q4_K) woff = (int64_t)(g >> 2) * 144 + (g & 3) * 32;
-        else woff = (int64_t)g * Raw<TYPE>::kRowBytes;
-#pragma unroll
-        for (int j = 0; j < NLW; j++) {
-            const uint8_t *src = wlive[j] ? wsrc[j] + woff : wsrc[j];
-            if constexpr (TYPE == JL_Q4_K)
-                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(rdst + (j * 256 + wave * 64) * 16), 16, 0, 0);
-            else
-                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(rdst + (j * 256 + wave * 64) * 4), 4, 0, 0);
-        }
-        if constexpr (TYPE == JL_Q4_K) {
-            const uint8_t *src = hlive ? hsrc + (int64_t)(g >> 2) * 144 : hsrc;
-            uint8_t *hdst = hdr_ring + (s % NS) * HDR_BYTES;
-            __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(hdst + wave * 64 * 16), 16, 0, 0);
-        }
-        uint8_t *adst = a_ring + st * ABYTES;
-#pragma unroll
-        for (int j = 0; j < NLA; j++)
-            __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)g * 128),
-                                             (lvoid *)(adst + (j * 256 + wave * 64) * 16), 16, 0, 0);
-    };
-
-    // ---- decode role: tile row tid % 128, half tid / 128 (uniform per wave) ----
-    const int drow = tid & 127;
-    const int dhalf = tid >> 7;
-    auto dequant = [&](int s) {
-        half8 v[4];
-        const uint32_t rr = raw0 + (s % NS) * RAWB + drow * Raw<TYPE>::kRowBytes;
-        const uint32_t hh = hdr0 + (s % NS) * HDR_BYTES + drow * 16;
-        decode_half_slice<TYPE>(rr, hh, dhalf, ((kbase + s) & 3) * 2 + dhalf, v);
-        lds_write_4xh8(w16_0 + (s & 1) * W16_BYTES + drow * W16_STRIDE + dhalf * 64, v);
-    };
-
-    floatx4 acc[MB][NB];
-#pragma unroll
-    for (int i = 0; i < MB; i++)
-#pragma unroll
-        for (int j = 0; j < NB; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
+    // ---- consumers ----
     // LDS row of each of the wave's column blocks
     int brow[NB];
 #pragma unroll
@@ -506,137 +544,112 @@ jl_gemm_f16(GemmParams p) {
         if (swiglu) brow[j] = (j / (NB / 2)) * 64 + wn * (TN / 2) + (j % (NB / 2)) * 16;
         else brow[j] = wn * TN + j * 16;
     }
+    for (int item = slot; item < items; item += slots) {
+        int mt, nt, split;
+        if (!locate(item, mt, nt, split)) continue;
+        const int m0 = mt * BM;
+        const int n0 = nt * cols_per_tile;
 
-    // A step is two 32-column halves.  The second half's fragment reads are in flight while the
-    // first half's MFMAs run.
-    half8 fa[2][MB], fb[2][NB];
-    auto issue_frags = [&](int s, int ks) {
-        const uint32_t abase = a0 + (s % NS) * ABYTES;
-        const uint32_t wbase = w16_0 + (s & 1) * W16_BYTES;
-        const int chunk = ks * 4 + (lane >> 4);
-        uint32_t aa[MB], ba[NB];
-#pragma unroll
-        for (int i = 0; i < MB; i++) {
-            const int r = wm * TM + i * 16 + (lane & 15);
-            aa[i] = abase + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4);
-        }
-#pragma unroll
-        for (int j = 0; j < NB; j++) ba[j] = wbase + (brow[j] + (lane & 15)) * W16_STRIDE + chunk * 16;
-        lds_issue_h8n<MB>(aa, fa[ks]);
-        lds_issue_h8n<NB>(ba, fb[ks]);
-    };
-    auto mfma_half = [&](int ks) {
+        floatx4 acc[MB][NB];
 #pragma unroll
         for (int i = 0; i < MB; i++)
 #pragma unroll
-            for (int j = 0; j < NB; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
-    };
-    auto consume = [&](int s) {
-        issue_frags(s, 0);
-        lds_wait_frags<MB, NB>(fa[0], fb[0]);
-        issue_frags(s, 1);
-        mfma_half(0);
-        lds_wait_frags<MB, NB>(fa[1], fb[1]);
-        mfma_half(1);
-    };
+            for (int j = 0; j < NB; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // ---- pipeline ----
-    // Step s occupies operand stage s % NS.  Producers keep NS - 1 steps of loads in flight and
-    // decode one step ahead of the consumers; the barrier at the top of iteration kt publishes the
-    // decoded slice of step kt and the landed activations of step kt, and frees what step kt - 1 used.
-    int issued = 0;
-    if (producer) {
-        for (; issued < NS - 1 && issued < ksteps; issued++) issue(issued);
-        wait_vm((issued - 1) * LPS);
-    }
-    __builtin_amdgcn_s_barrier();
-    if (producer) dequant(0);
+        // A step is two 32-column halves.  The second half's fragment reads are in flight while
+        // the first half's MFMAs run.
+        half8 fa[2][MB], fb[2][NB];
+        auto issue_frags = [&](int s, int ks) {
+            const uint32_t abase = a0 + (s % NSA) * ABYTES;
+            const uint32_t wbase = w16_0 + (s & 1) * W16_BYTES;
+            const int chunk = ks * 4 + (lane >> 4);
+            uint32_t aa[MB], ba[NB];
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                const int r = wm * TM + i * 16 + (lane & 15);
+                aa[i] = abase + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4);
+            }
+#pragma unroll
+            for (int j = 0; j < NB; j++) ba[j] = wbase + (brow[j] + (lane & 15)) * W16_STRIDE + chunk * 16;
+            lds_issue_h8n<MB>(aa, fa[ks]);
+            lds_issue_h8n<NB>(ba, fb[ks]);
+        };
+        auto mfma_half = [&](int ks) {
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+        };
 
-    // steady state: step kt + NS - 1 is issued in iteration kt, so when step kt + 1 is awaited
-    // exactly NS - 3 younger steps are in flight -- the wait is an immediate
-    const int steady = ksteps - (NS - 1) > 0 ? ksteps - (NS - 1) : 0;
-    int kt = 0;
-    for (; kt < steady; kt++) {
-        if (producer) JL_WAIT_VM((NS - 3) * LPS);
         __builtin_amdgcn_s_barrier();
-        if (producer) {
-            issue(kt + NS - 1);
-            dequant(kt + 1);
-        } else {
-            consume(kt);
-        }
-    }
-    // drain: nothing left to issue
-    for (; kt < ksteps; kt++) {
-        if (producer) {
-            const int ahead = ksteps - (kt + 2);
-            wait_vm(ahead > 0 ? ahead * LPS : 0);
+        for (int s = 0; s < ksteps; s++) {
+            __builtin_amdgcn_s_barrier();
+            issue_frags(s, 0);
+            lds_wait_frags<MB, NB>(fa[0], fb[0]);
+            issue_frags(s, 1);
+            mfma_half(0);
+            lds_wait_frags<MB, NB>(fa[1], fb[1]);
+            mfma_half(1);
         }
         __builtin_amdgcn_s_barrier();
-        if (producer) {
-            if (kt + 1 < ksteps) dequant(kt + 1);
-        } else {
-            consume(kt);
-        }
-    }
-    if (producer) return;
 
-    // ---- epilogue (consumers) ----
-    // The weight fragment went in as the MFMA's row operand, so a lane holds four consecutive
-    // output columns 4 * (lane / 16) .. + 3 of activation row lane % 16 of each block: one
-    // 16-byte store per block.
-    if (p.splits > 1) {
-        // partial sums of this run of K: plain 16-byte stores into the scratch plane of this split;
-        // jl_gemm_reduce adds the planes in order and applies the epilogue
-        const int64_t plane = (int64_t)p.mtiles * BM * p.ntiles * BN;
-        float *pp = p.partial + split * plane;
+        // ---- epilogue ----
+        // The weight fragment went in as the MFMA's row operand, so a lane holds four consecutive
+        // output columns 4 * (lane / 16) .. + 3 of activation row lane % 16 of each block: one
+        // 16-byte store per block.
+        if (p.splits > 1) {
+            // partial sums of this run of K: plain 16-byte stores into the scratch plane of this
+            // split; jl_gemm_reduce adds the planes in order and applies the epilogue
+            const int64_t plane = (int64_t)p.mtiles * BM * p.ntiles * BN;
+            float *pp = p.partial + split * plane;
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                const int m = m0 + wm * TM + i * 16 + (lane & 15);
+                float *prow = pp + (int64_t)m * (p.ntiles * BN) + nt * BN;
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    const int c = brow[j] + (lane >> 4) * 4;  // column inside the 128-wide tile
+                    *(float4 *)(prow + c) = float4{acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+                }
+            }
+            continue;
+        }
 #pragma unroll
         for (int i = 0; i < MB; i++) {
             const int m = m0 + wm * TM + i * 16 + (lane & 15);
-            float *prow = pp + (int64_t)m * (p.ntiles * BN) + nt * BN;
+            if (m >= p.rows) continue;
+            const float rs = p.row_scale[m];
+            float *crow = p.C + (int64_t)m * p.ldo + p.col_offset;
+            if (swiglu) {
 #pragma unroll
-            for (int j = 0; j < NB; j++) {
-                const int c = brow[j] + (lane >> 4) * 4;  // column inside the 128-wide tile
-                *(float4 *)(prow + c) = float4{acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
-            }
-        }
-        return;
-    }
+                for (int j = 0; j < NB / 2; j++) {
+                    const int col = n0 + wn * (TN / 2) + j * 16 + (lane >> 4) * 4;
 #pragma unroll
-    for (int i = 0; i < MB; i++) {
-        const int m = m0 + wm * TM + i * 16 + (lane & 15);
-        if (m >= p.rows) continue;
-        const float rs = p.row_scale[m];
-        float *crow = p.C + (int64_t)m * p.ldo + p.col_offset;
-        if (swiglu) {
+                    for (int e = 0; e < 4; e++)
+                        if (col + e < p.n_total)
+                            crow[col + e] = gemm_swiglu(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
+                }
+            } else {
 #pragma unroll
-            for (int j = 0; j < NB / 2; j++) {
-                const int col = n0 + wn * (TN / 2) + j * 16 + (lane >> 4) * 4;
+                for (int j = 0; j < NB; j++) {
+                    const int col = n0 + wn * TN + j * 16 + (lane >> 4) * 4;
+                    float4 v = {acc[i][j][0] * rs, acc[i][j][1] * rs, acc[i][j][2] * rs, acc[i][j][3] * rs};
+                    float *dst = crow + col;
+                    if (col + 3 < p.n_total && (((uintptr_t)dst) & 15) == 0) {
+                        if (p.epilogue == JL_RESIDUAL) {
+                            float4 o = *(const float4 *)dst;
+                            v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+                        }
+                        *(float4 *)dst = v;
+                    } else {
+                        const float ve[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (col + e < p.n_total)
-                        crow[col + e] = gemm_swiglu(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < NB; j++) {
-                const int col = n0 + wn * TN + j * 16 + (lane >> 4) * 4;
-                float4 v = {acc[i][j][0] * rs, acc[i][j][1] * rs, acc[i][j][2] * rs, acc[i][j][3] * rs};
-                float *dst = crow + col;
-                if (col + 3 < p.n_total && (((uintptr_t)dst) & 15) == 0) {
-                    if (p.epilogue == JL_RESIDUAL) {
-                        float4 o = *(const float4 *)dst;
-                        v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
-                    }
-                    *(float4 *)dst = v;
-                } else {
-                    const float ve[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        if (col + e < p.n_total) {
-                            if (p.epilogue == JL_RESIDUAL) dst[e] += ve[e];
-                            else dst[e] = ve[e];
+                        for (int e = 0; e < 4; e++) {
+                            if (col + e < p.n_total) {
+                                if (p.epilogue == JL_RESIDUAL) dst[e] += ve[e];
+                                else dst[e] = ve[e];
+                            }
                         }
                     }
                 }
@@ -683,14 +696,14 @@ size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 namespace {
 
 // Split-K factor for a skinny call (at most 64 activation rows): enough workgroups to cover the
-// chip, at least 8 steps (512 columns) per split, and partial-sum traffic (written once, read once)
+// chip, at least 2 raw stages (512 columns) per split, and partial-sum traffic (written once, read once)
 // no larger than the weight bytes themselves.  A divisor of the step count.
 int choose_splits(int rows, int k, int ntiles, int row_bytes, int compute_units) {
     if (rows > 64) return 1;
-    const int ksteps = k / BK;
+    const int ksteps = k / (BK * SUPER);  // raw stages of 256 columns
     const int padded = rows <= 32 ? 32 : 64;
     int want = (2 * compute_units + ntiles - 1) / ntiles;
-    int by_steps = ksteps / 8;
+    int by_steps = ksteps / 2;
     int by_traffic = row_bytes / (8 * padded);
     int s = want < by_steps ? want : by_steps;
     if (by_traffic < s) s = by_traffic;
@@ -718,10 +731,10 @@ size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_
 
 namespace {
 
-template <int TYPE, int BM, int NS>
+template <int TYPE, int BM>
 int launch_gemm(jl_context *ctx, const GemmParams &p, dim3 grid) {
-    auto fn = jl_gemm_f16<TYPE, BM, NS>;
-    constexpr int lds = gemm_lds_bytes<TYPE, BM, NS>();
+    auto fn = jl_gemm_f16<TYPE, BM>;
+    constexpr int lds = gemm_lds_bytes<TYPE, BM>();
     static_assert(lds <= 160 * 1024, "operand rings exceed the 160 KB of LDS");
     static bool configured[16] = {};
     if (ctx->device < 16 && !configured[ctx->device]) {
@@ -743,14 +756,16 @@ int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows, float *planes, si
     const int64_t plane = (int64_t)p.mtiles * bm * p.ntiles * BN;
     if (p.splits > 1 && (size_t)p.splits * plane * 4 > plane_bytes) p.splits = 1;
     p.partial = planes;
-    // one workgroup per (tile, split); the tile count is padded to a multiple of 8 so that each XCD
-    // gets the same number of launch slots per split
-    const unsigned per_split = (unsigned)((p.ntiles * p.mtiles + 7) / 8 * 8);
-    const dim3 grid(per_split * p.splits);
+    // persistent workgroups, one per compute unit (fewer when there is less work), a multiple of 8
+    // so that every XCD runs the same number of them
+    const int items = p.ntiles * p.mtiles * p.splits;
+    int wgs = items < ctx->compute_units ? items : ctx->compute_units;
+    wgs = (wgs + 7) / 8 * 8;
+    const dim3 grid(wgs);
     int st;
-    if (bm == 32) st = launch_gemm<TYPE, 32, 6>(ctx, p, grid);
-    else if (bm == 64) st = launch_gemm<TYPE, 64, 6>(ctx, p, grid);
-    else st = launch_gemm<TYPE, 128, 4>(ctx, p, grid);
+    if (bm == 32) st = launch_gemm<TYPE, 32>(ctx, p, grid);
+    else if (bm == 64) st = launch_gemm<TYPE, 64>(ctx, p, grid);
+    else st = launch_gemm<TYPE, 128>(ctx, p, grid);
     if (st != JL_OK || p.splits == 1) return st;
     hipLaunchKernelGGL(jl_gemm_reduce, dim3((p.n_total + 255) / 256, rows), dim3(256), 0, ctx->stream,
                        planes, p.row_scale, p.C, rows, p.n_total, p.ntiles, plane, p.splits, p.ldo,
@@ -769,7 +784,10 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     if (math == JL_MATH_INT8) {
         return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: the int8 kernels are not built into this library");
     }
-    JL_REQUIRE(k % 64 == 0, "jl_gemm: row length %d is not a multiple of 64", k);
+    if (k % 256 != 0) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "jl_gemm: no batched kernel for a row length of %d (a multiple of 256 is needed)", k);
+    }
     JL_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)workspace & 255) == 0,
                "jl_gemm: X must be 16-byte and the workspace 256-byte aligned");
     for (int i = 0; i < count; i++)
