@@ -138,11 +138,14 @@ __device__ __forceinline__ void lds_wait_frags(half8 (&a)[NA], half8 (&b)[NBF]) 
     }
 }
 
+// Four 16-byte chunks of one decoded row: chunk i goes to addr ^ (i << 4), i.e. the four stay inside
+// one aligned 64-byte group and are permuted by the row's swizzle key already folded into addr.
 __device__ __forceinline__ void lds_write_4xh8(uint32_t addr, const half8 (&v)[4]) {
+    const uint32_t a1 = addr ^ 16u, a2 = addr ^ 32u, a3 = addr ^ 48u;
     asm volatile(
-        "ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:16\n\tds_write_b128 %0, %3 offset:32\n\t"
-        "ds_write_b128 %0, %4 offset:48\n\ts_waitcnt lgkmcnt(0)"
-        : : "v"(addr), "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]) : "memory");
+        "ds_write_b128 %0, %4\n\tds_write_b128 %1, %5\n\tds_write_b128 %2, %6\n\t"
+        "ds_write_b128 %3, %7\n\ts_waitcnt lgkmcnt(0)"
+        : : "v"(addr), "v"(a1), "v"(a2), "v"(a3), "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]) : "memory");
 }
 
 __device__ __forceinline__ void lds_read_9dw(uint32_t addr, uint32_t (&w)[9]) {
@@ -305,8 +308,8 @@ struct GemmParams {
 
 constexpr int BN = 128, BK = 64;
 constexpr int SUPER = 4;                       // 64-column steps per raw-weight stage (256 columns)
-constexpr int W16_STRIDE = 144;                // bytes per decoded row: 64 halfs + 16 bytes of padding
-constexpr int W16_BYTES = BN * W16_STRIDE;     // 18432
+constexpr int W16_STRIDE = 128;                // bytes per decoded row: 64 halfs, chunks XOR-swizzled like A's
+constexpr int W16_BYTES = BN * W16_STRIDE;     // 16384
 
 // Raw weight bytes of one row for 256 columns -- always a whole number of 16-byte chunks, and
 // 16-byte aligned in the file layout, which is what lets the stage be fetched with 128-bit loads:
@@ -507,7 +510,8 @@ jl_gemm_f16(GemmParams p) {
                     decode_half_slice<TYPE>(row + 16 + q * 32, row, dhalf, q * 2 + dhalf, v);
                 else
                     decode_half_slice<TYPE>(row + q * Raw<TYPE>::kStepBytes, 0, dhalf, 0, v);
-                lds_write_4xh8(w16_0 + (s & 1) * W16_BYTES + drow * W16_STRIDE + dhalf * 64, v);
+                lds_write_4xh8(w16_0 + (s & 1) * W16_BYTES + drow * W16_STRIDE +
+                                   (((dhalf * 4) ^ ((drow >> 1) & 7)) << 4), v);
             };
 
             issue_raw(0);
@@ -570,7 +574,10 @@ jl_gemm_f16(GemmParams p) {
                 aa[i] = abase + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4);
             }
 #pragma unroll
-            for (int j = 0; j < NB; j++) ba[j] = wbase + (brow[j] + (lane & 15)) * W16_STRIDE + chunk * 16;
+            for (int j = 0; j < NB; j++) {
+                const int r = brow[j] + (lane & 15);
+                ba[j] = wbase + r * W16_STRIDE + ((chunk ^ ((r >> 1) & 7)) << 4);
+            }
             lds_issue_h8n<MB>(aa, fa[ks]);
             lds_issue_h8n<NB>(ba, fb[ks]);
         };
