@@ -193,13 +193,17 @@ def bench_gemm(ctx, hip, t, T, steps, warmup):
         proj.gateUp(X, hb, w["w1"], w["w3"], DIM, HIDDEN)
         proj.projection(H, res, w["w2"], HIDDEN, DIM, True)
 
+    # replayed as a HIP graph: Python cannot enqueue the layer's launches as fast as they run
+    layer()
+    ctx.sync()
+    graph = hip.capture(ctx.stream, layer)
     for _ in range(warmup):
-        layer()
+        hip.launch(graph, ctx.stream)
     ctx.sync()
     e0, e1 = hip.event(), hip.event()
     hip.record(e0, ctx.stream)
     for _ in range(steps):
-        layer()
+        hip.launch(graph, ctx.stream)
     hip.record(e1, ctx.stream)
     ms = hip.elapsed_ms(e0, e1) / steps
     flops = 2.0 * T * (DIM * (DIM + 2 * KV_DIM) + DIM * DIM + 2 * DIM * HIDDEN + HIDDEN * DIM)
@@ -238,13 +242,17 @@ def bench_batched_q4k(ctx, hip, B, steps, warmup):
         proj.gateUp(X, hb, w["w1"], w["w3"], dim, ffn)
         proj.projection(H, res, w["w2"], ffn, dim, True)
 
+    # replayed as a HIP graph: Python cannot enqueue the layer's launches as fast as they run
+    layer()
+    ctx.sync()
+    graph = hip.capture(ctx.stream, layer)
     for _ in range(warmup):
-        layer()
+        hip.launch(graph, ctx.stream)
     ctx.sync()
     e0, e1 = hip.event(), hip.event()
     hip.record(e0, ctx.stream)
     for _ in range(steps):
-        layer()
+        hip.launch(graph, ctx.stream)
     hip.record(e1, ctx.stream)
     ms = hip.elapsed_ms(e0, e1) / steps
     wbytes = sum(x.nbytes for x in w.values())

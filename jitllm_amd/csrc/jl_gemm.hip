@@ -809,6 +809,15 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     float *planes = (float *)((uint8_t *)workspace + head);
     const size_t plane_bytes = workspace_bytes > head ? workspace_bytes - head : 0;
 
+
+    if (rows <= 32) {
+        // batched decode of up to 32 rows: the weight-streaming kernel reads X itself
+        bool taken = false;
+        int st = jl_launch_gemm_skinny(ctx, weights, count, X, C, rows, ldo, col_offset, epilogue, planes,
+                                       plane_bytes, &taken);
+        if (st != JL_OK || taken) return st;
+    }
+
     hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
     JL_HIP(hipGetLastError());
 

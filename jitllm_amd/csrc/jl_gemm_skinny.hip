@@ -1,0 +1,635 @@
+// Batched decode (at most 64 activation rows): C = X . [W0 | W1 | ...]^T streamed at HBM speed.
+//
+// Replaces the reference's tiled batched-row kernels (matrixVectorTiledBatchQ4_0 / Q4_K,
+// J/backend/tornado/kernels/TransformerComputeKernelsQ4_0.java:1205-1292,
+// TransformerComputeKernelsQ4_K.java:1120-1221, driven by QuantizedBatchProjections.java:76-309).
+//
+// With so few rows the call is bound by reading the weights once, exactly like the single-token
+// matrix-vector kernels, so this kernel has their shape: a workgroup walks tiles of 16 weight rows,
+// a tile is copied into an LDS ring by LDS-DMA while the previous one is computed, and a thread
+// owns one 64-column slice of its weight row.  What differs is the arithmetic: the thread decodes
+// its slice to fp16 in registers -- eight fragments of eight consecutive columns -- and a wave (16
+// rows x 4 slices) multiplies them with the matching activation fragments on
+// v_mfma_f32_16x16x32_f16.  The MFMA sums over 32 "k slots"; slot (g, e) of MFMA i is column
+// 64 (slice of lane group g) + 8 i + e, the same for both operands, so no data crosses lanes.
+// The activation fragments (fp16 copy of X, made once per call) depend on the slice only and stay
+// in registers for the whole kernel.  A wave's result is a partial sum over its 256 columns; the
+// waves of a workgroup fold through LDS one tile later, rows wider than the workgroup's span are
+// cut across workgroups and folded by jl_skinny_reduce.
+#include "jl_device.h"
+#include "jl_internal.h"
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const void gvoid;
+typedef __attribute__((address_space(3))) void lvoid;
+
+constexpr int kMaxSeg = 8;
+constexpr int kGroup = 16;  // weight rows per tile: the MFMA's row count
+
+struct SkinnyParams {
+    const uint8_t *w[kMaxSeg];
+    int seg_rows[kMaxSeg];
+    int seg_group_begin[kMaxSeg + 1];  // first row group of each weight; [nseg] = all groups
+    int seg_col_begin[kMaxSeg];        // first output column of each weight
+    int nseg;
+    const uint8_t *w_up;      // JL_SWIGLU: the up weight (a group is 8 gate rows + 8 up rows)
+    const float *X;           // [rows x k] fp32 activations
+    float *C;
+    float *planes;            // Z > 1: [Z][16 * NBB][groups * 16] partial sums
+    int rows;                 // active activation rows
+    int k;
+    int64_t ldo, col_offset;
+    int epilogue;
+    int row_bytes;
+    int Ss;                   // 64-column slices one workgroup spans (a multiple of 4, at most 32)
+    int Z;                    // spans per row
+    int span_bytes;           // bytes of a weight row inside one span
+    int stages;               // depth of the tile ring
+};
+
+#define JL_WAIT_VM(N) \
+    __builtin_amdgcn_s_waitcnt(((N)&0xF) | (((N) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+// s_waitcnt vmcnt(n) for a run-time n (the instruction takes an immediate)
+__device__ __forceinline__ void wait_vm(int n) {
+    switch (n) {
+#define C(i) case i: JL_WAIT_VM(i); break;
+        C(0) C(1) C(2) C(3) C(4) C(5) C(6) C(7) C(8) C(9) C(10) C(11) C(12) C(13) C(14) C(15)
+        C(16) C(17) C(18) C(19) C(20) C(21) C(22) C(23) C(24) C(25) C(26) C(27) C(28) C(29) C(30)
+        C(31) C(32) C(33) C(34) C(35) C(36) C(37) C(38) C(39) C(40) C(41) C(42) C(43) C(44) C(45)
+        C(46) C(47) C(48) C(49) C(50) C(51) C(52) C(53) C(54) C(55) C(56) C(57) C(58) C(59) C(60)
+        C(61) C(62)
+#undef C
+        default: JL_WAIT_VM(63); break;
+    }
+}
+
+// ---- LDS access by hand (the compiler would drain the LDS-DMA ring before any LDS access it sees)
+
+__device__ __forceinline__ void lds_read_17(uint32_t addr, uint32_t (&w)[17]) {
+    uint2 p0, p1, p2, p3, p4, p5, p6, p7;
+    uint32_t last;
+    asm volatile(
+        "ds_read2_b32 %0, %9 offset0:0 offset1:1\n\tds_read2_b32 %1, %9 offset0:2 offset1:3\n\t"
+        "ds_read2_b32 %2, %9 offset0:4 offset1:5\n\tds_read2_b32 %3, %9 offset0:6 offset1:7\n\t"
+        "ds_read2_b32 %4, %9 offset0:8 offset1:9\n\tds_read2_b32 %5, %9 offset0:10 offset1:11\n\t"
+        "ds_read2_b32 %6, %9 offset0:12 offset1:13\n\tds_read2_b32 %7, %9 offset0:14 offset1:15\n\t"
+        "ds_read_b32 %8, %9 offset:64\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(p0), "=&v"(p1), "=&v"(p2), "=&v"(p3), "=&v"(p4), "=&v"(p5), "=&v"(p6), "=&v"(p7),
+          "=&v"(last)
+        : "v"(addr) : "memory");
+    w[0] = p0.x; w[1] = p0.y; w[2] = p1.x; w[3] = p1.y; w[4] = p2.x; w[5] = p2.y; w[6] = p3.x;
+    w[7] = p3.y; w[8] = p4.x; w[9] = p4.y; w[10] = p5.x; w[11] = p5.y; w[12] = p6.x; w[13] = p6.y;
+    w[14] = p7.x; w[15] = p7.y; w[16] = last;
+}
+
+__device__ __forceinline__ void lds_read_9(uint32_t addr, uint32_t (&w)[9]) {
+    uint2 p0, p1, p2, p3;
+    uint32_t last;
+    asm volatile(
+        "ds_read2_b32 %0, %5 offset0:0 offset1:1\n\tds_read2_b32 %1, %5 offset0:2 offset1:3\n\t"
+        "ds_read2_b32 %2, %5 offset0:4 offset1:5\n\tds_read2_b32 %3, %5 offset0:6 offset1:7\n\t"
+        "ds_read_b32 %4, %5 offset:32\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(p0), "=&v"(p1), "=&v"(p2), "=&v"(p3), "=&v"(last)
+        : "v"(addr) : "memory");
+    w[0] = p0.x; w[1] = p0.y; w[2] = p1.x; w[3] = p1.y; w[4] = p2.x; w[5] = p2.y; w[6] = p3.x;
+    w[7] = p3.y; w[8] = last;
+}
+
+__device__ __forceinline__ void lds_read_q4k(uint32_t hdr, uint32_t qs, uint4 &h, uint4 &q0, uint4 &q1) {
+    asm volatile(
+        "ds_read_b128 %0, %3\n\tds_read_b128 %1, %4\n\tds_read_b128 %2, %4 offset:16\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(h), "=&v"(q0), "=&v"(q1) : "v"(hdr), "v"(qs) : "memory");
+}
+
+// Never hand an MFMA result straight to this: the matrix pipe does not interlock with an LDS store
+// that reads its destination registers, and the compiler's hazard pass cannot see inside inline
+// assembly.  Callers pass values that went through ordinary vector arithmetic first.
+__device__ __forceinline__ void lds_write_f4(uint32_t addr, floatx4 v) {
+    asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                 : : "v"(addr), "v"(v) : "memory");
+}
+
+__device__ __forceinline__ floatx4 lds_read_f4(uint32_t addr) {
+    floatx4 v;
+    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+    return v;
+}
+
+__device__ __forceinline__ void lds_read_8xf4(const uint32_t (&a)[8], floatx4 (&v)[8]) {
+    asm volatile(
+        "ds_read_b128 %0, %8\n\tds_read_b128 %1, %9\n\tds_read_b128 %2, %10\n\tds_read_b128 %3, %11\n\t"
+        "ds_read_b128 %4, %12\n\tds_read_b128 %5, %13\n\tds_read_b128 %6, %14\n\tds_read_b128 %7, %15\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7]) : "memory");
+}
+
+// ---- slice decode: raw block bytes -> eight fp16 fragments of eight consecutive columns ---------
+//
+// A byte b in 0..255 under the exponent byte 0x64 is the fp16 number 1024 + b, exactly; a packed
+// subtract recentres it and a packed multiply applies the block scale.  Each product is exact
+// before its one rounding, so a decoded weight is the host's float decode rounded once to fp16.
+
+__device__ __forceinline__ h2 bytes_to_h2(uint32_t v, uint32_t sel) {
+    return __builtin_bit_cast(h2, __builtin_amdgcn_perm(v, 0x64646464u, sel));
+}
+
+// eight bytes (two dwords, already in 0..255 offset form) -> (byte - bias) * d
+__device__ __forceinline__ half8 frag_scaled(uint32_t q0, uint32_t q1, h2 bias, h2 d) {
+    h2 a = (bytes_to_h2(q0, 0x00050004u) - bias) * d;
+    h2 b = (bytes_to_h2(q0, 0x00070006u) - bias) * d;
+    h2 c = (bytes_to_h2(q1, 0x00050004u) - bias) * d;
+    h2 e = (bytes_to_h2(q1, 0x00070006u) - bias) * d;
+    return half8{a[0], a[1], b[0], b[1], c[0], c[1], e[0], e[1]};
+}
+
+// eight nibbles (two dwords of bytes 0..15) -> q * ds - dm, fused
+__device__ __forceinline__ half8 frag_affine(uint32_t q0, uint32_t q1, h2 ds, h2 dm) {
+    const h2 bias = {(_Float16)1024.f, (_Float16)1024.f};
+    h2 a = (bytes_to_h2(q0, 0x00050004u) - bias) * ds - dm;
+    h2 b = (bytes_to_h2(q0, 0x00070006u) - bias) * ds - dm;
+    h2 c = (bytes_to_h2(q1, 0x00050004u) - bias) * ds - dm;
+    h2 e = (bytes_to_h2(q1, 0x00070006u) - bias) * ds - dm;
+    return half8{a[0], a[1], b[0], b[1], c[0], c[1], e[0], e[1]};
+}
+
+// Decodes the 64-column slice `sl` of the tile row at LDS address `row`.
+template <int TYPE>
+__device__ __forceinline__ void decode_slice(uint32_t row, int sl, half8 (&f)[8]) {
+    if constexpr (TYPE == JL_Q8_0) {
+        // 68 bytes: scale A | 32 quants A | scale B | 32 quants B
+        uint32_t w[17];
+        lds_read_17(row + sl * 68, w);
+        const _Float16 dA = __builtin_bit_cast(_Float16, (unsigned short)(w[0] & 0xFFFF));
+        const _Float16 dB = __builtin_bit_cast(_Float16, (unsigned short)(w[8] >> 16));
+        const h2 bias = {(_Float16)1152.f, (_Float16)1152.f};
+        const h2 a2 = {dA, dA}, b2 = {dB, dB};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t q0 = __builtin_amdgcn_alignbit(w[2 * i + 1], w[2 * i], 16);
+            const uint32_t q1 = __builtin_amdgcn_alignbit(w[2 * i + 2], w[2 * i + 1], 16);
+            f[i] = frag_scaled(q0 ^ 0x80808080u, q1 ^ 0x80808080u, bias, a2);
+            f[4 + i] = frag_scaled(w[9 + 2 * i] ^ 0x80808080u, w[10 + 2 * i] ^ 0x80808080u, bias, b2);
+        }
+    } else if constexpr (TYPE == JL_Q4_0) {
+        // 36 bytes: scale A | 16 nibble bytes A | scale B | 16 nibble bytes B; element i < 16 of a
+        // block is the low nibble of byte i, element 16 + i the high nibble
+        uint32_t w[9];
+        lds_read_9(row + sl * 36, w);
+        const _Float16 dA = __builtin_bit_cast(_Float16, (unsigned short)(w[0] & 0xFFFF));
+        const _Float16 dB = __builtin_bit_cast(_Float16, (unsigned short)(w[4] >> 16));
+        const h2 bias = {(_Float16)1032.f, (_Float16)1032.f};
+        const h2 a2 = {dA, dA}, b2 = {dB, dB};
+        uint32_t qa[4], qb[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            qa[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
+            qb[i] = w[5 + i];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            f[i] = frag_scaled(qa[2 * i] & 0x0F0F0F0Fu, qa[2 * i + 1] & 0x0F0F0F0Fu, bias, a2);
+            f[2 + i] = frag_scaled((qa[2 * i] >> 4) & 0x0F0F0F0Fu, (qa[2 * i + 1] >> 4) & 0x0F0F0F0Fu, bias, a2);
+            f[4 + i] = frag_scaled(qb[2 * i] & 0x0F0F0F0Fu, qb[2 * i + 1] & 0x0F0F0F0Fu, bias, b2);
+            f[6 + i] = frag_scaled((qb[2 * i] >> 4) & 0x0F0F0F0Fu, (qb[2 * i + 1] >> 4) & 0x0F0F0F0Fu, bias, b2);
+        }
+    } else {
+        // a quarter of a super-block: 32 nibble bytes; low nibbles are sub-block 2 pair (columns
+        // 0..31 of the slice), high nibbles sub-block 2 pair + 1; w = (d sc) q - (dmin m)
+        uint4 h, q0, q1;
+        const uint32_t sb = row + (sl >> 2) * 144;
+        const int pair = sl & 3;
+        lds_read_q4k(sb, sb + 16 + pair * 32, h, q0, q1);
+        const float d = jl_half_bits_to_float(h.x);
+        const float dmin = jl_half_bits_to_float(h.x >> 16);
+        int sc0, mn0, sc1, mn1;
+        jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair, sc0, mn0);
+        jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair + 1, sc1, mn1);
+        const _Float16 ds0 = (_Float16)(d * (float)sc0), dm0 = (_Float16)(dmin * (float)mn0);
+        const _Float16 ds1 = (_Float16)(d * (float)sc1), dm1 = (_Float16)(dmin * (float)mn1);
+        const h2 s0 = {ds0, ds0}, m0 = {dm0, dm0}, s1 = {ds1, ds1}, m1 = {dm1, dm1};
+        const uint32_t qs[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            f[i] = frag_affine(qs[2 * i] & 0x0F0F0F0Fu, qs[2 * i + 1] & 0x0F0F0F0Fu, s0, m0);
+            f[4 + i] = frag_affine((qs[2 * i] >> 4) & 0x0F0F0F0Fu, (qs[2 * i + 1] >> 4) & 0x0F0F0F0Fu, s1, m1);
+        }
+    }
+}
+
+__device__ __forceinline__ float skinny_swiglu(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
+// Workgroup = 16 Ss compute threads (Ss / 4 waves) + kDmaWaves waves that do nothing but copy tiles.
+// An LDS-DMA load holds its wave at issue while the memory system is busy; issued from the compute
+// waves that time adds to the arithmetic instead of hiding behind it, so the copies have waves of
+// their own and the two kinds meet at one barrier per tile.
+constexpr int kDmaWaves = 2;
+constexpr int max_slices(int) { return 32; }
+
+// 16-byte loads per DMA wave and tile (upper bound): a tile row takes span_bytes + 16 bytes of LDS
+// (the padding spreads the 16 rows a wave reads at once over all banks), 16 rows, 128 lanes.
+template <int TYPE> struct Loads { static constexpr int kPerWave = TYPE == JL_Q8_0 ? 18 : 10; };
+
+// ZIN: spans of a row that one workgroup walks itself, one tile after the other, adding their
+// results in registers (it then holds ZIN sets of activation fragments); p.Z spans of ZIN each.
+template <int TYPE, int NBB, bool DUAL, int ZIN>
+__global__ void __launch_bounds__(512 + 64 * kDmaWaves) jl_gemm_skinny(SkinnyParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int LD = Loads<TYPE>::kPerWave;
+    const int tid = threadIdx.x;
+    const int waves = (blockDim.x >> 6) - kDmaWaves;   // compute waves
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int z = blockIdx.x % p.Z;            // this workgroup's run of ZIN spans
+    const int lds_row = p.span_bytes + 16;
+    const int slots_per_row = lds_row >> 4;
+    const int n_loads = (kGroup * slots_per_row + 64 * kDmaWaves - 1) / (64 * kDmaWaves);
+    const int stage_bytes = n_loads * 64 * kDmaWaves * 16;
+    const int partial_bytes = waves * NBB * 1024;  // one parity
+    const int total_groups = p.seg_group_begin[p.nseg];
+    const int out_rows = DUAL ? kGroup / 2 : kGroup;   // outputs per group
+
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
+    const uint32_t ring0 = lds0 + 2 * partial_bytes;
+    uint8_t *ring = lds + 2 * partial_bytes;
+
+    // The weight a row group belongs to.  The table is walked with constant indices: it then stays in
+    // scalar registers, where an index computed at run time would turn every use into a load from
+    // the argument buffer -- and a load's wait drains the whole tile ring.
+    struct Segment {
+        const uint8_t *w;
+        int rows, group_begin, col_begin;
+    };
+    auto segment_of = [&](int group) {
+        Segment sg = {p.w[0], p.seg_rows[0], 0, 0};
+#pragma unroll
+        for (int i = 1; i < kMaxSeg; i++) {
+            if (i < p.nseg && group >= p.seg_group_begin[i]) {
+                sg.w = p.w[i];
+                sg.rows = p.seg_rows[i];
+                sg.group_begin = p.seg_group_begin[i];
+                sg.col_begin = p.seg_col_begin[i];
+            }
+        }
+        return sg;
+    };
+
+    // my groups: wg, wg + stride, ... (workgroups of one span share a stride)
+    const int wg = blockIdx.x / p.Z;
+    const int stride = gridDim.x / p.Z;
+    const int mine = wg < total_groups ? (total_groups - wg + stride - 1) / stride : 0;
+
+    if (wave >= waves) {
+        // ---- copy waves.  Slot s of a tile is 16 bytes at LDS offset 16 s: row s / slots_per_row,
+        // byte 16 (s % slots_per_row) of the row's span.  A slot past the data (the padding behind
+        // each row, slots behind the last row) re-reads a neighbouring real slot -- never one
+        // shared address, which every compute unit would then hammer.
+        const int dw = wave - waves;
+        const int span_slots = p.span_bytes >> 4;
+        // the few instructions these waves issue go first: the copy is what everything waits for
+        __builtin_amdgcn_s_setprio(3);
+        int slot_in[LD], slot_row[LD];
+#pragma unroll
+        for (int j = 0; j < LD; j++) {
+            const int slot = (j * kDmaWaves + dw) * 64 + lane;
+            int row = slot / slots_per_row;
+            int within = slot - row * slots_per_row;
+            row = row < kGroup ? row : kGroup - 1;
+            within = within < span_slots ? within : span_slots - 1;
+            slot_row[j] = row;
+            slot_in[j] = z * ZIN * p.span_bytes + within * 16;
+        }
+        // tile t = span t % ZIN of group wg + (t / ZIN) stride
+        auto issue = [&](int t, int st) {
+            const int group = wg + (t / ZIN) * stride;
+            const int span_off = (t % ZIN) * p.span_bytes;
+            const Segment sg = segment_of(group);
+            const int first_row = (group - sg.group_begin) * out_rows;
+            const int64_t base_off = (int64_t)first_row * p.row_bytes + span_off;
+            const uint8_t *w_gate = sg.w + base_off;
+            const uint8_t *w_up = DUAL ? p.w_up + base_off : w_gate;
+            asm volatile("" : "+s"(w_gate), "+s"(w_up));   // both in registers before any per-lane choice
+            uint8_t *dst = ring + st * stage_bytes;
+#pragma unroll
+            for (int j = 0; j < LD; j++) {
+                if (j >= n_loads) break;
+                const int row = slot_row[j];
+                int wrow = DUAL ? (row & 7) : row;
+                if (first_row + wrow >= sg.rows) wrow = 0;  // past the weight's last row
+                const uint8_t *base = (DUAL && row >= 8) ? w_up : w_gate;
+                const uint8_t *src = base + wrow * p.row_bytes + slot_in[j];
+                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, 0);
+            }
+        };
+        const int tiles = mine * ZIN;
+        int issued = 0;
+        for (; issued < p.stages - 1 && issued < tiles; issued++) issue(issued, issued);
+        for (int t = 0; t < tiles; t++) {
+            // tiles issued after tile t may stay in flight
+            wait_vm((issued - t - 1) * n_loads);
+            __builtin_amdgcn_s_barrier();
+            // the stage of tile t - 1 is free now: every compute wave is past its reads
+            if (issued < tiles) {
+                issue(issued, issued % p.stages);
+                issued++;
+            }
+        }
+        if (mine > 0) __builtin_amdgcn_s_barrier();
+        return;
+    }
+
+    // ---- compute waves
+    const int c = lane & 15;                   // row of the group
+    const int g = lane >> 4;                   // which of the wave's four slices
+    const int sl = 4 * wave + g;               // slice inside the span
+
+    // Activation fragments: 64 consecutive columns of NBB x 16 rows, kept for the whole kernel.
+    // Read as fp32 (while the first tiles are on their way) and rounded to fp16 behind a
+    // power-of-two scale per row and wave: the largest magnitude of the row's 256 columns this wave
+    // multiplies is brought into [2^11, 2^12), which keeps huge rows finite and tiny rows out of
+    // fp16's subnormals.  The lane that holds activation row c as an operand also holds the results
+    // of that row (MFMA column c), so the scale is undone lane-locally, exactly.
+    half8 af[NBB][ZIN][8];
+    float undo[NBB][ZIN];
+#pragma unroll
+    for (int b = 0; b < NBB; b++) {
+#pragma unroll
+        for (int q = 0; q < ZIN; q++) {
+            const int m = 16 * b + c;
+            float4 x[16];
+            if (m < p.rows) {
+                const float4 *src = (const float4 *)(p.X + (int64_t)m * p.k + 64 * ((z * ZIN + q) * p.Ss + sl));
+#pragma unroll
+                for (int i = 0; i < 16; i++) x[i] = src[i];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; i++) x[i] = float4{0.f, 0.f, 0.f, 0.f};
+            }
+            float amax = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                amax = fmaxf(amax, fmaxf(fmaxf(fabsf(x[i].x), fabsf(x[i].y)), fmaxf(fabsf(x[i].z), fabsf(x[i].w))));
+            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            // amax = 1.f * 2^(E - 127): multiply by 2^(138 - E), undo with 2^(E - 138)
+            int E = (int)((__float_as_uint(amax) >> 23) & 0xFF);
+            E = E < 12 ? 12 : E;
+            const float inv = __uint_as_float((uint32_t)(265 - E) << 23);
+            undo[b][q] = __uint_as_float((uint32_t)(E - 11) << 23);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float4 lo = x[2 * i], hi = x[2 * i + 1];
+                af[b][q][i] = half8{(_Float16)(lo.x * inv), (_Float16)(lo.y * inv), (_Float16)(lo.z * inv),
+                                    (_Float16)(lo.w * inv), (_Float16)(hi.x * inv), (_Float16)(hi.y * inv),
+                                    (_Float16)(hi.z * inv), (_Float16)(hi.w * inv)};
+            }
+        }
+    }
+
+    // Folds the waves' partial sums of group `group` (parity `par`) and applies the epilogue.  A
+    // partial is what one lane of one wave held: weight rows 4 (o / 16) .. + 3 of activation row
+    // 16 b + o % 16, for lane o and row block b.  The (b, o) pairs are dealt out over all compute
+    // waves so that the fold is a few lanes' work in each instead of one wave's critical path.
+    // Gate/up groups: lanes o >= 32 hold the up rows of the outputs of lane o - 32.
+    auto finish = [&](int group, int par) {
+        const int lanes_out = DUAL ? 32 : 64;
+        const int per = (lanes_out + waves - 1) / waves;     // lanes o per wave
+        const Segment sg = segment_of(group);
+        for (int base = 0; base < per * NBB; base += 64) {
+            const int item = base + lane;
+            const int b = item / per;
+            const int o = wave * per + (item - b * per);
+            if (b >= NBB || o >= lanes_out) continue;
+            const uint32_t pb = lds0 + par * partial_bytes + b * 1024 + o * 16;
+            floatx4 sum = {0.f, 0.f, 0.f, 0.f}, sum_up = {0.f, 0.f, 0.f, 0.f};
+            // every wave's partial (there are at most eight waves): all reads in flight, one wait
+            uint32_t a[8];
+            float keep[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                keep[j] = j < waves ? 1.f : 0.f;
+                a[j] = pb + (j < waves ? j : 0) * (NBB * 1024);
+            }
+            floatx4 part[8];
+            lds_read_8xf4(a, part);
+#pragma unroll
+            for (int j = 0; j < 8; j++) sum += part[j] * keep[j];
+            if constexpr (DUAL) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) a[j] += 32 * 16;
+                lds_read_8xf4(a, part);
+#pragma unroll
+                for (int j = 0; j < 8; j++) sum_up += part[j] * keep[j];
+            }
+            const int m = 16 * b + (o & 15);
+            const int go = o >> 4;
+            const int local = (group - sg.group_begin) * out_rows + 4 * go;  // first of 4 outputs
+            if (p.Z > 1) {
+                // partial sums of this span: [z][row][group * 16 + weight row of the group]
+                float *pp = p.planes + ((int64_t)z * (16 * NBB) + m) * ((int64_t)total_groups * 16) + group * 16 + 4 * go;
+                *(floatx4 *)pp = sum;
+                if constexpr (DUAL) *(floatx4 *)(pp + 8) = sum_up;
+                continue;
+            }
+            if (m >= p.rows) continue;
+            float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + sg.col_begin + local;
+            const int left = sg.rows - local;
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = DUAL ? skinny_swiglu(sum[e], sum_up[e]) : sum[e];
+            if (p.epilogue == JL_RESIDUAL) {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (e < left) unsafeAtomicAdd(dst + e, v[e]);
+            } else if (left >= 4 && (((uintptr_t)dst) & 15) == 0) {
+                *(floatx4 *)dst = floatx4{v[0], v[1], v[2], v[3]};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (e < left) dst[e] = v[e];
+            }
+        }
+    };
+
+    for (int it = 0; it < mine; it++) {
+        const int group = wg + it * stride;
+        floatx4 total[NBB];
+#pragma unroll
+        for (int b = 0; b < NBB; b++) total[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < ZIN; q++) {
+            const int t = it * ZIN + q;
+            __builtin_amdgcn_s_barrier();   // tile t has landed; the partial sums of group it - 1 are complete
+            if (q == 0 && it > 0) finish(group - stride, (it - 1) & 1);
+
+            half8 wf[8];
+            decode_slice<TYPE>(ring0 + (t % p.stages) * stage_bytes + c * lds_row, sl, wf);
+#pragma unroll
+            for (int b = 0; b < NBB; b++) {
+                floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < 8; i += 2) {
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[i], af[b][q][i], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[i + 1], af[b][q][i + 1], acc1, 0, 0, 0);
+                }
+                total[b] += (acc0 + acc1) * undo[b][q];
+            }
+        }
+        // plain arithmetic happened on the MFMA results: the compiler placed the wait states itself
+        const uint32_t pw = lds0 + (it & 1) * partial_bytes + wave * (NBB * 1024) + lane * 16;
+#pragma unroll
+        for (int b = 0; b < NBB; b++) lds_write_f4(pw + b * 1024, total[b]);
+    }
+    if (mine > 0) {
+        __builtin_amdgcn_s_barrier();
+        finish(wg + (mine - 1) * stride, (mine - 1) & 1);
+    }
+}
+
+// Adds the spans' partial sums in span order and applies row scale and epilogue; one thread per
+// (activation row, weight row of a group).
+template <bool DUAL>
+__global__ void __launch_bounds__(256) jl_skinny_reduce(SkinnyParams p, int padded_rows) {
+    const int total_groups = p.seg_group_begin[p.nseg];
+    const int v = blockIdx.x * blockDim.x + threadIdx.x;  // group * 16 + row of the group
+    const int m = blockIdx.y;
+    if (v >= total_groups * 16 || m >= p.rows) return;
+    const int group = v >> 4, r = v & 15;
+    if (DUAL && r >= 8) return;
+    int seg = 0;
+    for (int i = 1; i < kMaxSeg; i++)
+        if (i < p.nseg && group >= p.seg_group_begin[i]) seg = i;
+    const int out_rows = DUAL ? 8 : 16;
+    const int local = (group - p.seg_group_begin[seg]) * out_rows + r;
+    if (local >= p.seg_rows[seg]) return;
+    const int64_t width = (int64_t)total_groups * 16;
+    const float *pp = p.planes + (int64_t)m * width + v;
+    float s = 0.f, u = 0.f;
+    for (int zz = 0; zz < p.Z; zz++) {
+        s += pp[(int64_t)zz * padded_rows * width];
+        if (DUAL) u += pp[(int64_t)zz * padded_rows * width + 8];
+    }
+    float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + p.seg_col_begin[seg] + local;
+    if (DUAL) *dst = skinny_swiglu(s, u);
+    else if (p.epilogue == JL_RESIDUAL) *dst += s;
+    else *dst = s;
+}
+
+template <int TYPE, int NBB, bool DUAL, int ZIN>
+int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int groups) {
+    auto fn = jl_gemm_skinny<TYPE, NBB, DUAL, ZIN>;
+    static bool configured[16] = {};
+    if (ctx->device < 16 && !configured[ctx->device]) {
+        JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        configured[ctx->device] = true;
+    }
+    // one workgroup per compute unit and span (the ring takes most of the LDS), fewer for less work
+    int per_span = ctx->compute_units / p.Z;
+    if (per_span < 1) per_span = 1;
+    if (per_span > groups) per_span = groups;
+    hipLaunchKernelGGL(fn, dim3(per_span * p.Z), dim3(threads + 64 * kDmaWaves), lds, ctx->stream, p);
+    JL_HIP(hipGetLastError());
+    if (p.Z > 1) {
+        hipLaunchKernelGGL(jl_skinny_reduce<DUAL>, dim3((groups * 16 + 255) / 256, p.rows), dim3(256), 0,
+                           ctx->stream, p, 16 * NBB);
+        JL_HIP(hipGetLastError());
+    }
+    return JL_OK;
+}
+
+template <int TYPE, bool DUAL>
+int launch_nbb(jl_context *ctx, const SkinnyParams &p, int nbb, int zin, int threads, int lds, int groups) {
+    if (nbb == 1) {
+        return zin == 2 ? launch<TYPE, 1, DUAL, 2>(ctx, p, threads, lds, groups)
+                        : launch<TYPE, 1, DUAL, 1>(ctx, p, threads, lds, groups);
+    }
+    return launch<TYPE, 2, DUAL, 1>(ctx, p, threads, lds, groups);
+}
+
+}  // namespace
+
+// Rows the fp16 activation copy must hold (zero past the active ones) for `rows` active rows.
+int jl_skinny_padded_rows(int rows) { return rows <= 16 ? 16 : 32; }
+
+// Sets *taken to false, launching nothing, when the shape is not one this kernel takes; the caller
+// then uses the tiled GEMM.
+int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
+                          float *C, int rows, int64_t ldo, int64_t col_offset, int epilogue,
+                          float *planes, size_t plane_bytes, bool *taken) {
+    *taken = false;
+    const int type = weights[0]->type;
+    const int k = (int)weights[0]->cols;
+    const bool dual = epilogue == JL_SWIGLU;
+    if (rows > 32 || k % 256 != 0 || count > kMaxSeg) return JL_OK;
+    const int S = k / 64;
+    const int nbb = jl_skinny_padded_rows(rows) / 16;
+    int Ss = max_slices(nbb);
+    while (Ss > 4 && S % Ss) Ss -= 4;
+    if (S % Ss) return JL_OK;
+    // up to 16 rows: a workgroup walks two spans itself (no partial sums to fold for rows of up to
+    // 4096 columns); more rows leave no registers for a second set of activation fragments
+    const int zin = (nbb == 1 && (S / Ss) % 2 == 0) ? 2 : 1;
+    const int Z = S / Ss / zin;
+
+    SkinnyParams p{};
+    p.nseg = dual ? 1 : count;
+    int groups = 0, col = 0;
+    const int per_group = dual ? 8 : 16;
+    for (int i = 0; i < p.nseg; i++) {
+        p.w[i] = weights[i]->blocks;
+        p.seg_rows[i] = (int)weights[i]->rows;
+        p.seg_group_begin[i] = groups;
+        p.seg_col_begin[i] = col;
+        groups += ((int)weights[i]->rows + per_group - 1) / per_group;
+        col += (int)weights[i]->rows;
+    }
+    p.seg_group_begin[p.nseg] = groups;
+    p.w_up = dual ? weights[1]->blocks : nullptr;
+    p.X = X;
+    p.C = C;
+    p.planes = planes;
+    p.rows = rows;
+    p.k = k;
+    p.ldo = ldo;
+    p.col_offset = col_offset;
+    p.epilogue = epilogue;
+    p.row_bytes = k / jl_block_elems(type) * jl_block_bytes(type);
+    p.Ss = Ss;
+    p.Z = Z;
+    p.span_bytes = Ss * (type == JL_Q8_0 ? 68 : 36);
+    if (Z > 1 && (size_t)Z * (16 * nbb) * groups * 16 * sizeof(float) > plane_bytes) return JL_OK;
+
+    const int threads = 16 * Ss;   // compute threads; the copy waves come on top
+    const int per_wave = type == JL_Q8_0 ? 18 : 10;
+    const int n_loads = (kGroup * ((p.span_bytes + 16) / 16) + 64 * kDmaWaves - 1) / (64 * kDmaWaves);
+    if (n_loads > per_wave) return JL_OK;
+    const int stage_bytes = n_loads * 64 * kDmaWaves * 16;
+    const int partial = 2 * (threads / 64) * nbb * 1024;
+    int stages = (160 * 1024 - partial) / stage_bytes;
+    if (stages > 4) stages = 4;
+    if (stages < 2) return JL_OK;
+    p.stages = stages;
+    const int lds = partial + stages * stage_bytes;
+    *taken = true;
+
+    switch (type) {
+        case JL_Q8_0:
+            return dual ? launch_nbb<JL_Q8_0, true>(ctx, p, nbb, zin, threads, lds, groups)
+                        : launch_nbb<JL_Q8_0, false>(ctx, p, nbb, zin, threads, lds, groups);
+        case JL_Q4_0:
+            return dual ? launch_nbb<JL_Q4_0, true>(ctx, p, nbb, zin, threads, lds, groups)
+                        : launch_nbb<JL_Q4_0, false>(ctx, p, nbb, zin, threads, lds, groups);
+        case JL_Q4_K:
+            return dual ? launch_nbb<JL_Q4_K, true>(ctx, p, nbb, zin, threads, lds, groups)
+                        : launch_nbb<JL_Q4_K, false>(ctx, p, nbb, zin, threads, lds, groups);
+        default:
+            *taken = false;
+            return JL_OK;
+    }
+}

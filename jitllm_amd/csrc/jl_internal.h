@@ -61,4 +61,9 @@ int jl_launch_fill(jl_context *ctx, float *dst, float value, size_t count);
 int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
                    int epilogue, int math, void *workspace, size_t workspace_bytes);
+// Batched decode (at most 64 rows): the weight-streaming kernel.  `taken` says whether the shape
+// was one it handles; when not, nothing was launched and the tiled GEMM must run instead.
+int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
+                          float *C, int rows, int64_t ldo, int64_t col_offset, int epilogue,
+                          float *planes, size_t plane_bytes, bool *taken);
 size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_cols, int math);
