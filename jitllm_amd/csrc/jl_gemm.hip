@@ -123,6 +123,24 @@ __device__ __forceinline__ void lds_issue_h8n(const uint32_t (&addr)[N], half8 (
     }
 }
 
+// Waits until at most LEFT of the fragment reads issued so far are outstanding (LDS reads return
+// in order) and hands the given arrays, whose reads are then complete, back to the compiler.
+template <int LEFT, int NA, int NBF>
+__device__ __forceinline__ void lds_wait_frags_left(half8 (&a)[NA], half8 (&b)[NBF]) {
+    static_assert(LEFT == 4 || LEFT == 6 || LEFT == 8, "outstanding reads");
+    if constexpr (NA == 4 && NBF == 4) {
+        asm volatile("s_waitcnt lgkmcnt(8)"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]),
+                       "+v"(b[2]), "+v"(b[3]) : : "memory");
+    } else if constexpr (NA == 4 && NBF == 2) {
+        asm volatile("s_waitcnt lgkmcnt(6)"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1])
+                     : : "memory");
+    } else {
+        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]) : : "memory");
+    }
+}
+
 template <int NA, int NBF>
 __device__ __forceinline__ void lds_wait_frags(half8 (&a)[NA], half8 (&b)[NBF]) {
     if constexpr (NA == 4 && NBF == 4) {
@@ -319,10 +337,13 @@ template <> struct Raw<JL_Q8_0> { static constexpr int kRowBytes = 272, kStepByt
 template <> struct Raw<JL_Q4_0> { static constexpr int kRowBytes = 144, kStepBytes = 36; };
 template <> struct Raw<JL_Q4_K> { static constexpr int kRowBytes = 144, kStepBytes = 32; };
 
-// 128-bit loads per thread (256 producer threads) for one raw stage, and the stage's LDS footprint
-// (every load slot has a place of its own, including the few past the last row)
-template <int TYPE> constexpr int raw_loads() { return (BN * Raw<TYPE>::kRowBytes / 16 + 255) / 256; }
-template <int TYPE> constexpr int raw_stage_bytes() { return raw_loads<TYPE>() * 256 * 16; }
+// Threads that do nothing but issue the LDS-DMA loads of both operands (two waves).
+constexpr int kCopyThreads = 128;
+
+// 128-bit loads per copy thread for one raw stage, and the stage's LDS footprint (every load slot
+// has a place of its own, including any past the last row)
+template <int TYPE> constexpr int raw_loads() { return (BN * Raw<TYPE>::kRowBytes / 16 + kCopyThreads - 1) / kCopyThreads; }
+template <int TYPE> constexpr int raw_stage_bytes() { return raw_loads<TYPE>() * kCopyThreads * 16; }
 
 // Activation stages: as many as the 160 KB of LDS leave room for (the Q8_0 raw stages are larger).
 template <int TYPE, int BM> constexpr int a_stages() {
@@ -330,7 +351,7 @@ template <int TYPE, int BM> constexpr int a_stages() {
 }
 
 // Loads that may still be in flight when step s = 4 u + q is awaited (steady state): everything
-// issued after the youngest load the step needs.  Producers issue, in iteration i (after its
+// issued after the youngest load the step needs.  The copy waves issue, in iteration i (after its
 // barrier), first the next raw stage if i % 4 == 0 (RL loads) and then activation step i + AHEAD
 // (NLA loads).  Step s needs activation step s (iteration s - AHEAD) and the raw stage of step s + 1
 // (iteration 4 u - 4, or 4 u when q == 3).
@@ -344,11 +365,15 @@ constexpr int gemm_lds_bytes() {
     return 2 * raw_stage_bytes<TYPE>() + a_stages<TYPE, BM>() * BM * 128 + 2 * W16_BYTES;
 }
 
-// Workgroup: 512 threads = 8 waves, two per SIMD, split by role so that one role's waits are
-// covered by the other's work: waves 0-3 are *producers* (issue the LDS-DMA loads of both operands
-// and decode the raw weight slice of the next step into fp16), waves 4-7 are *consumers* (read the
-// MFMA fragments and run the matrix pipe).  One barrier per 64-column step hands a decoded slice
-// from producers to consumers and a finished stage back.  Tile BM x 128 outputs:
+// Workgroup: 640 threads = 10 waves split by role, so that one role's waits are covered by the
+// others' work:
+//   waves 0-3  *decoders*: turn the raw weight slice of the next step into fp16 in LDS;
+//   waves 4-7  *consumers*: read the MFMA fragments and run the matrix pipe;
+//   waves 8-9  *copiers*: issue the LDS-DMA loads of both operands and wait for them.  An LDS-DMA
+//              load holds its wave at issue while the memory system is busy; in a wave of their
+//              own these stalls cost nobody else anything.
+// One barrier per 64-column step hands a landed stage from the copiers to the decoders, a decoded
+// slice from the decoders to the consumers, and a finished stage back.  Tile BM x 128 outputs:
 //   BM = 128: consumer waves 2 (M) x 2 (N), wave tile 64 x 64
 //   BM <= 64: consumer waves 1 x 4, wave tile BM x 32
 // For JL_SWIGLU the 128 tile columns are 64 gate rows followed by the 64 up rows of the same 64
@@ -359,7 +384,7 @@ constexpr int gemm_lds_bytes() {
 // 16-byte chunks XOR-swizzled by row so that fragment reads are bank-conflict free, fetched every
 // step (three or four stages).  Decoded weights: two buffers of 128 x 64 fp16.
 template <int TYPE, int BM>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ void __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3)))
 jl_gemm_f16(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int RAWB = raw_stage_bytes<TYPE>();
@@ -368,7 +393,7 @@ jl_gemm_f16(GemmParams p) {
     constexpr int RL = raw_loads<TYPE>();   // raw loads per thread and stage
     constexpr int NSA = a_stages<TYPE, BM>();
     constexpr int AHEAD = NSA - 1;          // activation steps in flight ahead of the one in use
-    constexpr int NLA = BM * 8 / 256;       // activation loads per thread and step
+    constexpr int NLA = BM * 8 / kCopyThreads;  // activation loads per copy thread and step
     constexpr int ABYTES = BM * 128;
     constexpr int WM = BM == 128 ? 2 : 1;
     constexpr int WN = 4 / WM;
@@ -381,8 +406,9 @@ jl_gemm_f16(GemmParams p) {
     // the role and the wave index are the same for every lane of a wave: keep them in scalar
     // registers so that the pipeline's bookkeeping (and the waits it selects) stays scalar code
     const int wave8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const bool producer = wave8 < 4;
-    const int tid = threadIdx.x & 255;  // index inside the role
+    const bool decoder = wave8 < 4;
+    const bool copier = wave8 >= 8;
+    const int tid = threadIdx.x & 255;  // index inside the role (decoders, consumers)
     const int lane = tid & 63;
     const int wave = wave8 & 3;
     const int wm = wave / WN, wn = wave % WN;
@@ -426,21 +452,23 @@ jl_gemm_f16(GemmParams p) {
         return true;
     };
 
-    // The two roles are separate loops (with the same barriers in the same order) rather than
-    // branches inside one loop: a wave only ever runs one of them, and written this way the
-    // register allocator sees that their states are never live together.
+    // The roles are separate loops (with the same barriers in the same order) rather than branches
+    // inside one loop: a wave only ever runs one of them, and written this way the register
+    // allocator sees that their states are never live together.
     //
-    // Local step s = 4 u + q uses raw stage u and activation stage s.  Producers issue
+    // Local step s = 4 u + q uses raw stage u and activation stage s.  The copiers issue
     //   at the head of an item   raw(0), A(0 .. AHEAD - 1)
     //   iteration s              [raw(u + 1) when q == 0]  A(s + AHEAD)     -- after the barrier of s
     // and before the barrier of s they wait until only allowed_in_flight(q) loads are outstanding.
-    // Barriers per item: one after the head loads, one per step, one at the end (every LDS read of
-    // the item is done before the next item's loads may land).
+    // The decoders decode step 0 at the head and step s + 1 in iteration s.  Barriers per item: one
+    // after the head loads, one per step, one at the end (every LDS read of the item is done before
+    // the next item's loads may land).
     static_assert(AHEAD >= 2 && AHEAD <= 4, "the wait table covers 2..4 steps of look-ahead");
+    static_assert(AHEAD * NLA + 2 * RL < 64, "outstanding loads must fit the 6-bit counter");
 
-    if (producer) {
-        const int drow = tid & 127;  // decode role: tile row tid % 128, half tid / 128
-        const int dhalf = tid >> 7;
+    if (copier) {
+        const int ctid = threadIdx.x - 512;   // 0 .. kCopyThreads - 1
+        const int cwave = ctid >> 6;
         for (int item = slot; item < items; item += slots) {
             int mt, nt, split;
             if (!locate(item, mt, nt, split)) continue;
@@ -469,21 +497,21 @@ jl_gemm_f16(GemmParams p) {
                 }
                 return base + (int64_t)(vcol - first) * p.row_bytes;
             };
-            // per-thread DMA sources (a slot with nothing to fetch re-reads the first weight bytes)
+            // per-thread DMA sources (a slot with nothing to fetch re-reads its own row 0 chunk)
             const uint8_t *wsrc[RL];
             int wstep[RL];  // bytes a slot's source advances per raw stage: RB, or 0 for a dummy slot
 #pragma unroll
             for (int j = 0; j < RL; j++) {
-                const int i = j * 256 + tid;
+                const int i = j * kCopyThreads + ctid;
                 const int r = i / CPR;
                 const uint8_t *rp = r < BN ? row_ptr(r) : nullptr;
                 wstep[j] = rp ? RB : 0;
-                wsrc[j] = rp ? rp + (int64_t)ubase * RB + (i - r * CPR) * 16 : p.w[0];
+                wsrc[j] = rp ? rp + (int64_t)ubase * RB + (i - r * CPR) * 16 : p.w[0] + (i & 63) * 16;
             }
             const uint8_t *asrc[NLA];
 #pragma unroll
             for (int j = 0; j < NLA; j++) {
-                const int i = j * 256 + tid;
+                const int i = j * kCopyThreads + ctid;
                 const int r = i >> 3, c = i & 7;
                 asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k + (int64_t)ubase * (BK * SUPER)) +
                           ((c ^ ((r >> 1) & 7)) << 4);
@@ -493,25 +521,14 @@ jl_gemm_f16(GemmParams p) {
 #pragma unroll
                 for (int j = 0; j < RL; j++)
                     __builtin_amdgcn_global_load_lds((gvoid *)(wsrc[j] + (int64_t)u * wstep[j]),
-                                                     (lvoid *)(dst + (j * 256 + wave * 64) * 16), 16, 0, 0);
+                                                     (lvoid *)(dst + (j * kCopyThreads + cwave * 64) * 16), 16, 0, 0);
             };
             auto issue_a = [&](int s) {  // activation step s (local index) -> ring slot s % NSA
                 uint8_t *dst = a_ring + (s % NSA) * ABYTES;
 #pragma unroll
                 for (int j = 0; j < NLA; j++)
                     __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)s * 128),
-                                                     (lvoid *)(dst + (j * 256 + wave * 64) * 16), 16, 0, 0);
-            };
-            auto dequant = [&](int s) {
-                half8 v[4];
-                const int u = s / SUPER, q = s % SUPER;
-                const uint32_t row = raw0 + (u & 1) * RAWB + drow * RB;
-                if constexpr (TYPE == JL_Q4_K)
-                    decode_half_slice<TYPE>(row + 16 + q * 32, row, dhalf, q * 2 + dhalf, v);
-                else
-                    decode_half_slice<TYPE>(row + q * Raw<TYPE>::kStepBytes, 0, dhalf, 0, v);
-                lds_write_4xh8(w16_0 + (s & 1) * W16_BYTES + drow * W16_STRIDE +
-                                   (((dhalf * 4) ^ ((drow >> 1) & 7)) << 4), v);
+                                                     (lvoid *)(dst + (j * kCopyThreads + cwave * 64) * 16), 16, 0, 0);
             };
 
             issue_raw(0);
@@ -520,7 +537,6 @@ jl_gemm_f16(GemmParams p) {
                 if (a < ksteps) issue_a(a);
             JL_WAIT_VM(0);
             __builtin_amdgcn_s_barrier();
-            dequant(0);
             for (int s = 0; s < ksteps; s++) {
                 const int u = s / SUPER, q = s % SUPER;
                 const bool last = u + 1 == usteps;
@@ -533,6 +549,33 @@ jl_gemm_f16(GemmParams p) {
                 __builtin_amdgcn_s_barrier();
                 if (q == 0 && !last) issue_raw(u + 1);
                 if (s + AHEAD < ksteps) issue_a(s + AHEAD);
+            }
+            __builtin_amdgcn_s_barrier();
+        }
+        return;
+    }
+
+    if (decoder) {
+        const int drow = tid & 127;  // tile row tid % 128, half tid / 128
+        const int dhalf = tid >> 7;
+        auto dequant = [&](int s) {
+            half8 v[4];
+            const int u = s / SUPER, q = s % SUPER;
+            const uint32_t row = raw0 + (u & 1) * RAWB + drow * RB;
+            if constexpr (TYPE == JL_Q4_K)
+                decode_half_slice<TYPE>(row + 16 + q * 32, row, dhalf, q * 2 + dhalf, v);
+            else
+                decode_half_slice<TYPE>(row + q * Raw<TYPE>::kStepBytes, 0, dhalf, 0, v);
+            lds_write_4xh8(w16_0 + (s & 1) * W16_BYTES + drow * W16_STRIDE +
+                               (((dhalf * 4) ^ ((drow >> 1) & 7)) << 4), v);
+        };
+        for (int item = slot; item < items; item += slots) {
+            int mt, nt, split;
+            if (!locate(item, mt, nt, split)) continue;
+            __builtin_amdgcn_s_barrier();
+            dequant(0);
+            for (int s = 0; s < ksteps; s++) {
+                __builtin_amdgcn_s_barrier();
                 if (s + 1 < ksteps) dequant(s + 1);
             }
             __builtin_amdgcn_s_barrier();
@@ -541,6 +584,8 @@ jl_gemm_f16(GemmParams p) {
     }
 
     // ---- consumers ----
+    // their instructions go first: the matrix pipe is what the other roles exist to feed
+    __builtin_amdgcn_s_setprio(2);
     // LDS row of each of the wave's column blocks
     int brow[NB];
 #pragma unroll
@@ -592,9 +637,11 @@ jl_gemm_f16(GemmParams p) {
         __builtin_amdgcn_s_barrier();
         for (int s = 0; s < ksteps; s++) {
             __builtin_amdgcn_s_barrier();
+            // both halves' reads go out at once; the first half's MFMAs start as soon as its own
+            // fragments are back (LDS reads return in order)
             issue_frags(s, 0);
-            lds_wait_frags<MB, NB>(fa[0], fb[0]);
             issue_frags(s, 1);
+            lds_wait_frags_left<MB + NB>(fa[0], fb[0]);
             mfma_half(0);
             lds_wait_frags<MB, NB>(fa[1], fb[1]);
             mfma_half(1);
@@ -748,7 +795,7 @@ int launch_gemm(jl_context *ctx, const GemmParams &p, dim3 grid) {
         JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         configured[ctx->device] = true;
     }
-    hipLaunchKernelGGL(fn, grid, dim3(512), lds, ctx->stream, p);
+    hipLaunchKernelGGL(fn, grid, dim3(640), lds, ctx->stream, p);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
