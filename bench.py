@@ -265,6 +265,41 @@ def bench_batched_q4k(ctx, hip, B, steps, warmup):
             "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "bytes": wbytes + io}
 
 
+# HBM bytes one gate/up launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
+# `bench.py --traffic-probe` (profiles/gemv_q8_0_gate_up_hbm_traffic.md): 17 522 KiB x 2.0 read
+# (the counter books 64 bytes for each of this chip's 128-byte requests; a 256 MiB plain copy reads
+# 131 087 KiB on it) + 64 KiB x 1.0 written.  The algorithmic figure is 35 733 504 bytes.
+GATE_UP_HBM_TRAFFIC_BYTES = 17522 * 1024 * 2 + 64 * 1024
+
+
+def traffic_probe(ctx, proj, layers):
+    """What `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` are collected on.
+
+    Launches, kernel by kernel (no graph, so every dispatch has a counter row of its own):
+      1. the calibration kernel: a plain device-to-device copy of 256 MiB of floats (torch's
+         elementwise copy kernel), which reads 268 435 456 bytes once and writes as many, so the
+         counters' units and the size of the memory requests they count can be read off a
+         transfer of known size;
+      2. the fused gate/up GEMV of each of the 16 layers (distinct weights, 35 651 584 bytes each),
+         three rounds.
+    Prints the byte counts the counter values are to be compared with.
+    """
+    import torch
+    src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0")
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        for w in layers:
+            proj.gateUp(w["w1"], w["w3"], DIM, HIDDEN)
+    ctx.sync()
+    print(json.dumps({"calibration": {"kernel": "torch copy_ of 64 Mi floats",
+                                      "read_bytes": src.numel() * 4, "write_bytes": src.numel() * 4},
+                      "gate_up": {"algorithmic_read_bytes": 2 * gemv_bytes(HIDDEN, DIM) + 4 * DIM,
+                                  "algorithmic_write_bytes": 4 * HIDDEN}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -272,6 +307,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill / batched legs")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="only launch what the HBM-traffic counters are read on (see traffic_probe)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path is built and measured on a single MI355X; "
@@ -289,6 +326,9 @@ def main():
         layers, wcls, acts, host, shapes = build_decode_set(ctx, t)
         ws = TornadoWorkspace(wrapX=acts["x"], wrapXb=acts["xb"], wrapHb=acts["hb"])
         proj = QuantizedProjections(ctx, ws)
+        if args.traffic_probe:
+            traffic_probe(ctx, proj, layers)
+            return
         total_bytes = decode_bytes()
         assert total_bytes == 1316320256, total_bytes
 
@@ -358,7 +398,7 @@ def main():
             "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
             "roofline": {"bound": "hbm", "kernel": "jl_gemv_tiles<Q8_0, gate/up> 2 x [8192 x 2048]",
                          "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
                          "bytes_per_launch": gate_up_bytes,
                          "avg_launch_us": round(gate_up_avg * 1e3, 3),
                          "launches_timed": len(gate_up_ms)},
