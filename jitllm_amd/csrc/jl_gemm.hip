@@ -749,16 +749,16 @@ size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 namespace {
 
-// Split-K factor for a skinny call (at most 64 activation rows): enough workgroups to cover the
-// chip, at least 2 raw stages (512 columns) per split, and partial-sum traffic (written once, read once)
-// no larger than the weight bytes themselves.  A divisor of the step count.
-int choose_splits(int rows, int k, int ntiles, int row_bytes, int compute_units) {
-    if (rows > 64) return 1;
+// Split-K factor: calls whose tile grid leaves compute units idle cut K across workgroups -- enough
+// work items to cover the chip, at least 2 raw stages (512 columns) per split, and partial-sum
+// traffic (written once, read once) bounded by the weight bytes: splits * padded_rows <=
+// row_bytes / 2.  A divisor of the stage count.
+int choose_splits(int rows, int bm, int k, int tiles, int row_bytes, int compute_units) {
     const int ksteps = k / (BK * SUPER);  // raw stages of 256 columns
-    const int padded = rows <= 32 ? 32 : 64;
-    int want = (2 * compute_units + ntiles - 1) / ntiles;
+    const int padded = (rows + bm - 1) / bm * bm;
+    int want = rows <= 64 ? (2 * compute_units + tiles - 1) / tiles : compute_units / tiles;
     int by_steps = ksteps / 2;
-    int by_traffic = row_bytes / (8 * padded);
+    int by_traffic = row_bytes / (2 * padded);
     int s = want < by_steps ? want : by_steps;
     if (by_traffic < s) s = by_traffic;
     if (s < 1) s = 1;
@@ -772,14 +772,14 @@ size_t scale_bytes(int64_t rows) { return round_up(round_up((size_t)rows, 128) *
 }  // namespace
 
 // Workspace: fp16 activations | row scales | split-K planes.  The planes are bounded by the
-// traffic rule in choose_splits: splits * padded_rows <= row_bytes / 8, so splits * padded_rows *
-// columns * 4 <= columns * row_bytes / 2 with row_bytes <= 34 * cols / 32.
+// traffic rule in choose_splits: splits * padded_rows <= row_bytes / 2, so splits * padded_rows *
+// columns * 4 <= columns * row_bytes * 2 with row_bytes <= 34 * cols / 32.
 size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_cols, int math) {
     if (math == JL_MATH_INT8) {
         size_t padded = round_up((size_t)max_rows, 128);
         return round_up(padded * (size_t)cols, 256) + round_up(padded * (size_t)(cols / 32) * 4, 256);
     }
-    size_t planes = round_up(round_up((size_t)out_cols, 128) * (size_t)cols * 17 / 32 + 64 * 128 * 4, 256);
+    size_t planes = round_up(round_up((size_t)out_cols, 128) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
     return a16_bytes(max_rows, cols) + scale_bytes(max_rows) + planes;
 }
 
@@ -806,7 +806,7 @@ int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows, float *planes, si
     p.ntiles = (p.n_total + cols_per_tile - 1) / cols_per_tile;
     const int bm = rows <= 32 ? 32 : rows <= 64 ? 64 : 128;
     p.mtiles = (rows + bm - 1) / bm;
-    p.splits = choose_splits(rows, p.k, p.ntiles, p.row_bytes, ctx->compute_units);
+    p.splits = choose_splits(rows, bm, p.k, p.ntiles * p.mtiles, p.row_bytes, ctx->compute_units);
     const int64_t plane = (int64_t)p.mtiles * bm * p.ntiles * BN;
     if (p.splits > 1 && (size_t)p.splits * plane * 4 > plane_bytes) p.splits = 1;
     p.partial = planes;
