@@ -155,9 +155,10 @@ int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
  * memory preflight equals what the call uses).  `max_rows` is the largest `batch`, `cols` the
  * largest row length, `out_cols` the largest number of output columns one call produces (a gate/up
  * pair counts both weights' rows), `math` a jl_gemm_math.  The scratch holds the fp16 copy of the
- * activations, one scale per row, and -- for calls of at most 64 rows, which cut K across
- * workgroups -- the partial sums of the cuts.  A smaller workspace that still holds the first two
- * is accepted; such calls simply do not cut K.
+ * activations, one scale per row, and -- for calls whose tile grid would leave compute units idle,
+ * which cut K across workgroups -- the partial sums of the cuts (at most about twice the weight
+ * bytes).  A smaller workspace that still holds the first two is accepted; such calls simply do
+ * not cut K.  Calls of at most 32 rows read X directly and use only the partial sums.
  */
 size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols, int math);
 
@@ -169,7 +170,8 @@ size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols,
  *   X    [batch x cols] fp32 row-major          C  fp32, row stride `ldo` floats
  *   epilogue JL_STORE / JL_RESIDUAL, or JL_SWIGLU with count == 2 (gate, up):
  *            C[b][col_offset + j] = SiLU(X_b.W0_j) * (X_b.W1_j)
- *   math     a jl_gemm_math; JL_MATH_INT8 with a Q4_K weight is JL_ERR_UNSUPPORTED
+ *   math     a jl_gemm_math; JL_MATH_INT8 is JL_ERR_UNSUPPORTED (not built)
+ * The row length must be a multiple of 256 columns, else JL_ERR_UNSUPPORTED.
  * This is Int8GemmKernels.gemmInt8Q8_0's contract (:651-676: epilogue, rowsHolder, ldo,
  * colOffset) and gemmMMAQ8's, behind one call.
  */
