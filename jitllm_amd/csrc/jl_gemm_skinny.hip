@@ -121,15 +121,6 @@ __device__ __forceinline__ floatx4 lds_read_f4(uint32_t addr) {
     return v;
 }
 
-__device__ __forceinline__ void lds_read_8xf4(const uint32_t (&a)[8], floatx4 (&v)[8]) {
-    asm volatile(
-        "ds_read_b128 %0, %8\n\tds_read_b128 %1, %9\n\tds_read_b128 %2, %10\n\tds_read_b128 %3, %11\n\t"
-        "ds_read_b128 %4, %12\n\tds_read_b128 %5, %13\n\tds_read_b128 %6, %14\n\tds_read_b128 %7, %15\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
-        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7]) : "memory");
-}
-
 // ---- slice decode: raw block bytes -> eight fp16 fragments of eight consecutive columns ---------
 //
 // A byte b in 0..255 under the exponent byte 0x64 is the fp16 number 1024 + b, exactly; a packed
@@ -223,7 +214,7 @@ __device__ __forceinline__ void decode_slice(uint32_t row, int sl, half8 (&f)[8]
     }
 }
 
-__device__ __forceinline__ float skinny_swiglu(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+__device__ __forceinline__ float skinny_swiglu(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
 
 // Workgroup = 16 Ss compute threads (Ss / 4 waves) + kDmaWaves waves that do nothing but copy tiles.
 // An LDS-DMA load holds its wave at issue while the memory system is busy; issued from the compute
@@ -394,51 +385,81 @@ __global__ void __launch_bounds__(512 + 64 * kDmaWaves) jl_gemm_skinny(SkinnyPar
 
     // Folds the waves' partial sums of group `group` (parity `par`) and applies the epilogue.  A
     // partial is what one lane of one wave held: weight rows 4 (o / 16) .. + 3 of activation row
-    // 16 b + o % 16, for lane o and row block b.  The (b, o) pairs are dealt out over all compute
-    // waves so that the fold is a few lanes' work in each instead of one wave's critical path.
-    // Gate/up groups: lanes o >= 32 hold the up rows of the outputs of lane o - 32.
+    // 16 b + o % 16, for lane o and row block b; in a gate/up group lanes o >= 32 hold the up rows of
+    // the outputs of lane o - 32.  The (b, o) pairs are dealt out over all compute waves, and inside
+    // a wave one lane reads one wave's partial of one pair: `waves` neighbouring lanes then add up
+    // with DPP moves in a fixed order, the first of them applies the epilogue.  Which lane does what
+    // never changes, so everything that depends on that only is worked out once, here.  (Wave
+    // counts that are not a power of two fold lane by lane instead, `serial` below.)
+    constexpr int kPasses = 2;   // at most 16 float4 sums per wave x 8 waves = 128 lanes' worth
+    const int lanes_out = DUAL ? 32 : 64;
+    const int per = (lanes_out + waves - 1) / waves;     // lanes o per wave
+    const bool serial = (waves & (waves - 1)) != 0;
+    const int wshift = 31 - __builtin_clz(waves | 1);
+    int fin_off[kPasses];      // LDS offset of what this lane reads (inside a parity), or -1
+    int fin_go[kPasses];       // o / 16: which four weight rows
+    bool fin_owner[kPasses];   // this lane applies the epilogue of its pair
+    float *fin_c[kPasses];     // output row of the pair (null when the row is not active)
+    float *fin_plane[kPasses]; // its row in this span's plane
+#pragma unroll
+    for (int ps = 0; ps < kPasses; ps++) {
+        const int idx = ps * 64 + lane;
+        const int wv = serial ? 0 : idx & (waves - 1);       // whose partial
+        const int unit = serial ? idx : idx >> wshift;        // which sum of this wave
+        const int pi = (DUAL && !serial) ? unit >> 1 : unit;  // which (b, o) pair
+        const int half = (DUAL && !serial) ? unit & 1 : 0;    // gate / up
+        const int b = pi / per;
+        const int o = wave * per + (pi - b * per);
+        const bool valid = b < NBB && o < lanes_out;
+        const int m = 16 * b + (o & 15);
+        fin_off[ps] = valid ? wv * (NBB * 1024) + b * 1024 + (o + 32 * half) * 16 : -1;
+        fin_go[ps] = o >> 4;
+        fin_owner[ps] = valid && wv == 0 && half == 0;
+        fin_c[ps] = m < p.rows ? p.C + (int64_t)m * p.ldo + p.col_offset : nullptr;
+        fin_plane[ps] = p.Z > 1 ? p.planes + ((int64_t)z * (16 * NBB) + m) * ((int64_t)total_groups * 16) : nullptr;
+    }
+    auto lane_sum = [&](float v) {   // over `waves` neighbouring lanes, every lane gets the total
+        if (waves >= 2) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
+        if (waves >= 4) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));
+        if (waves >= 8) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));
+        return v;
+    };
     auto finish = [&](int group, int par) {
-        const int lanes_out = DUAL ? 32 : 64;
-        const int per = (lanes_out + waves - 1) / waves;     // lanes o per wave
         const Segment sg = segment_of(group);
-        for (int base = 0; base < per * NBB; base += 64) {
-            const int item = base + lane;
-            const int b = item / per;
-            const int o = wave * per + (item - b * per);
-            if (b >= NBB || o >= lanes_out) continue;
-            const uint32_t pb = lds0 + par * partial_bytes + b * 1024 + o * 16;
+        const uint32_t pbase = lds0 + par * partial_bytes;
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ps++) {
+            if (ps * 64 >= (serial ? per * NBB : (per * NBB * (DUAL ? 2 : 1)) << wshift)) break;   // uniform
             floatx4 sum = {0.f, 0.f, 0.f, 0.f}, sum_up = {0.f, 0.f, 0.f, 0.f};
-            // every wave's partial (there are at most eight waves): all reads in flight, one wait
-            uint32_t a[8];
-            float keep[8];
+            if (serial) {
+                if (fin_off[ps] >= 0) {
+                    for (int w = 0; w < waves; w++) {
+                        sum += lds_read_f4(pbase + fin_off[ps] + w * (NBB * 1024));
+                        if constexpr (DUAL) sum_up += lds_read_f4(pbase + fin_off[ps] + w * (NBB * 1024) + 32 * 16);
+                    }
+                }
+            } else {
+                if (fin_off[ps] >= 0) sum = lds_read_f4(pbase + fin_off[ps]);
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                keep[j] = j < waves ? 1.f : 0.f;
-                a[j] = pb + (j < waves ? j : 0) * (NBB * 1024);
+                for (int e = 0; e < 4; e++) sum[e] = lane_sum(sum[e]);
+                if constexpr (DUAL) {
+                    // the up sums sit `waves` lanes further on
+#pragma unroll
+                    for (int e = 0; e < 4; e++) sum_up[e] = __shfl_down(sum[e], waves, 64);
+                }
             }
-            floatx4 part[8];
-            lds_read_8xf4(a, part);
-#pragma unroll
-            for (int j = 0; j < 8; j++) sum += part[j] * keep[j];
-            if constexpr (DUAL) {
-#pragma unroll
-                for (int j = 0; j < 8; j++) a[j] += 32 * 16;
-                lds_read_8xf4(a, part);
-#pragma unroll
-                for (int j = 0; j < 8; j++) sum_up += part[j] * keep[j];
-            }
-            const int m = 16 * b + (o & 15);
-            const int go = o >> 4;
+            if (!fin_owner[ps]) continue;
+            const int go = fin_go[ps];
             const int local = (group - sg.group_begin) * out_rows + 4 * go;  // first of 4 outputs
             if (p.Z > 1) {
                 // partial sums of this span: [z][row][group * 16 + weight row of the group]
-                float *pp = p.planes + ((int64_t)z * (16 * NBB) + m) * ((int64_t)total_groups * 16) + group * 16 + 4 * go;
+                float *pp = fin_plane[ps] + group * 16 + 4 * go;
                 *(floatx4 *)pp = sum;
                 if constexpr (DUAL) *(floatx4 *)(pp + 8) = sum_up;
                 continue;
             }
-            if (m >= p.rows) continue;
-            float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + sg.col_begin + local;
+            if (!fin_c[ps]) continue;
+            float *dst = fin_c[ps] + sg.col_begin + local;
             const int left = sg.rows - local;
             float v[4];
 #pragma unroll
