@@ -302,7 +302,7 @@ __device__ __forceinline__ void decode_half_slice(uint32_t raw_row, uint32_t hdr
 // form and three orders of magnitude inside the fp16 path's tolerance; the double-precision exp
 // costs about 150 instructions per output, which matters at T x hidden outputs per call.
 __device__ __forceinline__ float gemm_swiglu(float g, float u) {
-    return g / (1.0f + expf(-g)) * u;
+    return g / (1.0f + __expf(-g)) * u;
 }
 
 struct GemmParams {
@@ -679,10 +679,17 @@ jl_gemm_f16(GemmParams p) {
 #pragma unroll
                 for (int j = 0; j < NB / 2; j++) {
                     const int col = n0 + wn * (TN / 2) + j * 16 + (lane >> 4) * 4;
+                    float v[4];
 #pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (col + e < p.n_total)
-                            crow[col + e] = gemm_swiglu(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
+                    for (int e = 0; e < 4; e++) v[e] = gemm_swiglu(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
+                    float *dst = crow + col;
+                    if (col + 3 < p.n_total && (((uintptr_t)dst) & 15) == 0) {
+                        *(float4 *)dst = float4{v[0], v[1], v[2], v[3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (col + e < p.n_total) dst[e] = v[e];
+                    }
                 }
             } else {
 #pragma unroll
@@ -766,8 +773,8 @@ int choose_splits(int rows, int bm, int k, int tiles, int row_bytes, int compute
     return s;
 }
 
-size_t a16_bytes(int64_t rows, int64_t cols) { return round_up(round_up((size_t)rows, 128) * (size_t)cols * 2, 256); }
-size_t scale_bytes(int64_t rows) { return round_up(round_up((size_t)rows, 128) * 4, 256); }
+size_t a16_bytes(int64_t rows, int64_t cols) { return round_up(round_up((size_t)rows, 256) * (size_t)cols * 2, 256); }
+size_t scale_bytes(int64_t rows) { return round_up(round_up((size_t)rows, 256) * 4, 256); }
 
 }  // namespace
 
@@ -780,6 +787,11 @@ size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_
         return round_up(padded * (size_t)cols, 256) + round_up(padded * (size_t)(cols / 32) * 4, 256);
     }
     size_t planes = round_up(round_up((size_t)out_cols, 128) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
+    // calls of a thousand rows or more decode the weights to fp16 once, into the same region
+    if (max_rows >= 1024) {
+        const size_t copy = round_up(jl_dense_copy_bytes((int)cols, (int)out_cols), 256);
+        if (copy > planes) planes = copy;
+    }
     return a16_bytes(max_rows, cols) + scale_bytes(max_rows) + planes;
 }
 
@@ -865,8 +877,19 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
         if (st != JL_OK || taken) return st;
     }
 
-    hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
+    // a thousand rows or more: weights decoded to fp16 once per call, then the plain fp16 GEMM
+    int virt = 0;
+    for (int i = 0; i < count; i++) virt += (int)weights[i]->rows;
+    const int bn = jl_dense_column_tile(rows, k, virt, ctx->compute_units);
+    const bool dense = bn != 0 && jl_dense_copy_bytes(k, virt) <= plane_bytes;
+    const int padded_rows = dense ? (int)round_up((size_t)rows, 256) : padded;
+
+    hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded_rows), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
     JL_HIP(hipGetLastError());
+    if (dense) {
+        return jl_launch_gemm_dense(ctx, weights, count, A, row_scale, C, rows, ldo, col_offset, epilogue,
+                                    (_Float16 *)planes, bn);
+    }
 
     GemmParams p{};
     p.count = count;

@@ -1,0 +1,456 @@
+// Batched prefill over many rows: decode the weights to fp16 once per call, then a plain fp16 GEMM.
+//
+// This is the reference's own two-step shape (dequantize*ToFP16 followed by gemmMMA,
+// J/backend/tornado/kernels/TransformerBatchPrefillKernels.java:917-1076,2325-2363): with a
+// thousand or more activation rows the decode is a small fraction of the call when done once, and
+// the matrix loop without it affords 256-row tiles and 128 x 64 wave tiles, which halve the LDS
+// traffic per flop of the decode-in-the-loop kernel (jl_gemm.hip).  The decoded copy lives in the
+// caller's workspace for the duration of the call; in HBM the weights stay GGUF blocks.
+//
+//   jl_decode_to_f16   raw blocks -> [virtual rows x K] fp16, the host decode rounded once to fp16
+//                      (bit for bit what the fused kernel multiplies with)
+//   jl_gemm_hh<BN>     C = A16 . W16^T on v_mfma_f32_16x16x32_f16, 256 x BN x 32 steps, eight
+//                      identical waves that each bring in their share of both operands by LDS-DMA
+#include "jl_device.h"
+#include "jl_internal.h"
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const void gvoid;
+typedef __attribute__((address_space(3))) void lvoid;
+
+#define JL_WAIT_VM(N) \
+    __builtin_amdgcn_s_waitcnt(((N)&0xF) | (((N) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+// ---- weights -> fp16 ---------------------------------------------------------------------------
+
+__device__ __forceinline__ h2 bytes_to_h2(uint32_t v, uint32_t sel) {
+    return __builtin_bit_cast(h2, __builtin_amdgcn_perm(v, 0x64646464u, sel));
+}
+
+// four bytes in 0..255 offset form -> (byte - bias) * d, four fp16
+__device__ __forceinline__ void dword_scaled(uint32_t v, h2 bias, h2 d, h2 &lo, h2 &hi) {
+    lo = (bytes_to_h2(v, 0x00050004u) - bias) * d;
+    hi = (bytes_to_h2(v, 0x00070006u) - bias) * d;
+}
+
+struct DecodeParams {
+    const uint8_t *w;      // raw blocks of one weight
+    _Float16 *out;         // [virtual rows x k]
+    int rows, k, row_bytes;
+    int first_virtual;     // virtual row of the weight's row 0 (plain layout)
+    int swiglu_half;       // -1 plain; 0 gate / 1 up: row r goes to tile (r / half) * BN + half_sel * half + r % half
+    int half;              // BN / 2 of the GEMM that will read the copy
+};
+
+// One thread decodes 32 consecutive columns of one row (a Q8_0 / Q4_0 block, a Q4_K sub-block).
+// Reads are 2-byte (block scales sit on odd 2-byte boundaries); a 128-byte line serves ~4
+// neighbouring threads, so the cache turns them into whole-line traffic.
+template <int TYPE>
+__global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
+    const int per_row = p.k / 32;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)p.rows * per_row) return;
+    const int r = (int)(idx / per_row);
+    const int blk = (int)(idx - (int64_t)r * per_row);
+    const uint8_t *row = p.w + (int64_t)r * p.row_bytes;
+    int v = p.first_virtual + r;
+    if (p.swiglu_half >= 0) v = (r / p.half) * (2 * p.half) + p.swiglu_half * p.half + r % p.half;
+    h2 o[16];
+    if constexpr (TYPE == JL_Q8_0) {
+        const uint16_t *b = (const uint16_t *)(row + (int64_t)blk * 34);
+        const _Float16 d = __builtin_bit_cast(_Float16, b[0]);
+        const h2 bias = {(_Float16)1152.f, (_Float16)1152.f}, dd = {d, d};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t q = ((uint32_t)b[1 + 2 * i] | ((uint32_t)b[2 + 2 * i] << 16)) ^ 0x80808080u;
+            dword_scaled(q, bias, dd, o[2 * i], o[2 * i + 1]);
+        }
+    } else if constexpr (TYPE == JL_Q4_0) {
+        const uint16_t *b = (const uint16_t *)(row + (int64_t)blk * 18);
+        const _Float16 d = __builtin_bit_cast(_Float16, b[0]);
+        const h2 bias = {(_Float16)1032.f, (_Float16)1032.f}, dd = {d, d};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t q = (uint32_t)b[1 + 2 * i] | ((uint32_t)b[2 + 2 * i] << 16);
+            dword_scaled(q & 0x0F0F0F0Fu, bias, dd, o[2 * i], o[2 * i + 1]);              // elements 4i ..
+            dword_scaled((q >> 4) & 0x0F0F0F0Fu, bias, dd, o[8 + 2 * i], o[9 + 2 * i]);   // 16 + 4i ..
+        }
+    } else {
+        const uint8_t *sb = row + (int64_t)(blk >> 3) * 144;
+        const uint32_t *hdr = (const uint32_t *)sb;
+        const int sub = blk & 7;
+        const float d = jl_half_bits_to_float(hdr[0]);
+        const float dmin = jl_half_bits_to_float(hdr[0] >> 16);
+        int sc, mn;
+        jl_q4k_scale_min(hdr[1], hdr[2], hdr[3], sub, sc, mn);
+        const _Float16 ds = (_Float16)(d * (float)sc), dm = (_Float16)(dmin * (float)mn);
+        const h2 ds2 = {ds, ds}, dm2 = {dm, dm}, bias = {(_Float16)1024.f, (_Float16)1024.f};
+        const uint32_t *qs = (const uint32_t *)(sb + 16 + (sub >> 1) * 32);
+        const int shift = (sub & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t q = (qs[i] >> shift) & 0x0F0F0F0Fu;
+            o[2 * i] = (bytes_to_h2(q, 0x00050004u) - bias) * ds2 - dm2;
+            o[2 * i + 1] = (bytes_to_h2(q, 0x00070006u) - bias) * ds2 - dm2;
+        }
+    }
+    uint4 *dst = (uint4 *)(p.out + (int64_t)v * p.k + blk * 32);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint4 u;
+        u.x = __builtin_bit_cast(uint32_t, o[4 * i]);
+        u.y = __builtin_bit_cast(uint32_t, o[4 * i + 1]);
+        u.z = __builtin_bit_cast(uint32_t, o[4 * i + 2]);
+        u.w = __builtin_bit_cast(uint32_t, o[4 * i + 3]);
+        dst[i] = u;
+    }
+}
+
+// zero rows [first, first + count) of the decoded copy (padding up to the column tile)
+__global__ void __launch_bounds__(256) jl_zero_rows_f16(_Float16 *out, int64_t halfs) {
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (i < halfs) *(uint4 *)(out + i) = uint4{0, 0, 0, 0};
+}
+
+// ---- fp16 GEMM ----------------------------------------------------------------------------------
+
+struct DenseParams {
+    const _Float16 *A;       // [padded rows x k]
+    const _Float16 *W;       // [ntiles * BN x k], virtual row order
+    const float *row_scale;
+    float *C;
+    int rows, k, n_total;    // n_total: output columns (SWIGLU: of one weight)
+    int64_t ldo, col_offset;
+    int epilogue;
+    int ntiles, mtiles;
+};
+
+__device__ __forceinline__ float dense_swiglu(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
+
+constexpr int DBM = 256, DBK = 32, DNS = 5;
+
+// s_waitcnt lgkmcnt(LEFT) that hands the registers whose reads are now complete back to the compiler
+template <int LEFT>
+__device__ __forceinline__ void wait_lgkm(half8 &b0, half8 &b1, half8 &b2, half8 &b3, half8 &a0) {
+    static_assert(LEFT == 3 || LEFT == 7, "reads left in flight");
+    if constexpr (LEFT == 7)
+        asm volatile("s_waitcnt lgkmcnt(7)" : "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3), "+v"(a0) : : "memory");
+    else
+        asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3), "+v"(a0) : : "memory");
+}
+__device__ __forceinline__ void wait_lgkm_one(int left, half8 &a) {
+    switch (left) {
+        case 0: asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a) : : "memory"); break;
+        case 1: asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(a) : : "memory"); break;
+        case 2: asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(a) : : "memory"); break;
+        case 3: asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(a) : : "memory"); break;
+        case 4: asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(a) : : "memory"); break;
+        case 5: asm volatile("s_waitcnt lgkmcnt(5)" : "+v"(a) : : "memory"); break;
+        default: asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(a) : : "memory"); break;
+    }
+}
+
+// LDS stage: A rows then W rows, 64 bytes (four 16-byte chunks) per row; chunk c of row r sits at
+// position c ^ ((r >> 1) & 3): measured, this is the pairing of rows that lets a 128-bit fragment
+// read of 16 rows x 4 chunks run at the full 256 bytes per clock (c ^ (r >> 2) runs at half).
+template <int BN>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+jl_gemm_hh(DenseParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int WM = BN == 256 ? 2 : 4;     // waves along M
+    constexpr int WN = 8 / WM;
+    constexpr int TM = DBM / WM, TN = BN / WN;   // wave tile: 128 x 64 or 64 x 64
+    constexpr int MB = TM / 16, NB = TN / 16;
+    constexpr int STAGE = (DBM + BN) * 64;
+    constexpr int LA = DBM * 4 / 512;          // 16-byte loads per thread and stage, A part
+    constexpr int LW = BN * 4 / 512;
+    static_assert(NB == 4, "four column blocks per wave");
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int wm = wave / WN, wn = wave % WN;
+    const bool swiglu = p.epilogue == JL_SWIGLU;
+    const int cols_per_tile = swiglu ? BN / 2 : BN;
+    const int ksteps = p.k / DBK;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
+
+    // tile order: XCD x (workgroups blockIdx % 8 == x) takes the x-th eighth of the tiles, walked
+    // so that what its workgroups hold at any moment is a patch of few row tiles x many column tiles
+    const int total = p.ntiles * p.mtiles;
+    const int per_xcd = (total + 7) / 8;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = (gridDim.x + 7) >> 3;
+
+    // LDS row of each of the wave's column blocks (SWIGLU: first half of a tile gate, second up)
+    int brow[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        if (swiglu) brow[j] = (j / (NB / 2)) * (BN / 2) + wn * (TN / 2) + (j % (NB / 2)) * 16;
+        else brow[j] = wn * TN + j * 16;
+    }
+    // fragment read addresses inside a stage
+    const int fr = lane & 15, fg = lane >> 4;
+    uint32_t a_off[MB], w_off[NB];
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+        const int r = wm * TM + i * 16 + fr;
+        a_off[i] = r * 64 + ((fg ^ ((r >> 1) & 3)) << 4);
+    }
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        const int r = brow[j] + fr;
+        w_off[j] = DBM * 64 + r * 64 + ((fg ^ ((r >> 1) & 3)) << 4);
+    }
+
+    for (int item = slot; item < per_xcd; item += slots) {
+        const int logical = xcd * per_xcd + item;
+        if (logical >= total) continue;
+        constexpr int GM = 2;
+        const int group = logical / (GM * p.ntiles);
+        const int rest = logical - group * (GM * p.ntiles);
+        const int rows_in_group = p.mtiles - group * GM < GM ? p.mtiles - group * GM : GM;
+        const int nt = rest / rows_in_group;
+        const int mt = group * GM + rest - nt * rows_in_group;
+        const int m0 = mt * DBM;
+
+        // this thread's load slots: slot i = row i / 4, chunk position i % 4 (source chunk swizzled)
+        const uint8_t *asrc[LA], *wsrc[LW];
+#pragma unroll
+        for (int j = 0; j < LA; j++) {
+            const int i = j * 512 + tid, r = i >> 2, c = (i & 3) ^ ((r >> 1) & 3);
+            asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + c * 16;
+        }
+#pragma unroll
+        for (int j = 0; j < LW; j++) {
+            const int i = j * 512 + tid, r = i >> 2, c = (i & 3) ^ ((r >> 1) & 3);
+            wsrc[j] = (const uint8_t *)(p.W + ((int64_t)nt * BN + r) * p.k) + c * 16;
+        }
+        auto issue = [&](int s) {
+            uint8_t *dst = lds + (s % DNS) * STAGE;
+#pragma unroll
+            for (int j = 0; j < LA; j++)
+                __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)s * 64),
+                                                 (lvoid *)(dst + (j * 512 + wave * 64) * 16), 16, 0, 0);
+#pragma unroll
+            for (int j = 0; j < LW; j++)
+                __builtin_amdgcn_global_load_lds((gvoid *)(wsrc[j] + (int64_t)s * 64),
+                                                 (lvoid *)(dst + DBM * 64 + (j * 512 + wave * 64) * 16), 16, 0, 0);
+        };
+
+        floatx4 acc[MB][NB];
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int j = 0; j < NB; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+        // Two groups of four waves (waves w and w + 4 share a SIMD) run half a step apart: while
+        // one group's MFMAs occupy the matrix pipe, the other issues its loads and fragment reads,
+        // whose latency then hides behind the first group's arithmetic.  Two barriers per step
+        // swap the roles.  Step s reads stage s; stage s + 3 is issued in the memory phase of
+        // step s into the slot of stage s - 2, which both groups finished reading at least one
+        // barrier earlier; before the barrier that ends a memory phase every thread has waited for
+        // its loads of stage s + 1.
+        const int grp = wave >> 2;
+        __builtin_amdgcn_s_barrier();   // every LDS read of the previous item is done
+        issue(0);
+        if (ksteps > 1) issue(1);
+        if (ksteps > 2) issue(2);
+        if (ksteps > 2) JL_WAIT_VM(2 * (LA + LW));
+        else if (ksteps > 1) JL_WAIT_VM(LA + LW);
+        else JL_WAIT_VM(0);
+        __builtin_amdgcn_s_barrier();   // stage 0 has landed
+        if (grp == 1) __builtin_amdgcn_s_barrier();
+        for (int s = 0; s < ksteps; s++) {
+            // ---- memory phase
+            if (s + 3 < ksteps) issue(s + 3);
+            const uint32_t base = lds0 + (s % DNS) * STAGE;
+            half8 fa[MB], fb[NB];
+            {
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+                asm volatile("ds_read_b128 %0, %1" : "=&v"(fb[j]) : "v"(base + w_off[j]) : "memory");
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+                asm volatile("ds_read_b128 %0, %1" : "=&v"(fa[i]) : "v"(base + a_off[i]) : "memory");
+            }
+            // stage s + 1 landed (this thread's part); stages s + 2, s + 3 may be in flight
+            if (s + 3 < ksteps) JL_WAIT_VM(2 * (LA + LW));
+            else if (s + 2 < ksteps) JL_WAIT_VM(LA + LW);
+            else JL_WAIT_VM(0);
+            __builtin_amdgcn_s_barrier();
+            // ---- compute phase: LDS reads return in order, so row block i starts as soon as its
+            // own fragment is back
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                if (i == 0)
+                    wait_lgkm<MB - 1>(fb[0], fb[1], fb[2], fb[3], fa[0]);
+                else
+                    wait_lgkm_one(MB - 1 - i, fa[i]);
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+            }
+            __builtin_amdgcn_s_barrier();
+        }
+        if (grp == 0) __builtin_amdgcn_s_barrier();
+
+        // epilogue: a lane holds four consecutive output columns 4 (lane / 16) .. + 3 of activation
+        // row lane % 16 of each block
+        const int n0 = nt * cols_per_tile;
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+            const int m = m0 + wm * TM + i * 16 + (lane & 15);
+            if (m >= p.rows) continue;
+            const float rs = p.row_scale[m];
+            float *crow = p.C + (int64_t)m * p.ldo + p.col_offset;
+            if (swiglu) {
+#pragma unroll
+                for (int j = 0; j < NB / 2; j++) {
+                    const int col = n0 + wn * (TN / 2) + j * 16 + (lane >> 4) * 4;
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = dense_swiglu(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
+                    float *dst = crow + col;
+                    if (col + 3 < p.n_total && (((uintptr_t)dst) & 15) == 0) {
+                        *(float4 *)dst = float4{v[0], v[1], v[2], v[3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (col + e < p.n_total) dst[e] = v[e];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    const int col = n0 + wn * TN + j * 16 + (lane >> 4) * 4;
+                    float4 v = {acc[i][j][0] * rs, acc[i][j][1] * rs, acc[i][j][2] * rs, acc[i][j][3] * rs};
+                    float *dst = crow + col;
+                    if (col + 3 < p.n_total && (((uintptr_t)dst) & 15) == 0) {
+                        if (p.epilogue == JL_RESIDUAL) {
+                            float4 o = *(const float4 *)dst;
+                            v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+                        }
+                        *(float4 *)dst = v;
+                    } else {
+                        const float ve[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            if (col + e < p.n_total) {
+                                if (p.epilogue == JL_RESIDUAL) dst[e] += ve[e];
+                                else dst[e] = ve[e];
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int BN>
+int launch_dense(jl_context *ctx, const DenseParams &p) {
+    auto fn = jl_gemm_hh<BN>;
+    constexpr int lds = DNS * (DBM + BN) * 64;
+    static bool configured[16] = {};
+    if (ctx->device < 16 && !configured[ctx->device]) {
+        JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        configured[ctx->device] = true;
+    }
+    const int items = p.ntiles * p.mtiles;
+    int wgs = items < ctx->compute_units ? items : ctx->compute_units;
+    wgs = (wgs + 7) / 8 * 8;
+    hipLaunchKernelGGL(fn, dim3(wgs), dim3(512), lds, ctx->stream, p);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
+}
+
+template <int TYPE>
+int launch_decode(jl_context *ctx, const DecodeParams &d) {
+    const int64_t threads = (int64_t)d.rows * (d.k / 32);
+    hipLaunchKernelGGL(jl_decode_to_f16<TYPE>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                       ctx->stream, d);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
+}
+
+}  // namespace
+
+// Column tile the dense path would use for a call, 0 when the call is not one for it: it takes a
+// thousand rows or more and enough tiles to give most compute units one (narrow projections keep
+// the decode-in-the-loop kernel, whose 128-row tiles fill the chip better).
+int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int compute_units) {
+    if (rows < 1024 || k % 32 != 0) return 0;
+    const int mtiles = (rows + DBM - 1) / DBM;
+    // 256-wide tiles when they still give every compute unit work, else 128-wide ones
+    if ((int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units) return 256;
+    if ((int64_t)mtiles * ((out_cols_virtual + 127) / 128) * 10 >= (int64_t)compute_units * 7) return 128;
+    return 0;
+}
+
+// Bytes of the decoded copy for `out_cols_virtual` weight rows of `k` columns.
+size_t jl_dense_copy_bytes(int k, int out_cols_virtual) {
+    return ((size_t)(out_cols_virtual + 255) / 256 * 256) * (size_t)k * 2;
+}
+
+int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
+                         const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
+                         int epilogue, _Float16 *copy, int bn) {
+    const int type = weights[0]->type;
+    const int k = (int)weights[0]->cols;
+    const bool swiglu = epilogue == JL_SWIGLU;
+    int n_total = 0;
+    for (int i = 0; i < (swiglu ? 1 : count); i++) n_total += (int)weights[i]->rows;
+    const int virt = swiglu ? 2 * n_total : n_total;
+    const int cols_per_tile = swiglu ? bn / 2 : bn;
+    const int ntiles = (n_total + cols_per_tile - 1) / cols_per_tile;
+
+    // rows of the last tile that no weight row fills
+    if ((int64_t)ntiles * bn > virt) {
+        const int64_t first = swiglu ? (int64_t)(ntiles - 1) * bn : virt;
+        const int64_t halfs = ((int64_t)ntiles * bn - first) * k;
+        hipLaunchKernelGGL(jl_zero_rows_f16, dim3((unsigned)((halfs / 8 + 255) / 256)), dim3(256), 0, ctx->stream,
+                           copy + first * k, halfs);
+        JL_HIP(hipGetLastError());
+    }
+    int first_virtual = 0;
+    for (int i = 0; i < count; i++) {
+        DecodeParams d{};
+        d.w = weights[i]->blocks;
+        d.out = copy;
+        d.rows = (int)weights[i]->rows;
+        d.k = k;
+        d.row_bytes = k / jl_block_elems(type) * jl_block_bytes(type);
+        d.first_virtual = first_virtual;
+        d.swiglu_half = swiglu ? i : -1;
+        d.half = bn / 2;
+        first_virtual += d.rows;
+        int st;
+        switch (type) {
+            case JL_Q8_0: st = launch_decode<JL_Q8_0>(ctx, d); break;
+            case JL_Q4_0: st = launch_decode<JL_Q4_0>(ctx, d); break;
+            case JL_Q4_K: st = launch_decode<JL_Q4_K>(ctx, d); break;
+            default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
+        }
+        if (st != JL_OK) return st;
+    }
+
+    DenseParams p{};
+    p.A = A;
+    p.W = copy;
+    p.row_scale = row_scale;
+    p.C = C;
+    p.rows = rows;
+    p.k = k;
+    p.n_total = n_total;
+    p.ldo = ldo;
+    p.col_offset = col_offset;
+    p.epilogue = epilogue;
+    p.ntiles = ntiles;
+    p.mtiles = (rows + DBM - 1) / DBM;
+    int st = bn == 256 ? launch_dense<256>(ctx, p) : launch_dense<128>(ctx, p);
+    return st;
+}

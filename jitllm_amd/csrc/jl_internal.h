@@ -66,4 +66,10 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
 int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                           float *C, int rows, int64_t ldo, int64_t col_offset, int epilogue,
                           float *planes, size_t plane_bytes, bool *taken);
+// Many-row prefill: weights decoded to fp16 once per call into `copy`, then a plain fp16 GEMM.
+int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int compute_units);
+size_t jl_dense_copy_bytes(int k, int out_cols_virtual);
+int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
+                         const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
+                         int epilogue, _Float16 *copy, int bn);
 size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_cols, int math);

@@ -130,6 +130,67 @@ def test_batched_gate_up(ctx, t, d, n, T):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
 
 
+@pytest.mark.parametrize("t,d,n,T,residual", [
+    (O.Q8_0, 300, 512, 1100, False), (O.Q8_0, 300, 512, 1100, True), (O.Q4_K, 136, 1024, 1024, False),
+    (O.Q8_0, 16384, 256, 1024, False),
+])
+def test_many_row_prefill_matches_oracle(ctx, t, d, n, T, residual):
+    """A thousand rows or more: weights decoded to fp16 once per call, then the plain fp16 GEMM
+    (dequantize*ToFP16 + gemmMMA, TransformerBatchPrefillKernels.java:917-1076,2325-2363).  Same
+    arithmetic as the fused kernel, so the same bound; the last shape takes the 256-wide tiles."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("many-row prefill", NAMES[t], d, n, T, residual)
+    raw = synthetic.weight(t, d, n, seed=7300 + d)
+    X = synthetic.activations((T, n), seed=7400 + T)
+    ref = O.matmul_batch(t, raw, X, d, n)
+    out = ctx.float_array(T * d, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, d).projection(ctx.from_numpy(X), out, ctx.load_weight(t, raw, d, n),
+                                                       n, d, residual)
+    ctx.sync()
+    got = out.get().reshape(T, d)
+    want = ref + (UNTOUCHED if residual else np.float32(0))
+    err = rel_err(got, want, magnitude(t, raw, X, d, n) + (12345.5 * 6e-8 if residual else 0))
+    assert err < 2e-4, err
+
+
+def test_many_row_prefill_qkv_and_gate_up(ctx):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("many-row prefill qkv / gate_up")
+    t, n, T = O.Q4_0, 512, 1024
+    dims = (256, 96, 96)
+    raws = [synthetic.weight(t, d, n, seed=181 + i) for i, d in enumerate(dims)]
+    X = synthetic.activations((T, n), seed=185)
+    ws = [ctx.load_weight(t, r, d, n) for r, d in zip(raws, dims)]
+    ld = sum(dims)
+    out = ctx.float_array(T * ld, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, ld).fusedQKV(ctx.from_numpy(X), out, *ws)
+    ctx.sync()
+    got = out.get().reshape(T, ld)
+    col = 0
+    for raw, d in zip(raws, dims):
+        ref = O.matmul_batch(t, raw, X, d, n)
+        assert rel_err(got[:, col:col + d], ref, magnitude(t, raw, X, d, n)) < 2e-4
+        col += d
+    # gate/up with SwiGLU; 200 outputs do not fill the last tile
+    t, d, n, T = O.Q4_K, 200, 512, 1030
+    r1 = synthetic.weight(t, d, n, seed=191)
+    r3 = synthetic.weight(t, d, n, seed=192)
+    X = synthetic.activations((T, n), seed=193)
+    g = O.matmul_batch(t, r1, X, d, n)
+    u = O.matmul_batch(t, r3, X, d, n)
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(T, d)
+    hb = ctx.float_array(T * d, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, 2 * d).gateUp(ctx.from_numpy(X), hb, ctx.load_weight(t, r1, d, n),
+                                                ctx.load_weight(t, r3, d, n), n, d)
+    ctx.sync()
+    got = hb.get().reshape(T, d)
+    mg, mu = magnitude(t, r1, X, d, n), magnitude(t, r3, X, d, n)
+    bound = 2e-4 * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
+
+
 def test_huge_activation_rows_stay_finite(ctx):
     """Rows far outside fp16's range are rescaled by a power of two, not turned into infinities."""
     from jitllm_amd import synthetic
