@@ -50,7 +50,10 @@ def test_argument_checks_need_no_device(lib):
     assert lib.jl_gemm_workspace_bytes(100, 2048, 0, L.JL_MATH_F16) >= 128 * 2048 * 2
     # split-K planes grow with the output width, never beyond about twice the weight bytes
     wide = lib.jl_gemm_workspace_bytes(64, 4096, 12288, L.JL_MATH_F16)
-    assert f16 < wide <= 128 * 4096 * 2 + 1024 + 12288 * 4096 * 17 // 8 + (1 << 17)
+    assert f16 < wide <= 256 * 4096 * 2 + 2048 + 12288 * 4096 * 17 // 8 + (1 << 17)
+    # a thousand rows or more: room for the fp16 copy of the widest call's weights
+    many = lib.jl_gemm_workspace_bytes(2048, 2048, 16384, L.JL_MATH_F16)
+    assert many >= 2048 * 2048 * 2 + 16384 * 2048 * 2
     assert lib.jl_gemm_workspace_bytes(64, 4096, 12288, L.JL_MATH_DEFAULT) == wide
 
 
