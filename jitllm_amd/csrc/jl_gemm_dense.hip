@@ -131,32 +131,23 @@ struct DenseParams {
 
 __device__ __forceinline__ float dense_swiglu(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
 
-constexpr int DBM = 256, DBK = 32, DNS = 5;
+constexpr int DBM = 256, DBK = 64;
 
-// s_waitcnt lgkmcnt(LEFT) that hands the registers whose reads are now complete back to the compiler
-template <int LEFT>
-__device__ __forceinline__ void wait_lgkm(half8 &b0, half8 &b1, half8 &b2, half8 &b3, half8 &a0) {
-    static_assert(LEFT == 3 || LEFT == 7, "reads left in flight");
-    if constexpr (LEFT == 7)
-        asm volatile("s_waitcnt lgkmcnt(7)" : "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3), "+v"(a0) : : "memory");
+// hands fragment registers whose reads are complete back to the compiler
+template <int N>
+__device__ __forceinline__ void lds_settle(half8 (&f)[N]) {
+    if constexpr (N == 8)
+        asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]));
     else
-        asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3), "+v"(a0) : : "memory");
-}
-__device__ __forceinline__ void wait_lgkm_one(int left, half8 &a) {
-    switch (left) {
-        case 0: asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a) : : "memory"); break;
-        case 1: asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(a) : : "memory"); break;
-        case 2: asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(a) : : "memory"); break;
-        case 3: asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(a) : : "memory"); break;
-        case 4: asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(a) : : "memory"); break;
-        case 5: asm volatile("s_waitcnt lgkmcnt(5)" : "+v"(a) : : "memory"); break;
-        default: asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(a) : : "memory"); break;
-    }
+        asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
 }
 
-// LDS stage: A rows then W rows, 64 bytes (four 16-byte chunks) per row; chunk c of row r sits at
-// position c ^ ((r >> 1) & 3): measured, this is the pairing of rows that lets a 128-bit fragment
-// read of 16 rows x 4 chunks run at the full 256 bytes per clock (c ^ (r >> 2) runs at half).
+// LDS stage: A rows then W rows, 128 bytes (eight 16-byte chunks) per row; chunk c of row r sits
+// at position c ^ ((r >> 1) & 7) -- measured, this pairing of rows lets a 128-bit fragment read of
+// 16 rows x 4 chunks run at the full 256 bytes per clock.  A step is 64 columns = two MFMA
+// k-blocks: the second block's fragments are read while the first block's MFMAs run, one barrier
+// per step.  BN = 256: two stages of 64 KB (the next step's loads are issued right after the
+// barrier and have the whole step to land); BN = 128: three stages of 48 KB.
 template <int BN>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 jl_gemm_hh(DenseParams p) {
@@ -165,9 +156,11 @@ jl_gemm_hh(DenseParams p) {
     constexpr int WN = 8 / WM;
     constexpr int TM = DBM / WM, TN = BN / WN;   // wave tile: 128 x 64 or 64 x 64
     constexpr int MB = TM / 16, NB = TN / 16;
-    constexpr int STAGE = (DBM + BN) * 64;
-    constexpr int LA = DBM * 4 / 512;          // 16-byte loads per thread and stage, A part
-    constexpr int LW = BN * 4 / 512;
+    constexpr int STAGE = (DBM + BN) * 128;
+    constexpr int NS = BN == 256 ? 2 : 3;
+    constexpr int AHEAD = NS - 1;
+    constexpr int LA = DBM * 8 / 512;          // 16-byte loads per thread and stage, A part
+    constexpr int LW = BN * 8 / 512;
     static_assert(NB == 4, "four column blocks per wave");
 
     const int tid = threadIdx.x;
@@ -192,18 +185,19 @@ jl_gemm_hh(DenseParams p) {
         if (swiglu) brow[j] = (j / (NB / 2)) * (BN / 2) + wn * (TN / 2) + (j % (NB / 2)) * 16;
         else brow[j] = wn * TN + j * 16;
     }
-    // fragment read addresses inside a stage
+    // fragment read addresses inside a stage, k-block 0; k-block 1 is the same row, chunk + 4
     const int fr = lane & 15, fg = lane >> 4;
-    uint32_t a_off[MB], w_off[NB];
-#pragma unroll
-    for (int i = 0; i < MB; i++) {
-        const int r = wm * TM + i * 16 + fr;
-        a_off[i] = r * 64 + ((fg ^ ((r >> 1) & 3)) << 4);
+    // (row block i of the wave sits 16 rows = 2048 bytes further on with the same swizzle key, so
+    // the A fragments need one address register and immediate offsets)
+    uint32_t a_off0, w_off[NB];
+    {
+        const int r = wm * TM + fr;
+        a_off0 = r * 128 + ((fg ^ ((r >> 1) & 7)) << 4);
     }
 #pragma unroll
     for (int j = 0; j < NB; j++) {
         const int r = brow[j] + fr;
-        w_off[j] = DBM * 64 + r * 64 + ((fg ^ ((r >> 1) & 3)) << 4);
+        w_off[j] = DBM * 128 + r * 128 + ((fg ^ ((r >> 1) & 7)) << 4);
     }
 
     for (int item = slot; item < per_xcd; item += slots) {
@@ -217,28 +211,28 @@ jl_gemm_hh(DenseParams p) {
         const int mt = group * GM + rest - nt * rows_in_group;
         const int m0 = mt * DBM;
 
-        // this thread's load slots: slot i = row i / 4, chunk position i % 4 (source chunk swizzled)
+        // this thread's load slots: slot i = row i / 8, chunk position i % 8 (source chunk swizzled)
         const uint8_t *asrc[LA], *wsrc[LW];
 #pragma unroll
         for (int j = 0; j < LA; j++) {
-            const int i = j * 512 + tid, r = i >> 2, c = (i & 3) ^ ((r >> 1) & 3);
+            const int i = j * 512 + tid, r = i >> 3, c = (i & 7) ^ ((r >> 1) & 7);
             asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + c * 16;
         }
 #pragma unroll
         for (int j = 0; j < LW; j++) {
-            const int i = j * 512 + tid, r = i >> 2, c = (i & 3) ^ ((r >> 1) & 3);
+            const int i = j * 512 + tid, r = i >> 3, c = (i & 7) ^ ((r >> 1) & 7);
             wsrc[j] = (const uint8_t *)(p.W + ((int64_t)nt * BN + r) * p.k) + c * 16;
         }
         auto issue = [&](int s) {
-            uint8_t *dst = lds + (s % DNS) * STAGE;
+            uint8_t *dst = lds + (s % NS) * STAGE;
 #pragma unroll
             for (int j = 0; j < LA; j++)
-                __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)s * 64),
+                __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)s * 128),
                                                  (lvoid *)(dst + (j * 512 + wave * 64) * 16), 16, 0, 0);
 #pragma unroll
             for (int j = 0; j < LW; j++)
-                __builtin_amdgcn_global_load_lds((gvoid *)(wsrc[j] + (int64_t)s * 64),
-                                                 (lvoid *)(dst + DBM * 64 + (j * 512 + wave * 64) * 16), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gvoid *)(wsrc[j] + (int64_t)s * 128),
+                                                 (lvoid *)(dst + DBM * 128 + (j * 512 + wave * 64) * 16), 16, 0, 0);
         };
 
         floatx4 acc[MB][NB];
@@ -247,56 +241,50 @@ jl_gemm_hh(DenseParams p) {
 #pragma unroll
             for (int j = 0; j < NB; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-        // Two groups of four waves (waves w and w + 4 share a SIMD) run half a step apart: while
-        // one group's MFMAs occupy the matrix pipe, the other issues its loads and fragment reads,
-        // whose latency then hides behind the first group's arithmetic.  Two barriers per step
-        // swap the roles.  Step s reads stage s; stage s + 3 is issued in the memory phase of
-        // step s into the slot of stage s - 2, which both groups finished reading at least one
-        // barrier earlier; before the barrier that ends a memory phase every thread has waited for
-        // its loads of stage s + 1.
-        const int grp = wave >> 2;
         __builtin_amdgcn_s_barrier();   // every LDS read of the previous item is done
-        issue(0);
-        if (ksteps > 1) issue(1);
-        if (ksteps > 2) issue(2);
-        if (ksteps > 2) JL_WAIT_VM(2 * (LA + LW));
-        else if (ksteps > 1) JL_WAIT_VM(LA + LW);
-        else JL_WAIT_VM(0);
-        __builtin_amdgcn_s_barrier();   // stage 0 has landed
-        if (grp == 1) __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int a = 0; a < AHEAD; a++)
+            if (a < ksteps) issue(a);
         for (int s = 0; s < ksteps; s++) {
-            // ---- memory phase
-            if (s + 3 < ksteps) issue(s + 3);
-            const uint32_t base = lds0 + (s % DNS) * STAGE;
-            half8 fa[MB], fb[NB];
-            {
-#pragma unroll
-            for (int j = 0; j < NB; j++)
-                asm volatile("ds_read_b128 %0, %1" : "=&v"(fb[j]) : "v"(base + w_off[j]) : "memory");
-#pragma unroll
-            for (int i = 0; i < MB; i++)
-                asm volatile("ds_read_b128 %0, %1" : "=&v"(fa[i]) : "v"(base + a_off[i]) : "memory");
-            }
-            // stage s + 1 landed (this thread's part); stages s + 2, s + 3 may be in flight
-            if (s + 3 < ksteps) JL_WAIT_VM(2 * (LA + LW));
-            else if (s + 2 < ksteps) JL_WAIT_VM(LA + LW);
+            // stage s landed (this thread's part); the AHEAD - 1 younger stages may be in flight
+            if (AHEAD == 2 && s + 1 < ksteps) JL_WAIT_VM(LA + LW);
             else JL_WAIT_VM(0);
             __builtin_amdgcn_s_barrier();
-            // ---- compute phase: LDS reads return in order, so row block i starts as soon as its
-            // own fragment is back
+            // the slot of stage s - 1 was last read before this barrier
+            if (s + AHEAD < ksteps) issue(s + AHEAD);
+            const uint32_t base = lds0 + (s % NS) * STAGE;
+            half8 fa[2][MB], fb[2][NB];
 #pragma unroll
-            for (int i = 0; i < MB; i++) {
-                if (i == 0)
-                    wait_lgkm<MB - 1>(fb[0], fb[1], fb[2], fb[3], fa[0]);
-                else
-                    wait_lgkm_one(MB - 1 - i, fa[i]);
+            for (int h = 0; h < 2; h++) {
+                // k-block h: chunk position of chunk (4 h + fg) is the k-block-0 position ^ (4 h)
 #pragma unroll
                 for (int j = 0; j < NB; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                    asm volatile("ds_read_b128 %0, %1" : "=&v"(fb[h][j]) : "v"((base + w_off[j]) ^ (h << 6)) : "memory");
+                const uint32_t aa = (base + a_off0) ^ (h << 6);
+#pragma unroll
+                for (int i = 0; i < MB; i++)
+                    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(fa[h][i]) : "v"(aa), "n"(i * 2048) : "memory");
             }
-            __builtin_amdgcn_s_barrier();
+            // LDS reads return in order: the first k-block's MB + NB fragments are back when that
+            // many of the second's are still outstanding
+            if constexpr (MB == 8) asm volatile("s_waitcnt lgkmcnt(12)" ::: "memory");
+            else asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+            lds_settle(fa[0]);
+            lds_settle(fb[0]);
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[0][j], fa[0][i], acc[i][j], 0, 0, 0);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            lds_settle(fa[1]);
+            lds_settle(fb[1]);
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
         }
-        if (grp == 0) __builtin_amdgcn_s_barrier();
 
         // epilogue: a lane holds four consecutive output columns 4 (lane / 16) .. + 3 of activation
         // row lane % 16 of each block
@@ -354,7 +342,7 @@ jl_gemm_hh(DenseParams p) {
 template <int BN>
 int launch_dense(jl_context *ctx, const DenseParams &p) {
     auto fn = jl_gemm_hh<BN>;
-    constexpr int lds = DNS * (DBM + BN) * 64;
+    constexpr int lds = (BN == 256 ? 2 : 3) * (DBM + BN) * 128;
     static bool configured[16] = {};
     if (ctx->device < 16 && !configured[ctx->device]) {
         JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -383,7 +371,7 @@ int launch_decode(jl_context *ctx, const DecodeParams &d) {
 // thousand rows or more and enough tiles to give most compute units one (narrow projections keep
 // the decode-in-the-loop kernel, whose 128-row tiles fill the chip better).
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int compute_units) {
-    if (rows < 1024 || k % 32 != 0) return 0;
+    if (rows < 1024 || k % 64 != 0) return 0;
     const int mtiles = (rows + DBM - 1) / DBM;
     // 256-wide tiles when they still give every compute unit work, else 128-wide ones
     if ((int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units) return 256;
