@@ -31,10 +31,13 @@ constexpr int kMaxWeights = 8;
 
 // One workgroup per row: scale = the power of two that brings the row's largest magnitude into
 // [2^11, 2^12); a16 = half(x / scale) (the division is exact).  Rows past `rows` are zero-filled.
+// A row of up to 8192 columns is read once and kept in registers between the two passes (largest
+// magnitude, conversion); longer rows are read twice.
 __global__ void __launch_bounds__(256)
 jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__restrict__ row_scale,
                int rows, int k) {
     __shared__ float wave_max[4];
+    constexpr int kHeld = 8;   // float4 per thread held in registers: 256 x 8 x 4 = 8192 columns
     const int row = blockIdx.x;
     const int tid = threadIdx.x;
     _Float16 *a = A + (int64_t)row * k;
@@ -44,10 +47,21 @@ jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__r
         return;
     }
     const float *x = X + (int64_t)row * k;
+    const bool held = k <= kHeld * 1024;
+    float4 v[kHeld];
     float amax = 0.f;
-    for (int i = tid * 4; i < k; i += 1024) {
-        float4 v = *(const float4 *)(x + i);
-        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    if (held) {
+#pragma unroll
+        for (int j = 0; j < kHeld; j++) {
+            const int i = tid * 4 + j * 1024;
+            v[j] = i < k ? *(const float4 *)(x + i) : float4{0.f, 0.f, 0.f, 0.f};
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[j].x), fabsf(v[j].y)), fmaxf(fabsf(v[j].z), fabsf(v[j].w))));
+        }
+    } else {
+        for (int i = tid * 4; i < k; i += 1024) {
+            float4 w = *(const float4 *)(x + i);
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(w.x), fabsf(w.y)), fmaxf(fabsf(w.z), fabsf(w.w))));
+        }
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, JL_WAVE));
@@ -65,11 +79,20 @@ jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__r
         scale = ldexpf(1.f, e - 12);
         inv = ldexpf(1.f, 12 - e);
     }
-    for (int i = tid * 4; i < k; i += 1024) {
-        float4 v = *(const float4 *)(x + i);
-        half4 h = {(_Float16)(v.x * inv), (_Float16)(v.y * inv), (_Float16)(v.z * inv),
-                   (_Float16)(v.w * inv)};
-        *(half4 *)(a + i) = h;
+    if (held) {
+#pragma unroll
+        for (int j = 0; j < kHeld; j++) {
+            const int i = tid * 4 + j * 1024;
+            if (i < k)
+                *(half4 *)(a + i) = half4{(_Float16)(v[j].x * inv), (_Float16)(v[j].y * inv),
+                                          (_Float16)(v[j].z * inv), (_Float16)(v[j].w * inv)};
+        }
+    } else {
+        for (int i = tid * 4; i < k; i += 1024) {
+            float4 w = *(const float4 *)(x + i);
+            *(half4 *)(a + i) = half4{(_Float16)(w.x * inv), (_Float16)(w.y * inv), (_Float16)(w.z * inv),
+                                      (_Float16)(w.w * inv)};
+        }
     }
     if (tid == 0) row_scale[row] = scale;
 }
