@@ -811,9 +811,14 @@ size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_
     }
     size_t planes = round_up(round_up((size_t)out_cols, 128) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
     // calls of a thousand rows or more decode the weights to fp16 once, into the same region
+    // (and, for narrow projections with long rows, two planes of partial sums; such calls have at
+    // most 0.35 x 256 compute units' worth of 256 x 128 tiles)
     if (max_rows >= 1024) {
-        const size_t copy = round_up(jl_dense_copy_bytes((int)cols, (int)out_cols), 256);
-        if (copy > planes) planes = copy;
+        size_t two = jl_dense_plane_bytes((int)max_rows, (int)out_cols);
+        const size_t cap = 2 * (size_t)90 * 256 * 128 * sizeof(float);
+        if (two > cap) two = cap;
+        const size_t need = round_up(jl_dense_copy_bytes((int)cols, (int)out_cols), 256) + two;
+        if (need > planes) planes = need;
     }
     return a16_bytes(max_rows, cols) + scale_bytes(max_rows) + planes;
 }
@@ -865,6 +870,15 @@ int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows, float *planes, si
 
 }  // namespace
 
+int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row_scale, float *C, int rows,
+                          int n_total, int ntiles, int64_t plane, int splits, int64_t ldo, int64_t col_offset,
+                          int epilogue) {
+    hipLaunchKernelGGL(jl_gemm_reduce, dim3((n_total + 255) / 256, rows), dim3(256), 0, ctx->stream, planes,
+                       row_scale, C, rows, n_total, ntiles, plane, splits, ldo, col_offset, epilogue);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
+}
+
 int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
                    int epilogue, int math, void *workspace, size_t workspace_bytes) {
@@ -903,15 +917,17 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     // a thousand rows or more: weights decoded to fp16 once per call, then the plain fp16 GEMM
     int virt = 0;
     for (int i = 0; i < count; i++) virt += (int)weights[i]->rows;
-    const int bn = jl_dense_column_tile(rows, k, virt, ctx->compute_units);
-    const bool dense = bn != 0 && jl_dense_copy_bytes(k, virt) <= plane_bytes;
+    int dsplits = 1;
+    const int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits);
+    const size_t copy_bytes = round_up(jl_dense_copy_bytes(k, virt), 256);
+    const bool dense = bn != 0 && copy_bytes + (dsplits > 1 ? jl_dense_plane_bytes(rows, virt) : 0) <= plane_bytes;
     const int padded_rows = dense ? (int)round_up((size_t)rows, 256) : padded;
 
     hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded_rows), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
     JL_HIP(hipGetLastError());
     if (dense) {
         return jl_launch_gemm_dense(ctx, weights, count, A, row_scale, C, rows, ldo, col_offset, epilogue,
-                                    (_Float16 *)planes, bn);
+                                    (_Float16 *)planes, bn, dsplits, (float *)((uint8_t *)planes + copy_bytes));
     }
 
     GemmParams p{};

@@ -127,6 +127,8 @@ struct DenseParams {
     int64_t ldo, col_offset;
     int epilogue;
     int ntiles, mtiles;
+    int splits;              // K is cut into `splits` equal runs of steps, one work item each
+    float *partial;          // splits > 1: [splits][mtiles * 256][ntiles * BN] fp32 partial sums
 };
 
 __device__ __forceinline__ float dense_swiglu(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
@@ -169,7 +171,7 @@ jl_gemm_hh(DenseParams p) {
     const int wm = wave / WN, wn = wave % WN;
     const bool swiglu = p.epilogue == JL_SWIGLU;
     const int cols_per_tile = swiglu ? BN / 2 : BN;
-    const int ksteps = p.k / DBK;
+    const int ksteps = p.k / DBK / p.splits;   // steps of one work item
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
 
     // tile order: XCD x (workgroups blockIdx % 8 == x) takes the x-th eighth of the tiles, walked
@@ -200,9 +202,11 @@ jl_gemm_hh(DenseParams p) {
         w_off[j] = DBM * 128 + r * 128 + ((fg ^ ((r >> 1) & 7)) << 4);
     }
 
-    for (int item = slot; item < per_xcd; item += slots) {
-        const int logical = xcd * per_xcd + item;
+    for (int item = slot; item < per_xcd * p.splits; item += slots) {
+        const int split = item / per_xcd;
+        const int logical = xcd * per_xcd + (item - split * per_xcd);
         if (logical >= total) continue;
+        const int64_t kbytes = (int64_t)split * ksteps * (DBK * 2);   // first column of this run, in bytes
         constexpr int GM = 2;
         const int group = logical / (GM * p.ntiles);
         const int rest = logical - group * (GM * p.ntiles);
@@ -216,12 +220,12 @@ jl_gemm_hh(DenseParams p) {
 #pragma unroll
         for (int j = 0; j < LA; j++) {
             const int i = j * 512 + tid, r = i >> 3, c = (i & 7) ^ ((r >> 1) & 7);
-            asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + c * 16;
+            asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + kbytes + c * 16;
         }
 #pragma unroll
         for (int j = 0; j < LW; j++) {
             const int i = j * 512 + tid, r = i >> 3, c = (i & 7) ^ ((r >> 1) & 7);
-            wsrc[j] = (const uint8_t *)(p.W + ((int64_t)nt * BN + r) * p.k) + c * 16;
+            wsrc[j] = (const uint8_t *)(p.W + ((int64_t)nt * BN + r) * p.k) + kbytes + c * 16;
         }
         auto issue = [&](int s) {
             uint8_t *dst = lds + (s % NS) * STAGE;
@@ -289,6 +293,23 @@ jl_gemm_hh(DenseParams p) {
         // epilogue: a lane holds four consecutive output columns 4 (lane / 16) .. + 3 of activation
         // row lane % 16 of each block
         const int n0 = nt * cols_per_tile;
+        if (p.splits > 1) {
+            // partial sums of this run of K: plain 16-byte stores into the plane of this split; the
+            // planes are added in split order and the epilogue applied by the reduce kernel
+            const int64_t width = (int64_t)p.ntiles * BN;
+            float *pp = p.partial + (int64_t)split * p.mtiles * DBM * width;
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                const int m = m0 + wm * TM + i * 16 + (lane & 15);
+                float *prow = pp + (int64_t)m * width + nt * BN;
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    const int c = brow[j] + (lane >> 4) * 4;
+                    *(float4 *)(prow + c) = float4{acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+                }
+            }
+            continue;
+        }
 #pragma unroll
         for (int i = 0; i < MB; i++) {
             const int m = m0 + wm * TM + i * 16 + (lane & 15);
@@ -348,7 +369,7 @@ int launch_dense(jl_context *ctx, const DenseParams &p) {
         JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         configured[ctx->device] = true;
     }
-    const int items = p.ntiles * p.mtiles;
+    const int items = p.ntiles * p.mtiles * p.splits;
     int wgs = items < ctx->compute_units ? items : ctx->compute_units;
     wgs = (wgs + 7) / 8 * 8;
     hipLaunchKernelGGL(fn, dim3(wgs), dim3(512), lds, ctx->stream, p);
@@ -368,15 +389,27 @@ int launch_decode(jl_context *ctx, const DecodeParams &d) {
 }  // namespace
 
 // Column tile the dense path would use for a call, 0 when the call is not one for it: it takes a
-// thousand rows or more and enough tiles to give most compute units one (narrow projections keep
-// the decode-in-the-loop kernel, whose 128-row tiles fill the chip better).
-int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int compute_units) {
+// thousand rows or more and enough work items to give most compute units one.  Narrow projections
+// with long rows get there by cutting K in two (*splits = 2, plain store / residual only); what is
+// still too small keeps the decode-in-the-loop kernel, whose 128-row tiles fill the chip better.
+int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits) {
+    *splits = 1;
     if (rows < 1024 || k % 64 != 0) return 0;
     const int mtiles = (rows + DBM - 1) / DBM;
     // 256-wide tiles when they still give every compute unit work, else 128-wide ones
     if ((int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units) return 256;
-    if ((int64_t)mtiles * ((out_cols_virtual + 127) / 128) * 10 >= (int64_t)compute_units * 7) return 128;
+    const int64_t items = (int64_t)mtiles * ((out_cols_virtual + 127) / 128);
+    if (items * 10 >= (int64_t)compute_units * 7) return 128;
+    if (epilogue != JL_SWIGLU && k >= 4096 && k % 128 == 0 && items * 20 >= (int64_t)compute_units * 7) {
+        *splits = 2;
+        return 128;
+    }
     return 0;
+}
+
+// Bytes of the partial-sum planes of a call that cuts K in two.
+size_t jl_dense_plane_bytes(int rows, int out_cols_virtual) {
+    return 2 * (size_t)((rows + DBM - 1) / DBM * DBM) * (size_t)((out_cols_virtual + 127) / 128 * 128) * sizeof(float);
 }
 
 // Bytes of the decoded copy for `out_cols_virtual` weight rows of `k` columns.
@@ -386,7 +419,7 @@ size_t jl_dense_copy_bytes(int k, int out_cols_virtual) {
 
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
-                         int epilogue, _Float16 *copy, int bn) {
+                         int epilogue, _Float16 *copy, int bn, int splits, float *planes) {
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     const bool swiglu = epilogue == JL_SWIGLU;
@@ -439,6 +472,10 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
     p.epilogue = epilogue;
     p.ntiles = ntiles;
     p.mtiles = (rows + DBM - 1) / DBM;
-    int st = bn == 256 ? launch_dense<256>(ctx, p) : launch_dense<128>(ctx, p);
-    return st;
+    p.splits = splits;
+    p.partial = planes;
+    const int st = bn == 256 ? launch_dense<256>(ctx, p) : launch_dense<128>(ctx, p);
+    if (st != JL_OK || splits == 1) return st;
+    return jl_launch_gemm_reduce(ctx, planes, row_scale, C, rows, n_total, ntiles,
+                                 (int64_t)p.mtiles * DBM * ntiles * 128, splits, ldo, col_offset, epilogue);
 }

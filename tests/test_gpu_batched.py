@@ -132,12 +132,13 @@ def test_batched_gate_up(ctx, t, d, n, T):
 
 @pytest.mark.parametrize("t,d,n,T,residual", [
     (O.Q8_0, 300, 512, 1100, False), (O.Q8_0, 300, 512, 1100, True), (O.Q4_K, 136, 1024, 1024, False),
-    (O.Q8_0, 16384, 256, 1024, False),
+    (O.Q8_0, 16384, 256, 1024, False), (O.Q4_0, 2944, 4096, 1024, True),
 ])
 def test_many_row_prefill_matches_oracle(ctx, t, d, n, T, residual):
     """A thousand rows or more: weights decoded to fp16 once per call, then the plain fp16 GEMM
     (dequantize*ToFP16 + gemmMMA, TransformerBatchPrefillKernels.java:917-1076,2325-2363).  Same
-    arithmetic as the fused kernel, so the same bound; the last shape takes the 256-wide tiles."""
+    arithmetic as the fused kernel, so the same bound; the fourth shape takes the 256-wide tiles, the
+    fifth (few tiles, long rows) cuts K in two."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
     say("many-row prefill", NAMES[t], d, n, T, residual)
