@@ -743,33 +743,47 @@ jl_gemm_f16(GemmParams p) {
 }
 
 // Sums the split-K planes in split order (so the result does not depend on scheduling) and
-// applies row scale and epilogue.  One thread per output element.
+// applies row scale and epilogue.  One thread per four consecutive output columns.
 __global__ void __launch_bounds__(256)
 jl_gemm_reduce(const float *__restrict__ partial, const float *__restrict__ row_scale,
                float *__restrict__ C, int rows, int n_total, int ntiles, int64_t plane, int splits,
                int64_t ldo, int64_t col_offset, int epilogue) {
-    const int col = blockIdx.x * blockDim.x + threadIdx.x;
+    const int col = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
     const int m = blockIdx.y;
     if (col >= n_total || m >= rows) return;
     const int64_t width = (int64_t)ntiles * BN;
     float *out = C + (int64_t)m * ldo + col_offset + col;
+    const float rs = row_scale[m];
+    float v[4];
     if (epilogue == JL_SWIGLU) {
         // tile t holds gate columns 64 t .. 64 t + 63 in its first half and the up columns after
         const int64_t g = (int64_t)m * width + (col >> 6) * BN + (col & 63);
-        float sg = 0.f, su = 0.f;
+        float4 sg = {0.f, 0.f, 0.f, 0.f}, su = {0.f, 0.f, 0.f, 0.f};
         for (int z = 0; z < splits; z++) {
-            sg += partial[z * plane + g];
-            su += partial[z * plane + g + 64];
+            const float4 a = *(const float4 *)(partial + z * plane + g);
+            const float4 b = *(const float4 *)(partial + z * plane + g + 64);
+            sg.x += a.x; sg.y += a.y; sg.z += a.z; sg.w += a.w;
+            su.x += b.x; su.y += b.y; su.z += b.z; su.w += b.w;
         }
-        const float rs = row_scale[m];
-        *out = gemm_swiglu(sg * rs, su * rs);
+        v[0] = gemm_swiglu(sg.x * rs, su.x * rs);
+        v[1] = gemm_swiglu(sg.y * rs, su.y * rs);
+        v[2] = gemm_swiglu(sg.z * rs, su.z * rs);
+        v[3] = gemm_swiglu(sg.w * rs, su.w * rs);
     } else {
         const int64_t g = (int64_t)m * width + col;
-        float sum = 0.f;
-        for (int z = 0; z < splits; z++) sum += partial[z * plane + g];
-        sum *= row_scale[m];
-        if (epilogue == JL_RESIDUAL) *out += sum;
-        else *out = sum;
+        float4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int z = 0; z < splits; z++) {
+            const float4 a = *(const float4 *)(partial + z * plane + g);
+            sum.x += a.x; sum.y += a.y; sum.z += a.z; sum.w += a.w;
+        }
+        v[0] = sum.x * rs; v[1] = sum.y * rs; v[2] = sum.z * rs; v[3] = sum.w * rs;
+    }
+    const bool add = epilogue == JL_RESIDUAL;
+    if (col + 3 < n_total && (((uintptr_t)out) & 15) == 0) {
+        float4 o = add ? *(const float4 *)out : float4{0.f, 0.f, 0.f, 0.f};
+        *(float4 *)out = float4{o.x + v[0], o.y + v[1], o.z + v[2], o.w + v[3]};
+    } else {
+        for (int e = 0; e < 4 && col + e < n_total; e++) out[e] = add ? out[e] + v[e] : v[e];
     }
 }
 
@@ -861,7 +875,7 @@ int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows, float *planes, si
     else if (bm == 64) st = launch_gemm<TYPE, 64>(ctx, p, grid);
     else st = launch_gemm<TYPE, 128>(ctx, p, grid);
     if (st != JL_OK || p.splits == 1) return st;
-    hipLaunchKernelGGL(jl_gemm_reduce, dim3((p.n_total + 255) / 256, rows), dim3(256), 0, ctx->stream,
+    hipLaunchKernelGGL(jl_gemm_reduce, dim3((p.n_total + 1023) / 1024, rows), dim3(256), 0, ctx->stream,
                        planes, p.row_scale, p.C, rows, p.n_total, p.ntiles, plane, p.splits, p.ldo,
                        p.col_offset, p.epilogue);
     JL_HIP(hipGetLastError());
@@ -873,7 +887,7 @@ int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows, float *planes, si
 int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row_scale, float *C, int rows,
                           int n_total, int ntiles, int64_t plane, int splits, int64_t ldo, int64_t col_offset,
                           int epilogue) {
-    hipLaunchKernelGGL(jl_gemm_reduce, dim3((n_total + 255) / 256, rows), dim3(256), 0, ctx->stream, planes,
+    hipLaunchKernelGGL(jl_gemm_reduce, dim3((n_total + 1023) / 1024, rows), dim3(256), 0, ctx->stream, planes,
                        row_scale, C, rows, n_total, ntiles, plane, splits, ldo, col_offset, epilogue);
     JL_HIP(hipGetLastError());
     return JL_OK;

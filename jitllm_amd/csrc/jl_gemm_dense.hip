@@ -46,67 +46,96 @@ struct DecodeParams {
     int half;              // BN / 2 of the GEMM that will read the copy
 };
 
-// One thread decodes 32 consecutive columns of one row (a Q8_0 / Q4_0 block, a Q4_K sub-block).
-// Reads are 2-byte (block scales sit on odd 2-byte boundaries); a 128-byte line serves ~4
-// neighbouring threads, so the cache turns them into whole-line traffic.
+// eight bytes (two dwords in 0..255 offset form) -> (byte - bias) * d, eight fp16 as one 16-byte store
+__device__ __forceinline__ uint4 pack8_scaled(uint32_t q0, uint32_t q1, h2 bias, h2 d) {
+    h2 a, b, c, e;
+    dword_scaled(q0, bias, d, a, b);
+    dword_scaled(q1, bias, d, c, e);
+    return uint4{__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
+                 __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, e)};
+}
+__device__ __forceinline__ uint4 pack8_affine(uint32_t q0, uint32_t q1, h2 ds, h2 dm) {
+    const h2 bias = {(_Float16)1024.f, (_Float16)1024.f};
+    h2 a = (bytes_to_h2(q0, 0x00050004u) - bias) * ds - dm;
+    h2 b = (bytes_to_h2(q0, 0x00070006u) - bias) * ds - dm;
+    h2 c = (bytes_to_h2(q1, 0x00050004u) - bias) * ds - dm;
+    h2 e = (bytes_to_h2(q1, 0x00070006u) - bias) * ds - dm;
+    return uint4{__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
+                 __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, e)};
+}
+
+// One thread decodes 64 consecutive columns of one row -- a pair of Q8_0 / Q4_0 blocks (68 / 36
+// bytes, 4-byte aligned) or a quarter of a Q4_K super-block -- read with 128-bit loads, and writes
+// 128 bytes of fp16.
 template <int TYPE>
 __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
-    const int per_row = p.k / 32;
+    const int per_row = p.k / 64;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int64_t)p.rows * per_row) return;
     const int r = (int)(idx / per_row);
-    const int blk = (int)(idx - (int64_t)r * per_row);
+    const int sl = (int)(idx - (int64_t)r * per_row);
     const uint8_t *row = p.w + (int64_t)r * p.row_bytes;
     int v = p.first_virtual + r;
     if (p.swiglu_half >= 0) v = (r / p.half) * (2 * p.half) + p.swiglu_half * p.half + r % p.half;
-    h2 o[16];
+    uint4 *dst = (uint4 *)(p.out + (int64_t)v * p.k + sl * 64);
     if constexpr (TYPE == JL_Q8_0) {
-        const uint16_t *b = (const uint16_t *)(row + (int64_t)blk * 34);
-        const _Float16 d = __builtin_bit_cast(_Float16, b[0]);
-        const h2 bias = {(_Float16)1152.f, (_Float16)1152.f}, dd = {d, d};
+        // 68 bytes: scale A | 32 quants A | scale B | 32 quants B
+        const uint32_t *src = (const uint32_t *)(row + (int64_t)sl * 68);
+        uint32_t w[17];
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t q = ((uint32_t)b[1 + 2 * i] | ((uint32_t)b[2 + 2 * i] << 16)) ^ 0x80808080u;
-            dword_scaled(q, bias, dd, o[2 * i], o[2 * i + 1]);
-        }
-    } else if constexpr (TYPE == JL_Q4_0) {
-        const uint16_t *b = (const uint16_t *)(row + (int64_t)blk * 18);
-        const _Float16 d = __builtin_bit_cast(_Float16, b[0]);
-        const h2 bias = {(_Float16)1032.f, (_Float16)1032.f}, dd = {d, d};
+        for (int i = 0; i < 17; i++) w[i] = src[i];
+        const _Float16 dA = __builtin_bit_cast(_Float16, (unsigned short)(w[0] & 0xFFFF));
+        const _Float16 dB = __builtin_bit_cast(_Float16, (unsigned short)(w[8] >> 16));
+        const h2 bias = {(_Float16)1152.f, (_Float16)1152.f}, a2 = {dA, dA}, b2 = {dB, dB};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t q = (uint32_t)b[1 + 2 * i] | ((uint32_t)b[2 + 2 * i] << 16);
-            dword_scaled(q & 0x0F0F0F0Fu, bias, dd, o[2 * i], o[2 * i + 1]);              // elements 4i ..
-            dword_scaled((q >> 4) & 0x0F0F0F0Fu, bias, dd, o[8 + 2 * i], o[9 + 2 * i]);   // 16 + 4i ..
+            const uint32_t q0 = __builtin_amdgcn_alignbit(w[2 * i + 1], w[2 * i], 16);
+            const uint32_t q1 = __builtin_amdgcn_alignbit(w[2 * i + 2], w[2 * i + 1], 16);
+            dst[i] = pack8_scaled(q0 ^ 0x80808080u, q1 ^ 0x80808080u, bias, a2);
+            dst[4 + i] = pack8_scaled(w[9 + 2 * i] ^ 0x80808080u, w[10 + 2 * i] ^ 0x80808080u, bias, b2);
+        }
+    } else if constexpr (TYPE == JL_Q4_0) {
+        // 36 bytes: scale A | 16 nibble bytes A | scale B | 16 nibble bytes B
+        const uint32_t *src = (const uint32_t *)(row + (int64_t)sl * 36);
+        uint32_t w[9];
+#pragma unroll
+        for (int i = 0; i < 9; i++) w[i] = src[i];
+        const _Float16 dA = __builtin_bit_cast(_Float16, (unsigned short)(w[0] & 0xFFFF));
+        const _Float16 dB = __builtin_bit_cast(_Float16, (unsigned short)(w[4] >> 16));
+        const h2 bias = {(_Float16)1032.f, (_Float16)1032.f}, a2 = {dA, dA}, b2 = {dB, dB};
+        uint32_t qa[4], qb[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            qa[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
+            qb[i] = w[5 + i];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            dst[i] = pack8_scaled(qa[2 * i] & 0x0F0F0F0Fu, qa[2 * i + 1] & 0x0F0F0F0Fu, bias, a2);
+            dst[2 + i] = pack8_scaled((qa[2 * i] >> 4) & 0x0F0F0F0Fu, (qa[2 * i + 1] >> 4) & 0x0F0F0F0Fu, bias, a2);
+            dst[4 + i] = pack8_scaled(qb[2 * i] & 0x0F0F0F0Fu, qb[2 * i + 1] & 0x0F0F0F0Fu, bias, b2);
+            dst[6 + i] = pack8_scaled((qb[2 * i] >> 4) & 0x0F0F0F0Fu, (qb[2 * i + 1] >> 4) & 0x0F0F0F0Fu, bias, b2);
         }
     } else {
-        const uint8_t *sb = row + (int64_t)(blk >> 3) * 144;
-        const uint32_t *hdr = (const uint32_t *)sb;
-        const int sub = blk & 7;
-        const float d = jl_half_bits_to_float(hdr[0]);
-        const float dmin = jl_half_bits_to_float(hdr[0] >> 16);
-        int sc, mn;
-        jl_q4k_scale_min(hdr[1], hdr[2], hdr[3], sub, sc, mn);
-        const _Float16 ds = (_Float16)(d * (float)sc), dm = (_Float16)(dmin * (float)mn);
-        const h2 ds2 = {ds, ds}, dm2 = {dm, dm}, bias = {(_Float16)1024.f, (_Float16)1024.f};
-        const uint32_t *qs = (const uint32_t *)(sb + 16 + (sub >> 1) * 32);
-        const int shift = (sub & 1) * 4;
+        // a quarter of a super-block: low nibbles are sub-block 2 pair, high nibbles 2 pair + 1
+        const uint8_t *sb = row + (int64_t)(sl >> 2) * 144;
+        const int pair = sl & 3;
+        const uint4 h = *(const uint4 *)sb;
+        const uint4 q0 = *(const uint4 *)(sb + 16 + pair * 32), q1 = *(const uint4 *)(sb + 32 + pair * 32);
+        const float d = jl_half_bits_to_float(h.x);
+        const float dmin = jl_half_bits_to_float(h.x >> 16);
+        int sc0, mn0, sc1, mn1;
+        jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair, sc0, mn0);
+        jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair + 1, sc1, mn1);
+        const _Float16 ds0 = (_Float16)(d * (float)sc0), dm0 = (_Float16)(dmin * (float)mn0);
+        const _Float16 ds1 = (_Float16)(d * (float)sc1), dm1 = (_Float16)(dmin * (float)mn1);
+        const h2 s0 = {ds0, ds0}, m0 = {dm0, dm0}, s1 = {ds1, ds1}, m1 = {dm1, dm1};
+        const uint32_t qs[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t q = (qs[i] >> shift) & 0x0F0F0F0Fu;
-            o[2 * i] = (bytes_to_h2(q, 0x00050004u) - bias) * ds2 - dm2;
-            o[2 * i + 1] = (bytes_to_h2(q, 0x00070006u) - bias) * ds2 - dm2;
+        for (int i = 0; i < 4; i++) {
+            dst[i] = pack8_affine(qs[2 * i] & 0x0F0F0F0Fu, qs[2 * i + 1] & 0x0F0F0F0Fu, s0, m0);
+            dst[4 + i] = pack8_affine((qs[2 * i] >> 4) & 0x0F0F0F0Fu, (qs[2 * i + 1] >> 4) & 0x0F0F0F0Fu, s1, m1);
         }
-    }
-    uint4 *dst = (uint4 *)(p.out + (int64_t)v * p.k + blk * 32);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        uint4 u;
-        u.x = __builtin_bit_cast(uint32_t, o[4 * i]);
-        u.y = __builtin_bit_cast(uint32_t, o[4 * i + 1]);
-        u.z = __builtin_bit_cast(uint32_t, o[4 * i + 2]);
-        u.w = __builtin_bit_cast(uint32_t, o[4 * i + 3]);
-        dst[i] = u;
     }
 }
 
@@ -379,7 +408,7 @@ int launch_dense(jl_context *ctx, const DenseParams &p) {
 
 template <int TYPE>
 int launch_decode(jl_context *ctx, const DecodeParams &d) {
-    const int64_t threads = (int64_t)d.rows * (d.k / 32);
+    const int64_t threads = (int64_t)d.rows * (d.k / 64);
     hipLaunchKernelGGL(jl_decode_to_f16<TYPE>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
                        ctx->stream, d);
     JL_HIP(hipGetLastError());
