@@ -256,16 +256,19 @@ jl_gemm_hh(DenseParams p) {
             const int i = j * 512 + tid, r = i >> 3, c = (i & 7) ^ ((r >> 1) & 7);
             wsrc[j] = (const uint8_t *)(p.W + ((int64_t)nt * BN + r) * p.k) + kbytes + c * 16;
         }
-        auto issue = [&](int s) {
+        // load n (of LA + LW) of this thread for stage s
+        auto issue_one = [&](int s, int n) {
             uint8_t *dst = lds + (s % NS) * STAGE;
+            if (n < LA)
+                __builtin_amdgcn_global_load_lds((gvoid *)(asrc[n] + (int64_t)s * 128),
+                                                 (lvoid *)(dst + (n * 512 + wave * 64) * 16), 16, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds((gvoid *)(wsrc[n - LA] + (int64_t)s * 128),
+                                                 (lvoid *)(dst + DBM * 128 + ((n - LA) * 512 + wave * 64) * 16), 16, 0, 0);
+        };
+        auto issue = [&](int s) {
 #pragma unroll
-            for (int j = 0; j < LA; j++)
-                __builtin_amdgcn_global_load_lds((gvoid *)(asrc[j] + (int64_t)s * 128),
-                                                 (lvoid *)(dst + (j * 512 + wave * 64) * 16), 16, 0, 0);
-#pragma unroll
-            for (int j = 0; j < LW; j++)
-                __builtin_amdgcn_global_load_lds((gvoid *)(wsrc[j] + (int64_t)s * 128),
-                                                 (lvoid *)(dst + DBM * 128 + (j * 512 + wave * 64) * 16), 16, 0, 0);
+            for (int n = 0; n < LA + LW; n++) issue_one(s, n);
         };
 
         floatx4 acc[MB][NB];
@@ -283,8 +286,7 @@ jl_gemm_hh(DenseParams p) {
             if (AHEAD == 2 && s + 1 < ksteps) JL_WAIT_VM(LA + LW);
             else JL_WAIT_VM(0);
             __builtin_amdgcn_s_barrier();
-            // the slot of stage s - 1 was last read before this barrier
-            if (s + AHEAD < ksteps) issue(s + AHEAD);
+            const bool more = s + AHEAD < ksteps;   // the slot of stage s - 1 was last read before this barrier
             const uint32_t base = lds0 + (s % NS) * STAGE;
             half8 fa[2][MB], fb[2][NB];
 #pragma unroll
@@ -304,11 +306,21 @@ jl_gemm_hh(DenseParams p) {
             else asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
             lds_settle(fa[0]);
             lds_settle(fb[0]);
+            // The next stage's loads go out between the row blocks of the first k-block, a few at a
+            // time: every load occupies the address path for its 1 KB (64 bytes per clock per
+            // compute unit, i.e. half the step for a whole stage) and holds its wave at issue
+            // while that path is busy, which in one burst would leave the matrix pipe idle.
+            constexpr int PER = (LA + LW + MB - 1) / MB;
 #pragma unroll
-            for (int i = 0; i < MB; i++)
+            for (int i = 0; i < MB; i++) {
 #pragma unroll
                 for (int j = 0; j < NB; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[0][j], fa[0][i], acc[i][j], 0, 0, 0);
+                if (more) {
+#pragma unroll
+                    for (int n = i * PER; n < (i + 1) * PER && n < LA + LW; n++) issue_one(s + AHEAD, n);
+                }
+            }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             lds_settle(fa[1]);
             lds_settle(fb[1]);
