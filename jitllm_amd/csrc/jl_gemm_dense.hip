@@ -231,6 +231,7 @@ jl_gemm_hh(DenseParams p) {
         w_off[j] = DBM * 128 + r * 128 + ((fg ^ ((r >> 1) & 7)) << 4);
     }
 
+    const uint32_t toff = (uint32_t)(tid >> 3) * (uint32_t)(p.k * 2) + (uint32_t)(((tid & 7) ^ ((tid >> 4) & 7)) << 4);
     for (int item = slot; item < per_xcd * p.splits; item += slots) {
         const int split = item / per_xcd;
         const int logical = xcd * per_xcd + (item - split * per_xcd);
@@ -244,26 +245,20 @@ jl_gemm_hh(DenseParams p) {
         const int mt = group * GM + rest - nt * rows_in_group;
         const int m0 = mt * DBM;
 
-        // this thread's load slots: slot i = row i / 8, chunk position i % 8 (source chunk swizzled)
-        const uint8_t *asrc[LA], *wsrc[LW];
-#pragma unroll
-        for (int j = 0; j < LA; j++) {
-            const int i = j * 512 + tid, r = i >> 3, c = (i & 7) ^ ((r >> 1) & 7);
-            asrc[j] = (const uint8_t *)(p.A + (int64_t)(m0 + r) * p.k) + kbytes + c * 16;
-        }
-#pragma unroll
-        for (int j = 0; j < LW; j++) {
-            const int i = j * 512 + tid, r = i >> 3, c = (i & 7) ^ ((r >> 1) & 7);
-            wsrc[j] = (const uint8_t *)(p.W + ((int64_t)nt * BN + r) * p.k) + kbytes + c * 16;
-        }
+        // this thread's load slots: slot i = 512 n + tid is row i / 8, chunk position i % 8 (source
+        // chunk swizzled).  64 n rows do not change the swizzle key and A and W rows are equally
+        // long, so one 32-bit thread offset serves every slot on top of a uniform address.
+        const uint8_t *a_item = (const uint8_t *)(p.A + (int64_t)m0 * p.k) + kbytes;
+        const uint8_t *w_item = (const uint8_t *)(p.W + (int64_t)nt * BN * p.k) + kbytes;
+        const int64_t slot_stride = (int64_t)64 * p.k * 2;
         // load n (of LA + LW) of this thread for stage s
         auto issue_one = [&](int s, int n) {
             uint8_t *dst = lds + (s % NS) * STAGE;
             if (n < LA)
-                __builtin_amdgcn_global_load_lds((gvoid *)(asrc[n] + (int64_t)s * 128),
+                __builtin_amdgcn_global_load_lds((gvoid *)(a_item + n * slot_stride + (int64_t)s * 128 + toff),
                                                  (lvoid *)(dst + (n * 512 + wave * 64) * 16), 16, 0, 0);
             else
-                __builtin_amdgcn_global_load_lds((gvoid *)(wsrc[n - LA] + (int64_t)s * 128),
+                __builtin_amdgcn_global_load_lds((gvoid *)(w_item + (n - LA) * slot_stride + (int64_t)s * 128 + toff),
                                                  (lvoid *)(dst + DBM * 128 + ((n - LA) * 512 + wave * 64) * 16), 16, 0, 0);
         };
         auto issue = [&](int s) {
@@ -281,14 +276,13 @@ jl_gemm_hh(DenseParams p) {
 #pragma unroll
         for (int a = 0; a < AHEAD; a++)
             if (a < ksteps) issue(a);
-        for (int s = 0; s < ksteps; s++) {
-            // stage s landed (this thread's part); the AHEAD - 1 younger stages may be in flight
-            if (AHEAD == 2 && s + 1 < ksteps) JL_WAIT_VM(LA + LW);
-            else JL_WAIT_VM(0);
-            __builtin_amdgcn_s_barrier();
-            const bool more = s + AHEAD < ksteps;   // the slot of stage s - 1 was last read before this barrier
-            const uint32_t base = lds0 + (s % NS) * STAGE;
-            half8 fa[2][MB], fb[2][NB];
+        // The two waves of a SIMD (w and w + 4) run half a step apart, so that one of them has
+        // MFMAs to issue while the other waits for its fragments: after the barrier of step s the
+        // early wave reads the fragments of stage s and then multiplies them; the late wave first
+        // multiplies the fragments of stage s - 1, which it holds in registers, and then reads
+        // those of stage s.  Both have read stage s when they reach the next barrier.
+        half8 fa[2][MB], fb[2][NB];
+        auto read_frags = [&](uint32_t base) {
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 // k-block h: chunk position of chunk (4 h + fg) is the k-block-0 position ^ (4 h)
@@ -300,35 +294,70 @@ jl_gemm_hh(DenseParams p) {
                 for (int i = 0; i < MB; i++)
                     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(fa[h][i]) : "v"(aa), "n"(i * 2048) : "memory");
             }
-            // LDS reads return in order: the first k-block's MB + NB fragments are back when that
-            // many of the second's are still outstanding
-            if constexpr (MB == 8) asm volatile("s_waitcnt lgkmcnt(12)" ::: "memory");
-            else asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
-            lds_settle(fa[0]);
-            lds_settle(fb[0]);
-            // The next stage's loads go out between the row blocks of the first k-block, a few at a
-            // time: every load occupies the address path for its 1 KB (64 bytes per clock per
-            // compute unit, i.e. half the step for a whole stage) and holds its wave at issue
-            // while that path is busy, which in one burst would leave the matrix pipe idle.
+        };
+        // The MFMAs of k-block h.  With `loads`, stage `next`'s loads go out between the row
+        // blocks, a few at a time: every load occupies the address path for its 1 KB (64 bytes per
+        // clock per compute unit, i.e. half the step for a whole stage) and holds its wave at
+        // issue while that path is busy, which in one burst would leave the matrix pipe idle.
+        auto mfma_block = [&](int h, bool loads, int next) {
             constexpr int PER = (LA + LW + MB - 1) / MB;
 #pragma unroll
             for (int i = 0; i < MB; i++) {
 #pragma unroll
                 for (int j = 0; j < NB; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[0][j], fa[0][i], acc[i][j], 0, 0, 0);
-                if (more) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[h][j], fa[h][i], acc[i][j], 0, 0, 0);
+                if (loads) {
 #pragma unroll
-                    for (int n = i * PER; n < (i + 1) * PER && n < LA + LW; n++) issue_one(s + AHEAD, n);
+                    for (int n = i * PER; n < (i + 1) * PER && n < LA + LW; n++) issue_one(next, n);
                 }
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            lds_settle(fa[1]);
-            lds_settle(fb[1]);
-#pragma unroll
-            for (int i = 0; i < MB; i++)
-#pragma unroll
-                for (int j = 0; j < NB; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
+        };
+        // stage s landed (this thread's part); the AHEAD - 1 younger stages may be in flight
+        auto stage_ready = [&](int s) {
+            if (AHEAD == 2 && s + 1 < ksteps) JL_WAIT_VM(LA + LW);
+            else JL_WAIT_VM(0);
+            __builtin_amdgcn_s_barrier();
+        };
+        // (the slot that stage s + AHEAD goes to held stage s - 1, last read before barrier s)
+        if (wave < 4) {
+            for (int s = 0; s < ksteps; s++) {
+                stage_ready(s);
+                const bool more = s + AHEAD < ksteps;
+                read_frags(lds0 + (s % NS) * STAGE);
+                // LDS reads return in order: the first k-block's MB + NB fragments are back when
+                // that many of the second's are still outstanding
+                if constexpr (MB == 8) asm volatile("s_waitcnt lgkmcnt(12)" ::: "memory");
+                else asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+                lds_settle(fa[0]);
+                lds_settle(fb[0]);
+                mfma_block(0, more, s + AHEAD);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                lds_settle(fa[1]);
+                lds_settle(fb[1]);
+                mfma_block(1, false, 0);
+            }
+        } else {
+            auto read_all = [&](int s) {
+                read_frags(lds0 + (s % NS) * STAGE);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                lds_settle(fa[0]);
+                lds_settle(fb[0]);
+                lds_settle(fa[1]);
+                lds_settle(fb[1]);
+            };
+            stage_ready(0);
+            if (AHEAD < ksteps) issue(AHEAD);
+            read_all(0);
+            for (int s = 1; s < ksteps; s++) {
+                stage_ready(s);
+                __builtin_amdgcn_s_setprio(2);
+                mfma_block(0, s + AHEAD < ksteps, s + AHEAD);
+                mfma_block(1, false, 0);
+                __builtin_amdgcn_s_setprio(0);
+                read_all(s);
+            }
+            mfma_block(0, false, 0);
+            mfma_block(1, false, 0);
         }
 
         // epilogue: a lane holds four consecutive output columns 4 (lane / 16) .. + 3 of activation
