@@ -825,11 +825,11 @@ size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_
     }
     size_t planes = round_up(round_up((size_t)out_cols, 128) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
     // calls of a thousand rows or more decode the weights to fp16 once, into the same region
-    // (and, for narrow projections with long rows, two planes of partial sums; such calls have at
-    // most 0.35 x 256 compute units' worth of 256 x 128 tiles)
+    // (and, for narrow projections with long rows, two planes of partial sums; such calls have
+    // fewer 256 x 128 tiles than 0.7 x 256 compute units)
     if (max_rows >= 1024) {
         size_t two = jl_dense_plane_bytes((int)max_rows, (int)out_cols);
-        const size_t cap = 2 * (size_t)90 * 256 * 128 * sizeof(float);
+        const size_t cap = 2 * (size_t)180 * 256 * 128 * sizeof(float);
         if (two > cap) two = cap;
         const size_t need = round_up(jl_dense_copy_bytes((int)cols, (int)out_cols), 256) + two;
         if (need > planes) planes = need;

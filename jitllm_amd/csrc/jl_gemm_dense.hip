@@ -38,12 +38,14 @@ __device__ __forceinline__ void dword_scaled(uint32_t v, h2 bias, h2 d, h2 &lo, 
 }
 
 struct DecodeParams {
-    const uint8_t *w;      // raw blocks of one weight
-    _Float16 *out;         // [virtual rows x k]
-    int rows, k, row_bytes;
-    int first_virtual;     // virtual row of the weight's row 0 (plain layout)
-    int swiglu_half;       // -1 plain; 0 gate / 1 up: row r goes to tile (r / half) * BN + half_sel * half + r % half
-    int half;              // BN / 2 of the GEMM that will read the copy
+    const uint8_t *w[8];   // raw blocks of the call's weights
+    int begin[9];          // plain layout: weight i fills virtual rows [begin[i], begin[i + 1])
+    int count;
+    _Float16 *out;         // [ntiles * BN virtual rows x k]
+    int k, row_bytes;
+    int n_total;           // SWIGLU: rows of one weight
+    int half;              // SWIGLU: BN / 2 of the GEMM that will read the copy, else 0; virtual row
+                           // t * BN + sel * half + i is row t * half + i of weight sel (0 gate, 1 up)
 };
 
 // eight bytes (two dwords in 0..255 offset form) -> (byte - bias) * d, eight fp16 as one 16-byte store
@@ -64,85 +66,69 @@ __device__ __forceinline__ uint4 pack8_affine(uint32_t q0, uint32_t q1, h2 ds, h
                  __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, e)};
 }
 
-// One thread decodes 64 consecutive columns of one row -- a pair of Q8_0 / Q4_0 blocks (68 / 36
-// bytes, 4-byte aligned) or a quarter of a Q4_K super-block -- read with 128-bit loads, and writes
-// 128 bytes of fp16.
+// One thread decodes 8 consecutive columns of one row into one 16-byte store, so a wave writes
+// 1 KB of consecutive fp16 and reads a consecutive run of raw blocks (the 8 quant bytes of a
+// Q8_0 / Q4_0 chunk are only 2-byte aligned; the hardware takes unaligned dword loads).
+// blockIdx.x is the virtual row -- rows that no weight row fills (the end of the last column tile)
+// become zeros -- and blockIdx.y the run of 256 chunks within it.
+struct __attribute__((packed, aligned(2))) Quants8 { uint32_t lo, hi; };
+
 template <int TYPE>
 __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
-    const int per_row = p.k / 64;
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (int64_t)p.rows * per_row) return;
-    const int r = (int)(idx / per_row);
-    const int sl = (int)(idx - (int64_t)r * per_row);
-    const uint8_t *row = p.w + (int64_t)r * p.row_bytes;
-    int v = p.first_virtual + r;
-    if (p.swiglu_half >= 0) v = (r / p.half) * (2 * p.half) + p.swiglu_half * p.half + r % p.half;
-    uint4 *dst = (uint4 *)(p.out + (int64_t)v * p.k + sl * 64);
-    if constexpr (TYPE == JL_Q8_0) {
-        // 68 bytes: scale A | 32 quants A | scale B | 32 quants B
-        const uint32_t *src = (const uint32_t *)(row + (int64_t)sl * 68);
-        uint32_t w[17];
-#pragma unroll
-        for (int i = 0; i < 17; i++) w[i] = src[i];
-        const _Float16 dA = __builtin_bit_cast(_Float16, (unsigned short)(w[0] & 0xFFFF));
-        const _Float16 dB = __builtin_bit_cast(_Float16, (unsigned short)(w[8] >> 16));
-        const h2 bias = {(_Float16)1152.f, (_Float16)1152.f}, a2 = {dA, dA}, b2 = {dB, dB};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t q0 = __builtin_amdgcn_alignbit(w[2 * i + 1], w[2 * i], 16);
-            const uint32_t q1 = __builtin_amdgcn_alignbit(w[2 * i + 2], w[2 * i + 1], 16);
-            dst[i] = pack8_scaled(q0 ^ 0x80808080u, q1 ^ 0x80808080u, bias, a2);
-            dst[4 + i] = pack8_scaled(w[9 + 2 * i] ^ 0x80808080u, w[10 + 2 * i] ^ 0x80808080u, bias, b2);
-        }
-    } else if constexpr (TYPE == JL_Q4_0) {
-        // 36 bytes: scale A | 16 nibble bytes A | scale B | 16 nibble bytes B
-        const uint32_t *src = (const uint32_t *)(row + (int64_t)sl * 36);
-        uint32_t w[9];
-#pragma unroll
-        for (int i = 0; i < 9; i++) w[i] = src[i];
-        const _Float16 dA = __builtin_bit_cast(_Float16, (unsigned short)(w[0] & 0xFFFF));
-        const _Float16 dB = __builtin_bit_cast(_Float16, (unsigned short)(w[4] >> 16));
-        const h2 bias = {(_Float16)1032.f, (_Float16)1032.f}, a2 = {dA, dA}, b2 = {dB, dB};
-        uint32_t qa[4], qb[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            qa[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
-            qb[i] = w[5 + i];
-        }
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            dst[i] = pack8_scaled(qa[2 * i] & 0x0F0F0F0Fu, qa[2 * i + 1] & 0x0F0F0F0Fu, bias, a2);
-            dst[2 + i] = pack8_scaled((qa[2 * i] >> 4) & 0x0F0F0F0Fu, (qa[2 * i + 1] >> 4) & 0x0F0F0F0Fu, bias, a2);
-            dst[4 + i] = pack8_scaled(qb[2 * i] & 0x0F0F0F0Fu, qb[2 * i + 1] & 0x0F0F0F0Fu, bias, b2);
-            dst[6 + i] = pack8_scaled((qb[2 * i] >> 4) & 0x0F0F0F0Fu, (qb[2 * i + 1] >> 4) & 0x0F0F0F0Fu, bias, b2);
-        }
+    const int v = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;   // chunk of 8 columns
+    if (c >= p.k / 8) return;
+    uint4 *dst = (uint4 *)(p.out + (int64_t)v * p.k + c * 8);
+    // (the table is walked with constant indices so that it stays in scalar registers)
+    const uint8_t *w = nullptr;
+    int r = 0;
+    if (p.half) {
+        const int t = v / (2 * p.half), within = v - t * (2 * p.half);
+        const int sel = within >= p.half;
+        r = t * p.half + within - sel * p.half;
+        if (r < p.n_total) w = sel ? p.w[1] : p.w[0];
     } else {
-        // a quarter of a super-block: low nibbles are sub-block 2 pair, high nibbles 2 pair + 1
-        const uint8_t *sb = row + (int64_t)(sl >> 2) * 144;
-        const int pair = sl & 3;
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            if (i < p.count && v >= p.begin[i] && v < p.begin[i + 1]) {
+                w = p.w[i];
+                r = v - p.begin[i];
+            }
+    }
+    if (w == nullptr) {
+        *dst = uint4{0, 0, 0, 0};
+        return;
+    }
+    const uint8_t *row = w + (int64_t)r * p.row_bytes;
+    if constexpr (TYPE == JL_Q8_0) {
+        const uint8_t *blk = row + (c >> 2) * 34;
+        const _Float16 d = *(const _Float16 *)blk;
+        const Quants8 q = *(const Quants8 *)(blk + 2 + (c & 3) * 8);
+        const h2 bias = {(_Float16)1152.f, (_Float16)1152.f}, d2 = {d, d};
+        *dst = pack8_scaled(q.lo ^ 0x80808080u, q.hi ^ 0x80808080u, bias, d2);
+    } else if constexpr (TYPE == JL_Q4_0) {
+        // columns 0..15 of a block are the low nibbles of its 16 bytes, 16..31 the high nibbles
+        const uint8_t *blk = row + (c >> 2) * 18;
+        const _Float16 d = *(const _Float16 *)blk;
+        const Quants8 q = *(const Quants8 *)(blk + 2 + (c & 1) * 8);
+        const int shift = (c & 2) * 2;
+        const h2 bias = {(_Float16)1032.f, (_Float16)1032.f}, d2 = {d, d};
+        *dst = pack8_scaled((q.lo >> shift) & 0x0F0F0F0Fu, (q.hi >> shift) & 0x0F0F0F0Fu, bias, d2);
+    } else {
+        // sub-block c / 4 of super-block c / 32: low nibbles are the even sub-block of a pair of
+        // 32 bytes, high nibbles the odd one
+        const uint8_t *sb = row + (int64_t)(c >> 5) * 144;
+        const int sub = (c >> 2) & 7;
         const uint4 h = *(const uint4 *)sb;
-        const uint4 q0 = *(const uint4 *)(sb + 16 + pair * 32), q1 = *(const uint4 *)(sb + 32 + pair * 32);
+        const uint2 q = *(const uint2 *)(sb + 16 + (sub >> 1) * 32 + (c & 3) * 8);
         const float d = jl_half_bits_to_float(h.x);
         const float dmin = jl_half_bits_to_float(h.x >> 16);
-        int sc0, mn0, sc1, mn1;
-        jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair, sc0, mn0);
-        jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair + 1, sc1, mn1);
-        const _Float16 ds0 = (_Float16)(d * (float)sc0), dm0 = (_Float16)(dmin * (float)mn0);
-        const _Float16 ds1 = (_Float16)(d * (float)sc1), dm1 = (_Float16)(dmin * (float)mn1);
-        const h2 s0 = {ds0, ds0}, m0 = {dm0, dm0}, s1 = {ds1, ds1}, m1 = {dm1, dm1};
-        const uint32_t qs[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            dst[i] = pack8_affine(qs[2 * i] & 0x0F0F0F0Fu, qs[2 * i + 1] & 0x0F0F0F0Fu, s0, m0);
-            dst[4 + i] = pack8_affine((qs[2 * i] >> 4) & 0x0F0F0F0Fu, (qs[2 * i + 1] >> 4) & 0x0F0F0F0Fu, s1, m1);
-        }
+        int sc, mn;
+        jl_q4k_scale_min(h.y, h.z, h.w, sub, sc, mn);
+        const _Float16 ds = (_Float16)(d * (float)sc), dm = (_Float16)(dmin * (float)mn);
+        const int shift = (sub & 1) * 4;
+        *dst = pack8_affine((q.x >> shift) & 0x0F0F0F0Fu, (q.y >> shift) & 0x0F0F0F0Fu, h2{ds, ds}, h2{dm, dm});
     }
-}
-
-// zero rows [first, first + count) of the decoded copy (padding up to the column tile)
-__global__ void __launch_bounds__(256) jl_zero_rows_f16(_Float16 *out, int64_t halfs) {
-    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
-    if (i < halfs) *(uint4 *)(out + i) = uint4{0, 0, 0, 0};
 }
 
 // ---- fp16 GEMM ----------------------------------------------------------------------------------
@@ -448,10 +434,9 @@ int launch_dense(jl_context *ctx, const DenseParams &p) {
 }
 
 template <int TYPE>
-int launch_decode(jl_context *ctx, const DecodeParams &d) {
-    const int64_t threads = (int64_t)d.rows * (d.k / 64);
-    hipLaunchKernelGGL(jl_decode_to_f16<TYPE>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
-                       ctx->stream, d);
+int launch_decode(jl_context *ctx, const DecodeParams &d, int virtual_rows) {
+    hipLaunchKernelGGL(jl_decode_to_f16<TYPE>, dim3((unsigned)virtual_rows, (unsigned)((d.k / 8 + 255) / 256)),
+                       dim3(256), 0, ctx->stream, d);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
@@ -470,7 +455,7 @@ int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, in
     if ((int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units) return 256;
     const int64_t items = (int64_t)mtiles * ((out_cols_virtual + 127) / 128);
     if (items * 10 >= (int64_t)compute_units * 7) return 128;
-    if (epilogue != JL_SWIGLU && k >= 4096 && k % 128 == 0 && items * 20 >= (int64_t)compute_units * 7) {
+    if (epilogue != JL_SWIGLU && k >= 2048 && k % 128 == 0 && items * 20 >= (int64_t)compute_units * 7) {
         *splits = 2;
         return 128;
     }
@@ -495,39 +480,29 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
     const bool swiglu = epilogue == JL_SWIGLU;
     int n_total = 0;
     for (int i = 0; i < (swiglu ? 1 : count); i++) n_total += (int)weights[i]->rows;
-    const int virt = swiglu ? 2 * n_total : n_total;
     const int cols_per_tile = swiglu ? bn / 2 : bn;
     const int ntiles = (n_total + cols_per_tile - 1) / cols_per_tile;
 
-    // rows of the last tile that no weight row fills
-    if ((int64_t)ntiles * bn > virt) {
-        const int64_t first = swiglu ? (int64_t)(ntiles - 1) * bn : virt;
-        const int64_t halfs = ((int64_t)ntiles * bn - first) * k;
-        hipLaunchKernelGGL(jl_zero_rows_f16, dim3((unsigned)((halfs / 8 + 255) / 256)), dim3(256), 0, ctx->stream,
-                           copy + first * k, halfs);
-        JL_HIP(hipGetLastError());
-    }
-    int first_virtual = 0;
+    if (count > 8) return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: more than 8 weights in one call");
+    DecodeParams d{};
     for (int i = 0; i < count; i++) {
-        DecodeParams d{};
-        d.w = weights[i]->blocks;
-        d.out = copy;
-        d.rows = (int)weights[i]->rows;
-        d.k = k;
-        d.row_bytes = k / jl_block_elems(type) * jl_block_bytes(type);
-        d.first_virtual = first_virtual;
-        d.swiglu_half = swiglu ? i : -1;
-        d.half = bn / 2;
-        first_virtual += d.rows;
-        int st;
-        switch (type) {
-            case JL_Q8_0: st = launch_decode<JL_Q8_0>(ctx, d); break;
-            case JL_Q4_0: st = launch_decode<JL_Q4_0>(ctx, d); break;
-            case JL_Q4_K: st = launch_decode<JL_Q4_K>(ctx, d); break;
-            default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
-        }
-        if (st != JL_OK) return st;
+        d.w[i] = weights[i]->blocks;
+        d.begin[i + 1] = d.begin[i] + (int)weights[i]->rows;
     }
+    d.count = count;
+    d.out = copy;
+    d.k = k;
+    d.row_bytes = k / jl_block_elems(type) * jl_block_bytes(type);
+    d.n_total = n_total;
+    d.half = swiglu ? bn / 2 : 0;
+    int dst;
+    switch (type) {
+        case JL_Q8_0: dst = launch_decode<JL_Q8_0>(ctx, d, ntiles * bn); break;
+        case JL_Q4_0: dst = launch_decode<JL_Q4_0>(ctx, d, ntiles * bn); break;
+        case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, d, ntiles * bn); break;
+        default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
+    }
+    if (dst != JL_OK) return dst;
 
     DenseParams p{};
     p.A = A;
