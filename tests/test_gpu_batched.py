@@ -192,6 +192,74 @@ def test_many_row_prefill_qkv_and_gate_up(ctx):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
 
 
+@pytest.mark.parametrize("t,d,n,T,residual", [
+    (O.Q8_0, 5800, 256, 1024, False),    # 128-wide tiles, last tile 40 columns
+    (O.Q4_K, 6016, 256, 1024, True),     # 128-wide tiles, residual
+    (O.Q4_0, 16500, 256, 1100, False),   # 256-wide tiles, ragged rows and columns
+    (O.Q8_0, 3000, 2048, 1024, True),    # K cut in two, last tile 56 columns
+])
+def test_two_pass_prefill_tiles_and_edges(ctx, t, d, n, T, residual):
+    """Shapes with enough tiles for the decode-once path on 256 compute units, one per tiling it
+    can choose, with output columns and rows that do not fill the last tiles."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("two-pass prefill", NAMES[t], d, n, T, residual)
+    raw = synthetic.weight(t, d, n, seed=8300 + d)
+    X = synthetic.activations((T, n), seed=8400 + T)
+    ref = O.matmul_batch(t, raw, X, d, n)
+    out = ctx.float_array(T * d + 64, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, d).projection(ctx.from_numpy(X), out, ctx.load_weight(t, raw, d, n),
+                                                       n, d, residual)
+    ctx.sync()
+    flat = out.get()
+    assert np.all(flat[T * d:] == UNTOUCHED)   # nothing written past the last row
+    got = flat[:T * d].reshape(T, d)
+    want = ref.astype(np.float64) + (float(UNTOUCHED) if residual else 0.0)
+    # short rows average the fp16 rounding of the weights less: 5e-4 of sum |w x| (the path's bound
+    # is 2e-3); a residual adds the rounding of the fp32 sum, half an ulp of the value it is added to
+    slack = abs(np.spacing(np.float32(UNTOUCHED))) / 2 if residual else 0.0
+    excess = np.abs(got.astype(np.float64) - want) - slack
+    assert np.all(excess <= 5e-4 * magnitude(t, raw, X, d, n)), float(excess.max())
+
+
+def test_two_pass_prefill_qkv_and_gate_up(ctx):
+    """The decode-once path with several weights in one call: q|k|v of unequal widths side by side,
+    and gate/up interleaved by half tiles with a last tile of 8 outputs."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("two-pass prefill qkv / gate_up")
+    t, n, T = O.Q8_0, 256, 1024
+    dims = (4096, 1024, 1000)
+    raws = [synthetic.weight(t, d, n, seed=281 + i) for i, d in enumerate(dims)]
+    X = synthetic.activations((T, n), seed=285)
+    ws = [ctx.load_weight(t, r, d, n) for r, d in zip(raws, dims)]
+    ld = sum(dims)
+    out = ctx.float_array(T * ld, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, ld).fusedQKV(ctx.from_numpy(X), out, *ws)
+    ctx.sync()
+    got = out.get().reshape(T, ld)
+    col = 0
+    for raw, d in zip(raws, dims):
+        ref = O.matmul_batch(t, raw, X, d, n)
+        assert rel_err(got[:, col:col + d], ref, magnitude(t, raw, X, d, n)) < 2e-4
+        col += d
+    t, d, n, T = O.Q4_0, 8200, 256, 1024
+    r1 = synthetic.weight(t, d, n, seed=291)
+    r3 = synthetic.weight(t, d, n, seed=292)
+    X = synthetic.activations((T, n), seed=293)
+    g = O.matmul_batch(t, r1, X, d, n)
+    u = O.matmul_batch(t, r3, X, d, n)
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(T, d)
+    hb = ctx.float_array(T * d, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, 2 * d).gateUp(ctx.from_numpy(X), hb, ctx.load_weight(t, r1, d, n),
+                                                ctx.load_weight(t, r3, d, n), n, d)
+    ctx.sync()
+    got = hb.get().reshape(T, d)
+    mg, mu = magnitude(t, r1, X, d, n), magnitude(t, r3, X, d, n)
+    bound = 2e-4 * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
+
+
 def test_huge_activation_rows_stay_finite(ctx):
     """Rows far outside fp16's range are rescaled by a power of two, not turned into infinities."""
     from jitllm_amd import synthetic
