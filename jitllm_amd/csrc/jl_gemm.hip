@@ -824,10 +824,10 @@ size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_
         return round_up(padded * (size_t)cols, 256) + round_up(padded * (size_t)(cols / 32) * 4, 256);
     }
     size_t planes = round_up(round_up((size_t)out_cols, 128) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
-    // calls of a thousand rows or more decode the weights to fp16 once, into the same region
+    // calls of 512 rows or more may decode the weights to fp16 once, into the same region
     // (and, for narrow projections with long rows, two planes of partial sums; such calls have
     // fewer 256 x 128 tiles than 0.7 x 256 compute units)
-    if (max_rows >= 1024) {
+    if (max_rows >= 512) {
         size_t two = jl_dense_plane_bytes((int)max_rows, (int)out_cols);
         const size_t cap = 2 * (size_t)180 * 256 * 128 * sizeof(float);
         if (two > cap) two = cap;
@@ -928,7 +928,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
         if (st != JL_OK || taken) return st;
     }
 
-    // a thousand rows or more: weights decoded to fp16 once per call, then the plain fp16 GEMM
+    // many rows and enough tiles: weights decoded to fp16 once per call, then the plain fp16 GEMM
     int virt = 0;
     for (int i = 0; i < count; i++) virt += (int)weights[i]->rows;
     int dsplits = 1;

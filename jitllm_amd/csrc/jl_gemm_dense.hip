@@ -2,15 +2,16 @@
 //
 // This is the reference's own two-step shape (dequantize*ToFP16 followed by gemmMMA,
 // J/backend/tornado/kernels/TransformerBatchPrefillKernels.java:917-1076,2325-2363): with a
-// thousand or more activation rows the decode is a small fraction of the call when done once, and
+// few hundred or more activation rows the decode is a small fraction of the call when done once, and
 // the matrix loop without it affords 256-row tiles and 128 x 64 wave tiles, which halve the LDS
 // traffic per flop of the decode-in-the-loop kernel (jl_gemm.hip).  The decoded copy lives in the
 // caller's workspace for the duration of the call; in HBM the weights stay GGUF blocks.
 //
 //   jl_decode_to_f16   raw blocks -> [virtual rows x K] fp16, the host decode rounded once to fp16
-//                      (bit for bit what the fused kernel multiplies with)
-//   jl_gemm_hh<BN>     C = A16 . W16^T on v_mfma_f32_16x16x32_f16, 256 x BN x 32 steps, eight
-//                      identical waves that each bring in their share of both operands by LDS-DMA
+//                      (bit for bit what the fused kernel multiplies with); one launch per call
+//   jl_gemm_hh<BN>     C = A16 . W16^T on v_mfma_f32_16x16x32_f16, 256 x BN tiles in steps of 64
+//                      columns; eight waves that each bring in their share of both operands by
+//                      LDS-DMA, the two waves of a SIMD half a step apart
 #include "jl_device.h"
 #include "jl_internal.h"
 
@@ -443,13 +444,13 @@ int launch_decode(jl_context *ctx, const DecodeParams &d, int virtual_rows) {
 
 }  // namespace
 
-// Column tile the dense path would use for a call, 0 when the call is not one for it: it takes a
-// thousand rows or more and enough work items to give most compute units one.  Narrow projections
+// Column tile the dense path would use for a call, 0 when the call is not one for it: it takes
+// 512 rows or more and enough work items to give most compute units one.  Narrow projections
 // with long rows get there by cutting K in two (*splits = 2, plain store / residual only); what is
 // still too small keeps the decode-in-the-loop kernel, whose 128-row tiles fill the chip better.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits) {
     *splits = 1;
-    if (rows < 1024 || k % 64 != 0) return 0;
+    if (rows < 512 || k % 64 != 0) return 0;
     const int mtiles = (rows + DBM - 1) / DBM;
     // 256-wide tiles when they still give every compute unit work, else 128-wide ones
     if ((int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units) return 256;
