@@ -210,7 +210,7 @@ def bench_gemm(ctx, hip, t, T, steps, warmup):
     tflops = flops / (ms * 1e-3) / 1e12
     return {"tokens": T, "ms_per_layer": round(ms, 4), "tok_s_16_layers": round(T / (ms * 1e-3 * LAYERS), 1),
             "tflops": round(tflops, 1), "frac_f16_mfma_peak": round(tflops / F16_MFMA_PEAK_TFLOPS, 4),
-            "math": "f16 MFMA after in-LDS dequant"}
+            "math": "f16 MFMA, fp32 accumulate; weights decoded to fp16 inside the call (in LDS, or once per call into the workspace)"}
 
 
 def bench_batched_q4k(ctx, hip, B, steps, warmup):

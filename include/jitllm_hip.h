@@ -155,10 +155,13 @@ int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
  * memory preflight equals what the call uses).  `max_rows` is the largest `batch`, `cols` the
  * largest row length, `out_cols` the largest number of output columns one call produces (a gate/up
  * pair counts both weights' rows), `math` a jl_gemm_math.  The scratch holds the fp16 copy of the
- * activations, one scale per row, and -- for calls whose tile grid would leave compute units idle,
- * which cut K across workgroups -- the partial sums of the cuts (at most about twice the weight
- * bytes).  A smaller workspace that still holds the first two is accepted; such calls simply do
- * not cut K.  Calls of at most 32 rows read X directly and use only the partial sums.
+ * activations, one scale per row, and a third region of about 2.1 bytes per weight of the largest
+ * call that a call uses for one of two things: the partial sums of calls that cut K across
+ * workgroups (calls whose tile grid would leave compute units idle), or -- calls of 512 rows and
+ * more, the reference's dequantize-then-gemmMMA prefill shape -- an fp16 copy of the call's
+ * weights, decoded afresh by every such call and dead after it.  A smaller workspace that still
+ * holds the first two is accepted; such calls simply keep to one pass and do not cut K.  Calls of
+ * at most 32 rows read X directly and use only the partial sums.
  */
 size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols, int math);
 
