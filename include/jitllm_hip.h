@@ -147,6 +147,44 @@ int jl_gemv_gate_up(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, c
 /* gate[i] = SiLU(gate[i]) * up[i] (siluAndMultiply; the unfused tail of gateUp). */
 int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
 
+/* ---- the steps on either side of a decode projection ------------------------------------------ */
+
+/*
+ * scale[0] = (float)(1 / sqrt(sum_j x[j]^2 / n + eps)), a device scalar: the factor
+ * CpuOperations.rmsnorm applies (J/inference/op/CpuOperations.java:60-66) and what
+ * reductionOneBlockWithLayer leaves for the fused kernels
+ * (J/backend/tornado/kernels/TransformerComputeKernels.java:378-437).  The sum is taken in parallel,
+ * so its last bits may differ from the host's sequential sum.
+ */
+int jl_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale);
+
+/*
+ * The projections above with the RMS normalisation of x folded into the activation load:
+ * x_j is replaced by rms_weights[j] * (s * x_j) (CpuOperations.rmsnorm :67-72) and never written
+ * back.  jl_gemv_rms and jl_gemv_qkv_rms take s = rms_scale[0] from the device
+ * (fusedRmsNormQKVMatmulQ8, TransformerComputeKernelsLayered.java:2116-2220;
+ * reductionOneBlock2WithLogits + the vocabulary projection, TransformerComputeKernels.java:439-444,
+ * LogitsQ8_0Layer.java:85-97); jl_gemv_gate_up_rms computes s itself from x and eps, every
+ * workgroup for itself (fullyFusedRmsNormFFNGateUpQ8, TransformerComputeKernelsLayered.java:2866+).
+ * Row length: a multiple of 64 up to 8192, x and rms_weights 16-byte aligned; otherwise
+ * JL_ERR_UNSUPPORTED and the caller normalises first, as the unfused reference path does.
+ */
+int jl_gemv_rms(jl_context *ctx, const jl_weight *w, const float *x, const float *rms_weights,
+                const float *rms_scale, float *out, int epilogue);
+int jl_gemv_qkv_rms(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const jl_weight *wv,
+                    const float *x, const float *rms_weights, const float *rms_scale, float *q,
+                    float *k, float *v);
+int jl_gemv_gate_up_rms(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, const float *x,
+                        const float *rms_weights, float eps, float *hb);
+
+/*
+ * index[0] = position of the first maximum of values[0..n) (device int32): greedy sampling without
+ * bringing the logits to the host (argmaxLogits, TransformerComputeKernels.java:95-127;
+ * FloatTensor.argmax, J/tensor/standard/FloatTensor.java:168-181, whose tie and NaN behaviour --
+ * first of equals, 0 when element 0 is NaN -- this follows).
+ */
+int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
+
 /* ---- batched decode and batched prefill: `batch` activation rows ---------------------------- */
 
 /*

@@ -214,7 +214,7 @@ int jl_gemv(jl_context *ctx, const jl_weight *w, const float *x, float *out, int
     JL_REQUIRE(ctx && w && x && out, "jl_gemv: null argument");
     JL_REQUIRE(epilogue == JL_STORE || epilogue == JL_RESIDUAL,
                "jl_gemv: epilogue %d (JL_STORE or JL_RESIDUAL)", epilogue);
-    return jl_launch_gemv(ctx, &w, 1, &out, nullptr, x, epilogue);
+    return jl_launch_gemv(ctx, &w, 1, &out, nullptr, x, epilogue, nullptr);
 }
 
 int jl_gemv_qkv(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const jl_weight *wv,
@@ -230,7 +230,7 @@ int jl_gemv_qkv(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const
                (long long)wk->cols, (long long)wv->cols);
     const jl_weight *ws[3] = {wq, wk, wv};
     float *outs[3] = {q, k, v};
-    return jl_launch_gemv(ctx, ws, 3, outs, nullptr, x, JL_STORE);
+    return jl_launch_gemv(ctx, ws, 3, outs, nullptr, x, JL_STORE, nullptr);
 }
 
 int jl_gemv_gate_up(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, const float *x,
@@ -244,7 +244,60 @@ int jl_gemv_gate_up(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, c
     JL_REQUIRE(w1->rows == w3->rows && w1->cols == w3->cols,
                "jl_gemv_gate_up: gate is %lld x %lld, up is %lld x %lld", (long long)w1->rows,
                (long long)w1->cols, (long long)w3->rows, (long long)w3->cols);
-    return jl_launch_gemv(ctx, &w1, 1, &hb, w3, x, JL_SWIGLU);
+    return jl_launch_gemv(ctx, &w1, 1, &hb, w3, x, JL_SWIGLU, nullptr);
+}
+
+int jl_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale) {
+    JL_REQUIRE(ctx && x && scale && n > 0, "jl_rms_scale: bad argument");
+    return jl_launch_rms_scale(ctx, x, n, eps, scale);
+}
+
+int jl_gemv_rms(jl_context *ctx, const jl_weight *w, const float *x, const float *rms_weights,
+                const float *rms_scale, float *out, int epilogue) {
+    JL_REQUIRE(ctx && w && x && rms_weights && rms_scale && out, "jl_gemv_rms: null argument");
+    JL_REQUIRE(epilogue == JL_STORE || epilogue == JL_RESIDUAL,
+               "jl_gemv_rms: epilogue %d (JL_STORE or JL_RESIDUAL)", epilogue);
+    const jl_rms rms{rms_weights, rms_scale, 0.f};
+    return jl_launch_gemv(ctx, &w, 1, &out, nullptr, x, epilogue, &rms);
+}
+
+int jl_gemv_qkv_rms(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const jl_weight *wv,
+                    const float *x, const float *rms_weights, const float *rms_scale, float *q,
+                    float *k, float *v) {
+    JL_REQUIRE(ctx && wq && wk && wv && x && rms_weights && rms_scale && q && k && v,
+               "jl_gemv_qkv_rms: null argument");
+    if (wq->type != wk->type || wq->type != wv->type) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "jl_gemv_qkv_rms: no fused q|k|v kernel for mixed weights %s/%s/%s",
+                       jl_type_name(wq->type), jl_type_name(wk->type), jl_type_name(wv->type));
+    }
+    JL_REQUIRE(wq->cols == wk->cols && wq->cols == wv->cols,
+               "jl_gemv_qkv_rms: row lengths differ (%lld, %lld, %lld)", (long long)wq->cols,
+               (long long)wk->cols, (long long)wv->cols);
+    const jl_weight *ws[3] = {wq, wk, wv};
+    float *outs[3] = {q, k, v};
+    const jl_rms rms{rms_weights, rms_scale, 0.f};
+    return jl_launch_gemv(ctx, ws, 3, outs, nullptr, x, JL_STORE, &rms);
+}
+
+int jl_gemv_gate_up_rms(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, const float *x,
+                        const float *rms_weights, float eps, float *hb) {
+    JL_REQUIRE(ctx && w1 && w3 && x && rms_weights && hb, "jl_gemv_gate_up_rms: null argument");
+    if (w1->type != w3->type) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "jl_gemv_gate_up_rms: no fused gate/up kernel for a %s gate and a %s up weight",
+                       jl_type_name(w1->type), jl_type_name(w3->type));
+    }
+    JL_REQUIRE(w1->rows == w3->rows && w1->cols == w3->cols,
+               "jl_gemv_gate_up_rms: gate is %lld x %lld, up is %lld x %lld", (long long)w1->rows,
+               (long long)w1->cols, (long long)w3->rows, (long long)w3->cols);
+    const jl_rms rms{rms_weights, nullptr, eps};
+    return jl_launch_gemv(ctx, &w1, 1, &hb, w3, x, JL_SWIGLU, &rms);
+}
+
+int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
+    JL_REQUIRE(ctx && values && index && n > 0 && n <= INT32_MAX, "jl_argmax: bad argument");
+    return jl_launch_argmax(ctx, values, n, index);
 }
 
 int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count) {

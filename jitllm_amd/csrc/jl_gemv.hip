@@ -47,6 +47,11 @@ struct GemvParams {
     int row_bytes;
     int epilogue;
     int stages;     // depth of the LDS tile ring (2..8)
+    // RMS normalisation folded into the activation load: x_j becomes rms_w[j] * (scale * x_j).
+    const float *rms_w;      // null: x is used as it is
+    const float *rms_scale;  // device scalar; null with rms_w set: the kernel computes
+                             // 1 / sqrt(sum x^2 / n + rms_eps) itself, every workgroup for itself
+    float rms_eps;
 };
 
 template <int TYPE> struct Traits;
@@ -352,7 +357,9 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     // land on the same four).  Slot q holds floats 64 * (q / 17) + 4 * (q % 17) ... + 3.
     const int x_slots = p.S * 17;
     const int x_bytes = (x_slots + nthreads - 1) / nthreads * nthreads * 16;
-    const bool x_in_ring = x_bytes <= stage_bytes;  // else a region of its own after the ring
+    const bool rms = p.rms_w != nullptr;
+    // (with RMS weights alongside, both vectors get a region of their own after the ring)
+    const bool x_in_ring = !rms && x_bytes <= stage_bytes;  // else a region of its own after the ring
     uint8_t *xs = x_in_ring ? ring + (p.stages - 1) * stage_bytes : ring + p.stages * stage_bytes;
     const uint32_t xs0 = x_in_ring ? ring0 + (p.stages - 1) * stage_bytes : ring0 + p.stages * stage_bytes;
     for (int base = 0; base < x_bytes; base += nthreads * 16) {
@@ -361,33 +368,14 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         const int off = (sl < p.S && k < 16) ? (sl * 64 + k * 4) * 4 : 0;
         __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.x + off),
                                          (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
+        if (rms)
+            __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.rms_w + off),
+                                             (lvoid *)(xs + x_bytes + base + wave * JL_WAVE * 16), 16, 0, 0);
     }
     int issued = 0;
     for (; issued < p.stages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
     wait_vm_tiles<L>(issued);
     __builtin_amdgcn_s_barrier();
-
-    float x[64];
-    float sx[2] = {0.f, 0.f};
-    if (active) {
-#pragma unroll
-        for (int k = 0; k < 4; k++) lds_read_16f(xs0 + s * 272 + k * 64, &x[k * 16]);
-    } else {
-#pragma unroll
-        for (int k = 0; k < 64; k++) x[k] = 0.f;
-    }
-    if constexpr (TYPE != JL_Q8_0) {
-#pragma unroll
-        for (int k = 0; k < 32; k++) {
-            sx[0] += x[k];
-            sx[1] += x[32 + k];
-        }
-    }
-
-    // A row's Sp lane sums are folded over quads in registers, then one lane per quad leaves its
-    // partial in LDS and the row's finishing thread adds the P = Sp / 4 partials one tile later.
-    const int P = p.Sp >= 4 ? p.Sp / 4 : 1;
-    constexpr uint32_t kParity = kPartialBytes / 2;
 
     // Segmented sum over aligned groups of `width` lanes (a power of two): row-local DPP moves up
     // to 16 lanes, cross-row permutes beyond.
@@ -402,6 +390,63 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         if (width >= 64) v += __shfl_xor(v, 32, JL_WAVE);
         return v;
     };
+
+    float x[64];
+    float sx[2] = {0.f, 0.f};
+    if (active) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) lds_read_16f(xs0 + s * 272 + k * 64, &x[k * 16]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < 64; k++) x[k] = 0.f;
+    }
+    if (rms) {
+        // CpuOperations.rmsnorm (J/inference/op/CpuOperations.java:60-72): out = w * (ss * x) with
+        // ss = (float)(1 / sqrt(sum x^2 / n + eps)); the reference's fused kernels fold the same
+        // product into their activation load (TransformerComputeKernelsLayered.java:2168-2171).
+        float scale;
+        if (p.rms_scale) {
+            scale = *p.rms_scale;
+        } else {
+            float ss = 0.f;
+#pragma unroll
+            for (int k = 0; k < 64; k++) ss = fmaf(x[k], x[k], ss);   // lanes without a slice hold zeros
+            if (p.Sp <= JL_WAVE) {
+                ss = group_sum(ss, p.Sp);
+            } else {
+                // a row spans Sp / 64 waves: wave sums meet in LDS behind the two vectors
+                ss = group_sum(ss, JL_WAVE);
+                const uint32_t cell = xs0 + 2 * x_bytes;
+                if (lane == 0) lds_write_b32(cell + wave * 4, __float_as_uint(ss));
+                __builtin_amdgcn_s_barrier();
+                const int per_row = p.Sp / JL_WAVE, first_wave = (wave / per_row) * per_row;
+                ss = 0.f;
+                for (int i = 0; i < per_row; i++) ss += __uint_as_float(lds_read_b32(cell + (first_wave + i) * 4));
+            }
+            scale = (float)(1.0 / sqrt((double)(ss / (float)p.n + p.rms_eps)));
+        }
+        if (active) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float w16[16];
+                lds_read_16f(xs0 + x_bytes + s * 272 + k * 64, w16);
+#pragma unroll
+                for (int i = 0; i < 16; i++) x[k * 16 + i] = w16[i] * (scale * x[k * 16 + i]);
+            }
+        }
+    }
+    if constexpr (TYPE != JL_Q8_0) {
+#pragma unroll
+        for (int k = 0; k < 32; k++) {
+            sx[0] += x[k];
+            sx[1] += x[32 + k];
+        }
+    }
+
+    // A row's Sp lane sums are folded over quads in registers, then one lane per quad leaves its
+    // partial in LDS and the row's finishing thread adds the P = Sp / 4 partials one tile later.
+    const int P = p.Sp >= 4 ? p.Sp / 4 : 1;
+    constexpr uint32_t kParity = kPartialBytes / 2;
 
     // Finishes tile `t` from the partials of parity `par`.  The R * P partial slots are at most
     // 64 when P >= 1 quad per row, so wave 0 takes one slot per lane, folds each row's P lanes and
@@ -587,7 +632,7 @@ int launch_generic(jl_context *ctx, const jl_weight *w, const jl_weight *w_up, c
 }  // namespace
 
 int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *const *outs,
-                   const jl_weight *w_up, const float *x, int epilogue) {
+                   const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms) {
     const int type = w[0]->type;
     const int n = (int)w[0]->cols;
     const int row_bytes = n / jl_block_elems(type) * jl_block_bytes(type);
@@ -608,6 +653,14 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     }
     if (w_up && ((uintptr_t)w_up->blocks & 15) != 0) fast = false;
 
+    if (!fast && rms) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "no RMS-folding projection kernel for a row length of %d (a multiple of 64 up to "
+                       "8192 and 16-byte aligned operands are needed)", n);
+    }
+    if (rms && ((uintptr_t)rms->weights & 15) != 0) {
+        return jl_fail(JL_ERR_UNSUPPORTED, "the RMS weights must be 16-byte aligned");
+    }
     if (!fast) {
         for (int i = 0; i < nseg; i++) {
             int st;
@@ -643,16 +696,26 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     p.R = R;
     p.row_bytes = row_bytes;
     p.epilogue = epilogue;
+    if (rms) {
+        p.rms_w = rms->weights;
+        p.rms_scale = rms->scale;
+        p.rms_eps = rms->eps;
+    }
 
     const int threads = (R * Sp + 63) / 64 * 64;
     const int stage_bytes = threads * slice;
     const int x_bytes = (S * 17 + threads - 1) / threads * threads * 16;  // 17 slots per slice
-    const int x_extra = x_bytes <= stage_bytes ? 0 : x_bytes;
+    // (with RMS weights: both vectors and one cell per wave behind the ring)
+    const int x_extra = rms ? 2 * x_bytes + 64 : x_bytes <= stage_bytes ? 0 : x_bytes;
     // Ring depth 2: measured on every benchmark shape, a deeper ring at the lower occupancy its LDS
     // footprint forces is slower than two stages with up to four workgroups per compute unit.
     const int stages = 2;
     p.stages = stages;
     const int lds = kPartialBytes + stages * stage_bytes + x_extra;
+    if (rms && lds > 160 * 1024) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "no RMS-folding projection kernel for a row length of %d (up to 8192)", n);
+    }
 
     switch (type) {
         case JL_Q8_0:

@@ -54,8 +54,17 @@ int jl_fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3
 
 // Launchers implemented per translation unit; each returns a jl_status.
 int jl_launch_dequant(jl_context *ctx, const jl_weight *w, float *out);
+// RMS normalisation folded into a projection's activation load: x_j -> weights[j] * (s * x_j), with
+// s = scale[0] (device) or, when scale is null, 1 / sqrt(sum x^2 / n + eps) computed by the kernel.
+struct jl_rms {
+    const float *weights;
+    const float *scale;
+    float eps;
+};
 int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *const *outs,
-                   const jl_weight *w_up, const float *x, int epilogue);
+                   const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms);
+int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale);
+int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
 int jl_launch_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
 int jl_launch_fill(jl_context *ctx, float *dst, float value, size_t count);
 int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,

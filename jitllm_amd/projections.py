@@ -91,6 +91,45 @@ class QuantizedProjections:
         L.check(self._lib.jl_swiglu(self.context.handle, self.ws.wrapHb.ptr, self.ws.wrapHb2.ptr, d))
 
 
+    # ---- the reference's fused decode kernels: RMS normalisation folded into the projection ----
+
+    def rmsScale(self, x: FloatArray, n: int, eps: float, scale: FloatArray) -> None:
+        """``scale[0] = 1 / sqrt(sum x^2 / n + eps)`` on the device (reductionOneBlockWithLayer,
+        TransformerComputeKernels.java:378-437; CpuOperations.rmsnorm :60-66)."""
+        L.check(self._lib.jl_rms_scale(self.context.handle, x.ptr, n, float(eps), scale.ptr))
+
+    def rmsMatvec(self, x: FloatArray, rmsWeights: FloatArray, rmsScale: FloatArray, out: FloatArray,
+                  w: TornadoTensor, n: int, d: int) -> None:
+        """``out = w . (rmsWeights * (rmsScale[0] * x))``: the final norm folded into the vocabulary
+        projection (reductionOneBlock2WithLogits + the projection, LogitsQ8_0Layer.java:85-97)."""
+        _check_shape(w, n, d)
+        L.check(self._lib.jl_gemv_rms(self.context.handle, w.handle, x.ptr, rmsWeights.ptr,
+                                      rmsScale.ptr, out.ptr, L.JL_STORE))
+
+    def fusedRmsNormQKV(self, x: FloatArray, q: FloatArray, k: FloatArray, v: FloatArray,
+                        rmsWeights: FloatArray, rmsScale: FloatArray, wq: TornadoTensor,
+                        wk: TornadoTensor, wv: TornadoTensor) -> None:
+        """fusedRmsNormQKVMatmulQ8 (TransformerComputeKernelsLayered.java:2116-2220): q | k | v of
+        the normalised activations, which are never written out."""
+        L.check(self._lib.jl_gemv_qkv_rms(self.context.handle, wq.handle, wk.handle, wv.handle, x.ptr,
+                                          rmsWeights.ptr, rmsScale.ptr, q.ptr, k.ptr, v.ptr))
+
+    def fullyFusedRmsNormGateUp(self, x: FloatArray, rmsWeights: FloatArray, eps: float,
+                                w1: TornadoTensor, w3: TornadoTensor, n: int, d: int) -> None:
+        """fullyFusedRmsNormFFNGateUpQ8 (TransformerComputeKernelsLayered.java:2866+):
+        ``wrapHb = SiLU(w1 . xn) * (w3 . xn)`` with ``xn`` the RMS-normalised ``x``, the scale
+        computed inside the kernel."""
+        _check_shape(w1, n, d)
+        _check_shape(w3, n, d)
+        L.check(self._lib.jl_gemv_gate_up_rms(self.context.handle, w1.handle, w3.handle, x.ptr,
+                                              rmsWeights.ptr, float(eps), self.ws.wrapHb.ptr))
+
+    def argmax(self, logits: FloatArray, n: int, token: DeviceBuffer) -> None:
+        """``token[0]`` = index of the first maximum of the logits, an int32 on the device
+        (argmaxLogits, TransformerComputeKernels.java:95-127)."""
+        L.check(self._lib.jl_argmax(self.context.handle, logits.ptr, n, token.ptr))
+
+
 class QuantizedBatchProjections:
     """Projections of ``batchSize`` activation rows at once (batched decode, batched prefill)."""
 

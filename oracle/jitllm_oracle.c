@@ -430,6 +430,47 @@ void jo_swiglu(float *gate, const float *up, int64_t n) {
     }
 }
 
+/* ---- the steps on either side of a projection ---------------------------------------------- */
+
+/*
+ * J/inference/op/CpuOperations.java:60-66 with FloatTensor.reduce (J/tensor/standard/FloatTensor.java:
+ * 147-153): ss = sum x_i^2 sequentially in fp32 from 0f; ss /= size; ss += eps;
+ * ss = (float)(1.0 / Math.sqrt(ss)).
+ */
+float jo_rms_scale(const float *x, int64_t n, float eps) {
+    float ss = 0.0f;
+    for (int64_t i = 0; i < n; i++) {
+        float sq = x[i] * x[i];   /* acc + xi * xi: product rounded, then the sum (no FMA in the lambda) */
+        ss = ss + sq;
+    }
+    ss /= (float)n;
+    ss += eps;
+    return (float)(1.0 / sqrt((double)ss));
+}
+
+/* J/inference/op/CpuOperations.java:67-72: out[i] = weight[i] * (ss * x[i]) */
+void jo_rmsnorm(float *out, const float *x, const float *weight, int64_t n, float eps) {
+    float ss = jo_rms_scale(x, n, eps);
+    for (int64_t i = 0; i < n; i++) {
+        float scaled = ss * x[i];
+        out[i] = weight[i] * scaled;
+    }
+}
+
+/* J/tensor/standard/FloatTensor.java:168-181: the first maximum; a NaN never wins a comparison */
+int64_t jo_argmax(const float *x, int64_t n) {
+    int64_t max_index = 0;
+    float max_value = x[0];
+    for (int64_t i = 0; i < n; i++) {
+        float f = x[i];
+        if (f > max_value) {
+            max_value = f;
+            max_index = i;
+        }
+    }
+    return max_index;
+}
+
 /* ---- int8 activation path (the arithmetic the reference's int8 GEMM defines) -------------- */
 
 /*

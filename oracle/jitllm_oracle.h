@@ -49,6 +49,11 @@ void jo_matmul_batch(int type, int flavour, const uint8_t *w, const float *X, fl
 /* gate[i] = gate[i] / (float)(1.0 + exp(-gate[i])) * up[i] */
 void jo_swiglu(float *gate, const float *up, int64_t n);
 
+/* RMS normalisation as the host path computes it, and the first maximum of a vector */
+float   jo_rms_scale(const float *x, int64_t n, float eps);
+void    jo_rmsnorm(float *out, const float *x, const float *weight, int64_t n, float eps);
+int64_t jo_argmax(const float *x, int64_t n);
+
 /* per-32-block int8 quantisation of activations and the block-scaled int8 GEMM arithmetic */
 void jo_quantize_q8(const float *x, int8_t *q, float *scales, int64_t rows, int64_t k);
 void jo_gemm_int8_block_scaled(int type, const int8_t *aq, const float *ascale, const uint8_t *w,

@@ -65,6 +65,12 @@ def lib() -> C.CDLL:
     L.jo_matmul_batch.restype = None
     L.jo_swiglu.argtypes = [_f32p, _f32p, C.c_int64]
     L.jo_swiglu.restype = None
+    L.jo_rms_scale.argtypes = [_f32p, C.c_int64, C.c_float]
+    L.jo_rms_scale.restype = C.c_float
+    L.jo_rmsnorm.argtypes = [_f32p, _f32p, _f32p, C.c_int64, C.c_float]
+    L.jo_rmsnorm.restype = None
+    L.jo_argmax.argtypes = [_f32p, C.c_int64]
+    L.jo_argmax.restype = C.c_int64
     L.jo_quantize_q8.argtypes = [_f32p, _i8p, _f32p, C.c_int64, C.c_int64]
     L.jo_quantize_q8.restype = None
     L.jo_gemm_int8_block_scaled.argtypes = [C.c_int, _i8p, _f32p, _u8p, _f32p, C.c_int, C.c_int,
@@ -165,6 +171,27 @@ def swiglu(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
     u = np.ascontiguousarray(up, dtype=np.float32)
     lib().jo_swiglu(_f32(g), _f32(u), g.size)
     return g
+
+
+def rms_scale(x: np.ndarray, eps: float) -> np.float32:
+    """CpuOperations.rmsnorm's factor (J/inference/op/CpuOperations.java:60-66)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    return np.float32(lib().jo_rms_scale(_f32(x), x.size, eps))
+
+
+def rmsnorm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
+    """out = weight * (ss * x) (J/inference/op/CpuOperations.java:60-72)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().jo_rmsnorm(_f32(out), _f32(x), _f32(w), x.size, eps)
+    return out
+
+
+def argmax(x: np.ndarray) -> int:
+    """FloatTensor.argmax (J/tensor/standard/FloatTensor.java:168-181)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    return int(lib().jo_argmax(_f32(x), x.size))
 
 
 def quantize_q8(x: np.ndarray):

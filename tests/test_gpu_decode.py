@@ -180,6 +180,120 @@ def test_fused_gate_up(ctx, t, d, n):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + 1e-6)
 
 
+# ---- RMS normalisation folded into the projections, argmax -----------------------------------
+
+@pytest.mark.parametrize("n", [512, 2048, 4096, 8192, 16384, 1000])
+def test_rms_scale_on_device(ctx, n):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("rms scale", n)
+    x = synthetic.activations(n, seed=600 + n) * np.float32(2.5)
+    scale = ctx.float_array(1, fill=POISON)
+    QuantizedProjections(ctx, TornadoWorkspace()).rmsScale(ctx.from_numpy(x), n, 1e-5, scale)
+    ctx.sync()
+    want = float(O.rms_scale(x, 1e-5))
+    assert abs(float(scale.get()[0]) - want) <= 2e-6 * want   # parallel sum against the host's sequential one
+
+
+@pytest.mark.parametrize("t,dq,dkv,n", [(O.Q8_0, 2048, 512, 2048), (O.Q4_0, 4096, 1024, 4096),
+                                         (O.Q4_K, 4096, 1024, 4096), (O.Q8_0, 96, 32, 8192)])
+def test_fused_rms_qkv(ctx, t, dq, dkv, n):
+    """q | k | v of rmsnorm(x), held against the host's rmsnorm followed by three matVecs
+    (InferenceCore.java:86-91)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("rms qkv", NAMES[t], dq, dkv, n)
+    raws = [synthetic.weight(t, d, n, seed=631 + i) for i, d in enumerate((dq, dkv, dkv))]
+    x = synthetic.activations(n, seed=641) * np.float32(3.0)
+    rw = (1.0 + 0.25 * synthetic.activations(n, seed=642)).astype(np.float32)
+    xn = O.rmsnorm(x, rw, 1e-5)
+    ws = [upload(ctx, t, r, d, n) for r, d in zip(raws, (dq, dkv, dkv))]
+    outs = [ctx.float_array(d, fill=POISON) for d in (dq, dkv, dkv)]
+    proj = QuantizedProjections(ctx, TornadoWorkspace())
+    dx, drw, scale = ctx.from_numpy(x), ctx.from_numpy(rw), ctx.float_array(1, fill=POISON)
+    proj.rmsScale(dx, n, 1e-5, scale)
+    proj.fusedRmsNormQKV(dx, *outs, drw, scale, *ws)
+    ctx.sync()
+    assert np.array_equal(dx.get(), x)   # the normalised activations are never written back
+    for raw, d, out in zip(raws, (dq, dkv, dkv), outs):
+        ref = O.matmul(t, raw, xn, d, n)
+        assert rel_err(out.get(), ref, magnitude(t, raw, xn, d, n)) < 2e-5
+
+
+@pytest.mark.parametrize("t,d,n", [(O.Q8_0, 8192, 2048), (O.Q4_0, 14336, 4096),
+                                    (O.Q4_K, 12288, 4096), (O.Q8_0, 40, 8192), (O.Q4_K, 37, 512)])
+def test_fully_fused_rms_gate_up(ctx, t, d, n):
+    """hb = SiLU(w1 . xn) * (w3 . xn) with xn = rmsnorm(x), the scale computed inside the kernel:
+    against the host's rmsnorm, matVec, matVec, swiGLU (InferenceCore.java:124-129)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("rms gate_up", NAMES[t], d, n)
+    r1 = synthetic.weight(t, d, n, seed=651)
+    r3 = synthetic.weight(t, d, n, seed=652)
+    x = synthetic.activations(n, seed=653) * np.float32(0.2)
+    rw = (1.0 + 0.25 * synthetic.activations(n, seed=654)).astype(np.float32)
+    xn = O.rmsnorm(x, rw, 1e-5)
+    g = O.matmul(t, r1, xn, d, n)
+    u = O.matmul(t, r3, xn, d, n)
+    ref = O.swiglu(g, u)
+    hb = ctx.float_array(d, fill=POISON)
+    proj = QuantizedProjections(ctx, TornadoWorkspace(wrapHb=hb))
+    proj.fullyFusedRmsNormGateUp(ctx.from_numpy(x), ctx.from_numpy(rw), 1e-5, upload(ctx, t, r1, d, n),
+                                 upload(ctx, t, r3, d, n), n, d)
+    ctx.sync()
+    got = hb.get()
+    mg = magnitude(t, r1, xn, d, n)
+    mu = magnitude(t, r3, xn, d, n)
+    bound = 2e-5 * (mg * np.abs(u) + mu * np.abs(g) * 1.2 + 1e-6)
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + 1e-6)
+
+
+def test_rms_vocabulary_projection_and_argmax(ctx):
+    """Final norm folded into the vocabulary projection, then the greedy token on the device
+    (LogitsQ8_0Layer.java:85-110) against rmsnorm, matVec and FloatTensor.argmax on the host."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    t, d, n = O.Q8_0, 32000, 2048
+    say("rms vocabulary + argmax", d, n)
+    raw = synthetic.weight(t, d, n, seed=661)
+    x = synthetic.activations(n, seed=662)
+    rw = (1.0 + 0.25 * synthetic.activations(n, seed=663)).astype(np.float32)
+    xn = O.rmsnorm(x, rw, 1e-5)
+    ref = O.matmul(t, raw, xn, d, n)
+    proj = QuantizedProjections(ctx, TornadoWorkspace())
+    dx, drw, scale = ctx.from_numpy(x), ctx.from_numpy(rw), ctx.float_array(1, fill=POISON)
+    logits = ctx.float_array(d, fill=POISON)
+    token = ctx.raw_buffer(4)
+    proj.rmsScale(dx, n, 1e-5, scale)
+    proj.rmsMatvec(dx, drw, scale, logits, upload(ctx, t, raw, d, n), n, d)
+    proj.argmax(logits, d, token)
+    ctx.sync()
+    got = logits.get()
+    assert rel_err(got, ref, magnitude(t, raw, xn, d, n)) < 2e-5
+    assert int(token.download(np.int32, 1)[0]) == O.argmax(got)
+
+
+@pytest.mark.parametrize("n", [1, 5, 1023, 4097, 128256])
+def test_argmax_ties_and_edges(ctx, n):
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("argmax", n)
+    proj = QuantizedProjections(ctx, TornadoWorkspace())
+    token = ctx.raw_buffer(4)
+    rng = np.random.default_rng(n)
+    cases = [rng.standard_normal(n).astype(np.float32)]
+    tied = rng.integers(0, 4, n).astype(np.float32)           # many equal maxima: the first wins
+    cases.append(tied)
+    cases.append(np.full(n, -np.inf, dtype=np.float32))        # nothing above -inf: index 0
+    if n > 2:
+        nan_first = cases[0].copy(); nan_first[0] = np.nan     # nothing beats a NaN at index 0
+        nan_mid = cases[0].copy(); nan_mid[n // 2] = np.nan    # a NaN elsewhere never wins
+        cases += [nan_first, nan_mid]
+    for v in cases:
+        proj.argmax(ctx.from_numpy(v), n, token)
+        ctx.sync()
+        assert int(token.download(np.int32, 1)[0]) == O.argmax(v)
+
+
 def test_mixed_gate_up_runs_two_projections_and_swiglu(ctx):
     """QuantizedProjections.gateUp's unfused branch: gate and up of different types."""
     from jitllm_amd import synthetic

@@ -257,6 +257,54 @@ def test_swiglu_form():
     assert got[2] == 0.0 and got[5] == 40.0
 
 
+# ---- RMS normalisation and argmax -----------------------------------------------------------
+
+def test_rms_scale_closed_forms():
+    """Cases whose answer is known without the formula under test: a constant vector c has
+    sum x^2 / n = c^2 exactly when c^2 n is exact in fp32; a power-of-two factor on x with eps = 0
+    moves the scale by exactly its inverse; and a float64 evaluation bounds a generic vector."""
+    n = 2048
+    for c, eps in ((1.0, 0.0), (2.0, 0.0), (0.5, 1e-5), (3.0, 1e-6)):
+        x = np.full(n, c, dtype=np.float32)
+        want = 1.0 / np.sqrt(np.float64(np.float32(np.float32(c * c) + np.float32(eps))))
+        assert O.rms_scale(x, eps) == np.float32(want), (c, eps)
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal(4096).astype(np.float32)
+    base = O.rms_scale(x, 0.0)
+    for k in (-3, 1, 5):
+        assert O.rms_scale(np.ldexp(x, k).astype(np.float32), 0.0) == np.float32(np.ldexp(base, -k))
+    for eps in (1e-5, 1e-6):
+        exact = 1.0 / np.sqrt(np.mean(x.astype(np.float64) ** 2) + eps)
+        assert abs(float(O.rms_scale(x, eps)) - exact) <= 3e-6 * exact
+    # eps matters where the vector is small, and is added after the division by n
+    tiny = np.full(64, 1e-4, dtype=np.float32)
+    assert abs(float(O.rms_scale(tiny, 1e-5)) - 1.0 / np.sqrt(1e-8 + 1e-5)) < 1e-2
+    assert abs(float(O.rms_scale(tiny, 0.0)) - 1e4) < 1.0
+
+
+def test_rmsnorm_is_weight_times_scaled_x():
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal(1024).astype(np.float32) * 3
+    w = rng.uniform(0.5, 1.5, 1024).astype(np.float32)
+    out = O.rmsnorm(x, w, 1e-5)
+    ss = O.rms_scale(x, 1e-5)
+    assert_bit_equal(out, (w * (ss * x).astype(np.float32)).astype(np.float32))
+    # with unit weights and no eps the result has unit mean square
+    unit = O.rmsnorm(x, np.ones_like(x), 0.0)
+    assert abs(np.mean(unit.astype(np.float64) ** 2) - 1.0) < 1e-5
+
+
+def test_argmax_first_maximum_and_nan():
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal(5000).astype(np.float32)
+    assert O.argmax(x) == int(np.argmax(x))
+    x[[17, 400, 4999]] = 9.0
+    assert O.argmax(x) == 17
+    assert O.argmax(np.array([-np.inf, -np.inf], dtype=np.float32)) == 0
+    assert O.argmax(np.array([np.nan, 5.0, 7.0], dtype=np.float32)) == 0      # nothing beats a NaN
+    assert O.argmax(np.array([1.0, np.nan, 7.0, 7.0], dtype=np.float32)) == 2  # a NaN never wins
+
+
 # ---- int8 activation path -------------------------------------------------------------------
 
 def test_quantize_q8_definition():
