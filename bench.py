@@ -132,6 +132,45 @@ def decode_step(proj, layers, wcls, acts):
     proj.floatMatvec(acts["xb"], acts["logits"], wcls, DIM, VOCAB)
 
 
+def decode_step_fused_rms(proj, layers, wcls, acts):
+    """The same token with the reference's fused decode kernels: the attention norm folded into
+    q|k|v behind its own scale (fusedRmsNormQKVMatmulQ8), the FFN norm computed and folded inside
+    gate/up (fullyFusedRmsNormFFNGateUpQ8), the final norm folded into the vocabulary projection,
+    and the greedy token picked on the device (LogitsQ8_0Layer.java:85-110)."""
+    for w in layers:
+        proj.fusedRmsNormQKV(acts["x"], acts["q"], acts["k"], acts["v"], acts["rms_att"], None,
+                             w["wq"], w["wk"], w["wv"], eps=1e-5)
+        proj.residualMatvec(acts["xb"], w["wo"], DIM, DIM)
+        proj.fullyFusedRmsNormGateUp(acts["x"], acts["rms_ffn"], 1e-5, w["w1"], w["w3"], DIM, HIDDEN)
+        proj.residualMatvec(acts["hb"], w["w2"], HIDDEN, DIM)
+    proj.rmsMatvec(acts["x"], acts["rms_final"], None, acts["logits"], wcls, DIM, VOCAB, eps=1e-5)
+    proj.argmax(acts["logits"], VOCAB, acts["token"])
+
+
+def bench_fused_rms(ctx, hip, proj, layers, wcls, acts, steps, warmup):
+    from jitllm_amd import synthetic
+    for i, k in enumerate(("rms_att", "rms_ffn", "rms_final")):
+        acts[k] = ctx.from_numpy((1.0 + 0.1 * synthetic.activations(DIM, 31 + i)).astype("float32"))
+    acts["token"] = ctx.raw_buffer(4)
+    stream = ctx.stream
+    decode_step_fused_rms(proj, layers, wcls, acts)
+    ctx.sync()
+    graph = hip.capture(stream, lambda: decode_step_fused_rms(proj, layers, wcls, acts))
+    for _ in range(warmup):
+        hip.launch(graph, stream)
+    e0, e1 = hip.event(), hip.event()
+    hip.record(e0, stream)
+    for _ in range(steps):
+        hip.launch(graph, stream)
+    hip.record(e1, stream)
+    ctx.sync()
+    ms = hip.elapsed_ms(e0, e1) / steps
+    return {"ms_per_step": round(ms, 4), "tok_s": round(1e3 / ms, 1), "launches": 4 * LAYERS + 2,
+            "what": "decode set with the 33 RMS normalisations folded into q|k|v, gate/up and the "
+                    "vocabulary projection (scale computed inside each kernel, no normalised vector "
+                    "written) and the greedy token chosen on the device"}
+
+
 def decode_bytes():
     """Algorithmic bytes of a step: every one of the 7 projections of a layer counted on its own
     (weight blocks + fp32 input + fp32 output), as the benchmark's definition does, even where one
@@ -404,6 +443,8 @@ def main():
                          "launches_timed": len(gate_up_ms)},
         }
         if not args.no_extra:
+            out["decode_fused_rms"] = bench_fused_rms(ctx, hip, proj, layers, wcls, acts, args.steps,
+                                                      args.warmup)
             out["prefill"] = [bench_gemm(ctx, hip, t, T, max(3, args.steps // 10), 2)
                               for T in (512, 2048)]
             out["batched_q4k"] = [bench_batched_q4k(ctx, hip, B, max(5, args.steps // 5), 3)

@@ -161,19 +161,20 @@ int jl_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *s
 /*
  * The projections above with the RMS normalisation of x folded into the activation load:
  * x_j is replaced by rms_weights[j] * (s * x_j) (CpuOperations.rmsnorm :67-72) and never written
- * back.  jl_gemv_rms and jl_gemv_qkv_rms take s = rms_scale[0] from the device
- * (fusedRmsNormQKVMatmulQ8, TransformerComputeKernelsLayered.java:2116-2220;
- * reductionOneBlock2WithLogits + the vocabulary projection, TransformerComputeKernels.java:439-444,
- * LogitsQ8_0Layer.java:85-97); jl_gemv_gate_up_rms computes s itself from x and eps, every
- * workgroup for itself (fullyFusedRmsNormFFNGateUpQ8, TransformerComputeKernelsLayered.java:2866+).
- * Row length: a multiple of 64 up to 8192, x and rms_weights 16-byte aligned; otherwise
+ * back.  s = rms_scale[0], a device scalar such as jl_rms_scale leaves (fusedRmsNormQKVMatmulQ8,
+ * TransformerComputeKernelsLayered.java:2116-2220; reductionOneBlock2WithLogits + the vocabulary
+ * projection, TransformerComputeKernels.java:439-444, LogitsQ8_0Layer.java:85-97); or, with
+ * rms_scale null, s = 1 / sqrt(sum x^2 / n + eps) computed from x by every workgroup for itself,
+ * which saves the reduction's launch (fullyFusedRmsNormFFNGateUpQ8,
+ * TransformerComputeKernelsLayered.java:2866+, always works this way: jl_gemv_gate_up_rms).
+ * Row length: a multiple of 64 up to 16384, x and rms_weights 16-byte aligned; otherwise
  * JL_ERR_UNSUPPORTED and the caller normalises first, as the unfused reference path does.
  */
 int jl_gemv_rms(jl_context *ctx, const jl_weight *w, const float *x, const float *rms_weights,
-                const float *rms_scale, float *out, int epilogue);
+                const float *rms_scale, float eps, float *out, int epilogue);
 int jl_gemv_qkv_rms(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const jl_weight *wv,
-                    const float *x, const float *rms_weights, const float *rms_scale, float *q,
-                    float *k, float *v);
+                    const float *x, const float *rms_weights, const float *rms_scale, float eps,
+                    float *q, float *k, float *v);
 int jl_gemv_gate_up_rms(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, const float *x,
                         const float *rms_weights, float eps, float *hb);
 

@@ -47,8 +47,8 @@ SYMBOLS = {
     "jl_gemv_gate_up": (C.c_int, [vp, vp, vp, vp, vp]),
     "jl_swiglu": (C.c_int, [vp, vp, vp, i64]),
     "jl_rms_scale": (C.c_int, [vp, vp, i64, C.c_float, vp]),
-    "jl_gemv_rms": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_int]),
-    "jl_gemv_qkv_rms": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]),
+    "jl_gemv_rms": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp, C.c_int]),
+    "jl_gemv_qkv_rms": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_float, vp, vp, vp]),
     "jl_gemv_gate_up_rms": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp]),
     "jl_argmax": (C.c_int, [vp, vp, i64, vp]),
     "jl_gemm_workspace_bytes": (C.c_size_t, [i64, i64, i64, C.c_int]),

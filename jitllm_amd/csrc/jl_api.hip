@@ -53,6 +53,14 @@ static int context_create(int device, hipStream_t borrowed, bool borrow, jl_cont
         }
         ctx->owns_stream = true;
     }
+    hipError_t e = hipMalloc(&ctx->scratch, JL_CONTEXT_SCRATCH_BYTES);
+    if (e == hipSuccess) e = hipMemset(ctx->scratch, 0, JL_CONTEXT_SCRATCH_BYTES);
+    if (e == hipSuccess) e = hipDeviceSynchronize();   // the context's stream does not wait for the null stream
+    if (e != hipSuccess) {
+        if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return jl_fail(JL_ERR_OOM, "jl_context_create: scratch allocation failed: %s", hipGetErrorString(e));
+    }
     *out = ctx;
     return JL_OK;
 }
@@ -70,6 +78,7 @@ int jl_context_destroy(jl_context *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+    (void)hipFree(ctx->scratch);
     delete ctx;
     return JL_OK;
 }
@@ -253,18 +262,18 @@ int jl_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *s
 }
 
 int jl_gemv_rms(jl_context *ctx, const jl_weight *w, const float *x, const float *rms_weights,
-                const float *rms_scale, float *out, int epilogue) {
-    JL_REQUIRE(ctx && w && x && rms_weights && rms_scale && out, "jl_gemv_rms: null argument");
+                const float *rms_scale, float eps, float *out, int epilogue) {
+    JL_REQUIRE(ctx && w && x && rms_weights && out, "jl_gemv_rms: null argument");
     JL_REQUIRE(epilogue == JL_STORE || epilogue == JL_RESIDUAL,
                "jl_gemv_rms: epilogue %d (JL_STORE or JL_RESIDUAL)", epilogue);
-    const jl_rms rms{rms_weights, rms_scale, 0.f};
+    const jl_rms rms{rms_weights, rms_scale, eps};
     return jl_launch_gemv(ctx, &w, 1, &out, nullptr, x, epilogue, &rms);
 }
 
 int jl_gemv_qkv_rms(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const jl_weight *wv,
-                    const float *x, const float *rms_weights, const float *rms_scale, float *q,
-                    float *k, float *v) {
-    JL_REQUIRE(ctx && wq && wk && wv && x && rms_weights && rms_scale && q && k && v,
+                    const float *x, const float *rms_weights, const float *rms_scale, float eps,
+                    float *q, float *k, float *v) {
+    JL_REQUIRE(ctx && wq && wk && wv && x && rms_weights && q && k && v,
                "jl_gemv_qkv_rms: null argument");
     if (wq->type != wk->type || wq->type != wv->type) {
         return jl_fail(JL_ERR_UNSUPPORTED,
@@ -276,7 +285,7 @@ int jl_gemv_qkv_rms(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, c
                (long long)wk->cols, (long long)wv->cols);
     const jl_weight *ws[3] = {wq, wk, wv};
     float *outs[3] = {q, k, v};
-    const jl_rms rms{rms_weights, rms_scale, 0.f};
+    const jl_rms rms{rms_weights, rms_scale, eps};
     return jl_launch_gemv(ctx, ws, 3, outs, nullptr, x, JL_STORE, &rms);
 }
 

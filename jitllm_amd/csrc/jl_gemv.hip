@@ -190,6 +190,11 @@ __device__ __forceinline__ void lds_write_b32(uint32_t addr, uint32_t v) {
     asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(addr), "v"(v) : "memory");
 }
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void lds_write_x4(uint32_t addr, floatx4 v) {
+    asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(addr), "v"(v) : "memory");
+}
+
 __device__ __forceinline__ void lds_read_x4(uint32_t addr, uint32_t (&w)[4]) {
     asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)"
                  : "=&v"(*(uint4 *)w) : "v"(addr) : "memory");
@@ -281,7 +286,9 @@ __device__ __forceinline__ float quad_xor2(float v) {
     return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));
 }
 
-template <int TYPE, bool DUAL>
+// RMS: the activations are RMS-normalised on their way in (a variant of its own, so that the plain
+// kernel's registers and schedule are not touched by it).
+template <int TYPE, bool DUAL, bool RMS>
 __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
@@ -351,32 +358,6 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     const int first = blockIdx.x;
     const int mine = first < total_tiles ? (total_tiles - first + gridDim.x - 1) / gridDim.x : 0;
 
-    // Activations first (oldest loads), then the first stages - 1 tiles.  In LDS a thread's 64
-    // activations take 17 sixteen-byte slots, the last one padding: slices then start 272 bytes
-    // apart and the 128-bit reads below spread over all banks (256 bytes apart they would all
-    // land on the same four).  Slot q holds floats 64 * (q / 17) + 4 * (q % 17) ... + 3.
-    const int x_slots = p.S * 17;
-    const int x_bytes = (x_slots + nthreads - 1) / nthreads * nthreads * 16;
-    const bool rms = p.rms_w != nullptr;
-    // (with RMS weights alongside, both vectors get a region of their own after the ring)
-    const bool x_in_ring = !rms && x_bytes <= stage_bytes;  // else a region of its own after the ring
-    uint8_t *xs = x_in_ring ? ring + (p.stages - 1) * stage_bytes : ring + p.stages * stage_bytes;
-    const uint32_t xs0 = x_in_ring ? ring0 + (p.stages - 1) * stage_bytes : ring0 + p.stages * stage_bytes;
-    for (int base = 0; base < x_bytes; base += nthreads * 16) {
-        const int q = base / 16 + tid;
-        const int sl = q / 17, k = q - sl * 17;
-        const int off = (sl < p.S && k < 16) ? (sl * 64 + k * 4) * 4 : 0;
-        __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.x + off),
-                                         (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
-        if (rms)
-            __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.rms_w + off),
-                                             (lvoid *)(xs + x_bytes + base + wave * JL_WAVE * 16), 16, 0, 0);
-    }
-    int issued = 0;
-    for (; issued < p.stages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
-    wait_vm_tiles<L>(issued);
-    __builtin_amdgcn_s_barrier();
-
     // Segmented sum over aligned groups of `width` lanes (a power of two): row-local DPP moves up
     // to 16 lanes, cross-row permutes beyond.
     auto group_sum = [&](float v, int width) {
@@ -391,6 +372,99 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         return v;
     };
 
+    constexpr bool rms = RMS;
+
+    // Activations first (oldest loads), then the first stages - 1 tiles.  In LDS a thread's 64
+    // activations take 17 sixteen-byte slots, the last one padding: slices then start 272 bytes
+    // apart and the 128-bit reads below spread over all banks (256 bytes apart they would all
+    // land on the same four).  Slot q holds floats 64 * (q / 17) + 4 * (q % 17) ... + 3.
+    const int x_slots = p.S * 17;
+    const int x_bytes = (x_slots + nthreads - 1) / nthreads * nthreads * 16;
+    const bool x_in_ring = x_bytes <= stage_bytes;  // else a region of its own after the ring
+    uint8_t *xs = x_in_ring ? ring + (p.stages - 1) * stage_bytes : ring + p.stages * stage_bytes;
+    const uint32_t xs0 = x_in_ring ? ring0 + (p.stages - 1) * stage_bytes : ring0 + p.stages * stage_bytes;
+    if constexpr (!rms) {
+        for (int base = 0; base < x_bytes; base += nthreads * 16) {
+            const int q = base / 16 + tid;
+            const int sl = q / 17, k = q - sl * 17;
+            const int off = (sl < p.S && k < 16) ? (sl * 64 + k * 4) * 4 : 0;
+            __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.x + off),
+                                             (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
+        }
+    }
+    int issued = 0;
+    for (; issued < p.stages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
+    if constexpr (rms) {
+        // RMS normalisation folded into the activation load.  CpuOperations.rmsnorm
+        // (J/inference/op/CpuOperations.java:60-72): out = w * (ss * x) with
+        // ss = (float)(1 / sqrt(sum x^2 / n + eps)); the reference's fused kernels fold the same
+        // product into their activation reads (TransformerComputeKernelsLayered.java:2168-2171).
+        // The workgroup reads x and the weights with coalesced 16-byte loads and leaves the
+        // product in the LDS region the plain path fills with x, so everything after is shared
+        // and the LDS footprint (workgroups per compute unit) is that of the plain path.
+        const int nvec = p.n / 4;
+        const float4 *xv = (const float4 *)p.x, *wv = (const float4 *)p.rms_w;
+        // rows of up to 4 x 4 x nthreads columns are read once and held in registers from the
+        // sum of squares to the product; longer ones are read again for the product
+        const bool held = nvec <= nthreads * 4;
+        float4 v[4], w[4];
+        auto load = [&](int base) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int i = base + j * nthreads + tid;
+                v[j] = i < nvec ? xv[i] : float4{0.f, 0.f, 0.f, 0.f};
+                w[j] = i < nvec ? wv[i] : float4{0.f, 0.f, 0.f, 0.f};
+            }
+        };
+        if (held) load(0);
+        float scale;
+        if (p.rms_scale) {
+            scale = *p.rms_scale;
+        } else {
+            float ss = 0.f;
+            if (held) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    ss = fmaf(v[j].x, v[j].x, ss);
+                    ss = fmaf(v[j].y, v[j].y, ss);
+                    ss = fmaf(v[j].z, v[j].z, ss);
+                    ss = fmaf(v[j].w, v[j].w, ss);
+                }
+            } else {
+                for (int i = tid; i < nvec; i += nthreads) {
+                    const float4 u = xv[i];
+                    ss = fmaf(u.x, u.x, ss);
+                    ss = fmaf(u.y, u.y, ss);
+                    ss = fmaf(u.z, u.z, ss);
+                    ss = fmaf(u.w, u.w, ss);
+                }
+            }
+            // wave sums meet in the last words of the partial-sum region, which nothing else
+            // touches before the first tile is finished
+            ss = group_sum(ss, JL_WAVE);
+            const uint32_t cell = lds0 + kPartialBytes - 64;
+            if (lane == 0) lds_write_b32(cell + wave * 4, __float_as_uint(ss));
+            __builtin_amdgcn_s_barrier();
+            ss = 0.f;
+            for (int i = 0; i < nthreads / JL_WAVE; i++) ss += __uint_as_float(lds_read_b32(cell + i * 4));
+            scale = (float)(1.0 / sqrt((double)(ss / (float)p.n + p.rms_eps)));
+        }
+        for (int base = 0; base < nvec; base += nthreads * 4) {
+            if (!held) load(base);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int i = base + j * nthreads + tid;
+                if (i < nvec) {
+                    const floatx4 o = {w[j].x * (scale * v[j].x), w[j].y * (scale * v[j].y),
+                                       w[j].z * (scale * v[j].z), w[j].w * (scale * v[j].w)};
+                    lds_write_x4(xs0 + ((i >> 4) * 17 + (i & 15)) * 16, o);
+                }
+            }
+        }
+    }
+    wait_vm_tiles<L>(issued);
+    __builtin_amdgcn_s_barrier();
+
     float x[64];
     float sx[2] = {0.f, 0.f};
     if (active) {
@@ -399,41 +473,6 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     } else {
 #pragma unroll
         for (int k = 0; k < 64; k++) x[k] = 0.f;
-    }
-    if (rms) {
-        // CpuOperations.rmsnorm (J/inference/op/CpuOperations.java:60-72): out = w * (ss * x) with
-        // ss = (float)(1 / sqrt(sum x^2 / n + eps)); the reference's fused kernels fold the same
-        // product into their activation load (TransformerComputeKernelsLayered.java:2168-2171).
-        float scale;
-        if (p.rms_scale) {
-            scale = *p.rms_scale;
-        } else {
-            float ss = 0.f;
-#pragma unroll
-            for (int k = 0; k < 64; k++) ss = fmaf(x[k], x[k], ss);   // lanes without a slice hold zeros
-            if (p.Sp <= JL_WAVE) {
-                ss = group_sum(ss, p.Sp);
-            } else {
-                // a row spans Sp / 64 waves: wave sums meet in LDS behind the two vectors
-                ss = group_sum(ss, JL_WAVE);
-                const uint32_t cell = xs0 + 2 * x_bytes;
-                if (lane == 0) lds_write_b32(cell + wave * 4, __float_as_uint(ss));
-                __builtin_amdgcn_s_barrier();
-                const int per_row = p.Sp / JL_WAVE, first_wave = (wave / per_row) * per_row;
-                ss = 0.f;
-                for (int i = 0; i < per_row; i++) ss += __uint_as_float(lds_read_b32(cell + (first_wave + i) * 4));
-            }
-            scale = (float)(1.0 / sqrt((double)(ss / (float)p.n + p.rms_eps)));
-        }
-        if (active) {
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                float w16[16];
-                lds_read_16f(xs0 + x_bytes + s * 272 + k * 64, w16);
-#pragma unroll
-                for (int i = 0; i < 16; i++) x[k * 16 + i] = w16[i] * (scale * x[k * 16 + i]);
-            }
-        }
     }
     if constexpr (TYPE != JL_Q8_0) {
 #pragma unroll
@@ -607,9 +646,9 @@ int blocks_per_cu(const void *fn, int device, int threads, int lds) {
     return nb;
 }
 
-template <int TYPE, bool DUAL>
-int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds) {
-    auto fn = jl_gemv_tiles<TYPE, DUAL>;
+template <int TYPE, bool DUAL, bool RMS>
+int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) {
+    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS>;
     int per_cu = blocks_per_cu((const void *)fn, ctx->device, threads, lds);
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
@@ -617,6 +656,12 @@ int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds) {
     hipLaunchKernelGGL(fn, dim3(grid), dim3(threads), lds, ctx->stream, p);
     JL_HIP(hipGetLastError());
     return JL_OK;
+}
+
+template <int TYPE, bool DUAL>
+int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds) {
+    return p.rms_w ? launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds)
+                   : launch_tiles_of<TYPE, DUAL, false>(ctx, p, threads, lds);
 }
 
 template <int TYPE>
@@ -656,7 +701,7 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     if (!fast && rms) {
         return jl_fail(JL_ERR_UNSUPPORTED,
                        "no RMS-folding projection kernel for a row length of %d (a multiple of 64 up to "
-                       "8192 and 16-byte aligned operands are needed)", n);
+                       "16384 and 16-byte aligned operands are needed)", n);
     }
     if (rms && ((uintptr_t)rms->weights & 15) != 0) {
         return jl_fail(JL_ERR_UNSUPPORTED, "the RMS weights must be 16-byte aligned");
@@ -705,17 +750,12 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     const int threads = (R * Sp + 63) / 64 * 64;
     const int stage_bytes = threads * slice;
     const int x_bytes = (S * 17 + threads - 1) / threads * threads * 16;  // 17 slots per slice
-    // (with RMS weights: both vectors and one cell per wave behind the ring)
-    const int x_extra = rms ? 2 * x_bytes + 64 : x_bytes <= stage_bytes ? 0 : x_bytes;
+    const int x_extra = x_bytes <= stage_bytes ? 0 : x_bytes;
     // Ring depth 2: measured on every benchmark shape, a deeper ring at the lower occupancy its LDS
     // footprint forces is slower than two stages with up to four workgroups per compute unit.
     const int stages = 2;
     p.stages = stages;
     const int lds = kPartialBytes + stages * stage_bytes + x_extra;
-    if (rms && lds > 160 * 1024) {
-        return jl_fail(JL_ERR_UNSUPPORTED,
-                       "no RMS-folding projection kernel for a row length of %d (up to 8192)", n);
-    }
 
     switch (type) {
         case JL_Q8_0:

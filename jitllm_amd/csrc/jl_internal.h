@@ -13,7 +13,10 @@ struct jl_context {
     bool owns_stream;
     int compute_units;
     char name[128];
+    void *scratch;   // JL_CONTEXT_SCRATCH_BYTES of device memory for results handed from one launch of
+                     // a call to the next (calls on a context are ordered on its stream)
 };
+#define JL_CONTEXT_SCRATCH_BYTES 4096
 
 struct jl_weight {
     jl_context *ctx;

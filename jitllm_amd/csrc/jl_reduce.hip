@@ -8,7 +8,8 @@
 //   jl_argmax      index of the first maximum of the logits -- argmaxLogits (:95-127) on the device,
 //                  FloatTensor.argmax (J/tensor/standard/FloatTensor.java:168-181) on the host.
 //
-// Both are one workgroup: the inputs are a few KB to half a MB and the result is one word.
+// jl_rms_scale is one workgroup (a few KB of input); jl_argmax spreads the half MB of logits over
+// up to 128 workgroups and folds their results in a second, single-workgroup launch.
 #include "jl_device.h"
 #include "jl_internal.h"
 
@@ -51,23 +52,17 @@ __device__ __forceinline__ void keep_better(float &v, int &i, float ov, int oi) 
     }
 }
 
-__global__ void __launch_bounds__(kThreads) jl_argmax_kernel(const float *values, int n, int32_t *index) {
-    __shared__ float pv[kThreads / JL_WAVE];
-    __shared__ int pi[kThreads / JL_WAVE];
-    const int tid = threadIdx.x;
-    float best = -INFINITY;
-    int at = INT_MAX;
-    const int n4 = ((uintptr_t)values & 15) == 0 ? n / 4 : 0;
-    for (int i = tid; i < n4; i += kThreads) {
-        const float4 v = ((const float4 *)values)[i];
-        // ascending index inside a thread: a strict comparison keeps the first of equals
-        if (v.x > best) { best = v.x; at = 4 * i; }
-        if (v.y > best) { best = v.y; at = 4 * i + 1; }
-        if (v.z > best) { best = v.z; at = 4 * i + 2; }
-        if (v.w > best) { best = v.w; at = 4 * i + 3; }
-    }
-    for (int i = n4 * 4 + tid; i < n; i += kThreads)
-        if (values[i] > best) { best = values[i]; at = i; }
+// Two launches: workgroup g scans the float4s g, g + G, ... and leaves its best (value, index) in
+// the context's scratch; one small workgroup then folds the G cells.  (A single launch whose last
+// workgroup folds needs device-scope fences, which cost more here than the second launch.)
+constexpr int kArgmaxGroups = 128, kArgmaxThreads = 256;
+
+struct ArgmaxCells {
+    float value[kArgmaxGroups];
+    int index[kArgmaxGroups];
+};
+
+__device__ __forceinline__ void fold_waves(float &best, int &at, float *pv, int *pi, int tid, int waves) {
 #pragma unroll
     for (int o = JL_WAVE / 2; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, JL_WAVE);
@@ -79,8 +74,43 @@ __global__ void __launch_bounds__(kThreads) jl_argmax_kernel(const float *values
         pi[tid / JL_WAVE] = at;
     }
     __syncthreads();
+    if (tid == 0)
+        for (int w = 1; w < waves; w++) keep_better(best, at, pv[w], pi[w]);
+}
+
+__global__ void __launch_bounds__(kArgmaxThreads) jl_argmax_scan(const float *values, int n, ArgmaxCells *cells) {
+    __shared__ float pv[kArgmaxThreads / JL_WAVE];
+    __shared__ int pi[kArgmaxThreads / JL_WAVE];
+    const int tid = threadIdx.x;
+    float best = -INFINITY;
+    int at = INT_MAX;
+    const int n4 = ((uintptr_t)values & 15) == 0 ? n / 4 : 0;
+    for (int i = blockIdx.x * kArgmaxThreads + tid; i < n4; i += gridDim.x * kArgmaxThreads) {
+        const float4 v = ((const float4 *)values)[i];
+        // ascending index inside a thread: a strict comparison keeps the first of equals
+        if (v.x > best) { best = v.x; at = 4 * i; }
+        if (v.y > best) { best = v.y; at = 4 * i + 1; }
+        if (v.z > best) { best = v.z; at = 4 * i + 2; }
+        if (v.w > best) { best = v.w; at = 4 * i + 3; }
+    }
+    for (int i = n4 * 4 + blockIdx.x * kArgmaxThreads + tid; i < n; i += gridDim.x * kArgmaxThreads)
+        if (values[i] > best) { best = values[i]; at = i; }
+    fold_waves(best, at, pv, pi, tid, kArgmaxThreads / JL_WAVE);
     if (tid == 0) {
-        for (int w = 1; w < kThreads / JL_WAVE; w++) keep_better(best, at, pv[w], pi[w]);
+        cells->value[blockIdx.x] = best;
+        cells->index[blockIdx.x] = at;
+    }
+}
+
+__global__ void __launch_bounds__(kArgmaxGroups) jl_argmax_fold(const float *values, const ArgmaxCells *cells,
+                                                                int groups, int32_t *index) {
+    __shared__ float pv[kArgmaxGroups / JL_WAVE];
+    __shared__ int pi[kArgmaxGroups / JL_WAVE];
+    const int tid = threadIdx.x;
+    float best = tid < groups ? cells->value[tid] : -INFINITY;
+    int at = tid < groups ? cells->index[tid] : INT_MAX;
+    fold_waves(best, at, pv, pi, tid, kArgmaxGroups / JL_WAVE);
+    if (tid == 0) {
         // the host scan starts from element 0 and moves only on a strictly larger value: nothing
         // beats a NaN there, and with no value above -inf it stays at 0
         if (at == INT_MAX || values[0] != values[0]) at = 0;
@@ -97,7 +127,13 @@ int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, f
 }
 
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
-    hipLaunchKernelGGL(jl_argmax_kernel, dim3(1), dim3(kThreads), 0, ctx->stream, values, (int)n, index);
+    static_assert(sizeof(ArgmaxCells) <= JL_CONTEXT_SCRATCH_BYTES, "argmax cells exceed the context scratch");
+    int groups = (int)((n / 4 + kArgmaxThreads - 1) / kArgmaxThreads);
+    groups = groups < 1 ? 1 : groups > kArgmaxGroups ? kArgmaxGroups : groups;
+    ArgmaxCells *cells = (ArgmaxCells *)ctx->scratch;
+    hipLaunchKernelGGL(jl_argmax_scan, dim3(groups), dim3(kArgmaxThreads), 0, ctx->stream, values, (int)n, cells);
+    JL_HIP(hipGetLastError());
+    hipLaunchKernelGGL(jl_argmax_fold, dim3(1), dim3(kArgmaxGroups), 0, ctx->stream, values, cells, groups, index);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }

@@ -98,21 +98,26 @@ class QuantizedProjections:
         TransformerComputeKernels.java:378-437; CpuOperations.rmsnorm :60-66)."""
         L.check(self._lib.jl_rms_scale(self.context.handle, x.ptr, n, float(eps), scale.ptr))
 
-    def rmsMatvec(self, x: FloatArray, rmsWeights: FloatArray, rmsScale: FloatArray, out: FloatArray,
-                  w: TornadoTensor, n: int, d: int) -> None:
-        """``out = w . (rmsWeights * (rmsScale[0] * x))``: the final norm folded into the vocabulary
-        projection (reductionOneBlock2WithLogits + the projection, LogitsQ8_0Layer.java:85-97)."""
+    def rmsMatvec(self, x: FloatArray, rmsWeights: FloatArray, rmsScale: FloatArray | None,
+                  out: FloatArray, w: TornadoTensor, n: int, d: int, eps: float = 0.0) -> None:
+        """``out = w . (rmsWeights * (s * x))``: the final norm folded into the vocabulary
+        projection (reductionOneBlock2WithLogits + the projection, LogitsQ8_0Layer.java:85-97).
+        ``s`` is ``rmsScale[0]``, or with ``rmsScale`` None computed in the kernel from ``eps``."""
         _check_shape(w, n, d)
         L.check(self._lib.jl_gemv_rms(self.context.handle, w.handle, x.ptr, rmsWeights.ptr,
-                                      rmsScale.ptr, out.ptr, L.JL_STORE))
+                                      rmsScale.ptr if rmsScale is not None else None, float(eps),
+                                      out.ptr, L.JL_STORE))
 
     def fusedRmsNormQKV(self, x: FloatArray, q: FloatArray, k: FloatArray, v: FloatArray,
-                        rmsWeights: FloatArray, rmsScale: FloatArray, wq: TornadoTensor,
-                        wk: TornadoTensor, wv: TornadoTensor) -> None:
+                        rmsWeights: FloatArray, rmsScale: FloatArray | None, wq: TornadoTensor,
+                        wk: TornadoTensor, wv: TornadoTensor, eps: float = 0.0) -> None:
         """fusedRmsNormQKVMatmulQ8 (TransformerComputeKernelsLayered.java:2116-2220): q | k | v of
-        the normalised activations, which are never written out."""
+        the normalised activations, which are never written out.  With ``rmsScale`` None the scale
+        is computed in the kernel from ``eps`` and the separate reduction is not needed."""
         L.check(self._lib.jl_gemv_qkv_rms(self.context.handle, wq.handle, wk.handle, wv.handle, x.ptr,
-                                          rmsWeights.ptr, rmsScale.ptr, q.ptr, k.ptr, v.ptr))
+                                          rmsWeights.ptr,
+                                          rmsScale.ptr if rmsScale is not None else None, float(eps),
+                                          q.ptr, k.ptr, v.ptr))
 
     def fullyFusedRmsNormGateUp(self, x: FloatArray, rmsWeights: FloatArray, eps: float,
                                 w1: TornadoTensor, w3: TornadoTensor, n: int, d: int) -> None:

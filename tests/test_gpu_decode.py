@@ -215,8 +215,15 @@ def test_fused_rms_qkv(ctx, t, dq, dkv, n):
     proj.fusedRmsNormQKV(dx, *outs, drw, scale, *ws)
     ctx.sync()
     assert np.array_equal(dx.get(), x)   # the normalised activations are never written back
-    for raw, d, out in zip(raws, (dq, dkv, dkv), outs):
-        ref = O.matmul(t, raw, xn, d, n)
+    refs = [O.matmul(t, raw, xn, d, n) for raw, d in zip(raws, (dq, dkv, dkv))]
+    for raw, d, out, ref in zip(raws, (dq, dkv, dkv), outs, refs):
+        assert rel_err(out.get(), ref, magnitude(t, raw, xn, d, n)) < 2e-5
+    # the same with the scale computed inside the kernel
+    for out in outs:
+        out.init(POISON)
+    proj.fusedRmsNormQKV(dx, *outs, drw, None, *ws, eps=1e-5)
+    ctx.sync()
+    for raw, d, out, ref in zip(raws, (dq, dkv, dkv), outs, refs):
         assert rel_err(out.get(), ref, magnitude(t, raw, xn, d, n)) < 2e-5
 
 
@@ -271,6 +278,10 @@ def test_rms_vocabulary_projection_and_argmax(ctx):
     got = logits.get()
     assert rel_err(got, ref, magnitude(t, raw, xn, d, n)) < 2e-5
     assert int(token.download(np.int32, 1)[0]) == O.argmax(got)
+    logits.init(POISON)
+    proj.rmsMatvec(dx, drw, None, logits, upload(ctx, t, raw, d, n), n, d, eps=1e-5)
+    ctx.sync()
+    assert rel_err(logits.get(), ref, magnitude(t, raw, xn, d, n)) < 2e-5
 
 
 @pytest.mark.parametrize("n", [1, 5, 1023, 4097, 128256])
@@ -292,6 +303,26 @@ def test_argmax_ties_and_edges(ctx, n):
         proj.argmax(ctx.from_numpy(v), n, token)
         ctx.sync()
         assert int(token.download(np.int32, 1)[0]) == O.argmax(v)
+
+
+def test_rms_folding_refuses_what_it_has_no_kernel_for(ctx):
+    """A row length the tile kernel does not take is refused by name, never normalised some other
+    way (the caller then runs the unfused sequence, as the reference does)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd._lib import UnsupportedProjection
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("rms unsupported")
+    t, d, n = O.Q8_0, 16, 96
+    w = upload(ctx, t, synthetic.weight(t, d, n, seed=671), d, n)
+    x, rw = ctx.from_numpy(synthetic.activations(n, seed=672)), ctx.float_array(n, fill=1.0)
+    out = ctx.float_array(d, fill=POISON)
+    proj = QuantizedProjections(ctx, TornadoWorkspace(wrapHb=out))
+    with pytest.raises(UnsupportedProjection, match="row length of 96"):
+        proj.rmsMatvec(x, rw, None, out, w, n, d, eps=1e-5)
+    with pytest.raises(UnsupportedProjection, match="row length of 96"):
+        proj.fullyFusedRmsNormGateUp(x, rw, 1e-5, w, w, n, d)
+    ctx.sync()
+    assert np.all(out.get() == POISON)
 
 
 def test_mixed_gate_up_runs_two_projections_and_swiglu(ctx):
