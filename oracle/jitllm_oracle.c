@@ -19,6 +19,8 @@
  *                              zero is used here (what the JDK's own fallback does) and the result
  *                              is held to a few ulp, not bit equality: "parity unpinned" for the
  *                              last bits of that one addition chain only.
+ *   rmsnorm, argmax            closed forms (constant vectors, powers of two, eps-dominated input), a
+ *                              float64 evaluation, numpy's argmax with ties, -inf and NaN cases.
  *   java.util.Random           published first outputs for seeds 0 and 42.
  */
 #include "jitllm_oracle.h"
