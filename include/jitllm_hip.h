@@ -221,6 +221,52 @@ int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const f
             int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
             int math, void *workspace, size_t workspace_bytes);
 
+/* ---- GGUF files: the caller either side of jl_weight_upload --------------------------------- */
+
+/*
+ * Parses a GGUF file's header, metadata and tensor infos and keeps the file mapped read-only
+ * (GGUF.loadGGUFMetadata, J/format/GGUF.java:40-115; versions 2 and 3, general.alignment or 32).
+ * A file the reference refuses is refused with the same words: "unsupported header.magic ...",
+ * "unsupported header.version ...", "Model file not found: ...".  Host work only; needs no GPU.
+ */
+typedef struct jl_gguf jl_gguf;
+int jl_gguf_open(const char *path, jl_gguf **out);
+int jl_gguf_close(jl_gguf *g);
+int jl_gguf_version(const jl_gguf *g);
+int jl_gguf_alignment(const jl_gguf *g);
+int64_t jl_gguf_data_offset(const jl_gguf *g);   /* file offset of the tensor-data section (:71-96) */
+int64_t jl_gguf_tensor_count(const jl_gguf *g);
+int64_t jl_gguf_metadata_count(const jl_gguf *g);
+
+/*
+ * Tensor `index` in file order, or by name (jl_gguf_find: index, -1 if absent): GGUFTensorInfo
+ * (J/format/GGUF.java:297-322, 520).  `dims` are in GGUF ne order (dims[0] = row length), unused
+ * ones 1; `file_offset` is absolute; `bytes` follows the block geometry of J/format/GGMLType.java:5-54
+ * and is -1 for a type the reference cannot read either.  `name` stays valid until jl_gguf_close.
+ */
+int64_t jl_gguf_find(const jl_gguf *g, const char *name);
+int jl_gguf_tensor_info(const jl_gguf *g, int64_t index, const char **name, int *ggml_type, int *n_dims,
+                        int64_t dims[4], int64_t *file_offset, int64_t *bytes);
+
+/*
+ * Metadata by key (GGUF.readHeader / readMetadataValueOfType, :365-474): integers and booleans as
+ * int64, floats as double, strings by pointer (valid until jl_gguf_close); of an array only the
+ * element type (gguf_metadata_value_type) and the count are kept.  A missing key or a value of
+ * another kind is JL_ERR_INVALID.
+ */
+int jl_gguf_metadata_int(const jl_gguf *g, const char *key, int64_t *value);
+int jl_gguf_metadata_float(const jl_gguf *g, const char *key, double *value);
+int jl_gguf_metadata_string(const jl_gguf *g, const char *key, const char **value, int64_t *length);
+int jl_gguf_metadata_array(const jl_gguf *g, const char *key, int *element_type, int64_t *count);
+
+/*
+ * jl_weight_upload of a two-dimensional Q8_0 / Q4_0 / Q4_K tensor straight from the mapped file
+ * (ModelLoader.loadTornadoTensorNative, J/model/loader/ModelLoader.java:246-290, without the
+ * 16-byte array header the reference's segments carry, GGUF.java:214-268).  Another type is
+ * JL_ERR_UNSUPPORTED naming it; a tensor that runs past the end of the file is refused (:236-247).
+ */
+int jl_gguf_upload(jl_context *ctx, const jl_gguf *g, const char *name, jl_weight **out);
+
 #ifdef __cplusplus
 }
 #endif

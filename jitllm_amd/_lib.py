@@ -51,6 +51,21 @@ SYMBOLS = {
     "jl_gemv_qkv_rms": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_float, vp, vp, vp]),
     "jl_gemv_gate_up_rms": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp]),
     "jl_argmax": (C.c_int, [vp, vp, i64, vp]),
+    "jl_gguf_open": (C.c_int, [C.c_char_p, C.POINTER(vp)]),
+    "jl_gguf_close": (C.c_int, [vp]),
+    "jl_gguf_version": (C.c_int, [vp]),
+    "jl_gguf_alignment": (C.c_int, [vp]),
+    "jl_gguf_data_offset": (i64, [vp]),
+    "jl_gguf_tensor_count": (i64, [vp]),
+    "jl_gguf_metadata_count": (i64, [vp]),
+    "jl_gguf_find": (i64, [vp, C.c_char_p]),
+    "jl_gguf_tensor_info": (C.c_int, [vp, i64, C.POINTER(C.c_char_p), C.POINTER(C.c_int),
+                                      C.POINTER(C.c_int), C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)]),
+    "jl_gguf_metadata_int": (C.c_int, [vp, C.c_char_p, C.POINTER(i64)]),
+    "jl_gguf_metadata_float": (C.c_int, [vp, C.c_char_p, C.POINTER(C.c_double)]),
+    "jl_gguf_metadata_string": (C.c_int, [vp, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(i64)]),
+    "jl_gguf_metadata_array": (C.c_int, [vp, C.c_char_p, C.POINTER(C.c_int), C.POINTER(i64)]),
+    "jl_gguf_upload": (C.c_int, [vp, vp, C.c_char_p, C.POINTER(vp)]),
     "jl_gemm_workspace_bytes": (C.c_size_t, [i64, i64, i64, C.c_int]),
     "jl_gemm": (C.c_int, [vp, C.POINTER(vp), C.c_int, vp, vp, i64, i64, i64, i64, C.c_int, C.c_int,
                           vp, C.c_size_t]),

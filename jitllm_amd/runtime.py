@@ -142,6 +142,14 @@ class TornadoTensor:
         self.handle = h
         self.nbytes = want
 
+    @classmethod
+    def adopt(cls, ctx: Context, handle, ggml_type: GGMLType, rows: int, cols: int, nbytes: int) -> "TornadoTensor":
+        """Wraps a jl_weight the library created itself (e.g. from a mapped GGUF file)."""
+        self = cls.__new__(cls)
+        self.ctx, self.ggml_type = ctx, GGMLType(ggml_type)
+        self.rows, self.cols, self.handle, self.nbytes = int(rows), int(cols), handle, int(nbytes)
+        return self
+
     def data_type(self) -> GGMLType:
         return self.ggml_type
 

@@ -1,0 +1,127 @@
+"""The GGUF reader behind the C ABI, held against files written by an independent writer
+(tests/gguf_writer.py).  Parsing is host work: no GPU is needed."""
+import numpy as np
+import pytest
+
+import gguf_writer as W
+from jitllm_amd import synthetic
+from jitllm_amd._lib import JitllmHipError
+from jitllm_amd.ggml import GGMLType
+from jitllm_amd.gguf import GGUF
+
+META = [
+    ("general.architecture", W.STRING, "llama"),
+    ("general.name", W.STRING, "tiny é中"),           # non-ASCII UTF-8 in a value
+    ("llama.block_count", W.U32, 2),
+    ("llama.context_length", W.U64, 1 << 33),
+    ("llama.attention.layer_norm_rms_epsilon", W.F32, 1e-5),
+    ("llama.rope.freq_base", W.F64, 500000.0),
+    ("llama.some_i8", W.I8, -7),
+    ("llama.some_i16", W.I16, -300),
+    ("llama.some_u16", W.U16, 65535),
+    ("llama.some_i32", W.I32, -123456),
+    ("llama.some_i64", W.I64, -(1 << 40)),
+    ("llama.flag", W.BOOL, True),
+    ("tokenizer.ggml.tokens", W.ARRAY, (W.STRING, ["<s>", "</s>", "a", "bc", ""])),
+    ("tokenizer.ggml.scores", W.ARRAY, (W.F32, [0.0, -1.0, -2.5])),
+    ("tokenizer.ggml.token_type", W.ARRAY, (W.I32, [1, 2, 3, 4])),
+    ("nested.arrays", W.ARRAY, (W.ARRAY, [(W.U8, [1, 2, 3]), (W.STRING, ["x", "yz"])])),
+]
+
+
+def tensors():
+    d, n = 8, 256
+    return [
+        ("blk.0.attn_q.weight", (n, d), 8, synthetic.weight(GGMLType.Q8_0, d, n, seed=1)),
+        ("blk.0.ffn_gate.weight", (n, 2 * d), 2, synthetic.weight(GGMLType.Q4_0, 2 * d, n, seed=2)),
+        ("blk.0.ffn_down.weight", (n, d), 12, synthetic.weight(GGMLType.Q4_K, d, n, seed=3)),
+        ("blk.0.attn_norm.weight", (n,), 0, np.arange(n, dtype=np.float32)),
+        ("token_embd.weight", (n, 3), 14, np.zeros(3 * 210, dtype=np.uint8)),          # Q6_K: 210 B / 256
+        ("odd.iq2", (256,), 16, np.zeros(10, dtype=np.uint8)),                         # a type with no geometry
+    ]
+
+
+@pytest.mark.parametrize("version,alignment", [(3, None), (2, None), (3, 64), (3, 4096)])
+def test_reader_agrees_with_what_was_written(tmp_path, version, alignment):
+    path = tmp_path / "m.gguf"
+    ts = tensors()
+    where = W.write_gguf(path, META, ts, version=version, alignment=alignment)
+    with GGUF(path) as g:
+        assert g.version == version
+        assert g.getAlignment() == (alignment or 32)
+        assert g.getTensorDataOffset() % g.getAlignment() == 0
+        assert g.tensor_count() == len(ts)
+        assert g.metadata_count() == len(META) + (1 if alignment else 0)
+        assert g.metadata_string("general.architecture") == "llama"
+        assert g.metadata_string("general.name") == "tiny é中"
+        assert g.metadata_int("llama.block_count") == 2
+        assert g.metadata_int("llama.context_length") == 1 << 33
+        assert g.metadata_float("llama.attention.layer_norm_rms_epsilon") == float(np.float32(1e-5))
+        assert g.metadata_float("llama.rope.freq_base") == 500000.0
+        assert (g.metadata_int("llama.some_i8"), g.metadata_int("llama.some_i16")) == (-7, -300)
+        assert (g.metadata_int("llama.some_u16"), g.metadata_int("llama.some_i32")) == (65535, -123456)
+        assert g.metadata_int("llama.some_i64") == -(1 << 40)
+        assert g.metadata_int("llama.flag") == 1
+        assert g.metadata_array("tokenizer.ggml.tokens") == (W.STRING, 5)
+        assert g.metadata_array("tokenizer.ggml.scores") == (W.F32, 3)
+        assert g.metadata_array("nested.arrays") == (W.ARRAY, 2)
+        infos = g.getTensorInfos()
+        raw_file = path.read_bytes()
+        for name, dims, gtype, raw in ts:
+            ti = infos[name]
+            assert (ti.dimensions, ti.ggml_type, ti.file_offset) == (tuple(dims), gtype, where[name])
+            assert ti.file_offset % g.getAlignment() == 0
+            want = np.ascontiguousarray(raw).tobytes()
+            if gtype == 16:
+                assert ti.nbytes == -1
+            else:
+                assert ti.nbytes == len(want)
+                assert raw_file[ti.file_offset:ti.file_offset + ti.nbytes] == want
+        assert g.find("blk.0.attn_q.weight") == 0 and g.find("no.such.tensor") == -1
+        for i, (name, *_rest) in enumerate(ts):     # file order is kept
+            assert g.tensor_info(i).name == name
+
+
+def test_wrong_kinds_and_missing_keys_are_errors(tmp_path):
+    path = tmp_path / "m.gguf"
+    W.write_gguf(path, META, tensors())
+    with GGUF(path) as g:
+        with pytest.raises(JitllmHipError, match="no metadata key"):
+            g.metadata_int("llama.absent")
+        with pytest.raises(JitllmHipError, match="not an integer"):
+            g.metadata_int("general.architecture")
+        with pytest.raises(JitllmHipError, match="not a string"):
+            g.metadata_string("llama.block_count")
+        with pytest.raises(JitllmHipError, match="not a float"):
+            g.metadata_float("llama.block_count")
+        with pytest.raises(JitllmHipError, match="not an array"):
+            g.metadata_array("llama.block_count")
+        with pytest.raises(JitllmHipError):
+            g.tensor_info(99)
+
+
+def test_files_the_reference_refuses_are_refused_in_its_words(tmp_path):
+    bad_magic = tmp_path / "magic.gguf"
+    W.write_gguf(bad_magic, META, tensors(), magic=b"GGML")
+    with pytest.raises(JitllmHipError, match="unsupported header.magic"):
+        GGUF(bad_magic)
+    v1 = tmp_path / "v1.gguf"
+    W.write_gguf(v1, META, tensors(), version=1)
+    with pytest.raises(JitllmHipError, match="unsupported header.version 1"):
+        GGUF(v1)
+    with pytest.raises(JitllmHipError, match="Model file not found"):
+        GGUF(tmp_path / "absent.gguf")
+    cut = tmp_path / "cut.gguf"
+    W.write_gguf(cut, META, tensors())
+    blob = cut.read_bytes()
+    cut.write_bytes(blob[:200])                      # ends inside the metadata
+    with pytest.raises(JitllmHipError, match="ends early|malformed"):
+        GGUF(cut)
+    odd = tmp_path / "align.gguf"
+    W.write_gguf(odd, META, tensors(), alignment=48)
+    with pytest.raises(JitllmHipError, match="not a power of two"):
+        GGUF(odd)
+    tiny = tmp_path / "tiny.gguf"
+    tiny.write_bytes(b"GGUF")
+    with pytest.raises(JitllmHipError, match="too short"):
+        GGUF(tiny)
