@@ -12,10 +12,11 @@
 // rows x 4 slices) multiplies them with the matching activation fragments on
 // v_mfma_f32_16x16x32_f16.  The MFMA sums over 32 "k slots"; slot (g, e) of MFMA i is column
 // 64 (slice of lane group g) + 8 i + e, the same for both operands, so no data crosses lanes.
-// The activation fragments (fp16 copy of X, made once per call) depend on the slice only and stay
-// in registers for the whole kernel.  A wave's result is a partial sum over its 256 columns; the
-// waves of a workgroup fold through LDS one tile later, rows wider than the workgroup's span are
-// cut across workgroups and folded by jl_skinny_reduce.
+// The activation fragments (read as fp32 and rounded to fp16 by the kernel itself) depend on the
+// slice only and stay in registers for the whole kernel.  A wave's result is a partial sum over its
+// 256 columns; a wave of its own folds the compute waves' partials through LDS one tile later and
+// applies the epilogue, rows wider than the workgroup's span are cut across workgroups and folded
+// by jl_skinny_reduce.
 #include "jl_device.h"
 #include "jl_internal.h"
 
@@ -221,6 +222,9 @@ __device__ __forceinline__ float skinny_swiglu(float g, float u) { return g / (1
 // waves that time adds to the arithmetic instead of hiding behind it, so the copies have waves of
 // their own and the two kinds meet at one barrier per tile.
 constexpr int kDmaWaves = 2;
+// ... and so has the fold of the compute waves' partial sums with the epilogue: a chain of LDS
+// round trips, exponentials and stores that would otherwise stall the decode of the next tile.
+constexpr int kFoldWaves = 1;
 constexpr int max_slices(int) { return 32; }
 
 // 16-byte loads per DMA wave and tile (upper bound): a tile row takes span_bytes + 16 bytes of LDS
@@ -230,11 +234,11 @@ template <int TYPE> struct Loads { static constexpr int kPerWave = TYPE == JL_Q8
 // ZIN: spans of a row that one workgroup walks itself, one tile after the other, adding their
 // results in registers (it then holds ZIN sets of activation fragments); p.Z spans of ZIN each.
 template <int TYPE, int NBB, bool DUAL, int ZIN>
-__global__ void __launch_bounds__(512 + 64 * kDmaWaves) jl_gemm_skinny(SkinnyParams p) {
+__global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_skinny(SkinnyParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int LD = Loads<TYPE>::kPerWave;
     const int tid = threadIdx.x;
-    const int waves = (blockDim.x >> 6) - kDmaWaves;   // compute waves
+    const int waves = (blockDim.x >> 6) - kDmaWaves - kFoldWaves;   // compute waves
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int z = blockIdx.x % p.Z;            // this workgroup's run of ZIN spans
@@ -276,7 +280,7 @@ __global__ void __launch_bounds__(512 + 64 * kDmaWaves) jl_gemm_skinny(SkinnyPar
     const int stride = gridDim.x / p.Z;
     const int mine = wg < total_groups ? (total_groups - wg + stride - 1) / stride : 0;
 
-    if (wave >= waves) {
+    if (wave >= waves && wave < waves + kDmaWaves) {
         // ---- copy waves.  Slot s of a tile is 16 bytes at LDS offset 16 s: row s / slots_per_row,
         // byte 16 (s % slots_per_row) of the row's span.  A slot past the data (the padding behind
         // each row, slots behind the last row) re-reads a neighbouring real slot -- never one
@@ -335,6 +339,83 @@ __global__ void __launch_bounds__(512 + 64 * kDmaWaves) jl_gemm_skinny(SkinnyPar
         return;
     }
 
+    if (wave >= waves + kDmaWaves) {
+        // ---- fold wave.  After the barrier that opens group it + 1 the partial sums of group it
+        // (parity it & 1) are complete; they are overwritten two groups later, behind barriers this
+        // wave takes part in, so it has one group's time.  A partial is what one lane of one
+        // compute wave held: weight rows 4 (o / 16) .. + 3 of activation row 16 b + o % 16, for
+        // lane o and row block b; in a gate/up group lanes o >= 32 hold the up rows of the outputs
+        // of lane o - 32.  Lane o of this wave adds the waves' partials of its (b, o) in wave
+        // order and applies the epilogue.
+        const int o = lane;
+        const int go = o >> 4;
+        auto fold = [&](int group, int par) {
+            const Segment sg = segment_of(group);
+            const uint32_t pbase = lds0 + par * partial_bytes + o * 16;
+            const int local = (group - sg.group_begin) * out_rows + 4 * go;  // first of 4 outputs
+#pragma unroll
+            for (int b = 0; b < NBB; b++) {
+                if (DUAL && o >= 32) break;
+                floatx4 sum = {0.f, 0.f, 0.f, 0.f}, sum_up = {0.f, 0.f, 0.f, 0.f};
+                for (int w0 = 0; w0 < waves; w0 += 4) {
+                    floatx4 v[4], u[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const uint32_t a = pbase + (w0 + j < waves ? w0 + j : w0) * (NBB * 1024) + b * 1024;
+                        asm volatile("ds_read_b128 %0, %1" : "=&v"(v[j]) : "v"(a) : "memory");
+                        if constexpr (DUAL) asm volatile("ds_read_b128 %0, %1 offset:512" : "=&v"(u[j]) : "v"(a) : "memory");
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
+                    if constexpr (DUAL) asm volatile("" : "+v"(u[0]), "+v"(u[1]), "+v"(u[2]), "+v"(u[3]));
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (w0 + j < waves) {
+                            sum += v[j];
+                            if constexpr (DUAL) sum_up += u[j];
+                        }
+                    }
+                }
+                const int m = 16 * b + (o & 15);
+                if (p.Z > 1) {
+                    // partial sums of this span: [z][row][group * 16 + weight row of the group]
+                    float *pp = p.planes + ((int64_t)z * (16 * NBB) + m) * ((int64_t)total_groups * 16) + group * 16 + 4 * go;
+                    *(floatx4 *)pp = sum;
+                    if constexpr (DUAL) *(floatx4 *)(pp + 8) = sum_up;
+                    continue;
+                }
+                if (m >= p.rows) continue;
+                float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + sg.col_begin + local;
+                const int left = sg.rows - local;
+                float r[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = DUAL ? skinny_swiglu(sum[e], sum_up[e]) : sum[e];
+                if (p.epilogue == JL_RESIDUAL) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (e < left) unsafeAtomicAdd(dst + e, r[e]);   // one add per element, no load to wait for
+                } else if (left >= 4 && (((uintptr_t)dst) & 15) == 0) {
+                    *(floatx4 *)dst = floatx4{r[0], r[1], r[2], r[3]};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (e < left) dst[e] = r[e];
+                }
+            }
+        };
+        for (int it = 0; it < mine; it++) {
+#pragma unroll
+            for (int q = 0; q < ZIN; q++) {
+                __builtin_amdgcn_s_barrier();
+                if (q == 0 && it > 0) fold(wg + (it - 1) * stride, (it - 1) & 1);
+            }
+        }
+        if (mine > 0) {
+            __builtin_amdgcn_s_barrier();
+            fold(wg + (mine - 1) * stride, (mine - 1) & 1);
+        }
+        return;
+    }
+
     // ---- compute waves
     const int c = lane & 15;                   // row of the group
     const int g = lane >> 4;                   // which of the wave's four slices
@@ -383,111 +464,14 @@ __global__ void __launch_bounds__(512 + 64 * kDmaWaves) jl_gemm_skinny(SkinnyPar
         }
     }
 
-    // Folds the waves' partial sums of group `group` (parity `par`) and applies the epilogue.  A
-    // partial is what one lane of one wave held: weight rows 4 (o / 16) .. + 3 of activation row
-    // 16 b + o % 16, for lane o and row block b; in a gate/up group lanes o >= 32 hold the up rows of
-    // the outputs of lane o - 32.  The (b, o) pairs are dealt out over all compute waves, and inside
-    // a wave one lane reads one wave's partial of one pair: `waves` neighbouring lanes then add up
-    // with DPP moves in a fixed order, the first of them applies the epilogue.  Which lane does what
-    // never changes, so everything that depends on that only is worked out once, here.  (Wave
-    // counts that are not a power of two fold lane by lane instead, `serial` below.)
-    constexpr int kPasses = 2;   // at most 16 float4 sums per wave x 8 waves = 128 lanes' worth
-    const int lanes_out = DUAL ? 32 : 64;
-    const int per = (lanes_out + waves - 1) / waves;     // lanes o per wave
-    const bool serial = (waves & (waves - 1)) != 0;
-    const int wshift = 31 - __builtin_clz(waves | 1);
-    int fin_off[kPasses];      // LDS offset of what this lane reads (inside a parity), or -1
-    int fin_go[kPasses];       // o / 16: which four weight rows
-    bool fin_owner[kPasses];   // this lane applies the epilogue of its pair
-    float *fin_c[kPasses];     // output row of the pair (null when the row is not active)
-    float *fin_plane[kPasses]; // its row in this span's plane
-#pragma unroll
-    for (int ps = 0; ps < kPasses; ps++) {
-        const int idx = ps * 64 + lane;
-        const int wv = serial ? 0 : idx & (waves - 1);       // whose partial
-        const int unit = serial ? idx : idx >> wshift;        // which sum of this wave
-        const int pi = (DUAL && !serial) ? unit >> 1 : unit;  // which (b, o) pair
-        const int half = (DUAL && !serial) ? unit & 1 : 0;    // gate / up
-        const int b = pi / per;
-        const int o = wave * per + (pi - b * per);
-        const bool valid = b < NBB && o < lanes_out;
-        const int m = 16 * b + (o & 15);
-        fin_off[ps] = valid ? wv * (NBB * 1024) + b * 1024 + (o + 32 * half) * 16 : -1;
-        fin_go[ps] = o >> 4;
-        fin_owner[ps] = valid && wv == 0 && half == 0;
-        fin_c[ps] = m < p.rows ? p.C + (int64_t)m * p.ldo + p.col_offset : nullptr;
-        fin_plane[ps] = p.Z > 1 ? p.planes + ((int64_t)z * (16 * NBB) + m) * ((int64_t)total_groups * 16) : nullptr;
-    }
-    auto lane_sum = [&](float v) {   // over `waves` neighbouring lanes, every lane gets the total
-        if (waves >= 2) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
-        if (waves >= 4) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));
-        if (waves >= 8) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));
-        return v;
-    };
-    auto finish = [&](int group, int par) {
-        const Segment sg = segment_of(group);
-        const uint32_t pbase = lds0 + par * partial_bytes;
-#pragma unroll
-        for (int ps = 0; ps < kPasses; ps++) {
-            if (ps * 64 >= (serial ? per * NBB : (per * NBB * (DUAL ? 2 : 1)) << wshift)) break;   // uniform
-            floatx4 sum = {0.f, 0.f, 0.f, 0.f}, sum_up = {0.f, 0.f, 0.f, 0.f};
-            if (serial) {
-                if (fin_off[ps] >= 0) {
-                    for (int w = 0; w < waves; w++) {
-                        sum += lds_read_f4(pbase + fin_off[ps] + w * (NBB * 1024));
-                        if constexpr (DUAL) sum_up += lds_read_f4(pbase + fin_off[ps] + w * (NBB * 1024) + 32 * 16);
-                    }
-                }
-            } else {
-                if (fin_off[ps] >= 0) sum = lds_read_f4(pbase + fin_off[ps]);
-#pragma unroll
-                for (int e = 0; e < 4; e++) sum[e] = lane_sum(sum[e]);
-                if constexpr (DUAL) {
-                    // the up sums sit `waves` lanes further on
-#pragma unroll
-                    for (int e = 0; e < 4; e++) sum_up[e] = __shfl_down(sum[e], waves, 64);
-                }
-            }
-            if (!fin_owner[ps]) continue;
-            const int go = fin_go[ps];
-            const int local = (group - sg.group_begin) * out_rows + 4 * go;  // first of 4 outputs
-            if (p.Z > 1) {
-                // partial sums of this span: [z][row][group * 16 + weight row of the group]
-                float *pp = fin_plane[ps] + group * 16 + 4 * go;
-                *(floatx4 *)pp = sum;
-                if constexpr (DUAL) *(floatx4 *)(pp + 8) = sum_up;
-                continue;
-            }
-            if (!fin_c[ps]) continue;
-            float *dst = fin_c[ps] + sg.col_begin + local;
-            const int left = sg.rows - local;
-            float v[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = DUAL ? skinny_swiglu(sum[e], sum_up[e]) : sum[e];
-            if (p.epilogue == JL_RESIDUAL) {
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (e < left) unsafeAtomicAdd(dst + e, v[e]);
-            } else if (left >= 4 && (((uintptr_t)dst) & 15) == 0) {
-                *(floatx4 *)dst = floatx4{v[0], v[1], v[2], v[3]};
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (e < left) dst[e] = v[e];
-            }
-        }
-    };
-
     for (int it = 0; it < mine; it++) {
-        const int group = wg + it * stride;
         floatx4 total[NBB];
 #pragma unroll
         for (int b = 0; b < NBB; b++) total[b] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int q = 0; q < ZIN; q++) {
             const int t = it * ZIN + q;
-            __builtin_amdgcn_s_barrier();   // tile t has landed; the partial sums of group it - 1 are complete
-            if (q == 0 && it > 0) finish(group - stride, (it - 1) & 1);
+            __builtin_amdgcn_s_barrier();   // tile t has landed; the fold wave takes the sums of group it - 1
 
             half8 wf[8];
             decode_slice<TYPE>(ring0 + (t % p.stages) * stage_bytes + c * lds_row, sl, wf);
@@ -507,10 +491,7 @@ __global__ void __launch_bounds__(512 + 64 * kDmaWaves) jl_gemm_skinny(SkinnyPar
 #pragma unroll
         for (int b = 0; b < NBB; b++) lds_write_f4(pw + b * 1024, total[b]);
     }
-    if (mine > 0) {
-        __builtin_amdgcn_s_barrier();
-        finish(wg + (mine - 1) * stride, (mine - 1) & 1);
-    }
+    if (mine > 0) __builtin_amdgcn_s_barrier();
 }
 
 // Adds the spans' partial sums in span order and applies row scale and epilogue; one thread per
@@ -554,7 +535,7 @@ int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int gro
     int per_span = ctx->compute_units / p.Z;
     if (per_span < 1) per_span = 1;
     if (per_span > groups) per_span = groups;
-    hipLaunchKernelGGL(fn, dim3(per_span * p.Z), dim3(threads + 64 * kDmaWaves), lds, ctx->stream, p);
+    hipLaunchKernelGGL(fn, dim3(per_span * p.Z), dim3(threads + 64 * (kDmaWaves + kFoldWaves)), lds, ctx->stream, p);
     JL_HIP(hipGetLastError());
     if (p.Z > 1) {
         hipLaunchKernelGGL(jl_skinny_reduce<DUAL>, dim3((groups * 16 + 255) / 256, p.rows), dim3(256), 0,
@@ -626,7 +607,7 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     p.span_bytes = Ss * (type == JL_Q8_0 ? 68 : 36);
     if (Z > 1 && (size_t)Z * (16 * nbb) * groups * 16 * sizeof(float) > plane_bytes) return JL_OK;
 
-    const int threads = 16 * Ss;   // compute threads; the copy waves come on top
+    const int threads = 16 * Ss;   // compute threads; the copy and fold waves come on top
     const int per_wave = type == JL_Q8_0 ? 18 : 10;
     const int n_loads = (kGroup * ((p.span_bytes + 16) / 16) + 64 * kDmaWaves - 1) / (64 * kDmaWaves);
     if (n_loads > per_wave) return JL_OK;
