@@ -369,7 +369,7 @@ int jl_gguf_upload(jl_context *ctx, const jl_gguf *g, const char *name, jl_weigh
     const int64_t i = jl_gguf_find(g, name);
     JL_REQUIRE(i >= 0, "no tensor %s in the file", name);
     const TensorInfo &t = g->tensors[(size_t)i];
-    if (t.type != JL_Q8_0 && t.type != JL_Q4_0 && t.type != JL_Q4_K) {
+    if (jl_block_elems(t.type) == 0) {
         return jl_fail(JL_ERR_UNSUPPORTED, "tensor %s is ggml type %d, which has no projection kernel here",
                        name, t.type);
     }

@@ -1,7 +1,7 @@
-"""GGUF block geometry of the three weight representations on the path.
+"""GGUF block geometry of the weight representations on the path.
 
 Mirrors ``GGMLType`` of the reference (src/main/java/org/beehive/jitllm/format/GGMLType.java:7,13,
-18-20): a type is (elements per block, bytes per block); a ``[d x n]`` weight is ``d`` rows of
+18-20,27-29): a type is (elements per block, bytes per block); a ``[d x n]`` weight is ``d`` rows of
 ``n / block_elems`` blocks each, row-major, exactly as the file stores them.  The integer values
 are ggml's type ids, the ones a GGUF tensor-info record carries.
 """
@@ -14,6 +14,7 @@ class GGMLType(enum.IntEnum):
     Q4_0 = 2
     Q8_0 = 8
     Q4_K = 12
+    Q6_K = 14   # single-token projection and decode only
 
     @property
     def block_elems(self) -> int:
@@ -38,4 +39,5 @@ _GEOMETRY = {
     GGMLType.Q4_0: (32, 18),
     GGMLType.Q8_0: (32, 34),
     GGMLType.Q4_K: (256, 144),
+    GGMLType.Q6_K: (256, 210),
 }

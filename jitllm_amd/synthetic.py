@@ -6,6 +6,8 @@ Block value distributions:
   Q4_K  fp16 d ~ U(1e-3, 2e-2)/63, fp16 dmin ~ U(1e-3, 2e-2)*8/63 per super-block (so the largest
         weight magnitude d*63*15 stays near 0.3 and the minimum term roughly centres the range),
         8 (scale, min) pairs ~ U{0..63} packed into the 12 scale bytes, 128 bytes of nibbles
+  Q6_K  fp16 d ~ U(2e-5, 1e-4) per super-block (largest weight d*127*32 near 0.4), 16 signed
+        scales ~ U{-128..127}, 128 + 64 bytes of quant bits
   x     fp32 ~ N(0, 1)
 One seed makes one tensor (numpy PCG64).
 """
@@ -45,6 +47,10 @@ def weight(t: GGMLType, rows: int, cols: int, seed: int) -> np.ndarray:
     elif t == GGMLType.Q4_0:
         raw[:, 0:2] = _scales_f16(rng, blocks, 1e-3, 2e-2).view(np.uint8).reshape(blocks, 2)
         raw[:, 2:] = rng.integers(0, 256, size=(blocks, 16), dtype=np.uint8)
+    elif t == GGMLType.Q6_K:
+        raw[:, 0:192] = rng.integers(0, 256, size=(blocks, 192), dtype=np.uint8)
+        raw[:, 192:208] = rng.integers(-128, 128, size=(blocks, 16), dtype=np.int8).view(np.uint8)
+        raw[:, 208:210] = _scales_f16(rng, blocks, 2e-5, 1e-4).view(np.uint8).reshape(blocks, 2)
     else:
         raw[:, 0:2] = _scales_f16(rng, blocks, 1e-3 / 63, 2e-2 / 63).view(np.uint8).reshape(blocks, 2)
         raw[:, 2:4] = _scales_f16(rng, blocks, 8e-3 / 63, 16e-2 / 63).view(np.uint8).reshape(blocks, 2)

@@ -35,6 +35,7 @@
 #define Q4_0_BYTES 18
 #define QK_K 256
 #define Q4_K_BYTES 144
+#define Q6_K_BYTES 210
 
 int jo_max_threads(void) { return omp_get_max_threads(); }
 
@@ -44,6 +45,7 @@ int jo_block_elems(int type) {
         case JO_Q4_0: return Q_BLOCK;
         case JO_Q8_0: return Q_BLOCK;
         case JO_Q4_K: return QK_K;
+        case JO_Q6_K: return QK_K;
         default: return 0;
     }
 }
@@ -53,6 +55,7 @@ int jo_block_bytes(int type) {
         case JO_Q4_0: return Q4_0_BYTES;
         case JO_Q8_0: return Q8_0_BYTES;
         case JO_Q4_K: return Q4_K_BYTES;
+        case JO_Q6_K: return Q6_K_BYTES;
         default: return 0;
     }
 }
@@ -174,11 +177,42 @@ static inline float q4_k_get(const uint8_t *w, int64_t index) {
     return t - u;
 }
 
+/*
+ * J/tensor/standard/Q6_KFloatTensor.java:66-122.  A super-block is ql[128] | qh[64] | 16 signed
+ * scales | fp16 d; two halves of 128 elements, four groups of 32 in each: the group picks the ql
+ * plane (0 / 32), the nibble (low for groups 0-1, high for 2-3) and the bit pair of qh;
+ * w = d * scale * (q - 32), left to right in fp32.
+ */
+static inline float q6_k_get(const uint8_t *w, int64_t index) {
+    int64_t block_index = index / QK_K;
+    int within = (int)(index % QK_K);
+    const uint8_t *blk = w + block_index * Q6_K_BYTES;
+    float d = jo_f16_to_f32(read_u16(blk + 208));
+    int half_index = within / 128;
+    int pos_in_half = within % 128;
+    int group = pos_in_half / 32;
+    int pos = pos_in_half % 32;
+    const uint8_t *ql = blk + half_index * 64;
+    const uint8_t *qh = blk + 128 + half_index * 32;
+    const int8_t *sc = (const int8_t *)(blk + 192 + half_index * 8);
+    int is = pos / 16;
+    int q;
+    switch (group) {
+        case 0: q = ((ql[pos] & 0xF) | (((qh[pos] >> 0) & 3) << 4)) - 32; break;
+        case 1: q = ((ql[32 + pos] & 0xF) | (((qh[pos] >> 2) & 3) << 4)) - 32; break;
+        case 2: q = ((ql[pos] >> 4) | (((qh[pos] >> 4) & 3) << 4)) - 32; break;
+        default: q = ((ql[32 + pos] >> 4) | (((qh[pos] >> 6) & 3) << 4)) - 32; break;
+    }
+    float t = d * (float)sc[is + 2 * group];
+    return t * (float)q;
+}
+
 float jo_get_float(int type, const uint8_t *w, int64_t index) {
     switch (type) {
         case JO_Q8_0: return q8_0_get(w, index);
         case JO_Q4_0: return q4_0_get(w, index);
         case JO_Q4_K: return q4_k_get(w, index);
+        case JO_Q6_K: return q6_k_get(w, index);
         default: return NAN;
     }
 }
@@ -236,6 +270,28 @@ float jo_get_float_alt(int type, const uint8_t *w, int64_t index) {
         float b = dmin * (float)m;
         return a - b;
     }
+    if (type == JO_Q6_K) {
+        /* J/backend/tornado/kernels/TransformerComputeKernelsQ6_K.java:195-232 */
+        const uint8_t *blk = w + (index / 256) * Q6_K_BYTES;
+        int within = (int)(index % 256);
+        float d = jo_f16_to_f32(read_u16(blk + 208));
+        int half_index = within / 128;
+        int pos_in_half = within - half_index * 128;
+        int group = pos_in_half / 32;
+        int pos = pos_in_half - group * 32;
+        int ql_base = half_index * 64, qh_base = 128 + half_index * 32, sc_base = 192 + half_index * 8;
+        int is = pos / 16;
+        int qh = blk[qh_base + pos] & 0xFF;
+        int second_plane = group & 1, high_nibble = group >> 1;
+        int ql = blk[ql_base + second_plane * 32 + pos] & 0xFF;
+        int low_bits = high_nibble ? ((ql >> 4) & 0xF) : (ql & 0xF);
+        int high_pair = (qh >> (2 * group)) & 3;
+        int q = (low_bits | (high_pair << 4)) - 32;
+        int scale = blk[sc_base + is + group * 2] & 0xFF;
+        if (scale > 127) scale -= 256;
+        float a = d * (float)scale;
+        return a * (float)q;
+    }
     return NAN;
 }
 
@@ -261,6 +317,12 @@ static float scalar_dot(int type, const uint8_t *w, int64_t this_offset, const f
         case JO_Q4_K:
             for (int64_t j = 0; j < size; j++) {
                 float p = q4_k_get(w, this_offset + j) * x[that_offset + j];
+                result += p;
+            }
+            break;
+        case JO_Q6_K:   /* Q6_KFloatTensor.dot :124-127 is scalarDot */
+            for (int64_t j = 0; j < size; j++) {
+                float p = q6_k_get(w, this_offset + j) * x[that_offset + j];
                 result += p;
             }
             break;
@@ -393,7 +455,7 @@ static float vector_dot(int type, int bits, const uint8_t *w, int64_t this_offse
  */
 float jo_dot(int type, int flavour, const uint8_t *w, int64_t this_offset, const float *x,
              int64_t that_offset, int64_t size) {
-    if (type != JO_Q4_K && (flavour == JO_DOT_VEC128 || flavour == JO_DOT_VEC256)) {
+    if (type != JO_Q4_K && type != JO_Q6_K && (flavour == JO_DOT_VEC128 || flavour == JO_DOT_VEC256)) {
         return vector_dot(type, flavour, w, this_offset, x, that_offset, size);
     }
     return scalar_dot(type, w, this_offset, x, that_offset, size);

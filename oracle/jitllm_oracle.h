@@ -18,13 +18,13 @@ extern "C" {
 #endif
 
 /* ggml type ids, the numbering GGUF files carry (J/format/GGMLType.java:7,13,18 by ordinal). */
-enum { JO_Q4_0 = 2, JO_Q8_0 = 8, JO_Q4_K = 12 };
+enum { JO_Q4_0 = 2, JO_Q8_0 = 8, JO_Q4_K = 12, JO_Q6_K = 14 };
 
 /* dot flavours: which branch of Q8_0FloatTensor.dot / Q4_0FloatTensor.dot runs. */
 enum { JO_DOT_SCALAR = 0, JO_DOT_VEC128 = 128, JO_DOT_VEC256 = 256 };
 
-int jo_block_elems(int type);  /* 32 / 32 / 256 */
-int jo_block_bytes(int type);  /* 18 / 34 / 144 */
+int jo_block_elems(int type);  /* 32 / 32 / 256 / 256 */
+int jo_block_bytes(int type);  /* 18 / 34 / 144 / 210 */
 
 float    jo_f16_to_f32(uint16_t bits);
 uint16_t jo_f32_to_f16(float value);

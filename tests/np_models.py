@@ -65,7 +65,29 @@ def dequant_q4_k(raw: np.ndarray) -> np.ndarray:
     return out.reshape(-1)
 
 
-DEQUANT = {8: dequant_q8_0, 2: dequant_q4_0, 12: dequant_q4_k}
+def dequant_q6_k(raw: np.ndarray) -> np.ndarray:
+    """ggml's dequantize_row_q6_K, vectorised: per half of 128, y[l + 32 g] for l < 32 takes its low
+    four bits from ql (plane g % 2, nibble g // 2), bits 4-5 from qh >> 2 g, the scale
+    sc[l // 16 + 2 g]; w = d * sc * (q - 32) with every product rounded to fp32."""
+    b = raw.reshape(-1, 210)
+    nb = b.shape[0]
+    ql = b[:, 0:128].reshape(nb, 2, 2, 32).astype(np.int32)       # [block, half, plane, l]
+    qh = b[:, 128:192].reshape(nb, 2, 32).astype(np.int32)        # [block, half, l]
+    sc = b[:, 192:208].copy().view(np.int8).reshape(nb, 2, 8).astype(np.float32)
+    d = half_bits_to_f32(b[:, 208:210].copy().view(np.uint16)[:, 0])
+    out = np.empty((nb, 2, 4, 32), dtype=np.float32)
+    l16 = np.arange(32) // 16
+    with np.errstate(invalid="ignore", over="ignore"):
+        for g in range(4):
+            low = (ql[:, :, g % 2, :] >> (4 * (g // 2))) & 0xF
+            q = (low | (((qh >> (2 * g)) & 3) << 4)) - 32
+            scale = sc[:, :, l16 + 2 * g]                          # [block, half, l]
+            t = (d[:, None, None] * scale).astype(np.float32)
+            out[:, :, g, :] = (t * q.astype(np.float32)).astype(np.float32)
+    return out.reshape(-1)
+
+
+DEQUANT = {8: dequant_q8_0, 2: dequant_q4_0, 12: dequant_q4_k, 14: dequant_q6_k}
 
 
 def scalar_dot_rows(w_deq: np.ndarray, x: np.ndarray) -> np.ndarray:

@@ -180,6 +180,63 @@ def test_fused_gate_up(ctx, t, d, n):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + 1e-6)
 
 
+# ---- Q6_K: decode and the single-token projection ---------------------------------------------
+
+def test_q6_k_decode_bit_exact(ctx):
+    """Arbitrary bytes, special fp16 scales and a synthetic weight: the device decode equals
+    Q6_KFloatTensor.getFloat bit for bit."""
+    from jitllm_amd import synthetic
+    say("q6_K decode")
+    for raw, rows in ((FX.random_bytes(20260914, 12 * 210), 12),
+                      (FX.adversarial_blocks(O.Q6_K, 24, 20260908 + O.java_string_hash("Q6_K")), 24),
+                      (synthetic.weight(O.Q6_K, 40, 512, seed=701), 80)):
+        w = upload(ctx, O.Q6_K, raw, rows, raw.size // 210 // rows * 256)
+        assert bits_equal(w.dequantize(), O.dequant(O.Q6_K, raw))
+
+
+@pytest.mark.parametrize("d,n", [(2048, 2048), (32000, 2048), (2048, 8192), (37, 512), (1000, 256), (4, 4096)])
+def test_q6_k_gemv_matches_oracle(ctx, d, n):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("q6_K gemv", d, n)
+    raw = synthetic.weight(O.Q6_K, d, n, seed=710 + d % 97)
+    x = synthetic.activations(n, seed=720)
+    ref = O.matmul(O.Q6_K, raw, x, d, n)
+    mag = magnitude(O.Q6_K, raw, x, d, n)
+    w = upload(ctx, O.Q6_K, raw, d, n)
+    out = ctx.float_array(d, fill=POISON)
+    acc = ctx.from_numpy(np.full(d, 0.75, dtype=np.float32))
+    proj = QuantizedProjections(ctx, TornadoWorkspace(wrapX=acc))
+    dx = ctx.from_numpy(x)
+    proj.floatMatvec(dx, out, w, n, d)
+    proj.residualMatvec(dx, w, n, d)
+    ctx.sync()
+    assert rel_err(out.get(), ref, mag) < 2e-5
+    assert rel_err(acc.get(), ref.astype(np.float64) + 0.75, mag + 0.75 * 6e-8) < 2e-5
+
+
+def test_q6_k_has_no_fused_or_batched_kernels(ctx):
+    """What has no kernel is refused by name (QuantizedProjections.java:386-393 keeps Q6_K out of
+    the fused gate/up as well)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd._lib import UnsupportedProjection
+    from jitllm_amd.projections import QuantizedBatchProjections, QuantizedProjections, TornadoWorkspace
+    say("q6_K unsupported")
+    d, n = 16, 256
+    w = upload(ctx, O.Q6_K, synthetic.weight(O.Q6_K, d, n, seed=731), d, n)
+    x = ctx.from_numpy(synthetic.activations(n, seed=732))
+    out = ctx.float_array(d, fill=POISON)
+    proj = QuantizedProjections(ctx, TornadoWorkspace(wrapXb=x, wrapHb=out, wrapHb2=ctx.float_array(d)))
+    with pytest.raises(UnsupportedProjection, match="Q6_K"):
+        proj.fusedQKV(x, out, out, out, w, w, w)
+    assert not proj.fusedGateUp(w, w)
+    with pytest.raises(UnsupportedProjection, match="Q6_K"):
+        proj.rmsMatvec(x, x, None, out, w, n, d, eps=1e-5)
+    X = ctx.from_numpy(synthetic.activations((4, n), seed=733))
+    with pytest.raises(UnsupportedProjection, match="Q6_K"):
+        QuantizedBatchProjections(ctx, 4, n, d).projection(X, ctx.float_array(4 * d), w, n, d, False)
+
+
 # ---- RMS normalisation folded into the projections, argmax -----------------------------------
 
 @pytest.mark.parametrize("n", [512, 2048, 4096, 8192, 16384, 1000])
@@ -353,8 +410,8 @@ def test_errors_name_the_cause(ctx):
     lib = L.load()
     h = C.c_void_p()
     raw = np.zeros(64, dtype=np.uint8)
-    st = lib.jl_weight_upload(ctx.handle, 14, raw.ctypes.data, 1, 32, C.byref(h))  # Q6_K: no kernel
-    assert st == L.JL_ERR_UNSUPPORTED and b"ggml type 14" in lib.jl_last_error()
+    st = lib.jl_weight_upload(ctx.handle, 13, raw.ctypes.data, 1, 32, C.byref(h))  # Q5_K: no kernel
+    assert st == L.JL_ERR_UNSUPPORTED and b"ggml type 13" in lib.jl_last_error()
     st = lib.jl_weight_upload(ctx.handle, O.Q8_0, raw.ctypes.data, 1, 48, C.byref(h))
     assert st == L.JL_ERR_INVALID and b"whole number" in lib.jl_last_error()
     w8 = upload(ctx, O.Q8_0, synthetic.weight(O.Q8_0, 64, 256, 1), 64, 256)

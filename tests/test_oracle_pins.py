@@ -163,6 +163,79 @@ def test_q4_k_scale_unpacking_round_trip():
             assert np.all(out[:, other, :] == 0.0)
 
 
+# ---- Q6_K -----------------------------------------------------------------------------------
+
+def test_q6_k_decode_three_ways():
+    """Host wording (Q6_KFloatTensor.java:66-122) == device wording
+    (TransformerComputeKernelsQ6_K.java:195-232) == an independent numpy statement of ggml's
+    dequantize_row_q6_K, on arbitrary bytes and on blocks with special fp16 scales."""
+    raw = FX.random_bytes(20260914, 12 * 210)
+    main = O.dequant(O.Q6_K, raw)
+    assert_bit_equal(main, O.dequant_alt(O.Q6_K, raw))
+    assert_bit_equal(main, NP.DEQUANT[O.Q6_K](raw))
+    adv = FX.adversarial_blocks(O.Q6_K, 24, 20260908 + O.java_string_hash("Q6_K"))
+    main = O.dequant(O.Q6_K, adv)
+    assert_bit_equal(main, O.dequant_alt(O.Q6_K, adv))
+    assert_bit_equal(main, NP.DEQUANT[O.Q6_K](adv))
+
+
+def test_q6_k_layout_known_answers():
+    """Where each bit of a super-block lands, written out from the format's description rather
+    than from any decoder: byte p of ql plane 0 / 1 of half h holds element 128 h + p (+ 32) in
+    its low nibble and 128 h + 64 + p (+ 32) in its high nibble; qh byte p of half h holds bits
+    4-5 of elements 128 h + p + 32 g in bit pair g; scale byte 8 h + 2 g + p // 16 applies."""
+    def block(d_bits=0x3C00):               # d = 1.0, all scales 1, every q = 0 -> w = -32
+        b = np.zeros(210, dtype=np.uint8)
+        b[192:208] = 1
+        b[208], b[209] = d_bits & 0xFF, d_bits >> 8
+        return b
+    base = O.dequant(O.Q6_K, block())
+    assert np.all(base == -32.0)
+    cases = []
+    for h in (0, 1):
+        for p in (0, 5, 17, 31):
+            cases += [(64 * h + p, 0x07, 128 * h + p, 7), (64 * h + p, 0x70, 128 * h + 64 + p, 7),
+                      (64 * h + 32 + p, 0x0B, 128 * h + 32 + p, 11), (64 * h + 32 + p, 0xB0, 128 * h + 96 + p, 11)]
+            for g in range(4):
+                cases.append((128 + 32 * h + p, 2 << (2 * g), 128 * h + 32 * g + p, 32))
+    for byte, value, element, q in cases:
+        b = block()
+        b[byte] = value
+        out = O.dequant(O.Q6_K, b)
+        want = base.copy()
+        want[element] = q - 32
+        assert np.array_equal(out, want), (byte, value, element)
+    # scales: signed bytes, one per 16 elements in the order half, group, l // 16
+    b = block()
+    b[192:208] = np.arange(-8, 8, dtype=np.int8).view(np.uint8)
+    out = O.dequant(O.Q6_K, b).reshape(2, 4, 2, 16)
+    for h in range(2):
+        for g in range(4):
+            for half16 in range(2):
+                sc = -8 + 8 * h + 2 * g + half16
+                assert np.all(out[h, g, half16] == np.float32(sc) * np.float32(-32))
+    # d is applied first: (d * sc) rounded, then times q
+    b = block(0x3555)                                     # d = 0.33325195
+    b[192:208] = 3
+    b[0] = 0x0F                                           # element 0: q = 15
+    d = NP.half_bits_to_f32(np.array([0x3555], dtype=np.uint16))[0]
+    want = np.float32(np.float32(d * np.float32(3)) * np.float32(15 - 32))
+    assert O.dequant(O.Q6_K, b)[0] == want
+
+
+def test_q6_k_scalar_dot_and_matmul():
+    """Q6_KFloatTensor.dot is scalarDot (:124-127): a strictly sequential fp32 sum of decoded
+    weight times x, whatever flavour is asked for; rows are independent."""
+    from jitllm_amd import synthetic
+    d, n = 5, 512
+    raw = synthetic.weight(O.Q6_K, d, n, seed=77)
+    x = synthetic.activations(n, seed=78)
+    w = NP.DEQUANT[O.Q6_K](raw).reshape(d, n)
+    want = NP.scalar_dot_rows(w, x)
+    for flavour in (O.DOT_SCALAR, O.DOT_VEC256):
+        assert_bit_equal(O.matmul(O.Q6_K, raw, x, d, n, flavour=flavour), want)
+
+
 # ---- dot products -------------------------------------------------------------------------
 
 @pytest.mark.parametrize("t,name", [(O.Q4_0, "q4_0"), (O.Q4_K, "q4_K"), (O.Q8_0, "q8_0")])
