@@ -46,8 +46,10 @@ typedef enum jl_status {
 /* ggml type ids as a GGUF tensor-info record carries them (GGMLType ordinals). */
 /* Q8_0, Q4_0 and Q4_K have every entry point below.  Q6_K (210 B / 256, J/format/GGMLType.java:27-29:
  * the vocabulary projection and some attention / feed-forward tensors of "Q4_K_M" files) has
- * jl_dequant_f32 and jl_gemv; the fused and batched entry points return JL_ERR_UNSUPPORTED for it,
- * as the reference's own fused kernels do not take it either (QuantizedProjections.java:386-393). */
+ * jl_dequant_f32, jl_gemv and jl_gemm -- the latter always by decoding the weights to fp16 into the
+ * workspace first, whatever the row count -- while the fused single-token entry points return
+ * JL_ERR_UNSUPPORTED for it, as the reference's own fused kernels do not take it either
+ * (QuantizedProjections.java:386-393). */
 typedef enum jl_ggml_type { JL_Q4_0 = 2, JL_Q8_0 = 8, JL_Q4_K = 12, JL_Q6_K = 14 } jl_ggml_type;
 
 /* What a projection does with its result (Int8GemmKernels.java:617-621 EPILOGUE_*). */

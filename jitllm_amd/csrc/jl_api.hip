@@ -348,10 +348,6 @@ int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const f
     JL_REQUIRE(col_offset >= 0 && ldo >= col_offset + total,
                "jl_gemm: ldo %lld < col_offset %lld + %lld output columns", (long long)ldo,
                (long long)col_offset, (long long)total);
-    if (!jl_has_fused_kernels(weights[0]->type)) {
-        return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no batched kernel for a %s weight",
-                       jl_type_name(weights[0]->type));
-    }
     if (math == JL_MATH_DEFAULT) math = JL_MATH_F16;
     JL_REQUIRE(math == JL_MATH_F16 || math == JL_MATH_INT8, "jl_gemm: math %d", math);
     if (math == JL_MATH_INT8 && weights[0]->type == JL_Q4_K) {

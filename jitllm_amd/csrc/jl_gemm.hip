@@ -823,7 +823,9 @@ size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_
         size_t padded = round_up((size_t)max_rows, 128);
         return round_up(padded * (size_t)cols, 256) + round_up(padded * (size_t)(cols / 32) * 4, 256);
     }
-    size_t planes = round_up(round_up((size_t)out_cols, 128) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
+    // (256: the fp16 copy of a call's weights, which calls of a type without a decode-in-the-loop
+    // kernel always make, is padded to whole 256-row column tiles)
+    size_t planes = round_up(round_up((size_t)out_cols, 256) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
     // calls of 512 rows or more may decode the weights to fp16 once, into the same region
     // (and, for narrow projections with long rows, two planes of partial sums; such calls have
     // fewer 256 x 128 tiles than 0.7 x 256 compute units)
@@ -920,7 +922,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const size_t plane_bytes = workspace_bytes > head ? workspace_bytes - head : 0;
 
 
-    if (rows <= 32) {
+    if (rows <= 32 && jl_has_fused_kernels(type)) {
         // batched decode of up to 32 rows: the weight-streaming kernel reads X itself
         bool taken = false;
         int st = jl_launch_gemm_skinny(ctx, weights, count, X, C, rows, ldo, col_offset, epilogue, planes,
@@ -932,11 +934,22 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     int virt = 0;
     for (int i = 0; i < count; i++) virt += (int)weights[i]->rows;
     int dsplits = 1;
-    const int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits);
+    int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits);
+    // A type without a decode-in-the-loop kernel (Q6_K) takes the decode-once path whatever the
+    // shape: correct for any row count, tuned for none but prefill.
+    const bool dense_only = !jl_has_fused_kernels(type);
+    if (dense_only && bn == 0) {
+        bn = 128;
+        dsplits = 1;
+    }
     const size_t copy_bytes = round_up(jl_dense_copy_bytes(k, virt), 256);
     const bool dense = bn != 0 && copy_bytes + (dsplits > 1 ? jl_dense_plane_bytes(rows, virt) : 0) <= plane_bytes;
     const int padded_rows = dense ? (int)round_up((size_t)rows, 256) : padded;
 
+    if (dense_only && !dense) {
+        return jl_fail(JL_ERR_WORKSPACE, "jl_gemm: a %s weight needs room for its fp16 copy (%zu bytes) in the workspace",
+                       jl_type_name(type), copy_bytes);
+    }
     hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded_rows), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
     JL_HIP(hipGetLastError());
     if (dense) {

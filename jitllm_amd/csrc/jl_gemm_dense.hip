@@ -115,6 +115,26 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
         const int shift = (c & 2) * 2;
         const h2 bias = {(_Float16)1032.f, (_Float16)1032.f}, d2 = {d, d};
         *dst = pack8_scaled((q.lo >> shift) & 0x0F0F0F0Fu, (q.hi >> shift) & 0x0F0F0F0Fu, bias, d2);
+    } else if constexpr (TYPE == JL_Q6_K) {
+        // chunk c % 32 of super-block c / 32 (ql[128] | qh[64] | 16 signed scales | d): half h,
+        // group g, positions pos .. pos + 7 of the group; the value is the host decode
+        // (d * scale) * (q - 32) in fp32 (Q6_KFloatTensor.java:66-122), rounded once to fp16
+        const uint8_t *sb = row + (int64_t)(c >> 5) * 210;
+        const int e0 = (c & 31) * 8, h = e0 >> 7, g = (e0 >> 5) & 3, pos = e0 & 31;
+        const Quants8 ql = *(const Quants8 *)(sb + 64 * h + 32 * (g & 1) + pos);
+        const Quants8 qh = *(const Quants8 *)(sb + 128 + 32 * h + pos);
+        const float ds = __fmul_rn(jl_half_bits_to_float(*(const unsigned short *)(sb + 208)),
+                                   (float)(int)(int8_t)sb[192 + 8 * h + (pos >> 4) + 2 * g]);
+        const int nib = (g >> 1) * 4;
+        const uint32_t q0 = ((ql.lo >> nib) & 0x0F0F0F0Fu) | (((qh.lo >> (2 * g)) & 0x03030303u) << 4);
+        const uint32_t q1 = ((ql.hi >> nib) & 0x0F0F0F0Fu) | (((qh.hi >> (2 * g)) & 0x03030303u) << 4);
+        _Float16 v[8];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            v[e] = (_Float16)__fmul_rn(ds, (float)((int)((q0 >> (8 * e)) & 0xFF) - 32));
+            v[4 + e] = (_Float16)__fmul_rn(ds, (float)((int)((q1 >> (8 * e)) & 0xFF) - 32));
+        }
+        *dst = *(const uint4 *)v;
     } else {
         // sub-block c / 4 of super-block c / 32: low nibbles are the even sub-block of a pair of
         // 32 bytes, high nibbles the odd one
@@ -501,6 +521,7 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
         case JL_Q8_0: dst = launch_decode<JL_Q8_0>(ctx, d, ntiles * bn); break;
         case JL_Q4_0: dst = launch_decode<JL_Q4_0>(ctx, d, ntiles * bn); break;
         case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, d, ntiles * bn); break;
+        case JL_Q6_K: dst = launch_decode<JL_Q6_K>(ctx, d, ntiles * bn); break;
         default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
     }
     if (dst != JL_OK) return dst;

@@ -260,6 +260,55 @@ def test_two_pass_prefill_qkv_and_gate_up(ctx):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
 
 
+@pytest.mark.parametrize("d,n,T,residual", [(300, 512, 8, False), (1000, 2048, 100, True), (4096, 256, 600, False)])
+def test_q6_k_batched_rows_take_the_decode_once_path(ctx, d, n, T, residual):
+    """A Q6_K weight has no decode-in-the-loop kernel: every batched call decodes it to fp16 into
+    the workspace and runs the fp16 GEMM, few rows or many; partial batches leave the rest alone."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("q6_K batched", d, n, T, residual)
+    raw = synthetic.weight(O.Q6_K, d, n, seed=9300 + d)
+    X = synthetic.activations((T, n), seed=9400 + T)
+    active = T - 3
+    ref = O.matmul_batch(O.Q6_K, raw, X, d, n)
+    out = ctx.float_array(T * d, fill=UNTOUCHED)
+    proj = QuantizedBatchProjections(ctx, T, n, d)
+    proj.projection(ctx.from_numpy(X), out, ctx.load_weight(O.Q6_K, raw, d, n), n, d, residual, activeRows=active)
+    ctx.sync()
+    got = out.get().reshape(T, d)
+    assert np.all(got[active:] == UNTOUCHED)
+    want = ref.astype(np.float64) + (float(UNTOUCHED) if residual else 0.0)
+    slack = abs(np.spacing(np.float32(UNTOUCHED))) / 2 if residual else 0.0
+    excess = np.abs(got[:active].astype(np.float64) - want[:active]) - slack
+    assert np.all(excess <= 5e-4 * magnitude(O.Q6_K, raw, X, d, n)[:active]), float(excess.max())
+
+
+def test_q6_k_batched_gate_up(ctx):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("q6_K batched gate_up")
+    t, d, n, T = O.Q6_K, 200, 512, 40
+    r1 = synthetic.weight(t, d, n, seed=9501)
+    r3 = synthetic.weight(t, d, n, seed=9502)
+    X = synthetic.activations((T, n), seed=9503)
+    g = O.matmul_batch(t, r1, X, d, n)
+    u = O.matmul_batch(t, r3, X, d, n)
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(T, d)
+    hb = ctx.float_array(T * d, fill=UNTOUCHED)
+    # (the host mirror keeps the reference's rule that gate/up is fused for Q8_0 / Q4_0 / Q4_K
+    # pairs only; the library's jl_gemm takes the Q6_K pair, so it is called directly)
+    from jitllm_amd import _lib as L
+    proj = QuantizedBatchProjections(ctx, T, n, 2 * d)
+    assert not proj.fusedGateUp(ctx.load_weight(t, r1, d, n), ctx.load_weight(t, r3, d, n))
+    proj._gemm([ctx.load_weight(t, r1, d, n), ctx.load_weight(t, r3, d, n)], ctx.from_numpy(X), hb, T, d, 0,
+               L.JL_SWIGLU)
+    ctx.sync()
+    got = hb.get().reshape(T, d)
+    mg, mu = magnitude(t, r1, X, d, n), magnitude(t, r3, X, d, n)
+    bound = 5e-4 * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
+
+
 def test_huge_activation_rows_stay_finite(ctx):
     """Rows far outside fp16's range are rescaled by a power of two, not turned into infinities."""
     from jitllm_amd import synthetic

@@ -215,12 +215,12 @@ def test_q6_k_gemv_matches_oracle(ctx, d, n):
     assert rel_err(acc.get(), ref.astype(np.float64) + 0.75, mag + 0.75 * 6e-8) < 2e-5
 
 
-def test_q6_k_has_no_fused_or_batched_kernels(ctx):
+def test_q6_k_has_no_fused_single_token_kernels(ctx):
     """What has no kernel is refused by name (QuantizedProjections.java:386-393 keeps Q6_K out of
     the fused gate/up as well)."""
     from jitllm_amd import synthetic
     from jitllm_amd._lib import UnsupportedProjection
-    from jitllm_amd.projections import QuantizedBatchProjections, QuantizedProjections, TornadoWorkspace
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
     say("q6_K unsupported")
     d, n = 16, 256
     w = upload(ctx, O.Q6_K, synthetic.weight(O.Q6_K, d, n, seed=731), d, n)
@@ -232,9 +232,6 @@ def test_q6_k_has_no_fused_or_batched_kernels(ctx):
     assert not proj.fusedGateUp(w, w)
     with pytest.raises(UnsupportedProjection, match="Q6_K"):
         proj.rmsMatvec(x, x, None, out, w, n, d, eps=1e-5)
-    X = ctx.from_numpy(synthetic.activations((4, n), seed=733))
-    with pytest.raises(UnsupportedProjection, match="Q6_K"):
-        QuantizedBatchProjections(ctx, 4, n, d).projection(X, ctx.float_array(4 * d), w, n, d, False)
 
 
 # ---- RMS normalisation folded into the projections, argmax -----------------------------------
