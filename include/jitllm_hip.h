@@ -44,13 +44,14 @@ typedef enum jl_status {
 } jl_status;
 
 /* ggml type ids as a GGUF tensor-info record carries them (GGMLType ordinals). */
-/* Q8_0, Q4_0 and Q4_K have every entry point below.  Q6_K (210 B / 256, J/format/GGMLType.java:27-29:
- * the vocabulary projection and some attention / feed-forward tensors of "Q4_K_M" files) has
+/* Q8_0, Q4_0 and Q4_K have every entry point below.  Q6_K (210 B / 256) and Q5_K (176 B / 256;
+ * J/format/GGMLType.java:21-29: the vocabulary projection and some attention / feed-forward tensors
+ * of "Q4_K_M" files are Q6_K, "Q5_K_M" files are Q5_K with Q6_K) have
  * jl_dequant_f32, jl_gemv and jl_gemm -- the latter always by decoding the weights to fp16 into the
  * workspace first, whatever the row count -- while the fused single-token entry points return
- * JL_ERR_UNSUPPORTED for it, as the reference's own fused kernels do not take it either
- * (QuantizedProjections.java:386-393). */
-typedef enum jl_ggml_type { JL_Q4_0 = 2, JL_Q8_0 = 8, JL_Q4_K = 12, JL_Q6_K = 14 } jl_ggml_type;
+ * JL_ERR_UNSUPPORTED for them (the reference fuses gate/up for Q5_K but not Q6_K,
+ * QuantizedProjections.java:386-393; a caller that gets JL_ERR_UNSUPPORTED runs the unfused steps). */
+typedef enum jl_ggml_type { JL_Q4_0 = 2, JL_Q8_0 = 8, JL_Q4_K = 12, JL_Q5_K = 13, JL_Q6_K = 14 } jl_ggml_type;
 
 /* What a projection does with its result (Int8GemmKernels.java:617-621 EPILOGUE_*). */
 typedef enum jl_epilogue {
@@ -266,7 +267,7 @@ int jl_gguf_metadata_string(const jl_gguf *g, const char *key, const char **valu
 int jl_gguf_metadata_array(const jl_gguf *g, const char *key, int *element_type, int64_t *count);
 
 /*
- * jl_weight_upload of a two-dimensional Q8_0 / Q4_0 / Q4_K / Q6_K tensor straight from the mapped file
+ * jl_weight_upload of a two-dimensional Q8_0 / Q4_0 / Q4_K / Q5_K / Q6_K tensor straight from the mapped file
  * (ModelLoader.loadTornadoTensorNative, J/model/loader/ModelLoader.java:246-290, without the
  * 16-byte array header the reference's segments carry, GGUF.java:214-268).  Another type is
  * JL_ERR_UNSUPPORTED naming it; a tensor that runs past the end of the file is refused (:236-247).

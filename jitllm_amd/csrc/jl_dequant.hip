@@ -86,7 +86,8 @@ int jl_launch_dequant(jl_context *ctx, const jl_weight *w, float *out) {
                                total);
             break;
         case JL_Q6_K:
-            return jl_launch_dequant_q6k(ctx, w, out);
+        case JL_Q5_K:
+            return jl_launch_dequant_direct(ctx, w, out);
         default:
             return jl_fail(JL_ERR_UNSUPPORTED, "jl_dequant_f32: no decode kernel for ggml type %d",
                            w->type);

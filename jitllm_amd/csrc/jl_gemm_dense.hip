@@ -115,6 +115,29 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
         const int shift = (c & 2) * 2;
         const h2 bias = {(_Float16)1032.f, (_Float16)1032.f}, d2 = {d, d};
         *dst = pack8_scaled((q.lo >> shift) & 0x0F0F0F0Fu, (q.hi >> shift) & 0x0F0F0F0Fu, bias, d2);
+    } else if constexpr (TYPE == JL_Q5_K) {
+        // chunk c % 32 of super-block c / 32 (d, dmin | 12 scale bytes | qh[32] | qs[128]): sub-block
+        // sub, positions pos .. pos + 7; the value is the host decode ((d * sc) * q) - (dmin * m) in
+        // fp32 (Q5_KFloatTensor.java:78-122), rounded once to fp16
+        const uint8_t *sb = row + (int64_t)(c >> 5) * 176;
+        const int sub = (c >> 2) & 7, pos = (c & 3) * 8;
+        const uint4 h = *(const uint4 *)sb;
+        const uint2 qs = *(const uint2 *)(sb + 48 + (sub >> 1) * 32 + pos);
+        const uint2 qh = *(const uint2 *)(sb + 16 + pos);
+        int sc, mn;
+        jl_q4k_scale_min(h.y, h.z, h.w, sub, sc, mn);
+        const float ds = __fmul_rn(jl_half_bits_to_float(h.x), (float)sc);
+        const float dm = __fmul_rn(jl_half_bits_to_float(h.x >> 16), (float)mn);
+        const int nib = (sub & 1) * 4;
+        const uint32_t q0 = ((qs.x >> nib) & 0x0F0F0F0Fu) | (((qh.x >> sub) & 0x01010101u) << 4);
+        const uint32_t q1 = ((qs.y >> nib) & 0x0F0F0F0Fu) | (((qh.y >> sub) & 0x01010101u) << 4);
+        _Float16 v[8];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            v[e] = (_Float16)__fsub_rn(__fmul_rn(ds, (float)((q0 >> (8 * e)) & 0xFF)), dm);
+            v[4 + e] = (_Float16)__fsub_rn(__fmul_rn(ds, (float)((q1 >> (8 * e)) & 0xFF)), dm);
+        }
+        *dst = *(const uint4 *)v;
     } else if constexpr (TYPE == JL_Q6_K) {
         // chunk c % 32 of super-block c / 32 (ql[128] | qh[64] | 16 signed scales | d): half h,
         // group g, positions pos .. pos + 7 of the group; the value is the host decode
@@ -521,6 +544,7 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
         case JL_Q8_0: dst = launch_decode<JL_Q8_0>(ctx, d, ntiles * bn); break;
         case JL_Q4_0: dst = launch_decode<JL_Q4_0>(ctx, d, ntiles * bn); break;
         case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, d, ntiles * bn); break;
+        case JL_Q5_K: dst = launch_decode<JL_Q5_K>(ctx, d, ntiles * bn); break;
         case JL_Q6_K: dst = launch_decode<JL_Q6_K>(ctx, d, ntiles * bn); break;
         default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
     }

@@ -681,12 +681,12 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     const int type = w[0]->type;
     const int n = (int)w[0]->cols;
     const int row_bytes = n / jl_block_elems(type) * jl_block_bytes(type);
-    if (type == JL_Q6_K) {
+    if (!jl_has_fused_kernels(type)) {
         if (nseg != 1 || w_up || rms) {
-            return jl_fail(JL_ERR_UNSUPPORTED, "no fused single-token kernel for a Q6_K weight "
-                                               "(plain and residual projections only)");
+            return jl_fail(JL_ERR_UNSUPPORTED, "no fused single-token kernel for a %s weight "
+                                               "(plain and residual projections only)", jl_type_name(type));
         }
-        return jl_launch_gemv_q6k(ctx, w[0], x, outs[0], epilogue);
+        return jl_launch_gemv_direct(ctx, w[0], x, outs[0], epilogue);
     }
 
     const bool dual = w_up != nullptr;

@@ -30,15 +30,16 @@ struct jl_weight {
 
 // Block geometry (reference: J/format/GGMLType.java:7,13,18-20).
 static inline int jl_block_elems(int type) {
-    return (type == JL_Q4_K || type == JL_Q6_K) ? 256 : (type == JL_Q8_0 || type == JL_Q4_0) ? 32 : 0;
+    return (type == JL_Q4_K || type == JL_Q6_K || type == JL_Q5_K) ? 256 : (type == JL_Q8_0 || type == JL_Q4_0) ? 32 : 0;
 }
 static inline int jl_block_bytes(int type) {
-    return type == JL_Q4_K ? 144 : type == JL_Q6_K ? 210 : type == JL_Q8_0 ? 34 : type == JL_Q4_0 ? 18 : 0;
+    return type == JL_Q4_K ? 144 : type == JL_Q6_K ? 210 : type == JL_Q5_K ? 176 : type == JL_Q8_0 ? 34 : type == JL_Q4_0 ? 18 : 0;
 }
 static inline const char *jl_type_name(int type) {
-    return type == JL_Q4_K ? "Q4_K" : type == JL_Q6_K ? "Q6_K" : type == JL_Q8_0 ? "Q8_0" : type == JL_Q4_0 ? "Q4_0" : "?";
+    return type == JL_Q4_K ? "Q4_K" : type == JL_Q6_K ? "Q6_K" : type == JL_Q5_K ? "Q5_K" : type == JL_Q8_0 ? "Q8_0" : type == JL_Q4_0 ? "Q4_0" : "?";
 }
-// Q8_0, Q4_0 and Q4_K have the whole kernel family; Q6_K the single-token projection only.
+// Q8_0, Q4_0 and Q4_K have the whole kernel family; Q6_K and Q5_K the plain single-token
+// projection and the decode-once batched path.
 static inline bool jl_has_fused_kernels(int type) {
     return type == JL_Q8_0 || type == JL_Q4_0 || type == JL_Q4_K;
 }
@@ -70,8 +71,8 @@ struct jl_rms {
 };
 int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *const *outs,
                    const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms);
-int jl_launch_gemv_q6k(jl_context *ctx, const jl_weight *w, const float *x, float *out, int epilogue);
-int jl_launch_dequant_q6k(jl_context *ctx, const jl_weight *w, float *out);
+int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const float *x, float *out, int epilogue);
+int jl_launch_dequant_direct(jl_context *ctx, const jl_weight *w, float *out);
 int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale);
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
 int jl_launch_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);

@@ -14,7 +14,8 @@ class GGMLType(enum.IntEnum):
     Q4_0 = 2
     Q8_0 = 8
     Q4_K = 12
-    Q6_K = 14   # single-token projection and decode only
+    Q5_K = 13   # plain single-token projection and the decode-once batched path
+    Q6_K = 14   # likewise
 
     @property
     def block_elems(self) -> int:
@@ -39,5 +40,6 @@ _GEOMETRY = {
     GGMLType.Q4_0: (32, 18),
     GGMLType.Q8_0: (32, 34),
     GGMLType.Q4_K: (256, 144),
+    GGMLType.Q5_K: (256, 176),
     GGMLType.Q6_K: (256, 210),
 }

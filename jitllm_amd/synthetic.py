@@ -6,6 +6,7 @@ Block value distributions:
   Q4_K  fp16 d ~ U(1e-3, 2e-2)/63, fp16 dmin ~ U(1e-3, 2e-2)*8/63 per super-block (so the largest
         weight magnitude d*63*15 stays near 0.3 and the minimum term roughly centres the range),
         8 (scale, min) pairs ~ U{0..63} packed into the 12 scale bytes, 128 bytes of nibbles
+  Q5_K  as Q4_K with d and dmin halved (values reach 31), plus 32 bytes of fifth bits
   Q6_K  fp16 d ~ U(2e-5, 1e-4) per super-block (largest weight d*127*32 near 0.4), 16 signed
         scales ~ U{-128..127}, 128 + 64 bytes of quant bits
   x     fp32 ~ N(0, 1)
@@ -47,6 +48,13 @@ def weight(t: GGMLType, rows: int, cols: int, seed: int) -> np.ndarray:
     elif t == GGMLType.Q4_0:
         raw[:, 0:2] = _scales_f16(rng, blocks, 1e-3, 2e-2).view(np.uint8).reshape(blocks, 2)
         raw[:, 2:] = rng.integers(0, 256, size=(blocks, 16), dtype=np.uint8)
+    elif t == GGMLType.Q5_K:
+        raw[:, 0:2] = _scales_f16(rng, blocks, 5e-4 / 63, 1e-2 / 63).view(np.uint8).reshape(blocks, 2)
+        raw[:, 2:4] = _scales_f16(rng, blocks, 8e-3 / 63, 16e-2 / 63).view(np.uint8).reshape(blocks, 2)
+        sc = rng.integers(0, 64, size=(blocks, 8), dtype=np.uint8)
+        m = rng.integers(0, 64, size=(blocks, 8), dtype=np.uint8)
+        raw[:, 4:16] = pack_q4_k_scales(sc, m)
+        raw[:, 16:] = rng.integers(0, 256, size=(blocks, 160), dtype=np.uint8)
     elif t == GGMLType.Q6_K:
         raw[:, 0:192] = rng.integers(0, 256, size=(blocks, 192), dtype=np.uint8)
         raw[:, 192:208] = rng.integers(-128, 128, size=(blocks, 16), dtype=np.int8).view(np.uint8)

@@ -36,6 +36,7 @@
 #define QK_K 256
 #define Q4_K_BYTES 144
 #define Q6_K_BYTES 210
+#define Q5_K_BYTES 176
 
 int jo_max_threads(void) { return omp_get_max_threads(); }
 
@@ -46,6 +47,7 @@ int jo_block_elems(int type) {
         case JO_Q8_0: return Q_BLOCK;
         case JO_Q4_K: return QK_K;
         case JO_Q6_K: return QK_K;
+        case JO_Q5_K: return QK_K;
         default: return 0;
     }
 }
@@ -56,6 +58,7 @@ int jo_block_bytes(int type) {
         case JO_Q8_0: return Q8_0_BYTES;
         case JO_Q4_K: return Q4_K_BYTES;
         case JO_Q6_K: return Q6_K_BYTES;
+        case JO_Q5_K: return Q5_K_BYTES;
         default: return 0;
     }
 }
@@ -207,12 +210,47 @@ static inline float q6_k_get(const uint8_t *w, int64_t index) {
     return t * (float)q;
 }
 
+/*
+ * J/tensor/standard/Q5_KFloatTensor.java:78-122.  A super-block is fp16 d, dmin | 12 packed scale /
+ * min bytes (as Q4_K) | qh[32] | qs[128]: element pos < 32 of pair p is the low nibble of
+ * qs[32 p + pos] with bit 2 p of qh[pos] as its fifth bit (sub-block 2 p), element 32 + pos the high
+ * nibble with bit 2 p + 1 (sub-block 2 p + 1); w = d * sc * q - dmin * m, left to right in fp32.
+ */
+static inline float q5_k_get(const uint8_t *w, int64_t index) {
+    int64_t block_index = index / QK_K;
+    int within = (int)(index % QK_K);
+    const uint8_t *blk = w + block_index * Q5_K_BYTES;
+    float d = jo_f16_to_f32(read_u16(blk));
+    float dmin = jo_f16_to_f32(read_u16(blk + 2));
+    const uint8_t *scales = blk + 4;
+    int pair = within / 64;
+    int pos = within % 64;
+    int sub, q, high_bit;
+    if (pos < 32) {
+        sub = pair * 2;
+        q = blk[48 + pair * 32 + pos] & 0xF;
+        high_bit = (blk[16 + pos] >> (pair * 2)) & 1;
+    } else {
+        sub = pair * 2 + 1;
+        q = (blk[48 + pair * 32 + (pos - 32)] >> 4) & 0xF;
+        high_bit = (blk[16 + (pos - 32)] >> (pair * 2 + 1)) & 1;
+    }
+    q += high_bit * 16;
+    int sc = q4_k_scale(sub, scales);
+    int m = q4_k_min(sub, scales);
+    float t = d * (float)sc;
+    t = t * (float)q;
+    float u = dmin * (float)m;
+    return t - u;
+}
+
 float jo_get_float(int type, const uint8_t *w, int64_t index) {
     switch (type) {
         case JO_Q8_0: return q8_0_get(w, index);
         case JO_Q4_0: return q4_0_get(w, index);
         case JO_Q4_K: return q4_k_get(w, index);
         case JO_Q6_K: return q6_k_get(w, index);
+        case JO_Q5_K: return q5_k_get(w, index);
         default: return NAN;
     }
 }
@@ -270,6 +308,38 @@ float jo_get_float_alt(int type, const uint8_t *w, int64_t index) {
         float b = dmin * (float)m;
         return a - b;
     }
+    if (type == JO_Q5_K) {
+        /* J/backend/tornado/kernels/TransformerComputeKernelsQ5_K.java:144-220 */
+        const uint8_t *blk = w + (index / 256) * Q5_K_BYTES;
+        int within = (int)(index % 256);
+        float d = jo_f16_to_f32(read_u16(blk));
+        float dmin = jo_f16_to_f32(read_u16(blk + 2));
+        int pair = within / 64;
+        int pos_in_pair = within - pair * 64;
+        int high_nibble = pos_in_pair / 32;
+        int sub = pair * 2 + high_nibble;
+        int pos = pos_in_pair - high_nibble * 32;
+        int qs = blk[48 + pair * 32 + pos] & 0xFF;
+        int q = high_nibble == 0 ? (qs & 0xF) : ((qs >> 4) & 0xF);
+        int bits = blk[16 + pos] & 0xFF;
+        if (pair >= 2) bits >>= 4;
+        if ((pair & 1) == 1) bits >>= 2;
+        if (high_nibble == 1) bits >>= 1;
+        q += (bits & 1) * 16;
+        const uint8_t *s = blk + 4;
+        int sc, m;
+        if (sub < 4) {
+            sc = s[sub] & 63;
+            m = s[sub + 4] & 63;
+        } else {
+            sc = (s[sub + 4] & 0xF) | ((s[sub - 4] >> 6) << 4);
+            m = ((s[sub + 4] >> 4) & 0xF) | ((s[sub] >> 6) << 4);
+        }
+        float a = d * (float)sc;
+        a = a * (float)q;
+        float b = dmin * (float)m;
+        return a - b;
+    }
     if (type == JO_Q6_K) {
         /* J/backend/tornado/kernels/TransformerComputeKernelsQ6_K.java:195-232 */
         const uint8_t *blk = w + (index / 256) * Q6_K_BYTES;
@@ -317,6 +387,12 @@ static float scalar_dot(int type, const uint8_t *w, int64_t this_offset, const f
         case JO_Q4_K:
             for (int64_t j = 0; j < size; j++) {
                 float p = q4_k_get(w, this_offset + j) * x[that_offset + j];
+                result += p;
+            }
+            break;
+        case JO_Q5_K:   /* Q5_KFloatTensor.dot is scalarDot */
+            for (int64_t j = 0; j < size; j++) {
+                float p = q5_k_get(w, this_offset + j) * x[that_offset + j];
                 result += p;
             }
             break;
@@ -455,7 +531,7 @@ static float vector_dot(int type, int bits, const uint8_t *w, int64_t this_offse
  */
 float jo_dot(int type, int flavour, const uint8_t *w, int64_t this_offset, const float *x,
              int64_t that_offset, int64_t size) {
-    if (type != JO_Q4_K && type != JO_Q6_K && (flavour == JO_DOT_VEC128 || flavour == JO_DOT_VEC256)) {
+    if (type != JO_Q4_K && type != JO_Q6_K && type != JO_Q5_K && (flavour == JO_DOT_VEC128 || flavour == JO_DOT_VEC256)) {
         return vector_dot(type, flavour, w, this_offset, x, that_offset, size);
     }
     return scalar_dot(type, w, this_offset, x, that_offset, size);

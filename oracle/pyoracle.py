@@ -12,7 +12,7 @@ import subprocess
 
 import numpy as np
 
-Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
 DOT_SCALAR, DOT_VEC128, DOT_VEC256 = 0, 128, 256
 
 _HERE = os.path.dirname(os.path.abspath(__file__))

@@ -65,6 +65,28 @@ def dequant_q4_k(raw: np.ndarray) -> np.ndarray:
     return out.reshape(-1)
 
 
+def dequant_q5_k(raw: np.ndarray) -> np.ndarray:
+    """ggml's dequantize_row_q5_K, vectorised: sub-block j of 32 takes its low four bits from
+    nibble j % 2 of qs[32 (j // 2) ...], its fifth bit from bit j of qh, scale and min as Q4_K;
+    w = d * sc * q - dmin * m with every product and the difference rounded to fp32."""
+    b = raw.reshape(-1, 176)
+    nb = b.shape[0]
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    dmin = half_bits_to_f32(b[:, 2:4].copy().view(np.uint16)[:, 0])
+    sc, mn = q4_k_scales_mins(b[:, 4:16])
+    qh = b[:, 16:48].astype(np.int32)
+    qs = b[:, 48:].reshape(nb, 4, 32).astype(np.int32)
+    out = np.empty((nb, 8, 32), dtype=np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        for j in range(8):
+            q = ((qs[:, j // 2, :] >> (4 * (j % 2))) & 0xF) + (((qh >> j) & 1) << 4)
+            d1 = (d * sc[:, j].astype(np.float32)).astype(np.float32)
+            m1 = (dmin * mn[:, j].astype(np.float32)).astype(np.float32)
+            t = (d1[:, None] * q.astype(np.float32)).astype(np.float32)
+            out[:, j, :] = (t - m1[:, None]).astype(np.float32)
+    return out.reshape(-1)
+
+
 def dequant_q6_k(raw: np.ndarray) -> np.ndarray:
     """ggml's dequantize_row_q6_K, vectorised: per half of 128, y[l + 32 g] for l < 32 takes its low
     four bits from ql (plane g % 2, nibble g // 2), bits 4-5 from qh >> 2 g, the scale
@@ -87,7 +109,7 @@ def dequant_q6_k(raw: np.ndarray) -> np.ndarray:
     return out.reshape(-1)
 
 
-DEQUANT = {8: dequant_q8_0, 2: dequant_q4_0, 12: dequant_q4_k, 14: dequant_q6_k}
+DEQUANT = {8: dequant_q8_0, 2: dequant_q4_0, 12: dequant_q4_k, 13: dequant_q5_k, 14: dequant_q6_k}
 
 
 def scalar_dot_rows(w_deq: np.ndarray, x: np.ndarray) -> np.ndarray:

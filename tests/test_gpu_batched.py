@@ -260,27 +260,28 @@ def test_two_pass_prefill_qkv_and_gate_up(ctx):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
 
 
+@pytest.mark.parametrize("t", [O.Q5_K, O.Q6_K])
 @pytest.mark.parametrize("d,n,T,residual", [(300, 512, 8, False), (1000, 2048, 100, True), (4096, 256, 600, False)])
-def test_q6_k_batched_rows_take_the_decode_once_path(ctx, d, n, T, residual):
-    """A Q6_K weight has no decode-in-the-loop kernel: every batched call decodes it to fp16 into
+def test_k_quant_batched_rows_take_the_decode_once_path(ctx, t, d, n, T, residual):
+    """A Q6_K / Q5_K weight has no decode-in-the-loop kernel: every batched call decodes it to fp16 into
     the workspace and runs the fp16 GEMM, few rows or many; partial batches leave the rest alone."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
-    say("q6_K batched", d, n, T, residual)
-    raw = synthetic.weight(O.Q6_K, d, n, seed=9300 + d)
+    say("k-quant batched", t, d, n, T, residual)
+    raw = synthetic.weight(t, d, n, seed=9300 + d)
     X = synthetic.activations((T, n), seed=9400 + T)
     active = T - 3
-    ref = O.matmul_batch(O.Q6_K, raw, X, d, n)
+    ref = O.matmul_batch(t, raw, X, d, n)
     out = ctx.float_array(T * d, fill=UNTOUCHED)
     proj = QuantizedBatchProjections(ctx, T, n, d)
-    proj.projection(ctx.from_numpy(X), out, ctx.load_weight(O.Q6_K, raw, d, n), n, d, residual, activeRows=active)
+    proj.projection(ctx.from_numpy(X), out, ctx.load_weight(t, raw, d, n), n, d, residual, activeRows=active)
     ctx.sync()
     got = out.get().reshape(T, d)
     assert np.all(got[active:] == UNTOUCHED)
     want = ref.astype(np.float64) + (float(UNTOUCHED) if residual else 0.0)
     slack = abs(np.spacing(np.float32(UNTOUCHED))) / 2 if residual else 0.0
     excess = np.abs(got[:active].astype(np.float64) - want[:active]) - slack
-    assert np.all(excess <= 5e-4 * magnitude(O.Q6_K, raw, X, d, n)[:active]), float(excess.max())
+    assert np.all(excess <= 5e-4 * magnitude(t, raw, X, d, n)[:active]), float(excess.max())
 
 
 def test_q6_k_batched_gate_up(ctx):

@@ -180,30 +180,38 @@ def test_fused_gate_up(ctx, t, d, n):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + 1e-6)
 
 
-# ---- Q6_K: decode and the single-token projection ---------------------------------------------
+# ---- Q6_K and Q5_K: decode and the plain single-token projection ------------------------------
 
-def test_q6_k_decode_bit_exact(ctx):
+KQ = [O.Q5_K, O.Q6_K]
+KQ_NAMES = {O.Q5_K: "Q5_K", O.Q6_K: "Q6_K"}
+
+
+@pytest.mark.parametrize("t", KQ)
+def test_k_quant_decode_bit_exact(ctx, t):
     """Arbitrary bytes, special fp16 scales and a synthetic weight: the device decode equals
-    Q6_KFloatTensor.getFloat bit for bit."""
+    Q6_KFloatTensor.getFloat / Q5_KFloatTensor.getFloat bit for bit."""
     from jitllm_amd import synthetic
-    say("q6_K decode")
-    for raw, rows in ((FX.random_bytes(20260914, 12 * 210), 12),
-                      (FX.adversarial_blocks(O.Q6_K, 24, 20260908 + O.java_string_hash("Q6_K")), 24),
-                      (synthetic.weight(O.Q6_K, 40, 512, seed=701), 80)):
-        w = upload(ctx, O.Q6_K, raw, rows, raw.size // 210 // rows * 256)
-        assert bits_equal(w.dequantize(), O.dequant(O.Q6_K, raw))
+    say("decode", KQ_NAMES[t])
+    bb = O.block_bytes(t)
+    for raw, rows in ((FX.random_bytes(20260914, 12 * bb), 12),
+                      (FX.adversarial_blocks(t, 24, 20260908 + O.java_string_hash(KQ_NAMES[t])), 24),
+                      (synthetic.weight(t, 40, 512, seed=701), 80)):
+        w = upload(ctx, t, raw, rows, raw.size // bb // rows * 256)
+        assert bits_equal(w.dequantize(), O.dequant(t, raw))
 
 
-@pytest.mark.parametrize("d,n", [(2048, 2048), (32000, 2048), (2048, 8192), (37, 512), (1000, 256), (4, 4096)])
-def test_q6_k_gemv_matches_oracle(ctx, d, n):
+@pytest.mark.parametrize("t", KQ)
+@pytest.mark.parametrize("d,n", [(2048, 2048), (32000, 2048), (2048, 8192), (37, 512), (1000, 256), (4, 4096),
+                                 (64, 1024)])
+def test_k_quant_gemv_matches_oracle(ctx, t, d, n):
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
-    say("q6_K gemv", d, n)
-    raw = synthetic.weight(O.Q6_K, d, n, seed=710 + d % 97)
+    say("gemv", KQ_NAMES[t], d, n)
+    raw = synthetic.weight(t, d, n, seed=710 + d % 97)
     x = synthetic.activations(n, seed=720)
-    ref = O.matmul(O.Q6_K, raw, x, d, n)
-    mag = magnitude(O.Q6_K, raw, x, d, n)
-    w = upload(ctx, O.Q6_K, raw, d, n)
+    ref = O.matmul(t, raw, x, d, n)
+    mag = magnitude(t, raw, x, d, n)
+    w = upload(ctx, t, raw, d, n)
     out = ctx.float_array(d, fill=POISON)
     acc = ctx.from_numpy(np.full(d, 0.75, dtype=np.float32))
     proj = QuantizedProjections(ctx, TornadoWorkspace(wrapX=acc))
@@ -215,23 +223,29 @@ def test_q6_k_gemv_matches_oracle(ctx, d, n):
     assert rel_err(acc.get(), ref.astype(np.float64) + 0.75, mag + 0.75 * 6e-8) < 2e-5
 
 
-def test_q6_k_has_no_fused_single_token_kernels(ctx):
-    """What has no kernel is refused by name (QuantizedProjections.java:386-393 keeps Q6_K out of
-    the fused gate/up as well)."""
+@pytest.mark.parametrize("t", KQ)
+def test_k_quants_have_no_fused_single_token_kernels(ctx, t):
+    """What has no kernel is refused by name; the caller runs the unfused steps
+    (QuantizedProjections.java:386-393, 400-480)."""
     from jitllm_amd import synthetic
     from jitllm_amd._lib import UnsupportedProjection
     from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
-    say("q6_K unsupported")
+    say("unsupported", KQ_NAMES[t])
     d, n = 16, 256
-    w = upload(ctx, O.Q6_K, synthetic.weight(O.Q6_K, d, n, seed=731), d, n)
+    w = upload(ctx, t, synthetic.weight(t, d, n, seed=731), d, n)
     x = ctx.from_numpy(synthetic.activations(n, seed=732))
     out = ctx.float_array(d, fill=POISON)
     proj = QuantizedProjections(ctx, TornadoWorkspace(wrapXb=x, wrapHb=out, wrapHb2=ctx.float_array(d)))
-    with pytest.raises(UnsupportedProjection, match="Q6_K"):
+    with pytest.raises(UnsupportedProjection, match=KQ_NAMES[t]):
         proj.fusedQKV(x, out, out, out, w, w, w)
     assert not proj.fusedGateUp(w, w)
-    with pytest.raises(UnsupportedProjection, match="Q6_K"):
+    with pytest.raises(UnsupportedProjection, match=KQ_NAMES[t]):
         proj.rmsMatvec(x, x, None, out, w, n, d, eps=1e-5)
+    # ... and the unfused gate/up sequence works: two projections and an element-wise SwiGLU
+    proj.gateUp(w, w, n, d)
+    ctx.sync()
+    ref = O.matmul(t, synthetic.weight(t, d, n, seed=731), synthetic.activations(n, seed=732), d, n)
+    assert np.allclose(out.get(), O.swiglu(ref, ref), rtol=1e-4, atol=1e-5)
 
 
 # ---- RMS normalisation folded into the projections, argmax -----------------------------------
@@ -407,8 +421,8 @@ def test_errors_name_the_cause(ctx):
     lib = L.load()
     h = C.c_void_p()
     raw = np.zeros(64, dtype=np.uint8)
-    st = lib.jl_weight_upload(ctx.handle, 13, raw.ctypes.data, 1, 32, C.byref(h))  # Q5_K: no kernel
-    assert st == L.JL_ERR_UNSUPPORTED and b"ggml type 13" in lib.jl_last_error()
+    st = lib.jl_weight_upload(ctx.handle, 3, raw.ctypes.data, 1, 32, C.byref(h))  # Q4_1: no kernel
+    assert st == L.JL_ERR_UNSUPPORTED and b"ggml type 3" in lib.jl_last_error()
     st = lib.jl_weight_upload(ctx.handle, O.Q8_0, raw.ctypes.data, 1, 48, C.byref(h))
     assert st == L.JL_ERR_INVALID and b"whole number" in lib.jl_last_error()
     w8 = upload(ctx, O.Q8_0, synthetic.weight(O.Q8_0, 64, 256, 1), 64, 256)

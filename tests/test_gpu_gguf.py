@@ -27,7 +27,8 @@ def test_upload_from_file_then_project(ctx, tmp_path):
     raws = {"blk.0.attn_q.weight": (O.Q8_0, synthetic.weight(O.Q8_0, d, n, seed=901)),
             "blk.0.ffn_up.weight": (O.Q4_0, synthetic.weight(O.Q4_0, d, n, seed=902)),
             "blk.0.ffn_down.weight": (O.Q4_K, synthetic.weight(O.Q4_K, d, n, seed=903)),
-            "output.weight": (O.Q6_K, synthetic.weight(O.Q6_K, d, n, seed=906))}
+            "output.weight": (O.Q6_K, synthetic.weight(O.Q6_K, d, n, seed=906)),
+            "blk.0.attn_v.weight": (O.Q5_K, synthetic.weight(O.Q5_K, d, n, seed=907))}
     tensors = [("pad.me", (5,), 24, np.arange(5, dtype=np.uint8))]       # pushes the next offset off 32
     tensors += [(name, (n, d), int(t), raw) for name, (t, raw) in raws.items()]
     path = tmp_path / "m.gguf"
@@ -53,12 +54,12 @@ def test_upload_refuses_other_types_and_truncated_files(ctx, tmp_path):
     raw = synthetic.weight(O.Q8_0, d, n, seed=905)
     path = tmp_path / "m.gguf"
     W.write_gguf(path, [], [("norm.weight", (n,), 0, np.ones(n, dtype=np.float32)),
-                            ("emb.weight", (n, 3), 13, np.zeros(3 * 176, dtype=np.uint8)),   # Q5_K
+                            ("emb.weight", (n, 3), 3, np.zeros(3 * 8 * 20, dtype=np.uint8)),   # Q4_1
                             ("q.weight", (n, d), 8, raw)], truncate_data_by=100)
     with GGUF(path) as g:
         with pytest.raises(UnsupportedProjection, match="ggml type 0"):
             g.load_weight(ctx, "norm.weight")
-        with pytest.raises(UnsupportedProjection, match="ggml type 13"):
+        with pytest.raises(UnsupportedProjection, match="ggml type 3"):
             g.load_weight(ctx, "emb.weight")
         with pytest.raises(JitllmHipError, match="runs past the end of the file"):
             g.load_weight(ctx, "q.weight")

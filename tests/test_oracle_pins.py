@@ -223,17 +223,56 @@ def test_q6_k_layout_known_answers():
     assert O.dequant(O.Q6_K, b)[0] == want
 
 
-def test_q6_k_scalar_dot_and_matmul():
-    """Q6_KFloatTensor.dot is scalarDot (:124-127): a strictly sequential fp32 sum of decoded
-    weight times x, whatever flavour is asked for; rows are independent."""
+def test_q5_k_decode_three_ways_and_layout():
+    """Host wording (Q5_KFloatTensor.java:78-122) == device wording
+    (TransformerComputeKernelsQ5_K.java:144-220) == an independent numpy statement of ggml's
+    dequantize_row_q5_K; and the fifth bit's place written out from the format: bit j of qh[pos]
+    belongs to element 32 j + pos (sub-block j), worth 16."""
+    for raw in (FX.random_bytes(20260913, 10 * 176),
+                FX.adversarial_blocks(O.Q5_K, 24, 20260908 + O.java_string_hash("Q5_K"))):
+        main = O.dequant(O.Q5_K, raw)
+        assert_bit_equal(main, O.dequant_alt(O.Q5_K, raw))
+        assert_bit_equal(main, NP.DEQUANT[O.Q5_K](raw))
+    from jitllm_amd import synthetic
+    def block():
+        b = np.zeros(176, dtype=np.uint8)
+        b[0:2] = [0x00, 0x3C]                                        # d = 1, dmin = 0
+        b[4:16] = synthetic.pack_q4_k_scales(np.full(8, 1, np.uint8), np.zeros(8, np.uint8))
+        return b
+    assert np.all(O.dequant(O.Q5_K, block()) == 0.0)
+    for pos in (0, 7, 31):
+        for j in range(8):
+            b = block()
+            b[16 + pos] = 1 << j
+            want = np.zeros(256, dtype=np.float32)
+            want[32 * j + pos] = 16.0
+            assert np.array_equal(O.dequant(O.Q5_K, b), want), (pos, j)
+        for pair in range(4):
+            b = block()
+            b[48 + 32 * pair + pos] = 0x93                           # low nibble 3, high nibble 9
+            want = np.zeros(256, dtype=np.float32)
+            want[64 * pair + pos], want[64 * pair + 32 + pos] = 3.0, 9.0
+            assert np.array_equal(O.dequant(O.Q5_K, b), want), (pos, pair)
+    # the minimum is subtracted after the product: (d sc) q - dmin m
+    b = block()
+    b[2:4] = [0x00, 0x38]                                            # dmin = 0.5
+    b[4:16] = synthetic.pack_q4_k_scales(np.full(8, 3, np.uint8), np.full(8, 5, np.uint8))
+    b[48] = 0x02
+    assert O.dequant(O.Q5_K, b)[0] == np.float32(3 * 2 - 0.5 * 5)
+
+
+@pytest.mark.parametrize("t", [O.Q5_K, O.Q6_K])
+def test_k_quant_scalar_dot_and_matmul(t):
+    """Q6_KFloatTensor.dot / Q5_KFloatTensor.dot are scalarDot: a strictly sequential fp32 sum of
+    decoded weight times x, whatever flavour is asked for; rows are independent."""
     from jitllm_amd import synthetic
     d, n = 5, 512
-    raw = synthetic.weight(O.Q6_K, d, n, seed=77)
+    raw = synthetic.weight(t, d, n, seed=77)
     x = synthetic.activations(n, seed=78)
-    w = NP.DEQUANT[O.Q6_K](raw).reshape(d, n)
+    w = NP.DEQUANT[t](raw).reshape(d, n)
     want = NP.scalar_dot_rows(w, x)
     for flavour in (O.DOT_SCALAR, O.DOT_VEC256):
-        assert_bit_equal(O.matmul(O.Q6_K, raw, x, d, n, flavour=flavour), want)
+        assert_bit_equal(O.matmul(t, raw, x, d, n, flavour=flavour), want)
 
 
 # ---- dot products -------------------------------------------------------------------------
