@@ -228,6 +228,24 @@ int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const f
             int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
             int math, void *workspace, size_t workspace_bytes);
 
+/*
+ * jl_gemm with a resident fp16 copy of the call's weights: the reference's "residency choice" for
+ * the batched prefill (dequantize*ToFP16Once, TransformerBatchPrefillKernels.java:2336-2366: "the
+ * copy outlives the chunk, so it is decoded on the first one only"; BatchPrefillWorkspace).  Calls
+ * that decode their weights to fp16 (512 rows and more with enough output columns, and every Q6_K /
+ * Q5_K call) put the copy into `resident` instead of the workspace, and skip the decode when
+ * `*resident_state` says the buffer already holds what they need.  The caller owns one buffer of
+ * jl_gemm_resident_bytes(weights, count) bytes (2 per weight) and one int32 per set of weights it
+ * passes together, zeroes the int before the first call and whenever the weights' contents change,
+ * and never shares a buffer between different sets.  Calls that do not decode ignore both.  Results
+ * are the same as jl_gemm's, bit for bit.
+ */
+size_t jl_gemm_resident_bytes(const jl_weight *const *weights, int count);
+int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
+                     int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
+                     int math, void *workspace, size_t workspace_bytes, void *resident,
+                     size_t resident_bytes, int32_t *resident_state);
+
 /* ---- GGUF files: the caller either side of jl_weight_upload --------------------------------- */
 
 /*

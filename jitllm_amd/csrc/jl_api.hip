@@ -320,9 +320,9 @@ size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols,
     return jl_gemm_workspace_bytes_impl(max_rows, cols, out_cols, math == JL_MATH_DEFAULT ? JL_MATH_F16 : math);
 }
 
-int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
-            int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
-            int math, void *workspace, size_t workspace_bytes) {
+static int gemm_checked(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
+                        int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
+                        int math, void *workspace, size_t workspace_bytes, const jl_resident *resident) {
     JL_REQUIRE(ctx && weights && X && C, "jl_gemm: null argument");
     JL_REQUIRE(count >= 1 && count <= 8, "jl_gemm: %d weights (1..8)", count);
     JL_REQUIRE(batch >= 1 && active_rows >= 0 && active_rows <= batch,
@@ -363,7 +363,36 @@ int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const f
                        need);
     }
     return jl_launch_gemm(ctx, weights, count, X, C, batch, active_rows, ldo, col_offset, epilogue,
-                          math, workspace, workspace_bytes);
+                          math, workspace, workspace_bytes, resident);
+}
+
+int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
+            int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
+            int math, void *workspace, size_t workspace_bytes) {
+    return gemm_checked(ctx, weights, count, X, C, batch, active_rows, ldo, col_offset, epilogue, math,
+                        workspace, workspace_bytes, nullptr);
+}
+
+size_t jl_gemm_resident_bytes(const jl_weight *const *weights, int count) {
+    if (!weights || count < 1) return 0;
+    int64_t rows = 0;
+    for (int i = 0; i < count; i++) {
+        if (!weights[i]) return 0;
+        rows += weights[i]->rows;
+    }
+    // 2 bytes per weight, rows padded to whole 256-row tiles of either layout
+    return (size_t)((rows + 511) / 256 * 256) * (size_t)weights[0]->cols * 2;
+}
+
+int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
+                     int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
+                     int math, void *workspace, size_t workspace_bytes, void *resident,
+                     size_t resident_bytes, int32_t *resident_state) {
+    JL_REQUIRE(resident && resident_state, "jl_gemm_resident: null resident buffer or state");
+    JL_REQUIRE(((uintptr_t)resident & 255) == 0, "jl_gemm_resident: the resident buffer must be 256-byte aligned");
+    const jl_resident r{resident, resident_bytes, resident_state};
+    return gemm_checked(ctx, weights, count, X, C, batch, active_rows, ldo, col_offset, epilogue, math,
+                        workspace, workspace_bytes, &r);
 }
 
 }  // extern "C"

@@ -897,7 +897,8 @@ int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row
 
 int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
-                   int epilogue, int math, void *workspace, size_t workspace_bytes) {
+                   int epilogue, int math, void *workspace, size_t workspace_bytes,
+                   const jl_resident *resident) {
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     if (math == JL_MATH_INT8) {
@@ -943,7 +944,12 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
         dsplits = 1;
     }
     const size_t copy_bytes = round_up(jl_dense_copy_bytes(k, virt), 256);
-    const bool dense = bn != 0 && copy_bytes + (dsplits > 1 ? jl_dense_plane_bytes(rows, virt) : 0) <= plane_bytes;
+    // the decoded copy goes to the caller's resident buffer when there is one that holds it,
+    // otherwise to the head of the workspace's third region
+    const bool kept = resident && resident->copy && resident->state && resident->bytes >= copy_bytes &&
+                      ((uintptr_t)resident->copy & 255) == 0;
+    const size_t in_workspace = kept ? 0 : copy_bytes;
+    const bool dense = bn != 0 && in_workspace + (dsplits > 1 ? jl_dense_plane_bytes(rows, virt) : 0) <= plane_bytes;
     const int padded_rows = dense ? (int)round_up((size_t)rows, 256) : padded;
 
     if (dense_only && !dense) {
@@ -953,8 +959,14 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded_rows), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
     JL_HIP(hipGetLastError());
     if (dense) {
-        return jl_launch_gemm_dense(ctx, weights, count, A, row_scale, C, rows, ldo, col_offset, epilogue,
-                                    (_Float16 *)planes, bn, dsplits, (float *)((uint8_t *)planes + copy_bytes));
+        // what a kept copy looks like: gate / up interleaved by half tiles of this BN, or plain
+        const int32_t layout = epilogue == JL_SWIGLU ? bn : 1;
+        const bool decode = !kept || *resident->state != layout;
+        const int st = jl_launch_gemm_dense(ctx, weights, count, A, row_scale, C, rows, ldo, col_offset, epilogue,
+                                            kept ? (_Float16 *)resident->copy : (_Float16 *)planes, decode, bn,
+                                            dsplits, (float *)((uint8_t *)planes + in_workspace));
+        if (st == JL_OK && kept) *resident->state = layout;
+        return st;
     }
 
     GemmParams p{};

@@ -518,7 +518,7 @@ size_t jl_dense_copy_bytes(int k, int out_cols_virtual) {
 
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
-                         int epilogue, _Float16 *copy, int bn, int splits, float *planes) {
+                         int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes) {
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     const bool swiglu = epilogue == JL_SWIGLU;
@@ -539,14 +539,19 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
     d.row_bytes = k / jl_block_elems(type) * jl_block_bytes(type);
     d.n_total = n_total;
     d.half = swiglu ? bn / 2 : 0;
-    int dst;
-    switch (type) {
-        case JL_Q8_0: dst = launch_decode<JL_Q8_0>(ctx, d, ntiles * bn); break;
-        case JL_Q4_0: dst = launch_decode<JL_Q4_0>(ctx, d, ntiles * bn); break;
-        case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, d, ntiles * bn); break;
-        case JL_Q5_K: dst = launch_decode<JL_Q5_K>(ctx, d, ntiles * bn); break;
-        case JL_Q6_K: dst = launch_decode<JL_Q6_K>(ctx, d, ntiles * bn); break;
-        default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
+    // plain layout: always whole 256-row tiles, so the copy does not depend on the column tile
+    // (a copy that is kept across calls stays valid when the row count, hence BN, changes)
+    const int decoded_rows = swiglu ? ntiles * bn : (n_total + 255) / 256 * 256;
+    int dst = JL_OK;
+    if (decode) {
+        switch (type) {
+            case JL_Q8_0: dst = launch_decode<JL_Q8_0>(ctx, d, decoded_rows); break;
+            case JL_Q4_0: dst = launch_decode<JL_Q4_0>(ctx, d, decoded_rows); break;
+            case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, d, decoded_rows); break;
+            case JL_Q5_K: dst = launch_decode<JL_Q5_K>(ctx, d, decoded_rows); break;
+            case JL_Q6_K: dst = launch_decode<JL_Q6_K>(ctx, d, decoded_rows); break;
+            default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
+        }
     }
     if (dst != JL_OK) return dst;
 

@@ -77,9 +77,17 @@ int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, f
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
 int jl_launch_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
 int jl_launch_fill(jl_context *ctx, float *dst, float value, size_t count);
+// A caller-owned fp16 copy of one projection's weights that outlives the call: decoded when
+// *state does not name the layout the call needs (0 = empty), reused otherwise.
+struct jl_resident {
+    void *copy;
+    size_t bytes;
+    int32_t *state;
+};
 int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
-                   int epilogue, int math, void *workspace, size_t workspace_bytes);
+                   int epilogue, int math, void *workspace, size_t workspace_bytes,
+                   const jl_resident *resident);
 // Batched decode (at most 64 rows): the weight-streaming kernel.  `taken` says whether the shape
 // was one it handles; when not, nothing was launched and the tiled GEMM must run instead.
 int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
@@ -91,7 +99,7 @@ size_t jl_dense_copy_bytes(int k, int out_cols_virtual);
 size_t jl_dense_plane_bytes(int rows, int out_cols_virtual);
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
-                         int epilogue, _Float16 *copy, int bn, int splits, float *planes);
+                         int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes);
 // Adds split-K planes [splits][rows padded][ntiles * 128] in split order and applies the epilogue.
 int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row_scale, float *C, int rows,
                           int n_total, int ntiles, int64_t plane, int splits, int64_t ldo, int64_t col_offset,

@@ -139,7 +139,7 @@ class QuantizedBatchProjections:
     """Projections of ``batchSize`` activation rows at once (batched decode, batched prefill)."""
 
     def __init__(self, context: Context, batchSize: int, max_cols: int, max_out_cols: int = 0,
-                 math: int = L.JL_MATH_DEFAULT):
+                 math: int = L.JL_MATH_DEFAULT, resident: bool = False):
         """``max_cols`` is the longest row any projection reads, ``max_out_cols`` the most output
         columns one call produces (gate + up rows for a fused gate/up); together they size the
         workspace once, before anything runs (Implementation.needs)."""
@@ -150,6 +150,10 @@ class QuantizedBatchProjections:
         self._max_cols = int(max_cols)
         nbytes = self._lib.jl_gemm_workspace_bytes(self.batchSize, self._max_cols, int(max_out_cols), math)
         self.workspace = DeviceBuffer(context, max(nbytes, 256))
+        # the reference's residency choice for the batched prefill (BatchPrefillWorkspace;
+        # dequantize*ToFP16Once): an fp16 copy per set of weights that outlives the call
+        self.resident = bool(resident)
+        self._copies: dict = {}
 
     def workspace_bytes(self) -> int:
         return self.workspace.nbytes
@@ -160,9 +164,20 @@ class QuantizedBatchProjections:
         if n > self._max_cols:
             raise ValueError(f"row length {n} exceeds the {self._max_cols} the workspace was sized for")
         arr = (C.c_void_p * len(weights))(*[w.handle for w in weights])
-        L.check(self._lib.jl_gemm(self.context.handle, arr, len(weights), x.ptr, out.ptr,
-                                  self.batchSize, activeRows, ldo, colOffset, epilogue, self.math,
-                                  self.workspace.ptr, self.workspace.nbytes))
+        if not self.resident:
+            L.check(self._lib.jl_gemm(self.context.handle, arr, len(weights), x.ptr, out.ptr,
+                                      self.batchSize, activeRows, ldo, colOffset, epilogue, self.math,
+                                      self.workspace.ptr, self.workspace.nbytes))
+            return
+        key = tuple(w.handle.value for w in weights) + (epilogue == L.JL_SWIGLU,)
+        if key not in self._copies:
+            nbytes = self._lib.jl_gemm_resident_bytes(arr, len(weights))
+            self._copies[key] = (DeviceBuffer(self.context, nbytes), C.c_int32(0))
+        copy, state = self._copies[key]
+        L.check(self._lib.jl_gemm_resident(self.context.handle, arr, len(weights), x.ptr, out.ptr,
+                                           self.batchSize, activeRows, ldo, colOffset, epilogue, self.math,
+                                           self.workspace.ptr, self.workspace.nbytes, copy.ptr, copy.nbytes,
+                                           C.byref(state)))
 
     def projection(self, x: FloatArray, out: FloatArray, w: TornadoTensor, n: int, d: int,
                    residual: bool, activeRows: int | None = None) -> None:

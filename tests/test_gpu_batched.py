@@ -310,6 +310,36 @@ def test_q6_k_batched_gate_up(ctx):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
 
 
+def test_resident_fp16_copy_gives_the_same_bits(ctx):
+    """The reference's residency choice: the decoded copy is kept in a caller-owned buffer and
+    decoded on the first call only.  Same results as without, on the first call, on the second
+    (no decode), and after the row count -- hence the gate/up layout -- changes."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("resident copy")
+    t, d, n = O.Q8_0, 5800, 256
+    raw = synthetic.weight(t, d, n, seed=9601)
+    w = ctx.load_weight(t, raw, d, n)
+    r1, r3 = synthetic.weight(t, 8200, n, seed=9602), synthetic.weight(t, 8200, n, seed=9603)
+    w1, w3 = ctx.load_weight(t, r1, 8200, n), ctx.load_weight(t, r3, 8200, n)
+    T = 2048
+    X = ctx.from_numpy(synthetic.activations((T, n), seed=9604))
+    plain = QuantizedBatchProjections(ctx, T, n, 2 * 8200)
+    kept = QuantizedBatchProjections(ctx, T, n, 2 * 8200, resident=True)
+    def run(p, rows):
+        out = ctx.float_array(T * d, fill=UNTOUCHED)
+        hb = ctx.float_array(T * 8200, fill=UNTOUCHED)
+        p.projection(X, out, w, n, d, False, activeRows=rows)
+        p.gateUp(X, hb, w1, w3, n, 8200, activeRows=rows)
+        ctx.sync()
+        return out.get(), hb.get()
+    for rows in (2048, 2048, 1024, 2048, 700):      # 1024 rows pick another column tile for gate/up
+        a, b = run(plain, rows), run(kept, rows)
+        assert np.array_equal(a[0].view(np.uint32), b[0].view(np.uint32)), rows
+        assert np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32)), rows
+    assert len(kept._copies) == 2
+
+
 def test_huge_activation_rows_stay_finite(ctx):
     """Rows far outside fp16's range are rescaled by a power of two, not turned into infinities."""
     from jitllm_amd import synthetic
