@@ -53,9 +53,7 @@ static int context_create(int device, hipStream_t borrowed, bool borrow, jl_cont
         }
         ctx->owns_stream = true;
     }
-    hipError_t e = hipMalloc(&ctx->scratch, JL_CONTEXT_SCRATCH_BYTES);
-    if (e == hipSuccess) e = hipMemset(ctx->scratch, 0, JL_CONTEXT_SCRATCH_BYTES);
-    if (e == hipSuccess) e = hipDeviceSynchronize();   // the context's stream does not wait for the null stream
+    const hipError_t e = hipMalloc(&ctx->scratch, JL_CONTEXT_SCRATCH_BYTES);   // written before it is read
     if (e != hipSuccess) {
         if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
         delete ctx;
