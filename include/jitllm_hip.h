@@ -46,12 +46,16 @@ typedef enum jl_status {
 /* ggml type ids as a GGUF tensor-info record carries them (GGMLType ordinals). */
 /* Q8_0, Q4_0 and Q4_K have every entry point below.  Q6_K (210 B / 256) and Q5_K (176 B / 256;
  * J/format/GGMLType.java:21-29: the vocabulary projection and some attention / feed-forward tensors
- * of "Q4_K_M" files are Q6_K, "Q5_K_M" files are Q5_K with Q6_K) have
+ * of "Q4_K_M" files are Q6_K, "Q5_K_M" files are Q5_K with Q6_K), and the types quantisers mix
+ * into other files -- Q4_1 (20 B / 32, GGMLType.java:8), Q5_0 (22 B / 32, :11) and IQ4_XS
+ * (136 B / 256, :39-41) -- have
  * jl_dequant_f32, jl_gemv and jl_gemm -- the latter always by decoding the weights to fp16 into the
  * workspace first, whatever the row count -- while the fused single-token entry points return
  * JL_ERR_UNSUPPORTED for them (the reference fuses gate/up for Q5_K but not Q6_K,
  * QuantizedProjections.java:386-393; a caller that gets JL_ERR_UNSUPPORTED runs the unfused steps). */
-typedef enum jl_ggml_type { JL_Q4_0 = 2, JL_Q8_0 = 8, JL_Q4_K = 12, JL_Q5_K = 13, JL_Q6_K = 14 } jl_ggml_type;
+typedef enum jl_ggml_type {
+    JL_Q4_0 = 2, JL_Q4_1 = 3, JL_Q5_0 = 6, JL_Q8_0 = 8, JL_Q4_K = 12, JL_Q5_K = 13, JL_Q6_K = 14, JL_IQ4_XS = 23
+} jl_ggml_type;
 
 /* What a projection does with its result (Int8GemmKernels.java:617-621 EPILOGUE_*). */
 typedef enum jl_epilogue {

@@ -87,6 +87,9 @@ int jl_launch_dequant(jl_context *ctx, const jl_weight *w, float *out) {
             break;
         case JL_Q6_K:
         case JL_Q5_K:
+        case JL_Q4_1:
+        case JL_Q5_0:
+        case JL_IQ4_XS:
             return jl_launch_dequant_direct(ctx, w, out);
         default:
             return jl_fail(JL_ERR_UNSUPPORTED, "jl_dequant_f32: no decode kernel for ggml type %d",

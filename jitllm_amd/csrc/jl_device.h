@@ -31,6 +31,29 @@ __device__ __forceinline__ void jl_q4k_scale_min(uint32_t s0, uint32_t s1, uint3
     }
 }
 
+// Hands a value back to the compiler as one it knows nothing about.  Used on words of four
+// byte-sized quants after their nibble mask: the byte -> float conversions then stay the
+// single-instruction v_cvt_f32_ubyteN, where the compiler would otherwise see through the mask and
+// extract each 4-bit field on its own (a bit-field extract plus a conversion per weight).
+__device__ __forceinline__ uint32_t jl_opaque(uint32_t v) {
+    asm("" : "+v"(v));
+    return v;
+}
+
+// The bits 0..3 of x, one to a byte (bit k of x at bit 0 of byte k).
+__device__ __forceinline__ uint32_t jl_spread4(uint32_t x) { return ((x & 0xFu) * 0x00204081u) & 0x01010101u; }
+
+// ggml's kvalues_iq4nl (-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113;
+// J/tensor/standard/IQ4_XSFloatTensor.java:30-32) of the four nibbles held one to a byte in `idx`,
+// as four signed bytes: two byte permutes pick entry idx & 7 of each half of the table, a third
+// picks the half by bit 3.
+__device__ __forceinline__ uint32_t jl_iq4nl_lookup4(uint32_t idx) {
+    const uint32_t low3 = idx & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, low3);   // entries 0..7
+    const uint32_t hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, low3);   // entries 8..15
+    return __builtin_amdgcn_perm(hi, lo, 0x03020100u | ((idx & 0x08080808u) >> 1));
+}
+
 // Sum over the lanes of each aligned group of `width` lanes (a power of two, at most 64).  Every
 // lane of a group ends with the group's total.
 template <int WIDTH>

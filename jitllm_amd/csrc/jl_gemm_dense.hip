@@ -115,6 +115,51 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
         const int shift = (c & 2) * 2;
         const h2 bias = {(_Float16)1032.f, (_Float16)1032.f}, d2 = {d, d};
         *dst = pack8_scaled((q.lo >> shift) & 0x0F0F0F0Fu, (q.hi >> shift) & 0x0F0F0F0Fu, bias, d2);
+    } else if constexpr (TYPE == JL_Q4_1 || TYPE == JL_Q5_0 || TYPE == JL_IQ4_XS) {
+        // chunk c % 4 of the group of 32 c / 4: the low (chunks 0, 1) or high (2, 3) nibbles of
+        // eight of the group's sixteen bytes; the value is the host decode in fp32 --
+        // (q * d) + m (Q4_1FloatTensor.java:73-94), d * (q - 16) (Q5_0FloatTensor.java:61-85),
+        // (d * (ls - 32)) * kvalues[q] (IQ4_XSFloatTensor.java:72-100) -- rounded once to fp16
+        const int shift = (c & 2) * 2;
+        uint32_t q0, q1;
+        float a, b = 0.f;
+        if constexpr (TYPE == JL_Q4_1) {
+            const uint8_t *blk = row + (c >> 2) * 20;
+            const uint32_t dm = *(const uint32_t *)blk;
+            q0 = (*(const uint32_t *)(blk + 4 + (c & 1) * 8) >> shift) & 0x0F0F0F0Fu;
+            q1 = (*(const uint32_t *)(blk + 8 + (c & 1) * 8) >> shift) & 0x0F0F0F0Fu;
+            a = jl_half_bits_to_float(dm);
+            b = jl_half_bits_to_float(dm >> 16);
+        } else if constexpr (TYPE == JL_Q5_0) {
+            const uint8_t *blk = row + (c >> 2) * 22;
+            const Quants8 q = *(const Quants8 *)(blk + 6 + (c & 1) * 8);
+            const uint32_t qh = (uint32_t)*(const unsigned short *)(blk + 2) |
+                                ((uint32_t)*(const unsigned short *)(blk + 4) << 16);
+            const uint32_t bits = qh >> (8 * (c & 3));        // the fifth bits of columns 8 (c % 4) ..
+            q0 = ((q.lo >> shift) & 0x0F0F0F0Fu) | (jl_spread4(bits) << 4);
+            q1 = ((q.hi >> shift) & 0x0F0F0F0Fu) | (jl_spread4(bits >> 4) << 4);
+            a = jl_half_bits_to_float(*(const unsigned short *)blk);
+        } else {
+            const uint8_t *sb = row + (int64_t)(c >> 5) * 136;
+            const int g = (c >> 2) & 7;
+            const uint2 hdr = *(const uint2 *)sb;
+            const uint2 q = *(const uint2 *)(sb + 8 + 16 * g + (c & 1) * 8);
+            const int ls = (int)(((hdr.y >> (4 * g)) & 0xFu) | ((((hdr.x >> 16) >> (2 * g)) & 3u) << 4));
+            a = __fmul_rn(jl_half_bits_to_float(hdr.x), (float)(ls - 32));
+            q0 = jl_iq4nl_lookup4((q.x >> shift) & 0x0F0F0F0Fu);
+            q1 = jl_iq4nl_lookup4((q.y >> shift) & 0x0F0F0F0Fu);
+        }
+        _Float16 v[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const uint32_t byte = ((e < 4 ? q0 : q1) >> (8 * (e & 3))) & 0xFF;
+            float f;
+            if constexpr (TYPE == JL_Q4_1) f = __fadd_rn(__fmul_rn((float)byte, a), b);
+            else if constexpr (TYPE == JL_Q5_0) f = __fmul_rn(a, (float)((int)byte - 16));
+            else f = __fmul_rn(a, (float)(int)(int8_t)byte);
+            v[e] = (_Float16)f;
+        }
+        *dst = *(const uint4 *)v;
     } else if constexpr (TYPE == JL_Q5_K) {
         // chunk c % 32 of super-block c / 32 (d, dmin | 12 scale bytes | qh[32] | qs[128]): sub-block
         // sub, positions pos .. pos + 7; the value is the host decode ((d * sc) * q) - (dmin * m) in
@@ -550,6 +595,9 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
             case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, d, decoded_rows); break;
             case JL_Q5_K: dst = launch_decode<JL_Q5_K>(ctx, d, decoded_rows); break;
             case JL_Q6_K: dst = launch_decode<JL_Q6_K>(ctx, d, decoded_rows); break;
+            case JL_Q4_1: dst = launch_decode<JL_Q4_1>(ctx, d, decoded_rows); break;
+            case JL_Q5_0: dst = launch_decode<JL_Q5_0>(ctx, d, decoded_rows); break;
+            case JL_IQ4_XS: dst = launch_decode<JL_IQ4_XS>(ctx, d, decoded_rows); break;
             default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
         }
     }

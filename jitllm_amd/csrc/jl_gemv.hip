@@ -95,8 +95,8 @@ __device__ __forceinline__ float slice_dot_q4_0(const uint32_t (&dw)[9], const f
 #pragma unroll
     for (int i = 0; i < 9; i++) {
         uint32_t v = dw[i];
-        lo[i] = v & 0x0F0F0F0Fu;
-        hi[i] = (v >> 4) & 0x0F0F0F0Fu;
+        lo[i] = jl_opaque(v & 0x0F0F0F0Fu);
+        hi[i] = jl_opaque((v >> 4) & 0x0F0F0F0Fu);
     }
     float dA = jl_half_bits_to_float(w0);
     float dB = jl_half_bits_to_float(w4 >> 16);
@@ -134,8 +134,8 @@ __device__ __forceinline__ float slice_dot_q4_k(const uint4 &h, const uint4 &q0,
     float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        uint32_t lo = w[i] & 0x0F0F0F0Fu;
-        uint32_t hi = (w[i] >> 4) & 0x0F0F0F0Fu;
+        uint32_t lo = jl_opaque(w[i] & 0x0F0F0F0Fu);
+        uint32_t hi = jl_opaque((w[i] >> 4) & 0x0F0F0F0Fu);
         a0 = fmaf(ubyte(lo, 0), x[4 * i + 0], a0);
         a1 = fmaf(ubyte(lo, 1), x[4 * i + 1], a1);
         a0 = fmaf(ubyte(lo, 2), x[4 * i + 2], a0);

@@ -1,4 +1,4 @@
-// Single-token projection over Q6_K and Q5_K weights: out (+)= W . x.
+// Single-token projection over Q6_K, Q5_K, Q4_1, Q5_0 and IQ4_XS weights: out (+)= W . x.
 //
 // Files quantised "Q4_K_M" / "Q5_K_M" keep their vocabulary projection and some attention /
 // feed-forward tensors in Q6_K, and the reference reads a projection "by its own representation,
@@ -10,6 +10,14 @@
 //         (J/tensor/standard/Q6_KFloatTensor.java:66-122)
 //   Q5_K  fp16 d, dmin | 12 packed scale/min bytes | qh[32] | qs[128]   w = d * sc * q - dmin * m,
 //         q = nibble + 16 * (bit 2 pair + nibble half of qh)  (Q5_KFloatTensor.java:78-122)
+// and the types quantisers mix into Q4_0 / K-quant files (matrixVectorGenericQ4_1 / Q5_0 / IQ4_XS,
+// TransformerComputeKernelsQ4_1.java:272-290, ...Q5_0.java:261-279, ...IQ4_XS.java:248-266):
+//   Q4_1  fp16 d, m | 16 nibble bytes                w = d * q + m      (Q4_1FloatTensor.java:73-94)
+//   Q5_0  fp16 d | 32 fifth bits | 16 nibble bytes   w = d * (q - 16)   (Q5_0FloatTensor.java:61-85)
+//   IQ4_XS fp16 d | scales_h | scales_l[4] | qs[128] w = d * (ls - 32) * kvalues_iq4nl[q]
+//         (IQ4_XSFloatTensor.java:72-100)
+// whose 16 nibble bytes hold elements 0..15 of a group of 32 in their low halves and 16..31 in
+// their high halves: a lane takes eight consecutive bytes of one group.
 //
 // One wave per weight row, sixteen lanes per super-block.  A lane reads eight consecutive bytes of
 // the low-bit plane and the eight high-bit bytes of the same positions, which hold sixteen
@@ -29,8 +37,9 @@ struct __attribute__((packed, aligned(2))) U64a2 { uint32_t lo, hi; };
 
 __device__ __forceinline__ float ub(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
 
-// sum over the four bytes of q (values 0..63) times x
+// sum over the four bytes of q (values 0..255) times x
 __device__ __forceinline__ float dot4(uint32_t q, const float4 x) {
+    q = jl_opaque(q);   // keeps the four conversions byte selects of one register
     return fmaf(ub(q, 0), x.x, fmaf(ub(q, 1), x.y, fmaf(ub(q, 2), x.z, ub(q, 3) * x.w)));
 }
 
@@ -51,12 +60,30 @@ template <> struct Raw<JL_Q5_K> {
     uint2 qs, qh;
     uint4 hdr;
 };
+// Q4_1 / Q5_0 / IQ4_XS, lane j = (group, half) with group = j / 2: bytes 8 half .. 8 half + 7 of the
+// group's sixteen.  Q4_1 blocks are 4-byte aligned, Q5_0 blocks 2-byte, IQ4_XS super-blocks 8-byte.
+struct __attribute__((packed, aligned(4))) U64a4 { uint32_t lo, hi; };
+template <> struct Raw<JL_Q4_1> {
+    U64a4 qs;
+    uint32_t dm;           // d, m
+};
+template <> struct Raw<JL_Q5_0> {
+    U64a2 qs;
+    U32a2 qh;
+    unsigned short d;
+};
+template <> struct Raw<JL_IQ4_XS> {
+    uint2 qs;
+    uint2 hdr;             // d, scales_h | scales_l
+};
 // The sixteen activations that go with it: eight consecutive ones of the low-nibble group and
 // eight of the high-nibble group, with -32 times their sums (the "- 32" of every weight, applied
 // to the group's sum).
 struct Xs {
     float4 x[4];
-    float m32[2];   // Q6_K: -32 times the sum of each group's eight; Q5_K: the plain sums
+    float m32[2];   // the sum of each eight, times the constant the type takes off every weight:
+                    // Q6_K -32, Q5_0 -16, IQ4_XS -128 (its table is used with 128 added); Q5_K and
+                    // Q4_1, whose minimum is per block, the plain sums
 };
 
 template <int TYPE>
@@ -68,11 +95,23 @@ __device__ __forceinline__ Raw<TYPE> load_raw(const uint8_t *blk, int j) {
         r.qh = *(const U64a2 *)(blk + 128 + 32 * h + 8 * (i & 3));
         r.s8 = *(const U64a2 *)(blk + 192 + 8 * h);
         r.d = *(const unsigned short *)(blk + 208);
-    } else {
+    } else if constexpr (TYPE == JL_Q5_K) {
         const int pair = j >> 2, i = j & 3;   // super-blocks are 176 bytes: everything is aligned
         r.hdr = *(const uint4 *)blk;
         r.qh = *(const uint2 *)(blk + 16 + 8 * i);
         r.qs = *(const uint2 *)(blk + 48 + 32 * pair + 8 * i);
+    } else if constexpr (TYPE == JL_Q4_1) {
+        const uint8_t *b = blk + 20 * (j >> 1);
+        r.dm = *(const uint32_t *)b;
+        r.qs = *(const U64a4 *)(b + 4 + 8 * (j & 1));
+    } else if constexpr (TYPE == JL_Q5_0) {
+        const uint8_t *b = blk + 22 * (j >> 1);
+        r.d = *(const unsigned short *)b;
+        r.qh = *(const U32a2 *)(b + 2);
+        r.qs = *(const U64a2 *)(b + 6 + 8 * (j & 1));
+    } else {
+        r.hdr = *(const uint2 *)blk;
+        r.qs = *(const uint2 *)(blk + 8 + 8 * j);
     }
     return r;
 }
@@ -87,9 +126,12 @@ __device__ __forceinline__ Xs load_x(const float *x, int j) {
         const int h = j >> 3, i = j & 7;
         first = 128 * h + 32 * (i >> 2) + 8 * (i & 3);
         apart = 64;
-    } else {
+    } else if constexpr (TYPE == JL_Q5_K) {
         first = 64 * (j >> 2) + 8 * (j & 3);
         apart = 32;
+    } else {
+        first = 32 * (j >> 1) + 8 * (j & 1);
+        apart = 16;
     }
     const float4 *xs = (const float4 *)(x + first);
     v.x[0] = xs[0];
@@ -100,7 +142,7 @@ __device__ __forceinline__ Xs load_x(const float *x, int j) {
     for (int g = 0; g < 2; g++) {
         const float4 p = v.x[2 * g], q = v.x[2 * g + 1];
         const float sum = ((p.x + p.y) + (p.z + p.w)) + ((q.x + q.y) + (q.z + q.w));
-        v.m32[g] = TYPE == JL_Q6_K ? -32.f * sum : sum;
+        v.m32[g] = TYPE == JL_Q6_K ? -32.f * sum : TYPE == JL_Q5_0 ? -16.f * sum : TYPE == JL_IQ4_XS ? -128.f * sum : sum;
     }
     return v;
 }
@@ -125,6 +167,34 @@ __device__ __forceinline__ float block_part(const Raw<TYPE> &r, const Xs &v, int
         const float lo = (dot4(lo0, v.x[0]) + dot4(lo1, v.x[1])) + v.m32[0];
         const float hi = (dot4(hi0, v.x[2]) + dot4(hi1, v.x[3])) + v.m32[1];
         return d * fmaf(sc_hi, hi, sc_lo * lo);
+    } else if constexpr (TYPE == JL_Q4_1) {
+        const float d = jl_half_bits_to_float(r.dm), m = jl_half_bits_to_float(r.dm >> 16);
+        const float lo = dot4(r.qs.lo & 0x0F0F0F0Fu, v.x[0]) + dot4(r.qs.hi & 0x0F0F0F0Fu, v.x[1]);
+        const float hi = dot4((r.qs.lo >> 4) & 0x0F0F0F0Fu, v.x[2]) + dot4((r.qs.hi >> 4) & 0x0F0F0F0Fu, v.x[3]);
+        return fmaf(d, lo + hi, m * (v.m32[0] + v.m32[1]));
+    } else if constexpr (TYPE == JL_Q5_0) {
+        // fifth bits: byte `half` of qh for the low-nibble eight, byte 2 + half for the high-nibble eight
+        const uint32_t bl = r.qh.v >> (8 * (j & 1)), bh = r.qh.v >> (16 + 8 * (j & 1));
+        const uint32_t lo0 = (r.qs.lo & 0x0F0F0F0Fu) | (jl_spread4(bl) << 4);
+        const uint32_t lo1 = (r.qs.hi & 0x0F0F0F0Fu) | (jl_spread4(bl >> 4) << 4);
+        const uint32_t hi0 = ((r.qs.lo >> 4) & 0x0F0F0F0Fu) | (jl_spread4(bh) << 4);
+        const uint32_t hi1 = ((r.qs.hi >> 4) & 0x0F0F0F0Fu) | (jl_spread4(bh >> 4) << 4);
+        const float lo = (dot4(lo0, v.x[0]) + dot4(lo1, v.x[1])) + v.m32[0];
+        const float hi = (dot4(hi0, v.x[2]) + dot4(hi1, v.x[3])) + v.m32[1];
+        return jl_half_bits_to_float(r.d) * (lo + hi);
+    } else if constexpr (TYPE == JL_IQ4_XS) {
+        const int g = j >> 1;
+        const uint32_t scales_h = r.hdr.x >> 16, scales_l = r.hdr.y;
+        const int ls = (int)(((scales_l >> (4 * g)) & 0xFu) | (((scales_h >> (2 * g)) & 3u) << 4));
+        const float dl = jl_half_bits_to_float(r.hdr.x) * (float)(ls - 32);
+        // table values with 128 added are bytes 1..241; the 128 comes off through m32
+        const uint32_t lo0 = jl_iq4nl_lookup4(r.qs.x & 0x0F0F0F0Fu) ^ 0x80808080u;
+        const uint32_t lo1 = jl_iq4nl_lookup4(r.qs.y & 0x0F0F0F0Fu) ^ 0x80808080u;
+        const uint32_t hi0 = jl_iq4nl_lookup4((r.qs.x >> 4) & 0x0F0F0F0Fu) ^ 0x80808080u;
+        const uint32_t hi1 = jl_iq4nl_lookup4((r.qs.y >> 4) & 0x0F0F0F0Fu) ^ 0x80808080u;
+        const float lo = (dot4(lo0, v.x[0]) + dot4(lo1, v.x[1])) + v.m32[0];
+        const float hi = (dot4(hi0, v.x[2]) + dot4(hi1, v.x[3])) + v.m32[1];
+        return dl * (lo + hi);
     } else {
         const int pair = j >> 2;
         const float d = jl_half_bits_to_float(r.hdr.x), dmin = jl_half_bits_to_float(r.hdr.x >> 16);
@@ -148,6 +218,10 @@ __device__ __forceinline__ float block_part(const Raw<TYPE> &r, const Xs &v, int
 template <int TYPE> struct Geometry;
 template <> struct Geometry<JL_Q6_K> { static constexpr int kBytes = 210; };
 template <> struct Geometry<JL_Q5_K> { static constexpr int kBytes = 176; };
+// bytes per 256 elements: eight blocks of Q4_1 / Q5_0, one super-block of IQ4_XS
+template <> struct Geometry<JL_Q4_1> { static constexpr int kBytes = 160; };
+template <> struct Geometry<JL_Q5_0> { static constexpr int kBytes = 176; };
+template <> struct Geometry<JL_IQ4_XS> { static constexpr int kBytes = 136; };
 
 template <int TYPE>
 __global__ void __launch_bounds__(256)
@@ -253,6 +327,38 @@ jl_dequant_q5_k(const uint8_t *__restrict__ w, float *__restrict__ out, int64_t 
     out[e] = __fsub_rn(t, __fmul_rn(dmin, (float)mn));
 }
 
+// J/tensor/standard/Q4_1FloatTensor.java:73-94: (nibble * d) + m, Q5_0FloatTensor.java:61-85:
+// d * (q - 16), IQ4_XSFloatTensor.java:72-100: (d * (ls - 32)) * kvalues[q]; one thread per element,
+// every operation rounded to fp32.
+template <int TYPE>
+__global__ void __launch_bounds__(256)
+jl_dequant_nibbles(const uint8_t *__restrict__ w, float *__restrict__ out, int64_t total) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    const int within = (int)(e & 31);       // position in the group of 32
+    const int byte_at = within & 15, shift = (within >> 4) * 4;
+    if constexpr (TYPE == JL_Q4_1) {
+        const uint8_t *blk = w + (e >> 5) * 20;
+        const uint32_t dm = *(const uint32_t *)blk;
+        const int q = (blk[4 + byte_at] >> shift) & 0xF;
+        out[e] = __fadd_rn(__fmul_rn((float)q, jl_half_bits_to_float(dm)), jl_half_bits_to_float(dm >> 16));
+    } else if constexpr (TYPE == JL_Q5_0) {
+        const uint8_t *blk = w + (e >> 5) * 22;
+        const uint32_t qh = blk[2] | (blk[3] << 8) | (blk[4] << 16) | ((uint32_t)blk[5] << 24);
+        const int q = ((blk[6 + byte_at] >> shift) & 0xF) | (int)(((qh >> within) & 1u) << 4);
+        out[e] = __fmul_rn(jl_half_bits_to_float(blk[0] | (blk[1] << 8)), (float)(q - 16));
+    } else {
+        const uint8_t *blk = w + (e >> 8) * 136;
+        const int g = (int)((e >> 5) & 7);
+        const uint2 hdr = *(const uint2 *)blk;
+        const int ls = (int)(((hdr.y >> (4 * g)) & 0xFu) | ((((hdr.x >> 16) >> (2 * g)) & 3u) << 4));
+        const float dl = __fmul_rn(jl_half_bits_to_float(hdr.x), (float)(ls - 32));
+        const uint32_t q = (blk[8 + 16 * g + byte_at] >> shift) & 0xFu;
+        const int kv = (int)(int8_t)(jl_iq4nl_lookup4(q) & 0xFFu);
+        out[e] = __fmul_rn(dl, (float)kv);
+    }
+}
+
 template <int TYPE>
 int launch_direct(jl_context *ctx, const jl_weight *w, const float *x, float *out, int epilogue) {
     const int rows = (int)w->rows, n = (int)w->cols;
@@ -279,15 +385,27 @@ int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const float *x, f
         return jl_fail(JL_ERR_UNSUPPORTED, "no %s projection kernel for a row length of %lld or an unaligned vector",
                        jl_type_name(w->type), (long long)w->cols);
     }
-    return w->type == JL_Q6_K ? launch_direct<JL_Q6_K>(ctx, w, x, out, epilogue)
-                              : launch_direct<JL_Q5_K>(ctx, w, x, out, epilogue);
+    switch (w->type) {
+        case JL_Q6_K: return launch_direct<JL_Q6_K>(ctx, w, x, out, epilogue);
+        case JL_Q5_K: return launch_direct<JL_Q5_K>(ctx, w, x, out, epilogue);
+        case JL_Q4_1: return launch_direct<JL_Q4_1>(ctx, w, x, out, epilogue);
+        case JL_Q5_0: return launch_direct<JL_Q5_0>(ctx, w, x, out, epilogue);
+        case JL_IQ4_XS: return launch_direct<JL_IQ4_XS>(ctx, w, x, out, epilogue);
+        default: return jl_fail(JL_ERR_UNSUPPORTED, "no projection kernel for a ggml type %d weight", w->type);
+    }
 }
 
 int jl_launch_dequant_direct(jl_context *ctx, const jl_weight *w, float *out) {
     const int64_t total = w->rows * w->cols;
     const dim3 g((unsigned)((total + 255) / 256)), b(256);
-    if (w->type == JL_Q6_K) hipLaunchKernelGGL(jl_dequant_q6_k, g, b, 0, ctx->stream, w->blocks, out, total);
-    else hipLaunchKernelGGL(jl_dequant_q5_k, g, b, 0, ctx->stream, w->blocks, out, total);
+    switch (w->type) {
+        case JL_Q6_K: hipLaunchKernelGGL(jl_dequant_q6_k, g, b, 0, ctx->stream, w->blocks, out, total); break;
+        case JL_Q5_K: hipLaunchKernelGGL(jl_dequant_q5_k, g, b, 0, ctx->stream, w->blocks, out, total); break;
+        case JL_Q4_1: hipLaunchKernelGGL(jl_dequant_nibbles<JL_Q4_1>, g, b, 0, ctx->stream, w->blocks, out, total); break;
+        case JL_Q5_0: hipLaunchKernelGGL(jl_dequant_nibbles<JL_Q5_0>, g, b, 0, ctx->stream, w->blocks, out, total); break;
+        case JL_IQ4_XS: hipLaunchKernelGGL(jl_dequant_nibbles<JL_IQ4_XS>, g, b, 0, ctx->stream, w->blocks, out, total); break;
+        default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_dequant_f32: no decode kernel for ggml type %d", w->type);
+    }
     JL_HIP(hipGetLastError());
     return JL_OK;
 }

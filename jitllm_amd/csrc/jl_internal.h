@@ -30,16 +30,40 @@ struct jl_weight {
 
 // Block geometry (reference: J/format/GGMLType.java:7,13,18-20).
 static inline int jl_block_elems(int type) {
-    return (type == JL_Q4_K || type == JL_Q6_K || type == JL_Q5_K) ? 256 : (type == JL_Q8_0 || type == JL_Q4_0) ? 32 : 0;
+    switch (type) {
+        case JL_Q4_K: case JL_Q5_K: case JL_Q6_K: case JL_IQ4_XS: return 256;
+        case JL_Q8_0: case JL_Q4_0: case JL_Q4_1: case JL_Q5_0: return 32;
+        default: return 0;
+    }
 }
 static inline int jl_block_bytes(int type) {
-    return type == JL_Q4_K ? 144 : type == JL_Q6_K ? 210 : type == JL_Q5_K ? 176 : type == JL_Q8_0 ? 34 : type == JL_Q4_0 ? 18 : 0;
+    switch (type) {
+        case JL_Q4_0: return 18;
+        case JL_Q4_1: return 20;
+        case JL_Q5_0: return 22;
+        case JL_Q8_0: return 34;
+        case JL_Q4_K: return 144;
+        case JL_Q5_K: return 176;
+        case JL_Q6_K: return 210;
+        case JL_IQ4_XS: return 136;
+        default: return 0;
+    }
 }
 static inline const char *jl_type_name(int type) {
-    return type == JL_Q4_K ? "Q4_K" : type == JL_Q6_K ? "Q6_K" : type == JL_Q5_K ? "Q5_K" : type == JL_Q8_0 ? "Q8_0" : type == JL_Q4_0 ? "Q4_0" : "?";
+    switch (type) {
+        case JL_Q4_0: return "Q4_0";
+        case JL_Q4_1: return "Q4_1";
+        case JL_Q5_0: return "Q5_0";
+        case JL_Q8_0: return "Q8_0";
+        case JL_Q4_K: return "Q4_K";
+        case JL_Q5_K: return "Q5_K";
+        case JL_Q6_K: return "Q6_K";
+        case JL_IQ4_XS: return "IQ4_XS";
+        default: return "?";
+    }
 }
-// Q8_0, Q4_0 and Q4_K have the whole kernel family; Q6_K and Q5_K the plain single-token
-// projection and the decode-once batched path.
+// Q8_0, Q4_0 and Q4_K have the whole kernel family; Q4_1, Q5_0, Q5_K, Q6_K and IQ4_XS the plain
+// single-token projection and the decode-once batched path.
 static inline bool jl_has_fused_kernels(int type) {
     return type == JL_Q8_0 || type == JL_Q4_0 || type == JL_Q4_K;
 }

@@ -12,10 +12,13 @@ import enum
 
 class GGMLType(enum.IntEnum):
     Q4_0 = 2
+    Q4_1 = 3    # plain single-token projection and the decode-once batched path
+    Q5_0 = 6    # likewise
     Q8_0 = 8
     Q4_K = 12
     Q5_K = 13   # plain single-token projection and the decode-once batched path
     Q6_K = 14   # likewise
+    IQ4_XS = 23  # likewise
 
     @property
     def block_elems(self) -> int:
@@ -38,6 +41,9 @@ class GGMLType(enum.IntEnum):
 
 _GEOMETRY = {
     GGMLType.Q4_0: (32, 18),
+    GGMLType.Q4_1: (32, 20),
+    GGMLType.Q5_0: (32, 22),
+    GGMLType.IQ4_XS: (256, 136),
     GGMLType.Q8_0: (32, 34),
     GGMLType.Q4_K: (256, 144),
     GGMLType.Q5_K: (256, 176),

@@ -248,7 +248,7 @@ class Implementation:
         return self.create(steps, target, context, prepacking)
 
 
-SUPPORTED = frozenset({GGMLType.Q8_0, GGMLType.Q4_0, GGMLType.Q4_K, GGMLType.Q5_K, GGMLType.Q6_K})
+SUPPORTED = frozenset(GGMLType)
 
 
 def _sizes(steps: Sequence[Step]):

@@ -6,6 +6,11 @@ Block value distributions:
   Q4_K  fp16 d ~ U(1e-3, 2e-2)/63, fp16 dmin ~ U(1e-3, 2e-2)*8/63 per super-block (so the largest
         weight magnitude d*63*15 stays near 0.3 and the minimum term roughly centres the range),
         8 (scale, min) pairs ~ U{0..63} packed into the 12 scale bytes, 128 bytes of nibbles
+  Q4_1  fp16 d ~ U(1e-3, 2e-2), fp16 m = -7.5 d * U(0.5, 1.5) per block (the minimum roughly centres
+        the range), 16 bytes of nibbles
+  Q5_0  fp16 d ~ U(5e-4, 1e-2) per block, 4 bytes of fifth bits, 16 bytes of nibbles
+  IQ4_XS fp16 d ~ U(2e-5, 1e-4) per super-block (largest weight d*31*127 near 0.4), 8 six-bit group
+        scales split over scales_h / scales_l, 128 bytes of nibbles
   Q5_K  as Q4_K with d and dmin halved (values reach 31), plus 32 bytes of fifth bits
   Q6_K  fp16 d ~ U(2e-5, 1e-4) per super-block (largest weight d*127*32 near 0.4), 16 signed
         scales ~ U{-128..127}, 128 + 64 bytes of quant bits
@@ -48,6 +53,18 @@ def weight(t: GGMLType, rows: int, cols: int, seed: int) -> np.ndarray:
     elif t == GGMLType.Q4_0:
         raw[:, 0:2] = _scales_f16(rng, blocks, 1e-3, 2e-2).view(np.uint8).reshape(blocks, 2)
         raw[:, 2:] = rng.integers(0, 256, size=(blocks, 16), dtype=np.uint8)
+    elif t == GGMLType.Q4_1:
+        d = rng.uniform(1e-3, 2e-2, size=blocks).astype(np.float32)
+        m = (-7.5 * d * rng.uniform(0.5, 1.5, size=blocks)).astype(np.float32)
+        raw[:, 0:2] = d.astype(np.float16).view(np.uint16).view(np.uint8).reshape(blocks, 2)
+        raw[:, 2:4] = m.astype(np.float16).view(np.uint16).view(np.uint8).reshape(blocks, 2)
+        raw[:, 4:] = rng.integers(0, 256, size=(blocks, 16), dtype=np.uint8)
+    elif t == GGMLType.Q5_0:
+        raw[:, 0:2] = _scales_f16(rng, blocks, 5e-4, 1e-2).view(np.uint8).reshape(blocks, 2)
+        raw[:, 2:] = rng.integers(0, 256, size=(blocks, 20), dtype=np.uint8)
+    elif t == GGMLType.IQ4_XS:
+        raw[:, 0:2] = _scales_f16(rng, blocks, 2e-5, 1e-4).view(np.uint8).reshape(blocks, 2)
+        raw[:, 2:] = rng.integers(0, 256, size=(blocks, 134), dtype=np.uint8)
     elif t == GGMLType.Q5_K:
         raw[:, 0:2] = _scales_f16(rng, blocks, 5e-4 / 63, 1e-2 / 63).view(np.uint8).reshape(blocks, 2)
         raw[:, 2:4] = _scales_f16(rng, blocks, 8e-3 / 63, 16e-2 / 63).view(np.uint8).reshape(blocks, 2)

@@ -19,6 +19,10 @@
  *                              zero is used here (what the JDK's own fallback does) and the result
  *                              is held to a few ulp, not bit equality: "parity unpinned" for the
  *                              last bits of that one addition chain only.
+ *   Q4_1, Q5_0, IQ4_XS         decode: the reference's own known answers (Q4_1FloatTensorTest,
+ *                              QuantizedDeviceDecodeParityTest q5_0 / iq4_XS ReadsGgmlsLayout), second
+ *                              wordings, numpy statements of ggml's dequantize_row_*; dots: Q4_1 lane
+ *                              model as above, Q5_0 / IQ4_XS block sums bit-equal to a numpy loop.
  *   rmsnorm, argmax            closed forms (constant vectors, powers of two, eps-dominated input), a
  *                              float64 evaluation, numpy's argmax with ties, -inf and NaN cases.
  *   java.util.Random           published first outputs for seeds 0 and 42.
@@ -37,6 +41,9 @@
 #define Q4_K_BYTES 144
 #define Q6_K_BYTES 210
 #define Q5_K_BYTES 176
+#define Q4_1_BYTES 20
+#define Q5_0_BYTES 22
+#define IQ4_XS_BYTES 136
 
 int jo_max_threads(void) { return omp_get_max_threads(); }
 
@@ -48,6 +55,9 @@ int jo_block_elems(int type) {
         case JO_Q4_K: return QK_K;
         case JO_Q6_K: return QK_K;
         case JO_Q5_K: return QK_K;
+        case JO_Q4_1: return Q_BLOCK;
+        case JO_Q5_0: return Q_BLOCK;
+        case JO_IQ4_XS: return QK_K;
         default: return 0;
     }
 }
@@ -59,6 +69,9 @@ int jo_block_bytes(int type) {
         case JO_Q4_K: return Q4_K_BYTES;
         case JO_Q6_K: return Q6_K_BYTES;
         case JO_Q5_K: return Q5_K_BYTES;
+        case JO_Q4_1: return Q4_1_BYTES;
+        case JO_Q5_0: return Q5_0_BYTES;
+        case JO_IQ4_XS: return IQ4_XS_BYTES;
         default: return 0;
     }
 }
@@ -244,8 +257,75 @@ static inline float q5_k_get(const uint8_t *w, int64_t index) {
     return t - u;
 }
 
+/*
+ * J/tensor/standard/Q4_1FloatTensor.java:73-94.  fp16 d | fp16 m | 16 nibble bytes: element i < 16 is
+ * the low nibble of byte i, element i >= 16 the high nibble of byte i - 16; w = nibble * d + m,
+ * product rounded, then the sum (the nibble is never recentred).
+ */
+static inline float q4_1_get(const uint8_t *w, int64_t index) {
+    const uint8_t *blk = w + (index / Q_BLOCK) * Q4_1_BYTES;
+    int within = (int)(index % Q_BLOCK);
+    float scale = jo_f16_to_f32(read_u16(blk));
+    float min = jo_f16_to_f32(read_u16(blk + 2));
+    int nibble = within < 16 ? (blk[4 + within] & 0x0F) : ((blk[4 + within - 16] >> 4) & 0x0F);
+    float t = (float)nibble * scale;
+    return t + min;
+}
+
+/*
+ * J/tensor/standard/Q5_0FloatTensor.java:61-85.  fp16 d | 32 fifth bits (little-endian word, bit i
+ * belongs to element i) | 16 nibble bytes laid out as Q4_0's; w = d * (q - 16).
+ */
+static inline float q5_0_decode(const uint8_t *blk, float scale, uint32_t qh, int within) {
+    int half = within / 16;
+    int packed = blk[6 + within - half * 16];
+    int q = ((packed >> (half * 4)) & 0x0F) | (int)(((qh >> within) & 1u) << 4);
+    return scale * (float)(q - 16);
+}
+
+static inline uint32_t q5_0_high_bits(const uint8_t *blk) {
+    return (uint32_t)blk[2] | ((uint32_t)blk[3] << 8) | ((uint32_t)blk[4] << 16) | ((uint32_t)blk[5] << 24);
+}
+
+static inline float q5_0_get(const uint8_t *w, int64_t index) {
+    const uint8_t *blk = w + (index / Q_BLOCK) * Q5_0_BYTES;
+    return q5_0_decode(blk, jo_f16_to_f32(read_u16(blk)), q5_0_high_bits(blk), (int)(index % Q_BLOCK));
+}
+
+/*
+ * J/tensor/standard/IQ4_XSFloatTensor.java:27-100.  fp16 d | 16 bits scales_h (two high bits of
+ * each of the 8 group scales, group g at bit 2 g) | 4 bytes scales_l (low four bits, group g in
+ * byte g / 2) | 128 nibble bytes, 16 per group of 32 (elements 0..15 low nibbles, 16..31 high);
+ * w = (d * (ls - 32)) * kvalues_iq4nl[nibble].
+ */
+static const int8_t IQ4NL_VALUES[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+static inline float iq4_xs_group_scale(const uint8_t *blk, float d, int g) {
+    int scales_h = read_u16(blk + 2);
+    int low = blk[4 + g / 2];
+    int ls = ((low >> (4 * (g % 2))) & 0xF) | (((scales_h >> (2 * g)) & 3) << 4);
+    return d * (float)(ls - 32);
+}
+
+static inline float iq4_xs_decode(const uint8_t *blk, float dl, int g, int within) {
+    int half = within / 16;
+    int packed = blk[8 + g * 16 + within - half * 16];
+    return dl * (float)IQ4NL_VALUES[(packed >> (half * 4)) & 0xF];
+}
+
+static inline float iq4_xs_get(const uint8_t *w, int64_t index) {
+    const uint8_t *blk = w + (index / QK_K) * IQ4_XS_BYTES;
+    int within_block = (int)(index % QK_K);
+    int g = within_block / 32;
+    float d = jo_f16_to_f32(read_u16(blk));
+    return iq4_xs_decode(blk, iq4_xs_group_scale(blk, d, g), g, within_block % 32);
+}
+
 float jo_get_float(int type, const uint8_t *w, int64_t index) {
     switch (type) {
+        case JO_Q4_1: return q4_1_get(w, index);
+        case JO_Q5_0: return q5_0_get(w, index);
+        case JO_IQ4_XS: return iq4_xs_get(w, index);
         case JO_Q8_0: return q8_0_get(w, index);
         case JO_Q4_0: return q4_0_get(w, index);
         case JO_Q4_K: return q4_k_get(w, index);
@@ -340,6 +420,48 @@ float jo_get_float_alt(int type, const uint8_t *w, int64_t index) {
         float b = dmin * (float)m;
         return a - b;
     }
+    if (type == JO_Q4_1) {
+        /* J/backend/tornado/kernels/TransformerComputeKernelsQ4_1.java:59-67 */
+        const uint8_t *blk = w + (index / 32) * Q4_1_BYTES;
+        int within = (int)(index % 32);
+        float d = jo_f16_to_f32(read_u16(blk));
+        float m = jo_f16_to_f32(read_u16(blk + 2));
+        int half = within / 16;
+        int packed = blk[4 + (within - half * 16)] & 0xFF;
+        int q = (half == 0) ? (packed & 0xF) : ((packed >> 4) & 0xF);
+        float a = d * (float)q;
+        return a + m;
+    }
+    if (type == JO_Q5_0) {
+        /* J/backend/tornado/kernels/TransformerComputeKernelsQ5_0.java:56-70: the fifth bits are
+           read as two 16-bit halves */
+        const uint8_t *blk = w + (index / 32) * Q5_0_BYTES;
+        int within = (int)(index % 32);
+        float d = jo_f16_to_f32(read_u16(blk));
+        uint32_t qh = (uint32_t)read_u16(blk + 2) | ((uint32_t)read_u16(blk + 4) << 16);
+        int half = within / 16;
+        int packed = blk[6 + within - half * 16] & 0xFF;
+        int q = ((packed >> (half * 4)) & 0xF) | (int)(((qh >> within) & 1u) << 4);
+        return d * (float)(q - 16);
+    }
+    if (type == JO_IQ4_XS) {
+        /* J/backend/tornado/kernels/TransformerComputeKernelsIQ4_XS.java:62-96: the table as four
+           little-endian words of four signed bytes */
+        const uint8_t *blk = w + (index / 256) * IQ4_XS_BYTES;
+        int within_block = (int)(index % 256);
+        int g = within_block >> 5;
+        int within = within_block & 31;
+        int half = within >> 4;
+        int packed = blk[8 + (g << 4) + (within & 15)] & 0xFF;
+        int scales_h = read_u16(blk + 2);
+        int low = blk[4 + (g >> 1)] & 0xFF;
+        int ls = ((low >> ((g & 1) << 2)) & 0xF) | (((scales_h >> (g << 1)) & 3) << 4);
+        float dl = jo_f16_to_f32(read_u16(blk)) * (float)(ls - 32);
+        int q = (packed >> (half << 2)) & 0xF;
+        uint32_t word = q < 8 ? (q < 4 ? 0xBFAD9881u : 0xF6EADDCFu) : (q < 12 ? 0x26190D01u : 0x71594535u);
+        int kvalue = (int)(int8_t)(word >> ((q & 3) << 3));
+        return dl * (float)kvalue;
+    }
     if (type == JO_Q6_K) {
         /* J/backend/tornado/kernels/TransformerComputeKernelsQ6_K.java:195-232 */
         const uint8_t *blk = w + (index / 256) * Q6_K_BYTES;
@@ -393,6 +515,24 @@ static float scalar_dot(int type, const uint8_t *w, int64_t this_offset, const f
         case JO_Q5_K:   /* Q5_KFloatTensor.dot is scalarDot */
             for (int64_t j = 0; j < size; j++) {
                 float p = q5_k_get(w, this_offset + j) * x[that_offset + j];
+                result += p;
+            }
+            break;
+        case JO_Q4_1:
+            for (int64_t j = 0; j < size; j++) {
+                float p = q4_1_get(w, this_offset + j) * x[that_offset + j];
+                result += p;
+            }
+            break;
+        case JO_Q5_0:
+            for (int64_t j = 0; j < size; j++) {
+                float p = q5_0_get(w, this_offset + j) * x[that_offset + j];
+                result += p;
+            }
+            break;
+        case JO_IQ4_XS:
+            for (int64_t j = 0; j < size; j++) {
+                float p = iq4_xs_get(w, this_offset + j) * x[that_offset + j];
                 result += p;
             }
             break;
@@ -456,6 +596,42 @@ block_step_128(const float *wf, const float *x, float d, float *val) {
     }
 }
 
+/*
+ * Q4_1's block step (J/tensor/standard/Q4_1FloatTensor.java:141-182): the same four products, summed
+ * left to right, scaled into val by d; then the four activation slices, summed left to right,
+ * scaled into val by the block's minimum.
+ */
+static inline __attribute__((always_inline)) void
+block_step_256_affine(const float *wf, const float *x, float d, float m, float *val) {
+    for (int l = 0; l < 8; l++) {
+        float products = ((x[l] * wf[l] + x[8 + l] * wf[8 + l]) + x[16 + l] * wf[16 + l]) + x[24 + l] * wf[24 + l];
+        float activations = ((x[l] + x[8 + l]) + x[16 + l]) + x[24 + l];
+        val[l] = fmaf(products, d, val[l]);
+        val[l] = fmaf(activations, m, val[l]);
+    }
+}
+
+static inline __attribute__((always_inline)) void
+block_step_128_affine(const float *wf, const float *x, float d, float m, float *val) {
+    for (int i = 0; i < 2; i++) {
+        const float *wh = wf + 16 * i;
+        const float *xh = x + 16 * i;
+        for (int l = 0; l < 4; l++) {
+            float products = ((xh[l] * wh[l] + xh[4 + l] * wh[4 + l]) + xh[8 + l] * wh[8 + l]) + xh[12 + l] * wh[12 + l];
+            float activations = ((xh[l] + xh[4 + l]) + xh[8 + l]) + xh[12 + l];
+            val[l] = fmaf(products, d, val[l]);
+            val[l] = fmaf(activations, m, val[l]);
+        }
+    }
+}
+
+static inline __attribute__((always_inline)) void widen_q4_1(const uint8_t *blk, float *wf) {
+    for (int i = 0; i < 16; i++) {
+        wf[i] = (float)(blk[4 + i] & 0xF);       /* unsigned nibbles: no recentring */
+        wf[16 + i] = (float)(blk[4 + i] >> 4);
+    }
+}
+
 static inline __attribute__((always_inline)) void widen_q8_0(const uint8_t *blk, float *wf) {
     for (int i = 0; i < 32; i++) wf[i] = (float)(int8_t)blk[2 + i];
 }
@@ -470,11 +646,11 @@ static inline __attribute__((always_inline)) void widen_q4_0(const uint8_t *blk,
     }
 }
 
-/* J/tensor/standard/Q8_0FloatTensor.java:142-229 and Q4_0FloatTensor.java:90-174 */
+/* J/tensor/standard/Q8_0FloatTensor.java:142-229, Q4_0FloatTensor.java:90-174, Q4_1FloatTensor.java:105-192 */
 static inline __attribute__((always_inline)) float
 vector_dot_body(int type, int bits, const uint8_t *w, int64_t this_offset, const float *x,
            int64_t that_offset, int64_t size) {
-    const int block_bytes = (type == JO_Q8_0) ? Q8_0_BYTES : Q4_0_BYTES;
+    const int block_bytes = (type == JO_Q8_0) ? Q8_0_BYTES : (type == JO_Q4_1) ? Q4_1_BYTES : Q4_0_BYTES;
     float result = 0.0f;
     int64_t j = 0;
     int64_t alignment_bound = (-this_offset) & (Q_BLOCK - 1);
@@ -492,6 +668,13 @@ vector_dot_body(int type, int bits, const uint8_t *w, int64_t this_offset, const
     for (; j < upper_bound && j + Q_BLOCK <= size; j += Q_BLOCK, block_offset += block_bytes) {
         const uint8_t *blk = w + block_offset;
         float d = jo_f16_to_f32(read_u16(blk));
+        if (type == JO_Q4_1) {
+            float m = jo_f16_to_f32(read_u16(blk + 2));
+            widen_q4_1(blk, wf);
+            if (bits == 256) block_step_256_affine(wf, x + that_offset + j, d, m, val);
+            else block_step_128_affine(wf, x + that_offset + j, d, m, val);
+            continue;
+        }
         if (type == JO_Q8_0) widen_q8_0(blk, wf); else widen_q4_0(blk, wf);
         if (bits == 256) block_step_256(wf, x + that_offset + j, d, val);
         else block_step_128(wf, x + that_offset + j, d, val);
@@ -524,6 +707,52 @@ static float vector_dot(int type, int bits, const uint8_t *w, int64_t this_offse
 }
 
 /*
+ * Q5_0FloatTensor.dot (J/tensor/standard/Q5_0FloatTensor.java:87-112) and IQ4_XSFloatTensor.dot
+ * (IQ4_XSFloatTensor.java:102-126): no vector kernel, but not scalarDot either -- a block's (Q5_0)
+ * or a group's (IQ4_XS) 32 products are summed on their own from zero and that sum is added to the
+ * result; elements before the first whole block and after the last one go through scalarDot.
+ */
+static float block_sum_dot(int type, const uint8_t *w, int64_t this_offset, const float *x,
+                           int64_t that_offset, int64_t size) {
+    const int elems = (type == JO_Q5_0) ? Q_BLOCK : QK_K;
+    const int bytes = (type == JO_Q5_0) ? Q5_0_BYTES : IQ4_XS_BYTES;
+    float result = 0.0f;
+    int64_t j = 0;
+    int64_t alignment_bound = (-this_offset) & (elems - 1);
+    if (alignment_bound > size) alignment_bound = size;
+    if (alignment_bound > 0) {
+        result += scalar_dot(type, w, this_offset, x, that_offset, alignment_bound);
+        j += alignment_bound;
+    }
+    int64_t block_offset = (this_offset + j) / elems * bytes;
+    for (; j + elems <= size; j += elems, block_offset += bytes) {
+        const uint8_t *blk = w + block_offset;
+        float d = jo_f16_to_f32(read_u16(blk));
+        if (type == JO_Q5_0) {
+            uint32_t qh = q5_0_high_bits(blk);
+            float block = 0.0f;
+            for (int i = 0; i < Q_BLOCK; i++) {
+                float p = q5_0_decode(blk, d, qh, i) * x[that_offset + j + i];
+                block += p;
+            }
+            result += block;
+        } else {
+            for (int g = 0; g < QK_K / 32; g++) {
+                float dl = iq4_xs_group_scale(blk, d, g);
+                float group = 0.0f;
+                for (int i = 0; i < 32; i++) {
+                    float p = iq4_xs_decode(blk, dl, g, i) * x[that_offset + j + g * 32 + i];
+                    group += p;
+                }
+                result += group;
+            }
+        }
+    }
+    if (j < size) result += scalar_dot(type, w, this_offset + j, x, that_offset + j, size - j);
+    return result;
+}
+
+/*
  * Q8_0FloatTensor.dot (J/tensor/standard/Q8_0FloatTensor.java:89-99), Q4_0FloatTensor.dot
  * (Q4_0FloatTensor.java:82-88), Q4_KFloatTensor.dot (Q4_KFloatTensor.java:124-127).  The flavour
  * is the branch a JVM would take: vector kernels exist for 128- and 256-bit species only
@@ -531,7 +760,9 @@ static float vector_dot(int type, int bits, const uint8_t *w, int64_t this_offse
  */
 float jo_dot(int type, int flavour, const uint8_t *w, int64_t this_offset, const float *x,
              int64_t that_offset, int64_t size) {
-    if (type != JO_Q4_K && type != JO_Q6_K && type != JO_Q5_K && (flavour == JO_DOT_VEC128 || flavour == JO_DOT_VEC256)) {
+    /* Q5_0 and IQ4_XS have one dot for every JVM (the flavour only matters to the vector kernels) */
+    if (type == JO_Q5_0 || type == JO_IQ4_XS) return block_sum_dot(type, w, this_offset, x, that_offset, size);
+    if ((type == JO_Q8_0 || type == JO_Q4_0 || type == JO_Q4_1) && (flavour == JO_DOT_VEC128 || flavour == JO_DOT_VEC256)) {
         return vector_dot(type, flavour, w, this_offset, x, that_offset, size);
     }
     return scalar_dot(type, w, this_offset, x, that_offset, size);

@@ -18,7 +18,7 @@ extern "C" {
 #endif
 
 /* ggml type ids, the numbering GGUF files carry (J/format/GGMLType.java:7,13,18 by ordinal). */
-enum { JO_Q4_0 = 2, JO_Q8_0 = 8, JO_Q4_K = 12, JO_Q5_K = 13, JO_Q6_K = 14 };
+enum { JO_Q4_0 = 2, JO_Q4_1 = 3, JO_Q5_0 = 6, JO_Q8_0 = 8, JO_Q4_K = 12, JO_Q5_K = 13, JO_Q6_K = 14, JO_IQ4_XS = 23 };
 
 /* dot flavours: which branch of Q8_0FloatTensor.dot / Q4_0FloatTensor.dot runs. */
 enum { JO_DOT_SCALAR = 0, JO_DOT_VEC128 = 128, JO_DOT_VEC256 = 256 };

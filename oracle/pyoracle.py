@@ -13,6 +13,7 @@ import subprocess
 import numpy as np
 
 Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
+Q4_1, Q5_0, IQ4_XS = 3, 6, 23
 DOT_SCALAR, DOT_VEC128, DOT_VEC256 = 0, 128, 256
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -227,6 +228,10 @@ class JavaRandom:
         if bound is None:
             return lib().jo_jrandom_next_int(C.byref(self._s))
         return lib().jo_jrandom_next_int_bound(C.byref(self._s), bound)
+
+    def next_float(self) -> float:
+        """``next(24) / (float)(1 << 24)``: the top 24 of the 32 bits ``nextInt()`` would return."""
+        return ((self.next_int() & 0xFFFFFFFF) >> 8) / float(1 << 24)
 
     def next_boolean(self) -> bool:
         return bool(lib().jo_jrandom_next_boolean(C.byref(self._s)))

@@ -15,8 +15,10 @@ N_PROBE, D_PROBE = 512, 37  # T/backend/tornado/kernels/NativeQuantizedKernelAcc
 SPECIAL_HALVES = [0x0000, 0x8000, 0x0001, 0x03FF, 0x3C00, 0xBC00, 0x7BFF, 0xFBFF]
 PAYLOAD_PATTERNS = [0x00, 0xFF, 0xAA, 0x55]
 
-SCALE_OFFSETS = {O.Q4_0: [0], O.Q8_0: [0], O.Q4_K: [0, 2], O.Q5_K: [0, 2], O.Q6_K: [208]}
-TYPE_NAMES = {O.Q4_0: "Q4_0", O.Q8_0: "Q8_0", O.Q4_K: "Q4_K", O.Q5_K: "Q5_K", O.Q6_K: "Q6_K"}
+SCALE_OFFSETS = {O.Q4_0: [0], O.Q8_0: [0], O.Q4_K: [0, 2], O.Q5_K: [0, 2], O.Q6_K: [208],
+                 O.Q4_1: [0, 2], O.Q5_0: [0], O.IQ4_XS: [0]}
+TYPE_NAMES = {O.Q4_0: "Q4_0", O.Q8_0: "Q8_0", O.Q4_K: "Q4_K", O.Q5_K: "Q5_K", O.Q6_K: "Q6_K",
+              O.Q4_1: "Q4_1", O.Q5_0: "Q5_0", O.IQ4_XS: "IQ4_XS"}
 
 
 def random_bytes(seed: int, n: int) -> np.ndarray:

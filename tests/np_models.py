@@ -109,7 +109,55 @@ def dequant_q6_k(raw: np.ndarray) -> np.ndarray:
     return out.reshape(-1)
 
 
-DEQUANT = {8: dequant_q8_0, 2: dequant_q4_0, 12: dequant_q4_k, 13: dequant_q5_k, 14: dequant_q6_k}
+def dequant_q4_1(raw: np.ndarray) -> np.ndarray:
+    """ggml's dequantize_row_q4_1: y[j] = (qs[j] & 0xF) * d + m, y[j + 16] = (qs[j] >> 4) * d + m."""
+    b = raw.reshape(-1, 20)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    m = half_bits_to_f32(b[:, 2:4].copy().view(np.uint16)[:, 0])
+    q = np.concatenate([b[:, 4:] & 0x0F, b[:, 4:] >> 4], axis=1).astype(np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        return ((q * d[:, None]).astype(np.float32) + m[:, None]).astype(np.float32).reshape(-1)
+
+
+def dequant_q5_0(raw: np.ndarray) -> np.ndarray:
+    """ggml's dequantize_row_q5_0: qh is a little-endian 32-bit word; y[j] takes bit j of it as its
+    fifth bit and the low nibble of qs[j], y[j + 16] bit j + 16 and the high nibble; w = (q - 16) d."""
+    b = raw.reshape(-1, 22)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    qh = b[:, 2:6].copy().view("<u4")[:, 0].astype(np.int64)
+    bits = (qh[:, None] >> np.arange(32)[None, :]) & 1
+    nib = np.concatenate([b[:, 6:] & 0x0F, b[:, 6:] >> 4], axis=1).astype(np.int64)
+    q = ((nib | (bits << 4)) - 16).astype(np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        return (d[:, None] * q).astype(np.float32).reshape(-1)
+
+
+KVALUES_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113],
+                         dtype=np.float32)
+
+
+def dequant_iq4_xs(raw: np.ndarray) -> np.ndarray:
+    """ggml's dequantize_row_iq4_xs: for group ib of 32, ls = low four bits from scales_l[ib / 2]
+    (nibble ib % 2) | two bits of scales_h at 2 ib << 4, dl = d * (ls - 32); y[j] = dl *
+    kvalues_iq4nl[qs[j] & 0xF], y[j + 16] = dl * kvalues_iq4nl[qs[j] >> 4] over the group's 16 bytes."""
+    b = raw.reshape(-1, 136)
+    nb = b.shape[0]
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    scales_h = b[:, 2:4].copy().view("<u2")[:, 0].astype(np.int32)
+    scales_l = b[:, 4:8].astype(np.int32)
+    qs = b[:, 8:].reshape(nb, 8, 16)
+    out = np.empty((nb, 8, 32), dtype=np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        for ib in range(8):
+            ls = ((scales_l[:, ib // 2] >> (4 * (ib % 2))) & 0xF) | (((scales_h >> (2 * ib)) & 3) << 4)
+            dl = (d * (ls - 32).astype(np.float32)).astype(np.float32)
+            out[:, ib, 0:16] = (dl[:, None] * KVALUES_IQ4NL[qs[:, ib, :] & 0xF]).astype(np.float32)
+            out[:, ib, 16:32] = (dl[:, None] * KVALUES_IQ4NL[qs[:, ib, :] >> 4]).astype(np.float32)
+    return out.reshape(-1)
+
+
+DEQUANT = {8: dequant_q8_0, 2: dequant_q4_0, 12: dequant_q4_k, 13: dequant_q5_k, 14: dequant_q6_k,
+           3: dequant_q4_1, 6: dequant_q5_0, 23: dequant_iq4_xs}
 
 
 def scalar_dot_rows(w_deq: np.ndarray, x: np.ndarray) -> np.ndarray:
@@ -130,9 +178,14 @@ def _fma32(a: np.ndarray, b: np.ndarray, c: np.ndarray) -> np.ndarray:
 
 def vector_lane_values(t: int, raw: np.ndarray, x: np.ndarray, bits: int) -> np.ndarray:
     """Lane accumulators of the reference's vector dot for one row, before reduceLanes."""
+    m = None
     if t == 8:
         b = raw.reshape(-1, 34)
         wf = b[:, 2:].view(np.int8).astype(np.float32)
+    elif t == 3:
+        b = raw.reshape(-1, 20)
+        wf = np.concatenate([b[:, 4:] & 0xF, b[:, 4:] >> 4], axis=1).astype(np.float32)
+        m = half_bits_to_f32(b[:, 2:4].copy().view(np.uint16)[:, 0])
     else:
         b = raw.reshape(-1, 18)
         qs = b[:, 2:]
@@ -149,4 +202,22 @@ def vector_lane_values(t: int, raw: np.ndarray, x: np.ndarray, bits: int) -> np.
             s = ((p[0] + p[1]).astype(np.float32) + p[2]).astype(np.float32)
             s = (s + p[3]).astype(np.float32)
             val = _fma32(s, np.full(lanes, d[k], dtype=np.float32), val)
+            if m is not None:   # Q4_1: the activation slices, summed the same way, times the minimum
+                a = xb[k, lo:hi].reshape(4, lanes)
+                sa = ((a[0] + a[1]).astype(np.float32) + a[2]).astype(np.float32)
+                sa = (sa + a[3]).astype(np.float32)
+                val = _fma32(sa, np.full(lanes, m[k], dtype=np.float32), val)
     return val
+
+
+def block_sum_dot_rows(w_deq: np.ndarray, x: np.ndarray, group: int = 32) -> np.ndarray:
+    """Rows of ``w_deq`` [d x n] times ``x``: each run of ``group`` products summed sequentially in
+    float32 from zero, the runs' sums added sequentially to the result."""
+    d, n = w_deq.shape
+    acc = np.zeros(d, dtype=np.float32)
+    for g in range(n // group):
+        part = np.zeros(d, dtype=np.float32)
+        for j in range(g * group, (g + 1) * group):
+            part = (part + (w_deq[:, j] * x[j]).astype(np.float32)).astype(np.float32)
+        acc = (acc + part).astype(np.float32)
+    return acc

@@ -260,10 +260,10 @@ def test_two_pass_prefill_qkv_and_gate_up(ctx):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
 
 
-@pytest.mark.parametrize("t", [O.Q5_K, O.Q6_K])
+@pytest.mark.parametrize("t", [O.Q5_K, O.Q6_K, O.Q4_1, O.Q5_0, O.IQ4_XS])
 @pytest.mark.parametrize("d,n,T,residual", [(300, 512, 8, False), (1000, 2048, 100, True), (4096, 256, 600, False)])
 def test_k_quant_batched_rows_take_the_decode_once_path(ctx, t, d, n, T, residual):
-    """A Q6_K / Q5_K weight has no decode-in-the-loop kernel: every batched call decodes it to fp16 into
+    """A Q6_K / Q5_K / Q4_1 / Q5_0 / IQ4_XS weight has no decode-in-the-loop kernel: every batched call decodes it to fp16 into
     the workspace and runs the fp16 GEMM, few rows or many; partial batches leave the rest alone."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections

@@ -180,23 +180,23 @@ def test_fused_gate_up(ctx, t, d, n):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + 1e-6)
 
 
-# ---- Q6_K and Q5_K: decode and the plain single-token projection ------------------------------
+# ---- Q6_K, Q5_K, Q4_1, Q5_0, IQ4_XS: decode and the plain single-token projection --------------
 
-KQ = [O.Q5_K, O.Q6_K]
-KQ_NAMES = {O.Q5_K: "Q5_K", O.Q6_K: "Q6_K"}
+KQ = [O.Q5_K, O.Q6_K, O.Q4_1, O.Q5_0, O.IQ4_XS]
+KQ_NAMES = FX.TYPE_NAMES
 
 
 @pytest.mark.parametrize("t", KQ)
 def test_k_quant_decode_bit_exact(ctx, t):
-    """Arbitrary bytes, special fp16 scales and a synthetic weight: the device decode equals
-    Q6_KFloatTensor.getFloat / Q5_KFloatTensor.getFloat bit for bit."""
+    """Arbitrary bytes, special fp16 scales and a synthetic weight: the device decode equals the
+    host tensor's getFloat (Q6_K, Q5_K, Q4_1, Q5_0, IQ4_XSFloatTensor) bit for bit."""
     from jitllm_amd import synthetic
     say("decode", KQ_NAMES[t])
-    bb = O.block_bytes(t)
+    bb, be = O.block_bytes(t), O.block_elems(t)
     for raw, rows in ((FX.random_bytes(20260914, 12 * bb), 12),
                       (FX.adversarial_blocks(t, 24, 20260908 + O.java_string_hash(KQ_NAMES[t])), 24),
                       (synthetic.weight(t, 40, 512, seed=701), 80)):
-        w = upload(ctx, t, raw, rows, raw.size // bb // rows * 256)
+        w = upload(ctx, t, raw, rows, raw.size // bb // rows * be)
         assert bits_equal(w.dequantize(), O.dequant(t, raw))
 
 
@@ -421,8 +421,8 @@ def test_errors_name_the_cause(ctx):
     lib = L.load()
     h = C.c_void_p()
     raw = np.zeros(64, dtype=np.uint8)
-    st = lib.jl_weight_upload(ctx.handle, 3, raw.ctypes.data, 1, 32, C.byref(h))  # Q4_1: no kernel
-    assert st == L.JL_ERR_UNSUPPORTED and b"ggml type 3" in lib.jl_last_error()
+    st = lib.jl_weight_upload(ctx.handle, 7, raw.ctypes.data, 1, 32, C.byref(h))  # Q5_1: no kernel
+    assert st == L.JL_ERR_UNSUPPORTED and b"ggml type 7" in lib.jl_last_error()
     st = lib.jl_weight_upload(ctx.handle, O.Q8_0, raw.ctypes.data, 1, 48, C.byref(h))
     assert st == L.JL_ERR_INVALID and b"whole number" in lib.jl_last_error()
     w8 = upload(ctx, O.Q8_0, synthetic.weight(O.Q8_0, 64, 256, 1), 64, 256)

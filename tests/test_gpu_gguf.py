@@ -28,7 +28,10 @@ def test_upload_from_file_then_project(ctx, tmp_path):
             "blk.0.ffn_up.weight": (O.Q4_0, synthetic.weight(O.Q4_0, d, n, seed=902)),
             "blk.0.ffn_down.weight": (O.Q4_K, synthetic.weight(O.Q4_K, d, n, seed=903)),
             "output.weight": (O.Q6_K, synthetic.weight(O.Q6_K, d, n, seed=906)),
-            "blk.0.attn_v.weight": (O.Q5_K, synthetic.weight(O.Q5_K, d, n, seed=907))}
+            "blk.0.attn_v.weight": (O.Q5_K, synthetic.weight(O.Q5_K, d, n, seed=907)),
+            "blk.1.ffn_down.weight": (O.Q4_1, synthetic.weight(O.Q4_1, d, n, seed=908)),
+            "blk.1.attn_k.weight": (O.Q5_0, synthetic.weight(O.Q5_0, d, n, seed=909)),
+            "blk.1.attn_q.weight": (O.IQ4_XS, synthetic.weight(O.IQ4_XS, d, n, seed=910))}
     tensors = [("pad.me", (5,), 24, np.arange(5, dtype=np.uint8))]       # pushes the next offset off 32
     tensors += [(name, (n, d), int(t), raw) for name, (t, raw) in raws.items()]
     path = tmp_path / "m.gguf"
@@ -54,12 +57,12 @@ def test_upload_refuses_other_types_and_truncated_files(ctx, tmp_path):
     raw = synthetic.weight(O.Q8_0, d, n, seed=905)
     path = tmp_path / "m.gguf"
     W.write_gguf(path, [], [("norm.weight", (n,), 0, np.ones(n, dtype=np.float32)),
-                            ("emb.weight", (n, 3), 3, np.zeros(3 * 8 * 20, dtype=np.uint8)),   # Q4_1
+                            ("emb.weight", (n, 3), 9, np.zeros(3 * 8 * 40, dtype=np.uint8)),   # Q8_1
                             ("q.weight", (n, d), 8, raw)], truncate_data_by=100)
     with GGUF(path) as g:
         with pytest.raises(UnsupportedProjection, match="ggml type 0"):
             g.load_weight(ctx, "norm.weight")
-        with pytest.raises(UnsupportedProjection, match="ggml type 3"):
+        with pytest.raises(UnsupportedProjection, match="ggml type 9"):
             g.load_weight(ctx, "emb.weight")
         with pytest.raises(JitllmHipError, match="runs past the end of the file"):
             g.load_weight(ctx, "q.weight")

@@ -275,6 +275,165 @@ def test_k_quant_scalar_dot_and_matmul(t):
         assert_bit_equal(O.matmul(t, raw, x, d, n, flavour=flavour), want)
 
 
+# ---- Q4_1, Q5_0, IQ4_XS ---------------------------------------------------------------------
+
+NEW_TYPES = [(O.Q4_1, "Q4_1"), (O.Q5_0, "Q5_0"), (O.IQ4_XS, "IQ4_XS")]
+
+
+@pytest.mark.parametrize("t,name", NEW_TYPES)
+def test_minor_types_decode_three_ways(t, name):
+    """Host wording (Q4_1FloatTensor.java:73-94, Q5_0FloatTensor.java:61-85, IQ4_XSFloatTensor.java:
+    72-100) == device wording (TransformerComputeKernelsQ4_1.java:59-67, ...Q5_0.java:56-70,
+    ...IQ4_XS.java:62-96) == an independent numpy statement of ggml's dequantize_row_*; on random
+    bytes and on QuantizedDeviceDecodeParityTest's adversarial blocks."""
+    bb = O.block_bytes(t)
+    for raw in (FX.random_bytes(20260914 + t, 40 * bb),
+                FX.adversarial_blocks(t, 24, 20260908 + O.java_string_hash(name))):
+        main = O.dequant(t, raw)
+        assert_bit_equal(main, O.dequant_alt(t, raw))
+        assert_bit_equal(main, NP.DEQUANT[t](raw))
+
+
+def test_q4_1_known_answers():
+    """Q4_1FloatTensorTest.reconstructsScaleTimesNibblePlusMinimum: nibbles i % 16, d = 0.25,
+    m = -1.5 -> 0.25 * nibble - 1.5, exact in fp32; element i < 16 in the low nibble of byte i,
+    element i >= 16 in the high nibble of byte i - 16.  The nibble is not recentred (Q4_0 would give
+    0.25 * (nibble - 8))."""
+    b = np.zeros(20, dtype=np.uint8)
+    b[0:2] = np.array([0.25], np.float16).view(np.uint8)
+    b[2:4] = np.array([-1.5], np.float16).view(np.uint8)
+    nib = np.arange(32) % 16
+    b[4:20] = nib[:16] | (nib[16:] << 4)
+    want = (0.25 * nib - 1.5).astype(np.float32)
+    assert np.array_equal(O.dequant(O.Q4_1, b), want)
+    # distinct nibbles in the two halves tell the halves apart
+    b[4:20] = np.arange(16) | ((15 - np.arange(16)) << 4)
+    want = np.concatenate([0.25 * np.arange(16) - 1.5, 0.25 * (15 - np.arange(16)) - 1.5]).astype(np.float32)
+    assert np.array_equal(O.dequant(O.Q4_1, b), want)
+
+
+def test_q5_0_reads_ggmls_layout():
+    """QuantizedDeviceDecodeParityTest.q5_0ReadsGgmlsLayout: d = 1, qh = 0xFFFF0000, byte i =
+    i | i << 4 -> weight j is j - 16; and a single fifth bit lands on its own element."""
+    b = np.zeros(22, dtype=np.uint8)
+    b[0:2] = [0x00, 0x3C]
+    b[2:6] = [0x00, 0x00, 0xFF, 0xFF]
+    b[6:22] = np.arange(16) | (np.arange(16) << 4)
+    assert np.array_equal(O.dequant(O.Q5_0, b), (np.arange(32) - 16).astype(np.float32))
+    for j in (0, 5, 15, 16, 23, 31):
+        b = np.zeros(22, dtype=np.uint8)
+        b[0:2] = [0x00, 0x3C]
+        b[2 + j // 8] = 1 << (j % 8)
+        want = np.full(32, -16.0, dtype=np.float32)
+        want[j] = 0.0
+        assert np.array_equal(O.dequant(O.Q5_0, b), want), j
+
+
+def test_iq4_xs_reads_ggmls_layout():
+    """QuantizedDeviceDecodeParityTest.iq4_XSReadsGgmlsLayout: d = 1, group g's scale 33 + g, byte i
+    of each group i | (15 - i) << 4 -> weight j < 16 of group g is (1 + g) kvalues[j], weight 16 + i
+    is (1 + g) kvalues[15 - i]; the table is ggml's published kvalues_iq4nl."""
+    kvalues = [-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113]
+    b = np.zeros(136, dtype=np.uint8)
+    b[0:2] = [0x00, 0x3C]
+    scales_h = 0
+    for g in range(8):
+        ls = 33 + g
+        b[4 + g // 2] |= (ls & 0xF) << (4 * (g % 2))
+        scales_h |= (ls >> 4) << (2 * g)
+    b[2], b[3] = scales_h & 0xFF, scales_h >> 8
+    for g in range(8):
+        b[8 + 16 * g:8 + 16 * g + 16] = np.arange(16) | ((15 - np.arange(16)) << 4)
+    want = np.empty(256, dtype=np.float32)
+    for j in range(256):
+        g, within = divmod(j, 32)
+        q = within if within < 16 else 15 - (within - 16)
+        want[j] = (1 + g) * kvalues[q]
+    got = O.dequant(O.IQ4_XS, b)
+    assert np.array_equal(got, want)
+    assert np.array_equal(O.dequant_alt(O.IQ4_XS, b), want)
+    # a negative group scale: ls = 0 -> d * -32
+    b[2:8] = 0
+    assert np.array_equal(O.dequant(O.IQ4_XS, b)[:16], np.float32(-32) * np.array(kvalues, np.float32))
+
+
+@pytest.mark.parametrize("width", [128, 256])
+def test_q4_1_vector_dot_lane_model(width):
+    """Q4_1FloatTensor.vectorDot (:105-192): per-lane accumulators against an independent numpy
+    model; the lane fold held to a few ulp of the magnitude sum."""
+    from jitllm_amd import synthetic
+    n = 2048
+    raw = synthetic.weight(O.Q4_1, 4, n, seed=21)
+    x = synthetic.activations(n, seed=22)
+    rb = 20 * n // 32
+    for r in range(4):
+        row = raw[r * rb:(r + 1) * rb]
+        val = NP.vector_lane_values(O.Q4_1, row, x, width)
+        want_seq = np.float32(0)
+        for v in val:
+            want_seq = np.float32(want_seq + v)
+        got = O.dot(O.Q4_1, width, raw, r * n, x, 0, n)
+        deq = NP.DEQUANT[O.Q4_1](row)
+        # the affine form sums d * q * x and m * x apart: the magnitude that bounds its rounding
+        mag = np.abs(deq * x).sum() + np.abs(x).sum() * 0.3
+        assert abs(float(got) - float(want_seq)) <= 4 * np.finfo(np.float32).eps * mag
+        exact = (deq.astype(np.float64) * x).sum()
+        assert abs(float(got) - exact) <= 64 * np.finfo(np.float32).eps * mag
+
+
+def test_q4_1_vector_dot_agrees_with_elementwise_on_spans():
+    """Q4_1FloatTensorTest.vectorizedDotAgreesWithElementwise: five blocks, spans {0, size},
+    {32, 96}, {0, 100}, {64, 33} (whole, aligned inner, scalar tail, one block + one element), tolerance
+    max(1e-4, |expected| * 1e-5) against the float64 elementwise sum."""
+    rng = O.JavaRandom(4242)
+    blocks, size = 5, 160
+    nibbles = np.array([rng.next_int(16) for _ in range(size)])
+    raw = np.zeros(blocks * 20, dtype=np.uint8)
+    for b in range(blocks):
+        scale = np.float32(0.05) + np.float32(rng.next_float()) * np.float32(0.2)
+        mn = np.float32(rng.next_float()) - np.float32(0.5)
+        raw[20 * b:20 * b + 2] = np.array([scale], np.float16).view(np.uint8)
+        raw[20 * b + 2:20 * b + 4] = np.array([mn], np.float16).view(np.uint8)
+        nb = nibbles[32 * b:32 * b + 32]
+        raw[20 * b + 4:20 * b + 20] = nb[:16] | (nb[16:] << 4)
+    x = np.array([rng.next_gaussian() for _ in range(size)]).astype(np.float32)
+    deq = NP.DEQUANT[O.Q4_1](raw).astype(np.float64)
+    for offset, length in ((0, size), (32, 96), (0, 100), (64, 33)):
+        expected = float((deq[offset:offset + length] * x[offset:offset + length]).sum())
+        for flavour in (O.DOT_VEC128, O.DOT_VEC256, O.DOT_SCALAR):
+            got = float(O.dot(O.Q4_1, flavour, raw, offset, x, offset, length))
+            assert abs(got - np.float32(expected)) <= max(1e-4, abs(np.float32(expected)) * 1e-5), (offset, length)
+
+
+@pytest.mark.parametrize("t", [O.Q5_0, O.IQ4_XS])
+def test_block_sum_dots(t):
+    """Q5_0FloatTensor.dot (:87-112) sums a block's 32 products on their own and adds the sum to the
+    result, IQ4_XSFloatTensor.dot (:102-126) a group's 32; whatever flavour is asked for.  A span
+    that starts or ends inside a block goes through scalarDot there."""
+    from jitllm_amd import synthetic
+    d, n = 5, 1024
+    raw = synthetic.weight(t, d, n, seed=79)
+    x = synthetic.activations(n, seed=80)
+    w = NP.DEQUANT[t](raw).reshape(d, n)
+    want = NP.block_sum_dot_rows(w, x)
+    for flavour in (O.DOT_SCALAR, O.DOT_VEC256):
+        assert_bit_equal(O.matmul(t, raw, x, d, n, flavour=flavour), want)
+    # sequential and block-wise sums differ in the last bits: the form is visible
+    assert not np.array_equal(want, NP.scalar_dot_rows(w, x))
+    be = O.block_elems(t)
+    off, length = be - 5, 5 + be + 3          # 5 scalar, one whole block, 3 scalar
+    head = np.float32(0)
+    for j in range(off, off + 5):
+        head = np.float32(head + np.float32(w[0, j] * x[j]))
+    mid = NP.block_sum_dot_rows(w[0:1, be:2 * be], x[be:2 * be])[0]
+    tail = np.float32(0)
+    for j in range(2 * be, 2 * be + 3):
+        tail = np.float32(tail + np.float32(w[0, j] * x[j]))
+    want1 = np.float32(np.float32(np.float32(0) + head) + mid)
+    want1 = np.float32(want1 + tail)
+    assert O.dot(t, O.DOT_SCALAR, raw, off, x, off, length) == want1
+
+
 # ---- dot products -------------------------------------------------------------------------
 
 @pytest.mark.parametrize("t,name", [(O.Q4_0, "q4_0"), (O.Q4_K, "q4_K"), (O.Q8_0, "q8_0")])
