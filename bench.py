@@ -311,6 +311,74 @@ def bench_batched_q4k(ctx, hip, B, steps, warmup):
             "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "bytes": wbytes + io}
 
 
+def bench_decode_layers(ctx, hip, type_name, dim, kv, ffn, copies, steps, warmup):
+    """Single-token decode projections of one layer -- q|k|v, o (+=), gate/up SwiGLU, down (+=) --
+    over `copies` distinct layers' weights (more bytes than the 256 MB last-level cache holds),
+    replayed as one HIP graph.  Q4_0 at Llama-3-8B shapes and Q4_K at Qwen3-8B-like shapes: the
+    other two weight types the path is specified on.  Timed twice: the fp32-activation path (the one
+    held to the CPU path's results) and the reference's optional packed-integer path, whose four
+    activation quantisations per layer are launches of their own here and are counted."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.projections import PackedActivation, QuantizedProjections, TornadoWorkspace
+    t = GGMLType[type_name]
+    shapes = {"wq": (dim, dim), "wk": (kv, dim), "wv": (kv, dim), "wo": (dim, dim),
+              "w1": (ffn, dim), "w3": (ffn, dim), "w2": (dim, ffn)}
+    host = {k: synthetic.weight(t, r, c, 71 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
+    layers = [{k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes} for _ in range(copies)]
+    x = ctx.from_numpy(synthetic.activations(dim, 78))
+    xb = ctx.from_numpy(synthetic.activations(dim, 79))
+    q, k_, v = ctx.float_array(dim), ctx.float_array(kv), ctx.float_array(kv)
+    hb = ctx.from_numpy(synthetic.activations(ffn, 80) * np.float32(0.1))
+    hb2 = ctx.float_array(ffn)
+    proj = QuantizedProjections(ctx, TornadoWorkspace(wrapX=x, wrapXb=xb, wrapHb=hb2, wrapHb2=hb))
+    small = QuantizedProjections(ctx, TornadoWorkspace(wrapHb=hb2, packedX=PackedActivation(ctx, dim)), packed=True)
+    wide = QuantizedProjections(ctx, TornadoWorkspace(packedX=PackedActivation(ctx, ffn)), packed=True)
+
+    def step():
+        for w in layers:
+            proj.fusedQKV(xb, q, k_, v, w["wq"], w["wk"], w["wv"])
+            proj.residualMatvec(xb, w["wo"], dim, dim)
+            proj.gateUp(w["w1"], w["w3"], dim, ffn)
+            proj.residualMatvec(hb, w["w2"], ffn, dim)
+
+    def step_packed():
+        for w in layers:
+            small.quantize(xb, dim)
+            small.packedFusedQKV(q, k_, v, w["wq"], w["wk"], w["wv"])
+            small.quantize(xb, dim)                      # the attention output
+            small.packedMatvec(x, w["wo"], dim, dim, residual=True)
+            small.quantize(xb, dim)                      # the feed-forward input
+            small.packedGateUp(w["w1"], w["w3"], dim, ffn)
+            wide.quantize(hb, ffn)
+            wide.packedMatvec(x, w["w2"], ffn, dim, residual=True)
+
+    def timed(fn):
+        fn()
+        ctx.sync()
+        graph = hip.capture(ctx.stream, fn)
+        for _ in range(warmup):
+            hip.launch(graph, ctx.stream)
+        ctx.sync()
+        e0, e1 = hip.event(), hip.event()
+        hip.record(e0, ctx.stream)
+        for _ in range(steps):
+            hip.launch(graph, ctx.stream)
+        hip.record(e1, ctx.stream)
+        return hip.elapsed_ms(e0, e1) / steps / copies
+
+    ms = timed(step)
+    ms_packed = timed(step_packed)
+    wbytes = sum(a.size for a in host.values())
+    io = 4 * (dim + dim + 2 * kv + dim + dim + dim + ffn + ffn + dim)
+    gbs = (wbytes + io) / (ms * 1e-3) / 1e9
+    return {"type": type_name, "shapes": {"dim": dim, "kv": kv, "ffn": ffn}, "layers_swept": copies,
+            "ms_per_layer": round(ms, 4), "GB_s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+            "bytes_per_layer": wbytes + io,
+            "packed_activation_path": {"ms_per_layer": round(ms_packed, 4), "launches_per_layer": 8,
+                                       "GB_s": round((wbytes + io) / (ms_packed * 1e-3) / 1e9, 1)}}
+
+
 # HBM bytes one gate/up launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
 # `bench.py --traffic-probe` (profiles/gemv_q8_0_gate_up_hbm_traffic.md): 17 522 KiB x 2.0 read
 # (the counter books 64 bytes for each of this chip's 128-byte requests; a 256 MiB plain copy reads
@@ -455,6 +523,9 @@ def main():
             # (the matrix pipe's clock takes tens of milliseconds of load to settle: 100 untimed
             # replays of the layer before the timed ones)
             out["prefill"] = [bench_gemm(ctx, hip, t, T, args.steps, 100) for T in (512, 2048)]
+            out["decode_other_types"] = [
+                bench_decode_layers(ctx, hip, "Q4_0", 4096, 1024, 14336, 4, args.steps, args.warmup),
+                bench_decode_layers(ctx, hip, "Q4_K", 4096, 1024, 12288, 4, args.steps, args.warmup)]
             out["batched_q4k"] = [bench_batched_q4k(ctx, hip, B, max(5, args.steps // 5), 3)
                                   for B in (8, 32, 64)]
         if not args.no_cpu:

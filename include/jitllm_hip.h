@@ -197,6 +197,39 @@ int jl_gemv_gate_up_rms(jl_context *ctx, const jl_weight *w1, const jl_weight *w
  */
 int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
 
+/* ---- packed-activation ("dp4a") decode: faster, looser -------------------------------------- */
+/*
+ * The reference's optional packed-integer decode path (QuantizedProjections.packed(),
+ * J/backend/tornado/layers/QuantizedProjections.java:110-190,257-346): the activation is quantised
+ * once to Q8 blocks and every projection of it is a sum of exact int32 block dot products times
+ * the two block scales.  It does NOT meet the 1e-3 bound of the entry points above -- the
+ * activation keeps 8 bits -- and is held to the reference's own looser envelope for this path
+ * (src/test/.../golden/CpuGpuParity.java:115-116); what it is held to tightly is the reference's
+ * packed arithmetic itself.  Q8_0, Q4_0 and Q4_K weights; row lengths that are multiples of 64 up
+ * to 16384; `quants` 16-byte aligned, `scales` and `sums` 8-byte aligned.
+ *
+ * jl_quantize_q8: quantizeActivationQ8Blocks (TransformerComputeKernelsQ4_0.java:287-341).  Per
+ * block of 32: inverse = 127 / max|x| (0 for a block of zeros), q = (int)(x * inverse +- 0.5)
+ * clamped to +-127, scales[b] = max|x| / 127, sums[b] = sum of the block's q.  n must be a multiple
+ * of 32; quants holds n bytes in element order, scales and sums n / 32 entries.
+ */
+int jl_quantize_q8(jl_context *ctx, const float *x, int64_t n, int8_t *quants, float *scales, int32_t *sums);
+/*
+ * out (+)= W . x~ with x~ the quantised activation: matrixVectorGenericQ8_0DP4A / ...WithResidual
+ * (TransformerComputeKernelsQ8_0DP4A.java:71-97,245-268), ...Q4_0DP4A (TransformerComputeKernelsQ4_0.java:
+ * 466-524,773+), ...Q4_KDP4A (TransformerComputeKernelsQ4_K.java:446-515).  Per block:
+ * Q8_0 (dW sX) dot; Q4_0 (dW sX) (dot - 8 sum); Q4_K d (sc sX dot) - dmin (m sX sum).
+ */
+int jl_gemv_q8(jl_context *ctx, const jl_weight *w, const int8_t *quants, const float *scales,
+               const int32_t *sums, float *out, int epilogue);
+/* fusedQKVMatmulQ8_0DP4A (TransformerComputeKernelsQ8_0DP4A.java:129-176) and its siblings. */
+int jl_gemv_qkv_q8(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const jl_weight *wv,
+                   const int8_t *quants, const float *scales, const int32_t *sums, float *q, float *k, float *v);
+/* fusedFFNGateUpSiLUQ8_0DP4A (:295-346), ...Q4_0DP4A (TransformerComputeKernelsQ4_0.java:859-950),
+ * ...Q4_KDP4A (TransformerComputeKernelsQ4_K.java:520-574). */
+int jl_gemv_gate_up_q8(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, const int8_t *quants,
+                       const float *scales, const int32_t *sums, float *hb);
+
 /* ---- batched decode and batched prefill: `batch` activation rows ---------------------------- */
 
 /*

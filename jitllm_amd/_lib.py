@@ -51,6 +51,10 @@ SYMBOLS = {
     "jl_gemv_qkv_rms": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_float, vp, vp, vp]),
     "jl_gemv_gate_up_rms": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp]),
     "jl_argmax": (C.c_int, [vp, vp, i64, vp]),
+    "jl_quantize_q8": (C.c_int, [vp, vp, i64, vp, vp, vp]),
+    "jl_gemv_q8": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_int]),
+    "jl_gemv_qkv_q8": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]),
+    "jl_gemv_gate_up_q8": (C.c_int, [vp, vp, vp, vp, vp, vp, vp]),
     "jl_gemm_resident_bytes": (C.c_size_t, [C.POINTER(vp), C.c_int]),
     "jl_gemm_resident": (C.c_int, [vp, C.POINTER(vp), C.c_int, vp, vp, i64, i64, i64, i64, C.c_int, C.c_int,
                                    vp, C.c_size_t, vp, C.c_size_t, C.POINTER(C.c_int32)]),

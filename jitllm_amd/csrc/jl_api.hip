@@ -302,6 +302,50 @@ int jl_gemv_gate_up_rms(jl_context *ctx, const jl_weight *w1, const jl_weight *w
     return jl_launch_gemv(ctx, &w1, 1, &hb, w3, x, JL_SWIGLU, &rms);
 }
 
+int jl_quantize_q8(jl_context *ctx, const float *x, int64_t n, int8_t *quants, float *scales, int32_t *sums) {
+    JL_REQUIRE(ctx && x && quants && scales && sums, "jl_quantize_q8: null argument");
+    JL_REQUIRE(n > 0 && n % 32 == 0, "jl_quantize_q8: %lld activations are not a whole number of blocks of 32",
+               (long long)n);
+    return jl_launch_quantize_q8(ctx, x, n, quants, scales, sums);
+}
+
+int jl_gemv_q8(jl_context *ctx, const jl_weight *w, const int8_t *quants, const float *scales,
+               const int32_t *sums, float *out, int epilogue) {
+    JL_REQUIRE(ctx && w && quants && scales && sums && out, "jl_gemv_q8: null argument");
+    JL_REQUIRE(epilogue == JL_STORE || epilogue == JL_RESIDUAL,
+               "jl_gemv_q8: epilogue %d (JL_STORE or JL_RESIDUAL)", epilogue);
+    const jl_q8x xq{quants, scales, sums};
+    return jl_launch_gemv(ctx, &w, 1, &out, nullptr, nullptr, epilogue, nullptr, &xq);
+}
+
+int jl_gemv_qkv_q8(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const jl_weight *wv,
+                   const int8_t *quants, const float *scales, const int32_t *sums, float *q, float *k, float *v) {
+    JL_REQUIRE(ctx && wq && wk && wv && quants && scales && sums && q && k && v, "jl_gemv_qkv_q8: null argument");
+    if (wq->type != wk->type || wq->type != wv->type) {
+        return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemv_qkv_q8: no fused q|k|v kernel for mixed weights %s/%s/%s",
+                       jl_type_name(wq->type), jl_type_name(wk->type), jl_type_name(wv->type));
+    }
+    JL_REQUIRE(wq->cols == wk->cols && wq->cols == wv->cols, "jl_gemv_qkv_q8: row lengths differ (%lld, %lld, %lld)",
+               (long long)wq->cols, (long long)wk->cols, (long long)wv->cols);
+    const jl_weight *ws[3] = {wq, wk, wv};
+    float *outs[3] = {q, k, v};
+    const jl_q8x xq{quants, scales, sums};
+    return jl_launch_gemv(ctx, ws, 3, outs, nullptr, nullptr, JL_STORE, nullptr, &xq);
+}
+
+int jl_gemv_gate_up_q8(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, const int8_t *quants,
+                       const float *scales, const int32_t *sums, float *hb) {
+    JL_REQUIRE(ctx && w1 && w3 && quants && scales && sums && hb, "jl_gemv_gate_up_q8: null argument");
+    if (w1->type != w3->type) {
+        return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemv_gate_up_q8: no fused gate/up kernel for a %s gate and a %s up weight",
+                       jl_type_name(w1->type), jl_type_name(w3->type));
+    }
+    JL_REQUIRE(w1->rows == w3->rows && w1->cols == w3->cols, "jl_gemv_gate_up_q8: gate is %lld x %lld, up is %lld x %lld",
+               (long long)w1->rows, (long long)w1->cols, (long long)w3->rows, (long long)w3->cols);
+    const jl_q8x xq{quants, scales, sums};
+    return jl_launch_gemv(ctx, &w1, 1, &hb, w3, nullptr, JL_SWIGLU, nullptr, &xq);
+}
+
 int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
     JL_REQUIRE(ctx && values && index && n > 0 && n <= INT32_MAX, "jl_argmax: bad argument");
     return jl_launch_argmax(ctx, values, n, index);

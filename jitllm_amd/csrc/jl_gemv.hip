@@ -52,6 +52,11 @@ struct GemvParams {
     const float *rms_scale;  // device scalar; null with rms_w set: the kernel computes
                              // 1 / sqrt(sum x^2 / n + rms_eps) itself, every workgroup for itself
     float rms_eps;
+    // Packed-integer mode: the activation as Q8 blocks (32 signed bytes, an fp32 scale and the sum
+    // of the bytes per block) instead of x.
+    const int8_t *xq;
+    const float *xq_scales;
+    const int32_t *xq_sums;
 };
 
 template <int TYPE> struct Traits;
@@ -148,6 +153,106 @@ __device__ __forceinline__ float slice_dot_q4_k(const uint4 &h, const uint4 &q0,
     float lo_term = (d * (float)sc0) * (a0 + a1) - (dmin * (float)mn0) * sx[0];
     float hi_term = (d * (float)sc1) * (b0 + b1) - (dmin * (float)mn1) * sx[1];
     return lo_term + hi_term;
+}
+
+// ---- packed-integer mode -----------------------------------------------------------------------
+//
+// The reference's dp4a kernels (TransformerComputeKernelsQ8_0DP4A.java:35-68,
+// TransformerComputeKernelsQ4_0.java:466-510, TransformerComputeKernelsQ4_K.java:599-668): the
+// activation arrives quantised to Q8 blocks, a block's products are summed exactly in int32 by
+// four-byte dot instructions and the two scales are applied to the block's sum.  A thread keeps its
+// slice's 64 activation bytes in registers in the byte positions of the weights they meet, so the
+// raw LDS words feed the dot instruction unshifted; positions that hold a weight scale face zeros.
+
+struct PackedX {
+    uint32_t q[18];   // Q8_0: A 0..8, B 9..16 | Q4_0: A low 0..4, A high 5..9, B low 10..13, B high 14..17
+                      // | Q4_K: elements 0..31 in 0..7, 32..63 in 8..15
+    float scale[2];
+    float sum[2];     // the blocks' byte sums, as floats (|sum| <= 32 * 127)
+};
+
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// xa: the eight dwords of a block's 32 activation bytes.  The block's weights start two bytes into
+// their first dword (after the fp16 scale), so the bytes move up by two: nine dwords for 32 bytes
+// (Q8_0), five for each half of 16 (Q4_0).
+template <int N>
+__device__ __forceinline__ void shift_two_bytes(const uint32_t *xa, uint32_t *out) {
+    out[0] = xa[0] << 16;
+#pragma unroll
+    for (int i = 1; i < N; i++) out[i] = __builtin_amdgcn_alignbyte(xa[i], xa[i - 1], 2);
+    out[N] = xa[N - 1] >> 16;
+}
+
+template <int TYPE>
+__device__ __forceinline__ void pack_x(const uint32_t (&raw)[16], PackedX &x) {
+    if constexpr (TYPE == JL_Q8_0) {
+        shift_two_bytes<8>(&raw[0], &x.q[0]);
+#pragma unroll
+        for (int i = 0; i < 8; i++) x.q[9 + i] = raw[8 + i];
+        x.q[17] = 0;
+    } else if constexpr (TYPE == JL_Q4_0) {
+        shift_two_bytes<4>(&raw[0], &x.q[0]);    // elements 0..15 of block A face the low nibbles
+        shift_two_bytes<4>(&raw[4], &x.q[5]);    // elements 16..31 the high nibbles
+#pragma unroll
+        for (int i = 0; i < 8; i++) x.q[10 + i] = raw[8 + i];   // block B's nibble bytes are dword aligned
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; i++) x.q[i] = raw[i];
+        x.q[16] = x.q[17] = 0;
+    }
+}
+
+// (weightScale * xScale) * dot per block (TransformerComputeKernelsQ8_0DP4A.java:58-66)
+__device__ __forceinline__ float slice_dot_packed_q8_0(const uint32_t (&w)[17], const PackedX &x) {
+    int da = 0, db = 0;
+#pragma unroll
+    for (int i = 0; i < 9; i++) da = dot4(w[i], x.q[i], da);
+#pragma unroll
+    for (int i = 0; i < 8; i++) db = dot4(w[9 + i], x.q[9 + i], db);
+    const float sa = jl_half_bits_to_float(w[0]) * x.scale[0];
+    const float sb = jl_half_bits_to_float(w[8] >> 16) * x.scale[1];
+    return fmaf(sa, (float)da, sb * (float)db);
+}
+
+// weightScale * xScale * (dot - 8 * xSum) per block (TransformerComputeKernelsQ4_0.java:487-506)
+__device__ __forceinline__ float slice_dot_packed_q4_0(const uint32_t (&w)[9], const PackedX &x) {
+    int da = 0, db = 0;
+#pragma unroll
+    for (int i = 0; i < 5; i++) {
+        da = dot4(w[i] & 0x0F0F0F0Fu, x.q[i], da);
+        da = dot4((w[i] >> 4) & 0x0F0F0F0Fu, x.q[5 + i], da);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        db = dot4(w[5 + i] & 0x0F0F0F0Fu, x.q[10 + i], db);
+        db = dot4((w[5 + i] >> 4) & 0x0F0F0F0Fu, x.q[14 + i], db);
+    }
+    const float sa = jl_half_bits_to_float(w[0]) * x.scale[0];
+    const float sb = jl_half_bits_to_float(w[4] >> 16) * x.scale[1];
+    return fmaf(sa, fmaf(-8.f, x.sum[0], (float)da), sb * fmaf(-8.f, x.sum[1], (float)db));
+}
+
+// d * (sc0 xs0 dot0 + sc1 xs1 dot1) - dmin * (m0 xs0 sum0 + m1 xs1 sum1) for the two sub-blocks of a
+// pair (TransformerComputeKernelsQ4_K.java:651-667)
+__device__ __forceinline__ float slice_dot_packed_q4_k(const uint4 &h, const uint4 &q0, const uint4 &q1,
+                                                       int pair, const PackedX &x) {
+    const uint32_t w[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    int d0 = 0, d1 = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        d0 = dot4(w[i] & 0x0F0F0F0Fu, x.q[i], d0);
+        d1 = dot4((w[i] >> 4) & 0x0F0F0F0Fu, x.q[8 + i], d1);
+    }
+    int sc0, mn0, sc1, mn1;
+    jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair, sc0, mn0);
+    jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair + 1, sc1, mn1);
+    const float d = jl_half_bits_to_float(h.x), dmin = jl_half_bits_to_float(h.x >> 16);
+    const float scaled = fmaf((float)sc0 * x.scale[0], (float)d0, ((float)sc1 * x.scale[1]) * (float)d1);
+    const float mins = fmaf((float)mn0 * x.scale[0], x.sum[0], ((float)mn1 * x.scale[1]) * x.sum[1]);
+    return fmaf(d, scaled, -dmin * mins);
 }
 
 // ---- LDS access by hand ----------------------------------------------------------------------
@@ -273,6 +378,25 @@ __device__ __forceinline__ float slice_dot_lds(uint32_t stage, int r, int s, int
     }
 }
 
+template <int TYPE>
+__device__ __forceinline__ float slice_dot_lds_packed(uint32_t stage, int r, int s, int row_bytes, const PackedX &x) {
+    const uint32_t row = stage + (uint32_t)(r * row_bytes);
+    if constexpr (TYPE == JL_Q8_0) {
+        uint32_t w[17];
+        lds_read_17(row + s * 68, w);
+        return slice_dot_packed_q8_0(w, x);
+    } else if constexpr (TYPE == JL_Q4_0) {
+        uint32_t w[9];
+        lds_read_9(row + s * 36, w);
+        return slice_dot_packed_q4_0(w, x);
+    } else {
+        uint4 h, q0, q1;
+        uint32_t sb = row + (s >> 2) * 144;
+        lds_read_q4k(sb, sb + 16 + (s & 3) * 32, h, q0, q1);
+        return slice_dot_packed_q4_k(h, q0, q1, s & 3, x);
+    }
+}
+
 // LDS map: [0, kPartialBytes) row partial sums, two parities; then the stage ring.  The activation
 // vector is staged in the ring's last stage (or, when it is larger than a stage, in a region of
 // its own after the ring) until every thread holds its 64 activations in registers.
@@ -288,8 +412,9 @@ __device__ __forceinline__ float quad_xor2(float v) {
 
 // RMS: the activations are RMS-normalised on their way in (a variant of its own, so that the plain
 // kernel's registers and schedule are not touched by it).
-template <int TYPE, bool DUAL, bool RMS>
+template <int TYPE, bool DUAL, bool RMS, bool PACKED = false>
 __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
+    static_assert(!(RMS && PACKED), "the packed activation is normalised before it is quantised");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
     constexpr int L = X4 + 1;                     // plus one 4-byte load
@@ -383,7 +508,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     const bool x_in_ring = x_bytes <= stage_bytes;  // else a region of its own after the ring
     uint8_t *xs = x_in_ring ? ring + (p.stages - 1) * stage_bytes : ring + p.stages * stage_bytes;
     const uint32_t xs0 = x_in_ring ? ring0 + (p.stages - 1) * stage_bytes : ring0 + p.stages * stage_bytes;
-    if constexpr (!rms) {
+    if constexpr (!rms && !PACKED) {
         for (int base = 0; base < x_bytes; base += nthreads * 16) {
             const int q = base / 16 + tid;
             const int sl = q / 17, k = q - sl * 17;
@@ -467,18 +592,41 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
 
     float x[64];
     float sx[2] = {0.f, 0.f};
-    if (active) {
+    PackedX px;
+    if constexpr (PACKED) {
+        // the slice's 64 bytes, two scales and two sums straight from global memory (a few KB that
+        // every workgroup reads: they stay in the cache)
+        uint32_t raw[16];
 #pragma unroll
-        for (int k = 0; k < 4; k++) lds_read_16f(xs0 + s * 272 + k * 64, &x[k * 16]);
+        for (int k = 0; k < 16; k++) raw[k] = 0;
+        px.scale[0] = px.scale[1] = px.sum[0] = px.sum[1] = 0.f;
+        if (active) {
+            const uint4 *src = (const uint4 *)(p.xq + s * 64);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint4 v = src[k];
+                raw[4 * k] = v.x; raw[4 * k + 1] = v.y; raw[4 * k + 2] = v.z; raw[4 * k + 3] = v.w;
+            }
+            const float2 sc = *(const float2 *)(p.xq_scales + 2 * s);
+            const int2 sm = *(const int2 *)(p.xq_sums + 2 * s);
+            px.scale[0] = sc.x; px.scale[1] = sc.y;
+            px.sum[0] = (float)sm.x; px.sum[1] = (float)sm.y;
+        }
+        pack_x<TYPE>(raw, px);
     } else {
+        if (active) {
 #pragma unroll
-        for (int k = 0; k < 64; k++) x[k] = 0.f;
-    }
-    if constexpr (TYPE != JL_Q8_0) {
+            for (int k = 0; k < 4; k++) lds_read_16f(xs0 + s * 272 + k * 64, &x[k * 16]);
+        } else {
 #pragma unroll
-        for (int k = 0; k < 32; k++) {
-            sx[0] += x[k];
-            sx[1] += x[32 + k];
+            for (int k = 0; k < 64; k++) x[k] = 0.f;
+        }
+        if constexpr (TYPE != JL_Q8_0) {
+#pragma unroll
+            for (int k = 0; k < 32; k++) {
+                sx[0] += x[k];
+                sx[1] += x[32 + k];
+            }
         }
     }
 
@@ -535,7 +683,10 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         if (it > 0) finish(tile - gridDim.x, (it - 1) & 1);
 
         float v = 0.f;
-        if (active) v = slice_dot_lds<TYPE>(ring0 + (it % p.stages) * stage_bytes, r, s, p.row_bytes, x, sx);
+        if (active) {
+            if constexpr (PACKED) v = slice_dot_lds_packed<TYPE>(ring0 + (it % p.stages) * stage_bytes, r, s, p.row_bytes, px);
+            else v = slice_dot_lds<TYPE>(ring0 + (it % p.stages) * stage_bytes, r, s, p.row_bytes, x, sx);
+        }
         if (p.Sp >= 2) v += quad_xor1(v);
         if (p.Sp >= 4) v += quad_xor2(v);
         if (r < p.R && (p.Sp < 4 ? s == 0 : (s & 3) == 0)) {
@@ -646,9 +797,9 @@ int blocks_per_cu(const void *fn, int device, int threads, int lds) {
     return nb;
 }
 
-template <int TYPE, bool DUAL, bool RMS>
+template <int TYPE, bool DUAL, bool RMS, bool PACKED = false>
 int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) {
-    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS>;
+    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED>;
     int per_cu = blocks_per_cu((const void *)fn, ctx->device, threads, lds);
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
@@ -660,6 +811,7 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
 
 template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds) {
+    if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
     return p.rms_w ? launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds)
                    : launch_tiles_of<TYPE, DUAL, false>(ctx, p, threads, lds);
 }
@@ -677,10 +829,13 @@ int launch_generic(jl_context *ctx, const jl_weight *w, const jl_weight *w_up, c
 }  // namespace
 
 int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *const *outs,
-                   const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms) {
+                   const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms, const jl_q8x *xq) {
     const int type = w[0]->type;
     const int n = (int)w[0]->cols;
     const int row_bytes = n / jl_block_elems(type) * jl_block_bytes(type);
+    if (xq && !jl_has_fused_kernels(type)) {
+        return jl_fail(JL_ERR_UNSUPPORTED, "no packed-activation kernel for a %s weight", jl_type_name(type));
+    }
     if (!jl_has_fused_kernels(type)) {
         if (nseg != 1 || w_up || rms) {
             return jl_fail(JL_ERR_UNSUPPORTED, "no fused single-token kernel for a %s weight "
@@ -691,7 +846,10 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
 
     const bool dual = w_up != nullptr;
     const int slice = type == JL_Q8_0 ? 68 : 36;
-    bool fast = (n % 64 == 0) && (n / 64 <= 256) && (((uintptr_t)x & 15) == 0);
+    bool fast = (n % 64 == 0) && (n / 64 <= 256) &&
+                (xq ? (((uintptr_t)xq->quants & 15) == 0 && ((uintptr_t)xq->scales & 7) == 0 &&
+                       ((uintptr_t)xq->sums & 7) == 0)
+                    : (((uintptr_t)x & 15) == 0));
     int S = n / 64, Sp = 0, R = 0, half_rows = 0;
     if (fast) {
         Sp = next_pow2(S);
@@ -702,9 +860,17 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     }
     for (int i = 0; fast && i < nseg; i++) {
         if (((uintptr_t)w[i]->blocks & 15) != 0) fast = false;
+        // the last tile is brought in by whole 16-byte loads too: a weight whose bytes do not end on
+        // a 16-byte boundary (a few odd rows of a 64- or 128-column weight) would lose its tail
+        if ((w[i]->rows * (int64_t)row_bytes) % 16 != 0) fast = false;
     }
     if (w_up && ((uintptr_t)w_up->blocks & 15) != 0) fast = false;
 
+    if (!fast && xq) {
+        return jl_fail(JL_ERR_UNSUPPORTED,
+                       "no packed-activation kernel for a row length of %d (a multiple of 64 up to 16384 "
+                       "and aligned operands are needed)", n);
+    }
     if (!fast && rms) {
         return jl_fail(JL_ERR_UNSUPPORTED,
                        "no RMS-folding projection kernel for a row length of %d (a multiple of 64 up to "
@@ -748,6 +914,11 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     p.R = R;
     p.row_bytes = row_bytes;
     p.epilogue = epilogue;
+    if (xq) {
+        p.xq = xq->quants;
+        p.xq_scales = xq->scales;
+        p.xq_sums = xq->sums;
+    }
     if (rms) {
         p.rms_w = rms->weights;
         p.rms_scale = rms->scale;

@@ -8,6 +8,10 @@
 //   jl_argmax      index of the first maximum of the logits -- argmaxLogits (:95-127) on the device,
 //                  FloatTensor.argmax (J/tensor/standard/FloatTensor.java:168-181) on the host.
 //
+//   jl_quantize_q8 the activation as Q8 blocks for the packed-integer projections -- 32 signed bytes,
+//                  an fp32 scale and the sum of the bytes per block: quantizeActivationQ8Blocks
+//                  (J/backend/tornado/kernels/TransformerComputeKernelsQ4_0.java:287-341).
+//
 // jl_rms_scale is one workgroup (a few KB of input); jl_argmax spreads the half MB of logits over
 // up to 128 workgroups and folds their results in a second, single-workgroup launch.
 #include "jl_device.h"
@@ -118,6 +122,32 @@ __global__ void __launch_bounds__(kArgmaxGroups) jl_argmax_fold(const float *val
     }
 }
 
+// One lane per activation, 32 lanes per block: inverse = 127 / max|x| (0 for a block of zeros),
+// q = (int)(x * inverse +- 0.5) clamped to +-127, scale = max|x| / 127, sum = sum of q.
+__global__ void __launch_bounds__(256)
+jl_quantize_q8_kernel(const float *__restrict__ x, int64_t n, int8_t *__restrict__ quants,
+                      float *__restrict__ scales, int32_t *__restrict__ sums) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const float value = i < n ? x[i] : 0.f;
+    float max_abs = fabsf(value);
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) max_abs = fmaxf(max_abs, __shfl_xor(max_abs, o, JL_WAVE));
+    const float inverse = max_abs > 0.0f ? __fdiv_rn(127.0f, max_abs) : 0.0f;
+    const float scaled = __fmul_rn(value, inverse);
+    int q = (int)__fadd_rn(scaled, scaled >= 0.0f ? 0.5f : -0.5f);
+    q = min(127, max(-127, q));
+    int sum = q;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, JL_WAVE);
+    if (i < n) {
+        quants[i] = (int8_t)q;
+        if ((i & 31) == 0) {
+            scales[i >> 5] = __fdiv_rn(max_abs, 127.0f);
+            sums[i >> 5] = sum;
+        }
+    }
+}
+
 }  // namespace
 
 int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale) {
@@ -134,6 +164,13 @@ int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *i
     hipLaunchKernelGGL(jl_argmax_scan, dim3(groups), dim3(kArgmaxThreads), 0, ctx->stream, values, (int)n, cells);
     JL_HIP(hipGetLastError());
     hipLaunchKernelGGL(jl_argmax_fold, dim3(1), dim3(kArgmaxGroups), 0, ctx->stream, values, cells, groups, index);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
+}
+
+int jl_launch_quantize_q8(jl_context *ctx, const float *x, int64_t n, int8_t *quants, float *scales, int32_t *sums) {
+    hipLaunchKernelGGL(jl_quantize_q8_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, x, n,
+                       quants, scales, sums);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }

@@ -28,6 +28,28 @@ class TornadoWorkspace:
     wrapXb: FloatArray | None = None
     wrapHb: FloatArray | None = None
     wrapHb2: FloatArray | None = None
+    # the packed-integer path's view of the current activation (PackedActivationTasks' arrays)
+    packedX: "PackedActivation | None" = None
+
+
+class PackedActivation:
+    """An activation vector as Q8 blocks on the device: ``n`` signed bytes, ``n / 32`` fp32 scales
+    and ``n / 32`` int32 block sums (quantizeActivationQ8Blocks,
+    J/backend/tornado/kernels/TransformerComputeKernelsQ4_0.java:287-341)."""
+
+    def __init__(self, context: Context, n: int):
+        if n % 32:
+            raise ValueError(f"{n} activations are not a whole number of blocks of 32")
+        self.n = n
+        self.quants = context.raw_buffer(n)
+        self.scales = context.raw_buffer(n // 32 * 4)
+        self.sums = context.raw_buffer(n // 32 * 4)
+
+    def get(self):
+        """(int8 quants, float32 scales, int32 sums) on the host."""
+        import numpy as np
+        return (self.quants.download(np.int8, self.n), self.scales.download(np.float32, self.n // 32),
+                self.sums.download(np.int32, self.n // 32))
 
 
 def _check_shape(w: TornadoTensor, n: int, d: int) -> None:
@@ -38,15 +60,47 @@ def _check_shape(w: TornadoTensor, n: int, d: int) -> None:
 class QuantizedProjections:
     """Single-token projections over weights kept in the file's representations."""
 
-    def __init__(self, context: Context, ws: TornadoWorkspace):
+    def __init__(self, context: Context, ws: TornadoWorkspace, packed: bool = False):
         self.context = context
         self.ws = ws
         self._lib = context._lib
+        self._packed = packed
 
     def packed(self) -> bool:
-        """The packed-integer (quantised activation) decode path of the reference is not part of
-        this library: the projections read fp32 activations, as the CPU path does."""
-        return False
+        """Whether the projections take the packed-integer path (QuantizedProjections.java:110-112):
+        one answer for the whole layer, faster and looser -- the activation keeps 8 bits.  Off unless
+        asked for; the fp32 path is the one held to the CPU path's results."""
+        return self._packed
+
+    def quantize(self, x: FloatArray, n: int) -> None:
+        """``ws.packedX`` = ``x`` as Q8 blocks (PackedActivationTasks.quantize,
+        QuantizedProjections.java:296-298)."""
+        px = self.ws.packedX
+        if px is None or px.n != n:
+            raise RuntimeError("the packed path needs ws.packedX bound to a PackedActivation of the row length")
+        L.check(self._lib.jl_quantize_q8(self.context.handle, x.ptr, n, px.quants.ptr, px.scales.ptr, px.sums.ptr))
+
+    def packedMatvec(self, out: FloatArray, w: TornadoTensor, n: int, d: int, residual: bool = False) -> None:
+        """``out (+)= w . packedX`` (the packed arms of QuantizedProjections.java:156-190, 299-346)."""
+        _check_shape(w, n, d)
+        px = self.ws.packedX
+        L.check(self._lib.jl_gemv_q8(self.context.handle, w.handle, px.quants.ptr, px.scales.ptr, px.sums.ptr,
+                                     out.ptr, L.JL_RESIDUAL if residual else L.JL_STORE))
+
+    def packedFusedQKV(self, q: FloatArray, k: FloatArray, v: FloatArray, wq: TornadoTensor, wk: TornadoTensor,
+                       wv: TornadoTensor) -> None:
+        """fusedQKVMatmulQ8_0DP4A and its siblings over ``packedX``."""
+        px = self.ws.packedX
+        L.check(self._lib.jl_gemv_qkv_q8(self.context.handle, wq.handle, wk.handle, wv.handle, px.quants.ptr,
+                                         px.scales.ptr, px.sums.ptr, q.ptr, k.ptr, v.ptr))
+
+    def packedGateUp(self, w1: TornadoTensor, w3: TornadoTensor, n: int, d: int) -> None:
+        """``wrapHb = SiLU(w1 . packedX) * (w3 . packedX)`` (fusedFFNGateUpSiLUQ8_0DP4A and siblings)."""
+        _check_shape(w1, n, d)
+        _check_shape(w3, n, d)
+        px = self.ws.packedX
+        L.check(self._lib.jl_gemv_gate_up_q8(self.context.handle, w1.handle, w3.handle, px.quants.ptr,
+                                             px.scales.ptr, px.sums.ptr, self.ws.wrapHb.ptr))
 
     def matvec(self, out: FloatArray, w: TornadoTensor, n: int, d: int) -> None:
         """``out = w . wrapXb`` (QuantizedProjections.java:140-194)."""

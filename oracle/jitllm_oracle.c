@@ -23,6 +23,12 @@
  *                              QuantizedDeviceDecodeParityTest q5_0 / iq4_XS ReadsGgmlsLayout), second
  *                              wordings, numpy statements of ggml's dequantize_row_*; dots: Q4_1 lane
  *                              model as above, Q5_0 / IQ4_XS block sums bit-equal to a numpy loop.
+ *   packed path                quantiser: known answers (the maximum maps to +-127, halves round away
+ *                              from zero, a zero block gives zero scale and quants, sums = sum q);
+ *                              projections: an activation that lies on its own int8 grid makes the
+ *                              packed result the exact dot product, checked against the float64
+ *                              product of the decoded weights, and a numpy int64 evaluation of the
+ *                              three per-block formulas.
  *   rmsnorm, argmax            closed forms (constant vectors, powers of two, eps-dominated input), a
  *                              float64 evaluation, numpy's argmax with ties, -inf and NaN cases.
  *   java.util.Random           published first outputs for seeds 0 and 42.
@@ -908,6 +914,119 @@ void jo_gemm_int8_block_scaled(int type, const int8_t *aq, const float *ascale, 
             out[(int64_t)row * n + col] = acc;
         }
     }
+}
+
+/* ---- the packed-integer decode path ("dp4a") --------------------------------------------------- */
+
+/*
+ * quantizeActivationQ8Blocks, J/backend/tornado/kernels/TransformerComputeKernelsQ4_0.java:287-341:
+ * per block of 32, inverse = maxAbs > 0 ? 127 / maxAbs : 0; q = (int)(x * inverse + (+-0.5)) clamped
+ * to [-127, 127]; scales[b] = maxAbs / 127; sums[b] = sum of the block's q.  (A Java (int) cast
+ * sends NaN to 0 and saturates; both are spelled out, C leaves them undefined.)
+ */
+void jo_quantize_q8_blocks(const float *x, int64_t n, int8_t *q, float *scales, int32_t *sums) {
+    for (int64_t b = 0; b < n / 32; b++) {
+        const float *xb = x + b * 32;
+        float max_abs = 0.0f;
+        for (int i = 0; i < 32; i++) {
+            float a = fabsf(xb[i]);
+            if (a > max_abs) max_abs = a;   /* Math.max over a tree: order cannot matter */
+        }
+        float inverse = max_abs > 0.0f ? 127.0f / max_abs : 0.0f;
+        int32_t sum = 0;
+        for (int i = 0; i < 32; i++) {
+            float scaled = xb[i] * inverse;
+            float t = scaled + (scaled >= 0.0f ? 0.5f : -0.5f);
+            int qi;
+            if (t != t) qi = 0;
+            else if (t >= 128.0f) qi = 127;
+            else if (t <= -128.0f) qi = -127;
+            else qi = (int)t;
+            if (qi > 127) qi = 127;
+            if (qi < -127) qi = -127;
+            q[b * 32 + i] = (int8_t)qi;
+            sum += qi;
+        }
+        scales[b] = max_abs / 127.0f;
+        sums[b] = sum;
+    }
+}
+
+/*
+ * One row of the packed projections, the blocks (Q4_K: units of 16 weights) taken in order:
+ *   Q8_0  partial += weightScale * xScale * dot               TransformerComputeKernelsQ8_0DP4A.java:35-68
+ *   Q4_0  partial += weightScale * xScale * (dot - 8 * xSum)  TransformerComputeKernelsQ4_0.java:487-506
+ *   Q4_K  partial += dAll * (scale0 * xs0 * dot0 + scale1 * xs1 * dot1)
+ *                    - first * dMin * (min0 * xs0 * sum0 + min1 * xs1 * sum1)
+ *                                                             TransformerComputeKernelsQ4_K.java:599-668
+ * with every dot an exact int32 sum and Java's left-to-right float products.  The reference's
+ * kernels deal the blocks to lanes and fold the lanes' partials with shuffles, an order that
+ * depends on the launch's lane count; the sequential order here is one of them, and comparisons
+ * are held to a rounding tolerance, not to bit equality.
+ */
+static float packed_row(int type, const uint8_t *row, const int8_t *q, const float *xs, const int32_t *xsum, int n) {
+    float partial = 0.0f;
+    if (type == JO_Q8_0 || type == JO_Q4_0) {
+        const int bytes = type == JO_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES;
+        for (int b = 0; b < n / 32; b++) {
+            const uint8_t *blk = row + (int64_t)b * bytes;
+            float weight_scale = jo_f16_to_f32(read_u16(blk));
+            const int8_t *a = q + b * 32;
+            int32_t dot = 0;
+            if (type == JO_Q8_0) {
+                for (int i = 0; i < 32; i++) dot += (int32_t)(int8_t)blk[2 + i] * a[i];
+                float t = weight_scale * xs[b];
+                partial += t * (float)dot;
+            } else {
+                for (int i = 0; i < 16; i++) {
+                    dot += (int32_t)(blk[2 + i] & 0xF) * a[i];
+                    dot += (int32_t)(blk[2 + i] >> 4) * a[16 + i];
+                }
+                float t = weight_scale * xs[b];
+                partial += t * (float)(dot - 8 * xsum[b]);
+            }
+        }
+        return partial;
+    }
+    for (int unit = 0; unit < n / 16; unit++) {
+        int super_block = unit >> 4, in_block = unit & 15, pair = in_block >> 2, quarter = in_block & 3;
+        const uint8_t *blk = row + (int64_t)super_block * Q4_K_BYTES;
+        float d_all = jo_f16_to_f32(read_u16(blk));
+        float d_min = jo_f16_to_f32(read_u16(blk + 2));
+        int scale0 = q4_k_scale(2 * pair, blk + 4), min0 = q4_k_min(2 * pair, blk + 4);
+        int scale1 = q4_k_scale(2 * pair + 1, blk + 4), min1 = q4_k_min(2 * pair + 1, blk + 4);
+        const uint8_t *qs = blk + 16 + pair * 32 + quarter * 8;
+        int block0 = super_block * 8 + pair * 2, block1 = block0 + 1;
+        const int8_t *a0 = q + block0 * 32 + quarter * 8, *a1 = q + block1 * 32 + quarter * 8;
+        int32_t dot0 = 0, dot1 = 0;
+        for (int i = 0; i < 8; i++) {
+            dot0 += (int32_t)(qs[i] & 0xF) * a0[i];
+            dot1 += (int32_t)(qs[i] >> 4) * a1[i];
+        }
+        float xs0 = xs[block0], xs1 = xs[block1];
+        float first = (float)(1 - (quarter < 1 ? quarter : 1));
+        float t0 = (float)scale0 * xs0;
+        t0 = t0 * (float)dot0;
+        float t1 = (float)scale1 * xs1;
+        t1 = t1 * (float)dot1;
+        float lhs = d_all * (t0 + t1);
+        float m0 = (float)min0 * xs0;
+        m0 = m0 * (float)xsum[block0];
+        float m1 = (float)min1 * xs1;
+        m1 = m1 * (float)xsum[block1];
+        float rhs = first * d_min;
+        rhs = rhs * (m0 + m1);
+        partial += lhs - rhs;
+    }
+    return partial;
+}
+
+void jo_matmul_q8x(int type, const uint8_t *w, const int8_t *q, const float *scales, const int32_t *sums,
+                   float *out, int dim0, int dim1, int nthreads) {
+    if (nthreads < 1) nthreads = 1;
+    const int64_t row_bytes = (int64_t)dim1 / jo_block_elems(type) * jo_block_bytes(type);
+#pragma omp parallel for schedule(static) num_threads(nthreads)
+    for (int i = 0; i < dim0; i++) out[i] = packed_row(type, w + i * row_bytes, q, scales, sums, dim1);
 }
 
 /* ---- java.util.Random (the generator the reference's test fixtures are drawn from) --------- */

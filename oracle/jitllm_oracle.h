@@ -59,6 +59,11 @@ void jo_quantize_q8(const float *x, int8_t *q, float *scales, int64_t rows, int6
 void jo_gemm_int8_block_scaled(int type, const int8_t *aq, const float *ascale, const uint8_t *w,
                                float *out, int m, int n, int k, int nthreads);
 
+/* The packed-integer decode path: activation quantiser and the projections over it. */
+void jo_quantize_q8_blocks(const float *x, int64_t n, int8_t *q, float *scales, int32_t *sums);
+void jo_matmul_q8x(int type, const uint8_t *w, const int8_t *q, const float *scales, const int32_t *sums,
+                   float *out, int dim0, int dim1, int nthreads);
+
 /* java.util.Random */
 typedef struct { int64_t seed; double next_next_gaussian; int have_next_next_gaussian; } jo_jrandom;
 void    jo_jrandom_init(jo_jrandom *r, int64_t seed);

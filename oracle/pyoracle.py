@@ -77,6 +77,11 @@ def lib() -> C.CDLL:
     L.jo_gemm_int8_block_scaled.argtypes = [C.c_int, _i8p, _f32p, _u8p, _f32p, C.c_int, C.c_int,
                                             C.c_int, C.c_int]
     L.jo_gemm_int8_block_scaled.restype = None
+    _i32p = C.POINTER(C.c_int32)
+    L.jo_quantize_q8_blocks.argtypes = [_f32p, C.c_int64, _i8p, _f32p, _i32p]
+    L.jo_quantize_q8_blocks.restype = None
+    L.jo_matmul_q8x.argtypes = [C.c_int, _u8p, _i8p, _f32p, _i32p, _f32p, C.c_int, C.c_int, C.c_int]
+    L.jo_matmul_q8x.restype = None
     L.jo_jrandom_init.argtypes = [C.POINTER(_JRandomState), C.c_int64]
     L.jo_jrandom_next_int.argtypes = [C.POINTER(_JRandomState)]
     L.jo_jrandom_next_int.restype = C.c_int32
@@ -202,6 +207,28 @@ def quantize_q8(x: np.ndarray):
     s = np.empty((rows, k // 32), dtype=np.float32)
     lib().jo_quantize_q8(_f32(x), q.ctypes.data_as(_i8p), _f32(s), rows, k)
     return q, s
+
+
+def quantize_q8_blocks(x: np.ndarray):
+    """quantizeActivationQ8Blocks: (int8 quants [n], float32 scales [n / 32], int32 sums [n / 32])."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    q = np.empty(x.size, dtype=np.int8)
+    s = np.empty(x.size // 32, dtype=np.float32)
+    m = np.empty(x.size // 32, dtype=np.int32)
+    lib().jo_quantize_q8_blocks(_f32(x), x.size, q.ctypes.data_as(_i8p), _f32(s),
+                                m.ctypes.data_as(C.POINTER(C.c_int32)))
+    return q, s, m
+
+
+def matmul_q8x(t: int, w: np.ndarray, q: np.ndarray, scales: np.ndarray, sums: np.ndarray, dim0: int,
+               dim1: int, nthreads: int = 0) -> np.ndarray:
+    """The packed-integer projection of a quantised activation, one value per weight row."""
+    out = np.empty(dim0, dtype=np.float32)
+    q = np.ascontiguousarray(q, dtype=np.int8)
+    sums = np.ascontiguousarray(sums, dtype=np.int32)
+    lib().jo_matmul_q8x(t, _u8(w), q.ctypes.data_as(_i8p), _f32(scales), sums.ctypes.data_as(C.POINTER(C.c_int32)),
+                        _f32(out), dim0, dim1, nthreads or max_threads())
+    return out
 
 
 def gemm_int8_block_scaled(t: int, aq: np.ndarray, ascale: np.ndarray, w: np.ndarray, n: int,

@@ -114,6 +114,8 @@ SHAPES = [
     (O.Q4_K, 4096, 4096), (O.Q4_K, 1024, 4096), (O.Q4_K, 1536, 12288), (O.Q4_K, 3072, 4096),
     (O.Q8_0, 300, 3072), (O.Q4_0, 300, 5120), (O.Q4_K, 130, 1536),   # S not a power of two
     (O.Q8_0, 77, 96), (O.Q4_0, 5, 32), (O.Q4_K, 9, 256), (O.Q8_0, 3, 32768),  # catch-all kernel
+    (O.Q8_0, 5, 64), (O.Q8_0, 3, 128), (O.Q4_0, 7, 64), (O.Q4_0, 3, 192),  # bytes that end off a 16-byte boundary
+    (O.Q8_0, 8, 64), (O.Q4_0, 4, 64),                                       # ... and the same widths on one
 ]
 
 

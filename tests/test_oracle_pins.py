@@ -614,3 +614,96 @@ def test_int8_gemm_matches_fp64_product_of_the_quantised_operands():
     terms = dots.astype(np.float64) * s.astype(np.float64)[:, None, :] * dw[None, :, :]
     worst = np.max(np.abs(got - terms.sum(axis=2)) / np.abs(terms).sum(axis=2))
     assert worst < 1e-5
+
+
+# ---- the packed-integer decode path -----------------------------------------------------------
+
+def test_quantize_q8_blocks_known_answers():
+    """quantizeActivationQ8Blocks (TransformerComputeKernelsQ4_0.java:287-341).  With max|x| = 127 the
+    inverse is exactly 1, so the rounding rule shows: halves go away from zero, the maximum maps to
+    +-127, the scale is max|x| / 127 = 1 and the sum is the sum of the quants; a block of zeros has
+    zero scale, quants and sum."""
+    x = np.zeros(96, dtype=np.float32)
+    x[0:8] = [127.0, -127.0, 2.5, -2.5, 2.4999, -2.4999, 0.49, -0.51]
+    x[64:96] = np.linspace(-3, 3, 32)
+    q, s, m = O.quantize_q8_blocks(x)
+    assert list(q[0:8]) == [127, -127, 3, -3, 2, -2, 0, -1]
+    assert s[0] == 1.0 and m[0] == int(q[0:32].astype(np.int64).sum())
+    assert s[1] == 0.0 and m[1] == 0 and not q[32:64].any()
+    assert s[2] == np.float32(np.float32(3.0) / np.float32(127.0)) and abs(int(q[64])) == 127 and abs(int(q[95])) == 127
+    # the same definition as the prefill quantiser (Int8GemmKernels.java:75-129) on ordinary data
+    rng = np.random.default_rng(31)
+    v = (rng.standard_normal((4, 256)) * 3).astype(np.float32)
+    q1, s1, m1 = O.quantize_q8_blocks(v)
+    q2, s2 = O.quantize_q8(v)
+    assert np.array_equal(q1.reshape(4, 256), q2) and np.array_equal(s1.reshape(4, 8), s2)
+    assert np.array_equal(m1, q1.reshape(-1, 32).astype(np.int64).sum(axis=1))
+
+
+def _grid_activation(n, seed):
+    """An activation that lies on its own int8 grid: q random in [-127, 127] with +-127 present in
+    every block, times a power-of-two block scale -- quantising it loses nothing."""
+    rng = np.random.default_rng(seed)
+    q = rng.integers(-127, 128, size=(n // 32, 32)).astype(np.int64)
+    q[:, 0] = 127 * rng.choice([-1, 1], size=n // 32)
+    scale = np.ldexp(1.0, rng.integers(-9, -3, size=n // 32)).astype(np.float32)
+    return (q * scale[:, None]).astype(np.float32).reshape(-1), q.reshape(-1), scale
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_packed_projection_is_exact_on_the_grid(t):
+    """If the activation is exactly representable the packed projection computes the true dot
+    product: compared with the float64 product of the decoded weights (numpy statement of the
+    format) -- a wrong nibble half, a missing -8 or a swapped scale / minimum fails it."""
+    from jitllm_amd import synthetic
+    d, n = 12, 1024
+    raw = synthetic.weight(t, d, n, seed=41)
+    x, q, scale = _grid_activation(n, 42)
+    qq, ss, mm = O.quantize_q8_blocks(x)
+    assert np.array_equal(qq, q) and np.array_equal(ss, scale * np.float32(127) / np.float32(127))
+    w = NP.DEQUANT[t](raw).reshape(d, n).astype(np.float64)
+    exact = w @ x.astype(np.float64)
+    mag = np.abs(w) @ np.abs(x.astype(np.float64))
+    got = O.matmul_q8x(t, raw, qq, ss, mm, d, n)
+    # Q4_0 / Q4_K subtract 8 sum / min sum after the product: their terms are up to ~3x the magnitude
+    assert np.max(np.abs(got - exact) / mag) < 2e-6
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_packed_projection_numpy_model(t):
+    """The three per-block formulas evaluated independently in numpy (int64 dots, float64 scales)
+    on an ordinary activation."""
+    from jitllm_amd import synthetic
+    d, n = 7, 2048
+    raw = synthetic.weight(t, d, n, seed=43)
+    x = synthetic.activations(n, seed=44) * np.float32(1.7)
+    q, s, m = O.quantize_q8_blocks(x)
+    got = O.matmul_q8x(t, raw, q, s, m, d, n)
+    qi = q.astype(np.int64).reshape(n // 32, 32)
+    s64, m64 = s.astype(np.float64), m.astype(np.int64)
+    if t == O.Q8_0:
+        b = raw.reshape(d, n // 32, 34)
+        dw = NP.half_bits_to_f32(b[:, :, 0:2].copy().view(np.uint16)[:, :, 0]).astype(np.float64)
+        wq = b[:, :, 2:].view(np.int8).astype(np.int64)
+        want = (dw * s64 * (wq * qi).sum(axis=2)).sum(axis=1)
+        mag = (np.abs(dw) * s64 * (np.abs(wq) * np.abs(qi)).sum(axis=2)).sum(axis=1)
+    elif t == O.Q4_0:
+        b = raw.reshape(d, n // 32, 18)
+        dw = NP.half_bits_to_f32(b[:, :, 0:2].copy().view(np.uint16)[:, :, 0]).astype(np.float64)
+        nib = np.concatenate([b[:, :, 2:] & 0xF, b[:, :, 2:] >> 4], axis=2).astype(np.int64)
+        want = (dw * s64 * ((nib * qi).sum(axis=2) - 8 * m64)).sum(axis=1)
+        mag = (np.abs(dw) * s64 * ((nib * np.abs(qi)).sum(axis=2) + 8 * np.abs(m64))).sum(axis=1)
+    else:
+        b = raw.reshape(d, n // 256, 144)
+        dd = NP.half_bits_to_f32(b[:, :, 0:2].copy().view(np.uint16)[:, :, 0]).astype(np.float64)
+        dmin = NP.half_bits_to_f32(b[:, :, 2:4].copy().view(np.uint16)[:, :, 0]).astype(np.float64)
+        sc, mn = NP.q4_k_scales_mins(b[:, :, 4:16])
+        qs = b[:, :, 16:].reshape(d, n // 256, 4, 32)
+        nib = np.stack([qs & 0xF, qs >> 4], axis=3).reshape(d, n // 256, 8, 32).astype(np.int64)
+        qb = qi.reshape(n // 256, 8, 32)
+        sb, mb = s64.reshape(n // 256, 8), m64.reshape(n // 256, 8)
+        dots = (nib * qb).sum(axis=3)
+        want = (dd[:, :, None] * sc * sb * dots - dmin[:, :, None] * mn * sb * mb).sum(axis=(1, 2))
+        mag = (np.abs(dd[:, :, None]) * sc * sb * (nib * np.abs(qb)).sum(axis=3)
+               + np.abs(dmin[:, :, None]) * mn * sb * np.abs(mb)).sum(axis=(1, 2))
+    assert np.max(np.abs(got - want) / mag) < 2e-6
