@@ -24,6 +24,7 @@
 #include "jl_device.h"
 #include "jl_internal.h"
 
+#include <climits>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -46,7 +47,6 @@ struct GemvParams {
     int R;          // rows per tile
     int row_bytes;
     int epilogue;
-    int stages;     // depth of the LDS tile ring (2..8)
     // RMS normalisation folded into the activation load: x_j becomes rms_w[j] * (scale * x_j).
     const float *rms_w;      // null: x is used as it is
     const float *rms_scale;  // device scalar; null with rms_w set: the kernel computes
@@ -401,6 +401,10 @@ __device__ __forceinline__ float slice_dot_lds_packed(uint32_t stage, int r, int
 // vector is staged in the ring's last stage (or, when it is larger than a stage, in a region of
 // its own after the ring) until every thread holds its 64 activations in registers.
 constexpr int kPartialBytes = 2048;  // 2 parities x 256 floats
+// Depth of the LDS tile ring: one tile computed, one in flight.  Measured on every benchmark shape,
+// a deeper ring at the lower occupancy its LDS footprint forces is slower (and no faster where it
+// costs no occupancy: the 9 KB tiles of the 4-bit types at 3 and 4 stages).
+constexpr int kStages = 2;
 
 // v + (the value two quad neighbours hold): DPP quad permutes, VALU speed, no LDS round trip
 __device__ __forceinline__ float quad_xor1(float v) {
@@ -412,6 +416,18 @@ __device__ __forceinline__ float quad_xor2(float v) {
 
 // RMS: the activations are RMS-normalised on their way in (a variant of its own, so that the plain
 // kernel's registers and schedule are not touched by it).
+// Hands a loaded argument back as a plain scalar value.  Without it the compiler merges "this
+// local or that argument-array element" into one pointer and loads through it with a flat load,
+// whose wait drains the tile ring every tile.
+__device__ __forceinline__ uint32_t uniform_value(uint32_t v) {
+    asm volatile("" : "+s"(v));
+    return v;
+}
+__device__ __forceinline__ uintptr_t uniform_value(uintptr_t v) {
+    asm volatile("" : "+s"(v));
+    return v;
+}
+
 template <int TYPE, bool DUAL, bool RMS, bool PACKED = false>
 __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     static_assert(!(RMS && PACKED), "the packed activation is normalised before it is quantised");
@@ -422,7 +438,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
-    const int wave = tid / JL_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / JL_WAVE);   // uniform: LDS-DMA bases stay scalar
     const int lane = tid & (JL_WAVE - 1);
     const int r = tid / p.Sp;           // row of the tile this thread works on
     const int s = tid - r * p.Sp;       // its 64-column slice
@@ -452,16 +468,32 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     // Brings tile `tile` into stage `st`.  Every thread issues exactly L loads, whatever the tile:
     // lanes that have nothing to fetch re-read the segment's first bytes into their own slot, so
     // each wave's outstanding-load count is a compile-time constant per tile.
-    auto issue = [&](int tile, int st) {
+    // (a launch with one segment -- every one but the fused q|k|v -- never indexes the argument
+    // arrays with a run-time segment: that is a scalar memory load, and a wait, per tile)
+    const int nseg = p.nseg;
+    const uint8_t *const w0 = p.w[0];
+    const int rows0 = p.seg_rows[0];
+    float *const out0 = p.out[0];
+    auto segment_of = [&](int tile) {
         int seg = 0;
 #pragma unroll
         for (int i = 1; i < kMaxSeg; i++)
-            if (i < p.nseg && tile >= p.seg_tile_begin[i]) seg = i;
-        const int local = tile - p.seg_tile_begin[seg];
+            if (i < nseg && tile >= p.seg_tile_begin[i]) seg = i;
+        return seg;
+    };
+    auto issue = [&](int tile, int st) {
+        const uint8_t *wseg = w0;
+        int seg_rows = rows0, local = tile;
+        if (nseg > 1) {
+            const int seg = segment_of(tile);
+            wseg = (const uint8_t *)uniform_value((uintptr_t)p.w[seg]);
+            seg_rows = (int)uniform_value((uint32_t)p.seg_rows[seg]);
+            local = tile - (int)uniform_value((uint32_t)p.seg_tile_begin[seg]);
+        }
         const int64_t offset = (int64_t)local * half_bytes;
-        const int64_t remain = (int64_t)p.seg_rows[seg] * p.row_bytes - offset;
+        const int64_t remain = (int64_t)seg_rows * p.row_bytes - offset;
         const int bytes = remain < half_bytes ? (int)remain : half_bytes;
-        const uint8_t *base = p.w[seg] + offset;
+        const uint8_t *base = wseg + offset;
         const uint8_t *base_up = DUAL ? p.w_up + offset : base;
         uint8_t *dst = ring + st * stage_bytes;
         const bool whole = exact && bytes == half_bytes;  // uniform
@@ -471,7 +503,8 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
             const int wave_off = k < X4 ? (k * nthreads + wave * JL_WAVE) * 16
                                         : X4 * nthreads * 16 + wave * JL_WAVE * 4;
             const uint8_t *src = (DUAL && slot_up[k] ? base_up : base) + slot_off[k];
-            if (!whole && slot_off[k] + width > bytes) src = p.w[seg];
+            // (a whole tile -- the uniform, usual case -- has every slot inside it)
+            if (!whole && slot_off[k] + width > bytes) src = wseg;
             if (k < X4)
                 __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + wave_off), 16, 0, 0);
             else
@@ -506,8 +539,8 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     const int x_slots = p.S * 17;
     const int x_bytes = (x_slots + nthreads - 1) / nthreads * nthreads * 16;
     const bool x_in_ring = x_bytes <= stage_bytes;  // else a region of its own after the ring
-    uint8_t *xs = x_in_ring ? ring + (p.stages - 1) * stage_bytes : ring + p.stages * stage_bytes;
-    const uint32_t xs0 = x_in_ring ? ring0 + (p.stages - 1) * stage_bytes : ring0 + p.stages * stage_bytes;
+    uint8_t *xs = x_in_ring ? ring + (kStages - 1) * stage_bytes : ring + kStages * stage_bytes;
+    const uint32_t xs0 = x_in_ring ? ring0 + (kStages - 1) * stage_bytes : ring0 + kStages * stage_bytes;
     if constexpr (!rms && !PACKED) {
         for (int base = 0; base < x_bytes; base += nthreads * 16) {
             const int q = base / 16 + tid;
@@ -518,7 +551,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         }
     }
     int issued = 0;
-    for (; issued < p.stages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
+    for (; issued < kStages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
     if constexpr (rms) {
         // RMS normalisation folded into the activation load.  CpuOperations.rmsnorm
         // (J/inference/op/CpuOperations.java:60-72): out = w * (ss * x) with
@@ -641,10 +674,6 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     auto finish = [&](int t, int par) {
         const int slots = half_rows * P;
         if (tid < slots) {
-            int seg = 0;
-#pragma unroll
-            for (int i = 1; i < kMaxSeg; i++)
-                if (i < p.nseg && t >= p.seg_tile_begin[i]) seg = i;
             const uint32_t pb = lds0 + par * kParity;
             float v0 = __uint_as_float(lds_read_b32(pb + tid * 4));
             float v1 = 0.f;
@@ -655,9 +684,17 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
                 if constexpr (DUAL) v1 = group_sum(v1, width);
             }
             const int j = tid / P;  // row of the tile
-            const int row = (t - p.seg_tile_begin[seg]) * half_rows + j;
-            if (tid - j * P == 0 && row < p.seg_rows[seg]) {
-                float *o = p.out[seg] + row;
+            int local = t, seg_rows = rows0;
+            float *out = out0;
+            if (nseg > 1) {
+                const int seg = segment_of(t);
+                local = t - (int)uniform_value((uint32_t)p.seg_tile_begin[seg]);
+                seg_rows = (int)uniform_value((uint32_t)p.seg_rows[seg]);
+                out = (float *)uniform_value((uintptr_t)p.out[seg]);
+            }
+            const int row = local * half_rows + j;
+            if (tid - j * P == 0 && row < seg_rows) {
+                float *o = out + row;
                 if constexpr (DUAL) {
                     *o = jl_swiglu_value(v0, v1);
                 } else {
@@ -677,15 +714,15 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         // the stage that tile it - 1 (or, the first time round, the activation vector) occupied
         // is free now: every wave is past its reads
         if (issued < mine) {
-            issue(first + issued * gridDim.x, issued % p.stages);
+            issue(first + issued * gridDim.x, issued % kStages);
             issued++;
         }
         if (it > 0) finish(tile - gridDim.x, (it - 1) & 1);
 
         float v = 0.f;
         if (active) {
-            if constexpr (PACKED) v = slice_dot_lds_packed<TYPE>(ring0 + (it % p.stages) * stage_bytes, r, s, p.row_bytes, px);
-            else v = slice_dot_lds<TYPE>(ring0 + (it % p.stages) * stage_bytes, r, s, p.row_bytes, x, sx);
+            if constexpr (PACKED) v = slice_dot_lds_packed<TYPE>(ring0 + (it % kStages) * stage_bytes, r, s, p.row_bytes, px);
+            else v = slice_dot_lds<TYPE>(ring0 + (it % kStages) * stage_bytes, r, s, p.row_bytes, x, sx);
         }
         if (p.Sp >= 2) v += quad_xor1(v);
         if (p.Sp >= 4) v += quad_xor2(v);
@@ -929,11 +966,7 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     const int stage_bytes = threads * slice;
     const int x_bytes = (S * 17 + threads - 1) / threads * threads * 16;  // 17 slots per slice
     const int x_extra = x_bytes <= stage_bytes ? 0 : x_bytes;
-    // Ring depth 2: measured on every benchmark shape, a deeper ring at the lower occupancy its LDS
-    // footprint forces is slower than two stages with up to four workgroups per compute unit.
-    const int stages = 2;
-    p.stages = stages;
-    const int lds = kPartialBytes + stages * stage_bytes + x_extra;
+    const int lds = kPartialBytes + kStages * stage_bytes + x_extra;
 
     switch (type) {
         case JL_Q8_0:
