@@ -497,18 +497,31 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         const uint8_t *base_up = DUAL ? p.w_up + offset : base;
         uint8_t *dst = ring + st * stage_bytes;
         const bool whole = exact && bytes == half_bytes;  // uniform
+        if (whole) {
+            // the usual case (uniform): every slot is inside the tile, nothing to redirect
 #pragma unroll
-        for (int k = 0; k < L; k++) {
-            const int width = k < X4 ? 16 : 4;
-            const int wave_off = k < X4 ? (k * nthreads + wave * JL_WAVE) * 16
-                                        : X4 * nthreads * 16 + wave * JL_WAVE * 4;
-            const uint8_t *src = (DUAL && slot_up[k] ? base_up : base) + slot_off[k];
-            // (a whole tile -- the uniform, usual case -- has every slot inside it)
-            if (!whole && slot_off[k] + width > bytes) src = wseg;
-            if (k < X4)
-                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + wave_off), 16, 0, 0);
-            else
-                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + wave_off), 4, 0, 0);
+            for (int k = 0; k < L; k++) {
+                const int wave_off = k < X4 ? (k * nthreads + wave * JL_WAVE) * 16
+                                            : X4 * nthreads * 16 + wave * JL_WAVE * 4;
+                const uint8_t *src = (DUAL && slot_up[k] ? base_up : base) + slot_off[k];
+                if (k < X4)
+                    __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + wave_off), 16, 0, 0);
+                else
+                    __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + wave_off), 4, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < L; k++) {
+                const int width = k < X4 ? 16 : 4;
+                const int wave_off = k < X4 ? (k * nthreads + wave * JL_WAVE) * 16
+                                            : X4 * nthreads * 16 + wave * JL_WAVE * 4;
+                const uint8_t *src = (DUAL && slot_up[k] ? base_up : base) + slot_off[k];
+                if (slot_off[k] + width > bytes) src = wseg;
+                if (k < X4)
+                    __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + wave_off), 16, 0, 0);
+                else
+                    __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + wave_off), 4, 0, 0);
+            }
         }
     };
 
@@ -647,12 +660,10 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         }
         pack_x<TYPE>(raw, px);
     } else {
+        // (threads with no slice never use theirs: the dot product below is skipped for them)
         if (active) {
 #pragma unroll
             for (int k = 0; k < 4; k++) lds_read_16f(xs0 + s * 272 + k * 64, &x[k * 16]);
-        } else {
-#pragma unroll
-            for (int k = 0; k < 64; k++) x[k] = 0.f;
         }
         if constexpr (TYPE != JL_Q8_0) {
 #pragma unroll
@@ -708,8 +719,8 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
 
     for (int it = 0; it < mine; it++) {
         const int tile = first + it * gridDim.x;
-        // tiles issued after tile `it`: up to stages - 2 of them may stay in flight
-        wait_vm_tiles<L>(issued - it - 1);
+        // with two stages nothing was issued after tile `it`: its loads are the youngest
+        JL_WAIT_VM(0);
         __builtin_amdgcn_s_barrier();
         // the stage that tile it - 1 (or, the first time round, the activation vector) occupied
         // is free now: every wave is past its reads
