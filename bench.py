@@ -421,6 +421,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill / batched legs")
+    ap.add_argument("--extra", default="fused_rms,prefill,other_types,batched",
+                    help="comma-separated legs beside the decode set (a profiler run takes a few at a time)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="only launch what the HBM-traffic counters are read on (see traffic_probe)")
     args = ap.parse_args()
@@ -517,15 +519,19 @@ def main():
                          "avg_launch_us": round(gate_up_avg * 1e3, 3),
                          "launches_timed": len(gate_up_ms)},
         }
-        if not args.no_extra:
+        legs = set() if args.no_extra else set(args.extra.split(","))
+        if "fused_rms" in legs:
             out["decode_fused_rms"] = bench_fused_rms(ctx, hip, proj, layers, wcls, acts, args.steps,
                                                       args.warmup)
+        if "prefill" in legs:
             # (the matrix pipe's clock takes tens of milliseconds of load to settle: 100 untimed
             # replays of the layer before the timed ones)
             out["prefill"] = [bench_gemm(ctx, hip, t, T, args.steps, 100) for T in (512, 2048)]
+        if "other_types" in legs:
             out["decode_other_types"] = [
                 bench_decode_layers(ctx, hip, "Q4_0", 4096, 1024, 14336, 4, args.steps, args.warmup),
                 bench_decode_layers(ctx, hip, "Q4_K", 4096, 1024, 12288, 4, args.steps, args.warmup)]
+        if "batched" in legs:
             out["batched_q4k"] = [bench_batched_q4k(ctx, hip, B, max(5, args.steps // 5), 3)
                                   for B in (8, 32, 64)]
         if not args.no_cpu:
