@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 F16_MFMA_PEAK_TFLOPS = 2500.0
 INT8_MFMA_PEAK_TOPS = 5000.0
 
-# Llama-3.2-1B geometry (BASELINE.json configs[1])
+# Llama-3.2-1B geometry: the decode projection set the headline metric is quoted on
 DIM, KV_DIM, HIDDEN, VOCAB, LAYERS = 2048, 512, 8192, 128256, 16
 
 

@@ -289,7 +289,11 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         const int span_slots = p.span_bytes >> 4;
         // the few instructions these waves issue go first: the copy is what everything waits for
         __builtin_amdgcn_s_setprio(3);
-        int slot_in[LD], slot_row[LD];
+        // What a lane adds to the tile's first byte never changes: its row's offset, its place in
+        // the span and, for the up half of a gate/up group, the distance between the two weights
+        // (a gate/up call has one segment).  An issue is then one 64-bit add and the load.
+        int slot_in[LD], slot_wrow[LD];
+        int64_t slot_off[LD], slot_off_row0[LD];
 #pragma unroll
         for (int j = 0; j < LD; j++) {
             const int slot = (j * kDmaWaves + dw) * 64 + lane;
@@ -297,8 +301,11 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             int within = slot - row * slots_per_row;
             row = row < kGroup ? row : kGroup - 1;
             within = within < span_slots ? within : span_slots - 1;
-            slot_row[j] = row;
+            slot_wrow[j] = DUAL ? (row & 7) : row;
             slot_in[j] = z * ZIN * p.span_bytes + within * 16;
+            const int64_t up = (DUAL && row >= 8) ? (int64_t)(p.w_up - p.w[0]) : 0;
+            slot_off_row0[j] = up + slot_in[j];
+            slot_off[j] = slot_off_row0[j] + (int64_t)slot_wrow[j] * p.row_bytes;
         }
         // tile t = span t % ZIN of group wg + (t / ZIN) stride
         auto issue = [&](int t, int st) {
@@ -308,30 +315,41 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             const int first_row = (group - sg.group_begin) * out_rows;
             const int64_t base_off = (int64_t)first_row * p.row_bytes + span_off;
             const uint8_t *w_gate = sg.w + base_off;
-            const uint8_t *w_up = DUAL ? p.w_up + base_off : w_gate;
-            asm volatile("" : "+s"(w_gate), "+s"(w_up));   // both in registers before any per-lane choice
+            asm volatile("" : "+s"(w_gate));   // in scalar registers before any per-lane arithmetic
             uint8_t *dst = ring + st * stage_bytes;
+            if (first_row + out_rows <= sg.rows) {
+                // every row of the group exists (uniform; all groups but a weight's last)
 #pragma unroll
-            for (int j = 0; j < LD; j++) {
-                if (j >= n_loads) break;
-                const int row = slot_row[j];
-                int wrow = DUAL ? (row & 7) : row;
-                if (first_row + wrow >= sg.rows) wrow = 0;  // past the weight's last row
-                const uint8_t *base = (DUAL && row >= 8) ? w_up : w_gate;
-                const uint8_t *src = base + wrow * p.row_bytes + slot_in[j];
-                __builtin_amdgcn_global_load_lds((gvoid *)src, (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, 0);
+                for (int j = 0; j < LD; j++) {
+                    if (j >= n_loads) break;
+                    __builtin_amdgcn_global_load_lds((gvoid *)(w_gate + slot_off[j]),
+                                                     (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < LD; j++) {
+                    if (j >= n_loads) break;
+                    // past the weight's last row: re-read the group's first row
+                    const int wrow = first_row + slot_wrow[j] >= sg.rows ? 0 : slot_wrow[j];
+                    __builtin_amdgcn_global_load_lds((gvoid *)(w_gate + slot_off_row0[j] + (int64_t)wrow * p.row_bytes),
+                                                     (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, 0);
+                }
             }
         };
         const int tiles = mine * ZIN;
-        int issued = 0;
-        for (; issued < p.stages - 1 && issued < tiles; issued++) issue(issued, issued);
+        int issued = 0, next_stage = 0;
+        for (; issued < p.stages - 1 && issued < tiles; issued++) {
+            issue(issued, next_stage);
+            next_stage = next_stage + 1 == p.stages ? 0 : next_stage + 1;
+        }
         for (int t = 0; t < tiles; t++) {
             // tiles issued after tile t may stay in flight
             wait_vm((issued - t - 1) * n_loads);
             __builtin_amdgcn_s_barrier();
             // the stage of tile t - 1 is free now: every compute wave is past its reads
             if (issued < tiles) {
-                issue(issued, issued % p.stages);
+                issue(issued, next_stage);
+                next_stage = next_stage + 1 == p.stages ? 0 : next_stage + 1;
                 issued++;
             }
         }
