@@ -215,6 +215,15 @@ int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
  */
 int jl_quantize_q8(jl_context *ctx, const float *x, int64_t n, int8_t *quants, float *scales, int32_t *sums);
 /*
+ * The RMS-norm apply and the quantisation in one launch: xb[i] = rms_weights[i] * (rms_scale[0] * x[i])
+ * (both products rounded to fp32; rms_scale is the device scalar jl_rms_scale leaves) is written --
+ * non-packed readers still need it -- and quantised as above.  rmsApplyAndQuantizeActivationQ8Blocks
+ * (TransformerComputeKernelsQ4_0.java:374-432), dispatched by QuantizedProjections.rmsApply
+ * (QuantizedProjections.java:117-121) before the packed projections of a layer.
+ */
+int jl_rms_quantize_q8(jl_context *ctx, const float *x, const float *rms_weights, const float *rms_scale,
+                       int64_t n, float *xb, int8_t *quants, float *scales, int32_t *sums);
+/*
  * out (+)= W . x~ with x~ the quantised activation: matrixVectorGenericQ8_0DP4A / ...WithResidual
  * (TransformerComputeKernelsQ8_0DP4A.java:71-97,245-268), ...Q4_0DP4A (TransformerComputeKernelsQ4_0.java:
  * 466-524,773+), ...Q4_KDP4A (TransformerComputeKernelsQ4_K.java:446-515).  Per block:

@@ -306,7 +306,16 @@ int jl_quantize_q8(jl_context *ctx, const float *x, int64_t n, int8_t *quants, f
     JL_REQUIRE(ctx && x && quants && scales && sums, "jl_quantize_q8: null argument");
     JL_REQUIRE(n > 0 && n % 32 == 0, "jl_quantize_q8: %lld activations are not a whole number of blocks of 32",
                (long long)n);
-    return jl_launch_quantize_q8(ctx, x, n, quants, scales, sums);
+    return jl_launch_quantize_q8(ctx, x, nullptr, nullptr, nullptr, n, quants, scales, sums);
+}
+
+int jl_rms_quantize_q8(jl_context *ctx, const float *x, const float *rms_weights, const float *rms_scale,
+                       int64_t n, float *xb, int8_t *quants, float *scales, int32_t *sums) {
+    JL_REQUIRE(ctx && x && rms_weights && rms_scale && xb && quants && scales && sums,
+               "jl_rms_quantize_q8: null argument");
+    JL_REQUIRE(n > 0 && n % 32 == 0, "jl_rms_quantize_q8: %lld activations are not a whole number of blocks of 32",
+               (long long)n);
+    return jl_launch_quantize_q8(ctx, x, rms_weights, rms_scale, xb, n, quants, scales, sums);
 }
 
 int jl_gemv_q8(jl_context *ctx, const jl_weight *w, const int8_t *quants, const float *scales,

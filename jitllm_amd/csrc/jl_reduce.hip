@@ -123,12 +123,23 @@ __global__ void __launch_bounds__(kArgmaxGroups) jl_argmax_fold(const float *val
 }
 
 // One lane per activation, 32 lanes per block: inverse = 127 / max|x| (0 for a block of zeros),
-// q = (int)(x * inverse +- 0.5) clamped to +-127, scale = max|x| / 127, sum = sum of q.
+// q = (int)(x * inverse +- 0.5) clamped to +-127, scale = max|x| / 127, sum = sum of q.  With RMS
+// the lane first computes its element of the normalised vector, rms_w[i] * (rms_scale * x[i]) with
+// both products rounded to fp32, stores it to xb and quantises that
+// (rmsApplyAndQuantizeActivationQ8Blocks, TransformerComputeKernelsQ4_0.java:374-432).
+template <bool RMS>
 __global__ void __launch_bounds__(256)
-jl_quantize_q8_kernel(const float *__restrict__ x, int64_t n, int8_t *__restrict__ quants,
-                      float *__restrict__ scales, int32_t *__restrict__ sums) {
+jl_quantize_q8_kernel(const float *__restrict__ x, const float *__restrict__ rms_w,
+                      const float *__restrict__ rms_scale, float *__restrict__ xb, int64_t n,
+                      int8_t *__restrict__ quants, float *__restrict__ scales, int32_t *__restrict__ sums) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const float value = i < n ? x[i] : 0.f;
+    float value = i < n ? x[i] : 0.f;
+    if constexpr (RMS) {
+        if (i < n) {
+            value = __fmul_rn(rms_w[i], __fmul_rn(rms_scale[0], value));
+            xb[i] = value;
+        }
+    }
     float max_abs = fabsf(value);
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) max_abs = fmaxf(max_abs, __shfl_xor(max_abs, o, JL_WAVE));
@@ -168,9 +179,16 @@ int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *i
     return JL_OK;
 }
 
-int jl_launch_quantize_q8(jl_context *ctx, const float *x, int64_t n, int8_t *quants, float *scales, int32_t *sums) {
-    hipLaunchKernelGGL(jl_quantize_q8_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, x, n,
-                       quants, scales, sums);
+int jl_launch_quantize_q8(jl_context *ctx, const float *x, const float *rms_w, const float *rms_scale, float *xb,
+                          int64_t n, int8_t *quants, float *scales, int32_t *sums) {
+    const dim3 g((unsigned)((n + 255) / 256)), b(256);
+    if (rms_w) {
+        hipLaunchKernelGGL(jl_quantize_q8_kernel<true>, g, b, 0, ctx->stream, x, rms_w, rms_scale, xb, n, quants,
+                           scales, sums);
+    } else {
+        hipLaunchKernelGGL(jl_quantize_q8_kernel<false>, g, b, 0, ctx->stream, x, rms_w, rms_scale, xb, n, quants,
+                           scales, sums);
+    }
     JL_HIP(hipGetLastError());
     return JL_OK;
 }

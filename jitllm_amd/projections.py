@@ -80,6 +80,16 @@ class QuantizedProjections:
             raise RuntimeError("the packed path needs ws.packedX bound to a PackedActivation of the row length")
         L.check(self._lib.jl_quantize_q8(self.context.handle, x.ptr, n, px.quants.ptr, px.scales.ptr, px.sums.ptr))
 
+    def rmsApplyAndQuantize(self, x: FloatArray, rmsWeights: FloatArray, rmsScale: FloatArray, n: int) -> None:
+        """``wrapXb = rmsWeights * (rmsScale[0] * x)`` and ``packedX`` = its Q8 blocks, in one launch
+        (QuantizedProjections.rmsApply, QuantizedProjections.java:117-121 ->
+        PackedActivationTasks.rmsApplyAndQuantize)."""
+        px = self.ws.packedX
+        if px is None or px.n != n:
+            raise RuntimeError("the packed path needs ws.packedX bound to a PackedActivation of the row length")
+        L.check(self._lib.jl_rms_quantize_q8(self.context.handle, x.ptr, rmsWeights.ptr, rmsScale.ptr, n,
+                                             self.ws.wrapXb.ptr, px.quants.ptr, px.scales.ptr, px.sums.ptr))
+
     def packedMatvec(self, out: FloatArray, w: TornadoTensor, n: int, d: int, residual: bool = False) -> None:
         """``out (+)= w . packedX`` (the packed arms of QuantizedProjections.java:156-190, 299-346)."""
         _check_shape(w, n, d)
