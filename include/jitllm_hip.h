@@ -178,7 +178,8 @@ int jl_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *s
  * rms_scale null, s = 1 / sqrt(sum x^2 / n + eps) computed from x by every workgroup for itself,
  * which saves the reduction's launch (fullyFusedRmsNormFFNGateUpQ8,
  * TransformerComputeKernelsLayered.java:2866+, always works this way: jl_gemv_gate_up_rms).
- * Row length: a multiple of 64 up to 16384, x and rms_weights 16-byte aligned; otherwise
+ * Row length: a multiple of 64 up to 16384 (8192 for gate/up, whose tile holds a row of each
+ * matrix), x and rms_weights 16-byte aligned; otherwise
  * JL_ERR_UNSUPPORTED and the caller normalises first, as the unfused reference path does.
  */
 int jl_gemv_rms(jl_context *ctx, const jl_weight *w, const float *x, const float *rms_weights,
@@ -206,7 +207,7 @@ int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
  * activation keeps 8 bits -- and is held to the reference's own looser envelope for this path
  * (src/test/.../golden/CpuGpuParity.java:115-116); what it is held to tightly is the reference's
  * packed arithmetic itself.  Q8_0, Q4_0 and Q4_K weights; row lengths that are multiples of 64 up
- * to 16384; `quants` 16-byte aligned, `scales` and `sums` 8-byte aligned.
+ * to 16384 (8192 for gate/up); `quants` 16-byte aligned, `scales` and `sums` 8-byte aligned.
  *
  * jl_quantize_q8: quantizeActivationQ8Blocks (TransformerComputeKernelsQ4_0.java:287-341).  Per
  * block of 32: inverse = 127 / max|x| (0 for a block of zeros), q = (int)(x * inverse +- 0.5)

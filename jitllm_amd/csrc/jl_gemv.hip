@@ -916,13 +916,13 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
 
     if (!fast && xq) {
         return jl_fail(JL_ERR_UNSUPPORTED,
-                       "no packed-activation kernel for a row length of %d (a multiple of 64 up to 16384 "
-                       "and aligned operands are needed)", n);
+                       "no packed-activation kernel for a row length of %d (a multiple of 64 up to %d "
+                       "and aligned operands are needed)", n, dual ? 8192 : 16384);
     }
     if (!fast && rms) {
         return jl_fail(JL_ERR_UNSUPPORTED,
                        "no RMS-folding projection kernel for a row length of %d (a multiple of 64 up to "
-                       "16384 and 16-byte aligned operands are needed)", n);
+                       "%d and 16-byte aligned operands are needed)", n, dual ? 8192 : 16384);
     }
     if (rms && ((uintptr_t)rms->weights & 15) != 0) {
         return jl_fail(JL_ERR_UNSUPPORTED, "the RMS weights must be 16-byte aligned");

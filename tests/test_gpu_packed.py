@@ -189,6 +189,14 @@ def test_packed_path_refusals(ctx):
     w64 = ctx.load_weight(O.Q8_0, synthetic.weight(O.Q8_0, 5, 64, seed=1606), 5, 64)
     with pytest.raises(UnsupportedProjection, match="packed-activation"):
         proj64.packedMatvec(out, w64, 64, 5)
+    # a gate/up tile holds a row of each matrix: its longest row is half the plain projection's
+    n = 16384
+    projL, wsL = packed_projections(ctx, n, wrapHb=ctx.float_array(8))
+    projL.quantize(ctx.from_numpy(synthetic.activations(n, seed=1607)), n)
+    wL = ctx.load_weight(O.Q8_0, synthetic.weight(O.Q8_0, 8, n, seed=1608), 8, n)
+    projL.packedMatvec(out, wL, n, 8)
+    with pytest.raises(UnsupportedProjection, match="up to 8192"):
+        projL.packedGateUp(wL, wL, n, 8)
     with pytest.raises(JitllmHipError, match="blocks of 32"):
         from jitllm_amd import _lib as L
         L.check(ctx._lib.jl_quantize_q8(ctx.handle, out.ptr, 8, ws.packedX.quants.ptr, ws.packedX.scales.ptr,
