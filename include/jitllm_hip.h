@@ -293,6 +293,31 @@ int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count
                      int math, void *workspace, size_t workspace_bytes, void *resident,
                      size_t resident_bytes, int32_t *resident_state);
 
+/*
+ * jl_gemm / jl_gemm_resident over activations that are already fp16 -- what the reference's prefill
+ * plugin is handed: DecodedMatMul.project (J/backend/tornado/ops/DecodedMatMul.java:100-109) passes
+ * the step's input as a HalfFloatArray and its output as a FloatArray, gemmMMA / gemmMMAQ8 take
+ * `HalfFloatArray A` (TransformerBatchPrefillKernels.java:917-924, 2397+), and the producers write
+ * fp16 themselves (batchedRmsApplyFP16 :59-72, batchedDecodeAttentionFP16Out :1633+,
+ * batchedFFNSwiGLUFP16Packed :2183-2199).
+ *   X    [batch x cols] IEEE binary16 row-major, 16-byte aligned, multiplied as it is (jl_gemm
+ *        first rescales every fp32 row by a power of two; there is nothing to rescale here, so a
+ *        row whose products leave fp16's range is the producer's to avoid, as in the reference).
+ *        Calls that read whole 256-row tiles take X in place when `batch` covers the last tile,
+ *        otherwise the active rows are copied into the workspace first.
+ *   C    fp32 as in jl_gemm; with c_fp16 != 0 -- JL_SWIGLU only, the feed-forward hidden vector
+ *        batchedFFNSwiGLUFP16Packed writes -- binary16, `ldo` and `col_offset` counting fp16 values
+ *        and every result rounded once from its fp32 value.
+ *   resident / resident_state: as in jl_gemm_resident, or both null for jl_gemm's behaviour.
+ * The workspace is sized by jl_gemm_workspace_bytes as for jl_gemm.  On inputs that fp16 holds
+ * exactly and whose rows jl_gemm's rescaling does not push below fp16's normal range the fp32
+ * results equal jl_gemm's bit for bit.
+ */
+int jl_gemm_xf16(jl_context *ctx, const jl_weight *const *weights, int count, const uint16_t *X, void *C,
+                 int c_fp16, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
+                 void *workspace, size_t workspace_bytes, void *resident, size_t resident_bytes,
+                 int32_t *resident_state);
+
 /* ---- GGUF files: the caller either side of jl_weight_upload --------------------------------- */
 
 /*

@@ -373,8 +373,11 @@ size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols,
 
 static int gemm_checked(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
                         int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
-                        int math, void *workspace, size_t workspace_bytes, const jl_resident *resident) {
-    JL_REQUIRE(ctx && weights && X && C, "jl_gemm: null argument");
+                        int math, void *workspace, size_t workspace_bytes, const jl_resident *resident,
+                        const jl_half_io *half = nullptr) {
+    JL_REQUIRE(ctx && weights && (X || (half && half->x16)) && C, "jl_gemm: null argument");
+    JL_REQUIRE(!(half && half->c_f16) || epilogue == JL_SWIGLU,
+               "jl_gemm_xf16: only the JL_SWIGLU result can be written as fp16 (epilogue %d)", epilogue);
     JL_REQUIRE(count >= 1 && count <= 8, "jl_gemm: %d weights (1..8)", count);
     JL_REQUIRE(batch >= 1 && active_rows >= 0 && active_rows <= batch,
                "jl_gemm: active_rows %lld of batch %lld", (long long)active_rows, (long long)batch);
@@ -414,7 +417,7 @@ static int gemm_checked(jl_context *ctx, const jl_weight *const *weights, int co
                        need);
     }
     return jl_launch_gemm(ctx, weights, count, X, C, batch, active_rows, ldo, col_offset, epilogue,
-                          math, workspace, workspace_bytes, resident);
+                          math, workspace, workspace_bytes, resident, half);
 }
 
 int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
@@ -444,6 +447,20 @@ int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count
     const jl_resident r{resident, resident_bytes, resident_state};
     return gemm_checked(ctx, weights, count, X, C, batch, active_rows, ldo, col_offset, epilogue, math,
                         workspace, workspace_bytes, &r);
+}
+
+int jl_gemm_xf16(jl_context *ctx, const jl_weight *const *weights, int count, const uint16_t *X, void *C,
+                 int c_fp16, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
+                 void *workspace, size_t workspace_bytes, void *resident, size_t resident_bytes,
+                 int32_t *resident_state) {
+    JL_REQUIRE(X != nullptr, "jl_gemm_xf16: null argument");
+    JL_REQUIRE((resident == nullptr) == (resident_state == nullptr),
+               "jl_gemm_xf16: a resident buffer and its state go together");
+    JL_REQUIRE(((uintptr_t)resident & 255) == 0, "jl_gemm_xf16: the resident buffer must be 256-byte aligned");
+    const jl_resident r{resident, resident_bytes, resident_state};
+    const jl_half_io half{(const _Float16 *)X, c_fp16 != 0};
+    return gemm_checked(ctx, weights, count, nullptr, (float *)C, batch, active_rows, ldo, col_offset, epilogue,
+                        JL_MATH_F16, workspace, workspace_bytes, resident ? &r : nullptr, &half);
 }
 
 }  // extern "C"

@@ -74,3 +74,18 @@ __device__ __forceinline__ float jl_swiglu_value(float g, float u) {
     float denom = (float)(1.0 + exp(-(double)g));
     return __fmul_rn(__fdiv_rn(g, denom), u);
 }
+
+// Four consecutive results of an output row stored as binary16 (round to nearest even): one
+// 8-byte store when all four lie inside the row and the address allows it.
+__device__ __forceinline__ void jl_store4_f16(_Float16 *dst, const float (&v)[4], int valid) {
+    typedef _Float16 jl_half4 __attribute__((ext_vector_type(4)));
+    if (valid >= 4 && (((uintptr_t)dst) & 7) == 0) {
+        *(jl_half4 *)dst = jl_half4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if (e < valid) dst[e] = (_Float16)v[e];
+    }
+}
+
+

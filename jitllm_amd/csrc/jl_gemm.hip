@@ -97,6 +97,16 @@ jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__r
     if (tid == 0) row_scale[row] = scale;
 }
 
+// Activations that arrive as fp16 but in a buffer the kernels cannot read whole row tiles of: the
+// active rows copied as they are, the rows that pad the last tile zero-filled.  A thread moves 16 bytes.
+__global__ void __launch_bounds__(256)
+jl_rows_copy_f16(const _Float16 *__restrict__ X, _Float16 *__restrict__ A, int rows, int k) {
+    const int row = blockIdx.x;
+    const uint4 *x = (const uint4 *)(X + (int64_t)row * k);
+    uint4 *a = (uint4 *)(A + (int64_t)row * k);
+    for (int i = threadIdx.x; i < k / 8; i += 256) a[i] = row < rows ? x[i] : uint4{0u, 0u, 0u, 0u};
+}
+
 // ---- LDS access by hand ----------------------------------------------------------------------
 // Operand tiles arrive by LDS-DMA (global_load_lds_*).  The compiler answers any LDS access it can
 // see after such a load with a full vmcnt(0) wait, which would serialise the operand ring, so every
@@ -333,8 +343,9 @@ struct GemmParams {
     int w_begin[kMaxWeights + 1];  // first virtual output column of each weight
     int count;
     const _Float16 *A;       // [padded_rows x k] fp16
-    const float *row_scale;  // [padded_rows]
+    const float *row_scale;  // [padded_rows]; null: the activations came as fp16, every scale is 1
     float *C;
+    int c_f16;               // SWIGLU only: C holds binary16 values, ldo and col_offset count them
     int rows;                // active rows
     int k;
     int n_total;             // virtual output columns (SWIGLU: rows of one weight)
@@ -696,7 +707,7 @@ jl_gemm_f16(GemmParams p) {
         for (int i = 0; i < MB; i++) {
             const int m = m0 + wm * TM + i * 16 + (lane & 15);
             if (m >= p.rows) continue;
-            const float rs = p.row_scale[m];
+            const float rs = p.row_scale ? p.row_scale[m] : 1.f;
             float *crow = p.C + (int64_t)m * p.ldo + p.col_offset;
             if (swiglu) {
 #pragma unroll
@@ -705,6 +716,10 @@ jl_gemm_f16(GemmParams p) {
                     float v[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) v[e] = gemm_swiglu(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
+                    if (p.c_f16) {
+                        jl_store4_f16((_Float16 *)p.C + (int64_t)m * p.ldo + p.col_offset + col, v, p.n_total - col);
+                        continue;
+                    }
                     float *dst = crow + col;
                     if (col + 3 < p.n_total && (((uintptr_t)dst) & 15) == 0) {
                         *(float4 *)dst = float4{v[0], v[1], v[2], v[3]};
@@ -747,13 +762,13 @@ jl_gemm_f16(GemmParams p) {
 __global__ void __launch_bounds__(256)
 jl_gemm_reduce(const float *__restrict__ partial, const float *__restrict__ row_scale,
                float *__restrict__ C, int rows, int n_total, int ntiles, int64_t plane, int splits,
-               int64_t ldo, int64_t col_offset, int epilogue) {
+               int64_t ldo, int64_t col_offset, int epilogue, int c_f16) {
     const int col = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
     const int m = blockIdx.y;
     if (col >= n_total || m >= rows) return;
     const int64_t width = (int64_t)ntiles * BN;
     float *out = C + (int64_t)m * ldo + col_offset + col;
-    const float rs = row_scale[m];
+    const float rs = row_scale ? row_scale[m] : 1.f;
     float v[4];
     if (epilogue == JL_SWIGLU) {
         // tile t holds gate columns 64 t .. 64 t + 63 in its first half and the up columns after
@@ -769,6 +784,10 @@ jl_gemm_reduce(const float *__restrict__ partial, const float *__restrict__ row_
         v[1] = gemm_swiglu(sg.y * rs, su.y * rs);
         v[2] = gemm_swiglu(sg.z * rs, su.z * rs);
         v[3] = gemm_swiglu(sg.w * rs, su.w * rs);
+        if (c_f16) {
+            jl_store4_f16((_Float16 *)C + (int64_t)m * ldo + col_offset + col, v, n_total - col);
+            return;
+        }
     } else {
         const int64_t g = (int64_t)m * width + col;
         float4 sum = {0.f, 0.f, 0.f, 0.f};
@@ -879,7 +898,7 @@ int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows, float *planes, si
     if (st != JL_OK || p.splits == 1) return st;
     hipLaunchKernelGGL(jl_gemm_reduce, dim3((p.n_total + 1023) / 1024, rows), dim3(256), 0, ctx->stream,
                        planes, p.row_scale, p.C, rows, p.n_total, p.ntiles, plane, p.splits, p.ldo,
-                       p.col_offset, p.epilogue);
+                       p.col_offset, p.epilogue, p.c_f16);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
@@ -890,7 +909,7 @@ int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row
                           int n_total, int ntiles, int64_t plane, int splits, int64_t ldo, int64_t col_offset,
                           int epilogue) {
     hipLaunchKernelGGL(jl_gemm_reduce, dim3((n_total + 1023) / 1024, rows), dim3(256), 0, ctx->stream, planes,
-                       row_scale, C, rows, n_total, ntiles, plane, splits, ldo, col_offset, epilogue);
+                       row_scale, C, rows, n_total, ntiles, plane, splits, ldo, col_offset, epilogue, 0);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
@@ -898,7 +917,7 @@ int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row
 int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
                    int epilogue, int math, void *workspace, size_t workspace_bytes,
-                   const jl_resident *resident) {
+                   const jl_resident *resident, const jl_half_io *half) {
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     if (math == JL_MATH_INT8) {
@@ -908,7 +927,9 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
         return jl_fail(JL_ERR_UNSUPPORTED,
                        "jl_gemm: no batched kernel for a row length of %d (a multiple of 256 is needed)", k);
     }
-    JL_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)workspace & 255) == 0,
+    const _Float16 *X16 = half ? half->x16 : nullptr;
+    const bool c_f16 = half && half->c_f16;
+    JL_REQUIRE(((uintptr_t)(X16 ? (const void *)X16 : (const void *)X) & 15) == 0 && ((uintptr_t)workspace & 255) == 0,
                "jl_gemm: X must be 16-byte and the workspace 256-byte aligned");
     for (int i = 0; i < count; i++)
         JL_REQUIRE(((uintptr_t)weights[i]->blocks & 15) == 0, "jl_gemm: weight %d is not 16-byte aligned", i);
@@ -923,7 +944,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const size_t plane_bytes = workspace_bytes > head ? workspace_bytes - head : 0;
 
 
-    if (rows <= 32 && jl_has_fused_kernels(type)) {
+    if (rows <= 32 && jl_has_fused_kernels(type) && !X16) {
         // batched decode of up to 32 rows: the weight-streaming kernel reads X itself
         bool taken = false;
         int st = jl_launch_gemm_skinny(ctx, weights, count, X, C, rows, ldo, col_offset, epilogue, planes,
@@ -956,15 +977,28 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
         return jl_fail(JL_ERR_WORKSPACE, "jl_gemm: a %s weight needs room for its fp16 copy (%zu bytes) in the workspace",
                        jl_type_name(type), copy_bytes);
     }
-    hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded_rows), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
-    JL_HIP(hipGetLastError());
+    if (!X16) {
+        hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded_rows), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
+        JL_HIP(hipGetLastError());
+    } else {
+        // fp16 activations are multiplied as they are (no row scales).  The kernels bring in whole
+        // row tiles: the caller's buffer serves directly when its `batch` rows cover the last
+        // tile, else the active rows are copied into the workspace and padded with zeros there.
+        row_scale = nullptr;
+        if ((int64_t)padded_rows <= batch) {
+            A = const_cast<_Float16 *>(X16);
+        } else {
+            hipLaunchKernelGGL(jl_rows_copy_f16, dim3(padded_rows), dim3(256), 0, ctx->stream, X16, A, rows, k);
+            JL_HIP(hipGetLastError());
+        }
+    }
     if (dense) {
         // what a kept copy looks like: gate / up interleaved by half tiles of this BN, or plain
         const int32_t layout = epilogue == JL_SWIGLU ? bn : 1;
         const bool decode = !kept || *resident->state != layout;
         const int st = jl_launch_gemm_dense(ctx, weights, count, A, row_scale, C, rows, ldo, col_offset, epilogue,
                                             kept ? (_Float16 *)resident->copy : (_Float16 *)planes, decode, bn,
-                                            dsplits, (float *)((uint8_t *)planes + in_workspace));
+                                            dsplits, (float *)((uint8_t *)planes + in_workspace), c_f16);
         if (st == JL_OK && kept) *resident->state = layout;
         return st;
     }
@@ -981,6 +1015,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     p.A = A;
     p.row_scale = row_scale;
     p.C = C;
+    p.c_f16 = c_f16 ? 1 : 0;
     p.rows = rows;
     p.k = k;
     p.n_total = epilogue == JL_SWIGLU ? (int)weights[0]->rows : begin;

@@ -225,8 +225,9 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
 struct DenseParams {
     const _Float16 *A;       // [padded rows x k]
     const _Float16 *W;       // [ntiles * BN x k], virtual row order
-    const float *row_scale;
+    const float *row_scale;  // null: the activations came as fp16, every scale is 1
     float *C;
+    int c_f16;               // SWIGLU only: C holds binary16 values, ldo and col_offset count them
     int rows, k, n_total;    // n_total: output columns (SWIGLU: of one weight)
     int64_t ldo, col_offset;
     int epilogue;
@@ -459,7 +460,7 @@ jl_gemm_hh(DenseParams p) {
         for (int i = 0; i < MB; i++) {
             const int m = m0 + wm * TM + i * 16 + (lane & 15);
             if (m >= p.rows) continue;
-            const float rs = p.row_scale[m];
+            const float rs = p.row_scale ? p.row_scale[m] : 1.f;
             float *crow = p.C + (int64_t)m * p.ldo + p.col_offset;
             if (swiglu) {
 #pragma unroll
@@ -468,6 +469,10 @@ jl_gemm_hh(DenseParams p) {
                     float v[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) v[e] = dense_swiglu(acc[i][j][e] * rs, acc[i][j + NB / 2][e] * rs);
+                    if (p.c_f16) {
+                        jl_store4_f16((_Float16 *)p.C + (int64_t)m * p.ldo + p.col_offset + col, v, p.n_total - col);
+                        continue;
+                    }
                     float *dst = crow + col;
                     if (col + 3 < p.n_total && (((uintptr_t)dst) & 15) == 0) {
                         *(float4 *)dst = float4{v[0], v[1], v[2], v[3]};
@@ -563,7 +568,8 @@ size_t jl_dense_copy_bytes(int k, int out_cols_virtual) {
 
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
-                         int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes) {
+                         int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes,
+                         bool c_f16) {
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     const bool swiglu = epilogue == JL_SWIGLU;
@@ -608,6 +614,7 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
     p.W = copy;
     p.row_scale = row_scale;
     p.C = C;
+    p.c_f16 = c_f16 ? 1 : 0;
     p.rows = rows;
     p.k = k;
     p.n_total = n_total;

@@ -119,10 +119,16 @@ struct jl_resident {
     size_t bytes;
     int32_t *state;
 };
+// Activations that arrive as binary16 (`x16`, read instead of X) and a SWIGLU result wanted as
+// binary16 (`c_f16`: C is then an array of binary16 values).
+struct jl_half_io {
+    const _Float16 *x16;
+    bool c_f16;
+};
 int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
                    int epilogue, int math, void *workspace, size_t workspace_bytes,
-                   const jl_resident *resident);
+                   const jl_resident *resident, const jl_half_io *half = nullptr);
 // Batched decode (at most 64 rows): the weight-streaming kernel.  `taken` says whether the shape
 // was one it handles; when not, nothing was launched and the tiled GEMM must run instead.
 int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
@@ -134,7 +140,8 @@ size_t jl_dense_copy_bytes(int k, int out_cols_virtual);
 size_t jl_dense_plane_bytes(int rows, int out_cols_virtual);
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
-                         int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes);
+                         int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes,
+                         bool c_f16 = false);
 // Adds split-K planes [splits][rows padded][ntiles * 128] in split order and applies the epilogue.
 int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row_scale, float *C, int rows,
                           int n_total, int ntiles, int64_t plane, int splits, int64_t ldo, int64_t col_offset,

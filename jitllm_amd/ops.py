@@ -20,7 +20,7 @@ from typing import Callable, Dict, List, Optional, Sequence
 
 from . import _lib as L
 from .ggml import GGMLType
-from .runtime import Context, DeviceBuffer, FloatArray, TornadoTensor
+from .runtime import Context, DeviceBuffer, FloatArray, HalfFloatArray, TornadoTensor
 
 
 class OperationKind(enum.Enum):
@@ -342,16 +342,28 @@ class HipInstance(Instance):
         if step.tokens > self.batchSize:
             raise ValueError(f"a step of {step.tokens} tokens in an instance built for {self.batchSize}")
         arr = (C.c_void_p * len(weights))(*[w.handle for w in weights])
+        copy, state = None, None
+        if self.residency:
+            key = tuple(w.handle.value for w in weights) + (epilogue == L.JL_SWIGLU,)
+            if key not in self.copies:
+                nbytes = self._lib.jl_gemm_resident_bytes(arr, len(weights))
+                self.copies[key] = (DeviceBuffer(self.context, nbytes), C.c_int32(0))
+            copy, state = self.copies[key]
+        if isinstance(x, HalfFloatArray):
+            # the reference's own operand types: fp16 in (DecodedMatMul.java:100-109), fp32 out, or --
+            # the feed-forward hidden vector -- fp16 out (batchedFFNSwiGLUFP16Packed)
+            L.check(self._lib.jl_gemm_xf16(
+                self.context.handle, arr, len(weights), x.ptr, out.ptr, int(isinstance(out, HalfFloatArray)),
+                self.batchSize, step.tokens, ldo, 0, epilogue, self.workspace.ptr, self.workspace.nbytes,
+                copy.ptr if copy else None, copy.nbytes if copy else 0, C.byref(state) if copy else None))
+            return
+        if isinstance(out, HalfFloatArray):
+            raise ValueError("an fp16 output needs fp16 activations")
         args = (self.context.handle, arr, len(weights), x.ptr, out.ptr, self.batchSize, step.tokens, ldo, 0,
                 epilogue, L.JL_MATH_DEFAULT, self.workspace.ptr, self.workspace.nbytes)
         if not self.residency:
             L.check(self._lib.jl_gemm(*args))
             return
-        key = tuple(w.handle.value for w in weights) + (epilogue == L.JL_SWIGLU,)
-        if key not in self.copies:
-            nbytes = self._lib.jl_gemm_resident_bytes(arr, len(weights))
-            self.copies[key] = (DeviceBuffer(self.context, nbytes), C.c_int32(0))
-        copy, state = self.copies[key]
         L.check(self._lib.jl_gemm_resident(*args, copy.ptr, copy.nbytes, C.byref(state)))
 
 

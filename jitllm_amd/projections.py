@@ -15,7 +15,7 @@ from dataclasses import dataclass
 
 from . import _lib as L
 from .ggml import GGMLType
-from .runtime import Context, DeviceBuffer, FloatArray, TornadoTensor
+from .runtime import Context, DeviceBuffer, FloatArray, HalfFloatArray, TornadoTensor
 
 FUSED_GATE_UP_TYPES = (GGMLType.Q8_0, GGMLType.Q4_0, GGMLType.Q4_K)
 
@@ -228,16 +228,28 @@ class QuantizedBatchProjections:
         if n > self._max_cols:
             raise ValueError(f"row length {n} exceeds the {self._max_cols} the workspace was sized for")
         arr = (C.c_void_p * len(weights))(*[w.handle for w in weights])
+        copy, state = None, None
+        if self.resident:
+            key = tuple(w.handle.value for w in weights) + (epilogue == L.JL_SWIGLU,)
+            if key not in self._copies:
+                nbytes = self._lib.jl_gemm_resident_bytes(arr, len(weights))
+                self._copies[key] = (DeviceBuffer(self.context, nbytes), C.c_int32(0))
+            copy, state = self._copies[key]
+        if isinstance(x, HalfFloatArray):
+            # fp16 activations, the operand type of the reference's prefill GEMMs (gemmMMA's
+            # HalfFloatArray A); an fp16 ``out`` is the hidden vector batchedFFNSwiGLUFP16Packed writes
+            L.check(self._lib.jl_gemm_xf16(
+                self.context.handle, arr, len(weights), x.ptr, out.ptr, int(isinstance(out, HalfFloatArray)),
+                self.batchSize, activeRows, ldo, colOffset, epilogue, self.workspace.ptr, self.workspace.nbytes,
+                copy.ptr if copy else None, copy.nbytes if copy else 0, C.byref(state) if copy else None))
+            return
+        if isinstance(out, HalfFloatArray):
+            raise ValueError("an fp16 output needs fp16 activations")
         if not self.resident:
             L.check(self._lib.jl_gemm(self.context.handle, arr, len(weights), x.ptr, out.ptr,
                                       self.batchSize, activeRows, ldo, colOffset, epilogue, self.math,
                                       self.workspace.ptr, self.workspace.nbytes))
             return
-        key = tuple(w.handle.value for w in weights) + (epilogue == L.JL_SWIGLU,)
-        if key not in self._copies:
-            nbytes = self._lib.jl_gemm_resident_bytes(arr, len(weights))
-            self._copies[key] = (DeviceBuffer(self.context, nbytes), C.c_int32(0))
-        copy, state = self._copies[key]
         L.check(self._lib.jl_gemm_resident(self.context.handle, arr, len(weights), x.ptr, out.ptr,
                                            self.batchSize, activeRows, ldo, colOffset, epilogue, self.math,
                                            self.workspace.ptr, self.workspace.nbytes, copy.ptr, copy.nbytes,

@@ -61,6 +61,14 @@ class Context:
         a.set(values)
         return a
 
+    def half_array(self, size: int) -> "HalfFloatArray":
+        return HalfFloatArray(self, size)
+
+    def half_from_numpy(self, values: np.ndarray) -> "HalfFloatArray":
+        a = HalfFloatArray(self, np.asarray(values).size)
+        a.set(values)
+        return a
+
     def raw_buffer(self, nbytes: int) -> "DeviceBuffer":
         return DeviceBuffer(self, nbytes)
 
@@ -122,6 +130,23 @@ class FloatArray(DeviceBuffer):
 
     def get(self) -> np.ndarray:
         return self.download(np.float32, self.size)
+
+
+class HalfFloatArray(DeviceBuffer):
+    """IEEE binary16 device array: the activations of the batched prefill (TornadoVM's HalfFloatArray)."""
+
+    def __init__(self, ctx: Context, size: int):
+        super().__init__(ctx, int(size) * 2)
+        self.size = int(size)
+
+    def set(self, values: np.ndarray) -> None:
+        values = np.ascontiguousarray(values, dtype=np.float16).reshape(-1)
+        if values.size != self.size:
+            raise ValueError(f"{values.size} values for a HalfFloatArray of {self.size}")
+        self.upload(values)
+
+    def get(self) -> np.ndarray:
+        return self.download(np.float16, self.size)
 
 
 class TornadoTensor:

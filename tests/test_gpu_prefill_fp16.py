@@ -1,0 +1,226 @@
+"""GPU parity of the batched prefill over fp16 activations (jl_gemm_xf16): the operand types the
+reference's prefill GEMMs take (fp16 in, fp32 out; the feed-forward hidden vector fp16 out).  Pinned
+three ways: to the fp32 entry point bit for bit on inputs fp16 holds exactly, to the oracle on the
+widened inputs, and -- the fp16 output -- to the fp32 output rounded once."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from gpu_util import magnitude, rel_err, say
+from oracle import pyoracle as O
+
+pytestmark = pytest.mark.gpu
+
+F16_BOUND = 2e-3                  # fp16-MFMA path: max |d| / sum |w x|
+UNTOUCHED = np.float32(-12345.5)
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from jitllm_amd.runtime import Context
+    c = Context(0)
+    yield c
+    c.close()
+
+
+def half_activations(shape, seed):
+    from jitllm_amd import synthetic
+    return synthetic.activations(shape, seed=seed).astype(np.float16)
+
+
+# (type, weight rows, row length, batch, active rows, residual): whole-tile batches read in place by
+# the decode-once path (one with K cut in two), ragged ones copied into the workspace, small ones
+# on the decode-in-the-loop kernel, and a type that always decodes once
+CASES = [
+    (O.Q8_0, 3072, 2048, 512, 512, False),
+    (O.Q8_0, 2048, 2048, 2048, 2048, True),
+    (O.Q4_K, 4100, 1024, 600, 600, False),
+    (O.Q4_K, 4100, 1024, 768, 600, True),
+    (O.Q4_0, 1000, 512, 130, 130, True),
+    (O.Q8_0, 300, 256, 9, 9, False),
+    (O.Q8_0, 300, 256, 64, 40, True),
+    (O.Q6_K, 640, 512, 96, 90, False),
+]
+
+
+@pytest.mark.parametrize("t,d,n,batch,rows,residual", CASES)
+def test_fp16_activations_give_the_fp32_entry_points_bits(ctx, t, d, n, batch, rows, residual):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("xf16 projection", t, d, n, batch, rows, residual)
+    raw = synthetic.weight(t, d, n, seed=1700 + d % 97)
+    w = ctx.load_weight(t, raw, d, n)
+    X16 = half_activations((batch, n), 1701)
+    X32 = X16.astype(np.float32)
+    start = synthetic.activations((batch, d), seed=1702) if residual else np.full((batch, d), UNTOUCHED, np.float32)
+    p = QuantizedBatchProjections(ctx, batch, n, d)
+    a, b = ctx.from_numpy(start), ctx.from_numpy(start)
+    p.projection(ctx.from_numpy(X32), a, w, n, d, residual, activeRows=rows)
+    p.projection(ctx.half_from_numpy(X16), b, w, n, d, residual, activeRows=rows)
+    ctx.sync()
+    got32, got16 = a.get().reshape(batch, d), b.get().reshape(batch, d)
+    if rows > 32:       # up to 32 rows the fp32 entry point reads X itself, in another kernel
+        assert np.array_equal(got16.view(np.uint32), got32.view(np.uint32))
+    assert np.array_equal(got16[rows:], start[rows:])
+    ref = O.matmul_batch(t, raw, X32[:rows], d, n).astype(np.float64) + (start[:rows] if residual else 0.0)
+    mag = magnitude(t, raw, X32[:rows], d, n) + (np.abs(start[:rows]) * 1e-6 if residual else 0.0)
+    assert rel_err(got16[:rows], ref, mag) < F16_BOUND
+
+
+@pytest.mark.parametrize("t,dq,dkv,n,T,resident", [(O.Q8_0, 2048, 512, 2048, 512, True), (O.Q4_K, 256, 128, 1024, 70, False)])
+def test_fp16_activations_fused_qkv(ctx, t, dq, dkv, n, T, resident):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("xf16 qkv", t, T)
+    raws = [synthetic.weight(t, r, n, seed=1710 + i) for i, r in enumerate((dq, dkv, dkv))]
+    ws = [ctx.load_weight(t, raw, r, n) for raw, r in zip(raws, (dq, dkv, dkv))]
+    X16 = half_activations((T, n), 1713)
+    width = dq + 2 * dkv
+    p = QuantizedBatchProjections(ctx, T, n, width, resident=resident)
+    a, b = ctx.float_array(T * width, fill=UNTOUCHED), ctx.float_array(T * width, fill=UNTOUCHED)
+    for _ in range(2):                                   # the second call reuses the resident copy
+        p.fusedQKV(ctx.from_numpy(X16.astype(np.float32)), a, *ws)
+        p.fusedQKV(ctx.half_from_numpy(X16), b, *ws)
+        ctx.sync()
+        got = b.get().reshape(T, width)
+        assert np.array_equal(got.view(np.uint32), a.get().reshape(T, width).view(np.uint32))
+    col = 0
+    for raw, r in zip(raws, (dq, dkv, dkv)):
+        ref = O.matmul_batch(t, raw, X16.astype(np.float32), r, n)
+        assert rel_err(got[:, col:col + r], ref, magnitude(t, raw, X16.astype(np.float32), r, n)) < F16_BOUND
+        col += r
+
+
+@pytest.mark.parametrize("t,ffn,n,batch,rows", [(O.Q8_0, 8192, 2048, 512, 512), (O.Q4_K, 1002, 512, 768, 700),
+                                                (O.Q4_0, 1002, 1024, 96, 96), (O.Q5_K, 520, 256, 40, 33)])
+def test_fp16_hidden_vector_is_the_fp32_one_rounded_once(ctx, t, ffn, n, batch, rows):
+    """gate/up + SwiGLU with the result stored as fp16 (batchedFFNSwiGLUFP16Packed): every value is
+    the fp32 result of the same call rounded to nearest even, rows past the active ones untouched;
+    the fp32 result itself equals the fp32 entry point's and meets the oracle."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("xf16 gate/up", t, ffn, n, batch, rows)
+    r1, r3 = synthetic.weight(t, ffn, n, seed=1720), synthetic.weight(t, ffn, n, seed=1721)
+    w1, w3 = ctx.load_weight(t, r1, ffn, n), ctx.load_weight(t, r3, ffn, n)
+    X16 = half_activations((batch, n), 1722)
+    X32 = X16.astype(np.float32)
+    p = QuantizedBatchProjections(ctx, batch, n, 2 * ffn)
+    h32, h32x = ctx.float_array(batch * ffn, fill=UNTOUCHED), ctx.float_array(batch * ffn, fill=UNTOUCHED)
+    h16 = ctx.half_from_numpy(np.full(batch * ffn, 7.5, dtype=np.float16))
+    dx = ctx.half_from_numpy(X16)
+    # (called below the mirror's gateUp, which keeps the reference's rule that only Q8_0 / Q4_0 /
+    # Q4_K pairs are fused; the library takes the Q5_K pair)
+    from jitllm_amd import _lib as L
+    p._gemm([w1, w3], ctx.from_numpy(X32), h32, rows, ffn, 0, L.JL_SWIGLU)
+    p._gemm([w1, w3], dx, h32x, rows, ffn, 0, L.JL_SWIGLU)
+    p._gemm([w1, w3], dx, h16, rows, ffn, 0, L.JL_SWIGLU)
+    ctx.sync()
+    a, b, c = h32.get().reshape(batch, ffn), h32x.get().reshape(batch, ffn), h16.get().reshape(batch, ffn)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.array_equal(c[:rows].view(np.uint16), b[:rows].astype(np.float16).view(np.uint16))
+    assert np.all(c[rows:] == np.float16(7.5))
+    g = O.matmul_batch(t, r1, X32[:rows], ffn, n)
+    u = O.matmul_batch(t, r3, X32[:rows], ffn, n)
+    want = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(rows, ffn)
+    mg, mu = magnitude(t, r1, X32[:rows], ffn, n), magnitude(t, r3, X32[:rows], ffn, n)
+    bound = F16_BOUND * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(b[:rows].astype(np.float64) - want) <= bound)
+
+
+def test_fp16_hidden_vector_at_an_odd_offset(ctx):
+    """ldo and col_offset count fp16 values; an output row that starts on an odd element takes the
+    element-wise stores and leaves its neighbours alone."""
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("xf16 gate/up offset")
+    t, ffn, n, T, ldo, off = O.Q8_0, 130, 256, 40, 141, 3
+    r1, r3 = synthetic.weight(t, ffn, n, seed=1730), synthetic.weight(t, ffn, n, seed=1731)
+    w1, w3 = ctx.load_weight(t, r1, ffn, n), ctx.load_weight(t, r3, ffn, n)
+    dx = ctx.half_from_numpy(half_activations((T, n), 1732))
+    p = QuantizedBatchProjections(ctx, T, n, 2 * ffn)
+    h32 = ctx.float_array(T * ffn)
+    h16 = ctx.half_from_numpy(np.full(T * ldo, 7.5, dtype=np.float16))
+    p.gateUp(dx, h32, w1, w3, n, ffn)
+    arr = (C.c_void_p * 2)(w1.handle, w3.handle)
+    L.check(ctx._lib.jl_gemm_xf16(ctx.handle, arr, 2, dx.ptr, h16.ptr, 1, T, T, ldo, off, L.JL_SWIGLU,
+                                  p.workspace.ptr, p.workspace.nbytes, None, 0, None))
+    ctx.sync()
+    got = h16.get().reshape(T, ldo)
+    assert np.array_equal(got[:, off:off + ffn].view(np.uint16),
+                          h32.get().reshape(T, ffn).astype(np.float16).view(np.uint16))
+    assert np.all(got[:, :off] == np.float16(7.5)) and np.all(got[:, off + ffn:] == np.float16(7.5))
+
+
+def test_plugin_instance_takes_the_references_operand_types(ctx):
+    """A layer's steps through the plugin mirror with fp16 activations in, fp32 out and an fp16
+    hidden vector feeding the down projection, against the oracle on the same fp16 values."""
+    from jitllm_amd import ops, synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.ops import HipImplementation, MatMul, ResidualAdd, SwiGLU, Target, TensorRole as R
+    say("xf16 plugin layer")
+    t, T, dim, kv, ffn = O.Q8_0, 512, 512, 256, 4352
+    g = GGMLType(t)
+    shapes = {R.ATTENTION_QUERY: (dim, dim), R.ATTENTION_KEY: (kv, dim), R.ATTENTION_VALUE: (kv, dim),
+              R.FFN_GATE: (ffn, dim), R.FFN_UP: (ffn, dim), R.FFN_DOWN: (dim, ffn)}
+    raws = {r: synthetic.weight(g, d, n, seed=1740 + i) for i, (r, (d, n)) in enumerate(shapes.items())}
+    tensors = {r: ctx.load_weight(g, raws[r], *shapes[r]) for r in shapes}
+    program = [
+        MatMul(R.ATTENTION_QUERY, "xb", "qkv", dim, dim, T, g), MatMul(R.ATTENTION_KEY, "xb", "k", kv, dim, T, g),
+        MatMul(R.ATTENTION_VALUE, "xb", "v", kv, dim, T, g),
+        MatMul(R.FFN_GATE, "xb", "hb", ffn, dim, T, g), MatMul(R.FFN_UP, "xb", "hb2", ffn, dim, T, g),
+        SwiGLU("hb", "hb2", "hb"),
+        MatMul(R.FFN_DOWN, "hb", "xb2", dim, ffn, T, g), ResidualAdd("x", "xb2"),
+    ]
+    impl = HipImplementation(residency=True)
+    steps = [c.step for c in ops.split(program, 0, T, [impl], Target())]
+    xb = half_activations((T, dim), 1750)
+    x = synthetic.activations((T, dim), 1751)
+    acts = {"xb": ctx.half_from_numpy(xb), "x": ctx.from_numpy(x), "qkv": ctx.float_array(T * (dim + 2 * kv)),
+            "hb": ctx.half_array(T * ffn)}
+    inst = impl.create(steps, Target(), ctx)
+    operands = ops.Operands(acts, lambda role, layer: tensors[role])
+    for step in steps:
+        inst.emit(step, operands)
+    ctx.sync()
+    xb32 = xb.astype(np.float32)
+    got = acts["qkv"].get().reshape(T, dim + 2 * kv)
+    col = 0
+    for r in (R.ATTENTION_QUERY, R.ATTENTION_KEY, R.ATTENTION_VALUE):
+        d, n = shapes[r]
+        assert rel_err(got[:, col:col + d], O.matmul_batch(t, raws[r], xb32, d, n), magnitude(t, raws[r], xb32, d, n)) < F16_BOUND
+        col += d
+    hb = acts["hb"].get().reshape(T, ffn)
+    gt, up = O.matmul_batch(t, raws[R.FFN_GATE], xb32, ffn, dim), O.matmul_batch(t, raws[R.FFN_UP], xb32, ffn, dim)
+    want = O.swiglu(gt.reshape(-1), up.reshape(-1)).reshape(T, ffn)
+    mg, mu = magnitude(t, raws[R.FFN_GATE], xb32, ffn, dim), magnitude(t, raws[R.FFN_UP], xb32, ffn, dim)
+    bound = F16_BOUND * (mg * np.abs(up) + 1.2 * mu * np.abs(gt)) + np.abs(want) * 2.0 ** -11 + 1e-6
+    assert np.all(np.abs(hb.astype(np.float64) - want) <= bound)
+    # the down projection read exactly the fp16 hidden vector the device holds
+    hb32 = hb.astype(np.float32)
+    ref = O.matmul_batch(t, raws[R.FFN_DOWN], hb32, dim, ffn).astype(np.float64) + x
+    mag = magnitude(t, raws[R.FFN_DOWN], hb32, dim, ffn) + np.abs(x) * 1e-6
+    assert rel_err(acts["x"].get().reshape(T, dim), ref, mag) < F16_BOUND
+
+
+def test_xf16_refusals(ctx):
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("xf16 refusals")
+    t, d, n, T = O.Q8_0, 64, 256, 8
+    w = ctx.load_weight(t, synthetic.weight(t, d, n, seed=1760), d, n)
+    p = QuantizedBatchProjections(ctx, T, n, d)
+    dx = ctx.half_from_numpy(half_activations((T, n), 1761))
+    with pytest.raises(L.JitllmHipError, match="only the JL_SWIGLU result"):
+        p.projection(dx, ctx.half_array(T * d), w, n, d, False)
+    with pytest.raises(ValueError, match="fp16 output needs fp16 activations"):
+        p.projection(ctx.float_array(T * n), ctx.half_array(T * d), w, n, d, False)
+    arr = (C.c_void_p * 1)(w.handle)
+    out = ctx.float_array(T * d)
+    copy = ctx.raw_buffer(1 << 20)
+    with pytest.raises(L.JitllmHipError, match="go together"):
+        L.check(ctx._lib.jl_gemm_xf16(ctx.handle, arr, 1, dx.ptr, out.ptr, 0, T, T, d, 0, L.JL_STORE,
+                                      p.workspace.ptr, p.workspace.nbytes, copy.ptr, copy.nbytes, None))
+    with pytest.raises(L.JitllmHipError, match="null argument"):
+        L.check(ctx._lib.jl_gemm_xf16(ctx.handle, arr, 1, None, out.ptr, 0, T, T, d, 0, L.JL_STORE,
+                                      p.workspace.ptr, p.workspace.nbytes, None, 0, None))
