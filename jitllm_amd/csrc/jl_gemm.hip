@@ -846,10 +846,11 @@ size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_
     // kernel always make, is padded to whole 256-row column tiles)
     size_t planes = round_up(round_up((size_t)out_cols, 256) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
     // calls of 512 rows or more may decode the weights to fp16 once, into the same region
-    // (and, for narrow projections with long rows, two planes of partial sums; such calls have
-    // fewer 256 x 128 tiles than 0.7 x 256 compute units)
+    // (and, for narrow projections, up to eight planes of partial sums; such calls have fewer
+    // 256 x 128 tiles than 0.7 x 256 compute units and are cut no further than twice that many
+    // work items, which bounds the planes)
     if (max_rows >= 512) {
-        size_t two = jl_dense_plane_bytes((int)max_rows, (int)out_cols);
+        size_t two = jl_dense_plane_bytes((int)max_rows, (int)out_cols, 8);
         const size_t cap = 2 * (size_t)180 * 256 * 128 * sizeof(float);
         if (two > cap) two = cap;
         const size_t need = round_up(jl_dense_copy_bytes((int)cols, (int)out_cols), 256) + two;
@@ -970,7 +971,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const bool kept = resident && resident->copy && resident->state && resident->bytes >= copy_bytes &&
                       ((uintptr_t)resident->copy & 255) == 0;
     const size_t in_workspace = kept ? 0 : copy_bytes;
-    const bool dense = bn != 0 && in_workspace + (dsplits > 1 ? jl_dense_plane_bytes(rows, virt) : 0) <= plane_bytes;
+    const bool dense = bn != 0 && in_workspace + (dsplits > 1 ? jl_dense_plane_bytes(rows, virt, dsplits) : 0) <= plane_bytes;
     const int padded_rows = dense ? (int)round_up((size_t)rows, 256) : padded;
 
     if (dense_only && !dense) {

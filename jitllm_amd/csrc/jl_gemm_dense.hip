@@ -539,8 +539,9 @@ int launch_decode(jl_context *ctx, const DecodeParams &d, int virtual_rows) {
 
 // Column tile the dense path would use for a call, 0 when the call is not one for it: it takes
 // 512 rows or more and enough work items to give most compute units one.  Narrow projections
-// with long rows get there by cutting K in two (*splits = 2, plain store / residual only); what is
-// still too small keeps the decode-in-the-loop kernel, whose 128-row tiles fill the chip better.
+// get there by cutting K into 2, 4 or 8 runs of at least four steps (plain store / residual only);
+// what is still too small keeps the decode-in-the-loop kernel, whose 128-row tiles fill the chip
+// better.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits) {
     *splits = 1;
     if (rows < 512 || k % 64 != 0) return 0;
@@ -549,16 +550,21 @@ int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, in
     if ((int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units) return 256;
     const int64_t items = (int64_t)mtiles * ((out_cols_virtual + 127) / 128);
     if (items * 10 >= (int64_t)compute_units * 7) return 128;
-    if (epilogue != JL_SWIGLU && k >= 2048 && k % 128 == 0 && items * 20 >= (int64_t)compute_units * 7) {
-        *splits = 2;
-        return 128;
+    if (epilogue != JL_SWIGLU) {
+        for (int s = 2; s <= 8; s *= 2) {
+            if ((k / DBK) % s != 0 || k / s < 4 * DBK) break;
+            if (items * s * 10 >= (int64_t)compute_units * 7) {
+                *splits = s;
+                return 128;
+            }
+        }
     }
     return 0;
 }
 
-// Bytes of the partial-sum planes of a call that cuts K in two.
-size_t jl_dense_plane_bytes(int rows, int out_cols_virtual) {
-    return 2 * (size_t)((rows + DBM - 1) / DBM * DBM) * (size_t)((out_cols_virtual + 127) / 128 * 128) * sizeof(float);
+// Bytes of the partial-sum planes of a call that cuts K into `splits` runs.
+size_t jl_dense_plane_bytes(int rows, int out_cols_virtual, int splits) {
+    return (size_t)splits * (size_t)((rows + DBM - 1) / DBM * DBM) * (size_t)((out_cols_virtual + 127) / 128 * 128) * sizeof(float);
 }
 
 // Bytes of the decoded copy for `out_cols_virtual` weight rows of `k` columns.

@@ -137,7 +137,7 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
 // Many-row prefill: weights decoded to fp16 once per call into `copy`, then a plain fp16 GEMM.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits);
 size_t jl_dense_copy_bytes(int k, int out_cols_virtual);
-size_t jl_dense_plane_bytes(int rows, int out_cols_virtual);
+size_t jl_dense_plane_bytes(int rows, int out_cols_virtual, int splits);
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
                          int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes,

@@ -197,6 +197,8 @@ def test_many_row_prefill_qkv_and_gate_up(ctx):
     (O.Q4_K, 6016, 256, 1024, True),     # 128-wide tiles, residual
     (O.Q4_0, 16500, 256, 1100, False),   # 256-wide tiles, ragged rows and columns
     (O.Q8_0, 3000, 2048, 1024, True),    # K cut in two, last tile 56 columns
+    (O.Q4_K, 3000, 1024, 600, False),    # K cut in four runs of four steps, ragged rows
+    (O.Q8_0, 1500, 2048, 512, True),     # K cut in eight, last tile 92 columns
 ])
 def test_two_pass_prefill_tiles_and_edges(ctx, t, d, n, T, residual):
     """Shapes with enough tiles for the decode-once path on 256 compute units, one per tiling it
