@@ -318,6 +318,18 @@ int jl_gemm_xf16(jl_context *ctx, const jl_weight *const *weights, int count, co
                  void *workspace, size_t workspace_bytes, void *resident, size_t resident_bytes,
                  int32_t *resident_state);
 
+/*
+ * The producer of those fp16 activations: the batched prefill's RMS normalisation, reduction and
+ * apply in one launch.  batchedRmsReduceParallel (TransformerBatchPrefillKernels.java:1480-1510)
+ * in its own summation order -- work item t of 256 adds the squares of elements t, t + 256, ...,
+ * the partial sums fold as a binary tree, scales[b] = 1 / sqrt(sum / n + eps) in fp32 -- then
+ * batchedRmsApplyFP16 (:59-72): out[b][i] = fp16(rms_weights[i] * scales[b] * X[b][i]), products
+ * left to right in fp32, one rounding to fp16.  X [rows x n] fp32, out [rows x n] binary16;
+ * `scales` ([rows]) may be null.
+ */
+int jl_rms_apply_xf16(jl_context *ctx, const float *X, const float *rms_weights, float eps, int64_t rows,
+                      int64_t n, float *scales, uint16_t *out);
+
 /* ---- GGUF files: the caller either side of jl_weight_upload --------------------------------- */
 
 /*

@@ -449,6 +449,15 @@ int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count
                         workspace, workspace_bytes, &r);
 }
 
+int jl_rms_apply_xf16(jl_context *ctx, const float *X, const float *rms_weights, float eps, int64_t rows,
+                      int64_t n, float *scales, uint16_t *out) {
+    JL_REQUIRE(ctx && X && rms_weights && out, "jl_rms_apply_xf16: null argument");
+    JL_REQUIRE(rows >= 0 && n > 0 && n <= INT32_MAX && rows <= INT32_MAX, "jl_rms_apply_xf16: %lld rows of %lld",
+               (long long)rows, (long long)n);
+    if (rows == 0) return JL_OK;
+    return jl_launch_rms_apply_f16(ctx, X, rms_weights, eps, rows, n, scales, (_Float16 *)out);
+}
+
 int jl_gemm_xf16(jl_context *ctx, const jl_weight *const *weights, int count, const uint16_t *X, void *C,
                  int c_fp16, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,
                  void *workspace, size_t workspace_bytes, void *resident, size_t resident_bytes,

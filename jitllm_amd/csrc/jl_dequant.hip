@@ -4,9 +4,8 @@
 #include "jl_device.h"
 #include "jl_internal.h"
 
-// One thread per element; `*_rn` intrinsics keep every product and the subtraction a separately
-// rounded fp32 operation (the compiler may otherwise contract a*b-c into one fma, which Java
-// never does).
+// One thread per element; every product is a separately rounded fp32 operation (jl_mul_rn: the
+// compiler would otherwise contract a*b-c into one fma, which Java never does).
 
 // J/tensor/standard/Q8_0FloatTensor.java:52-61: quant * scale.
 __global__ void __launch_bounds__(256)
@@ -16,7 +15,7 @@ jl_dequant_q8_0(const uint8_t *__restrict__ w, float *__restrict__ out, int64_t 
     const uint8_t *blk = w + (i >> 5) * 34;
     float d = jl_half_bits_to_float(blk[0] | (blk[1] << 8));
     float q = (float)(int)(int8_t)blk[2 + (i & 31)];
-    out[i] = __fmul_rn(q, d);
+    out[i] = jl_mul_rn(q, d);
 }
 
 // J/tensor/standard/Q4_0FloatTensor.java:55-79: (nibble - 8) * scale; element i < 16 is the low
@@ -30,7 +29,7 @@ jl_dequant_q4_0(const uint8_t *__restrict__ w, float *__restrict__ out, int64_t 
     int e = (int)(i & 31);
     int byte = blk[2 + (e & 15)];
     int q = (e < 16 ? (byte & 0xF) : (byte >> 4)) - 8;
-    out[i] = __fmul_rn((float)q, d);
+    out[i] = jl_mul_rn((float)q, d);
 }
 
 // J/tensor/standard/Q4_KFloatTensor.java:87-122: ((d * sc) * q) - (dmin * m).
@@ -51,9 +50,9 @@ jl_dequant_q4_k(const uint8_t *__restrict__ w, float *__restrict__ out, int64_t 
     int q = high ? (byte >> 4) : (byte & 0xF);
     int sc, mn;
     jl_q4k_scale_min(hdr[1], hdr[2], hdr[3], pair * 2 + high, sc, mn);
-    float t = __fmul_rn(d, (float)sc);
-    t = __fmul_rn(t, (float)q);
-    float u = __fmul_rn(dmin, (float)mn);
+    float t = jl_mul_rn(d, (float)sc);
+    t = jl_mul_rn(t, (float)q);
+    float u = jl_mul_rn(dmin, (float)mn);
     out[i] = __fsub_rn(t, u);
 }
 

@@ -7,6 +7,17 @@
 
 #define JL_WAVE 64
 
+// A product rounded to fp32 on its own.  The compiler's default is to contract a * b + c into one
+// fma -- across statements, through the *_rn intrinsics (plain operators in this toolchain's
+// headers), and even into a mixed-precision fma when the sum is then narrowed to fp16 (with a +0
+// addend, which also loses the sign of a zero product).  Java never fuses, so wherever a result
+// has to carry the host's bits the product passes through a register the compiler cannot look past.
+__device__ __forceinline__ float jl_mul_rn(float a, float b) {
+    float r = a * b;
+    asm volatile("" : "+v"(r));
+    return r;
+}
+
 // IEEE half bits -> float, exact (subnormals included); the device form of Float.float16ToFloat.
 __device__ __forceinline__ float jl_half_bits_to_float(uint32_t bits) {
     return __half2float(__ushort_as_half((unsigned short)(bits & 0xFFFFu)));
@@ -72,7 +83,7 @@ __device__ __forceinline__ float jl_group_sum_dyn(float v, int width) {
 // divide and one float multiply (CpuOperations.swiGLU, J/inference/op/CpuOperations.java:255-260).
 __device__ __forceinline__ float jl_swiglu_value(float g, float u) {
     float denom = (float)(1.0 + exp(-(double)g));
-    return __fmul_rn(__fdiv_rn(g, denom), u);
+    return jl_mul_rn(__fdiv_rn(g, denom), u);
 }
 
 // Four consecutive results of an output row stored as binary16 (round to nearest even): one

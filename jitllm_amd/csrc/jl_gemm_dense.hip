@@ -145,7 +145,7 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
             const uint2 hdr = *(const uint2 *)sb;
             const uint2 q = *(const uint2 *)(sb + 8 + 16 * g + (c & 1) * 8);
             const int ls = (int)(((hdr.y >> (4 * g)) & 0xFu) | ((((hdr.x >> 16) >> (2 * g)) & 3u) << 4));
-            a = __fmul_rn(jl_half_bits_to_float(hdr.x), (float)(ls - 32));
+            a = jl_mul_rn(jl_half_bits_to_float(hdr.x), (float)(ls - 32));
             q0 = jl_iq4nl_lookup4((q.x >> shift) & 0x0F0F0F0Fu);
             q1 = jl_iq4nl_lookup4((q.y >> shift) & 0x0F0F0F0Fu);
         }
@@ -154,9 +154,9 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
         for (int e = 0; e < 8; e++) {
             const uint32_t byte = ((e < 4 ? q0 : q1) >> (8 * (e & 3))) & 0xFF;
             float f;
-            if constexpr (TYPE == JL_Q4_1) f = __fadd_rn(__fmul_rn((float)byte, a), b);
-            else if constexpr (TYPE == JL_Q5_0) f = __fmul_rn(a, (float)((int)byte - 16));
-            else f = __fmul_rn(a, (float)(int)(int8_t)byte);
+            if constexpr (TYPE == JL_Q4_1) f = __fadd_rn(jl_mul_rn((float)byte, a), b);
+            else if constexpr (TYPE == JL_Q5_0) f = jl_mul_rn(a, (float)((int)byte - 16));
+            else f = jl_mul_rn(a, (float)(int)(int8_t)byte);
             v[e] = (_Float16)f;
         }
         *dst = *(const uint4 *)v;
@@ -171,16 +171,16 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
         const uint2 qh = *(const uint2 *)(sb + 16 + pos);
         int sc, mn;
         jl_q4k_scale_min(h.y, h.z, h.w, sub, sc, mn);
-        const float ds = __fmul_rn(jl_half_bits_to_float(h.x), (float)sc);
-        const float dm = __fmul_rn(jl_half_bits_to_float(h.x >> 16), (float)mn);
+        const float ds = jl_mul_rn(jl_half_bits_to_float(h.x), (float)sc);
+        const float dm = jl_mul_rn(jl_half_bits_to_float(h.x >> 16), (float)mn);
         const int nib = (sub & 1) * 4;
         const uint32_t q0 = ((qs.x >> nib) & 0x0F0F0F0Fu) | (((qh.x >> sub) & 0x01010101u) << 4);
         const uint32_t q1 = ((qs.y >> nib) & 0x0F0F0F0Fu) | (((qh.y >> sub) & 0x01010101u) << 4);
         _Float16 v[8];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            v[e] = (_Float16)__fsub_rn(__fmul_rn(ds, (float)((q0 >> (8 * e)) & 0xFF)), dm);
-            v[4 + e] = (_Float16)__fsub_rn(__fmul_rn(ds, (float)((q1 >> (8 * e)) & 0xFF)), dm);
+            v[e] = (_Float16)__fsub_rn(jl_mul_rn(ds, (float)((q0 >> (8 * e)) & 0xFF)), dm);
+            v[4 + e] = (_Float16)__fsub_rn(jl_mul_rn(ds, (float)((q1 >> (8 * e)) & 0xFF)), dm);
         }
         *dst = *(const uint4 *)v;
     } else if constexpr (TYPE == JL_Q6_K) {
@@ -191,7 +191,7 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
         const int e0 = (c & 31) * 8, h = e0 >> 7, g = (e0 >> 5) & 3, pos = e0 & 31;
         const Quants8 ql = *(const Quants8 *)(sb + 64 * h + 32 * (g & 1) + pos);
         const Quants8 qh = *(const Quants8 *)(sb + 128 + 32 * h + pos);
-        const float ds = __fmul_rn(jl_half_bits_to_float(*(const unsigned short *)(sb + 208)),
+        const float ds = jl_mul_rn(jl_half_bits_to_float(*(const unsigned short *)(sb + 208)),
                                    (float)(int)(int8_t)sb[192 + 8 * h + (pos >> 4) + 2 * g]);
         const int nib = (g >> 1) * 4;
         const uint32_t q0 = ((ql.lo >> nib) & 0x0F0F0F0Fu) | (((qh.lo >> (2 * g)) & 0x03030303u) << 4);
@@ -199,8 +199,8 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
         _Float16 v[8];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            v[e] = (_Float16)__fmul_rn(ds, (float)((int)((q0 >> (8 * e)) & 0xFF) - 32));
-            v[4 + e] = (_Float16)__fmul_rn(ds, (float)((int)((q1 >> (8 * e)) & 0xFF) - 32));
+            v[e] = (_Float16)jl_mul_rn(ds, (float)((int)((q0 >> (8 * e)) & 0xFF) - 32));
+            v[4 + e] = (_Float16)jl_mul_rn(ds, (float)((int)((q1 >> (8 * e)) & 0xFF) - 32));
         }
         *dst = *(const uint4 *)v;
     } else {

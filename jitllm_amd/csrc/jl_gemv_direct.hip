@@ -303,7 +303,7 @@ jl_dequant_q6_k(const uint8_t *__restrict__ w, float *__restrict__ out, int64_t 
     const int q = (low | (((qh >> (2 * group)) & 3) << 4)) - 32;
     const int sc = (int)(int8_t)blk[192 + 8 * h + (pos >> 4) + 2 * group];
     const float d = jl_half_bits_to_float(blk[208] | (blk[209] << 8));
-    out[e] = __fmul_rn(__fmul_rn(d, (float)sc), (float)q);
+    out[e] = jl_mul_rn(jl_mul_rn(d, (float)sc), (float)q);
 }
 
 // J/tensor/standard/Q5_KFloatTensor.java:78-122, one thread per element: ((d * sc) * q) - (dmin * m),
@@ -322,9 +322,9 @@ jl_dequant_q5_k(const uint8_t *__restrict__ w, float *__restrict__ out, int64_t 
     q += ((blk[16 + pos] >> (2 * pair + high)) & 1) * 16;
     int sc, mn;
     jl_q4k_scale_min(hdr[1], hdr[2], hdr[3], 2 * pair + high, sc, mn);
-    float t = __fmul_rn(d, (float)sc);
-    t = __fmul_rn(t, (float)q);
-    out[e] = __fsub_rn(t, __fmul_rn(dmin, (float)mn));
+    float t = jl_mul_rn(d, (float)sc);
+    t = jl_mul_rn(t, (float)q);
+    out[e] = __fsub_rn(t, jl_mul_rn(dmin, (float)mn));
 }
 
 // J/tensor/standard/Q4_1FloatTensor.java:73-94: (nibble * d) + m, Q5_0FloatTensor.java:61-85:
@@ -341,21 +341,21 @@ jl_dequant_nibbles(const uint8_t *__restrict__ w, float *__restrict__ out, int64
         const uint8_t *blk = w + (e >> 5) * 20;
         const uint32_t dm = *(const uint32_t *)blk;
         const int q = (blk[4 + byte_at] >> shift) & 0xF;
-        out[e] = __fadd_rn(__fmul_rn((float)q, jl_half_bits_to_float(dm)), jl_half_bits_to_float(dm >> 16));
+        out[e] = __fadd_rn(jl_mul_rn((float)q, jl_half_bits_to_float(dm)), jl_half_bits_to_float(dm >> 16));
     } else if constexpr (TYPE == JL_Q5_0) {
         const uint8_t *blk = w + (e >> 5) * 22;
         const uint32_t qh = blk[2] | (blk[3] << 8) | (blk[4] << 16) | ((uint32_t)blk[5] << 24);
         const int q = ((blk[6 + byte_at] >> shift) & 0xF) | (int)(((qh >> within) & 1u) << 4);
-        out[e] = __fmul_rn(jl_half_bits_to_float(blk[0] | (blk[1] << 8)), (float)(q - 16));
+        out[e] = jl_mul_rn(jl_half_bits_to_float(blk[0] | (blk[1] << 8)), (float)(q - 16));
     } else {
         const uint8_t *blk = w + (e >> 8) * 136;
         const int g = (int)((e >> 5) & 7);
         const uint2 hdr = *(const uint2 *)blk;
         const int ls = (int)(((hdr.y >> (4 * g)) & 0xFu) | ((((hdr.x >> 16) >> (2 * g)) & 3u) << 4));
-        const float dl = __fmul_rn(jl_half_bits_to_float(hdr.x), (float)(ls - 32));
+        const float dl = jl_mul_rn(jl_half_bits_to_float(hdr.x), (float)(ls - 32));
         const uint32_t q = (blk[8 + 16 * g + byte_at] >> shift) & 0xFu;
         const int kv = (int)(int8_t)(jl_iq4nl_lookup4(q) & 0xFFu);
-        out[e] = __fmul_rn(dl, (float)kv);
+        out[e] = jl_mul_rn(dl, (float)kv);
     }
 }
 

@@ -12,6 +12,10 @@
 //                  an fp32 scale and the sum of the bytes per block: quantizeActivationQ8Blocks
 //                  (J/backend/tornado/kernels/TransformerComputeKernelsQ4_0.java:287-341).
 //
+//   jl_rms_apply_xf16  the batched prefill's normalisation, which hands the projections fp16 rows:
+//                  batchedRmsReduceParallel + batchedRmsApplyFP16
+//                  (J/backend/tornado/kernels/TransformerBatchPrefillKernels.java:1480-1510, 59-72).
+//
 // jl_rms_scale is one workgroup (a few KB of input); jl_argmax spreads the half MB of logits over
 // up to 128 workgroups and folds their results in a second, single-workgroup launch.
 #include "jl_device.h"
@@ -136,7 +140,7 @@ jl_quantize_q8_kernel(const float *__restrict__ x, const float *__restrict__ rms
     float value = i < n ? x[i] : 0.f;
     if constexpr (RMS) {
         if (i < n) {
-            value = __fmul_rn(rms_w[i], __fmul_rn(rms_scale[0], value));
+            value = jl_mul_rn(rms_w[i], jl_mul_rn(rms_scale[0], value));
             xb[i] = value;
         }
     }
@@ -144,7 +148,7 @@ jl_quantize_q8_kernel(const float *__restrict__ x, const float *__restrict__ rms
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) max_abs = fmaxf(max_abs, __shfl_xor(max_abs, o, JL_WAVE));
     const float inverse = max_abs > 0.0f ? __fdiv_rn(127.0f, max_abs) : 0.0f;
-    const float scaled = __fmul_rn(value, inverse);
+    const float scaled = jl_mul_rn(value, inverse);
     int q = (int)__fadd_rn(scaled, scaled >= 0.0f ? 0.5f : -0.5f);
     q = min(127, max(-127, q));
     int sum = q;
@@ -175,6 +179,65 @@ int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *i
     hipLaunchKernelGGL(jl_argmax_scan, dim3(groups), dim3(kArgmaxThreads), 0, ctx->stream, values, (int)n, cells);
     JL_HIP(hipGetLastError());
     hipLaunchKernelGGL(jl_argmax_fold, dim3(1), dim3(kArgmaxGroups), 0, ctx->stream, values, cells, groups, index);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
+}
+
+namespace {
+
+// One workgroup of 256 per activation row, and the reference kernel's own summation order (its
+// local size is 256 too): thread t adds the squares of elements t, t + 256, ... in turn -- product
+// rounded, then the sum -- and the 256 partial sums fold as the tree partial[t] += partial[t + s],
+// s = 128 ... 1.  With correctly rounded division and square root the scale, and so every fp16
+// output, has the bits the reference's source states.  Rows of up to 8192 columns are read once.
+__global__ void __launch_bounds__(256)
+jl_rms_apply_f16_kernel(const float *__restrict__ X, const float *__restrict__ w, float eps, int n,
+                        float *__restrict__ scales, _Float16 *__restrict__ out) {
+    __shared__ float partial[256];
+    constexpr int kHeld = 32;
+    const int tid = threadIdx.x;
+    const float *x = X + (int64_t)blockIdx.x * n;
+    _Float16 *o = out + (int64_t)blockIdx.x * n;
+    const bool held = n <= kHeld * 256;
+    float v[kHeld];
+    float ss = 0.f;
+    if (held) {
+#pragma unroll
+        for (int j = 0; j < kHeld; j++) {
+            const int i = tid + j * 256;
+            v[j] = i < n ? x[i] : 0.f;
+            if (i < n) ss = __fadd_rn(ss, jl_mul_rn(v[j], v[j]));
+        }
+    } else {
+        for (int i = tid; i < n; i += 256) ss = __fadd_rn(ss, jl_mul_rn(x[i], x[i]));
+    }
+    partial[tid] = ss;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (tid < s) partial[tid] = __fadd_rn(partial[tid], partial[tid + s]);
+        __syncthreads();
+    }
+    const float m = __fadd_rn(__fdiv_rn(partial[0], (float)n), eps);
+    // (the square root through double: correctly rounded to fp32, which __fsqrt_rn is not here)
+    const float scale = __fdiv_rn(1.0f, (float)sqrt((double)m));
+    if (tid == 0 && scales) scales[blockIdx.x] = scale;
+    if (held) {
+#pragma unroll
+        for (int j = 0; j < kHeld; j++) {
+            const int i = tid + j * 256;
+            if (i < n) o[i] = (_Float16)jl_mul_rn(jl_mul_rn(w[i], scale), v[j]);
+        }
+    } else {
+        for (int i = tid; i < n; i += 256) o[i] = (_Float16)jl_mul_rn(jl_mul_rn(w[i], scale), x[i]);
+    }
+}
+
+}  // namespace
+
+int jl_launch_rms_apply_f16(jl_context *ctx, const float *X, const float *w, float eps, int64_t rows, int64_t n,
+                            float *scales, _Float16 *out) {
+    hipLaunchKernelGGL(jl_rms_apply_f16_kernel, dim3((unsigned)rows), dim3(256), 0, ctx->stream, X, w, eps, (int)n,
+                       scales, out);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }

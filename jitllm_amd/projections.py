@@ -255,6 +255,15 @@ class QuantizedBatchProjections:
                                            self.workspace.ptr, self.workspace.nbytes, copy.ptr, copy.nbytes,
                                            C.byref(state)))
 
+    def rmsApplyFP16(self, x: FloatArray, rmsWeights: FloatArray, eps: float, out: HalfFloatArray, dim: int,
+                     scales: FloatArray | None = None, activeRows: int | None = None) -> None:
+        """``out[b] = fp16(rmsWeights * scale_b * x[b])`` with ``scale_b`` from the row's mean square:
+        batchedRmsReduceParallel + batchedRmsApplyFP16 (TransformerBatchPrefillKernels.java:1480-1510,
+        59-72), the step that hands the prefill projections their fp16 activations."""
+        rows = self.batchSize if activeRows is None else activeRows
+        L.check(self._lib.jl_rms_apply_xf16(self.context.handle, x.ptr, rmsWeights.ptr, eps, rows, dim,
+                                            scales.ptr if scales is not None else None, out.ptr))
+
     def projection(self, x: FloatArray, out: FloatArray, w: TornadoTensor, n: int, d: int,
                    residual: bool, activeRows: int | None = None) -> None:
         """``out = w . x`` over the batch, or ``out += w . x`` with ``residual``

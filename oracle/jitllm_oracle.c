@@ -834,6 +834,43 @@ void jo_rmsnorm(float *out, const float *x, const float *weight, int64_t n, floa
     }
 }
 
+/*
+ * The batched prefill's normalisation, which hands the projections fp16 activations:
+ * batchedRmsReduceParallel (J/backend/tornado/kernels/TransformerBatchPrefillKernels.java:1480-1510)
+ * with its local size of 256 -- work item t adds the squares of elements t, t + 256, ... in turn,
+ * the 256 partial sums fold as the binary tree partial[t] += partial[t + s], s = 128 ... 1, and
+ * scale = 1.0f / sqrt(partial[0] / dim + eps) in fp32 -- then batchedRmsApplyFP16 (:59-72):
+ * out = FP16(rmsWeights[i] * scale * x[i]), the products taken left to right and rounded to fp32,
+ * the result to the nearest fp16.  `scales` (one per row) may be null.
+ */
+void jo_batched_rms_apply_f16(const float *x, const float *weight, float eps, int64_t rows, int64_t n,
+                              float *scales, uint16_t *out) {
+    enum { LOCAL = 256 };
+    for (int64_t b = 0; b < rows; b++) {
+        const float *row = x + b * n;
+        float partial[LOCAL];
+        for (int t = 0; t < LOCAL; t++) {
+            float ss = 0.0f;
+            for (int64_t i = t; i < n; i += LOCAL) {
+                float sq = row[i] * row[i];
+                ss = ss + sq;
+            }
+            partial[t] = ss;
+        }
+        for (int s = LOCAL / 2; s > 0; s >>= 1)
+            for (int t = 0; t < s; t++) partial[t] = partial[t] + partial[t + s];
+        float m = partial[0] / (float)n;
+        m = m + eps;
+        float scale = 1.0f / sqrtf(m);
+        if (scales) scales[b] = scale;
+        for (int64_t i = 0; i < n; i++) {
+            float ws = weight[i] * scale;
+            float r = ws * row[i];
+            out[b * n + i] = jo_f32_to_f16(r);
+        }
+    }
+}
+
 /* J/tensor/standard/FloatTensor.java:168-181: the first maximum; a NaN never wins a comparison */
 int64_t jo_argmax(const float *x, int64_t n) {
     int64_t max_index = 0;

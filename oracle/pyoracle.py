@@ -70,6 +70,8 @@ def lib() -> C.CDLL:
     L.jo_rms_scale.restype = C.c_float
     L.jo_rmsnorm.argtypes = [_f32p, _f32p, _f32p, C.c_int64, C.c_float]
     L.jo_rmsnorm.restype = None
+    L.jo_batched_rms_apply_f16.argtypes = [_f32p, _f32p, C.c_float, C.c_int64, C.c_int64, _f32p, C.c_void_p]
+    L.jo_batched_rms_apply_f16.restype = None
     L.jo_argmax.argtypes = [_f32p, C.c_int64]
     L.jo_argmax.restype = C.c_int64
     L.jo_quantize_q8.argtypes = [_f32p, _i8p, _f32p, C.c_int64, C.c_int64]
@@ -183,6 +185,18 @@ def rms_scale(x: np.ndarray, eps: float) -> np.float32:
     """CpuOperations.rmsnorm's factor (J/inference/op/CpuOperations.java:60-66)."""
     x = np.ascontiguousarray(x, dtype=np.float32)
     return np.float32(lib().jo_rms_scale(_f32(x), x.size, eps))
+
+
+def batched_rms_apply_f16(x: np.ndarray, weight: np.ndarray, eps: float):
+    """batchedRmsReduceParallel + batchedRmsApplyFP16 (TransformerBatchPrefillKernels.java:1480-1510,
+    59-72) over the rows of ``x``: (scales [rows] fp32, out [rows x n] fp16)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, n = x.shape
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    scales = np.empty(rows, dtype=np.float32)
+    out = np.empty((rows, n), dtype=np.float16)
+    lib().jo_batched_rms_apply_f16(_f32(x), _f32(w), eps, rows, n, _f32(scales), out.ctypes.data)
+    return scales, out
 
 
 def rmsnorm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:

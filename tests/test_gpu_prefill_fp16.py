@@ -224,3 +224,54 @@ def test_xf16_refusals(ctx):
     with pytest.raises(L.JitllmHipError, match="null argument"):
         L.check(ctx._lib.jl_gemm_xf16(ctx.handle, arr, 1, None, out.ptr, 0, T, T, d, 0, L.JL_STORE,
                                       p.workspace.ptr, p.workspace.nbytes, None, 0, None))
+
+
+@pytest.mark.parametrize("rows,n", [(1, 2048), (70, 2048), (600, 1000), (33, 8192), (5, 8448), (3, 16384)])
+def test_rms_apply_to_fp16_has_the_oracles_bits(ctx, rows, n):
+    """batchedRmsReduceParallel + batchedRmsApplyFP16 in one launch: the kernel sums in the
+    reference kernel's own order, so scales and fp16 outputs equal the oracle's bit for bit (rows
+    held in registers up to 8192 columns, re-read beyond; a row length that is no multiple of 256)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("rms apply fp16", rows, n)
+    x = synthetic.activations((rows, n), seed=1800 + n) * np.float32(2.5)
+    x[0, :7] = [0.0, -0.0, 1e-30, 3e4, -3e4, 65504.0, 1e-8]
+    w = np.random.default_rng(1801).uniform(0.5, 1.5, n).astype(np.float32)
+    p = QuantizedBatchProjections(ctx, rows + 2, 256, 256)
+    out = ctx.half_from_numpy(np.full((rows + 2) * n, 7.5, dtype=np.float16))
+    scales = ctx.float_array(rows + 2, fill=UNTOUCHED)
+    p.rmsApplyFP16(ctx.from_numpy(np.concatenate([x, np.zeros((2, n), np.float32)])), ctx.from_numpy(w), 1e-5, out, n,
+                   scales=scales, activeRows=rows)
+    ctx.sync()
+    want_scales, want = O.batched_rms_apply_f16(x, w, 1e-5)
+    got_scales, got = scales.get(), out.get().reshape(rows + 2, n)
+    assert np.array_equal(got_scales[:rows].view(np.uint32), want_scales.view(np.uint32))
+    assert np.all(got_scales[rows:] == UNTOUCHED)
+    assert np.array_equal(got[:rows].view(np.uint16), want.view(np.uint16))
+    assert np.all(got[rows:] == np.float16(7.5))
+
+
+def test_normalise_then_project_in_fp16(ctx):
+    """The prefill plan's first two steps chained on the device -- RMS apply to fp16, then q|k|v over
+    the fp16 rows -- against the oracle's projection of the oracle's fp16 activations."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("rms apply fp16 -> qkv")
+    t, T, n, dq, dkv = O.Q8_0, 512, 2048, 2048, 512
+    raws = [synthetic.weight(t, r, n, seed=1810 + i) for i, r in enumerate((dq, dkv, dkv))]
+    ws = [ctx.load_weight(t, raw, r, n) for raw, r in zip(raws, (dq, dkv, dkv))]
+    x = synthetic.activations((T, n), seed=1813) * np.float32(4.0)
+    w = np.random.default_rng(1814).uniform(0.5, 1.5, n).astype(np.float32)
+    p = QuantizedBatchProjections(ctx, T, n, dq + 2 * dkv)
+    xb16 = ctx.half_array(T * n)
+    qkv = ctx.float_array(T * (dq + 2 * dkv), fill=UNTOUCHED)
+    p.rmsApplyFP16(ctx.from_numpy(x), ctx.from_numpy(w), 1e-5, xb16, n)
+    p.fusedQKV(xb16, qkv, *ws)
+    ctx.sync()
+    _, xb = O.batched_rms_apply_f16(x, w, 1e-5)
+    xb32 = xb.astype(np.float32)
+    got = qkv.get().reshape(T, dq + 2 * dkv)
+    col = 0
+    for raw, r in zip(raws, (dq, dkv, dkv)):
+        assert rel_err(got[:, col:col + r], O.matmul_batch(t, raw, xb32, r, n), magnitude(t, raw, xb32, r, n)) < F16_BOUND
+        col += r

@@ -565,6 +565,64 @@ def test_rmsnorm_is_weight_times_scaled_x():
     assert abs(np.mean(unit.astype(np.float64) ** 2) - 1.0) < 1e-5
 
 
+def test_batched_rms_apply_f16_closed_forms():
+    """batchedRmsReduceParallel + batchedRmsApplyFP16: answers that do not come from the formula.  A
+    row of +-2 has mean square exactly 4, so with eps = 0 the scale is exactly 0.5 and the output
+    is the weight itself (negated where x is -2) rounded to fp16; eps dominating a tiny row gives
+    1/sqrt(eps); a row scaled by a power of two has its scale divided by it and the same output."""
+    n = 1000
+    rng = np.random.default_rng(77)
+    w = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    signs = rng.choice(np.float32([-1.0, 1.0]), n)
+    scales, out = O.batched_rms_apply_f16((2.0 * signs)[None, :], w, 0.0)
+    assert scales[0] == np.float32(0.5)
+    assert np.array_equal(out[0].view(np.uint16), (w * signs).astype(np.float16).view(np.uint16))
+    scales, out = O.batched_rms_apply_f16(np.full((1, n), 1e-20, np.float32), w, 0.25)
+    assert scales[0] == np.float32(2.0)
+    x = rng.standard_normal((3, n)).astype(np.float32)
+    s1, o1 = O.batched_rms_apply_f16(x, w, 0.0)
+    s2, o2 = O.batched_rms_apply_f16(x * np.float32(8.0), w, 0.0)
+    assert np.array_equal(s1, s2 * np.float32(8.0))
+    # (w * s/8) * 8x == (w * s) * x exactly: both factors move by a power of two
+    assert np.array_equal(o1.view(np.uint16), o2.view(np.uint16))
+    # float64 evaluation: the scale to fp32 accuracy, the output to half an fp16 ulp and a little
+    want_scale = 1.0 / np.sqrt(np.mean(x.astype(np.float64) ** 2, axis=1))
+    assert np.all(np.abs(s1 - want_scale) <= 3e-6 * want_scale)
+    want = w.astype(np.float64) * want_scale[:, None] * x
+    assert np.all(np.abs(o1.astype(np.float64) - want) <= np.abs(want) * (2.0 ** -11 + 1e-5) + 2.0 ** -25)
+
+
+def test_batched_rms_apply_f16_summation_order():
+    """The order the reference's kernel states, in a second wording: numpy over the 256 work items at
+    once (element t + 256 j is step j of work item t), the partial sums folded as the tree
+    partial[:s] += partial[s:2s].  A sequential sum, or the products taken right to left, gives
+    other bits on some of these 64 x 4096 values."""
+    rng = np.random.default_rng(78)
+    for n in (4096, 1000):
+        x = (rng.standard_normal((64, n)) * 3.0).astype(np.float32)
+        w = rng.uniform(0.5, 1.5, n).astype(np.float32)
+        eps = np.float32(1e-5)
+        scales, out = O.batched_rms_apply_f16(x, w, float(eps))
+        pad = (-n) % 256
+        for b in range(x.shape[0]):
+            steps = np.concatenate([x[b], np.zeros(pad, np.float32)]).reshape(-1, 256)
+            p = np.zeros(256, np.float32)
+            for j in range(steps.shape[0]):
+                p = p + steps[j] * steps[j]
+            s = 128
+            while s:
+                p[:s] = p[:s] + p[s:2 * s]
+                s //= 2
+            scale = np.float32(1.0) / np.sqrt(np.float32(p[0] / np.float32(n)) + eps)
+            assert scale.dtype == np.float32 and scales[b] == scale
+            want = ((w * scale) * x[b]).astype(np.float16)
+            assert np.array_equal(out[b].view(np.uint16), want.view(np.uint16))
+    # and the order matters: the sequential fp32 sum gives another scale on some rows
+    sums = np.cumsum(x * x, axis=1, dtype=np.float32)[:, -1]
+    seq = np.float32(1.0) / np.sqrt(sums / np.float32(n) + eps)
+    assert seq.dtype == np.float32 and np.any(seq != scales)
+
+
 def test_argmax_first_maximum_and_nan():
     rng = np.random.default_rng(9)
     x = rng.standard_normal(5000).astype(np.float32)
