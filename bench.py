@@ -257,6 +257,26 @@ def bench_gemm(ctx, hip, t, T, steps, warmup):
     # the reference's own operand types on top of that: activations arrive as fp16 (its RMS apply,
     # attention and SwiGLU kernels write fp16) and the hidden vector leaves as fp16
     ms_half = timed(QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=True), X16, H16, hb16)
+    # what hands the projections those fp16 rows: the RMS reduction and fp16 apply of one [T x dim]
+    # activation (two per layer in the model), timed on its own
+    rms_w = ctx.from_numpy(np.ones(DIM, dtype=np.float32))
+    half_proj = QuantizedBatchProjections(ctx, T, DIM, DIM)
+    def rms_apply():
+        # (32 launches per graph: a one-kernel graph measures the graph launch, not the kernel)
+        for _ in range(32):
+            half_proj.rmsApplyFP16(X, rms_w, 1e-5, X16, DIM)
+    rms_apply()
+    ctx.sync()
+    graph = hip.capture(ctx.stream, rms_apply)
+    for _ in range(10):
+        hip.launch(graph, ctx.stream)
+    ctx.sync()
+    e0, e1 = hip.event(), hip.event()
+    hip.record(e0, ctx.stream)
+    for _ in range(steps):
+        hip.launch(graph, ctx.stream)
+    hip.record(e1, ctx.stream)
+    rms_us = hip.elapsed_ms(e0, e1) / steps / 32 * 1e3
     flops = 2.0 * T * (DIM * (DIM + 2 * KV_DIM) + DIM * DIM + 2 * DIM * HIDDEN + HIDDEN * DIM)
     tflops = flops / (ms * 1e-3) / 1e12
     tflops_kept = flops / (ms_kept * 1e-3) / 1e12
@@ -268,7 +288,8 @@ def bench_gemm(ctx, hip, t, T, steps, warmup):
                                         "frac_f16_mfma_peak": round(tflops_kept / F16_MFMA_PEAK_TFLOPS, 4)},
             "with_resident_copy_and_fp16_activations": {
                 "ms_per_layer": round(ms_half, 4), "tflops": round(tflops_half, 1),
-                "frac_f16_mfma_peak": round(tflops_half / F16_MFMA_PEAK_TFLOPS, 4)}}
+                "frac_f16_mfma_peak": round(tflops_half / F16_MFMA_PEAK_TFLOPS, 4),
+                "rms_apply_to_fp16_us": round(rms_us, 2)}}
 
 
 def bench_batched_q4k(ctx, hip, B, steps, warmup):

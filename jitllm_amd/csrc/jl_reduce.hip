@@ -190,23 +190,35 @@ namespace {
 // rounded, then the sum -- and the 256 partial sums fold as the tree partial[t] += partial[t + s],
 // s = 128 ... 1.  With correctly rounded division and square root the scale, and so every fp16
 // output, has the bits the reference's source states.  Rows of up to 8192 columns are read once.
+template <int STEPS>
 __global__ void __launch_bounds__(256)
 jl_rms_apply_f16_kernel(const float *__restrict__ X, const float *__restrict__ w, float eps, int n,
                         float *__restrict__ scales, _Float16 *__restrict__ out) {
     __shared__ float partial[256];
-    constexpr int kHeld = 32;
     const int tid = threadIdx.x;
     const float *x = X + (int64_t)blockIdx.x * n;
     _Float16 *o = out + (int64_t)blockIdx.x * n;
-    const bool held = n <= kHeld * 256;
-    float v[kHeld];
+    // STEPS > 0: the row fits STEPS elements per thread and is read once; every load goes out
+    // before the first sum needs one (a load and its use inside one predicated step would make
+    // the steps wait for each other: a round trip to memory per step)
+    constexpr int HELD = STEPS > 0 ? STEPS : 1;
+    float v[HELD], wv[HELD];
     float ss = 0.f;
-    if (held) {
+    if constexpr (STEPS > 0) {
 #pragma unroll
-        for (int j = 0; j < kHeld; j++) {
+        for (int j = 0; j < HELD; j++) {
             const int i = tid + j * 256;
-            v[j] = i < n ? x[i] : 0.f;
-            if (i < n) ss = __fadd_rn(ss, jl_mul_rn(v[j], v[j]));
+            v[j] = x[i < n ? i : 0];
+        }
+#pragma unroll
+        for (int j = 0; j < HELD; j++) {
+            const int i = tid + j * 256;
+            wv[j] = w[i < n ? i : 0];
+        }
+#pragma unroll
+        for (int j = 0; j < HELD; j++) {
+            const float next = __fadd_rn(ss, jl_mul_rn(v[j], v[j]));
+            ss = tid + j * 256 < n ? next : ss;
         }
     } else {
         for (int i = tid; i < n; i += 256) ss = __fadd_rn(ss, jl_mul_rn(x[i], x[i]));
@@ -221,11 +233,11 @@ jl_rms_apply_f16_kernel(const float *__restrict__ X, const float *__restrict__ w
     // (the square root through double: correctly rounded to fp32, which __fsqrt_rn is not here)
     const float scale = __fdiv_rn(1.0f, (float)sqrt((double)m));
     if (tid == 0 && scales) scales[blockIdx.x] = scale;
-    if (held) {
+    if constexpr (STEPS > 0) {
 #pragma unroll
-        for (int j = 0; j < kHeld; j++) {
+        for (int j = 0; j < HELD; j++) {
             const int i = tid + j * 256;
-            if (i < n) o[i] = (_Float16)jl_mul_rn(jl_mul_rn(w[i], scale), v[j]);
+            if (i < n) o[i] = (_Float16)jl_mul_rn(jl_mul_rn(wv[j], scale), v[j]);
         }
     } else {
         for (int i = tid; i < n; i += 256) o[i] = (_Float16)jl_mul_rn(jl_mul_rn(w[i], scale), x[i]);
@@ -236,8 +248,12 @@ jl_rms_apply_f16_kernel(const float *__restrict__ X, const float *__restrict__ w
 
 int jl_launch_rms_apply_f16(jl_context *ctx, const float *X, const float *w, float eps, int64_t rows, int64_t n,
                             float *scales, _Float16 *out) {
-    hipLaunchKernelGGL(jl_rms_apply_f16_kernel, dim3((unsigned)rows), dim3(256), 0, ctx->stream, X, w, eps, (int)n,
-                       scales, out);
+    const dim3 g((unsigned)rows), b(256);
+    const int ni = (int)n;
+    if (n <= 8 * 256) hipLaunchKernelGGL(jl_rms_apply_f16_kernel<8>, g, b, 0, ctx->stream, X, w, eps, ni, scales, out);
+    else if (n <= 16 * 256) hipLaunchKernelGGL(jl_rms_apply_f16_kernel<16>, g, b, 0, ctx->stream, X, w, eps, ni, scales, out);
+    else if (n <= 32 * 256) hipLaunchKernelGGL(jl_rms_apply_f16_kernel<32>, g, b, 0, ctx->stream, X, w, eps, ni, scales, out);
+    else hipLaunchKernelGGL(jl_rms_apply_f16_kernel<0>, g, b, 0, ctx->stream, X, w, eps, ni, scales, out);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
