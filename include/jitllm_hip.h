@@ -9,7 +9,8 @@
  *   batched prefill J/backend/tornado/ops/Implementation.java + Instance.java (needs/create/emit)
  * Weights are GGUF blocks in the file's own layout (Q8_0 34 B / 32, Q4_0 18 B / 32, Q4_K 144 B /
  * 256; J/format/GGMLType.java:7,13,18-20), uploaded once and never converted.  Activations and
- * outputs are fp32 device buffers that the caller owns and rebinds by value, never by address.
+ * outputs are fp32 device buffers that the caller owns and rebinds by value, never by address
+ * (the batched prefill also takes and leaves the fp16 buffers of the reference's plan: jl_gemm_xf16).
  *
  * Conventions
  *   - every entry point returns JL_OK (0) or a negative jl_status; jl_last_error() then names the
