@@ -326,10 +326,12 @@ int jl_gemm_xf16(jl_context *ctx, const jl_weight *const *weights, int count, co
  * the partial sums fold as a binary tree, scales[b] = 1 / sqrt(sum / n + eps) in fp32 -- then
  * batchedRmsApplyFP16 (:59-72): out[b][i] = fp16(rms_weights[i] * scales[b] * X[b][i]), products
  * left to right in fp32, one rounding to fp16.  X [rows x n] fp32, out [rows x n] binary16;
- * `scales` ([rows]) may be null.
+ * `scales` ([rows]) may be null.  With `delta` ([rows x n], else null) the pending residual add
+ * comes first -- batchedRmsReduceFusedResidual (:1519-1551): X[b][i] += delta[b][i] is written
+ * back and sums and outputs are those of the updated row; without it X is only read.
  */
-int jl_rms_apply_xf16(jl_context *ctx, const float *X, const float *rms_weights, float eps, int64_t rows,
-                      int64_t n, float *scales, uint16_t *out);
+int jl_rms_apply_xf16(jl_context *ctx, float *X, const float *delta, const float *rms_weights, float eps,
+                      int64_t rows, int64_t n, float *scales, uint16_t *out);
 
 /* ---- GGUF files: the caller either side of jl_weight_upload --------------------------------- */
 

@@ -61,7 +61,7 @@ SYMBOLS = {
                                    vp, C.c_size_t, vp, C.c_size_t, C.POINTER(C.c_int32)]),
     "jl_gemm_xf16": (C.c_int, [vp, C.POINTER(vp), C.c_int, vp, vp, C.c_int, i64, i64, i64, i64, C.c_int,
                                vp, C.c_size_t, vp, C.c_size_t, C.POINTER(C.c_int32)]),
-    "jl_rms_apply_xf16": (C.c_int, [vp, vp, vp, C.c_float, i64, i64, vp, vp]),
+    "jl_rms_apply_xf16": (C.c_int, [vp, vp, vp, vp, C.c_float, i64, i64, vp, vp]),
     "jl_gguf_open": (C.c_int, [C.c_char_p, C.POINTER(vp)]),
     "jl_gguf_close": (C.c_int, [vp]),
     "jl_gguf_version": (C.c_int, [vp]),

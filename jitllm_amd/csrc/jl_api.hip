@@ -449,13 +449,13 @@ int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count
                         workspace, workspace_bytes, &r);
 }
 
-int jl_rms_apply_xf16(jl_context *ctx, const float *X, const float *rms_weights, float eps, int64_t rows,
-                      int64_t n, float *scales, uint16_t *out) {
+int jl_rms_apply_xf16(jl_context *ctx, float *X, const float *delta, const float *rms_weights, float eps,
+                      int64_t rows, int64_t n, float *scales, uint16_t *out) {
     JL_REQUIRE(ctx && X && rms_weights && out, "jl_rms_apply_xf16: null argument");
     JL_REQUIRE(rows >= 0 && n > 0 && n <= INT32_MAX && rows <= INT32_MAX, "jl_rms_apply_xf16: %lld rows of %lld",
                (long long)rows, (long long)n);
     if (rows == 0) return JL_OK;
-    return jl_launch_rms_apply_f16(ctx, X, rms_weights, eps, rows, n, scales, (_Float16 *)out);
+    return jl_launch_rms_apply_f16(ctx, X, delta, rms_weights, eps, rows, n, scales, (_Float16 *)out);
 }
 
 int jl_gemm_xf16(jl_context *ctx, const jl_weight *const *weights, int count, const uint16_t *X, void *C,

@@ -106,8 +106,8 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
 // `rms_w` set: xb = rms_w * (rms_scale[0] * x) is written and quantised instead of x.
 int jl_launch_quantize_q8(jl_context *ctx, const float *x, const float *rms_w, const float *rms_scale, float *xb,
                           int64_t n, int8_t *quants, float *scales, int32_t *sums);
-int jl_launch_rms_apply_f16(jl_context *ctx, const float *X, const float *w, float eps, int64_t rows, int64_t n,
-                            float *scales, _Float16 *out);
+int jl_launch_rms_apply_f16(jl_context *ctx, float *X, const float *delta, const float *w, float eps, int64_t rows,
+                            int64_t n, float *scales, _Float16 *out);
 int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const float *x, float *out, int epilogue);
 int jl_launch_dequant_direct(jl_context *ctx, const jl_weight *w, float *out);
 int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale);

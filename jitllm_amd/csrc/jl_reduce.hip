@@ -190,13 +190,16 @@ namespace {
 // rounded, then the sum -- and the 256 partial sums fold as the tree partial[t] += partial[t + s],
 // s = 128 ... 1.  With correctly rounded division and square root the scale, and so every fp16
 // output, has the bits the reference's source states.  Rows of up to 8192 columns are read once.
-template <int STEPS>
+// ADD: the pending residual add first, batchedRmsReduceFusedResidual (:1519-1551): x += delta is
+// written back and everything after it runs over the updated row.
+template <int STEPS, bool ADD>
 __global__ void __launch_bounds__(256)
-jl_rms_apply_f16_kernel(const float *__restrict__ X, const float *__restrict__ w, float eps, int n,
-                        float *__restrict__ scales, _Float16 *__restrict__ out) {
+jl_rms_apply_f16_kernel(float *__restrict__ X, const float *__restrict__ delta, const float *__restrict__ w,
+                        float eps, int n, float *__restrict__ scales, _Float16 *__restrict__ out) {
     __shared__ float partial[256];
     const int tid = threadIdx.x;
-    const float *x = X + (int64_t)blockIdx.x * n;
+    float *x = X + (int64_t)blockIdx.x * n;
+    const float *dl = ADD ? delta + (int64_t)blockIdx.x * n : nullptr;
     _Float16 *o = out + (int64_t)blockIdx.x * n;
     // STEPS > 0: the row fits STEPS elements per thread and is read once; every load goes out
     // before the first sum needs one (a load and its use inside one predicated step would make
@@ -215,13 +218,34 @@ jl_rms_apply_f16_kernel(const float *__restrict__ X, const float *__restrict__ w
             const int i = tid + j * 256;
             wv[j] = w[i < n ? i : 0];
         }
+        if constexpr (ADD) {
+            float dv[HELD];
+#pragma unroll
+            for (int j = 0; j < HELD; j++) {
+                const int i = tid + j * 256;
+                dv[j] = dl[i < n ? i : 0];
+            }
+#pragma unroll
+            for (int j = 0; j < HELD; j++) {
+                const int i = tid + j * 256;
+                v[j] = __fadd_rn(v[j], dv[j]);
+                if (i < n) x[i] = v[j];
+            }
+        }
 #pragma unroll
         for (int j = 0; j < HELD; j++) {
             const float next = __fadd_rn(ss, jl_mul_rn(v[j], v[j]));
             ss = tid + j * 256 < n ? next : ss;
         }
     } else {
-        for (int i = tid; i < n; i += 256) ss = __fadd_rn(ss, jl_mul_rn(x[i], x[i]));
+        for (int i = tid; i < n; i += 256) {
+            float xi = x[i];
+            if constexpr (ADD) {
+                xi = __fadd_rn(xi, dl[i]);
+                x[i] = xi;
+            }
+            ss = __fadd_rn(ss, jl_mul_rn(xi, xi));
+        }
     }
     partial[tid] = ss;
     __syncthreads();
@@ -246,14 +270,20 @@ jl_rms_apply_f16_kernel(const float *__restrict__ X, const float *__restrict__ w
 
 }  // namespace
 
-int jl_launch_rms_apply_f16(jl_context *ctx, const float *X, const float *w, float eps, int64_t rows, int64_t n,
-                            float *scales, _Float16 *out) {
+template <bool ADD>
+static void launch_rms_apply(jl_context *ctx, float *X, const float *delta, const float *w, float eps, int64_t rows,
+                             int n, float *scales, _Float16 *out) {
     const dim3 g((unsigned)rows), b(256);
-    const int ni = (int)n;
-    if (n <= 8 * 256) hipLaunchKernelGGL(jl_rms_apply_f16_kernel<8>, g, b, 0, ctx->stream, X, w, eps, ni, scales, out);
-    else if (n <= 16 * 256) hipLaunchKernelGGL(jl_rms_apply_f16_kernel<16>, g, b, 0, ctx->stream, X, w, eps, ni, scales, out);
-    else if (n <= 32 * 256) hipLaunchKernelGGL(jl_rms_apply_f16_kernel<32>, g, b, 0, ctx->stream, X, w, eps, ni, scales, out);
-    else hipLaunchKernelGGL(jl_rms_apply_f16_kernel<0>, g, b, 0, ctx->stream, X, w, eps, ni, scales, out);
+    if (n <= 8 * 256) hipLaunchKernelGGL((jl_rms_apply_f16_kernel<8, ADD>), g, b, 0, ctx->stream, X, delta, w, eps, n, scales, out);
+    else if (n <= 16 * 256) hipLaunchKernelGGL((jl_rms_apply_f16_kernel<16, ADD>), g, b, 0, ctx->stream, X, delta, w, eps, n, scales, out);
+    else if (n <= 32 * 256) hipLaunchKernelGGL((jl_rms_apply_f16_kernel<32, ADD>), g, b, 0, ctx->stream, X, delta, w, eps, n, scales, out);
+    else hipLaunchKernelGGL((jl_rms_apply_f16_kernel<0, ADD>), g, b, 0, ctx->stream, X, delta, w, eps, n, scales, out);
+}
+
+int jl_launch_rms_apply_f16(jl_context *ctx, float *X, const float *delta, const float *w, float eps, int64_t rows,
+                            int64_t n, float *scales, _Float16 *out) {
+    if (delta) launch_rms_apply<true>(ctx, X, delta, w, eps, rows, (int)n, scales, out);
+    else launch_rms_apply<false>(ctx, X, delta, w, eps, rows, (int)n, scales, out);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }

@@ -256,12 +256,15 @@ class QuantizedBatchProjections:
                                            C.byref(state)))
 
     def rmsApplyFP16(self, x: FloatArray, rmsWeights: FloatArray, eps: float, out: HalfFloatArray, dim: int,
-                     scales: FloatArray | None = None, activeRows: int | None = None) -> None:
+                     scales: FloatArray | None = None, activeRows: int | None = None,
+                     delta: FloatArray | None = None) -> None:
         """``out[b] = fp16(rmsWeights * scale_b * x[b])`` with ``scale_b`` from the row's mean square:
         batchedRmsReduceParallel + batchedRmsApplyFP16 (TransformerBatchPrefillKernels.java:1480-1510,
-        59-72), the step that hands the prefill projections their fp16 activations."""
+        59-72), the step that hands the prefill projections their fp16 activations.  With ``delta``
+        the pending residual add ``x += delta`` comes first (batchedRmsReduceFusedResidual, :1519-1551)."""
         rows = self.batchSize if activeRows is None else activeRows
-        L.check(self._lib.jl_rms_apply_xf16(self.context.handle, x.ptr, rmsWeights.ptr, eps, rows, dim,
+        L.check(self._lib.jl_rms_apply_xf16(self.context.handle, x.ptr, delta.ptr if delta is not None else None,
+                                            rmsWeights.ptr, eps, rows, dim,
                                             scales.ptr if scales is not None else None, out.ptr))
 
     def projection(self, x: FloatArray, out: FloatArray, w: TornadoTensor, n: int, d: int,

@@ -841,13 +841,17 @@ void jo_rmsnorm(float *out, const float *x, const float *weight, int64_t n, floa
  * the 256 partial sums fold as the binary tree partial[t] += partial[t + s], s = 128 ... 1, and
  * scale = 1.0f / sqrt(partial[0] / dim + eps) in fp32 -- then batchedRmsApplyFP16 (:59-72):
  * out = FP16(rmsWeights[i] * scale * x[i]), the products taken left to right and rounded to fp32,
- * the result to the nearest fp16.  `scales` (one per row) may be null.
+ * the result to the nearest fp16.  `scales` (one per row) may be null.  With `delta` the pending
+ * residual add comes first, as in batchedRmsReduceFusedResidual (:1519-1551): x[b][i] += delta[b][i]
+ * is written back and the sums run over the updated row.
  */
-void jo_batched_rms_apply_f16(const float *x, const float *weight, float eps, int64_t rows, int64_t n,
-                              float *scales, uint16_t *out) {
+void jo_batched_rms_apply_f16(float *x, const float *delta, const float *weight, float eps, int64_t rows,
+                              int64_t n, float *scales, uint16_t *out) {
     enum { LOCAL = 256 };
     for (int64_t b = 0; b < rows; b++) {
-        const float *row = x + b * n;
+        float *row = x + b * n;
+        if (delta)
+            for (int64_t i = 0; i < n; i++) row[i] = row[i] + delta[b * n + i];
         float partial[LOCAL];
         for (int t = 0; t < LOCAL; t++) {
             float ss = 0.0f;

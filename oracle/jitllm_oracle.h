@@ -54,8 +54,8 @@ float   jo_rms_scale(const float *x, int64_t n, float eps);
 void    jo_rmsnorm(float *out, const float *x, const float *weight, int64_t n, float eps);
 int64_t jo_argmax(const float *x, int64_t n);
 /* the batched prefill's RMS reduction (parallel order, local size 256) and fp16 apply */
-void    jo_batched_rms_apply_f16(const float *x, const float *weight, float eps, int64_t rows, int64_t n,
-                                 float *scales, uint16_t *out);
+void    jo_batched_rms_apply_f16(float *x, const float *delta, const float *weight, float eps, int64_t rows,
+                                 int64_t n, float *scales, uint16_t *out);
 
 /* per-32-block int8 quantisation of activations and the block-scaled int8 GEMM arithmetic */
 void jo_quantize_q8(const float *x, int8_t *q, float *scales, int64_t rows, int64_t k);

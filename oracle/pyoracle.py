@@ -70,7 +70,7 @@ def lib() -> C.CDLL:
     L.jo_rms_scale.restype = C.c_float
     L.jo_rmsnorm.argtypes = [_f32p, _f32p, _f32p, C.c_int64, C.c_float]
     L.jo_rmsnorm.restype = None
-    L.jo_batched_rms_apply_f16.argtypes = [_f32p, _f32p, C.c_float, C.c_int64, C.c_int64, _f32p, C.c_void_p]
+    L.jo_batched_rms_apply_f16.argtypes = [_f32p, _f32p, _f32p, C.c_float, C.c_int64, C.c_int64, _f32p, C.c_void_p]
     L.jo_batched_rms_apply_f16.restype = None
     L.jo_argmax.argtypes = [_f32p, C.c_int64]
     L.jo_argmax.restype = C.c_int64
@@ -187,15 +187,22 @@ def rms_scale(x: np.ndarray, eps: float) -> np.float32:
     return np.float32(lib().jo_rms_scale(_f32(x), x.size, eps))
 
 
-def batched_rms_apply_f16(x: np.ndarray, weight: np.ndarray, eps: float):
+def batched_rms_apply_f16(x: np.ndarray, weight: np.ndarray, eps: float, delta: np.ndarray | None = None,
+                          updated: list | None = None):
     """batchedRmsReduceParallel + batchedRmsApplyFP16 (TransformerBatchPrefillKernels.java:1480-1510,
-    59-72) over the rows of ``x``: (scales [rows] fp32, out [rows x n] fp16)."""
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    59-72) over the rows of ``x``: (scales [rows] fp32, out [rows x n] fp16).  With ``delta`` the
+    residual add of batchedRmsReduceFusedResidual (:1519-1551) comes first; the updated rows are
+    appended to ``updated`` when a list is given (``x`` itself is never modified)."""
+    x = np.array(x, dtype=np.float32, order="C", copy=True)
     rows, n = x.shape
+    d = None if delta is None else np.ascontiguousarray(delta, dtype=np.float32)
     w = np.ascontiguousarray(weight, dtype=np.float32)
     scales = np.empty(rows, dtype=np.float32)
     out = np.empty((rows, n), dtype=np.float16)
-    lib().jo_batched_rms_apply_f16(_f32(x), _f32(w), eps, rows, n, _f32(scales), out.ctypes.data)
+    lib().jo_batched_rms_apply_f16(_f32(x), None if d is None else _f32(d), _f32(w), eps, rows, n, _f32(scales),
+                                   out.ctypes.data)
+    if updated is not None:
+        updated.append(x)
     return scales, out
 
 

@@ -275,3 +275,26 @@ def test_normalise_then_project_in_fp16(ctx):
     for raw, r in zip(raws, (dq, dkv, dkv)):
         assert rel_err(got[:, col:col + r], O.matmul_batch(t, raw, xb32, r, n), magnitude(t, raw, xb32, r, n)) < F16_BOUND
         col += r
+
+
+@pytest.mark.parametrize("rows,n", [(40, 2048), (7, 3000), (3, 8448)])
+def test_rms_apply_with_the_pending_residual(ctx, rows, n):
+    """batchedRmsReduceFusedResidual folded in: x += delta is written back (active rows only) and
+    scales and fp16 outputs are the oracle's for the updated rows, bit for bit."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("rms apply fp16 + residual", rows, n)
+    x = synthetic.activations((rows + 1, n), seed=1900 + n)
+    delta = synthetic.activations((rows + 1, n), seed=1901 + n) * np.float32(0.25)
+    w = np.random.default_rng(1902).uniform(0.5, 1.5, n).astype(np.float32)
+    p = QuantizedBatchProjections(ctx, rows + 1, 256, 256)
+    dx, out, scales = ctx.from_numpy(x), ctx.half_array((rows + 1) * n), ctx.float_array(rows + 1)
+    p.rmsApplyFP16(dx, ctx.from_numpy(w), 1e-5, out, n, scales=scales, activeRows=rows, delta=ctx.from_numpy(delta))
+    ctx.sync()
+    updated = []
+    want_scales, want = O.batched_rms_apply_f16(x[:rows], w, 1e-5, delta=delta[:rows], updated=updated)
+    got_x = dx.get().reshape(rows + 1, n)
+    assert np.array_equal(got_x[:rows].view(np.uint32), updated[0].view(np.uint32))
+    assert np.array_equal(got_x[rows], x[rows])
+    assert np.array_equal(scales.get()[:rows].view(np.uint32), want_scales.view(np.uint32))
+    assert np.array_equal(out.get().reshape(rows + 1, n)[:rows].view(np.uint16), want.view(np.uint16))

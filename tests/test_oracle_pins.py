@@ -623,6 +623,22 @@ def test_batched_rms_apply_f16_summation_order():
     assert seq.dtype == np.float32 and np.any(seq != scales)
 
 
+def test_batched_rms_apply_f16_with_the_pending_residual():
+    """batchedRmsReduceFusedResidual: the add is one fp32 operation per element, written back, and
+    everything after it is the plain form over the updated rows (numpy does the add here)."""
+    rng = np.random.default_rng(79)
+    x = rng.standard_normal((5, 1000)).astype(np.float32)
+    delta = (rng.standard_normal((5, 1000)) * 0.3).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, 1000).astype(np.float32)
+    kept = x.copy()
+    updated = []
+    s1, o1 = O.batched_rms_apply_f16(x, w, 1e-5, delta=delta, updated=updated)
+    assert np.array_equal(x, kept)
+    assert np.array_equal(updated[0].view(np.uint32), (x + delta).view(np.uint32))
+    s2, o2 = O.batched_rms_apply_f16(x + delta, w, 1e-5)
+    assert np.array_equal(s1.view(np.uint32), s2.view(np.uint32)) and np.array_equal(o1.view(np.uint16), o2.view(np.uint16))
+
+
 def test_argmax_first_maximum_and_nan():
     rng = np.random.default_rng(9)
     x = rng.standard_normal(5000).astype(np.float32)
