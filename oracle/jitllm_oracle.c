@@ -31,6 +31,10 @@
  *                              three per-block formulas.
  *   rmsnorm, argmax            closed forms (constant vectors, powers of two, eps-dominated input), a
  *                              float64 evaluation, numpy's argmax with ties, -inf and NaN cases.
+ *   batched RMS apply to fp16  closed forms (a row of +-2 returns the weights, eps-dominated rows,
+ *                              power-of-two scaling leaves every output bit), a float64 evaluation,
+ *                              and the kernel's summation order restated in numpy over the 256 work
+ *                              items at once, bit for bit; the residual form against numpy's add.
  *   java.util.Random           published first outputs for seeds 0 and 42.
  */
 #include "jitllm_oracle.h"
