@@ -262,13 +262,13 @@ def bench_gemm(ctx, hip, t, T, steps, warmup):
     rms_w = ctx.from_numpy(np.ones(DIM, dtype=np.float32))
     half_proj = QuantizedBatchProjections(ctx, T, DIM, DIM)
     def rms_apply():
-        # (32 launches per graph: a one-kernel graph measures the graph launch, not the kernel)
-        for _ in range(32):
+        # (8 launches per graph: a one-kernel graph measures the graph launch, not the kernel)
+        for _ in range(8):
             half_proj.rmsApplyFP16(X, rms_w, 1e-5, X16, DIM)
     rms_apply()
     ctx.sync()
     graph = hip.capture(ctx.stream, rms_apply)
-    for _ in range(10):
+    for _ in range(3):
         hip.launch(graph, ctx.stream)
     ctx.sync()
     e0, e1 = hip.event(), hip.event()
@@ -276,7 +276,7 @@ def bench_gemm(ctx, hip, t, T, steps, warmup):
     for _ in range(steps):
         hip.launch(graph, ctx.stream)
     hip.record(e1, ctx.stream)
-    rms_us = hip.elapsed_ms(e0, e1) / steps / 32 * 1e3
+    rms_us = hip.elapsed_ms(e0, e1) / steps / 8 * 1e3
     flops = 2.0 * T * (DIM * (DIM + 2 * KV_DIM) + DIM * DIM + 2 * DIM * HIDDEN + HIDDEN * DIM)
     tflops = flops / (ms * 1e-3) / 1e12
     tflops_kept = flops / (ms_kept * 1e-3) / 1e12
