@@ -20,7 +20,7 @@ from typing import Callable, Dict, List, Optional, Sequence
 
 from . import _lib as L
 from .ggml import GGMLType
-from .runtime import Context, DeviceBuffer, FloatArray, HalfFloatArray, TornadoTensor
+from .runtime import Context, DeviceBuffer, FloatArray, HalfFloatArray, ResidentCopies, TornadoTensor
 
 
 class OperationKind(enum.Enum):
@@ -304,7 +304,7 @@ class HipImplementation(Implementation):
             raise RuntimeError("the hip implementation reads the file's blocks, not prepacked tiles")
         need = self.needs(steps, target)
         return HipInstance(context, max(s.tokens for s in steps), DeviceBuffer(context, max(need.bytes, 256)),
-                           self.residency, {})
+                           self.residency, ResidentCopies(context))
 
     def narrowed(self, primary: Instance, steps: Sequence[Step], target: Target, context: Context,
                  prepacking=None) -> Instance:
@@ -314,7 +314,7 @@ class HipImplementation(Implementation):
 
 
 class HipInstance(Instance):
-    def __init__(self, context: Context, batchSize: int, workspace: DeviceBuffer, residency: bool, copies: dict):
+    def __init__(self, context: Context, batchSize: int, workspace: DeviceBuffer, residency: bool, copies: ResidentCopies):
         self.context = context
         self.batchSize = int(batchSize)
         self.workspace = workspace
@@ -323,7 +323,7 @@ class HipInstance(Instance):
         self._lib = context._lib
 
     def buffers(self) -> list:
-        return [self.workspace] + [c for c, _ in self.copies.values()]
+        return [self.workspace] + self.copies.buffers()
 
     def emit(self, step: Step, operands: Operands) -> None:
         """One ``jl_gemm`` per step: q|k|v and gate|up write side by side into the first output's
@@ -344,11 +344,8 @@ class HipInstance(Instance):
         arr = (C.c_void_p * len(weights))(*[w.handle for w in weights])
         copy, state = None, None
         if self.residency:
-            key = tuple(w.handle.value for w in weights) + (epilogue == L.JL_SWIGLU,)
-            if key not in self.copies:
-                nbytes = self._lib.jl_gemm_resident_bytes(arr, len(weights))
-                self.copies[key] = (DeviceBuffer(self.context, nbytes), C.c_int32(0))
-            copy, state = self.copies[key]
+            copy, state = self.copies.lookup(weights, epilogue == L.JL_SWIGLU,
+                                             lambda: self._lib.jl_gemm_resident_bytes(arr, len(weights)))
         if isinstance(x, HalfFloatArray):
             # the reference's own operand types: fp16 in (DecodedMatMul.java:100-109), fp32 out, or --
             # the feed-forward hidden vector -- fp16 out (batchedFFNSwiGLUFP16Packed)

@@ -15,7 +15,7 @@ from dataclasses import dataclass
 
 from . import _lib as L
 from .ggml import GGMLType
-from .runtime import Context, DeviceBuffer, FloatArray, HalfFloatArray, TornadoTensor
+from .runtime import Context, DeviceBuffer, FloatArray, HalfFloatArray, ResidentCopies, TornadoTensor
 
 FUSED_GATE_UP_TYPES = (GGMLType.Q8_0, GGMLType.Q4_0, GGMLType.Q4_K)
 
@@ -217,7 +217,7 @@ class QuantizedBatchProjections:
         # the reference's residency choice for the batched prefill (BatchPrefillWorkspace;
         # dequantize*ToFP16Once): an fp16 copy per set of weights that outlives the call
         self.resident = bool(resident)
-        self._copies: dict = {}
+        self._copies = ResidentCopies(context)
 
     def workspace_bytes(self) -> int:
         return self.workspace.nbytes
@@ -230,11 +230,8 @@ class QuantizedBatchProjections:
         arr = (C.c_void_p * len(weights))(*[w.handle for w in weights])
         copy, state = None, None
         if self.resident:
-            key = tuple(w.handle.value for w in weights) + (epilogue == L.JL_SWIGLU,)
-            if key not in self._copies:
-                nbytes = self._lib.jl_gemm_resident_bytes(arr, len(weights))
-                self._copies[key] = (DeviceBuffer(self.context, nbytes), C.c_int32(0))
-            copy, state = self._copies[key]
+            copy, state = self._copies.lookup(weights, epilogue == L.JL_SWIGLU,
+                                              lambda: self._lib.jl_gemm_resident_bytes(arr, len(weights)))
         if isinstance(x, HalfFloatArray):
             # fp16 activations, the operand type of the reference's prefill GEMMs (gemmMMA's
             # HalfFloatArray A); an fp16 ``out`` is the hidden vector batchedFFNSwiGLUFP16Packed writes

@@ -201,3 +201,35 @@ class TornadoTensor:
         res = out.get().reshape(self.rows, self.cols)
         out.free()
         return res
+
+
+class ResidentCopies:
+    """The fp16 copies jl_gemm_resident keeps per set of weights, keyed on the weight objects.
+
+    An entry holds strong references to its ``TornadoTensor`` objects, so neither their identity nor
+    their jl_weight address can be handed to another weight while the entry lives; an entry whose
+    weights were freed is dropped (its device buffer with it) the next time the cache is asked, so a
+    copy never outlives the weights it was decoded from."""
+
+    def __init__(self, context: Context):
+        self.context = context
+        self._entries: dict = {}
+
+    def lookup(self, weights, swiglu: bool, nbytes_of) -> tuple:
+        """(device buffer, int32 state) for this set of weights; ``nbytes_of()`` sizes a new one."""
+        dead = [k for k, (ws, _, _) in self._entries.items() if any(not w.handle for w in ws)]
+        for k in dead:
+            self._entries.pop(k)[1].free()
+        if any(not w.handle for w in weights):
+            raise ValueError("a freed weight was passed to a resident projection")
+        key = tuple(id(w) for w in weights) + (bool(swiglu),)
+        if key not in self._entries:
+            self._entries[key] = (tuple(weights), DeviceBuffer(self.context, nbytes_of()), C.c_int32(0))
+        _, copy, state = self._entries[key]
+        return copy, state
+
+    def buffers(self) -> list:
+        return [copy for _, copy, _ in self._entries.values()]
+
+    def __len__(self) -> int:
+        return len(self._entries)
