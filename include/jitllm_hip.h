@@ -285,8 +285,11 @@ int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const f
  * `*resident_state` says the buffer already holds what they need.  The caller owns one buffer of
  * jl_gemm_resident_bytes(weights, count) bytes (2 per weight) and one int32 per set of weights it
  * passes together, zeroes the int before the first call and whenever the weights' contents change,
- * and never shares a buffer between different sets.  Calls that do not decode ignore both.  Results
- * are the same as jl_gemm's, bit for bit.
+ * and never shares a buffer between different sets.  The state records the layout of the copy, not
+ * whose weights it holds: reset *resident_state to 0 whenever the set of weights behind the buffer
+ * changes -- also when a weight is freed and another one is uploaded in its place, even if the new
+ * jl_weight comes back at the old address.  Calls that do not decode ignore both.  Results are the
+ * same as jl_gemm's, bit for bit.
  */
 size_t jl_gemm_resident_bytes(const jl_weight *const *weights, int count);
 int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
