@@ -199,6 +199,22 @@ int jl_gemv_gate_up_rms(jl_context *ctx, const jl_weight *w1, const jl_weight *w
  */
 int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
 
+/*
+ * jl_argmax for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The
+ * candidates that the first launch hands to the second -- one (value, index) cell per scanning
+ * workgroup, 1 KiB -- live in a device array that is part of the library's code object, so neither
+ * this call nor anything it relies on (hipMalloc, hipFree, an allocating library routine) allocates;
+ * jl_argmax keeps them in memory that jl_context_create allocated.  The result is jl_argmax's.
+ *   - at most JL_ARGMAX_STATIC_MAX_VALUES values; more is JL_ERR_INVALID, use jl_argmax.
+ *   - every call on one GPU shares that GPU's array, whatever the context or stream: calls that
+ *     overlap on one GPU race.  Calls ordered on one stream do not; a call reads no cell it has
+ *     not written itself, so nothing needs clearing between calls.
+ *   - the array's address is looked up per device by jl_context_create (devices 0..63).
+ */
+#define JL_ARGMAX_STATIC_MAX_VALUES ((int64_t)1 << 24)
+int jl_argmax_static(jl_context *ctx, const float *values, int64_t n, int32_t *index);
+
 /* ---- packed-activation ("dp4a") decode: faster, looser -------------------------------------- */
 /*
  * The reference's optional packed-integer decode path (QuantizedProjections.packed(),

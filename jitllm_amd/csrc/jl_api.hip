@@ -37,6 +37,10 @@ static int context_create(int device, hipStream_t borrowed, bool borrow, jl_cont
                        "device %d is %s; this library carries gfx950 (MI355X) code only", device,
                        prop.gcnArchName);
     }
+    {
+        const int st = jl_static_scratch_init(device);   // `device` is current
+        if (st != JL_OK) return st;
+    }
     jl_context *ctx = new (std::nothrow) jl_context();
     JL_REQUIRE(ctx != nullptr, "jl_context_create: host allocation failed");
     ctx->device = device;
@@ -358,6 +362,14 @@ int jl_gemv_gate_up_q8(jl_context *ctx, const jl_weight *w1, const jl_weight *w3
 int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
     JL_REQUIRE(ctx && values && index && n > 0 && n <= INT32_MAX, "jl_argmax: bad argument");
     return jl_launch_argmax(ctx, values, n, index);
+}
+
+int jl_argmax_static(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
+    JL_REQUIRE(ctx && values && index, "jl_argmax_static: null argument");
+    JL_REQUIRE(n > 0, "jl_argmax_static: %lld values", (long long)n);
+    JL_REQUIRE(n <= JL_ARGMAX_STATIC_MAX_VALUES, "jl_argmax_static: %lld values, at most %lld (use jl_argmax)",
+               (long long)n, (long long)JL_ARGMAX_STATIC_MAX_VALUES);
+    return jl_launch_argmax_static(ctx, values, n, index);
 }
 
 int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count) {

@@ -112,6 +112,12 @@ int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const float *x, f
 int jl_launch_dequant_direct(jl_context *ctx, const jl_weight *w, float *out);
 int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale);
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
+// jl_argmax with its (value, index) cells in a device array that is part of the library's code
+// object instead of the context's allocation.  jl_static_scratch_init looks that array's address
+// up on the current device (once per device; jl_context_create calls it).
+#define JL_MAX_DEVICES 64
+int jl_static_scratch_init(int device);
+int jl_launch_argmax_static(jl_context *ctx, const float *values, int64_t n, int32_t *index);
 int jl_launch_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
 int jl_launch_fill(jl_context *ctx, float *dst, float value, size_t count);
 // A caller-owned fp16 copy of one projection's weights that outlives the call: decoded when

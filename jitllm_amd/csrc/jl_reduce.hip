@@ -171,16 +171,52 @@ int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, f
     return JL_OK;
 }
 
-int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
-    static_assert(sizeof(ArgmaxCells) <= JL_CONTEXT_SCRATCH_BYTES, "argmax cells exceed the context scratch");
+static int argmax_launches(jl_context *ctx, const float *values, int64_t n, int32_t *index, ArgmaxCells *cells) {
     int groups = (int)((n / 4 + kArgmaxThreads - 1) / kArgmaxThreads);
     groups = groups < 1 ? 1 : groups > kArgmaxGroups ? kArgmaxGroups : groups;
-    ArgmaxCells *cells = (ArgmaxCells *)ctx->scratch;
+    // the fold reads cells 0 .. groups - 1 only, all of them written by this call's scan: whatever an
+    // earlier call left in the cells is never looked at, so nothing has to be cleared
     hipLaunchKernelGGL(jl_argmax_scan, dim3(groups), dim3(kArgmaxThreads), 0, ctx->stream, values, (int)n, cells);
     JL_HIP(hipGetLastError());
     hipLaunchKernelGGL(jl_argmax_fold, dim3(1), dim3(kArgmaxGroups), 0, ctx->stream, values, cells, groups, index);
     JL_HIP(hipGetLastError());
     return JL_OK;
+}
+
+int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
+    static_assert(sizeof(ArgmaxCells) <= JL_CONTEXT_SCRATCH_BYTES, "argmax cells exceed the context scratch");
+    return argmax_launches(ctx, values, n, index, (ArgmaxCells *)ctx->scratch);
+}
+
+// ---- jl_argmax_static: the same two launches with the cells in a device array of the library ----
+//
+// `scratch` lives in the code object: every device the library runs on holds its own copy at its
+// own address from the moment the code object is loaded there until the process ends.  In host code
+// the name is only a handle for hipGetSymbolAddress; the kernels take the address that call returns.
+#define JL_STATIC_SCRATCH_BYTES 1024
+static __device__ __align__(256) unsigned char scratch[JL_STATIC_SCRATCH_BYTES];
+static_assert(sizeof(ArgmaxCells) <= JL_STATIC_SCRATCH_BYTES, "argmax cells exceed the static scratch");
+
+static void *g_static_scratch[JL_MAX_DEVICES] = {};   // device address of `scratch`, per device
+
+int jl_static_scratch_init(int device) {
+    if (device < 0 || device >= JL_MAX_DEVICES) return JL_OK;   // such a device simply has no jl_argmax_static
+    if (__atomic_load_n(&g_static_scratch[device], __ATOMIC_ACQUIRE)) return JL_OK;
+    void *ptr = nullptr;
+    JL_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));   // the caller made `device` current
+    if (!ptr) return jl_fail(JL_ERR_HIP, "hipGetSymbolAddress returned a null address for the static scratch");
+    __atomic_store_n(&g_static_scratch[device], ptr, __ATOMIC_RELEASE);
+    return JL_OK;
+}
+
+int jl_launch_argmax_static(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
+    void *cells = ctx->device >= 0 && ctx->device < JL_MAX_DEVICES
+                      ? __atomic_load_n(&g_static_scratch[ctx->device], __ATOMIC_ACQUIRE) : nullptr;
+    if (!cells) {
+        return jl_fail(JL_ERR_UNSUPPORTED, "jl_argmax_static: device %d has no static scratch (the library keeps one "
+                       "for devices 0..%d, set up by jl_context_create)", ctx->device, JL_MAX_DEVICES - 1);
+    }
+    return argmax_launches(ctx, values, n, index, (ArgmaxCells *)cells);
 }
 
 namespace {
