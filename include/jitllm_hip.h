@@ -271,7 +271,7 @@ int jl_gemv_gate_up_q8(jl_context *ctx, const jl_weight *w1, const jl_weight *w3
  * more, the reference's dequantize-then-gemmMMA prefill shape -- an fp16 copy of the call's
  * weights, decoded afresh by every such call and dead after it.  A smaller workspace that still
  * holds the first two is accepted; such calls simply keep to one pass and do not cut K.  Calls of
- * at most 32 rows read X directly and use only the partial sums.
+ * at most 64 rows read X directly and use only the partial sums.
  */
 size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols, int math);
 

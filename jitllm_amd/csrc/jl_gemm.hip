@@ -945,8 +945,8 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const size_t plane_bytes = workspace_bytes > head ? workspace_bytes - head : 0;
 
 
-    if (rows <= 32 && jl_has_fused_kernels(type) && !X16) {
-        // batched decode of up to 32 rows: the weight-streaming kernel reads X itself
+    if (rows <= 64 && jl_has_fused_kernels(type) && !X16) {
+        // batched decode of up to 64 rows: the weight-streaming kernel reads X itself
         bool taken = false;
         int st = jl_launch_gemm_skinny(ctx, weights, count, X, C, rows, ldo, col_offset, epilogue, planes,
                                        plane_bytes, &taken);

@@ -7,16 +7,30 @@
 // With so few rows the call is bound by reading the weights once, exactly like the single-token
 // matrix-vector kernels, so this kernel has their shape: a workgroup walks tiles of 16 weight rows,
 // a tile is copied into an LDS ring by LDS-DMA while the previous one is computed, and a thread
-// owns one 64-column slice of its weight row.  What differs is the arithmetic: the thread decodes
-// its slice to fp16 in registers -- eight fragments of eight consecutive columns -- and a wave (16
-// rows x 4 slices) multiplies them with the matching activation fragments on
-// v_mfma_f32_16x16x32_f16.  The MFMA sums over 32 "k slots"; slot (g, e) of MFMA i is column
-// 64 (slice of lane group g) + 8 i + e, the same for both operands, so no data crosses lanes.
+// owns one 64-column slice of its weight row.  What differs is the arithmetic: the thread turns its
+// slice into eight fp16 fragments of eight consecutive columns in registers, and a wave (16 rows x
+// 4 slices) multiplies them with the matching activation fragments on v_mfma_f32_16x16x32_f16.  The
+// MFMA sums over 32 "k slots"; slot (g, e) of MFMA i is column 64 (slice of lane group g) + 8 i + e,
+// the same for both operands, so no data crosses lanes.  The activations are the MFMA's row operand
+// and the weights its column operand: a lane's four results belong to the weight row it decoded.
+//
+// Q8_0 / Q4_0 fragments are the decoded weights (q - bias) * d rounded once to fp16.  Q4_K fragments
+// are the exact integers sc * q (at most 945): a wave's four slices are the four nibble pairs of one
+// super-block, so d and dmin are common to everything its eight MFMAs add up and are applied to
+// their result -- the reference's blockDot formulation, TransformerComputeKernelsQ4_K.java:270-373 --
+// and the minimum term sum_j m_j * (sum of x over sub-block j) is a ninth MFMA over the sub-blocks'
+// activation sums.  That is 1.4 vector instructions per weight instead of 3, and no weight is
+// rounded at all.
+//
 // The activation fragments (read as fp32 and rounded to fp16 by the kernel itself) depend on the
 // slice only and stay in registers for the whole kernel.  A wave's result is a partial sum over its
 // 256 columns; a wave of its own folds the compute waves' partials through LDS one tile later and
 // applies the epilogue, rows wider than the workgroup's span are cut across workgroups and folded
-// by jl_skinny_reduce.
+// by jl_skinny_reduce.  Calls of 33..64 rows run as two row blocks of up to 32 on the two halves of
+// the chip; the halves walk the same tiles at the same time, so the second reader of a tile finds
+// it in the L2 of its XCD.
+#include <stdlib.h>
+
 #include "jl_device.h"
 #include "jl_internal.h"
 
@@ -50,7 +64,21 @@ struct SkinnyParams {
     int Z;                    // spans per row
     int span_bytes;           // bytes of a weight row inside one span
     int stages;               // depth of the tile ring
+    int row_blocks;           // gridDim.y: blocks of 16 NBB activation rows, each on its own workgroups
+#ifdef JL_SKINNY_PROBE
+    int probe;                // timing experiments: parts of the kernel switched off
+    uint32_t *stamps;         // cycle stamps of workgroup 8: [wave][96]
+    int lds_total;
+#endif
 };
+#ifdef JL_SKINNY_PROBE
+#define PROBE(x) (p.probe == (x))
+#define STAMP(slot) do { if (p.stamps && blockIdx.x == 8 && blockIdx.y == 0) { const uint32_t t_ = (uint32_t)__builtin_readcyclecounter(); \
+    if (lane == 0 && (slot) < 96) asm volatile("ds_write_b32 %0, %1" :: "v"(lds0 + p.lds_total + 4 * (wave * 96 + (slot))), "v"(t_) : "memory"); } } while (0)
+#else
+#define PROBE(x) false
+#define STAMP(slot) do { } while (0)
+#endif
 
 #define JL_WAIT_VM(N) \
     __builtin_amdgcn_s_waitcnt(((N)&0xF) | (((N) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
@@ -141,19 +169,26 @@ __device__ __forceinline__ half8 frag_scaled(uint32_t q0, uint32_t q1, h2 bias, 
     return half8{a[0], a[1], b[0], b[1], c[0], c[1], e[0], e[1]};
 }
 
-// eight nibbles (two dwords of bytes 0..15) -> q * ds - dm, fused
-__device__ __forceinline__ half8 frag_affine(uint32_t q0, uint32_t q1, h2 ds, h2 dm) {
-    const h2 bias = {(_Float16)1024.f, (_Float16)1024.f};
-    h2 a = (bytes_to_h2(q0, 0x00050004u) - bias) * ds - dm;
-    h2 b = (bytes_to_h2(q0, 0x00070006u) - bias) * ds - dm;
-    h2 c = (bytes_to_h2(q1, 0x00050004u) - bias) * ds - dm;
-    h2 e = (bytes_to_h2(q1, 0x00070006u) - bias) * ds - dm;
+// eight nibbles (two dwords of bytes 0..15) -> the exact integers q * sc: (1024 + q) * sc - 1024 sc
+// in one fused step, so the only rounding would be that of the (exact) result
+__device__ __forceinline__ half8 frag_times(uint32_t q0, uint32_t q1, h2 sc, h2 off) {
+    h2 a = __builtin_elementwise_fma(bytes_to_h2(q0, 0x00050004u), sc, off);
+    h2 b = __builtin_elementwise_fma(bytes_to_h2(q0, 0x00070006u), sc, off);
+    h2 c = __builtin_elementwise_fma(bytes_to_h2(q1, 0x00050004u), sc, off);
+    h2 e = __builtin_elementwise_fma(bytes_to_h2(q1, 0x00070006u), sc, off);
     return half8{a[0], a[1], b[0], b[1], c[0], c[1], e[0], e[1]};
 }
 
+// What a Q4_K slice needs beside its fragments: the super-block's d and dmin (applied to the MFMA
+// results) and the two sub-blocks' minimums as the k slots of the minimum MFMA.
+struct Q4KTail {
+    float d, dmin;
+    half8 mins;   // {m0, m0, m1, m1, 0, 0, 0, 0}: each minimum meets its sub-block's activation sum as hi + lo
+};
+
 // Decodes the 64-column slice `sl` of the tile row at LDS address `row`.
 template <int TYPE>
-__device__ __forceinline__ void decode_slice(uint32_t row, int sl, half8 (&f)[8]) {
+__device__ __forceinline__ void decode_slice(uint32_t row, int sl, half8 (&f)[8], Q4KTail &tail) {
     if constexpr (TYPE == JL_Q8_0) {
         // 68 bytes: scale A | 32 quants A | scale B | 32 quants B
         uint32_t w[17];
@@ -193,29 +228,73 @@ __device__ __forceinline__ void decode_slice(uint32_t row, int sl, half8 (&f)[8]
         }
     } else {
         // a quarter of a super-block: 32 nibble bytes; low nibbles are sub-block 2 pair (columns
-        // 0..31 of the slice), high nibbles sub-block 2 pair + 1; w = (d sc) q - (dmin m)
+        // 0..31 of the slice), high nibbles sub-block 2 pair + 1; w = d (sc q) - dmin m
         uint4 h, q0, q1;
         const uint32_t sb = row + (sl >> 2) * 144;
         const int pair = sl & 3;
         lds_read_q4k(sb, sb + 16 + pair * 32, h, q0, q1);
-        const float d = jl_half_bits_to_float(h.x);
-        const float dmin = jl_half_bits_to_float(h.x >> 16);
-        int sc0, mn0, sc1, mn1;
-        jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair, sc0, mn0);
-        jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair + 1, sc1, mn1);
-        const _Float16 ds0 = (_Float16)(d * (float)sc0), dm0 = (_Float16)(dmin * (float)mn0);
-        const _Float16 ds1 = (_Float16)(d * (float)sc1), dm1 = (_Float16)(dmin * (float)mn1);
-        const h2 s0 = {ds0, ds0}, m0 = {dm0, dm0}, s1 = {ds1, ds1}, m1 = {dm1, dm1};
+        tail.d = jl_half_bits_to_float(h.x);
+        tail.dmin = jl_half_bits_to_float(h.x >> 16);
+        // the scales / minimums of sub-blocks 2 pair and 2 pair + 1, two to a register (bytes 0 and
+        // 1): sub-blocks 0..3 keep them in the low six bits of bytes j and j + 4, sub-blocks 4..7
+        // in the nibbles of byte j + 4 with bits 4..5 in the top bits of bytes j - 4 and j
+        // (Q4_KFloatTensor.getScaleK4 / getMinK4, J/tensor/standard/Q4_KFloatTensor.java:68-85)
+        const int sh = 16 * (pair & 1);
+        const uint32_t a = h.y >> sh, b = h.z >> sh, c = h.w >> sh;
+        const uint32_t sc2 = pair < 2 ? (a & 0x3F3Fu) : ((c & 0x0F0Fu) | ((a >> 2) & 0x3030u));
+        const uint32_t mn2 = pair < 2 ? (b & 0x3F3Fu) : (((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u));
+        // small integers as fp16: bits 0x6400 | v are 1024 + v
+        const h2 k1024 = {(_Float16)1024.f, (_Float16)1024.f};
+        const h2 s0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(sc2, 0x64646464u, 0x00040004u)) - k1024;
+        const h2 s1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(sc2, 0x64646464u, 0x00050005u)) - k1024;
+        const h2 m01 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(mn2, 0x64646464u, 0x00040004u)) - k1024;
+        const h2 m11 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(mn2, 0x64646464u, 0x00050005u)) - k1024;
+        const _Float16 z = (_Float16)0.f;
+        tail.mins = half8{m01[0], m01[1], m11[0], m11[1], z, z, z, z};
+        const h2 o0 = s0 * h2{(_Float16)-1024.f, (_Float16)-1024.f};   // exact: at most 63 * 1024
+        // the high nibbles stay where they are: a byte 16 q is 1024 + 16 q, times sc / 16 (exact)
+        const h2 s1x = s1 * h2{(_Float16)0.0625f, (_Float16)0.0625f};
+        const h2 o1 = s1 * h2{(_Float16)-64.f, (_Float16)-64.f};
         const uint32_t qs[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            f[i] = frag_affine(qs[2 * i] & 0x0F0F0F0Fu, qs[2 * i + 1] & 0x0F0F0F0Fu, s0, m0);
-            f[4 + i] = frag_affine((qs[2 * i] >> 4) & 0x0F0F0F0Fu, (qs[2 * i + 1] >> 4) & 0x0F0F0F0Fu, s1, m1);
+            f[i] = frag_times(qs[2 * i] & 0x0F0F0F0Fu, qs[2 * i + 1] & 0x0F0F0F0Fu, s0, o0);
+            f[4 + i] = frag_times(qs[2 * i] & 0xF0F0F0F0u, qs[2 * i + 1] & 0xF0F0F0F0u, s1x, o1);
         }
     }
 }
 
-__device__ __forceinline__ float skinny_swiglu(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
+// t[a] of lane group g (lanes 16 g .. 16 g + 15)  <-  t[g] of lane group a, for the four dwords
+// of each float4: two swaps of lane halves (lane bit 5 against a's high bit), then two swaps of
+// lane quarters (lane bit 4 against a's low bit).
+__device__ __forceinline__ void lane_group_transpose(float4 (&t)[4]) {
+    uint32_t v[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+        v[a][0] = __float_as_uint(t[a].x); v[a][1] = __float_as_uint(t[a].y);
+        v[a][2] = __float_as_uint(t[a].z); v[a][3] = __float_as_uint(t[a].w);
+    }
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+#pragma unroll
+        for (int a0 = 0; a0 < 2; a0++) {   // upper lanes of t[a0] <-> lower lanes of t[2 + a0]
+            const auto r = __builtin_amdgcn_permlane32_swap(v[a0][d], v[2 + a0][d], false, false);
+            v[a0][d] = r[0];
+            v[2 + a0][d] = r[1];
+        }
+#pragma unroll
+        for (int a1 = 0; a1 < 2; a1++) {   // odd lane groups of t[2 a1] <-> even lane groups of t[2 a1 + 1]
+            const auto r = __builtin_amdgcn_permlane16_swap(v[2 * a1][d], v[2 * a1 + 1][d], false, false);
+            v[2 * a1][d] = r[0];
+            v[2 * a1 + 1][d] = r[1];
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+        t[a] = float4{__uint_as_float(v[a][0]), __uint_as_float(v[a][1]), __uint_as_float(v[a][2]), __uint_as_float(v[a][3])};
+}
+
+__device__ __forceinline__ float skinny_swiglu(float g, float u) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u; }
 
 // Workgroup = 16 Ss compute threads (Ss / 4 waves) + kDmaWaves waves that do nothing but copy tiles.
 // An LDS-DMA load holds its wave at issue while the memory system is busy; issued from the compute
@@ -242,6 +321,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int z = blockIdx.x % p.Z;            // this workgroup's run of ZIN spans
+    const int row0 = blockIdx.y * (16 * NBB);  // first activation row of this workgroup's row block
     const int lds_row = p.span_bytes + 16;
     const int slots_per_row = lds_row >> 4;
     const int n_loads = (kGroup * slots_per_row + 64 * kDmaWaves - 1) / (64 * kDmaWaves);
@@ -278,7 +358,9 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     // my groups: wg, wg + stride, ... (workgroups of one span share a stride)
     const int wg = blockIdx.x / p.Z;
     const int stride = gridDim.x / p.Z;
-    const int mine = wg < total_groups ? (total_groups - wg + stride - 1) / stride : 0;
+    int mine = wg < total_groups ? (total_groups - wg + stride - 1) / stride : 0;
+    if (PROBE(4)) return;          // launch only
+    if (PROBE(3)) mine = 0;        // launch + activation prologue
 
     if (wave >= waves && wave < waves + kDmaWaves) {
         // ---- copy waves.  Slot s of a tile is 16 bytes at LDS offset 16 s: row s / slots_per_row,
@@ -294,18 +376,26 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         // (a gate/up call has one segment).  An issue is then one 64-bit add and the load.
         int slot_in[LD], slot_wrow[LD];
         int64_t slot_off[LD], slot_off_row0[LD];
+        // slot (j kDmaWaves + dw) 64 + lane: one division for j = 0, then steps of 64 kDmaWaves slots
+        const int step_rows = (64 * kDmaWaves) / slots_per_row, step_within = (64 * kDmaWaves) % slots_per_row;
+        int srow = (dw * 64 + lane) / slots_per_row;
+        int swithin = dw * 64 + lane - srow * slots_per_row;
+        const int64_t up_distance = DUAL ? (int64_t)(p.w_up - p.w[0]) : 0;
 #pragma unroll
         for (int j = 0; j < LD; j++) {
-            const int slot = (j * kDmaWaves + dw) * 64 + lane;
-            int row = slot / slots_per_row;
-            int within = slot - row * slots_per_row;
-            row = row < kGroup ? row : kGroup - 1;
-            within = within < span_slots ? within : span_slots - 1;
+            const int row = srow < kGroup ? srow : kGroup - 1;
+            const int within = swithin < span_slots ? swithin : span_slots - 1;
             slot_wrow[j] = DUAL ? (row & 7) : row;
             slot_in[j] = z * ZIN * p.span_bytes + within * 16;
-            const int64_t up = (DUAL && row >= 8) ? (int64_t)(p.w_up - p.w[0]) : 0;
+            const int64_t up = (DUAL && row >= 8) ? up_distance : 0;
             slot_off_row0[j] = up + slot_in[j];
-            slot_off[j] = slot_off_row0[j] + (int64_t)slot_wrow[j] * p.row_bytes;
+            slot_off[j] = slot_off_row0[j] + (int64_t)(slot_wrow[j] * p.row_bytes);
+            srow += step_rows;
+            swithin += step_within;
+            if (swithin >= slots_per_row) {
+                swithin -= slots_per_row;
+                srow++;
+            }
         }
         // tile t = span t % ZIN of group wg + (t / ZIN) stride
         auto issue = [&](int t, int st) {
@@ -321,7 +411,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                 // every row of the group exists (uniform; all groups but a weight's last)
 #pragma unroll
                 for (int j = 0; j < LD; j++) {
-                    if (j >= n_loads) break;
+                    if (j >= n_loads || PROBE(2)) break;
                     __builtin_amdgcn_global_load_lds((gvoid *)(w_gate + slot_off[j]),
                                                      (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, 0);
                 }
@@ -342,16 +432,20 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             issue(issued, next_stage);
             next_stage = next_stage + 1 == p.stages ? 0 : next_stage + 1;
         }
+        STAMP(0);
         for (int t = 0; t < tiles; t++) {
             // tiles issued after tile t may stay in flight
             wait_vm((issued - t - 1) * n_loads);
+            STAMP(1 + 3 * t);
             __builtin_amdgcn_s_barrier();
+            STAMP(2 + 3 * t);
             // the stage of tile t - 1 is free now: every compute wave is past its reads
             if (issued < tiles) {
                 issue(issued, next_stage);
                 next_stage = next_stage + 1 == p.stages ? 0 : next_stage + 1;
                 issued++;
             }
+            STAMP(3 + 3 * t);
         }
         if (mine > 0) __builtin_amdgcn_s_barrier();
         return;
@@ -361,62 +455,61 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         // ---- fold wave.  After the barrier that opens group it + 1 the partial sums of group it
         // (parity it & 1) are complete; they are overwritten two groups later, behind barriers this
         // wave takes part in, so it has one group's time.  A partial is what one lane of one
-        // compute wave held: weight rows 4 (o / 16) .. + 3 of activation row 16 b + o % 16, for
-        // lane o and row block b; in a gate/up group lanes o >= 32 hold the up rows of the outputs
-        // of lane o - 32.  Lane o of this wave adds the waves' partials of its (b, o) in wave
-        // order and applies the epilogue.
+        // compute wave held: weight row o % 16 of the group against activation rows
+        // 16 b + 4 (o / 16) .. + 3, for lane o and row block b; in a gate/up group weight rows 8..15
+        // are the up rows of outputs 0..7.  Lane o of this wave adds the waves' partials of its
+        // (b, o) in wave order and applies the epilogue.
         const int o = lane;
+        const int n = o & 15;
         const int go = o >> 4;
+        // its few instructions go ahead of the compute waves' on the SIMD they share: every
+        // barrier between two folds waits for this wave
+        __builtin_amdgcn_s_setprio(2);
+        float *const c_lane = p.C + (int64_t)(row0 + 4 * go) * p.ldo + p.col_offset + n;
         auto fold = [&](int group, int par) {
             const Segment sg = segment_of(group);
             const uint32_t pbase = lds0 + par * partial_bytes + o * 16;
-            const int local = (group - sg.group_begin) * out_rows + 4 * go;  // first of 4 outputs
+            const int local = (group - sg.group_begin) * out_rows + n;   // output column inside the weight
 #pragma unroll
             for (int b = 0; b < NBB; b++) {
-                if (DUAL && o >= 32) break;
-                floatx4 sum = {0.f, 0.f, 0.f, 0.f}, sum_up = {0.f, 0.f, 0.f, 0.f};
-                for (int w0 = 0; w0 < waves; w0 += 4) {
-                    floatx4 v[4], u[4];
+                // all of the (at most eight) compute waves' partials in one round trip
+                floatx4 v[8], u[8];
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const uint32_t a = pbase + (w0 + j < waves ? w0 + j : w0) * (NBB * 1024) + b * 1024;
-                        asm volatile("ds_read_b128 %0, %1" : "=&v"(v[j]) : "v"(a) : "memory");
-                        if constexpr (DUAL) asm volatile("ds_read_b128 %0, %1 offset:512" : "=&v"(u[j]) : "v"(a) : "memory");
-                    }
-                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
-                    if constexpr (DUAL) asm volatile("" : "+v"(u[0]), "+v"(u[1]), "+v"(u[2]), "+v"(u[3]));
+                for (int j = 0; j < 8; j++) {
+                    const uint32_t a = pbase + (j < waves ? j : 0) * (NBB * 1024) + b * 1024;
+                    asm volatile("ds_read_b128 %0, %1" : "=&v"(v[j]) : "v"(a) : "memory");
+                    // (lanes 56..63 read past their own row block here; in range, and unused)
+                    if constexpr (DUAL) asm volatile("ds_read_b128 %0, %1 offset:128" : "=&v"(u[j]) : "v"(a) : "memory");
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
+                             : : "memory");
+                if constexpr (DUAL)
+                    asm volatile("" : "+v"(u[0]), "+v"(u[1]), "+v"(u[2]), "+v"(u[3]), "+v"(u[4]), "+v"(u[5]), "+v"(u[6]), "+v"(u[7]));
+                floatx4 sum = v[0], sum_up = u[0];
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        if (w0 + j < waves) {
-                            sum += v[j];
-                            if constexpr (DUAL) sum_up += u[j];
-                        }
+                for (int j = 1; j < 8; j++) {
+                    if (j < waves) {
+                        sum += v[j];
+                        if constexpr (DUAL) sum_up += u[j];
                     }
                 }
-                const int m = 16 * b + (o & 15);
+                const int m0 = row0 + 16 * b + 4 * go;   // first of this lane's four activation rows
                 if (p.Z > 1) {
                     // partial sums of this span: [z][row][group * 16 + weight row of the group]
-                    float *pp = p.planes + ((int64_t)z * (16 * NBB) + m) * ((int64_t)total_groups * 16) + group * 16 + 4 * go;
-                    *(floatx4 *)pp = sum;
-                    if constexpr (DUAL) *(floatx4 *)(pp + 8) = sum_up;
+                    float *pp = p.planes + ((int64_t)z * (16 * NBB * p.row_blocks) + m0) * ((int64_t)total_groups * 16) + group * 16 + n;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) pp[(int64_t)e * total_groups * 16] = sum[e];
                     continue;
                 }
-                if (m >= p.rows) continue;
-                float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + sg.col_begin + local;
-                const int left = sg.rows - local;
-                float r[4];
+                if ((DUAL && n >= 8) || local >= sg.rows) continue;
+                float *dst = c_lane + (int64_t)(16 * b) * p.ldo + sg.col_begin + (local - n);
 #pragma unroll
-                for (int e = 0; e < 4; e++) r[e] = DUAL ? skinny_swiglu(sum[e], sum_up[e]) : sum[e];
-                if (p.epilogue == JL_RESIDUAL) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (e < left) unsafeAtomicAdd(dst + e, r[e]);   // one add per element, no load to wait for
-                } else if (left >= 4 && (((uintptr_t)dst) & 15) == 0) {
-                    *(floatx4 *)dst = floatx4{r[0], r[1], r[2], r[3]};
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (e < left) dst[e] = r[e];
+                for (int e = 0; e < 4; e++) {
+                    if (m0 + e >= p.rows) break;
+                    const float r = DUAL ? skinny_swiglu(sum[e], sum_up[e]) : sum[e];
+                    if (p.epilogue == JL_RESIDUAL) unsafeAtomicAdd(dst + e * p.ldo, r);   // one add per element, no load to wait for
+                    else dst[e * p.ldo] = r;
                 }
             }
         };
@@ -424,7 +517,9 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
 #pragma unroll
             for (int q = 0; q < ZIN; q++) {
                 __builtin_amdgcn_s_barrier();
+                STAMP(2 * it);
                 if (q == 0 && it > 0) fold(wg + (it - 1) * stride, (it - 1) & 1);
+                if (q == 0) STAMP(2 * it + 1);
             }
         }
         if (mine > 0) {
@@ -435,53 +530,99 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     }
 
     // ---- compute waves
-    const int c = lane & 15;                   // row of the group
+    const int c = lane & 15;                   // weight row of the group; activation row of a row block
     const int g = lane >> 4;                   // which of the wave's four slices
     const int sl = 4 * wave + g;               // slice inside the span
 
     // Activation fragments: 64 consecutive columns of NBB x 16 rows, kept for the whole kernel.
     // Read as fp32 (while the first tiles are on their way) and rounded to fp16 behind a
     // power-of-two scale per row and wave: the largest magnitude of the row's 256 columns this wave
-    // multiplies is brought into [2^11, 2^12), which keeps huge rows finite and tiny rows out of
-    // fp16's subnormals.  The lane that holds activation row c as an operand also holds the results
-    // of that row (MFMA column c), so the scale is undone lane-locally, exactly.
+    // multiplies is brought into [2^9, 2^10), which keeps huge rows finite, tiny rows out of
+    // fp16's subnormals and the sum of a sub-block's 32 activations inside fp16's range.  The
+    // results of activation row r sit in lane group r / 4 of every weight row's lanes, so each lane
+    // fetches the four scales it has to undo from the lanes that computed them.
+    STAMP(0);
     half8 af[NBB][ZIN][8];
-    float undo[NBB][ZIN];
+    half8 sums[NBB][ZIN];     // Q4_K: the two sub-blocks' activation sums, each as hi + lo, as k slots
+    floatx4 undo[NBB][ZIN];
+    {
+        // Every load of the prologue is issued before the first value is used.  Load n = 4 a + b
+        // of a lane fetches the 16-byte chunk 16 a + 4 b + g of its row's 256 columns, so that the
+        // four lanes of a row read 64 consecutive bytes (a lane reading its own slice chunk by
+        // chunk would touch 64 cache lines per instruction, and the cache looks up one line per
+        // clock: that alone took 4-7 us per launch).  The chunks are then dealt out by transposing
+        // a with g across the lane groups: afterwards register 4 a + b holds chunk 4 b + a of the
+        // lane's own slice.
+        float4 x[NBB * ZIN][16];
 #pragma unroll
-    for (int b = 0; b < NBB; b++) {
+        for (int b = 0; b < NBB; b++) {
 #pragma unroll
-        for (int q = 0; q < ZIN; q++) {
-            const int m = 16 * b + c;
-            float4 x[16];
-            if (m < p.rows) {
-                const float4 *src = (const float4 *)(p.X + (int64_t)m * p.k + 64 * ((z * ZIN + q) * p.Ss + sl));
+            for (int q = 0; q < ZIN; q++) {
+                const int m = row0 + 16 * b + c;
+                float4 raw[16];
+                if (m < p.rows) {
+                    const float4 *src = (const float4 *)(p.X + (int64_t)m * p.k + 64 * ((z * ZIN + q) * p.Ss + 4 * wave)) + g;
 #pragma unroll
-                for (int i = 0; i < 16; i++) x[i] = src[i];
-            } else {
+                    for (int n = 0; n < 16; n++) raw[n] = src[16 * (n >> 2) + 4 * (n & 3)];
+                } else {
 #pragma unroll
-                for (int i = 0; i < 16; i++) x[i] = float4{0.f, 0.f, 0.f, 0.f};
+                    for (int n = 0; n < 16; n++) raw[n] = float4{0.f, 0.f, 0.f, 0.f};
+                }
+#pragma unroll
+                for (int bb = 0; bb < 4; bb++) {
+                    float4 t[4] = {raw[bb], raw[4 + bb], raw[8 + bb], raw[12 + bb]};
+                    lane_group_transpose(t);
+#pragma unroll
+                    for (int a = 0; a < 4; a++) x[b * ZIN + q][4 * bb + a] = t[a];
+                }
             }
-            float amax = 0.f;
+        }
 #pragma unroll
-            for (int i = 0; i < 16; i++)
-                amax = fmaxf(amax, fmaxf(fmaxf(fabsf(x[i].x), fabsf(x[i].y)), fmaxf(fabsf(x[i].z), fabsf(x[i].w))));
-            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-            // amax = 1.f * 2^(E - 127): multiply by 2^(138 - E), undo with 2^(E - 138)
-            int E = (int)((__float_as_uint(amax) >> 23) & 0xFF);
-            E = E < 12 ? 12 : E;
-            const float inv = __uint_as_float((uint32_t)(265 - E) << 23);
-            undo[b][q] = __uint_as_float((uint32_t)(E - 11) << 23);
+        for (int b = 0; b < NBB; b++) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float4 lo = x[2 * i], hi = x[2 * i + 1];
-                af[b][q][i] = half8{(_Float16)(lo.x * inv), (_Float16)(lo.y * inv), (_Float16)(lo.z * inv),
-                                    (_Float16)(lo.w * inv), (_Float16)(hi.x * inv), (_Float16)(hi.y * inv),
-                                    (_Float16)(hi.z * inv), (_Float16)(hi.w * inv)};
+            for (int q = 0; q < ZIN; q++) {
+                const float4 (&xs)[16] = x[b * ZIN + q];
+                float amax = 0.f;
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fabsf(xs[i].x)), __builtin_fabsf(xs[i].y));
+                    amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fabsf(xs[i].z)), __builtin_fabsf(xs[i].w));
+                }
+                amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                // amax = 1.f * 2^(E - 127): multiply by 2^(136 - E), undo with 2^(E - 136)
+                int E = (int)((__float_as_uint(amax) >> 23) & 0xFF);
+                E = E < 12 ? 12 : E;
+                const float inv = __uint_as_float((uint32_t)(263 - E) << 23);
+                const float un = __uint_as_float((uint32_t)(E - 9) << 23);
+#pragma unroll
+                for (int e = 0; e < 4; e++) undo[b][q][e] = __shfl(un, 4 * g + e, 64);
+                float part[2] = {0.f, 0.f};
+                const h2 ones = {(_Float16)1.f, (_Float16)1.f};
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float4 lo = xs[2 * i], hi = xs[2 * i + 1];
+                    const half8 h = half8{(_Float16)(lo.x * inv), (_Float16)(lo.y * inv), (_Float16)(lo.z * inv),
+                                          (_Float16)(lo.w * inv), (_Float16)(hi.x * inv), (_Float16)(hi.y * inv),
+                                          (_Float16)(hi.z * inv), (_Float16)(hi.w * inv)};
+                    af[b][q][i] = h;
+                    if constexpr (TYPE == JL_Q4_K) {
+                        // sums of the values the MFMAs will see: at most 32 x 2^10, exact in fp32
+#pragma unroll
+                        for (int e = 0; e < 8; e += 2)
+                            part[i >> 2] = __builtin_amdgcn_fdot2(h2{h[e], h[e + 1]}, ones, part[i >> 2], false);
+                    }
+                }
+                if constexpr (TYPE == JL_Q4_K) {
+                    const _Float16 z16 = (_Float16)0.f;
+                    const _Float16 h0 = (_Float16)part[0], h1 = (_Float16)part[1];
+                    sums[b][q] = half8{h0, (_Float16)(part[0] - (float)h0), h1, (_Float16)(part[1] - (float)h1), z16, z16, z16, z16};
+                }
             }
         }
     }
 
+    STAMP(1);
     for (int it = 0; it < mine; it++) {
         floatx4 total[NBB];
 #pragma unroll
@@ -489,27 +630,51 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
 #pragma unroll
         for (int q = 0; q < ZIN; q++) {
             const int t = it * ZIN + q;
+            STAMP(2 + 4 * t);
             __builtin_amdgcn_s_barrier();   // tile t has landed; the fold wave takes the sums of group it - 1
+            STAMP(3 + 4 * t);
 
+            if (PROBE(1)) continue;   // copy only
             half8 wf[8];
-            decode_slice<TYPE>(ring0 + (t % p.stages) * stage_bytes + c * lds_row, sl, wf);
+            Q4KTail tail;
+            decode_slice<TYPE>(ring0 + (t % p.stages) * stage_bytes + c * lds_row, sl, wf, tail);
+            asm volatile("" : "+v"(wf[0]), "+v"(wf[7]));
+            STAMP(4 + 4 * t);
 #pragma unroll
             for (int b = 0; b < NBB; b++) {
                 floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int i = 0; i < 8; i += 2) {
-                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[i], af[b][q][i], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[i + 1], af[b][q][i + 1], acc1, 0, 0, 0);
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[b][q][i], wf[i], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[b][q][i + 1], wf[i + 1], acc1, 0, 0, 0);
                 }
-                total[b] += (acc0 + acc1) * undo[b][q];
+                if constexpr (TYPE == JL_Q4_K) {
+                    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                    const floatx4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[b][q], tail.mins, zero, 0, 0, 0);
+                    total[b] += ((acc0 + acc1) * tail.d - accm * tail.dmin) * undo[b][q];
+                } else {
+                    total[b] += (acc0 + acc1) * undo[b][q];
+                }
             }
         }
+        asm volatile("" : "+v"(total[0]));
+        STAMP(5 + 4 * (it * ZIN + ZIN - 1));
         // plain arithmetic happened on the MFMA results: the compiler placed the wait states itself
         const uint32_t pw = lds0 + (it & 1) * partial_bytes + wave * (NBB * 1024) + lane * 16;
 #pragma unroll
         for (int b = 0; b < NBB; b++) lds_write_f4(pw + b * 1024, total[b]);
     }
     if (mine > 0) __builtin_amdgcn_s_barrier();
+#ifdef JL_SKINNY_PROBE
+    if (p.stamps && blockIdx.x == 8 && blockIdx.y == 0 && wave == 0) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        for (int i = lane; i < 16 * 96; i += 64) {
+            uint32_t v;
+            asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds0 + p.lds_total + 4 * i) : "memory");
+            p.stamps[i] = v;
+        }
+    }
+#endif
 }
 
 // Adds the spans' partial sums in span order and applies row scale and epilogue; one thread per
@@ -541,6 +706,11 @@ __global__ void __launch_bounds__(256) jl_skinny_reduce(SkinnyParams p, int padd
     else *dst = s;
 }
 
+#ifdef JL_SKINNY_PROBE
+#define JL_PROBE_LDS 6144
+#else
+#define JL_PROBE_LDS 0
+#endif
 template <int TYPE, int NBB, bool DUAL, int ZIN>
 int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int groups) {
     auto fn = jl_gemm_skinny<TYPE, NBB, DUAL, ZIN>;
@@ -550,14 +720,19 @@ int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int gro
         configured[ctx->device] = true;
     }
     // one workgroup per compute unit and span (the ring takes most of the LDS), fewer for less work
-    int per_span = ctx->compute_units / p.Z;
+    // The row blocks of a call share the chip: workgroup (x, y) runs beside (x, y + 1), and with a
+    // grid width that is a multiple of 8 both land on the same XCD, whose L2 then serves the second
+    // reader of every tile.
+    int per_span = ctx->compute_units / p.row_blocks / p.Z;
+    if (p.row_blocks > 1) per_span = per_span / 8 * 8;
     if (per_span < 1) per_span = 1;
     if (per_span > groups) per_span = groups;
-    hipLaunchKernelGGL(fn, dim3(per_span * p.Z), dim3(threads + 64 * (kDmaWaves + kFoldWaves)), lds, ctx->stream, p);
+    hipLaunchKernelGGL(fn, dim3(per_span * p.Z, p.row_blocks), dim3(threads + 64 * (kDmaWaves + kFoldWaves)), lds + JL_PROBE_LDS,
+                       ctx->stream, p);
     JL_HIP(hipGetLastError());
     if (p.Z > 1) {
         hipLaunchKernelGGL(jl_skinny_reduce<DUAL>, dim3((groups * 16 + 255) / 256, p.rows), dim3(256), 0,
-                           ctx->stream, p, 16 * NBB);
+                           ctx->stream, p, 16 * NBB * p.row_blocks);
         JL_HIP(hipGetLastError());
     }
     return JL_OK;
@@ -574,7 +749,7 @@ int launch_nbb(jl_context *ctx, const SkinnyParams &p, int nbb, int zin, int thr
 
 }  // namespace
 
-// Rows the fp16 activation copy must hold (zero past the active ones) for `rows` active rows.
+// Activation rows one workgroup multiplies: 16 or 32; calls of more rows run as two row blocks.
 int jl_skinny_padded_rows(int rows) { return rows <= 16 ? 16 : 32; }
 
 // Sets *taken to false, launching nothing, when the shape is not one this kernel takes; the caller
@@ -586,8 +761,9 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     const bool dual = epilogue == JL_SWIGLU;
-    if (rows > 32 || k % 256 != 0 || count > kMaxSeg) return JL_OK;
+    if (rows > 64 || k % 256 != 0 || count > kMaxSeg) return JL_OK;
     const int S = k / 64;
+    const int row_blocks = rows > 32 ? 2 : 1;
     const int nbb = jl_skinny_padded_rows(rows) / 16;
     int Ss = max_slices(nbb);
     while (Ss > 4 && S % Ss) Ss -= 4;
@@ -622,8 +798,12 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     p.row_bytes = k / jl_block_elems(type) * jl_block_bytes(type);
     p.Ss = Ss;
     p.Z = Z;
+    p.row_blocks = row_blocks;
+#ifdef JL_SKINNY_PROBE
+    p.probe = getenv("JL_SKINNY_PROBE") ? atoi(getenv("JL_SKINNY_PROBE")) : 0;
+#endif
     p.span_bytes = Ss * (type == JL_Q8_0 ? 68 : 36);
-    if (Z > 1 && (size_t)Z * (16 * nbb) * groups * 16 * sizeof(float) > plane_bytes) return JL_OK;
+    if (Z > 1 && (size_t)Z * (16 * nbb * row_blocks) * groups * 16 * sizeof(float) > plane_bytes) return JL_OK;
 
     const int threads = 16 * Ss;   // compute threads; the copy and fold waves come on top
     const int per_wave = type == JL_Q8_0 ? 18 : 10;
@@ -637,6 +817,21 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     p.stages = stages;
     const int lds = partial + stages * stage_bytes;
     *taken = true;
+#ifdef JL_SKINNY_PROBE
+    p.lds_total = lds;
+    {
+        static uint32_t *stamp_buf = nullptr;
+        if (!stamp_buf && getenv("JL_SKINNY_STAMPS")) (void)hipMalloc(&stamp_buf, 16 * 96 * 4);
+        p.stamps = stamp_buf;
+        if (stamp_buf && getenv("JL_SKINNY_STAMPS_DUMP")) {
+            static uint32_t host[16 * 96];
+            (void)hipDeviceSynchronize();
+            (void)hipMemcpy(host, stamp_buf, sizeof host, hipMemcpyDeviceToHost);
+            FILE *f = fopen(getenv("JL_SKINNY_STAMPS_DUMP"), "wb");
+            if (f) { fwrite(host, 1, sizeof host, f); fclose(f); }
+        }
+    }
+#endif
 
     switch (type) {
         case JL_Q8_0:

@@ -137,7 +137,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
                    int epilogue, int math, void *workspace, size_t workspace_bytes,
                    const jl_resident *resident, const jl_half_io *half = nullptr);
-// Batched decode (at most 32 rows): the weight-streaming kernel.  `taken` says whether the shape
+// Batched decode (at most 64 rows): the weight-streaming kernel.  `taken` says whether the shape
 // was one it handles; when not, nothing was launched and the tiled GEMM must run instead.
 int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                           float *C, int rows, int64_t ldo, int64_t col_offset, int epilogue,
