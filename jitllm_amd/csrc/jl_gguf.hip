@@ -18,8 +18,10 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <cstdint>
 #include <cstring>
 #include <map>
+#include <new>
 #include <string>
 #include <vector>
 
@@ -27,6 +29,7 @@ namespace {
 
 constexpr uint32_t kMagic = 0x46554747u;  // "GGUF", little-endian
 constexpr int kDefaultAlignment = 32;
+constexpr int kMaxAlignment = 1 << 20;
 
 // gguf_metadata_value_type
 enum ValueType { U8, I8, U16, I16, U32, I32, F32, BOOL, STRING, ARRAY, U64, I64, F64, VALUE_TYPES };
@@ -200,26 +203,19 @@ void close_file(jl_gguf *g) {
 
 extern "C" {
 
-int jl_gguf_open(const char *path, jl_gguf **out) {
-    JL_REQUIRE(path && out, "jl_gguf_open: null argument");
-    *out = nullptr;
-    jl_gguf *g = new (std::nothrow) jl_gguf();
-    JL_REQUIRE(g != nullptr, "jl_gguf_open: host allocation failed");
+// Fills `g` from the file; the caller closes it when this fails or throws.
+static int parse_file(const char *path, jl_gguf *g) {
     g->fd = open(path, O_RDONLY | O_CLOEXEC);
     if (g->fd < 0) {
-        close_file(g);
         return jl_fail(JL_ERR_INVALID, "Model file not found: %s", path);
     }
     struct stat st;
     if (fstat(g->fd, &st) != 0 || st.st_size < 24) {
-        close_file(g);
         return jl_fail(JL_ERR_INVALID, "%s is too short to be a GGUF file", path);
     }
     g->size = (int64_t)st.st_size;
     void *m = mmap(nullptr, (size_t)g->size, PROT_READ, MAP_PRIVATE, g->fd, 0);
     if (m == MAP_FAILED) {
-        g->base = nullptr;
-        close_file(g);
         return jl_fail(JL_ERR_INVALID, "mapping %s failed", path);
     }
     g->base = (const uint8_t *)m;
@@ -227,19 +223,16 @@ int jl_gguf_open(const char *path, jl_gguf **out) {
     Cursor c{g->base, g->size};
     const uint32_t magic = c.get<uint32_t>();
     if (magic != kMagic) {
-        close_file(g);
         return jl_fail(JL_ERR_INVALID, "unsupported header.magic %u", magic);
     }
     g->version = (int)c.get<uint32_t>();
     if (g->version != 2 && g->version != 3) {
         const int v = g->version;
-        close_file(g);
         return jl_fail(JL_ERR_INVALID, "unsupported header.version %d", v);
     }
     const uint64_t tensor_count = c.get<uint64_t>();
     const uint64_t kv_count = c.get<uint64_t>();
     if (!c.ok || tensor_count > (uint64_t)g->size || kv_count > (uint64_t)g->size) {
-        close_file(g);
         return jl_fail(JL_ERR_INVALID, "GGUF header of %s holds impossible counts", path);
     }
     for (uint64_t i = 0; i < kv_count; i++) {
@@ -247,18 +240,23 @@ int jl_gguf_open(const char *path, jl_gguf **out) {
         Value v;
         if (!c.ok || !read_value(c, v)) {
             const long long at = (long long)c.pos;
-            close_file(g);
-            return jl_fail(JL_ERR_INVALID, "GGUF metadata ends early or is malformed at byte %lld", at);
+                return jl_fail(JL_ERR_INVALID, "GGUF metadata ends early or is malformed at byte %lld", at);
         }
         g->metadata[key] = v;
     }
     auto al = g->metadata.find("general.alignment");
-    if (al != g->metadata.end() && al->second.type != STRING && al->second.type != ARRAY && al->second.i > 0)
-        g->alignment = (int)al->second.i;
-    if (g->alignment & (g->alignment - 1)) {
-        const int a = g->alignment;
-        close_file(g);
-        return jl_fail(JL_ERR_INVALID, "general.alignment %d is not a power of two", a);
+    if (al != g->metadata.end() && al->second.type != STRING && al->second.type != ARRAY && al->second.i > 0) {
+        // range-checked as 64 bits before it is narrowed: 2^32 must not become 0
+        const int64_t a = al->second.i;
+        if (a > kMaxAlignment || (a & (a - 1))) {
+                return jl_fail(JL_ERR_INVALID, "general.alignment %lld is not a power of two of at most %d",
+                           (long long)a, kMaxAlignment);
+        }
+        g->alignment = (int)a;
+    }
+    // a tensor info takes at least 24 bytes (name length, dimension count, type, offset)
+    if (tensor_count > (uint64_t)(g->size - c.pos) / 24) {
+        return jl_fail(JL_ERR_INVALID, "GGUF header of %s holds impossible counts", path);
     }
     g->tensors.reserve((size_t)tensor_count);
     for (uint64_t i = 0; i < tensor_count; i++) {
@@ -266,27 +264,53 @@ int jl_gguf_open(const char *path, jl_gguf **out) {
         t.name = c.str();
         t.n_dims = (int)c.get<uint32_t>();
         if (!c.ok || t.n_dims < 0 || t.n_dims > 4) {
-            close_file(g);
-            return jl_fail(JL_ERR_INVALID, "GGUF tensor info %llu is malformed", (unsigned long long)i);
+                return jl_fail(JL_ERR_INVALID, "GGUF tensor info %llu is malformed", (unsigned long long)i);
         }
         for (int k = 0; k < t.n_dims; k++) t.dims[k] = (int64_t)c.get<uint64_t>();
         t.type = (int)c.get<uint32_t>();
         t.offset = (int64_t)c.get<uint64_t>();
         if (!c.ok) {
-            close_file(g);
-            return jl_fail(JL_ERR_INVALID, "GGUF tensor infos end early at byte %lld", (long long)c.pos);
+                return jl_fail(JL_ERR_INVALID, "GGUF tensor infos end early at byte %lld", (long long)c.pos);
         }
         const TypeGeometry geo = geometry(t.type);
         if (geo.bytes) {
-            int64_t n = 1;
-            for (int k = 0; k < t.n_dims; k++) n *= t.dims[k];
-            t.bytes = n / geo.elems * geo.bytes;
+            // element count without overflow: a product past 2^62 leaves the tensor without a size,
+            // and every later use refuses it
+            uint64_t n = 1;
+            bool fits = true;
+            for (int k = 0; k < t.n_dims; k++) {
+                const uint64_t dim = (uint64_t)t.dims[k];
+                if (dim != 0 && n > (UINT64_C(1) << 62) / dim) fits = false;
+                else n *= dim;
+            }
+            if (fits && n / geo.elems <= (UINT64_C(1) << 62) / geo.bytes) t.bytes = (int64_t)(n / geo.elems * geo.bytes);
         }
         g->by_name[t.name] = (int64_t)g->tensors.size();
         g->tensors.push_back(t);
     }
     // padding to the nearest multiple of the alignment, then the tensor data
     g->data_offset = (c.pos + g->alignment - 1) / g->alignment * g->alignment;
+    return JL_OK;
+}
+
+int jl_gguf_open(const char *path, jl_gguf **out) {
+    JL_REQUIRE(path && out, "jl_gguf_open: null argument");
+    *out = nullptr;
+    jl_gguf *g = new (std::nothrow) jl_gguf();
+    JL_REQUIRE(g != nullptr, "jl_gguf_open: host allocation failed");
+    int st;
+    // strings, maps and the tensor table allocate: nothing may leave an extern "C" function by throwing
+    try {
+        st = parse_file(path, g);
+    } catch (const std::bad_alloc &) {
+        st = jl_fail(JL_ERR_OOM, "jl_gguf_open: out of host memory while reading %s", path);
+    } catch (...) {
+        st = jl_fail(JL_ERR_INVALID, "jl_gguf_open: reading %s failed", path);
+    }
+    if (st != JL_OK) {
+        close_file(g);
+        return st;
+    }
     *out = g;
     return JL_OK;
 }
@@ -319,7 +343,7 @@ int jl_gguf_tensor_info(const jl_gguf *g, int64_t index, const char **name, int 
     if (n_dims) *n_dims = t.n_dims;
     if (dims)
         for (int k = 0; k < 4; k++) dims[k] = t.dims[k];
-    if (file_offset) *file_offset = g->data_offset + t.offset;
+    if (file_offset) *file_offset = (t.offset < 0 || t.offset > INT64_MAX - g->data_offset) ? -1 : g->data_offset + t.offset;
     if (bytes) *bytes = t.bytes;
     return JL_OK;
 }
@@ -364,7 +388,7 @@ int jl_gguf_metadata_array(const jl_gguf *g, const char *key, int *element_type,
 }
 
 int jl_gguf_upload(jl_context *ctx, const jl_gguf *g, const char *name, jl_weight **out) {
-    JL_REQUIRE(ctx && g && name && out, "jl_gguf_upload: null argument");
+    JL_REQUIRE(g && name && out, "jl_gguf_upload: null argument");
     *out = nullptr;
     const int64_t i = jl_gguf_find(g, name);
     JL_REQUIRE(i >= 0, "no tensor %s in the file", name);
@@ -374,11 +398,16 @@ int jl_gguf_upload(jl_context *ctx, const jl_gguf *g, const char *name, jl_weigh
                        name, t.type);
     }
     JL_REQUIRE(t.n_dims == 2, "tensor %s has %d dimensions, a projection weight has 2", name, t.n_dims);
+    // compared as unsigned quantities against what is left of the file: a sum of offsets near
+    // 2^63 would wrap and pass
+    const uint64_t room = g->data_offset <= g->size ? (uint64_t)(g->size - g->data_offset) : 0;
     const int64_t begin = g->data_offset + t.offset;
-    if (t.offset < 0 || t.bytes < 0 || begin + t.bytes > g->size) {
+    if (t.offset < 0 || t.bytes < 0 || (uint64_t)t.offset > room || (uint64_t)t.bytes > room - (uint64_t)t.offset) {
         return jl_fail(JL_ERR_INVALID, "tensor %s (%s, %lld bytes) runs past the end of the file", name,
                        jl_type_name(t.type), (long long)t.bytes);
     }
+    // (the file's own faults are reported before a missing context is)
+    JL_REQUIRE(ctx != nullptr, "jl_gguf_upload: null context");
     // GGUF dimensions are in ne order: dims[0] is the row length
     return jl_weight_upload(ctx, t.type, g->base + begin, t.dims[1], t.dims[0], out);
 }

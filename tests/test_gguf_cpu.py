@@ -125,3 +125,56 @@ def test_files_the_reference_refuses_are_refused_in_its_words(tmp_path):
     tiny.write_bytes(b"GGUF")
     with pytest.raises(JitllmHipError, match="too short"):
         GGUF(tiny)
+
+
+def _crafted(tmp_path, name, tensor_count=1, kv=(), offset=0, dims=(256, 8), gtype=8, data=b"\0" * 4096):
+    """A file put together by hand so that single header fields can hold hostile values."""
+    import struct
+    head = b"GGUF" + struct.pack("<IQQ", 3, tensor_count, len(kv))
+    for key, vtype, v in kv:
+        head += W._string(key) + struct.pack("<I", vtype) + W._value(vtype, v)
+    head += W._string("t") + struct.pack("<I", len(dims)) + b"".join(struct.pack("<Q", d) for d in dims)
+    head += struct.pack("<IQ", gtype, offset)
+    blob = head + b"\0" * (-len(head) % 32) + data
+    path = tmp_path / name
+    path.write_bytes(blob)
+    return path
+
+
+def _upload_without_context(g, name="t"):
+    """jl_gguf_upload reports what is wrong with the file's tensor before it looks at the context,
+    so the bounds checks run without a GPU."""
+    import ctypes as C
+    from jitllm_amd import _lib as L
+    h = C.c_void_p()
+    L.check(g._lib.jl_gguf_upload(None, g.handle, name.encode(), C.byref(h)))
+
+
+def test_hostile_header_fields_are_refused_not_followed(tmp_path):
+    # a sane file first: the only thing missing is the context
+    with GGUF(_crafted(tmp_path, "ok.gguf")) as g:
+        assert g.tensor_info(0).nbytes == 8 * 256 // 32 * 34
+        with pytest.raises(JitllmHipError, match="null context"):
+            _upload_without_context(g)
+    # a tensor offset near 2^63: data_offset + offset wraps negative in signed arithmetic
+    for off in ((1 << 63) - 40, (1 << 63) - 1, 1 << 63, (1 << 64) - 32, 4096 - 2175):
+        with GGUF(_crafted(tmp_path, "far.gguf", offset=off)) as g:
+            with pytest.raises(JitllmHipError, match="runs past the end"):
+                _upload_without_context(g)
+            g.tensor_info(0)         # reporting it must not trap either
+    # the last byte of the tensor is the last byte of the file: still inside
+    with GGUF(_crafted(tmp_path, "edge.gguf", offset=4096 - 2176)) as g:
+        with pytest.raises(JitllmHipError, match="null context"):
+            _upload_without_context(g)
+    # dimensions whose product overflows 64 bits leave no size to trust
+    with GGUF(_crafted(tmp_path, "dims.gguf", dims=(1 << 40, 1 << 40))) as g:
+        with pytest.raises(JitllmHipError, match="runs past the end"):
+            _upload_without_context(g)
+    # general.alignment = 2^32 narrows to 0 in 32 bits (and 0 divides); 2^40 is a power of two too
+    for a in (1 << 32, 1 << 40, (1 << 32) + 32):
+        with pytest.raises(JitllmHipError, match="general.alignment"):
+            GGUF(_crafted(tmp_path, "al.gguf", kv=[("general.alignment", W.U64, a)]))
+    # a tensor count that the file could not possibly hold must not size the tensor table
+    for count in (1 << 40, 400):
+        with pytest.raises(JitllmHipError, match="impossible counts|malformed|end early"):
+            GGUF(_crafted(tmp_path, "count.gguf", tensor_count=count))
