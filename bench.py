@@ -8,10 +8,16 @@ launches, 1 316 320 256 algorithmic bytes (weights in GGUF block layout + fp32 i
 each once).  Inputs are resident in HBM before the timed region.  Every layer owns distinct device
 buffers, so the 1.3 GB sweep cannot live in the 256 MB memory-side cache.
 
-Prints one JSON line.  `value` is GB/s of algorithmic bytes; `roofline` is the dominant kernel
-(the fused gate/up GEMV) against the 8 TB/s HBM peak; `cpu_baseline` is the oracle's restatement of
-the reference's Java CPU matmul timed on this machine's host cores; `prefill` and `batched` carry
-the MFMA side of the metric.
+Prints one JSON line.  `value` is GB/s of algorithmic bytes; `roofline` is the largest single
+launch shape of the step (the fused gate/up GEMV) against the 8 TB/s HBM peak; `cpu_baseline` is the
+oracle's restatement of the reference's Java CPU matmul timed on this machine's host cores;
+`prefill` and `batched` carry the MFMA side of the metric.
+
+Every timed leg is a HIP graph replayed in REPS repetitions of K replays each; the figure reported
+is the median repetition, its spread (max - min over the median) is given beside it and a spread
+above 10 % is flagged "unstable" (the reference's rule, docs/architecture/verification.md:116-131).
+Before a leg is timed, one of its outputs is downloaded and a sample of it compared with the CPU
+oracle: a line cannot come from a kernel that computes something else.
 """
 from __future__ import annotations
 
@@ -32,6 +38,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 F16_MFMA_PEAK_TFLOPS = 2500.0
 INT8_MFMA_PEAK_TOPS = 5000.0
+F16_MFMA_FLOPS_PER_CU_CLK = 4096     # dense fp16 MFMA flops per compute unit and clock (2.5 PFLOP/s over 256 CUs at 2.4 GHz)
+REPS = 5                             # timed repetitions per leg (median reported)
+UNSTABLE_SPREAD = 0.10
 
 # Llama-3.2-1B geometry: the decode projection set the headline metric is quoted on
 DIM, KV_DIM, HIDDEN, VOCAB, LAYERS = 2048, 512, 8192, 128256, 16
@@ -55,6 +64,19 @@ class Hip:
         self.lib.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
         self.lib.hipGraphExecDestroy.argtypes = [C.c_void_p]
         self.lib.hipGraphDestroy.argtypes = [C.c_void_p]
+        self.lib.hipDeviceGetAttribute.argtypes = [C.POINTER(C.c_int), C.c_int, C.c_int]
+
+    def clock_khz(self, device=0) -> int:
+        """hipDeviceAttributeClockRate (enumerator 5): the device's peak shader clock."""
+        v = C.c_int()
+        assert self.lib.hipDeviceGetAttribute(C.byref(v), 5, device) == 0
+        return int(v.value)
+
+    def destroy_graph(self, exe):
+        assert self.lib.hipGraphExecDestroy(exe) == 0
+
+    def destroy_event(self, e):
+        assert self.lib.hipEventDestroy(e) == 0
 
     def capture(self, stream, fn):
         """Records the kernel launches `fn` enqueues on `stream` into an executable graph."""
@@ -83,6 +105,87 @@ class Hip:
         ms = C.c_float()
         assert self.lib.hipEventElapsedTime(C.byref(ms), a, b) == 0
         return float(ms.value)
+
+
+def under_tracer() -> bool:
+    """True when a profiler's tool library rides along (rocprofv3 preloads one)."""
+    return ("rocprof" in os.environ.get("LD_PRELOAD", "").lower()
+            or any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ))
+
+
+def spread_stats(samples, scale=1.0, digits=4):
+    """Median, range and relative spread of the repetitions."""
+    med = statistics.median(samples)
+    spread = (max(samples) - min(samples)) / med if med > 0 else 0.0
+    return {"median": round(med * scale, digits), "min": round(min(samples) * scale, digits),
+            "max": round(max(samples) * scale, digits), "spread": round(spread, 4),
+            "unstable": bool(spread > UNSTABLE_SPREAD), "repetitions": len(samples)}
+
+
+def timed_graph(ctx, hip, fn, steps, warmup, reps=REPS):
+    """`fn`'s launches captured into one graph; `warmup` untimed replays, then `reps` repetitions
+    of exactly `steps` replays between two events on the context's stream.  Returns the
+    milliseconds per replay of each repetition.  The graph and the events are destroyed."""
+    fn()
+    ctx.sync()
+    graph = hip.capture(ctx.stream, fn)
+    for _ in range(warmup):
+        hip.launch(graph, ctx.stream)
+    ctx.sync()
+    out = []
+    for _ in range(reps):
+        e0, e1 = hip.event(), hip.event()
+        hip.record(e0, ctx.stream)
+        for _ in range(steps):
+            hip.launch(graph, ctx.stream)
+        hip.record(e1, ctx.stream)
+        out.append(hip.elapsed_ms(e0, e1) / steps)
+        hip.destroy_event(e0)
+        hip.destroy_event(e1)
+    ctx.sync()
+    hip.destroy_graph(graph)
+    return out
+
+
+# ---- result checks against the CPU oracle (never inside a timed region) --------------------------
+
+def sample_rows(d, count, seed):
+    """Sorted row indices: the first 16, the last 16 and a seeded random remainder."""
+    rng = np.random.default_rng(seed)
+    edge = np.concatenate([np.arange(min(16, d)), np.arange(max(0, d - 16), d)])
+    return np.unique(np.concatenate([edge, rng.choice(d, size=min(count, d), replace=False)]))
+
+
+def gather_rows(raw, t, cols, rows):
+    """The blocks of the given weight rows as a small weight of its own (rows are independent)."""
+    row_bytes = cols // t.block_elems * t.block_bytes
+    return np.ascontiguousarray(raw.reshape(-1, row_bytes)[rows]).reshape(-1)
+
+
+def oracle_rows(t, raw, cols, rows, X):
+    """(reference, magnitude) of the sampled weight rows against activation rows X [B x cols]:
+    the oracle's matmul in the CPU path's own summation order, and sum_j |w_ij x_bj| in float64."""
+    from jitllm_amd.ggml import GGMLType
+    from oracle import pyoracle as O
+    sub = gather_rows(raw, t, cols, rows)
+    X = np.ascontiguousarray(np.atleast_2d(X), dtype=np.float32)
+    mode = O.DOT_SCALAR if t == GGMLType.Q4_K else O.DOT_VEC256
+    ref = O.matmul_batch(int(t), sub, X, rows.size, cols, mode).astype(np.float64)
+    w = np.abs(O.dequant(int(t), sub).reshape(rows.size, cols).astype(np.float64))
+    return ref, np.abs(X.astype(np.float64)) @ w.T
+
+
+def check(name, got, ref, mag, bound):
+    """max |got - ref| / sum |w x| over the sample; the benchmark stops if it exceeds `bound`."""
+    err = float(np.max(np.abs(np.asarray(got, dtype=np.float64) - ref) / np.maximum(mag, 1e-30)))
+    if not err < bound:
+        raise SystemExit(f"bench.py: {name} differs from the CPU oracle: {err:.3e} of the magnitude sum "
+                         f"(bound {bound:.0e}); no figure is reported for a wrong result")
+    return float(f"{err:.3e}")
+
+
+def swiglu64(g, u):
+    return g / (1.0 + np.exp(-g)) * u
 
 
 def q8_bytes(rows, cols):
@@ -147,25 +250,30 @@ def decode_step_fused_rms(proj, layers, wcls, acts):
     proj.argmax(acts["logits"], VOCAB, acts["token"])
 
 
-def bench_fused_rms(ctx, hip, proj, layers, wcls, acts, steps, warmup):
+def bench_fused_rms(ctx, hip, proj, layers, wcls, acts, host, steps, warmup):
     from jitllm_amd import synthetic
+    from jitllm_amd.ggml import GGMLType
+    from oracle import pyoracle as O
+    rms_host = {}
     for i, k in enumerate(("rms_att", "rms_ffn", "rms_final")):
-        acts[k] = ctx.from_numpy((1.0 + 0.1 * synthetic.activations(DIM, 31 + i)).astype("float32"))
+        rms_host[k] = (1.0 + 0.1 * synthetic.activations(DIM, 31 + i)).astype("float32")
+        acts[k] = ctx.from_numpy(rms_host[k])
     acts["token"] = ctx.raw_buffer(4)
-    stream = ctx.stream
-    decode_step_fused_rms(proj, layers, wcls, acts)
+    # check: the vocabulary projection of the normalised vector, and the token picked from it
+    x0 = acts["x"].get()
+    proj.rmsMatvec(acts["x"], acts["rms_final"], None, acts["logits"], wcls, DIM, VOCAB, eps=1e-5)
+    proj.argmax(acts["logits"], VOCAB, acts["token"])
     ctx.sync()
-    graph = hip.capture(stream, lambda: decode_step_fused_rms(proj, layers, wcls, acts))
-    for _ in range(warmup):
-        hip.launch(graph, stream)
-    e0, e1 = hip.event(), hip.event()
-    hip.record(e0, stream)
-    for _ in range(steps):
-        hip.launch(graph, stream)
-    hip.record(e1, stream)
-    ctx.sync()
-    ms = hip.elapsed_ms(e0, e1) / steps
-    return {"ms_per_step": round(ms, 4), "tok_s": round(1e3 / ms, 1), "launches": 4 * LAYERS + 2,
+    logits = acts["logits"].get()
+    rows = sample_rows(VOCAB, 128, 7)
+    ref, mag = oracle_rows(GGMLType.Q8_0, host["wcls"], DIM, rows, O.rmsnorm(x0, rms_host["rms_final"], 1e-5))
+    err = check("rms-folded vocabulary projection", logits[rows], ref[0], mag[0], 1e-3)
+    if int(acts["token"].download(np.int32, 1)[0]) != int(np.argmax(logits)):
+        raise SystemExit("bench.py: the device's greedy token is not the first maximum of its logits")
+    ms = timed_graph(ctx, hip, lambda: decode_step_fused_rms(proj, layers, wcls, acts), steps, warmup)
+    st = spread_stats(ms)
+    return {"ms_per_step": st["median"], "ms_stats": st, "tok_s": round(1e3 / statistics.median(ms), 1),
+            "launches": 4 * LAYERS + 2, "check_rel_err": err,
             "what": "decode set with the 33 RMS normalisations folded into q|k|v, gate/up and the "
                     "vocabulary projection (scale computed inside each kernel, no normalised vector "
                     "written) and the greedy token chosen on the device"}
@@ -180,6 +288,19 @@ def decode_bytes():
     return LAYERS * per_layer + gemv_bytes(VOCAB, DIM)
 
 
+def cpu_timed(fn, budget_s, min_passes=3):
+    """Runs `fn` once untimed, then for about `budget_s` seconds (at least `min_passes` passes);
+    returns (median seconds per pass, passes, wall seconds)."""
+    begin = time.perf_counter()
+    fn()
+    times = []
+    while len(times) < min_passes or (time.perf_counter() - begin < budget_s and len(times) < 5000):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return statistics.median(times), len(times), time.perf_counter() - begin
+
+
 def cpu_baseline(host, shapes, t, budget_s=10.0):
     """The oracle (a C restatement of FloatTensor.matmul with the 256-bit vectorDot lane order,
     rows spread over the host cores) on one layer's seven projections plus the vocabulary
@@ -191,160 +312,227 @@ def cpu_baseline(host, shapes, t, budget_s=10.0):
     x_hid = synthetic.activations(HIDDEN, 32)
     names = ["wq", "wk", "wv", "wo", "w1", "w3", "w2", "wcls"]
     nbytes = sum(gemv_bytes(*shapes[k]) for k in names)
-    times = []
-    begin = time.perf_counter()
-    while len(times) < 4 or (time.perf_counter() - begin < budget_s and len(times) < 5000):
-        t0 = time.perf_counter()
+
+    def one_pass():
         for k in names:
             rows, cols = shapes[k]
-            O.matmul(int(t), host[k], x_hid if cols == HIDDEN else x_dim, rows, cols,
-                     O.DOT_VEC256, threads)
-        times.append(time.perf_counter() - t0)
-    med = statistics.median(times[1:])
+            O.matmul(int(t), host[k], x_hid if cols == HIDDEN else x_dim, rows, cols, O.DOT_VEC256, threads)
+    med, passes, wall = cpu_timed(one_pass, budget_s)
     return {"value": round(nbytes / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"one layer's 7 projections + vocabulary projection ({nbytes} B), "
-                      f"median of {len(times) - 1} passes after 1 warm-up "
-                      f"({time.perf_counter() - begin:.1f} s of wall time), 256-bit vectorDot order",
+                      f"median of {passes} passes after 1 warm-up "
+                      f"({wall:.1f} s of wall time), 256-bit vectorDot order",
             "tok_s_equiv": round(nbytes / med / decode_bytes(), 3)}
 
 
-def bench_gemm(ctx, hip, t, T, steps, warmup):
+def cpu_baseline_rows(t, raw, cols, rows, X, total_rows, budget_s, what):
+    """The oracle's batched matmul (FloatTensor.matmul(context, ...): one dot per activation row and
+    weight row, rows spread over the host cores) on a sample of a weight's rows, scaled to the
+    whole weight by the row count."""
+    from jitllm_amd.ggml import GGMLType
+    from oracle import pyoracle as O
+    threads = O.max_threads()
+    sub = gather_rows(raw, t, cols, rows)
+    X = np.ascontiguousarray(np.atleast_2d(X), dtype=np.float32)
+    mode = O.DOT_SCALAR if t == GGMLType.Q4_K else O.DOT_VEC256
+    med, passes, wall = cpu_timed(lambda: O.matmul_batch(int(t), sub, X, rows.size, cols, mode, threads), budget_s)
+    flops = 2.0 * X.shape[0] * rows.size * cols
+    return {"gflops": round(flops / med / 1e9, 1), "cores": threads, "kind": "port",
+            "ms_whole_weight_equiv": round(med * 1e3 * total_rows / rows.size, 3),
+            "sample": f"{what}: {rows.size} of {total_rows} weight rows x {X.shape[0]} activation rows, median of "
+                      f"{passes} passes ({wall:.1f} s), "
+                      + ("scalar dot (the type has no vector dot on the host)" if mode == O.DOT_SCALAR
+                         else "256-bit vectorDot order")}
+
+
+def check_swiglu(name, got, g, u, mag_g, mag_u, bound):
+    """SwiGLU of two projections: the tolerance is the projections' bound carried through the
+    activation (|d silu| <= 1.1 |d g|) plus, for an fp16 result, its rounding."""
+    ref = swiglu64(g, u)
+    mag = 1.1 * mag_g * np.abs(u) + mag_u * np.abs(g / (1.0 + np.exp(-g))) + np.abs(ref)
+    return check(name, got, ref, mag, bound)
+
+
+def bench_gemm(ctx, hip, t, T, steps, warmup, cpu, clock_khz, cu):
     """Batched prefill of one Llama-3.2-1B layer (q|k|v, o, gate/up SwiGLU, down) over T tokens."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
-    w = {
-        "wq": ctx.load_weight(t, synthetic.weight(t, DIM, DIM, 41), DIM, DIM),
-        "wk": ctx.load_weight(t, synthetic.weight(t, KV_DIM, DIM, 42), KV_DIM, DIM),
-        "wv": ctx.load_weight(t, synthetic.weight(t, KV_DIM, DIM, 43), KV_DIM, DIM),
-        "wo": ctx.load_weight(t, synthetic.weight(t, DIM, DIM, 44), DIM, DIM),
-        "w1": ctx.load_weight(t, synthetic.weight(t, HIDDEN, DIM, 45), HIDDEN, DIM),
-        "w3": ctx.load_weight(t, synthetic.weight(t, HIDDEN, DIM, 46), HIDDEN, DIM),
-        "w2": ctx.load_weight(t, synthetic.weight(t, DIM, HIDDEN, 47), DIM, HIDDEN),
-    }
-    X = ctx.from_numpy(synthetic.activations((T, DIM), 48))
-    H = ctx.from_numpy(synthetic.activations((T, HIDDEN), 49) * np.float32(0.1))
+    shapes = {"wq": (DIM, DIM), "wk": (KV_DIM, DIM), "wv": (KV_DIM, DIM), "wo": (DIM, DIM),
+              "w1": (HIDDEN, DIM), "w3": (HIDDEN, DIM), "w2": (DIM, HIDDEN)}
+    host = {k: synthetic.weight(t, r, c, 41 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
+    w = {k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes}
+    Xh = synthetic.activations((T, DIM), 48)
+    Hh = synthetic.activations((T, HIDDEN), 49) * np.float32(0.1)
+    X, H = ctx.from_numpy(Xh), ctx.from_numpy(Hh)
     qkv = ctx.float_array(T * (DIM + 2 * KV_DIM))
     res = ctx.float_array(T * DIM, fill=0.0)
     hb = ctx.float_array(T * HIDDEN)
-    X16 = ctx.half_from_numpy(synthetic.activations((T, DIM), 48))
-    H16 = ctx.half_from_numpy(synthetic.activations((T, HIDDEN), 49) * np.float32(0.1))
+    X16, H16 = ctx.half_from_numpy(Xh), ctx.half_from_numpy(Hh)
     hb16 = ctx.half_array(T * HIDDEN)
-    def timed(proj, X=X, H=H, hb=hb):
+    arows = sample_rows(T, 8, 50)          # activation rows checked
+    F16_BOUND = 2e-3
+
+    def run(proj, X=X, H=H, hb=hb, widen=False):
         def layer():
             proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
             proj.projection(X, res, w["wo"], DIM, DIM, True)
             proj.gateUp(X, hb, w["w1"], w["w3"], DIM, HIDDEN)
             proj.projection(H, res, w["w2"], HIDDEN, DIM, True)
-
-        # replayed as a HIP graph: Python cannot enqueue the layer's launches as fast as they run
+        # result check first: q and v columns, o + down accumulated from zero, SwiGLU hidden vector
+        res.init(0.0)
         layer()
         ctx.sync()
-        graph = hip.capture(ctx.stream, layer)
-        for _ in range(warmup):
-            hip.launch(graph, ctx.stream)
-        ctx.sync()
-        e0, e1 = hip.event(), hip.event()
-        hip.record(e0, ctx.stream)
-        for _ in range(steps):
-            hip.launch(graph, ctx.stream)
-        hip.record(e1, ctx.stream)
-        return hip.elapsed_ms(e0, e1) / steps
+        xs = (Xh.astype(np.float16).astype(np.float32) if widen else Xh)[arows]
+        hs = (Hh.astype(np.float16).astype(np.float32) if widen else Hh)[arows]
+        errs = {}
+        got = qkv.get().reshape(T, DIM + 2 * KV_DIM)[arows]
+        rq, rv = sample_rows(DIM, 48, 51), sample_rows(KV_DIM, 48, 52)
+        ref, mag = oracle_rows(t, host["wq"], DIM, rq, xs)
+        errs["q"] = check(f"prefill T={T} q", got[:, rq], ref, mag, F16_BOUND)
+        ref, mag = oracle_rows(t, host["wv"], DIM, rv, xs)
+        errs["v"] = check(f"prefill T={T} v", got[:, DIM + KV_DIM + rv], ref, mag, F16_BOUND)
+        ro = sample_rows(DIM, 48, 53)
+        ref_o, mag_o = oracle_rows(t, host["wo"], DIM, ro, xs)
+        ref_d, mag_d = oracle_rows(t, host["w2"], HIDDEN, ro, hs)
+        errs["o+down"] = check(f"prefill T={T} o + down", res.get().reshape(T, DIM)[arows][:, ro], ref_o + ref_d,
+                               mag_o + mag_d, F16_BOUND)
+        rh = sample_rows(HIDDEN, 48, 54)
+        g, mg = oracle_rows(t, host["w1"], DIM, rh, xs)
+        u, mu = oracle_rows(t, host["w3"], DIM, rh, xs)
+        errs["gate/up"] = check_swiglu(f"prefill T={T} gate/up", hb.get().astype(np.float32).reshape(T, HIDDEN)[arows][:, rh],
+                                       g, u, mg, mu, F16_BOUND)
+        # replayed as a HIP graph: Python cannot enqueue the layer's launches as fast as they run
+        return timed_graph(ctx, hip, layer, steps, warmup), errs
 
-    ms = timed(QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN))
+    flops = 2.0 * T * (DIM * (DIM + 2 * KV_DIM) + DIM * DIM + 2 * DIM * HIDDEN + HIDDEN * DIM)
+
+    def mode(ms_list, errs):
+        ms = statistics.median(ms_list)
+        tf = flops / (ms * 1e-3) / 1e12
+        return {"ms_per_layer": round(ms, 4), "ms_stats": spread_stats(ms_list), "tflops": round(tf, 1),
+                "frac_f16_mfma_peak": round(tf / F16_MFMA_PEAK_TFLOPS, 4), "check_rel_err": errs}
+
+    default = mode(*run(QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN)))
     # the reference's residency choice: an fp16 copy per projection kept across calls (2 bytes per
     # weight of HBM), decoded by the first call only -- reported beside the default, not instead
-    ms_kept = timed(QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=True))
+    kept = mode(*run(QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=True)))
     # the reference's own operand types on top of that: activations arrive as fp16 (its RMS apply,
     # attention and SwiGLU kernels write fp16) and the hidden vector leaves as fp16
-    ms_half = timed(QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=True), X16, H16, hb16)
+    half_proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=True)
+    half = mode(*run(half_proj, X16, H16, hb16, widen=True))
+    # the dominant kernel on its own: the gate/up call of that last mode is one launch of the fp16
+    # GEMM and nothing else (four to a graph)
+    def gate_ups():
+        for _ in range(4):
+            half_proj.gateUp(X16, hb16, w["w1"], w["w3"], DIM, HIDDEN)
+    gu = [m / 4 for m in timed_graph(ctx, hip, gate_ups, steps, 20)]
+    gu_flops = 2.0 * T * 2 * HIDDEN * DIM
+    gu_tf = gu_flops / (statistics.median(gu) * 1e-3) / 1e12
+    peak_box = cu * clock_khz * 1e3 * F16_MFMA_FLOPS_PER_CU_CLK / 1e12
+    roofline = {"bound": "mfma", "kernel": f"jl_gemm_hh gate/up SwiGLU [{T} x {DIM}] x [{2 * HIDDEN} x {DIM}]^T, fp16 in / fp16 out",
+                "achieved": round(gu_tf, 1), "peak": F16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(gu_tf / F16_MFMA_PEAK_TFLOPS, 4), "flops_per_launch": gu_flops,
+                "avg_launch_us": round(statistics.median(gu) * 1e3, 2), "launch_us_stats": spread_stats(gu, 1e3, 2),
+                "peak_from_box": {"compute_units": cu, "peak_clock_khz": clock_khz,
+                                  "flops_per_cu_clk": F16_MFMA_FLOPS_PER_CU_CLK, "tflops": round(peak_box, 1),
+                                  "frac": round(gu_tf / peak_box, 4)}}
     # what hands the projections those fp16 rows: the RMS reduction and fp16 apply of one [T x dim]
     # activation (two per layer in the model), timed on its own
     rms_w = ctx.from_numpy(np.ones(DIM, dtype=np.float32))
-    half_proj = QuantizedBatchProjections(ctx, T, DIM, DIM)
+    rms_proj = QuantizedBatchProjections(ctx, T, DIM, DIM)
     def rms_apply():
         # (8 launches per graph: a one-kernel graph measures the graph launch, not the kernel)
         for _ in range(8):
-            half_proj.rmsApplyFP16(X, rms_w, 1e-5, X16, DIM)
-    rms_apply()
-    ctx.sync()
-    graph = hip.capture(ctx.stream, rms_apply)
-    for _ in range(3):
-        hip.launch(graph, ctx.stream)
-    ctx.sync()
-    e0, e1 = hip.event(), hip.event()
-    hip.record(e0, ctx.stream)
-    for _ in range(steps):
-        hip.launch(graph, ctx.stream)
-    hip.record(e1, ctx.stream)
-    rms_us = hip.elapsed_ms(e0, e1) / steps / 8 * 1e3
-    flops = 2.0 * T * (DIM * (DIM + 2 * KV_DIM) + DIM * DIM + 2 * DIM * HIDDEN + HIDDEN * DIM)
-    tflops = flops / (ms * 1e-3) / 1e12
-    tflops_kept = flops / (ms_kept * 1e-3) / 1e12
-    tflops_half = flops / (ms_half * 1e-3) / 1e12
-    return {"tokens": T, "ms_per_layer": round(ms, 4), "tok_s_16_layers": round(T / (ms * 1e-3 * LAYERS), 1),
-            "tflops": round(tflops, 1), "frac_f16_mfma_peak": round(tflops / F16_MFMA_PEAK_TFLOPS, 4),
-            "math": "f16 MFMA, fp32 accumulate; weights decoded to fp16 inside the call (in LDS, or once per call into the workspace)",
-            "with_resident_fp16_copy": {"ms_per_layer": round(ms_kept, 4), "tflops": round(tflops_kept, 1),
-                                        "frac_f16_mfma_peak": round(tflops_kept / F16_MFMA_PEAK_TFLOPS, 4)},
-            "with_resident_copy_and_fp16_activations": {
-                "ms_per_layer": round(ms_half, 4), "tflops": round(tflops_half, 1),
-                "frac_f16_mfma_peak": round(tflops_half / F16_MFMA_PEAK_TFLOPS, 4),
-                "rms_apply_to_fp16_us": round(rms_us, 2)}}
+            rms_proj.rmsApplyFP16(X, rms_w, 1e-5, X16, DIM)
+    rms_us = statistics.median(timed_graph(ctx, hip, rms_apply, steps, 3)) / 8 * 1e3
+    half["rms_apply_to_fp16_us"] = round(rms_us, 2)
+    out = {"tokens": T, "ms_per_layer": default["ms_per_layer"], "ms_stats": default["ms_stats"],
+           "tok_s_16_layers": round(T / (default["ms_per_layer"] * 1e-3 * LAYERS), 1),
+           "tflops": default["tflops"], "frac_f16_mfma_peak": default["frac_f16_mfma_peak"],
+           "check_rel_err": default["check_rel_err"],
+           "math": "f16 MFMA, fp32 accumulate; weights decoded to fp16 inside the call (in LDS, or once per call into the workspace)",
+           "with_resident_fp16_copy": kept, "with_resident_copy_and_fp16_activations": half,
+           "roofline": roofline}
+    if cpu:
+        rows = sample_rows(HIDDEN, 224, 55)
+        out["cpu_baseline"] = cpu_baseline_rows(t, host["w1"], DIM, rows, Xh, HIDDEN, 2.0, f"gate projection at T={T}")
+        out["cpu_baseline"]["ms_per_layer_equiv"] = round(
+            flops / (out["cpu_baseline"]["gflops"] * 1e9) * 1e3, 1)
+    for x in w.values():
+        x.free()
+    return out
 
 
-def bench_batched_q4k(ctx, hip, B, steps, warmup):
+def bench_batched_q4k(ctx, hip, B, steps, warmup, cpu):
     """Q4_K batched decode, Qwen3-8B-like shapes (dim 4096, ffn 12288, kv 1024), B sequences."""
     from jitllm_amd import synthetic
     from jitllm_amd.ggml import GGMLType
     from jitllm_amd.projections import QuantizedBatchProjections
     t = GGMLType.Q4_K
     dim, kv, ffn = 4096, 1024, 12288
-    w = {
-        "wq": ctx.load_weight(t, synthetic.weight(t, dim, dim, 61), dim, dim),
-        "wk": ctx.load_weight(t, synthetic.weight(t, kv, dim, 62), kv, dim),
-        "wv": ctx.load_weight(t, synthetic.weight(t, kv, dim, 63), kv, dim),
-        "wo": ctx.load_weight(t, synthetic.weight(t, dim, dim, 64), dim, dim),
-        "w1": ctx.load_weight(t, synthetic.weight(t, ffn, dim, 65), ffn, dim),
-        "w3": ctx.load_weight(t, synthetic.weight(t, ffn, dim, 66), ffn, dim),
-        "w2": ctx.load_weight(t, synthetic.weight(t, dim, ffn, 67), dim, ffn),
-    }
-    X = ctx.from_numpy(synthetic.activations((B, dim), 68))
-    H = ctx.from_numpy(synthetic.activations((B, ffn), 69) * np.float32(0.1))
+    shapes = {"wq": (dim, dim), "wk": (kv, dim), "wv": (kv, dim), "wo": (dim, dim),
+              "w1": (ffn, dim), "w3": (ffn, dim), "w2": (dim, ffn)}
+    host = {k: synthetic.weight(t, r, c, 61 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
+    # enough copies of the layer that a replay cannot be served from the 256 MB memory-side cache
+    copies = 3
+    layers = [{k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes} for _ in range(copies)]
+    Xh = synthetic.activations((B, dim), 68)
+    Hh = synthetic.activations((B, ffn), 69) * np.float32(0.1)
+    X, H = ctx.from_numpy(Xh), ctx.from_numpy(Hh)
     qkv = ctx.float_array(B * (dim + 2 * kv))
     res = ctx.float_array(B * dim, fill=0.0)
     hb = ctx.float_array(B * ffn)
     proj = QuantizedBatchProjections(ctx, B, ffn, 2 * ffn)
 
-    def layer():
+    def layer(w):
         proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
         proj.projection(X, res, w["wo"], dim, dim, True)
         proj.gateUp(X, hb, w["w1"], w["w3"], dim, ffn)
         proj.projection(H, res, w["w2"], ffn, dim, True)
 
-    # replayed as a HIP graph: Python cannot enqueue the layer's launches as fast as they run
-    layer()
+    layer(layers[0])
     ctx.sync()
-    graph = hip.capture(ctx.stream, layer)
-    for _ in range(warmup):
-        hip.launch(graph, ctx.stream)
-    ctx.sync()
-    e0, e1 = hip.event(), hip.event()
-    hip.record(e0, ctx.stream)
-    for _ in range(steps):
-        hip.launch(graph, ctx.stream)
-    hip.record(e1, ctx.stream)
-    ms = hip.elapsed_ms(e0, e1) / steps
-    wbytes = sum(x.nbytes for x in w.values())
+    errs = {}
+    got = qkv.get().reshape(B, dim + 2 * kv)
+    rq, rk = sample_rows(dim, 32, 71), sample_rows(kv, 32, 72)
+    ref, mag = oracle_rows(t, host["wq"], dim, rq, Xh)
+    errs["q"] = check(f"batched B={B} q", got[:, rq], ref, mag, 2e-3)
+    ref, mag = oracle_rows(t, host["wk"], dim, rk, Xh)
+    errs["k"] = check(f"batched B={B} k", got[:, dim + rk], ref, mag, 2e-3)
+    ro = sample_rows(dim, 32, 73)
+    ref_o, mag_o = oracle_rows(t, host["wo"], dim, ro, Xh)
+    ref_d, mag_d = oracle_rows(t, host["w2"], ffn, ro, Hh)
+    errs["o+down"] = check(f"batched B={B} o + down", res.get().reshape(B, dim)[:, ro], ref_o + ref_d,
+                           mag_o + mag_d, 2e-3)
+    rh = sample_rows(ffn, 32, 74)
+    g, mg = oracle_rows(t, host["w1"], dim, rh, Xh)
+    u, mu = oracle_rows(t, host["w3"], dim, rh, Xh)
+    errs["gate/up"] = check_swiglu(f"batched B={B} gate/up", hb.get().reshape(B, ffn)[:, rh], g, u, mg, mu, 2e-3)
+
+    def sweep():
+        for w in layers:
+            layer(w)
+    ms_list = [m / copies for m in timed_graph(ctx, hip, sweep, steps, warmup)]
+    ms = statistics.median(ms_list)
+    wbytes = sum(a.size for a in host.values())
     # fp32 activations in and out, once per projection
     io = 4 * B * (dim + dim + 2 * kv + dim + dim + dim + ffn + ffn + dim)
     flops = 2.0 * B * (dim * (dim + 2 * kv) + dim * dim + 2 * dim * ffn + ffn * dim)
     gbs = (wbytes + io) / (ms * 1e-3) / 1e9
-    return {"B": B, "ms_per_layer": round(ms, 4), "GB_s": round(gbs, 1),
-            "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-            "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "bytes": wbytes + io}
+    out = {"B": B, "ms_per_layer": round(ms, 4), "ms_stats": spread_stats(ms_list), "layers_swept": copies,
+           "GB_s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+           "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "bytes": wbytes + io, "check_rel_err": errs}
+    if cpu and B == 8:
+        rows = sample_rows(ffn, 480, 75)
+        out["cpu_baseline"] = cpu_baseline_rows(t, host["w1"], dim, rows, Xh, ffn, 2.0, "gate projection at B=8")
+        out["cpu_baseline"]["ms_per_layer_equiv"] = round(flops / (out["cpu_baseline"]["gflops"] * 1e9) * 1e3, 1)
+    for w in layers:
+        for x in w.values():
+            x.free()
+    return out
 
 
-def bench_decode_layers(ctx, hip, type_name, dim, kv, ffn, copies, steps, warmup):
+def bench_decode_layers(ctx, hip, type_name, dim, kv, ffn, copies, steps, warmup, cpu):
     """Single-token decode projections of one layer -- q|k|v, o (+=), gate/up SwiGLU, down (+=) --
     over `copies` distinct layers' weights (more bytes than the 256 MB last-level cache holds),
     replayed as one HIP graph.  Q4_0 at Llama-3-8B shapes and Q4_K at Qwen3-8B-like shapes: the
@@ -354,26 +542,31 @@ def bench_decode_layers(ctx, hip, type_name, dim, kv, ffn, copies, steps, warmup
     from jitllm_amd import synthetic
     from jitllm_amd.ggml import GGMLType
     from jitllm_amd.projections import PackedActivation, QuantizedProjections, TornadoWorkspace
+    from oracle import pyoracle as O
     t = GGMLType[type_name]
     shapes = {"wq": (dim, dim), "wk": (kv, dim), "wv": (kv, dim), "wo": (dim, dim),
               "w1": (ffn, dim), "w3": (ffn, dim), "w2": (dim, ffn)}
     host = {k: synthetic.weight(t, r, c, 71 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
     layers = [{k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes} for _ in range(copies)]
-    x = ctx.from_numpy(synthetic.activations(dim, 78))
-    xb = ctx.from_numpy(synthetic.activations(dim, 79))
+    xh, xbh = synthetic.activations(dim, 78), synthetic.activations(dim, 79)
+    hbh = synthetic.activations(ffn, 80) * np.float32(0.1)
+    x, xb = ctx.from_numpy(xh), ctx.from_numpy(xbh)
     q, k_, v = ctx.float_array(dim), ctx.float_array(kv), ctx.float_array(kv)
-    hb = ctx.from_numpy(synthetic.activations(ffn, 80) * np.float32(0.1))
+    hb = ctx.from_numpy(hbh)
     hb2 = ctx.float_array(ffn)
     proj = QuantizedProjections(ctx, TornadoWorkspace(wrapX=x, wrapXb=xb, wrapHb=hb2, wrapHb2=hb))
     small = QuantizedProjections(ctx, TornadoWorkspace(wrapHb=hb2, packedX=PackedActivation(ctx, dim)), packed=True)
     wide = QuantizedProjections(ctx, TornadoWorkspace(packedX=PackedActivation(ctx, ffn)), packed=True)
 
+    def layer(w):
+        proj.fusedQKV(xb, q, k_, v, w["wq"], w["wk"], w["wv"])
+        proj.residualMatvec(xb, w["wo"], dim, dim)
+        proj.gateUp(w["w1"], w["w3"], dim, ffn)
+        proj.residualMatvec(hb, w["w2"], ffn, dim)
+
     def step():
         for w in layers:
-            proj.fusedQKV(xb, q, k_, v, w["wq"], w["wk"], w["wv"])
-            proj.residualMatvec(xb, w["wo"], dim, dim)
-            proj.gateUp(w["w1"], w["w3"], dim, ffn)
-            proj.residualMatvec(hb, w["w2"], ffn, dim)
+            layer(w)
 
     def step_packed():
         for w in layers:
@@ -386,30 +579,95 @@ def bench_decode_layers(ctx, hip, type_name, dim, kv, ffn, copies, steps, warmup
             wide.quantize(hb, ffn)
             wide.packedMatvec(x, w["w2"], ffn, dim, residual=True)
 
-    def timed(fn):
-        fn()
-        ctx.sync()
-        graph = hip.capture(ctx.stream, fn)
-        for _ in range(warmup):
-            hip.launch(graph, ctx.stream)
-        ctx.sync()
-        e0, e1 = hip.event(), hip.event()
-        hip.record(e0, ctx.stream)
-        for _ in range(steps):
-            hip.launch(graph, ctx.stream)
-        hip.record(e1, ctx.stream)
-        return hip.elapsed_ms(e0, e1) / steps / copies
+    # check one layer of the fp32-activation path: q, the two residual projections, gate/up
+    layer(layers[0])
+    ctx.sync()
+    errs = {}
+    rq, ro, rh = sample_rows(dim, 64, 81), sample_rows(dim, 64, 82), sample_rows(ffn, 64, 83)
+    ref, mag = oracle_rows(t, host["wq"], dim, rq, xbh)
+    errs["q"] = check(f"{type_name} decode q", q.get()[rq], ref[0], mag[0], 1e-3)
+    ref_o, mag_o = oracle_rows(t, host["wo"], dim, ro, xbh)
+    ref_d, mag_d = oracle_rows(t, host["w2"], ffn, ro, hbh)
+    errs["o+down"] = check(f"{type_name} decode o + down", x.get()[ro] - xh[ro].astype(np.float64), (ref_o + ref_d)[0],
+                           (mag_o + mag_d + np.abs(xh[ro]) * 1e-6)[0], 1e-3)
+    g, mg = oracle_rows(t, host["w1"], dim, rh, xbh)
+    u, mu = oracle_rows(t, host["w3"], dim, rh, xbh)
+    errs["gate/up"] = check_swiglu(f"{type_name} decode gate/up", hb2.get()[rh], g[0], u[0], mg[0], mu[0], 1e-3)
 
-    ms = timed(step)
-    ms_packed = timed(step_packed)
+    ms_list = [m / copies for m in timed_graph(ctx, hip, step, steps, warmup)]
+    packed_list = [m / copies for m in timed_graph(ctx, hip, step_packed, steps, warmup)]
+    ms, ms_packed = statistics.median(ms_list), statistics.median(packed_list)
     wbytes = sum(a.size for a in host.values())
     io = 4 * (dim + dim + 2 * kv + dim + dim + dim + ffn + ffn + dim)
     gbs = (wbytes + io) / (ms * 1e-3) / 1e9
-    return {"type": type_name, "shapes": {"dim": dim, "kv": kv, "ffn": ffn}, "layers_swept": copies,
-            "ms_per_layer": round(ms, 4), "GB_s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-            "bytes_per_layer": wbytes + io,
-            "packed_activation_path": {"ms_per_layer": round(ms_packed, 4), "launches_per_layer": 8,
-                                       "GB_s": round((wbytes + io) / (ms_packed * 1e-3) / 1e9, 1)}}
+    out = {"type": type_name, "shapes": {"dim": dim, "kv": kv, "ffn": ffn}, "layers_swept": copies,
+           "ms_per_layer": round(ms, 4), "ms_stats": spread_stats(ms_list), "GB_s": round(gbs, 1),
+           "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "bytes_per_layer": wbytes + io, "check_rel_err": errs,
+           "packed_activation_path": {"ms_per_layer": round(ms_packed, 4), "ms_stats": spread_stats(packed_list),
+                                      "launches_per_layer": 8,
+                                      "GB_s": round((wbytes + io) / (ms_packed * 1e-3) / 1e9, 1)}}
+    if cpu:
+        threads = O.max_threads()
+        mode = O.DOT_SCALAR if t == GGMLType.Q4_K else O.DOT_VEC256
+
+        def one_pass():
+            for name, (r, c) in shapes.items():
+                O.matmul(int(t), host[name], hbh if c == ffn else xbh, r, c, mode, threads)
+        med, passes, wall = cpu_timed(one_pass, 2.0)
+        out["cpu_baseline"] = {"value": round((wbytes + io) / med / 1e9, 2), "unit": "GB/s", "cores": threads,
+                               "kind": "port",
+                               "sample": f"the layer's 7 projections ({wbytes + io} B), median of {passes} passes "
+                                         f"({wall:.1f} s), "
+                                         + ("scalar dot" if mode == O.DOT_SCALAR else "256-bit vectorDot order")}
+    for w in layers:
+        for a in w.values():
+            a.free()
+    return out
+
+
+def bench_wq_shape(ctx, hip, t, steps, warmup, cpu):
+    """The single 2048 x 2048 Q8_0 projection (Llama-3.2-1B wq), two ways: *hot* -- the same weight
+    replayed, 4.5 MB that stay in the L2 / memory-side cache, labelled as such -- and *cold* --
+    rotating over 96 device copies (428 MB, more than the 256 MB memory-side cache holds), the
+    model-free form of the reference's SyntheticKernelBench."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    from oracle import pyoracle as O
+    raw = synthetic.weight(t, DIM, DIM, 11)
+    xh = synthetic.activations(DIM, 21)
+    copies = [ctx.load_weight(t, raw, DIM, DIM) for _ in range(96)]
+    x, out = ctx.from_numpy(xh), ctx.float_array(DIM)
+    proj = QuantizedProjections(ctx, TornadoWorkspace())
+    proj.floatMatvec(x, out, copies[-1], DIM, DIM)
+    ctx.sync()
+    rows = sample_rows(DIM, 256, 9)
+    ref, mag = oracle_rows(t, raw, DIM, rows, xh)
+    err = check("2048 x 2048 projection", out.get()[rows], ref[0], mag[0], 1e-3)
+
+    def hot():
+        for _ in range(96):
+            proj.floatMatvec(x, out, copies[0], DIM, DIM)
+
+    def cold():
+        for w in copies:
+            proj.floatMatvec(x, out, w, DIM, DIM)
+    nbytes = gemv_bytes(DIM, DIM)
+    res = {"shape": "Q8_0 [2048 x 2048], batch 1", "bytes_per_launch": nbytes, "check_rel_err": err}
+    for name, fn, note in (("hot", hot, "same weight every launch: served from L2 / the memory-side cache, not HBM"),
+                           ("cold_rotating", cold, "96 device copies in turn (428 MB): every launch reads HBM")):
+        us = [m / 96 * 1e3 for m in timed_graph(ctx, hip, fn, steps, warmup)]
+        med = statistics.median(us)
+        res[name] = {"us_per_launch": round(med, 3), "us_stats": spread_stats(us, 1.0, 3),
+                     "GB_s": round(nbytes / med / 1e3, 1), "frac_hbm_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4),
+                     "note": note}
+    if cpu:
+        threads = O.max_threads()
+        med, passes, wall = cpu_timed(lambda: O.matmul(int(t), raw, xh, DIM, DIM, O.DOT_VEC256, threads), 1.0)
+        res["cpu_baseline"] = {"value": round(nbytes / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+                               "sample": f"the same projection, median of {passes} passes ({wall:.1f} s), host caches warm"}
+    for w in copies:
+        w.free()
+    return res
 
 
 # HBM bytes one gate/up launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
@@ -447,17 +705,48 @@ def traffic_probe(ctx, proj, layers):
                                   "algorithmic_write_bytes": 4 * HIDDEN}}))
 
 
+def prefill_probe(ctx, t, T=2048):
+    """What the matrix-pipe counters (`rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F16 SQ_VALU_MFMA_BUSY_CYCLES
+    SQ_BUSY_CU_CYCLES GRBM_GUI_ACTIVE`) are collected on: one Llama-3.2-1B layer's four prefill calls at
+    T tokens with the resident fp16 copy and fp16 activations (every call is then one launch of the
+    fp16 GEMM, plus a fold for o and down), launched kernel by kernel -- no graph, so that every
+    dispatch has a counter row of its own -- three times after one call that decodes the copy."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    shapes = {"wq": (DIM, DIM), "wk": (KV_DIM, DIM), "wv": (KV_DIM, DIM), "wo": (DIM, DIM),
+              "w1": (HIDDEN, DIM), "w3": (HIDDEN, DIM), "w2": (DIM, HIDDEN)}
+    w = {k: ctx.load_weight(t, synthetic.weight(t, r, c, 41 + i), r, c) for i, (k, (r, c)) in enumerate(shapes.items())}
+    X16 = ctx.half_from_numpy(synthetic.activations((T, DIM), 48))
+    H16 = ctx.half_from_numpy(synthetic.activations((T, HIDDEN), 49) * np.float32(0.1))
+    qkv, res = ctx.float_array(T * (DIM + 2 * KV_DIM)), ctx.float_array(T * DIM, fill=0.0)
+    hb16 = ctx.half_array(T * HIDDEN)
+    proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=True)
+    for _ in range(4):
+        proj.fusedQKV(X16, qkv, w["wq"], w["wk"], w["wv"])
+        proj.projection(X16, res, w["wo"], DIM, DIM, True)
+        proj.gateUp(X16, hb16, w["w1"], w["w3"], DIM, HIDDEN)
+        proj.projection(H16, res, w["w2"], HIDDEN, DIM, True)
+        ctx.sync()
+    print(json.dumps({"tokens": T, "flops": {"q|k|v": 2.0 * T * DIM * (DIM + 2 * KV_DIM), "o": 2.0 * T * DIM * DIM,
+                                             "gate/up": 2.0 * T * 2 * HIDDEN * DIM, "down": 2.0 * T * HIDDEN * DIM},
+                      "mfma_f16_flops_per_instruction_16x16x32": 2 * 16 * 16 * 32}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-extra", action="store_true", help="skip the prefill / batched legs")
-    ap.add_argument("--extra", default="fused_rms,prefill,other_types,batched",
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-extra", action="store_true", help="skip the legs beside the decode set")
+    ap.add_argument("--extra", default="wq_shape,fused_rms,prefill,other_types,batched",
                     help="comma-separated legs beside the decode set (a profiler run takes a few at a time)")
+    ap.add_argument("--prefill-warmup", type=int, default=-1,
+                    help="untimed replays before the prefill legs (default 100; 10 under a profiler)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="only launch what the HBM-traffic counters are read on (see traffic_probe)")
+    ap.add_argument("--prefill-probe", action="store_true",
+                    help="only launch what the matrix-pipe counters are read on (see prefill_probe)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path is built and measured on a single MI355X; "
@@ -470,8 +759,16 @@ def main():
 
     t = GGMLType.Q8_0
     hip = Hip()
+    cpu = not args.no_cpu
+    # (the matrix pipe's clock takes tens of milliseconds of load to settle: 100 untimed replays of
+    # the layer before the timed ones; a kernel tracer records every one of them, so few then)
+    prefill_warmup = args.prefill_warmup if args.prefill_warmup >= 0 else (10 if under_tracer() else 100)
     with Context(0) as ctx:
         cu, name = ctx.device_info()
+        clock_khz = hip.clock_khz(0)
+        if args.prefill_probe:
+            prefill_probe(ctx, t)
+            return
         layers, wcls, acts, host, shapes = build_decode_set(ctx, t)
         ws = TornadoWorkspace(wrapX=acts["x"], wrapXb=acts["xb"], wrapHb=acts["hb"])
         proj = QuantizedProjections(ctx, ws)
@@ -480,6 +777,26 @@ def main():
             return
         total_bytes = decode_bytes()
         assert total_bytes == 1316320256, total_bytes
+
+        # result check, before anything is timed: the gate/up launch and the vocabulary projection
+        x0, xb0 = acts["x"].get(), acts["xb"].get()
+        proj.gateUp(layers[-1]["w1"], layers[-1]["w3"], DIM, HIDDEN)
+        proj.floatMatvec(acts["xb"], acts["logits"], wcls, DIM, VOCAB)
+        proj.fusedQKV(acts["xb"], acts["q"], acts["k"], acts["v"], layers[0]["wq"], layers[0]["wk"], layers[0]["wv"])
+        proj.residualMatvec(acts["xb"], layers[0]["wo"], DIM, DIM)
+        ctx.sync()
+        checks = {}
+        rh, rv, rd = sample_rows(HIDDEN, 96, 1), sample_rows(VOCAB, 160, 2), sample_rows(DIM, 96, 3)
+        g, mg = oracle_rows(t, host["w1"], DIM, rh, xb0)
+        u, mu = oracle_rows(t, host["w3"], DIM, rh, xb0)
+        checks["gate/up"] = check_swiglu("decode gate/up", acts["hb"].get()[rh], g[0], u[0], mg[0], mu[0], 1e-3)
+        ref, mag = oracle_rows(t, host["wcls"], DIM, rv, xb0)
+        checks["vocabulary"] = check("vocabulary projection", acts["logits"].get()[rv], ref[0], mag[0], 1e-3)
+        ref, mag = oracle_rows(t, host["wq"], DIM, rd, xb0)
+        checks["q"] = check("decode q", acts["q"].get()[rd], ref[0], mag[0], 1e-3)
+        ref, mag = oracle_rows(t, host["wo"], DIM, rd, xb0)
+        checks["o (residual)"] = check("decode o", acts["x"].get()[rd] - x0[rd].astype(np.float64), ref[0],
+                                       mag[0] + np.abs(x0[rd]) * 1e-6, 1e-3)
 
         for _ in range(max(1, args.warmup)):
             decode_step(proj, layers, wcls, acts)
@@ -493,42 +810,72 @@ def main():
             hip.launch(step_graph, stream)
         ctx.sync()
 
-        # timed region: exactly K steps
-        e0, e1 = hip.event(), hip.event()
-        t0 = time.perf_counter()
-        hip.record(e0, stream)
-        for _ in range(args.steps):
-            hip.launch(step_graph, stream)
-        hip.record(e1, stream)
-        ctx.sync()
-        wall = time.perf_counter() - t0
-        ms_step_clean = hip.elapsed_ms(e0, e1) / args.steps
+        # timed region: REPS repetitions of exactly K steps each; the median repetition is reported
+        step_ms, walls = [], []
+        for _ in range(REPS):
+            e0, e1 = hip.event(), hip.event()
+            ctx.sync()
+            t0 = time.perf_counter()
+            hip.record(e0, stream)
+            for _ in range(args.steps):
+                hip.launch(step_graph, stream)
+            hip.record(e1, stream)
+            ctx.sync()
+            walls.append((time.perf_counter() - t0) * 1e3 / args.steps)
+            step_ms.append(hip.elapsed_ms(e0, e1) / args.steps)
+            hip.destroy_event(e0)
+            hip.destroy_event(e1)
+        hip.destroy_graph(step_graph)
+        ms = statistics.median(step_ms)
 
-        # the same K steps launched kernel by kernel from Python, for comparison
+        # the same K steps launched kernel by kernel from Python, for comparison (never the headline)
+        e0, e1 = hip.event(), hip.event()
         hip.record(e0, stream)
         for _ in range(args.steps):
             decode_step(proj, layers, wcls, acts)
         hip.record(e1, stream)
-        ms_step = hip.elapsed_ms(e0, e1) / args.steps
+        ms_python = hip.elapsed_ms(e0, e1) / args.steps
+        hip.destroy_event(e0)
+        hip.destroy_event(e1)
 
-        # dominant kernel: the fused gate/up GEMV, 16 launches over the 16 layers' own weights
-        # (571 MB, so nothing is served from the 256 MB memory-side cache), replayed K times
+        # the step's kernels on their own, each as a graph over the 16 layers' own weights (so
+        # nothing is served from the 256 MB memory-side cache)
+        def per_kernel(fn, launches, nbytes):
+            us = [m / launches * 1e3 for m in timed_graph(ctx, hip, fn, args.steps, 2)]
+            med = statistics.median(us)
+            return {"avg_launch_us": round(med, 3), "us_stats": spread_stats(us, 1.0, 3),
+                    "bytes_per_launch": nbytes, "GB_s": round(nbytes / med / 1e3, 1),
+                    "frac_hbm_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+
         def gate_ups():
             for w in layers:
                 proj.gateUp(w["w1"], w["w3"], DIM, HIDDEN)
-        gu_graph = hip.capture(stream, gate_ups)
-        hip.launch(gu_graph, stream)
-        hip.record(e0, stream)
-        for _ in range(args.steps):
-            hip.launch(gu_graph, stream)
-        hip.record(e1, stream)
-        gate_up_avg = hip.elapsed_ms(e0, e1) / (args.steps * LAYERS)
-        gate_up_ms = [gate_up_avg] * (args.steps * LAYERS)
-        gate_up_bytes = 2 * gemv_bytes(HIDDEN, DIM)
 
-        ms = min(ms_step, ms_step_clean)
+        def qkvs():
+            for w in layers:
+                proj.fusedQKV(acts["xb"], acts["q"], acts["k"], acts["v"], w["wq"], w["wk"], w["wv"])
+
+        def os_():
+            for w in layers:
+                proj.residualMatvec(acts["xb"], w["wo"], DIM, DIM)
+
+        def downs():
+            for w in layers:
+                proj.residualMatvec(acts["hb"], w["w2"], HIDDEN, DIM)
+        gate_up_bytes = 2 * gemv_bytes(HIDDEN, DIM)
+        gu = per_kernel(gate_ups, LAYERS, gate_up_bytes)
+        kernels = {
+            "gate/up 2 x [8192 x 2048]": gu,
+            "q|k|v [3072 x 2048]": per_kernel(qkvs, LAYERS, gemv_bytes(DIM, DIM) + 2 * gemv_bytes(KV_DIM, DIM)),
+            "o [2048 x 2048] +=": per_kernel(os_, LAYERS, gemv_bytes(DIM, DIM)),
+            "down [2048 x 8192] +=": per_kernel(downs, LAYERS, gemv_bytes(DIM, HIDDEN)),
+        }
+        # the single-weight instances of the tile kernel (q|k|v, o, down, vocabulary) together:
+        # everything in the step that is not a gate/up launch
+        single_bytes = total_bytes - LAYERS * gate_up_bytes
+        single_ms = ms - LAYERS * gu["avg_launch_us"] * 1e-3
         gbs = total_bytes / (ms * 1e-3) / 1e9
-        achieved = gate_up_bytes / (gate_up_avg * 1e-3) / 1e9
+        achieved = gu["GB_s"]
         out = {
             "metric": "Q-GEMV HBM GB/s (% of peak) + prefill tok/s (% MFMA peak), 1xMI355X",
             "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -539,38 +886,48 @@ def main():
             "config": {"workload": "Q8_0 Llama-3.2-1B decode projection set, batch 1: 16 x (q|k|v, o, "
                                    "gate/up SwiGLU, down) + vocabulary projection, 65 launches/token "
                                    "replayed as one HIP graph",
-                       "bytes_per_step": total_bytes, "device": name, "compute_units": cu},
+                       "bytes_per_step": total_bytes, "device": name, "compute_units": cu,
+                       "peak_clock_khz": clock_khz},
             "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
             "tok_s": round(1e3 / ms, 1),
-            "ms_per_step_graph": round(ms_step_clean, 4),
-            "ms_per_step_python_launches": round(ms_step, 4),
-            "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
-            "roofline": {"bound": "hbm", "kernel": "jl_gemv_tiles<Q8_0, gate/up> 2 x [8192 x 2048]",
-                         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "ms_per_step_stats": spread_stats(step_ms),
+            "ms_per_step_python_launches": round(ms_python, 4),
+            "host_wall_ms_per_step": round(statistics.median(walls), 4),
+            "checks_rel_err": checks,
+            "roofline": {"bound": "hbm",
+                         "kernel": "jl_gemv_tiles<Q8_0, gate/up> 2 x [8192 x 2048]: the largest launch "
+                                   "shape of the step (16 of its 65 launches, 43 % of its bytes), not its "
+                                   "slowest -- see step_frac and single_weight_launches",
+                         "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
                          "bytes_per_launch": gate_up_bytes,
-                         "avg_launch_us": round(gate_up_avg * 1e3, 3),
-                         "launches_timed": len(gate_up_ms)},
+                         "avg_launch_us": gu["avg_launch_us"], "launch_us_stats": gu["us_stats"],
+                         "launches_timed": args.steps * LAYERS * REPS,
+                         "step_frac": round(gbs / HBM_PEAK_GBS, 4),
+                         "single_weight_launches": {
+                             "what": "the 49 launches of a step that are not gate/up (q|k|v, o, down, vocabulary)",
+                             "bytes": single_bytes, "ms": round(single_ms, 4),
+                             "GB_s": round(single_bytes / (single_ms * 1e-3) / 1e9, 1),
+                             "frac": round(single_bytes / (single_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}},
+            "decode_kernels": kernels,
         }
         legs = set() if args.no_extra else set(args.extra.split(","))
+        if "wq_shape" in legs:
+            out["wq_shape"] = bench_wq_shape(ctx, hip, t, args.steps, args.warmup, cpu)
         if "fused_rms" in legs:
-            out["decode_fused_rms"] = bench_fused_rms(ctx, hip, proj, layers, wcls, acts, args.steps,
+            out["decode_fused_rms"] = bench_fused_rms(ctx, hip, proj, layers, wcls, acts, host, args.steps,
                                                       args.warmup)
         if "prefill" in legs:
-            # (the matrix pipe's clock takes tens of milliseconds of load to settle: 100 untimed
-            # replays of the layer before the timed ones)
-            out["prefill"] = [bench_gemm(ctx, hip, t, T, args.steps, 100) for T in (512, 2048)]
+            out["prefill"] = [bench_gemm(ctx, hip, t, T, max(4, args.steps // 2), prefill_warmup, cpu and T == 512,
+                                         clock_khz, cu) for T in (512, 2048)]
         if "other_types" in legs:
             out["decode_other_types"] = [
-                bench_decode_layers(ctx, hip, "Q4_0", 4096, 1024, 14336, 4, args.steps, args.warmup),
-                bench_decode_layers(ctx, hip, "Q4_K", 4096, 1024, 12288, 4, args.steps, args.warmup)]
+                bench_decode_layers(ctx, hip, "Q4_0", 4096, 1024, 14336, 4, args.steps, args.warmup, cpu),
+                bench_decode_layers(ctx, hip, "Q4_K", 4096, 1024, 12288, 4, args.steps, args.warmup, cpu)]
         if "batched" in legs:
-            out["batched_q4k"] = [bench_batched_q4k(ctx, hip, B, max(5, args.steps // 5), 3)
+            out["batched_q4k"] = [bench_batched_q4k(ctx, hip, B, max(5, args.steps // 5), 3, cpu)
                                   for B in (8, 32, 64)]
-        if not args.no_cpu:
-            out["cpu_baseline"] = cpu_baseline(host, shapes, t)
-        else:
-            out["cpu_baseline"] = None
+        out["cpu_baseline"] = cpu_baseline(host, shapes, t) if cpu else None
     print(json.dumps(out))
 
 
