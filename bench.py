@@ -420,6 +420,33 @@ def bench_gemm(ctx, hip, t, T, steps, warmup, cpu, clock_khz, cu):
     # attention and SwiGLU kernels write fp16) and the hidden vector leaves as fp16
     half_proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=True)
     half = mode(*run(half_proj, X16, H16, hb16, widen=True))
+    # the block-scaled int8 path (JL_MATH_INT8: activations quantised per 32-block inside the call,
+    # int8 MFMA over the raw blocks, one fp32 scale product per block; Int8GemmKernels): its
+    # results are fixed bit for bit, so the check is equality with the oracle's int8 statement
+    from jitllm_amd import _lib as L
+    from oracle import pyoracle as O
+    i8_proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, math=L.JL_MATH_INT8)
+
+    def i8_layer():
+        i8_proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
+        i8_proj.projection(X, res, w["wo"], DIM, DIM, True)
+        i8_proj.gateUp(X, hb, w["w1"], w["w3"], DIM, HIDDEN)
+        i8_proj.projection(H, res, w["w2"], HIDDEN, DIM, True)
+    res.init(0.0)
+    i8_layer()
+    ctx.sync()
+    xq, xs = O.quantize_q8(Xh[arows])
+    hq, hs = O.quantize_q8(Hh[arows])
+    ro = sample_rows(DIM, 48, 56)
+    ref_o = O.gemm_int8_block_scaled(int(t), xq, xs, gather_rows(host["wo"], t, DIM, ro), ro.size)
+    ref_d = O.gemm_int8_block_scaled(int(t), hq, hs, gather_rows(host["w2"], t, HIDDEN, ro), ro.size)
+    got = res.get().reshape(T, DIM)[arows][:, ro]
+    if not np.array_equal(got.view(np.uint32), (ref_o + ref_d).astype(np.float32).view(np.uint32)):
+        raise SystemExit(f"bench.py: the int8 prefill path at T={T} differs from the oracle's int8 arithmetic")
+    int8 = mode(timed_graph(ctx, hip, i8_layer, steps, warmup), {"o+down": "bit-equal to the oracle's int8 statement"})
+    int8["frac_int8_mfma_peak"] = round(int8["tflops"] / INT8_MFMA_PEAK_TOPS, 4)
+    int8["math"] = ("int8 MFMA over the raw blocks, fp32 (float) dot * dA fused-multiplied by dW per 32-block in k order; "
+                    "bound by the three vector-ALU operations per int32 result at one sixth of the int8 MFMA peak")
     # the dominant kernel on its own: the gate/up call of that last mode is one launch of the fp16
     # GEMM and nothing else (four to a graph)
     def gate_ups():
@@ -452,7 +479,7 @@ def bench_gemm(ctx, hip, t, T, steps, warmup, cpu, clock_khz, cu):
            "check_rel_err": default["check_rel_err"],
            "math": "f16 MFMA, fp32 accumulate; weights decoded to fp16 inside the call (in LDS, or once per call into the workspace)",
            "with_resident_fp16_copy": kept, "with_resident_copy_and_fp16_activations": half,
-           "roofline": roofline}
+           "int8_block_scaled": int8, "roofline": roofline}
     if cpu:
         rows = sample_rows(HIDDEN, 224, 55)
         out["cpu_baseline"] = cpu_baseline_rows(t, host["w1"], DIM, rows, Xh, HIDDEN, 2.0, f"gate projection at T={T}")

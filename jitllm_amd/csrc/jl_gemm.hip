@@ -838,10 +838,7 @@ size_t scale_bytes(int64_t rows) { return round_up(round_up((size_t)rows, 256) *
 // traffic rule in choose_splits: splits * padded_rows <= row_bytes / 2, so splits * padded_rows *
 // columns * 4 <= columns * row_bytes * 2 with row_bytes <= 34 * cols / 32.
 size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_cols, int math) {
-    if (math == JL_MATH_INT8) {
-        size_t padded = round_up((size_t)max_rows, 128);
-        return round_up(padded * (size_t)cols, 256) + round_up(padded * (size_t)(cols / 32) * 4, 256);
-    }
+    if (math == JL_MATH_INT8) return jl_gemm_i8_workspace_bytes(max_rows, cols);
     // (256: the fp16 copy of a call's weights, which calls of a type without a decode-in-the-loop
     // kernel always make, is padded to whole 256-row column tiles)
     size_t planes = round_up(round_up((size_t)out_cols, 256) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
@@ -922,7 +919,11 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     if (math == JL_MATH_INT8) {
-        return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: the int8 kernels are not built into this library");
+        // block-scaled int8 arithmetic (Int8GemmKernels): a path of its own; fp16 operands and a
+        // resident fp16 copy have no meaning for it
+        if (half && half->x16) return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: the int8 path takes fp32 activations");
+        return jl_launch_gemm_i8(ctx, weights, count, X, C, batch, (int)active_rows, ldo, col_offset, epilogue,
+                                 workspace, workspace_bytes);
     }
     if (k % 256 != 0) {
         return jl_fail(JL_ERR_UNSUPPORTED,

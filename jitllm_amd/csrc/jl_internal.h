@@ -154,4 +154,10 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
 int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row_scale, float *C, int rows,
                           int n_total, int ntiles, int64_t plane, int splits, int64_t ldo, int64_t col_offset,
                           int epilogue);
+// JL_MATH_INT8: activations quantised per 32-block, int8 MFMA over the raw Q8_0 / Q4_0 blocks, one
+// fp32 scale product per block in k order.
+size_t jl_gemm_i8_workspace_bytes(int64_t max_rows, int64_t cols);
+int jl_launch_gemm_i8(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
+                      int64_t batch, int rows, int64_t ldo, int64_t col_offset, int epilogue, void *workspace,
+                      size_t workspace_bytes);
 size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_cols, int math);
