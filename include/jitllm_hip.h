@@ -283,8 +283,17 @@ size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols,
  *   X    [batch x cols] fp32 row-major          C  fp32, row stride `ldo` floats
  *   epilogue JL_STORE / JL_RESIDUAL, or JL_SWIGLU with count == 2 (gate, up):
  *            C[b][col_offset + j] = SiLU(X_b.W0_j) * (X_b.W1_j)
- *   math     a jl_gemm_math; JL_MATH_INT8 is JL_ERR_UNSUPPORTED (not built)
- * The row length must be a multiple of 256 columns, else JL_ERR_UNSUPPORTED.
+ *   math     a jl_gemm_math.  JL_MATH_INT8 (Q8_0 and Q4_0 weights; other types JL_ERR_UNSUPPORTED) is
+ *            the block-scaled int8 arithmetic of Int8GemmKernels.java:17-23 -- activations quantised
+ *            per 32-block inside the call (quantizeActivationsQ8Warp :96-129), each block's dot
+ *            product exact in int32, acc = fma((float) dot * dA, dW, acc) over the blocks in k order,
+ *            SwiGLU as (g / (1 + exp(-g))) * u in fp32 -- reproduced step by step, K never cut: the
+ *            fp32 results of JL_STORE / JL_RESIDUAL are those of that arithmetic bit for bit.  It
+ *            reads the raw blocks where they lie (gemmInt8Q8_0 :651-676) and takes row lengths that
+ *            are multiples of 64.  An opt-in mode: an activation carries 7 bits, so against the
+ *            fp32 CPU path it is looser than JL_MATH_F16 (every output within sum over the blocks
+ *            of (dA / 2) * sum |w|).
+ * JL_MATH_F16: the row length must be a multiple of 256 columns, else JL_ERR_UNSUPPORTED.
  * This is Int8GemmKernels.gemmInt8Q8_0's contract (:651-676: epilogue, rowsHolder, ldo,
  * colOffset) and gemmMMAQ8's, behind one call.
  */

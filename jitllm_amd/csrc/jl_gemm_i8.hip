@@ -13,7 +13,7 @@
 //   jl_quantize_rows_i8   X fp32 [rows x k] -> int8 [padded rows x k], dA as [k / 32][padded rows]
 //                         (block-major, so that the 32 rows of a matrix tile are consecutive) and,
 //                         for Q4_0, -8 * (sum of the block's int8 activations) in the same layout
-//   jl_gemm_i8<TYPE,WM,WN> v_mfma_i32_32x32x32_i8: one instruction is exactly one 32-block of a
+//   jl_gemm_i8<TYPE,MI,NJ> v_mfma_i32_32x32x32_i8: one instruction is exactly one 32-block of a
 //                         32 x 32 output patch.  The weights are read where they lie: a stage is 64
 //                         columns = two blocks = 68 (Q8_0) or 36 (Q4_0) consecutive bytes of every
 //                         weight row of the tile, copied into LDS by LDS-DMA as four (two) 16-byte
@@ -124,14 +124,17 @@ template <int TYPE> struct Raw {
 
 __device__ __forceinline__ float i8_swiglu(float g, float u) { return (g / (1.0f + __expf(-g))) * u; }
 
-// Workgroup = WM x WN waves, each a 64 x 64 patch (2 x 2 MFMA tiles) of a (64 WM) x (64 WN) tile:
-// BM activation rows x BN weight rows.  JL_SWIGLU: a wave's 64 weight rows are 32 gate rows and the
-// 32 up rows of the same outputs, so both halves of an output meet in one lane.
-template <int TYPE, int WM, int WN>
-__global__ void __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// Workgroup = 2 x 2 waves, each a patch of MI x NJ MFMA tiles of 32 x 32: a tile of BM = 64 MI
+// activation rows x BN = 64 NJ weight rows (128 x 128 or 64 x 64).  JL_SWIGLU: the weight rows of a
+// tile are 32-row runs of gate rows and of the up rows of the same outputs in turn -- a wave with
+// two column patches holds both halves of an output in one lane, waves with one exchange them
+// through LDS at the end.
+template <int TYPE, int MI, int NJ>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, MI == 2 ? 2 : 4)))
 jl_gemm_i8(I8Params p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr int BM = 64 * WM, BN = 64 * WN;
+    constexpr int WM = 2, WN = 2, NW = 4;
+    constexpr int BM = 32 * MI * WM, BN = 32 * NJ * WN;
     constexpr int PAIR = Raw<TYPE>::kPair, NP = Raw<TYPE>::kPlanes;
     constexpr bool Q4 = TYPE == JL_Q4_0;
     // stage layout
@@ -144,8 +147,9 @@ jl_gemm_i8(I8Params p) {
     constexpr int STAGE = SS_OFF + (Q4 ? S_REGION : 0);
     constexpr int NS = 3, AHEAD = NS - 1;
     // loads of one wave and stage
-    constexpr int LA = 4 / WN;      // 16-byte loads of the activation tile
-    constexpr int LW = NP / WM;     // 16-byte loads of the weight pieces
+    constexpr int LA = MI;                       // 16-byte loads of the activation tile
+    constexpr int LW = (NP * NJ + NW - 1) / NW;  // 16-byte loads of the weight pieces (waves repeat
+                                                 // one another's when there are fewer than four)
     constexpr int NL = LA + LW + 1 + 1 + (Q4 ? 1 : 0);
 
     const int tid = threadIdx.x;
@@ -184,7 +188,7 @@ jl_gemm_i8(I8Params p) {
         const uint8_t *w = seg_w;
         int row;
         if (swiglu) {
-            w = ((r >> 5) & 1) ? p.w_up : seg_w;
+            w = ((r >> 5) & 1) ? p.w_up : seg_w;           // (JL_SWIGLU runs with NJ == 2)
             row = nt * (BN / 2) + 32 * (r >> 6) + (r & 31);
         } else {
             row = (nt - seg_tile0) * BN + r;
@@ -211,14 +215,14 @@ jl_gemm_i8(I8Params p) {
         }
 #pragma unroll
         for (int j = 0; j < LW; j++, n++) {
-            const int q = wave * LW + j;                       // piece q / WN, rows 64 (q % WN) ..
-            const int piece = q / WN, r0 = 64 * (q % WN);
+            const int q = (wave * LW + j) % (NP * NJ);         // piece q / NJ, rows 64 (q % NJ) ..
+            const int piece = q / NJ, r0 = 64 * (q % NJ);
             src[n] = weight_row(r0 + lane) + piece * 16;
             step[n] = PAIR;
             dst[n] = W_OFF + piece * BN * 16 + r0 * 16;
         }
         {
-            const int r0 = 64 * (wave % WN);                   // the dword behind the pieces
+            const int r0 = 64 * (wave % NJ);                   // the dword behind the pieces
             src[n] = weight_row(r0 + lane) + NP * 16;
             step[n] = PAIR;
             dst[n] = WD_OFF + r0 * 4;
@@ -253,15 +257,15 @@ jl_gemm_i8(I8Params p) {
     };
 
     // ---- fragment addresses inside a stage
-    // activations: row wm 64 + mi 32 + l, 16-byte chunk 2 b + h at position chunk ^ ((row >> 2) & 3)
+    // activations: row wm 32 MI + mi 32 + l, 16-byte chunk 2 b + h at position chunk ^ ((row >> 2) & 3)
     uint32_t a_addr[2];
 #pragma unroll
-    for (int b = 0; b < 2; b++) a_addr[b] = A_OFF + (wm * 64 + l) * 64 + (((2 * b + h) ^ ((l >> 2) & 3)) << 4);
-    const uint32_t s_addr = (wm * 64 + 4 * h) * 4;    // + block * BM * 4 + mi * 128 + g * 32
-    // weights: row r = wn 64 + nj 32 + l.  Even block: the quants are bytes 2 + 16 h .. of the pair,
+    for (int b = 0; b < 2; b++) a_addr[b] = A_OFF + (wm * 32 * MI + l) * 64 + (((2 * b + h) ^ ((l >> 2) & 3)) << 4);
+    const uint32_t s_addr = (wm * 32 * MI + 4 * h) * 4;    // + block * BM * 4 + mi * 128 + g * 32
+    // weights: row r = wn 32 NJ + nj 32 + l.  Even block: the quants are bytes 2 + 16 h .. of the pair,
     // piece h from byte 2 on and the first two bytes of piece h + 1; odd block: bytes 36 + 16 h ..
     // (Q8_0; 20 .. for Q4_0, both halves), the last three dwords of a piece and the first of the next.
-    const int wr = wn * 64 + l;
+    const int wr = wn * 32 * NJ + l;
     uint32_t w1[2], w2[2], w3[2];
     if constexpr (!Q4) {
         w1[0] = W_OFF + h * BN * 16 + wr * 16;
@@ -279,11 +283,11 @@ jl_gemm_i8(I8Params p) {
         w3[1] = 0;
     }
 
-    floatx4 acc[2][2][4];
+    floatx4 acc[MI][NJ][4];
 #pragma unroll
-    for (int mi = 0; mi < 2; mi++)
+    for (int mi = 0; mi < MI; mi++)
 #pragma unroll
-        for (int nj = 0; nj < 2; nj++)
+        for (int nj = 0; nj < NJ; nj++)
 #pragma unroll
             for (int g = 0; g < 4; g++) acc[mi][nj][g] = floatx4{0.f, 0.f, 0.f, 0.f};
 
@@ -301,14 +305,14 @@ jl_gemm_i8(I8Params p) {
         const uint32_t base = lds0 + (s % NS) * STAGE;
 #pragma unroll
         for (int b = 0; b < 2; b++) {
-            intx4 fa[2], fb[2];
-            floatx4 da[2][4];
-            intx4 ss[2][4];
-            float dw[2];
+            intx4 fa[MI], fb[NJ];
+            floatx4 da[MI][4];
+            intx4 ss[MI][4];
+            float dw[NJ];
             // -- reads (by hand: the compiler would wait for the LDS-DMA loads before any LDS
             // access it can see)
 #pragma unroll
-            for (int mi = 0; mi < 2; mi++) {
+            for (int mi = 0; mi < MI; mi++) {
                 asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(fa[mi]) : "v"(base + a_addr[b]), "n"(mi * 2048) : "memory");
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
@@ -319,10 +323,10 @@ jl_gemm_i8(I8Params p) {
                                      : "v"(base + SS_OFF + b * BM * 4 + s_addr), "n"(mi * 128 + g * 32) : "memory");
                 }
             }
-            intx4 r1[2];
-            uint32_t r2[2], r3[2];
+            intx4 r1[NJ];
+            uint32_t r2[NJ], r3[NJ];
 #pragma unroll
-            for (int nj = 0; nj < 2; nj++) {
+            for (int nj = 0; nj < NJ; nj++) {
                 asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(r1[nj]) : "v"(base + w1[b]), "n"(nj * 512) : "memory");
                 // (the dword plane has 4-byte rows: 32 rows on are 128 bytes, not 512)
                 if (b == 1) {
@@ -335,16 +339,19 @@ jl_gemm_i8(I8Params p) {
                     asm volatile("ds_read_b32 %0, %1 offset:%2" : "=&v"(r3[nj]) : "v"(base + w3[b]), "n"(nj * 512) : "memory");
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            asm volatile("" : "+v"(fa[0]), "+v"(fa[1]), "+v"(r1[0]), "+v"(r1[1]), "+v"(r2[0]), "+v"(r2[1]));
-            if constexpr (!Q4) asm volatile("" : "+v"(r3[0]), "+v"(r3[1]));
 #pragma unroll
-            for (int mi = 0; mi < 2; mi++) {
-                asm volatile("" : "+v"(da[mi][0]), "+v"(da[mi][1]), "+v"(da[mi][2]), "+v"(da[mi][3]));
+            for (int nj = 0; nj < NJ; nj++) {
+                asm volatile("" : "+v"(r1[nj]), "+v"(r2[nj]));
+                if constexpr (!Q4) asm volatile("" : "+v"(r3[nj]));
+            }
+#pragma unroll
+            for (int mi = 0; mi < MI; mi++) {
+                asm volatile("" : "+v"(fa[mi]), "+v"(da[mi][0]), "+v"(da[mi][1]), "+v"(da[mi][2]), "+v"(da[mi][3]));
                 if constexpr (Q4) asm volatile("" : "+v"(ss[mi][0]), "+v"(ss[mi][1]), "+v"(ss[mi][2]), "+v"(ss[mi][3]));
             }
             // -- the weight operand and its scale
 #pragma unroll
-            for (int nj = 0; nj < 2; nj++) {
+            for (int nj = 0; nj < NJ; nj++) {
                 intx4 q;
                 if (b == 0) {
                     q[0] = (int)__builtin_amdgcn_alignbit((uint32_t)r1[nj][1], (uint32_t)r1[nj][0], 16);
@@ -371,20 +378,20 @@ jl_gemm_i8(I8Params p) {
             }
             // -- one MFMA per 32 x 32 patch and block, then (float) dot * dA, fused-multiplied by dW
             // into the accumulator: register 4 g + j of a patch is activation row 8 g + 4 h + j
-            intx16 dot[2][2];
+            intx16 dot[MI][NJ];
 #pragma unroll
-            for (int nj = 0; nj < 2; nj++)
+            for (int nj = 0; nj < NJ; nj++)
 #pragma unroll
-                for (int mi = 0; mi < 2; mi++) {
+                for (int mi = 0; mi < MI; mi++) {
                     intx16 c;
 #pragma unroll
                     for (int i = 0; i < 16; i++) c[i] = Q4 ? ss[mi][i >> 2][i & 3] : 0;
                     dot[mi][nj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[mi], fb[nj], c, 0, 0, 0);
                 }
 #pragma unroll
-            for (int nj = 0; nj < 2; nj++)
+            for (int nj = 0; nj < NJ; nj++)
 #pragma unroll
-                for (int mi = 0; mi < 2; mi++)
+                for (int mi = 0; mi < MI; mi++)
 #pragma unroll
                     for (int i = 0; i < 16; i++) {
                         const float t = (float)dot[mi][nj][i] * da[mi][i >> 2][i & 3];
@@ -395,27 +402,27 @@ jl_gemm_i8(I8Params p) {
 
     // ---- epilogue: a lane holds one output column and 16 activation rows of each patch
 #pragma unroll
-    for (int mi = 0; mi < 2; mi++) {
+    for (int mi = 0; mi < MI; mi++) {
 #pragma unroll
-        for (int nj = 0; nj < (2); nj++) {
+        for (int nj = 0; nj < NJ; nj++) {
             if (swiglu && nj == 1) continue;
             int col, limit;
             if (swiglu) {
                 col = nt * (BN / 2) + 32 * wn + l;
                 limit = seg_rows;
             } else {
-                col = (nt - seg_tile0) * BN + wn * 64 + nj * 32 + l;
+                col = (nt - seg_tile0) * BN + wn * 32 * NJ + nj * 32 + l;
                 limit = seg_rows;
             }
             if (col >= limit) continue;
             float *cbase = p.C + p.col_offset + seg_col0 + col;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int m = m0 + wm * 64 + mi * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
+                const int m = m0 + wm * 32 * MI + mi * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
                 if (m >= p.rows) continue;
                 float *dstp = cbase + (int64_t)m * p.ldo;
                 const float v = acc[mi][nj][i >> 2][i & 3];
-                if (swiglu) *dstp = i8_swiglu(v, acc[mi][1][i >> 2][i & 3]);
+                if (swiglu) *dstp = i8_swiglu(v, acc[mi][NJ - 1][i >> 2][i & 3]);
                 else if (p.epilogue == JL_RESIDUAL) *dstp += v;
                 else *dstp = v;
             }
@@ -423,10 +430,10 @@ jl_gemm_i8(I8Params p) {
     }
 }
 
-template <int TYPE, int WM, int WN>
+template <int TYPE, int MI, int NJ>
 int launch_i8(jl_context *ctx, const I8Params &p) {
-    auto fn = jl_gemm_i8<TYPE, WM, WN>;
-    constexpr int BM = 64 * WM, BN = 64 * WN;
+    auto fn = jl_gemm_i8<TYPE, MI, NJ>;
+    constexpr int BM = 64 * MI, BN = 64 * NJ;
     constexpr int region = 8 * BM < 1024 ? 1024 : 8 * BM;
     constexpr int stage = BM * 64 + Raw<TYPE>::kPlanes * BN * 16 + BN * 4 + region * (TYPE == JL_Q4_0 ? 2 : 1);
     constexpr int lds = 3 * stage;
@@ -437,9 +444,15 @@ int launch_i8(jl_context *ctx, const I8Params &p) {
     }
     const int total = p.ntiles * p.mtiles;
     const int grid = (total + 7) / 8 * 8;
-    hipLaunchKernelGGL(fn, dim3(grid), dim3(64 * WM * WN), lds, ctx->stream, p);
+    hipLaunchKernelGGL(fn, dim3(grid), dim3(256), lds, ctx->stream, p);
     JL_HIP(hipGetLastError());
     return JL_OK;
+}
+
+template <int TYPE>
+int launch_i8_tile(jl_context *ctx, const I8Params &p, int bm, int bn) {
+    if (bm == 128) return launch_i8<TYPE, 2, 2>(ctx, p);
+    return bn == 128 ? launch_i8<TYPE, 1, 2>(ctx, p) : launch_i8<TYPE, 1, 1>(ctx, p);
 }
 
 size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -475,16 +488,14 @@ int jl_launch_gemm_i8(jl_context *ctx, const jl_weight *const *weights, int coun
                        jl_gemm_i8_workspace_bytes(batch, k), workspace_bytes);
     }
     const bool swiglu = epilogue == JL_SWIGLU;
-    // Tile: 128 x 128 (four waves) when that gives most compute units a workgroup or two, else
-    // 64 x 64 (one wave), which cuts a narrow projection into four times as many.
-    int n_tiles_128 = 0, n_tiles_64 = 0;
-    for (int i = 0; i < (swiglu ? 1 : count); i++) {
-        const int r = (int)weights[i]->rows;
-        n_tiles_128 += (r + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128);
-        n_tiles_64 += (r + (swiglu ? 31 : 63)) / (swiglu ? 32 : 64);
-    }
-    const bool big = (int64_t)n_tiles_128 * ((rows + 127) / 128) >= (int64_t)ctx->compute_units * 3 / 2;
-    const int bm = big ? 128 : 64, bn = big ? 128 : 64;
+    // Tile: 128 x 128 when that gives most compute units a workgroup, else 64 rows x 64 columns
+    // (x 128 for gate/up, whose halves must meet in one wave), which cuts a narrow projection or a
+    // short batch into four (two) times as many workgroups.
+    int n_tiles_128 = 0;
+    for (int i = 0; i < (swiglu ? 1 : count); i++)
+        n_tiles_128 += ((int)weights[i]->rows + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128);
+    const bool big = (int64_t)n_tiles_128 * ((rows + 127) / 128) * 2 >= (int64_t)ctx->compute_units * 3;
+    const int bm = big ? 128 : 64, bn = (big || swiglu) ? 128 : 64;
     const int padded = (rows + bm - 1) / bm * bm;   // at most the 128-row padding the workspace holds
 
     int8_t *A8 = (int8_t *)workspace;
@@ -526,7 +537,5 @@ int jl_launch_gemm_i8(jl_context *ctx, const jl_weight *const *weights, int coun
     p.row_bytes = k / 32 * jl_block_bytes(type);
     p.ntiles = tiles;
     p.mtiles = padded / bm;
-    (void)n_tiles_64;
-    if (type == JL_Q8_0) return big ? launch_i8<JL_Q8_0, 2, 2>(ctx, p) : launch_i8<JL_Q8_0, 1, 1>(ctx, p);
-    return big ? launch_i8<JL_Q4_0, 2, 2>(ctx, p) : launch_i8<JL_Q4_0, 1, 1>(ctx, p);
+    return type == JL_Q8_0 ? launch_i8_tile<JL_Q8_0>(ctx, p, bm, bn) : launch_i8_tile<JL_Q4_0>(ctx, p, bm, bn);
 }
