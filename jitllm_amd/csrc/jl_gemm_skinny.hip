@@ -264,36 +264,6 @@ __device__ __forceinline__ void decode_slice(uint32_t row, int sl, half8 (&f)[8]
     }
 }
 
-// t[a] of lane group g (lanes 16 g .. 16 g + 15)  <-  t[g] of lane group a, for the four dwords
-// of each float4: two swaps of lane halves (lane bit 5 against a's high bit), then two swaps of
-// lane quarters (lane bit 4 against a's low bit).
-__device__ __forceinline__ void lane_group_transpose(float4 (&t)[4]) {
-    uint32_t v[4][4];
-#pragma unroll
-    for (int a = 0; a < 4; a++) {
-        v[a][0] = __float_as_uint(t[a].x); v[a][1] = __float_as_uint(t[a].y);
-        v[a][2] = __float_as_uint(t[a].z); v[a][3] = __float_as_uint(t[a].w);
-    }
-#pragma unroll
-    for (int d = 0; d < 4; d++) {
-#pragma unroll
-        for (int a0 = 0; a0 < 2; a0++) {   // upper lanes of t[a0] <-> lower lanes of t[2 + a0]
-            const auto r = __builtin_amdgcn_permlane32_swap(v[a0][d], v[2 + a0][d], false, false);
-            v[a0][d] = r[0];
-            v[2 + a0][d] = r[1];
-        }
-#pragma unroll
-        for (int a1 = 0; a1 < 2; a1++) {   // odd lane groups of t[2 a1] <-> even lane groups of t[2 a1 + 1]
-            const auto r = __builtin_amdgcn_permlane16_swap(v[2 * a1][d], v[2 * a1 + 1][d], false, false);
-            v[2 * a1][d] = r[0];
-            v[2 * a1 + 1][d] = r[1];
-        }
-    }
-#pragma unroll
-    for (int a = 0; a < 4; a++)
-        t[a] = float4{__uint_as_float(v[a][0]), __uint_as_float(v[a][1]), __uint_as_float(v[a][2]), __uint_as_float(v[a][3])};
-}
-
 __device__ __forceinline__ float skinny_swiglu(float g, float u) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u; }
 
 // Workgroup = 16 Ss compute threads (Ss / 4 waves) + kDmaWaves waves that do nothing but copy tiles.
@@ -305,6 +275,9 @@ constexpr int kDmaWaves = 2;
 // round trips, exponentials and stores that would otherwise stall the decode of the next tile.
 constexpr int kFoldWaves = 1;
 constexpr int max_slices(int) { return 32; }
+// The prologue's staging area of a compute wave: 8 activation rows x 256 columns as fp16, rows 16
+// bytes apart from a multiple of 256 so that the fragment reads of 16 lanes hit all banks.
+constexpr int kScratchRow = 528, kScratchPerWave = 8 * kScratchRow;
 
 // 16-byte loads per DMA wave and tile (upper bound): a tile row takes span_bytes + 16 bytes of LDS
 // (the padding spreads the 16 rows a wave reads at once over all banks), 16 rows, 128 lanes.
@@ -330,9 +303,11 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     const int total_groups = p.seg_group_begin[p.nseg];
     const int out_rows = DUAL ? kGroup / 2 : kGroup;   // outputs per group
 
+    // LDS: the tile ring, then the partial sums (two parities)
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
-    const uint32_t ring0 = lds0 + 2 * partial_bytes;
-    uint8_t *ring = lds + 2 * partial_bytes;
+    const uint32_t ring0 = lds0;
+    uint8_t *ring = lds;
+    const uint32_t part0 = lds0 + p.stages * stage_bytes;
 
     // The weight a row group belongs to.  The table is walked with constant indices: it then stays in
     // scalar registers, where an index computed at run time would turn every use into a load from
@@ -468,7 +443,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         float *const c_lane = p.C + (int64_t)(row0 + 4 * go) * p.ldo + p.col_offset + n;
         auto fold = [&](int group, int par) {
             const Segment sg = segment_of(group);
-            const uint32_t pbase = lds0 + par * partial_bytes + o * 16;
+            const uint32_t pbase = part0 + par * partial_bytes + o * 16;
             const int local = (group - sg.group_begin) * out_rows + n;   // output column inside the weight
 #pragma unroll
             for (int b = 0; b < NBB; b++) {
@@ -546,34 +521,26 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     half8 sums[NBB][ZIN];     // Q4_K: the two sub-blocks' activation sums, each as hi + lo, as k slots
     floatx4 undo[NBB][ZIN];
     {
-        // Every load of the prologue is issued before the first value is used.  Load n = 4 a + b
-        // of a lane fetches the 16-byte chunk 16 a + 4 b + g of its row's 256 columns, so that the
-        // four lanes of a row read 64 consecutive bytes (a lane reading its own slice chunk by
-        // chunk would touch 64 cache lines per instruction, and the cache looks up one line per
-        // clock: that alone took 4-7 us per launch).  The chunks are then dealt out by transposing
-        // a with g across the lane groups: afterwards register 4 a + b holds chunk 4 b + a of the
-        // lane's own slice.
+        // Every load of the prologue is issued before the first value is used, and every load
+        // instruction reads one row's 1 KB run of the wave's 256 columns: lane l holds columns
+        // 4 l .. 4 l + 3 of row r in register r.  (Loads shaped like the fragments -- a lane
+        // fetching pieces of its own row and slice -- touch 16 rows per instruction and took
+        // 2 us longer per launch: the cache looks up one line per clock.)  The rows are scaled,
+        // rounded to fp16 and turned into fragments through LDS, eight rows at a time, in a
+        // region of the wave's own: the last ring stage and the partial sums behind it, neither of
+        // which anybody touches before the first tile has been multiplied.
+        uint8_t *scr = lds + (p.stages - 1) * stage_bytes + wave * kScratchPerWave;
         float4 x[NBB * ZIN][16];
 #pragma unroll
         for (int b = 0; b < NBB; b++) {
 #pragma unroll
             for (int q = 0; q < ZIN; q++) {
-                const int m = row0 + 16 * b + c;
-                float4 raw[16];
-                if (m < p.rows) {
-                    const float4 *src = (const float4 *)(p.X + (int64_t)m * p.k + 64 * ((z * ZIN + q) * p.Ss + 4 * wave)) + g;
+                const float4 *src = (const float4 *)(p.X + 64 * ((z * ZIN + q) * p.Ss + 4 * wave)) + lane;
 #pragma unroll
-                    for (int n = 0; n < 16; n++) raw[n] = src[16 * (n >> 2) + 4 * (n & 3)];
-                } else {
-#pragma unroll
-                    for (int n = 0; n < 16; n++) raw[n] = float4{0.f, 0.f, 0.f, 0.f};
-                }
-#pragma unroll
-                for (int bb = 0; bb < 4; bb++) {
-                    float4 t[4] = {raw[bb], raw[4 + bb], raw[8 + bb], raw[12 + bb]};
-                    lane_group_transpose(t);
-#pragma unroll
-                    for (int a = 0; a < 4; a++) x[b * ZIN + q][4 * bb + a] = t[a];
+                for (int r = 0; r < 16; r++) {
+                    const int m = row0 + 16 * b + r;   // (uniform: a scalar branch)
+                    if (m < p.rows) x[b * ZIN + q][r] = *(const float4 *)((const float *)src + (int64_t)m * p.k);
+                    else x[b * ZIN + q][r] = float4{0.f, 0.f, 0.f, 0.f};
                 }
             }
         }
@@ -582,38 +549,80 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
 #pragma unroll
             for (int q = 0; q < ZIN; q++) {
                 const float4 (&xs)[16] = x[b * ZIN + q];
-                float amax = 0.f;
+                // The largest magnitude of each row's 256 columns.  Sixteen registers of per-lane
+                // maxima are folded over the lanes and halved twice on the way (a swap of lane
+                // halves puts row r and row r + 8 side by side, a swap of lane quarters rows r and
+                // r + 4), so lane group g ends with the maxima of rows 4 g .. 4 g + 3 -- the rows
+                // whose results its lanes will hold.
+                float v16[16];
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fabsf(xs[i].x)), __builtin_fabsf(xs[i].y));
-                    amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fabsf(xs[i].z)), __builtin_fabsf(xs[i].w));
+                for (int r = 0; r < 16; r++)
+                    v16[r] = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(xs[r].x), __builtin_fabsf(xs[r].y)),
+                                             __builtin_fmaxf(__builtin_fabsf(xs[r].z), __builtin_fabsf(xs[r].w)));
+                float v8[8], v4[4];
+#pragma unroll
+                for (int r = 0; r < 8; r++) {
+                    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v16[r]), __float_as_uint(v16[r + 8]), false, false);
+                    v8[r] = __builtin_fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
                 }
-                amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-                // amax = 1.f * 2^(E - 127): multiply by 2^(136 - E), undo with 2^(E - 136)
-                int E = (int)((__float_as_uint(amax) >> 23) & 0xFF);
-                E = E < 12 ? 12 : E;
-                const float inv = __uint_as_float((uint32_t)(263 - E) << 23);
-                const float un = __uint_as_float((uint32_t)(E - 9) << 23);
 #pragma unroll
-                for (int e = 0; e < 4; e++) undo[b][q][e] = __shfl(un, 4 * g + e, 64);
-                float part[2] = {0.f, 0.f};
-                const h2 ones = {(_Float16)1.f, (_Float16)1.f};
+                for (int r = 0; r < 4; r++) {
+                    const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v8[r]), __float_as_uint(v8[r + 4]), false, false);
+                    v4[r] = __builtin_fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                }
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const float4 lo = xs[2 * i], hi = xs[2 * i + 1];
-                    const half8 h = half8{(_Float16)(lo.x * inv), (_Float16)(lo.y * inv), (_Float16)(lo.z * inv),
-                                          (_Float16)(lo.w * inv), (_Float16)(hi.x * inv), (_Float16)(hi.y * inv),
-                                          (_Float16)(hi.z * inv), (_Float16)(hi.w * inv)};
-                    af[b][q][i] = h;
-                    if constexpr (TYPE == JL_Q4_K) {
-                        // sums of the values the MFMAs will see: at most 32 x 2^10, exact in fp32
+                for (int j = 0; j < 4; j++) {
+                    // rotations within the 16 lanes (DPP row_ror 8, 4, 2, 1): every lane ends with the maximum
+                    v4[j] = __builtin_fmaxf(v4[j], __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v4[j]), 0x128, 0xF, 0xF, false)));
+                    v4[j] = __builtin_fmaxf(v4[j], __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v4[j]), 0x124, 0xF, 0xF, false)));
+                    v4[j] = __builtin_fmaxf(v4[j], __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v4[j]), 0x122, 0xF, 0xF, false)));
+                    v4[j] = __builtin_fmaxf(v4[j], __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v4[j]), 0x121, 0xF, 0xF, false)));
+                }
+                // amax = 1.f * 2^(E - 127): multiply by 2^(136 - E), undo with 2^(E - 136); the
+                // row's largest value lands in [2^9, 2^10), which keeps huge rows finite, tiny rows
+                // out of fp16's subnormals and a sub-block's sum of 32 inside fp16's range
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    int E = (int)((__float_as_uint(v4[e]) >> 23) & 0xFF);
+                    E = E < 12 ? 12 : E;
+                    undo[b][q][e] = __uint_as_float((uint32_t)(E - 9) << 23);
+                }
+                float inv[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const uint32_t bits = __builtin_amdgcn_readlane(__float_as_uint(v4[r & 3]), 16 * (r >> 2));
+                    int E = (int)((bits >> 23) & 0xFF);
+                    E = E < 12 ? 12 : E;
+                    inv[r] = __uint_as_float((uint32_t)(263 - E) << 23);
+                }
+#pragma unroll
+                for (int pass = 0; pass < 2; pass++) {
+#pragma unroll
+                    for (int rr = 0; rr < 8; rr++) {
+                        const int r = 8 * pass + rr;
+                        typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+                        const half4 h = {(_Float16)(xs[r].x * inv[r]), (_Float16)(xs[r].y * inv[r]),
+                                         (_Float16)(xs[r].z * inv[r]), (_Float16)(xs[r].w * inv[r])};
+                        *(half4 *)(scr + rr * kScratchRow + lane * 8) = h;
+                    }
+                    __builtin_amdgcn_wave_barrier();   // (LDS serves a wave's accesses in order)
+                    if ((c >> 3) == pass) {
+#pragma unroll
+                        for (int i = 0; i < 8; i++) af[b][q][i] = *(const half8 *)(scr + (c & 7) * kScratchRow + 128 * g + 16 * i);
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+                if constexpr (TYPE == JL_Q4_K) {
+                    // sums of the values the MFMAs will see: at most 32 x 2^10, exact in fp32
+                    float part[2] = {0.f, 0.f};
+                    const h2 ones = {(_Float16)1.f, (_Float16)1.f};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const half8 h = af[b][q][i];
 #pragma unroll
                         for (int e = 0; e < 8; e += 2)
                             part[i >> 2] = __builtin_amdgcn_fdot2(h2{h[e], h[e + 1]}, ones, part[i >> 2], false);
                     }
-                }
-                if constexpr (TYPE == JL_Q4_K) {
                     const _Float16 z16 = (_Float16)0.f;
                     const _Float16 h0 = (_Float16)part[0], h1 = (_Float16)part[1];
                     sums[b][q] = half8{h0, (_Float16)(part[0] - (float)h0), h1, (_Float16)(part[1] - (float)h1), z16, z16, z16, z16};
@@ -660,7 +669,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         asm volatile("" : "+v"(total[0]));
         STAMP(5 + 4 * (it * ZIN + ZIN - 1));
         // plain arithmetic happened on the MFMA results: the compiler placed the wait states itself
-        const uint32_t pw = lds0 + (it & 1) * partial_bytes + wave * (NBB * 1024) + lane * 16;
+        const uint32_t pw = part0 + (it & 1) * partial_bytes + wave * (NBB * 1024) + lane * 16;
 #pragma unroll
         for (int b = 0; b < NBB; b++) lds_write_f4(pw + b * 1024, total[b]);
     }
@@ -814,6 +823,8 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     int stages = (160 * 1024 - partial) / stage_bytes;
     if (stages > 4) stages = 4;
     if (stages < 2) return JL_OK;
+    // the prologue's staging area is the last stage and the partial sums behind it
+    if ((threads / 64) * kScratchPerWave > stage_bytes + partial) return JL_OK;
     p.stages = stages;
     const int lds = partial + stages * stage_bytes;
     *taken = true;
