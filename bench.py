@@ -759,6 +759,57 @@ def prefill_probe(ctx, t, T=2048):
                       "mfma_f16_flops_per_instruction_16x16x32": 2 * 16 * 16 * 32}))
 
 
+def batched_probe(ctx):
+    """What the kernel trace of the batched-decode kernels is collected on: the four calls of one
+    Q4_K Qwen3-8B-like layer (q|k|v, o +=, gate/up SwiGLU, down +=) at 8, 32 and 64 rows, launched
+    kernel by kernel over three device copies of the layer in turn (325 MB, more than the
+    memory-side cache holds), four rounds each."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.projections import QuantizedBatchProjections
+    t = GGMLType.Q4_K
+    dim, kv, ffn = 4096, 1024, 12288
+    shapes = {"wq": (dim, dim), "wk": (kv, dim), "wv": (kv, dim), "wo": (dim, dim),
+              "w1": (ffn, dim), "w3": (ffn, dim), "w2": (dim, ffn)}
+    host = {k: synthetic.weight(t, r, c, 61 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
+    layers = [{k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes} for _ in range(3)]
+    for B in (8, 32, 64):
+        X = ctx.from_numpy(synthetic.activations((B, dim), 68))
+        H = ctx.from_numpy(synthetic.activations((B, ffn), 69) * np.float32(0.1))
+        qkv, res, hb = ctx.float_array(B * (dim + 2 * kv)), ctx.float_array(B * dim, fill=0.0), ctx.float_array(B * ffn)
+        proj = QuantizedBatchProjections(ctx, B, ffn, 2 * ffn)
+        for _ in range(4):
+            for w in layers:
+                proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
+                proj.projection(X, res, w["wo"], dim, dim, True)
+                proj.gateUp(X, hb, w["w1"], w["w3"], dim, ffn)
+                proj.projection(H, res, w["w2"], ffn, dim, True)
+            ctx.sync()
+    print(json.dumps({"weight_bytes": {k: int(v.size) for k, v in host.items()}}))
+
+
+def int8_probe(ctx, t, T=2048):
+    """What the counters and the kernel trace of the int8 prefill path are collected on: one
+    Llama-3.2-1B layer's four calls at T tokens with JL_MATH_INT8, kernel by kernel, four times."""
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    shapes = {"wq": (DIM, DIM), "wk": (KV_DIM, DIM), "wv": (KV_DIM, DIM), "wo": (DIM, DIM),
+              "w1": (HIDDEN, DIM), "w3": (HIDDEN, DIM), "w2": (DIM, HIDDEN)}
+    w = {k: ctx.load_weight(t, synthetic.weight(t, r, c, 41 + i), r, c) for i, (k, (r, c)) in enumerate(shapes.items())}
+    X = ctx.from_numpy(synthetic.activations((T, DIM), 48))
+    H = ctx.from_numpy(synthetic.activations((T, HIDDEN), 49) * np.float32(0.1))
+    qkv, res, hb = ctx.float_array(T * (DIM + 2 * KV_DIM)), ctx.float_array(T * DIM, fill=0.0), ctx.float_array(T * HIDDEN)
+    proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, math=L.JL_MATH_INT8)
+    for _ in range(4):
+        proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
+        proj.projection(X, res, w["wo"], DIM, DIM, True)
+        proj.gateUp(X, hb, w["w1"], w["w3"], DIM, HIDDEN)
+        proj.projection(H, res, w["w2"], HIDDEN, DIM, True)
+        ctx.sync()
+    print(json.dumps({"tokens": T, "macs": {"q|k|v": T * DIM * (DIM + 2 * KV_DIM), "o": T * DIM * DIM,
+                                            "gate/up": T * 2 * HIDDEN * DIM, "down": T * HIDDEN * DIM}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -774,6 +825,10 @@ def main():
                     help="only launch what the HBM-traffic counters are read on (see traffic_probe)")
     ap.add_argument("--prefill-probe", action="store_true",
                     help="only launch what the matrix-pipe counters are read on (see prefill_probe)")
+    ap.add_argument("--batched-probe", action="store_true",
+                    help="only launch the batched-decode calls, kernel by kernel (see batched_probe)")
+    ap.add_argument("--int8-probe", action="store_true",
+                    help="only launch the int8 prefill calls, kernel by kernel (see int8_probe)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path is built and measured on a single MI355X; "
@@ -795,6 +850,12 @@ def main():
         clock_khz = hip.clock_khz(0)
         if args.prefill_probe:
             prefill_probe(ctx, t)
+            return
+        if args.batched_probe:
+            batched_probe(ctx)
+            return
+        if args.int8_probe:
+            int8_probe(ctx, t)
             return
         layers, wcls, acts, host, shapes = build_decode_set(ctx, t)
         ws = TornadoWorkspace(wrapX=acts["x"], wrapXb=acts["xb"], wrapHb=acts["hb"])

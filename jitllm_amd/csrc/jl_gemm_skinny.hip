@@ -686,33 +686,58 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
 #endif
 }
 
-// Adds the spans' partial sums in span order and applies row scale and epilogue; one thread per
-// (activation row, weight row of a group).
+// Adds the spans' partial sums in span order and applies the epilogue; one thread per activation
+// row and four consecutive weight rows of a group (16-byte loads from the planes).
 template <bool DUAL>
 __global__ void __launch_bounds__(256) jl_skinny_reduce(SkinnyParams p, int padded_rows) {
     const int total_groups = p.seg_group_begin[p.nseg];
-    const int v = blockIdx.x * blockDim.x + threadIdx.x;  // group * 16 + row of the group
+    const int v = (blockIdx.x * blockDim.x + threadIdx.x) * 4;  // group * 16 + first row of the group
     const int m = blockIdx.y;
     if (v >= total_groups * 16 || m >= p.rows) return;
     const int group = v >> 4, r = v & 15;
     if (DUAL && r >= 8) return;
-    int seg = 0;
-    for (int i = 1; i < kMaxSeg; i++)
-        if (i < p.nseg && group >= p.seg_group_begin[i]) seg = i;
+    int seg_rows = p.seg_rows[0], seg_begin = 0, seg_col = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxSeg; i++) {
+        if (i < p.nseg && group >= p.seg_group_begin[i]) {
+            seg_rows = p.seg_rows[i];
+            seg_begin = p.seg_group_begin[i];
+            seg_col = p.seg_col_begin[i];
+        }
+    }
     const int out_rows = DUAL ? 8 : 16;
-    const int local = (group - p.seg_group_begin[seg]) * out_rows + r;
-    if (local >= p.seg_rows[seg]) return;
+    const int local = (group - seg_begin) * out_rows + r;
+    if (local >= seg_rows) return;
     const int64_t width = (int64_t)total_groups * 16;
     const float *pp = p.planes + (int64_t)m * width + v;
-    float s = 0.f, u = 0.f;
+    float4 s = {0.f, 0.f, 0.f, 0.f}, u = {0.f, 0.f, 0.f, 0.f};
     for (int zz = 0; zz < p.Z; zz++) {
-        s += pp[(int64_t)zz * padded_rows * width];
-        if (DUAL) u += pp[(int64_t)zz * padded_rows * width + 8];
+        const float4 a = *(const float4 *)(pp + (int64_t)zz * padded_rows * width);
+        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+        if (DUAL) {
+            const float4 c = *(const float4 *)(pp + (int64_t)zz * padded_rows * width + 8);
+            u.x += c.x; u.y += c.y; u.z += c.z; u.w += c.w;
+        }
     }
-    float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + p.seg_col_begin[seg] + local;
-    if (DUAL) *dst = skinny_swiglu(s, u);
-    else if (p.epilogue == JL_RESIDUAL) *dst += s;
-    else *dst = s;
+    float out[4] = {s.x, s.y, s.z, s.w};
+    if (DUAL) {
+        out[0] = skinny_swiglu(s.x, u.x); out[1] = skinny_swiglu(s.y, u.y);
+        out[2] = skinny_swiglu(s.z, u.z); out[3] = skinny_swiglu(s.w, u.w);
+    }
+    float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + seg_col + local;
+    const bool add = !DUAL && p.epilogue == JL_RESIDUAL;
+    if (local + 3 < seg_rows && (((uintptr_t)dst) & 15) == 0) {
+        if (add) {
+            const float4 o = *(const float4 *)dst;
+            *(float4 *)dst = float4{o.x + out[0], o.y + out[1], o.z + out[2], o.w + out[3]};
+        } else {
+            *(float4 *)dst = float4{out[0], out[1], out[2], out[3]};
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if (local + e < seg_rows) dst[e] = add ? dst[e] + out[e] : out[e];
+    }
 }
 
 #ifdef JL_SKINNY_PROBE
@@ -740,7 +765,7 @@ int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int gro
                        ctx->stream, p);
     JL_HIP(hipGetLastError());
     if (p.Z > 1) {
-        hipLaunchKernelGGL(jl_skinny_reduce<DUAL>, dim3((groups * 16 + 255) / 256, p.rows), dim3(256), 0,
+        hipLaunchKernelGGL(jl_skinny_reduce<DUAL>, dim3((groups * 4 + 255) / 256, p.rows), dim3(256), 0,
                            ctx->stream, p, 16 * NBB * p.row_blocks);
         JL_HIP(hipGetLastError());
     }
