@@ -428,9 +428,22 @@ __device__ __forceinline__ uintptr_t uniform_value(uintptr_t v) {
     return v;
 }
 
+#ifdef JL_GEMV_STAMPS
+// Timing experiments only: the 100 MHz real-time counter at eight points of every workgroup's
+// life, kept in scalar registers and written out when the workgroup is done.
+__device__ uint64_t *jl_gemv_stamp_buf = nullptr;
+#define GSTAMP(k) do { stamp[k] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define GSTAMP(k) do { } while (0)
+#endif
+
 template <int TYPE, bool DUAL, bool RMS, bool PACKED = false>
 __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     static_assert(!(RMS && PACKED), "the packed activation is normalised before it is quantised");
+#ifdef JL_GEMV_STAMPS
+    uint64_t stamp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
+    GSTAMP(0);
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
     constexpr int L = X4 + 1;                     // plus one 4-byte load
@@ -525,6 +538,10 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         }
     };
 
+#ifdef JL_GEMV_STAMPS
+    asm volatile("" :: "v"(slot_off[0]), "s"(total_tiles), "s"(half_bytes));   // the arguments have arrived
+#endif
+    GSTAMP(1);
     // my tiles: blockIdx.x, blockIdx.x + gridDim.x, ...
     const int first = blockIdx.x;
     const int mine = first < total_tiles ? (total_tiles - first + gridDim.x - 1) / gridDim.x : 0;
@@ -554,6 +571,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
     const bool x_in_ring = x_bytes <= stage_bytes;  // else a region of its own after the ring
     uint8_t *xs = x_in_ring ? ring + (kStages - 1) * stage_bytes : ring + kStages * stage_bytes;
     const uint32_t xs0 = x_in_ring ? ring0 + (kStages - 1) * stage_bytes : ring0 + kStages * stage_bytes;
+    int issued = 0;
     if constexpr (!rms && !PACKED) {
         for (int base = 0; base < x_bytes; base += nthreads * 16) {
             const int q = base / 16 + tid;
@@ -563,7 +581,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
                                              (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
         }
     }
-    int issued = 0;
+    GSTAMP(2);
     for (; issued < kStages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
     if constexpr (rms) {
         // RMS normalisation folded into the activation load.  CpuOperations.rmsnorm
@@ -633,8 +651,10 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
             }
         }
     }
+    GSTAMP(3);
     wait_vm_tiles<L>(issued);
     __builtin_amdgcn_s_barrier();
+    GSTAMP(4);
 
     float x[64];
     float sx[2] = {0.f, 0.f};
@@ -722,6 +742,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         // with two stages nothing was issued after tile `it`: its loads are the youngest
         JL_WAIT_VM(0);
         __builtin_amdgcn_s_barrier();
+        if (it == mine - 1) GSTAMP(5);
         // the stage that tile it - 1 (or, the first time round, the activation vector) occupied
         // is free now: every wave is past its reads
         if (issued < mine) {
@@ -735,6 +756,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
             if constexpr (PACKED) v = slice_dot_lds_packed<TYPE>(ring0 + (it % kStages) * stage_bytes, r, s, p.row_bytes, px);
             else v = slice_dot_lds<TYPE>(ring0 + (it % kStages) * stage_bytes, r, s, p.row_bytes, x, sx);
         }
+        if (it == mine - 1) GSTAMP(6);
         if (p.Sp >= 2) v += quad_xor1(v);
         if (p.Sp >= 4) v += quad_xor2(v);
         if (r < p.R && (p.Sp < 4 ? s == 0 : (s & 3) == 0)) {
@@ -746,6 +768,12 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         __builtin_amdgcn_s_barrier();
         finish(first + (mine - 1) * gridDim.x, (mine - 1) & 1);
     }
+    GSTAMP(7);
+#ifdef JL_GEMV_STAMPS
+    if (jl_gemv_stamp_buf && tid == 0) {
+        for (int k = 0; k < 8; k++) jl_gemv_stamp_buf[(size_t)blockIdx.x * 8 + k] = stamp[k];
+    }
+#endif
 }
 
 // Catch-all for shapes the tile kernel does not take (row length not a multiple of 64, rows wider
@@ -875,6 +903,12 @@ int launch_generic(jl_context *ctx, const jl_weight *w, const jl_weight *w_up, c
 }
 
 }  // namespace
+
+#ifdef JL_GEMV_STAMPS
+extern "C" int jl_probe_gemv_stamps(uint64_t *device_buffer) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(jl_gemv_stamp_buf), &device_buffer, sizeof(device_buffer));
+}
+#endif
 
 int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *const *outs,
                    const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms, const jl_q8x *xq) {
