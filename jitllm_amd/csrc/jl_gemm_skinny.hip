@@ -264,6 +264,31 @@ __device__ __forceinline__ void decode_slice(uint32_t row, int sl, half8 (&f)[8]
     }
 }
 
+// ---- the prologue's arithmetic, by hand.  Written with fmaxf / casts the compiler spends an
+// instruction on every |x| and on every operand of a maximum (it must quiet signalling NaNs), four
+// on a DPP step and seven on rounding four products to fp16; these are the instructions themselves.
+
+// max(|a|, |b|, |c|, |d|)
+__device__ __forceinline__ float max_abs4(const float4 &v) {
+    float m;
+    asm("v_max3_f32 %0, |%1|, |%2|, |%3|\n\tv_max_f32 %0, %0, |%4|" : "=&v"(m) : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w));
+    return m;
+}
+__device__ __forceinline__ float max_raw(float a, float b) {
+    float m;
+    asm("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(a), "v"(b));
+    return m;
+}
+// max(v, v rotated by N lanes within its row of 16); two wait states between a vector write and a
+// DPP read of the same register
+#define JL_MAX_ROR(v, N) asm("s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_ror:" #N " row_mask:0xf bank_mask:0xf" : "+v"(v))
+// fp16(a * scale) | fp16(b * scale) << 16, each product rounded once (the scale is a power of two)
+__device__ __forceinline__ uint32_t scaled_pair_f16(float a, float b, float scale) {
+    uint32_t r;
+    asm("v_fma_mixlo_f16 %0, %1, %3, 0\n\tv_fma_mixhi_f16 %0, %2, %3, 0" : "=&v"(r) : "v"(a), "v"(b), "s"(scale));
+    return r;
+}
+
 __device__ __forceinline__ float skinny_swiglu(float g, float u) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u; }
 
 // Workgroup = 16 Ss compute threads (Ss / 4 waves) + kDmaWaves waves that do nothing but copy tiles.
@@ -556,27 +581,25 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                 // whose results its lanes will hold.
                 float v16[16];
 #pragma unroll
-                for (int r = 0; r < 16; r++)
-                    v16[r] = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(xs[r].x), __builtin_fabsf(xs[r].y)),
-                                             __builtin_fmaxf(__builtin_fabsf(xs[r].z), __builtin_fabsf(xs[r].w)));
+                for (int r = 0; r < 16; r++) v16[r] = max_abs4(xs[r]);
                 float v8[8], v4[4];
 #pragma unroll
                 for (int r = 0; r < 8; r++) {
                     const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v16[r]), __float_as_uint(v16[r + 8]), false, false);
-                    v8[r] = __builtin_fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                    v8[r] = max_raw(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
                 }
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v8[r]), __float_as_uint(v8[r + 4]), false, false);
-                    v4[r] = __builtin_fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                    v4[r] = max_raw(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
                 }
+                // rotations within the 16 lanes: every lane ends with the maximum
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    // rotations within the 16 lanes (DPP row_ror 8, 4, 2, 1): every lane ends with the maximum
-                    v4[j] = __builtin_fmaxf(v4[j], __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v4[j]), 0x128, 0xF, 0xF, false)));
-                    v4[j] = __builtin_fmaxf(v4[j], __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v4[j]), 0x124, 0xF, 0xF, false)));
-                    v4[j] = __builtin_fmaxf(v4[j], __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v4[j]), 0x122, 0xF, 0xF, false)));
-                    v4[j] = __builtin_fmaxf(v4[j], __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v4[j]), 0x121, 0xF, 0xF, false)));
+                    JL_MAX_ROR(v4[j], 8);
+                    JL_MAX_ROR(v4[j], 4);
+                    JL_MAX_ROR(v4[j], 2);
+                    JL_MAX_ROR(v4[j], 1);
                 }
                 // amax = 1.f * 2^(E - 127): multiply by 2^(136 - E), undo with 2^(E - 136); the
                 // row's largest value lands in [2^9, 2^10), which keeps huge rows finite, tiny rows
@@ -600,10 +623,8 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
 #pragma unroll
                     for (int rr = 0; rr < 8; rr++) {
                         const int r = 8 * pass + rr;
-                        typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-                        const half4 h = {(_Float16)(xs[r].x * inv[r]), (_Float16)(xs[r].y * inv[r]),
-                                         (_Float16)(xs[r].z * inv[r]), (_Float16)(xs[r].w * inv[r])};
-                        *(half4 *)(scr + rr * kScratchRow + lane * 8) = h;
+                        *(uint2 *)(scr + rr * kScratchRow + lane * 8) =
+                            uint2{scaled_pair_f16(xs[r].x, xs[r].y, inv[r]), scaled_pair_f16(xs[r].z, xs[r].w, inv[r])};
                     }
                     __builtin_amdgcn_wave_barrier();   // (LDS serves a wave's accesses in order)
                     if ((c >> 3) == pass) {
