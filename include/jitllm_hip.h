@@ -50,10 +50,11 @@ typedef enum jl_status {
  * of "Q4_K_M" files are Q6_K, "Q5_K_M" files are Q5_K with Q6_K), and the types quantisers mix
  * into other files -- Q4_1 (20 B / 32, GGMLType.java:8), Q5_0 (22 B / 32, :11) and IQ4_XS
  * (136 B / 256, :39-41) -- have
- * jl_dequant_f32, jl_gemv and jl_gemm -- the latter always by decoding the weights to fp16 into the
- * workspace first, whatever the row count -- while the fused single-token entry points return
- * JL_ERR_UNSUPPORTED for them (the reference fuses gate/up for Q5_K but not Q6_K,
- * QuantizedProjections.java:386-393; a caller that gets JL_ERR_UNSUPPORTED runs the unfused steps). */
+ * jl_dequant_f32, jl_gemv, jl_gemv_gate_up and jl_gemm -- the latter always by decoding the weights
+ * to fp16 into the workspace first, whatever the row count.  (Of these the reference fuses gate/up
+ * for Q5_K only, QuantizedProjections.java:386-393; the one-launch form is there for all five.)  The
+ * fused q|k|v, RMS-folding and packed-activation single-token entry points return
+ * JL_ERR_UNSUPPORTED for them; a caller that gets JL_ERR_UNSUPPORTED runs the unfused steps. */
 typedef enum jl_ggml_type {
     JL_Q4_0 = 2, JL_Q4_1 = 3, JL_Q5_0 = 6, JL_Q8_0 = 8, JL_Q4_K = 12, JL_Q5_K = 13, JL_Q6_K = 14, JL_IQ4_XS = 23
 } jl_ggml_type;
@@ -150,8 +151,9 @@ int jl_gemv_qkv(jl_context *ctx, const jl_weight *wq, const jl_weight *wk, const
 /*
  * hb = SiLU(W1.x) * (W3.x) in one launch (fusedFeedForwardWithSiLUAndGLUActivationQ8_0Byte,
  * TransformerComputeKernelsLayered.java:2453-2479; fusedFFNGateUpSiLUQ4_0; fusedFFNGateUpSiLUQ4_K;
- * QuantizedProjections.gateUp :400-480).  Both weights share type and shape; a mixed pair is
- * JL_ERR_UNSUPPORTED and the caller runs two jl_gemv and jl_swiglu, as the reference does.
+ * the Q5_K sibling; QuantizedProjections.gateUp :400-480).  Every weight type with a jl_gemv has
+ * it.  Both weights share type and shape; a mixed pair is JL_ERR_UNSUPPORTED and the caller runs
+ * two jl_gemv and jl_swiglu, as the reference does.
  */
 int jl_gemv_gate_up(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, const float *x,
                     float *hb);

@@ -919,11 +919,11 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
         return jl_fail(JL_ERR_UNSUPPORTED, "no packed-activation kernel for a %s weight", jl_type_name(type));
     }
     if (!jl_has_fused_kernels(type)) {
-        if (nseg != 1 || w_up || rms) {
-            return jl_fail(JL_ERR_UNSUPPORTED, "no fused single-token kernel for a %s weight "
-                                               "(plain and residual projections only)", jl_type_name(type));
+        if (nseg != 1 || rms) {
+            return jl_fail(JL_ERR_UNSUPPORTED, "no fused q|k|v or RMS-folding single-token kernel for a %s weight "
+                                               "(plain, residual and gate/up projections only)", jl_type_name(type));
         }
-        return jl_launch_gemv_direct(ctx, w[0], x, outs[0], epilogue);
+        return jl_launch_gemv_direct(ctx, w[0], w_up, x, outs[0], epilogue);
     }
 
     const bool dual = w_up != nullptr;

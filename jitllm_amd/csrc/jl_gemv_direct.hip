@@ -223,10 +223,13 @@ template <> struct Geometry<JL_Q4_1> { static constexpr int kBytes = 160; };
 template <> struct Geometry<JL_Q5_0> { static constexpr int kBytes = 176; };
 template <> struct Geometry<JL_IQ4_XS> { static constexpr int kBytes = 136; };
 
-template <int TYPE>
+// DUAL: `w_up` is a second weight of the same shape and a row's result is SiLU(w . x) * (w_up . x),
+// the fused gate/up of the feed-forward block (the reference fuses it for Q5_K,
+// J/backend/tornado/layers/QuantizedProjections.java:386-393).
+template <int TYPE, bool DUAL>
 __global__ void __launch_bounds__(256)
-jl_gemv_direct(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out, int rows,
-               int n, int epilogue) {
+jl_gemv_direct(const uint8_t *__restrict__ w, const uint8_t *__restrict__ w_up, const float *__restrict__ x,
+               float *__restrict__ out, int rows, int n, int epilogue) {
     constexpr int BB = Geometry<TYPE>::kBytes;
     const int lane = threadIdx.x & 63;
     const int waves = (gridDim.x * blockDim.x) >> 6;
@@ -234,26 +237,33 @@ jl_gemv_direct(const uint8_t *__restrict__ w, const float *__restrict__ x, float
     const int j = lane & 15;
     for (int row = (blockIdx.x * blockDim.x + threadIdx.x) >> 6; row < rows; row += waves) {
         const uint8_t *wr = w + (int64_t)row * blocks * BB;
-        float acc = 0.f;
+        const uint8_t *ur = DUAL ? w_up + (int64_t)row * blocks * BB : nullptr;
+        float acc = 0.f, acc_up = 0.f;
         // two super-blocks per lane and trip: all their loads are issued before the first use
         for (int sb0 = lane >> 4; sb0 < blocks; sb0 += 8) {
-            Raw<TYPE> r[2];
+            Raw<TYPE> r[2], ru[2];
             Xs v[2];
 #pragma unroll
             for (int u = 0; u < 2; u++) {
                 const int sb = sb0 + 4 * u;
                 if (sb < blocks) {
                     r[u] = load_raw<TYPE>(wr + sb * BB, j);
+                    if constexpr (DUAL) ru[u] = load_raw<TYPE>(ur + sb * BB, j);
                     v[u] = load_x<TYPE>(x + sb * 256, j);
                 }
             }
 #pragma unroll
             for (int u = 0; u < 2; u++)
-                if (sb0 + 4 * u < blocks) acc += block_part<TYPE>(r[u], v[u], j);
+                if (sb0 + 4 * u < blocks) {
+                    acc += block_part<TYPE>(r[u], v[u], j);
+                    if constexpr (DUAL) acc_up += block_part<TYPE>(ru[u], v[u], j);
+                }
         }
         acc = jl_group_sum<JL_WAVE>(acc);
+        if constexpr (DUAL) acc_up = jl_group_sum<JL_WAVE>(acc_up);
         if (lane == 0) {
-            if (epilogue == JL_RESIDUAL) out[row] += acc;
+            if constexpr (DUAL) out[row] = jl_swiglu_value(acc, acc_up);
+            else if (epilogue == JL_RESIDUAL) out[row] += acc;
             else out[row] = acc;
         }
     }
@@ -261,10 +271,10 @@ jl_gemv_direct(const uint8_t *__restrict__ w, const float *__restrict__ x, float
 
 // Rows of 4 NIT super-blocks: a lane meets the same activations in every row, so they are read
 // once into registers, and a row's 6 NIT loads per lane are all in flight before the first use.
-template <int TYPE, int NIT>
+template <int TYPE, int NIT, bool DUAL>
 __global__ void __launch_bounds__(256)
-jl_gemv_direct_held(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out, int rows,
-                    int epilogue) {
+jl_gemv_direct_held(const uint8_t *__restrict__ w, const uint8_t *__restrict__ w_up, const float *__restrict__ x,
+                    float *__restrict__ out, int rows, int epilogue) {
     constexpr int BB = Geometry<TYPE>::kBytes;
     const int lane = threadIdx.x & 63;
     const int waves = (gridDim.x * blockDim.x) >> 6;
@@ -273,16 +283,29 @@ jl_gemv_direct_held(const uint8_t *__restrict__ w, const float *__restrict__ x, 
 #pragma unroll
     for (int k = 0; k < NIT; k++) v[k] = load_x<TYPE>(x + ((lane >> 4) + 4 * k) * 256, j);
     for (int row = (blockIdx.x * blockDim.x + threadIdx.x) >> 6; row < rows; row += waves) {
-        const uint8_t *wr = w + (int64_t)row * (4 * NIT * BB) + (lane >> 4) * BB;
+        const int64_t at = (int64_t)row * (4 * NIT * BB) + (lane >> 4) * BB;
         Raw<TYPE> r[NIT];
 #pragma unroll
-        for (int k = 0; k < NIT; k++) r[k] = load_raw<TYPE>(wr + k * 4 * BB, j);
-        float acc = 0.f;
+        for (int k = 0; k < NIT; k++) r[k] = load_raw<TYPE>(w + at + k * 4 * BB, j);
+        float acc = 0.f, acc_up = 0.f;
+        if constexpr (DUAL) {
+            // the up row's loads go out before the gate row is multiplied
+            Raw<TYPE> ru[NIT];
 #pragma unroll
-        for (int k = 0; k < NIT; k++) acc += block_part<TYPE>(r[k], v[k], j);
+            for (int k = 0; k < NIT; k++) ru[k] = load_raw<TYPE>(w_up + at + k * 4 * BB, j);
+#pragma unroll
+            for (int k = 0; k < NIT; k++) acc += block_part<TYPE>(r[k], v[k], j);
+#pragma unroll
+            for (int k = 0; k < NIT; k++) acc_up += block_part<TYPE>(ru[k], v[k], j);
+            acc_up = jl_group_sum<JL_WAVE>(acc_up);
+        } else {
+#pragma unroll
+            for (int k = 0; k < NIT; k++) acc += block_part<TYPE>(r[k], v[k], j);
+        }
         acc = jl_group_sum<JL_WAVE>(acc);
         if (lane == 0) {
-            if (epilogue == JL_RESIDUAL) out[row] += acc;
+            if constexpr (DUAL) out[row] = jl_swiglu_value(acc, acc_up);
+            else if (epilogue == JL_RESIDUAL) out[row] += acc;
             else out[row] = acc;
         }
     }
@@ -359,38 +382,52 @@ jl_dequant_nibbles(const uint8_t *__restrict__ w, float *__restrict__ out, int64
     }
 }
 
-template <int TYPE>
-int launch_direct(jl_context *ctx, const jl_weight *w, const float *x, float *out, int epilogue) {
+template <int TYPE, bool DUAL>
+int launch_direct(jl_context *ctx, const jl_weight *w, const jl_weight *w_up, const float *x, float *out, int epilogue) {
     const int rows = (int)w->rows, n = (int)w->cols;
+    const uint8_t *up = DUAL ? w_up->blocks : nullptr;
     // enough waves to hide the loads' latency, rows dealt round robin
     int groups = (rows + 3) / 4;
     const int cap = ctx->compute_units * 8;
     if (groups > cap) groups = cap;
     const dim3 g(groups), b(256);
+    // (a gate/up pair holds twice the raw registers: rows of 8192 columns take the general kernel)
     switch (n) {
-        case 1024: hipLaunchKernelGGL((jl_gemv_direct_held<TYPE, 1>), g, b, 0, ctx->stream, w->blocks, x, out, rows, epilogue); break;
-        case 2048: hipLaunchKernelGGL((jl_gemv_direct_held<TYPE, 2>), g, b, 0, ctx->stream, w->blocks, x, out, rows, epilogue); break;
-        case 4096: hipLaunchKernelGGL((jl_gemv_direct_held<TYPE, 4>), g, b, 0, ctx->stream, w->blocks, x, out, rows, epilogue); break;
-        case 8192: hipLaunchKernelGGL((jl_gemv_direct_held<TYPE, 8>), g, b, 0, ctx->stream, w->blocks, x, out, rows, epilogue); break;
-        default: hipLaunchKernelGGL(jl_gemv_direct<TYPE>, g, b, 0, ctx->stream, w->blocks, x, out, rows, n, epilogue); break;
+        case 1024: hipLaunchKernelGGL((jl_gemv_direct_held<TYPE, 1, DUAL>), g, b, 0, ctx->stream, w->blocks, up, x, out, rows, epilogue); break;
+        case 2048: hipLaunchKernelGGL((jl_gemv_direct_held<TYPE, 2, DUAL>), g, b, 0, ctx->stream, w->blocks, up, x, out, rows, epilogue); break;
+        case 4096: hipLaunchKernelGGL((jl_gemv_direct_held<TYPE, 4, DUAL>), g, b, 0, ctx->stream, w->blocks, up, x, out, rows, epilogue); break;
+        case 8192:
+            if constexpr (!DUAL) {
+                hipLaunchKernelGGL((jl_gemv_direct_held<TYPE, 8, false>), g, b, 0, ctx->stream, w->blocks, up, x, out, rows, epilogue);
+                break;
+            }
+            [[fallthrough]];
+        default: hipLaunchKernelGGL((jl_gemv_direct<TYPE, DUAL>), g, b, 0, ctx->stream, w->blocks, up, x, out, rows, n, epilogue); break;
     }
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
 
+template <int TYPE>
+int launch_direct_type(jl_context *ctx, const jl_weight *w, const jl_weight *w_up, const float *x, float *out, int epilogue) {
+    return w_up ? launch_direct<TYPE, true>(ctx, w, w_up, x, out, epilogue)
+                : launch_direct<TYPE, false>(ctx, w, nullptr, x, out, epilogue);
+}
+
 }  // namespace
 
-int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const float *x, float *out, int epilogue) {
+int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const jl_weight *w_up, const float *x, float *out,
+                          int epilogue) {
     if (w->cols % 256 != 0 || ((uintptr_t)x & 15) != 0) {
         return jl_fail(JL_ERR_UNSUPPORTED, "no %s projection kernel for a row length of %lld or an unaligned vector",
                        jl_type_name(w->type), (long long)w->cols);
     }
     switch (w->type) {
-        case JL_Q6_K: return launch_direct<JL_Q6_K>(ctx, w, x, out, epilogue);
-        case JL_Q5_K: return launch_direct<JL_Q5_K>(ctx, w, x, out, epilogue);
-        case JL_Q4_1: return launch_direct<JL_Q4_1>(ctx, w, x, out, epilogue);
-        case JL_Q5_0: return launch_direct<JL_Q5_0>(ctx, w, x, out, epilogue);
-        case JL_IQ4_XS: return launch_direct<JL_IQ4_XS>(ctx, w, x, out, epilogue);
+        case JL_Q6_K: return launch_direct_type<JL_Q6_K>(ctx, w, w_up, x, out, epilogue);
+        case JL_Q5_K: return launch_direct_type<JL_Q5_K>(ctx, w, w_up, x, out, epilogue);
+        case JL_Q4_1: return launch_direct_type<JL_Q4_1>(ctx, w, w_up, x, out, epilogue);
+        case JL_Q5_0: return launch_direct_type<JL_Q5_0>(ctx, w, w_up, x, out, epilogue);
+        case JL_IQ4_XS: return launch_direct_type<JL_IQ4_XS>(ctx, w, w_up, x, out, epilogue);
         default: return jl_fail(JL_ERR_UNSUPPORTED, "no projection kernel for a ggml type %d weight", w->type);
     }
 }

@@ -108,7 +108,9 @@ int jl_launch_quantize_q8(jl_context *ctx, const float *x, const float *rms_w, c
                           int64_t n, int8_t *quants, float *scales, int32_t *sums);
 int jl_launch_rms_apply_f16(jl_context *ctx, float *X, const float *delta, const float *w, float eps, int64_t rows,
                             int64_t n, float *scales, _Float16 *out);
-int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const float *x, float *out, int epilogue);
+// `w_up` set: out = SiLU(w . x) * (w_up . x) (the fused gate/up), `epilogue` ignored.
+int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const jl_weight *w_up, const float *x, float *out,
+                          int epilogue);
 int jl_launch_dequant_direct(jl_context *ctx, const jl_weight *w, float *out);
 int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale);
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);

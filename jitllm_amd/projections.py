@@ -17,7 +17,10 @@ from . import _lib as L
 from .ggml import GGMLType
 from .runtime import Context, DeviceBuffer, FloatArray, HalfFloatArray, ResidentCopies, TornadoTensor
 
-FUSED_GATE_UP_TYPES = (GGMLType.Q8_0, GGMLType.Q4_0, GGMLType.Q4_K)
+# QuantizedProjections.fusedGateUp (:386-393): Q8_0, Q4_0, Q4_K and Q5_K;
+# QuantizedBatchProjections.fusedGateUp (:315-321), the tiled answer: Q8_0, Q4_0 and Q4_K
+FUSED_GATE_UP_TYPES = (GGMLType.Q8_0, GGMLType.Q4_0, GGMLType.Q4_K, GGMLType.Q5_K)
+BATCH_FUSED_GATE_UP_TYPES = (GGMLType.Q8_0, GGMLType.Q4_0, GGMLType.Q4_K)
 
 
 @dataclass
@@ -282,7 +285,7 @@ class QuantizedBatchProjections:
 
     def fusedGateUp(self, w1: TornadoTensor, w3: TornadoTensor) -> bool:
         """QuantizedBatchProjections.java:315-321 (the tiled, non-SIMD-group answer)."""
-        return w1.data_type() == w3.data_type() and w1.data_type() in FUSED_GATE_UP_TYPES
+        return w1.data_type() == w3.data_type() and w1.data_type() in BATCH_FUSED_GATE_UP_TYPES
 
     def gateUp(self, x: FloatArray, hb: FloatArray, w1: TornadoTensor, w3: TornadoTensor, dim: int,
                hidDim: int, activeRows: int | None = None) -> None:

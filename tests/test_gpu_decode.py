@@ -240,14 +240,41 @@ def test_k_quants_have_no_fused_single_token_kernels(ctx, t):
     proj = QuantizedProjections(ctx, TornadoWorkspace(wrapXb=x, wrapHb=out, wrapHb2=ctx.float_array(d)))
     with pytest.raises(UnsupportedProjection, match=KQ_NAMES[t]):
         proj.fusedQKV(x, out, out, out, w, w, w)
-    assert not proj.fusedGateUp(w, w)
+    assert proj.fusedGateUp(w, w) == (t == O.Q5_K)     # QuantizedProjections.java:386-393
     with pytest.raises(UnsupportedProjection, match=KQ_NAMES[t]):
         proj.rmsMatvec(x, x, None, out, w, n, d, eps=1e-5)
-    # ... and the unfused gate/up sequence works: two projections and an element-wise SwiGLU
+    # ... and gate/up works either way: one launch for Q5_K, else two projections and an
+    # element-wise SwiGLU
     proj.gateUp(w, w, n, d)
     ctx.sync()
     ref = O.matmul(t, synthetic.weight(t, d, n, seed=731), synthetic.activations(n, seed=732), d, n)
     assert np.allclose(out.get(), O.swiglu(ref, ref), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("t", KQ)
+@pytest.mark.parametrize("d,n", [(12288, 4096), (2048, 2048), (37, 512), (300, 8192), (64, 1280)])
+def test_k_quant_fused_gate_up(ctx, t, d, n):
+    """hb = SiLU(w1 . x) * (w3 . x) in one launch for the remaining types (the reference fuses it for
+    Q5_K, QuantizedProjections.java:386-393), held against the host's matVec, matVec, swiGLU."""
+    import ctypes as C
+    from jitllm_amd import _lib as L, synthetic
+    say("gate_up", KQ_NAMES[t], d, n)
+    r1 = synthetic.weight(t, d, n, seed=741)
+    r3 = synthetic.weight(t, d, n, seed=742)
+    x = synthetic.activations(n, seed=743)
+    g = O.matmul(t, r1, x, d, n)
+    u = O.matmul(t, r3, x, d, n)
+    ref = O.swiglu(g, u)
+    hb = ctx.float_array(d, fill=POISON)
+    w1, w3 = upload(ctx, t, r1, d, n), upload(ctx, t, r3, d, n)
+    L.check(L.load().jl_gemv_gate_up(ctx.handle, w1.handle, w3.handle, ctx.from_numpy(x).ptr, hb.ptr))
+    ctx.sync()
+    got = hb.get()
+    mg, mu = magnitude(t, r1, x, d, n), magnitude(t, r3, x, d, n)
+    bound = 2e-5 * (mg * np.abs(u) + mu * np.abs(g) * 1.2 + 1e-6)
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + 1e-6)
+    w1.free()
+    w3.free()
 
 
 # ---- RMS normalisation folded into the projections, argmax -----------------------------------
