@@ -177,3 +177,32 @@ def test_int8_refusals(ctx):
     arr6 = (C.c_void_p * 1)(w6.handle)
     st = lib.jl_gemm(ctx.handle, arr6, 1, x.ptr, o.ptr, 1, 1, 64, 0, L.JL_STORE, L.JL_MATH_INT8, ws.ptr, ws.nbytes)
     assert st == L.JL_ERR_UNSUPPORTED and b"Q6_K" in lib.jl_last_error()
+
+
+def test_int8_row_stride_and_column_offset(ctx):
+    """Two calls fill one packed row side by side (ldo, col_offset: gemmInt8Q8_0's contract,
+    Int8GemmKernels.java:651-676); what lies between and beside them is left alone."""
+    import ctypes as C
+    from jitllm_amd import _lib as L, synthetic
+    say("int8 ldo / col_offset")
+    lib = L.load()
+    t, n, T, da, db, ldo = O.Q8_0, 192, 37, 70, 40, 128
+    ra, rb = synthetic.weight(t, da, n, seed=2140), synthetic.weight(t, db, n, seed=2141)
+    wa, wb = ctx.load_weight(t, ra, da, n), ctx.load_weight(t, rb, db, n)
+    X = synthetic.activations((T, n), seed=2142)
+    out = ctx.float_array(T * ldo, fill=UNTOUCHED)
+    nbytes = lib.jl_gemm_workspace_bytes(T, n, da, L.JL_MATH_INT8)
+    ws = ctx.raw_buffer(nbytes)
+    xd = ctx.from_numpy(X)
+    for w, off in ((wa, 4), (wb, 80)):
+        arr = (C.c_void_p * 1)(w.handle)
+        L.check(lib.jl_gemm(ctx.handle, arr, 1, xd.ptr, out.ptr, T, T, ldo, off, L.JL_STORE, L.JL_MATH_INT8,
+                            ws.ptr, ws.nbytes))
+    ctx.sync()
+    got = out.get().reshape(T, ldo)
+    assert np.array_equal(bits(got[:, 4:4 + da]), bits(int8_reference(t, ra, X, da, n)))
+    assert np.array_equal(bits(got[:, 80:80 + db]), bits(int8_reference(t, rb, X, db, n)))
+    mask = np.ones(ldo, dtype=bool)
+    mask[4:4 + da] = False
+    mask[80:80 + db] = False
+    assert np.all(got[:, mask] == UNTOUCHED)
