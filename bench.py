@@ -549,6 +549,12 @@ def bench_batched_q4k(ctx, hip, B, steps, warmup, cpu):
     out = {"B": B, "ms_per_layer": round(ms, 4), "ms_stats": spread_stats(ms_list), "layers_swept": copies,
            "GB_s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
            "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "bytes": wbytes + io, "check_rel_err": errs}
+    # which roof applies at this batch: the call's flop per byte against the chip's ridge
+    intensity = flops / (wbytes + io)
+    ridge = F16_MFMA_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+    out["flop_per_byte"] = round(intensity, 1)
+    out["bound"] = "hbm" if intensity < ridge else "mfma"
+    out["frac_f16_mfma_peak"] = round(out["tflops"] / F16_MFMA_PEAK_TFLOPS, 4)
     if cpu and B == 8:
         rows = sample_rows(ffn, 480, 75)
         out["cpu_baseline"] = cpu_baseline_rows(t, host["w1"], dim, rows, Xh, ffn, 2.0, "gate projection at B=8")

@@ -737,6 +737,13 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
         }
     };
 
+    // Rows of at most 64 slices lie inside one wave: their lane sums are folded in registers and the
+    // row's first lane applies the epilogue itself -- no partial sums in LDS, no finishing pass one
+    // tile later, no barrier behind the last tile.  For gate/up the rows are dealt gate 0, up 0,
+    // gate 1, up 1, ... so that both halves of an output sit in the same wave (rows of 64 slices
+    // fill a wave each, so gate/up keeps the LDS hand-over there).
+    const bool in_wave = p.Sp <= (DUAL ? 32 : 64);
+    const int r_lds = (DUAL && in_wave) ? (r & 1) * half_rows + (r >> 1) : r;   // tile row this thread reads
     for (int it = 0; it < mine; it++) {
         const int tile = first + it * gridDim.x;
         // with two stages nothing was issued after tile `it`: its loads are the youngest
@@ -749,14 +756,42 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
             issue(first + issued * gridDim.x, issued % kStages);
             issued++;
         }
-        if (it > 0) finish(tile - gridDim.x, (it - 1) & 1);
+        if (!in_wave && it > 0) finish(tile - gridDim.x, (it - 1) & 1);
 
         float v = 0.f;
         if (active) {
-            if constexpr (PACKED) v = slice_dot_lds_packed<TYPE>(ring0 + (it % kStages) * stage_bytes, r, s, p.row_bytes, px);
-            else v = slice_dot_lds<TYPE>(ring0 + (it % kStages) * stage_bytes, r, s, p.row_bytes, x, sx);
+            if constexpr (PACKED) v = slice_dot_lds_packed<TYPE>(ring0 + (it % kStages) * stage_bytes, r_lds, s, p.row_bytes, px);
+            else v = slice_dot_lds<TYPE>(ring0 + (it % kStages) * stage_bytes, r_lds, s, p.row_bytes, x, sx);
         }
         if (it == mine - 1) GSTAMP(6);
+        if (in_wave) {
+            v = group_sum(v, p.Sp);
+            float up = 0.f;
+            if constexpr (DUAL) up = __shfl(v, lane + p.Sp, JL_WAVE);   // the up row sits Sp lanes on
+            const int j = DUAL ? r >> 1 : r;   // output row of the tile
+            if (s == 0 && r < p.R && (!DUAL || (r & 1) == 0)) {
+                int local = tile, seg_rows = rows0;
+                float *out = out0;
+                if (nseg > 1) {
+                    const int seg = segment_of(tile);
+                    local = tile - (int)uniform_value((uint32_t)p.seg_tile_begin[seg]);
+                    seg_rows = (int)uniform_value((uint32_t)p.seg_rows[seg]);
+                    out = (float *)uniform_value((uintptr_t)p.out[seg]);
+                }
+                const int row = local * half_rows + j;
+                if (row < seg_rows) {
+                    float *o = out + row;
+                    if constexpr (DUAL) {
+                        *o = jl_swiglu_value(v, up);
+                    } else {
+                        // no read-modify-write through a load: a load's wait would drain the prefetch ring
+                        if (p.epilogue == JL_RESIDUAL) unsafeAtomicAdd(o, v);
+                        else *o = v;
+                    }
+                }
+            }
+            continue;
+        }
         if (p.Sp >= 2) v += quad_xor1(v);
         if (p.Sp >= 4) v += quad_xor2(v);
         if (r < p.R && (p.Sp < 4 ? s == 0 : (s & 3) == 0)) {
@@ -764,7 +799,7 @@ __global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
             lds_write_b32(lds0 + (it & 1) * kParity + slot * 4, __float_as_uint(v));
         }
     }
-    if (mine > 0) {
+    if (mine > 0 && !in_wave) {
         __builtin_amdgcn_s_barrier();
         finish(first + (mine - 1) * gridDim.x, (mine - 1) & 1);
     }
