@@ -29,72 +29,11 @@ constexpr int kMaxWeights = 8;
 
 // ---- activations: fp32 -> fp16 with a power-of-two row scale --------------------------------
 
-// One workgroup per row: scale = the power of two that brings the row's largest magnitude into
-// [2^11, 2^12); a16 = half(x / scale) (the division is exact).  Rows past `rows` are zero-filled.
-// A row of up to 8192 columns is read once and kept in registers between the two passes (largest
-// magnitude, conversion); longer rows are read twice.
+// One workgroup per row; see jl_row_to_f16.
 __global__ void __launch_bounds__(256)
 jl_rows_to_f16(const float *__restrict__ X, _Float16 *__restrict__ A, float *__restrict__ row_scale,
                int rows, int k) {
-    __shared__ float wave_max[4];
-    constexpr int kHeld = 8;   // float4 per thread held in registers: 256 x 8 x 4 = 8192 columns
-    const int row = blockIdx.x;
-    const int tid = threadIdx.x;
-    _Float16 *a = A + (int64_t)row * k;
-    if (row >= rows) {
-        for (int i = tid * 4; i < k; i += 1024) *(half4 *)(a + i) = half4{0, 0, 0, 0};
-        if (tid == 0) row_scale[row] = 1.f;
-        return;
-    }
-    const float *x = X + (int64_t)row * k;
-    const bool held = k <= kHeld * 1024;
-    float4 v[kHeld];
-    float amax = 0.f;
-    if (held) {
-#pragma unroll
-        for (int j = 0; j < kHeld; j++) {
-            const int i = tid * 4 + j * 1024;
-            v[j] = i < k ? *(const float4 *)(x + i) : float4{0.f, 0.f, 0.f, 0.f};
-            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[j].x), fabsf(v[j].y)), fmaxf(fabsf(v[j].z), fabsf(v[j].w))));
-        }
-    } else {
-        for (int i = tid * 4; i < k; i += 1024) {
-            float4 w = *(const float4 *)(x + i);
-            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(w.x), fabsf(w.y)), fmaxf(fabsf(w.z), fabsf(w.w))));
-        }
-    }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, JL_WAVE));
-    if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
-    __syncthreads();
-    amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
-    // Every row is brought to [2^11, 2^12) at its largest magnitude: huge rows stay finite in
-    // fp16, tiny rows keep their bits out of fp16's subnormal range, and the power of two is
-    // undone exactly in the epilogue.
-    float scale = 1.f, inv = 1.f;
-    if (amax > 0.f && amax < INFINITY) {
-        int e;
-        frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
-        e = e < -100 ? -100 : e;
-        scale = ldexpf(1.f, e - 12);
-        inv = ldexpf(1.f, 12 - e);
-    }
-    if (held) {
-#pragma unroll
-        for (int j = 0; j < kHeld; j++) {
-            const int i = tid * 4 + j * 1024;
-            if (i < k)
-                *(half4 *)(a + i) = half4{(_Float16)(v[j].x * inv), (_Float16)(v[j].y * inv),
-                                          (_Float16)(v[j].z * inv), (_Float16)(v[j].w * inv)};
-        }
-    } else {
-        for (int i = tid * 4; i < k; i += 1024) {
-            float4 w = *(const float4 *)(x + i);
-            *(half4 *)(a + i) = half4{(_Float16)(w.x * inv), (_Float16)(w.y * inv), (_Float16)(w.z * inv),
-                                      (_Float16)(w.w * inv)};
-        }
-    }
-    if (tid == 0) row_scale[row] = scale;
+    jl_row_to_f16(X, A, row_scale, rows, k, blockIdx.x);
 }
 
 // Activations that arrive as fp16 but in a buffer the kernels cannot read whole row tiles of: the
@@ -979,9 +918,16 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
         return jl_fail(JL_ERR_WORKSPACE, "jl_gemm: a %s weight needs room for its fp16 copy (%zu bytes) in the workspace",
                        jl_type_name(type), copy_bytes);
     }
+    // what a kept copy looks like: gate / up interleaved by half tiles of this BN, or plain
+    const int32_t layout = epilogue == JL_SWIGLU ? bn : 1;
+    const bool decode = dense && (!kept || *resident->state != layout);
+    // a call that decodes its weights converts its fp32 activations in that same launch
+    const bool ride_along = decode && !X16;
     if (!X16) {
-        hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded_rows), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
-        JL_HIP(hipGetLastError());
+        if (!ride_along) {
+            hipLaunchKernelGGL(jl_rows_to_f16, dim3(padded_rows), dim3(256), 0, ctx->stream, X, A, row_scale, rows, k);
+            JL_HIP(hipGetLastError());
+        }
     } else {
         // fp16 activations are multiplied as they are (no row scales).  The kernels bring in whole
         // row tiles: the caller's buffer serves directly when its `batch` rows cover the last
@@ -995,12 +941,10 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
         }
     }
     if (dense) {
-        // what a kept copy looks like: gate / up interleaved by half tiles of this BN, or plain
-        const int32_t layout = epilogue == JL_SWIGLU ? bn : 1;
-        const bool decode = !kept || *resident->state != layout;
         const int st = jl_launch_gemm_dense(ctx, weights, count, A, row_scale, C, rows, ldo, col_offset, epilogue,
                                             kept ? (_Float16 *)resident->copy : (_Float16 *)planes, decode, bn,
-                                            dsplits, (float *)((uint8_t *)planes + in_workspace), c_f16);
+                                            dsplits, (float *)((uint8_t *)planes + in_workspace), c_f16,
+                                            ride_along ? X : nullptr, ride_along ? row_scale : nullptr);
         if (st == JL_OK && kept) *resident->state = layout;
         return st;
     }

@@ -47,6 +47,13 @@ struct DecodeParams {
     int n_total;           // SWIGLU: rows of one weight
     int half;              // SWIGLU: BN / 2 of the GEMM that will read the copy, else 0; virtual row
                            // t * BN + sel * half + i is row t * half + i of weight sel (0 gate, 1 up)
+    // the call's activations, when they ride along (else virtual_rows = the grid's width):
+    // workgroups blockIdx.x >= virtual_rows convert activation row blockIdx.x - virtual_rows
+    int virtual_rows;
+    const float *X;        // [rows x k] fp32
+    _Float16 *A;           // [padded rows x k]
+    float *row_scale;
+    int rows;
 };
 
 // eight bytes (two dwords in 0..255 offset form) -> (byte - bias) * d, eight fp16 as one 16-byte store
@@ -76,6 +83,10 @@ struct __attribute__((packed, aligned(2))) Quants8 { uint32_t lo, hi; };
 
 template <int TYPE>
 __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
+    if ((int)blockIdx.x >= p.virtual_rows) {
+        if (blockIdx.y == 0) jl_row_to_f16(p.X, p.A, p.row_scale, p.rows, p.k, blockIdx.x - p.virtual_rows);
+        return;
+    }
     const int v = blockIdx.x;
     const int c = blockIdx.y * 256 + threadIdx.x;   // chunk of 8 columns
     if (c >= p.k / 8) return;
@@ -528,8 +539,9 @@ int launch_dense(jl_context *ctx, const DenseParams &p) {
 }
 
 template <int TYPE>
-int launch_decode(jl_context *ctx, const DecodeParams &d, int virtual_rows) {
-    hipLaunchKernelGGL(jl_decode_to_f16<TYPE>, dim3((unsigned)virtual_rows, (unsigned)((d.k / 8 + 255) / 256)),
+int launch_decode(jl_context *ctx, const DecodeParams &d, int activation_rows) {
+    hipLaunchKernelGGL(jl_decode_to_f16<TYPE>,
+                       dim3((unsigned)(d.virtual_rows + activation_rows), (unsigned)((d.k / 8 + 255) / 256)),
                        dim3(256), 0, ctx->stream, d);
     JL_HIP(hipGetLastError());
     return JL_OK;
@@ -575,7 +587,7 @@ size_t jl_dense_copy_bytes(int k, int out_cols_virtual) {
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
                          int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes,
-                         bool c_f16) {
+                         bool c_f16, const float *X32, float *row_scale_out) {
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     const bool swiglu = epilogue == JL_SWIGLU;
@@ -598,18 +610,29 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
     d.half = swiglu ? bn / 2 : 0;
     // plain layout: always whole 256-row tiles, so the copy does not depend on the column tile
     // (a copy that is kept across calls stays valid when the row count, hence BN, changes)
-    const int decoded_rows = swiglu ? ntiles * bn : (n_total + 255) / 256 * 256;
+    d.virtual_rows = swiglu ? ntiles * bn : (n_total + 255) / 256 * 256;
+    // fp32 activations of a call that decodes are converted by the same launch (X32 is null when
+    // the caller has converted them, or they came as fp16)
+    int xr = 0;
+    if (X32) {
+        if (!decode) return jl_fail(JL_ERR_INVALID, "jl_gemm: activations handed to a decode that is not due");
+        d.X = X32;
+        d.A = const_cast<_Float16 *>(A);
+        d.row_scale = row_scale_out;
+        d.rows = rows;
+        xr = (rows + DBM - 1) / DBM * DBM;
+    }
     int dst = JL_OK;
     if (decode) {
         switch (type) {
-            case JL_Q8_0: dst = launch_decode<JL_Q8_0>(ctx, d, decoded_rows); break;
-            case JL_Q4_0: dst = launch_decode<JL_Q4_0>(ctx, d, decoded_rows); break;
-            case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, d, decoded_rows); break;
-            case JL_Q5_K: dst = launch_decode<JL_Q5_K>(ctx, d, decoded_rows); break;
-            case JL_Q6_K: dst = launch_decode<JL_Q6_K>(ctx, d, decoded_rows); break;
-            case JL_Q4_1: dst = launch_decode<JL_Q4_1>(ctx, d, decoded_rows); break;
-            case JL_Q5_0: dst = launch_decode<JL_Q5_0>(ctx, d, decoded_rows); break;
-            case JL_IQ4_XS: dst = launch_decode<JL_IQ4_XS>(ctx, d, decoded_rows); break;
+            case JL_Q8_0: dst = launch_decode<JL_Q8_0>(ctx, d, xr); break;
+            case JL_Q4_0: dst = launch_decode<JL_Q4_0>(ctx, d, xr); break;
+            case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, d, xr); break;
+            case JL_Q5_K: dst = launch_decode<JL_Q5_K>(ctx, d, xr); break;
+            case JL_Q6_K: dst = launch_decode<JL_Q6_K>(ctx, d, xr); break;
+            case JL_Q4_1: dst = launch_decode<JL_Q4_1>(ctx, d, xr); break;
+            case JL_Q5_0: dst = launch_decode<JL_Q5_0>(ctx, d, xr); break;
+            case JL_IQ4_XS: dst = launch_decode<JL_IQ4_XS>(ctx, d, xr); break;
             default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
         }
     }

@@ -151,7 +151,7 @@ size_t jl_dense_plane_bytes(int rows, int out_cols_virtual, int splits);
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
                          int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes,
-                         bool c_f16 = false);
+                         bool c_f16 = false, const float *X32 = nullptr, float *row_scale_out = nullptr);
 // Adds split-K planes [splits][rows padded][ntiles * 128] in split order and applies the epilogue.
 int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row_scale, float *C, int rows,
                           int n_total, int ntiles, int64_t plane, int splits, int64_t ldo, int64_t col_offset,
