@@ -405,6 +405,7 @@ constexpr int kPartialBytes = 2048;  // 2 parities x 256 floats
 // a deeper ring at the lower occupancy its LDS footprint forces is slower (and no faster where it
 // costs no occupancy: the 9 KB tiles of the 4-bit types at 3 and 4 stages).
 constexpr int kStages = 2;
+constexpr int kWideThreads = 1024;   // workgroup of the plain kernel for rows of more than 128 slices
 
 // v + (the value two quad neighbours hold): DPP quad permutes, VALU speed, no LDS round trip
 __device__ __forceinline__ float quad_xor1(float v) {
@@ -437,8 +438,8 @@ __device__ uint64_t *jl_gemv_stamp_buf = nullptr;
 #define GSTAMP(k) do { } while (0)
 #endif
 
-template <int TYPE, bool DUAL, bool RMS, bool PACKED = false>
-__global__ void __launch_bounds__(256) jl_gemv_tiles(GemvParams p) {
+template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256>
+__global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     static_assert(!(RMS && PACKED), "the packed activation is normalised before it is quantised");
 #ifdef JL_GEMV_STAMPS
     uint64_t stamp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -875,6 +876,15 @@ jl_gemv_generic(const uint8_t *__restrict__ w, const uint8_t *__restrict__ w_up,
 
 // ---- host side ------------------------------------------------------------------------------
 
+// LDS of a workgroup of `threads`: partial sums, the tile ring, and the staged activation vector
+// where it is larger than a ring stage.
+int tile_lds_bytes(int threads, int slice, int S) {
+    const int stage_bytes = threads * slice;
+    const int x_bytes = (S * 17 + threads - 1) / threads * threads * 16;  // 17 slots per slice
+    const int x_extra = x_bytes <= stage_bytes ? 0 : x_bytes;
+    return kPartialBytes + kStages * stage_bytes + x_extra;
+}
+
 int next_pow2(int v) {
     int p = 1;
     while (p < v) p <<= 1;
@@ -908,9 +918,9 @@ int blocks_per_cu(const void *fn, int device, int threads, int lds) {
     return nb;
 }
 
-template <int TYPE, bool DUAL, bool RMS, bool PACKED = false>
+template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256>
 int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) {
-    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED>;
+    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED, THREADS>;
     int per_cu = blocks_per_cu((const void *)fn, ctx->device, threads, lds);
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
@@ -923,8 +933,11 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
 template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds) {
     if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
-    return p.rms_w ? launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds)
-                   : launch_tiles_of<TYPE, DUAL, false>(ctx, p, threads, lds);
+    if (p.rms_w) return launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds);
+    if constexpr (!DUAL) {
+        if (threads == kWideThreads) return launch_tiles_of<TYPE, false, false, false, kWideThreads>(ctx, p, threads, lds);
+    }
+    return launch_tiles_of<TYPE, DUAL, false>(ctx, p, threads, lds);
 }
 
 template <int TYPE>
@@ -970,7 +983,13 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     int S = n / 64, Sp = 0, R = 0, half_rows = 0;
     if (fast) {
         Sp = next_pow2(S);
-        R = 256 / Sp;
+        // Rows of more than 128 slices (8192 columns): a workgroup of 256 threads would hold one
+        // row per tile and stage the whole activation vector -- more bytes than its tiles -- for
+        // it, at one workgroup per compute unit for the LDS that takes.  Sixteen waves share the
+        // staged vector instead (plain and residual projections; the other variants keep 256).
+        // (when its LDS fits: Q8_0 rows of more than 15 360 columns do not)
+        const bool wide = Sp == 256 && !dual && !rms && !xq && tile_lds_bytes(kWideThreads, slice, S) <= 160 * 1024;
+        R = (wide ? kWideThreads : 256) / Sp;
         half_rows = dual ? R / 2 : R;
         if (half_rows < 1) fast = false;
         else if (((int64_t)half_rows * row_bytes) % 16 != 0) fast = false;
@@ -1043,10 +1062,7 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     }
 
     const int threads = (R * Sp + 63) / 64 * 64;
-    const int stage_bytes = threads * slice;
-    const int x_bytes = (S * 17 + threads - 1) / threads * threads * 16;  // 17 slots per slice
-    const int x_extra = x_bytes <= stage_bytes ? 0 : x_bytes;
-    const int lds = kPartialBytes + kStages * stage_bytes + x_extra;
+    const int lds = tile_lds_bytes(threads, slice, S);
 
     switch (type) {
         case JL_Q8_0:

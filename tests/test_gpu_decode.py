@@ -116,6 +116,10 @@ SHAPES = [
     (O.Q8_0, 77, 96), (O.Q4_0, 5, 32), (O.Q4_K, 9, 256), (O.Q8_0, 3, 32768),  # catch-all kernel
     (O.Q8_0, 5, 64), (O.Q8_0, 3, 128), (O.Q4_0, 7, 64), (O.Q4_0, 3, 192),  # bytes that end off a 16-byte boundary
     (O.Q8_0, 8, 64), (O.Q4_0, 4, 64),                                       # ... and the same widths on one
+    # rows of more than 8192 columns (workgroups of 1024 threads, four rows to a tile): whole and
+    # ragged tiles, a row length that leaves most of a row's lanes idle, the longest row each type takes
+    (O.Q8_0, 1026, 14336), (O.Q8_0, 37, 8256), (O.Q8_0, 21, 15360), (O.Q8_0, 64, 16384),
+    (O.Q4_0, 131, 16384), (O.Q4_K, 35, 11008), (O.Q4_K, 2, 16384),
 ]
 
 
@@ -137,6 +141,24 @@ def test_gemv_matches_oracle(ctx, t, d, n):
     err = rel_err(got, ref, magnitude(t, raw, x, d, n))
     assert err < 1e-3, err
     assert err < 2e-5, err  # fp32 arithmetic throughout: only the summation order differs
+
+
+@pytest.mark.parametrize("t,d,n", [(O.Q8_0, 130, 14336), (O.Q4_0, 1022, 14336), (O.Q4_K, 67, 12288)])
+def test_residual_matvec_on_long_rows(ctx, t, d, n):
+    """x += w . hb at the down projection's row lengths (the 1024-thread workgroups), ragged last tile."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("residual, long rows", NAMES[t], d, n)
+    raw = synthetic.weight(t, d, n, seed=1500 + d)
+    x = synthetic.activations(n, seed=1600 + n)
+    ref = O.matmul(t, raw, x, d, n, O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256)
+    mag = magnitude(t, raw, x, d, n)
+    w = upload(ctx, t, raw, d, n)
+    base = synthetic.activations(d, seed=1700)
+    acc = ctx.from_numpy(base)
+    QuantizedProjections(ctx, TornadoWorkspace(wrapX=acc)).residualMatvec(ctx.from_numpy(x), w, n, d)
+    ctx.sync()
+    assert rel_err(acc.get(), ref.astype(np.float64) + base, mag + np.abs(base) * 6e-8) < 2e-5
 
 
 @pytest.mark.parametrize("t,dq,dkv,n", [(O.Q8_0, 2048, 512, 2048), (O.Q4_0, 4096, 1024, 4096),
