@@ -89,38 +89,67 @@ __device__ __forceinline__ float slice_dot_q8_0(const uint32_t (&w)[17], const f
     return fmaf(a0 + a1, dA, (b0 + b1) * dB);
 }
 
+// The 4-bit kernels multiply without converting: a nibble left alone in the low ten bits of a
+// 16-bit half *is* a binary16 number -- the subnormal q * 2^-24 (q * 2^-20 for a high nibble, which
+// sits four bits up) -- and v_fma_mix_f32 takes a binary16 operand from either half of a register,
+// widens it exactly and fuses product and sum in fp32.  So a dword of eight nibbles costs five
+// mask / shift operations and eight multiply-adds, where byte -> float conversions took sixteen
+// more; the powers of two are taken out again, exactly, with the block scale.
+struct NibblePairs {
+    uint32_t lo02, hi02, lo13, hi13;   // low / high nibbles of bytes 0 and 2, of bytes 1 and 3
+};
+__device__ __forceinline__ NibblePairs nibble_pairs(uint32_t v) {
+    const uint32_t t = v >> 8;
+    return NibblePairs{v & 0x000F000Fu, v & 0x00F000F0u, t & 0x000F000Fu, t & 0x00F000F0u};
+}
+// acc += (binary16 in the low / high half of w) * x
+__device__ __forceinline__ void mix_low(float &acc, uint32_t w, float x) {
+    asm("v_fma_mix_f32 %0, %1, %2, %0 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "+v"(acc) : "v"(w), "v"(x));
+}
+__device__ __forceinline__ void mix_high(float &acc, uint32_t w, float x) {
+    asm("v_fma_mix_f32 %0, %1, %2, %0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(acc) : "v"(w), "v"(x));
+}
+// byte b (0..3) of the dword the pairs came from: acc_lo += low nibble * 2^-24 * x_lo,
+// acc_hi += high nibble * 2^-20 * x_hi
+__device__ __forceinline__ void mix_byte(const NibblePairs &n, int b, float x_lo, float x_hi, float &acc_lo,
+                                         float &acc_hi) {
+    const uint32_t lo = (b & 1) ? n.lo13 : n.lo02, hi = (b & 1) ? n.hi13 : n.hi02;
+    if (b & 2) {
+        mix_high(acc_lo, lo, x_lo);
+        mix_high(acc_hi, hi, x_hi);
+    } else {
+        mix_low(acc_lo, lo, x_lo);
+        mix_low(acc_hi, hi, x_hi);
+    }
+}
+constexpr float kTwo24 = 16777216.f, kTwoM24 = 1.f / 16777216.f;
+
 // Dot of one Q4_0 block pair (36 bytes) with 64 activations; sx[0], sx[1] are the sums of the
 // activations facing block A and block B, so that sum((q - 8) x) = sum(q x) - 8 sum(x).
 //   bytes 0..1 scale A | 2..17 nibbles A | 18..19 scale B | 20..35 nibbles B
 // element i < 16 of a block is the low nibble of its byte i, element 16 + i the high nibble.
 __device__ __forceinline__ float slice_dot_q4_0(const uint32_t (&dw)[9], const float (&x)[64],
                                                 const float (&sx)[2]) {
-    uint32_t lo[9], hi[9];
-    uint32_t w0 = dw[0], w4 = dw[4];
+    NibblePairs n[9];
 #pragma unroll
-    for (int i = 0; i < 9; i++) {
-        uint32_t v = dw[i];
-        lo[i] = jl_opaque(v & 0x0F0F0F0Fu);
-        hi[i] = jl_opaque((v >> 4) & 0x0F0F0F0Fu);
-    }
-    float dA = jl_half_bits_to_float(w0);
-    float dB = jl_half_bits_to_float(w4 >> 16);
+    for (int i = 0; i < 9; i++) n[i] = nibble_pairs(dw[i]);
+    const float dA = jl_half_bits_to_float(dw[0]);
+    const float dB = jl_half_bits_to_float(dw[4] >> 16);
+    // a0, b0: sum(q x) * 2^-24 over the low nibbles; a1, b1: * 2^-20 over the high nibbles
     float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-        int o = 2 + i;  // byte i of block A
-        a0 = fmaf(ubyte(lo[o >> 2], o & 3), x[i], a0);
-        a1 = fmaf(ubyte(hi[o >> 2], o & 3), x[16 + i], a1);
+        const int o = 2 + i;  // byte i of block A
+        mix_byte(n[o >> 2], o & 3, x[i], x[16 + i], a0, a1);
     }
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-        int o = 20 + i;  // byte i of block B
-        b0 = fmaf(ubyte(lo[o >> 2], o & 3), x[32 + i], b0);
-        b1 = fmaf(ubyte(hi[o >> 2], o & 3), x[48 + i], b1);
+        const int o = 20 + i;  // byte i of block B
+        mix_byte(n[o >> 2], o & 3, x[32 + i], x[48 + i], b0, b1);
     }
-    float da = fmaf(-8.f, sx[0], a0 + a1);
-    float db = fmaf(-8.f, sx[1], b0 + b1);
-    return fmaf(da, dA, db * dB);
+    const float da = fmaf(-8.f * kTwoM24, sx[0], fmaf(a1, 0.0625f, a0));
+    const float db = fmaf(-8.f * kTwoM24, sx[1], fmaf(b1, 0.0625f, b0));
+    return fmaf(da, dA * kTwo24, db * (dB * kTwo24));
 }
 
 // Dot of one quarter of a Q4_K super-block with 64 activations.  `hdr` is the super-block's first
@@ -130,28 +159,24 @@ __device__ __forceinline__ float slice_dot_q4_0(const uint32_t (&dw)[9], const f
 __device__ __forceinline__ float slice_dot_q4_k(const uint4 &h, const uint4 &q0, const uint4 &q1,
                                                 int pair, const float (&x)[64],
                                                 const float (&sx)[2]) {
-    uint32_t w[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-    float d = jl_half_bits_to_float(h.x);
-    float dmin = jl_half_bits_to_float(h.x >> 16);
+    const uint32_t w[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const float d = jl_half_bits_to_float(h.x);
+    const float dmin = jl_half_bits_to_float(h.x >> 16);
     int sc0, mn0, sc1, mn1;
     jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair, sc0, mn0);
     jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair + 1, sc1, mn1);
+    // a: sum(q x) * 2^-24 of the low sub-block, b: * 2^-20 of the high one; even and odd bytes apart
     float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        uint32_t lo = jl_opaque(w[i] & 0x0F0F0F0Fu);
-        uint32_t hi = jl_opaque((w[i] >> 4) & 0x0F0F0F0Fu);
-        a0 = fmaf(ubyte(lo, 0), x[4 * i + 0], a0);
-        a1 = fmaf(ubyte(lo, 1), x[4 * i + 1], a1);
-        a0 = fmaf(ubyte(lo, 2), x[4 * i + 2], a0);
-        a1 = fmaf(ubyte(lo, 3), x[4 * i + 3], a1);
-        b0 = fmaf(ubyte(hi, 0), x[32 + 4 * i + 0], b0);
-        b1 = fmaf(ubyte(hi, 1), x[32 + 4 * i + 1], b1);
-        b0 = fmaf(ubyte(hi, 2), x[32 + 4 * i + 2], b0);
-        b1 = fmaf(ubyte(hi, 3), x[32 + 4 * i + 3], b1);
+        const NibblePairs n = nibble_pairs(w[i]);
+        mix_byte(n, 0, x[4 * i + 0], x[32 + 4 * i + 0], a0, b0);
+        mix_byte(n, 1, x[4 * i + 1], x[32 + 4 * i + 1], a1, b1);
+        mix_byte(n, 2, x[4 * i + 2], x[32 + 4 * i + 2], a0, b0);
+        mix_byte(n, 3, x[4 * i + 3], x[32 + 4 * i + 3], a1, b1);
     }
-    float lo_term = (d * (float)sc0) * (a0 + a1) - (dmin * (float)mn0) * sx[0];
-    float hi_term = (d * (float)sc1) * (b0 + b1) - (dmin * (float)mn1) * sx[1];
+    float lo_term = ((d * (float)sc0) * kTwo24) * (a0 + a1) - (dmin * (float)mn0) * sx[0];
+    float hi_term = ((d * (float)sc1) * (kTwo24 * 0.0625f)) * (b0 + b1) - (dmin * (float)mn1) * sx[1];
     return lo_term + hi_term;
 }
 

@@ -143,6 +143,26 @@ def test_gemv_matches_oracle(ctx, t, d, n):
     assert err < 2e-5, err  # fp32 arithmetic throughout: only the summation order differs
 
 
+@pytest.mark.parametrize("scale", [1e-20, 1e-6, 1e6, 1e20])
+@pytest.mark.parametrize("t", [O.Q8_0, O.Q4_0, O.Q4_K])
+def test_gemv_over_activation_magnitudes(ctx, t, scale):
+    """The kernels move powers of two between the weights, the sums and the block scales (the 4-bit
+    ones multiply nibbles as binary16 subnormals): none of that may cost range or bits for
+    activations forty decades apart."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    d, n = 264, 4096
+    say("gemv, activations x", scale, NAMES[t])
+    raw = synthetic.weight(t, d, n, seed=1800)
+    x = (synthetic.activations(n, seed=1801).astype(np.float64) * scale).astype(np.float32)
+    ref = O.matmul(t, raw, x, d, n, O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256)
+    w = upload(ctx, t, raw, d, n)
+    out = ctx.float_array(d, fill=POISON)
+    QuantizedProjections(ctx, TornadoWorkspace()).floatMatvec(ctx.from_numpy(x), out, w, n, d)
+    ctx.sync()
+    assert rel_err(out.get(), ref, magnitude(t, raw, x, d, n)) < 2e-5
+
+
 @pytest.mark.parametrize("t,d,n", [(O.Q8_0, 130, 14336), (O.Q4_0, 1022, 14336), (O.Q4_K, 67, 12288)])
 def test_residual_matvec_on_long_rows(ctx, t, d, n):
     """x += w . hb at the down projection's row lengths (the 1024-thread workgroups), ragged last tile."""
