@@ -463,9 +463,18 @@ __device__ uint64_t *jl_gemv_stamp_buf = nullptr;
 #define GSTAMP(k) do { } while (0)
 #endif
 
-template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256>
+// SPT != 0 is the kernel for the usual launch, with its geometry known to the compiler: rows of
+// exactly SPT slices (a power of two), THREADS / SPT rows per tile and, in every segment, a row
+// count that is a multiple of that, so every thread has a slice, every tile is whole and every
+// output row exists.  Sizes, offsets, the lane folds and the choice between the two ways of
+// finishing a row are then constants and most of the loop's branches and scalar bookkeeping (226
+// scalar instructions per tile and wave in the general form, as many as the vector ones) are gone.
+// (SEGS: the fixed-geometry form of the fused q|k|v, up to three weights side by side.)
+template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false>
 __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     static_assert(!(RMS && PACKED), "the packed activation is normalised before it is quantised");
+    constexpr bool LEAN = SPT != 0;
+    static_assert(!LEAN || !PACKED, "the packed form has no fixed-geometry instances");
 #ifdef JL_GEMV_STAMPS
     uint64_t stamp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #endif
@@ -476,18 +485,22 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     constexpr int SLICE = X4 * 16 + 4;            // bytes of a tile one thread brings in
 
     const int tid = threadIdx.x;
-    const int nthreads = blockDim.x;
+    const int nthreads = LEAN ? THREADS : (int)blockDim.x;
+    // geometry: constants in the fixed-geometry form, launch arguments otherwise
+    const int Sp = LEAN ? SPT : p.Sp, S = LEAN ? SPT : p.S, R = LEAN ? THREADS / (LEAN ? SPT : 1) : p.R;
+    const int row_bytes = LEAN ? SPT * SLICE : p.row_bytes;
     const int wave = __builtin_amdgcn_readfirstlane(tid / JL_WAVE);   // uniform: LDS-DMA bases stay scalar
     const int lane = tid & (JL_WAVE - 1);
-    const int r = tid / p.Sp;           // row of the tile this thread works on
-    const int s = tid - r * p.Sp;       // its 64-column slice
-    const bool active = (s < p.S) && (r < p.R);
-    const int half_rows = DUAL ? p.R / 2 : p.R;       // output rows per tile
-    const int half_bytes = half_rows * p.row_bytes;   // bytes of a tile that come from one weight
-    const int total_tiles = p.seg_tile_begin[p.nseg];
+    const int r = tid / Sp;           // row of the tile this thread works on
+    const int s = tid - r * Sp;       // its 64-column slice
+    const bool active = LEAN || ((s < S) && (r < R));
+    const int half_rows = DUAL ? R / 2 : R;       // output rows per tile
+    const int half_bytes = half_rows * row_bytes;   // bytes of a tile that come from one weight
+    const int nseg = (LEAN && !SEGS) ? 1 : p.nseg;
+    const int total_tiles = (LEAN && !SEGS) ? p.seg_tile_begin[1] : p.seg_tile_begin[nseg];
     const int stage_bytes = nthreads * SLICE;
     // every thread of the workgroup owns a slice and every load slot is real data
-    const bool exact = (p.S == p.Sp) && (p.R * p.Sp == nthreads);
+    const bool exact = LEAN || ((S == Sp) && (R * Sp == nthreads));
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
     const uint32_t ring0 = lds0 + kPartialBytes;
@@ -509,7 +522,6 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     // each wave's outstanding-load count is a compile-time constant per tile.
     // (a launch with one segment -- every one but the fused q|k|v -- never indexes the argument
     // arrays with a run-time segment: that is a scalar memory load, and a wait, per tile)
-    const int nseg = p.nseg;
     const uint8_t *const w0 = p.w[0];
     const int rows0 = p.seg_rows[0];
     float *const out0 = p.out[0];
@@ -520,22 +532,45 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
             if (i < nseg && tile >= p.seg_tile_begin[i]) seg = i;
         return seg;
     };
+    // The fixed-geometry form keeps every segment's bases in scalar registers (the argument arrays
+    // read with constant indices, once) and picks by comparing the tile with the segments' first
+    // tiles: no memory access per tile at all.
+    const uint8_t *seg_w[kMaxSeg] = {};
+    float *seg_out[kMaxSeg] = {};
+    int seg_begin[kMaxSeg] = {};
+    if constexpr (LEAN && SEGS) {
+#pragma unroll
+        for (int i = 0; i < kMaxSeg; i++) {
+            seg_w[i] = p.w[i];
+            seg_out[i] = p.out[i];
+            seg_begin[i] = p.seg_tile_begin[i];
+        }
+    }
     auto issue = [&](int tile, int st) {
         const uint8_t *wseg = w0;
         int seg_rows = rows0, local = tile;
         if (nseg > 1) {
-            const int seg = segment_of(tile);
-            wseg = (const uint8_t *)uniform_value((uintptr_t)p.w[seg]);
-            seg_rows = (int)uniform_value((uint32_t)p.seg_rows[seg]);
-            local = tile - (int)uniform_value((uint32_t)p.seg_tile_begin[seg]);
+            if constexpr (LEAN) {
+#pragma unroll
+                for (int i = 1; i < kMaxSeg; i++)
+                    if (i < nseg && tile >= seg_begin[i]) {
+                        wseg = seg_w[i];
+                        local = tile - seg_begin[i];
+                    }
+            } else {
+                const int seg = segment_of(tile);
+                wseg = (const uint8_t *)uniform_value((uintptr_t)p.w[seg]);
+                seg_rows = (int)uniform_value((uint32_t)p.seg_rows[seg]);
+                local = tile - (int)uniform_value((uint32_t)p.seg_tile_begin[seg]);
+            }
         }
         const int64_t offset = (int64_t)local * half_bytes;
-        const int64_t remain = (int64_t)seg_rows * p.row_bytes - offset;
+        const int64_t remain = (int64_t)seg_rows * row_bytes - offset;
         const int bytes = remain < half_bytes ? (int)remain : half_bytes;
         const uint8_t *base = wseg + offset;
         const uint8_t *base_up = DUAL ? p.w_up + offset : base;
         uint8_t *dst = ring + st * stage_bytes;
-        const bool whole = exact && bytes == half_bytes;  // uniform
+        const bool whole = LEAN || (exact && bytes == half_bytes);  // uniform
         if (whole) {
             // the usual case (uniform): every slot is inside the tile, nothing to redirect
 #pragma unroll
@@ -592,7 +627,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     // activations take 17 sixteen-byte slots, the last one padding: slices then start 272 bytes
     // apart and the 128-bit reads below spread over all banks (256 bytes apart they would all
     // land on the same four).  Slot q holds floats 64 * (q / 17) + 4 * (q % 17) ... + 3.
-    const int x_slots = p.S * 17;
+    const int x_slots = S * 17;
     const int x_bytes = (x_slots + nthreads - 1) / nthreads * nthreads * 16;
     const bool x_in_ring = x_bytes <= stage_bytes;  // else a region of its own after the ring
     uint8_t *xs = x_in_ring ? ring + (kStages - 1) * stage_bytes : ring + kStages * stage_bytes;
@@ -602,7 +637,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
         for (int base = 0; base < x_bytes; base += nthreads * 16) {
             const int q = base / 16 + tid;
             const int sl = q / 17, k = q - sl * 17;
-            const int off = (sl < p.S && k < 16) ? (sl * 64 + k * 4) * 4 : 0;
+            const int off = (sl < S && k < 16) ? (sl * 64 + k * 4) * 4 : 0;
             __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.x + off),
                                              (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
         }
@@ -722,7 +757,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
 
     // A row's Sp lane sums are folded over quads in registers, then one lane per quad leaves its
     // partial in LDS and the row's finishing thread adds the P = Sp / 4 partials one tile later.
-    const int P = p.Sp >= 4 ? p.Sp / 4 : 1;
+    const int P = Sp >= 4 ? Sp / 4 : 1;
     constexpr uint32_t kParity = kPartialBytes / 2;
 
     // Finishes tile `t` from the partials of parity `par`.  The R * P partial slots are at most
@@ -744,13 +779,22 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
             int local = t, seg_rows = rows0;
             float *out = out0;
             if (nseg > 1) {
-                const int seg = segment_of(t);
-                local = t - (int)uniform_value((uint32_t)p.seg_tile_begin[seg]);
-                seg_rows = (int)uniform_value((uint32_t)p.seg_rows[seg]);
-                out = (float *)uniform_value((uintptr_t)p.out[seg]);
+                if constexpr (LEAN) {
+#pragma unroll
+                    for (int i = 1; i < kMaxSeg; i++)
+                        if (i < nseg && t >= seg_begin[i]) {
+                            out = seg_out[i];
+                            local = t - seg_begin[i];
+                        }
+                } else {
+                    const int seg = segment_of(t);
+                    local = t - (int)uniform_value((uint32_t)p.seg_tile_begin[seg]);
+                    seg_rows = (int)uniform_value((uint32_t)p.seg_rows[seg]);
+                    out = (float *)uniform_value((uintptr_t)p.out[seg]);
+                }
             }
             const int row = local * half_rows + j;
-            if (tid - j * P == 0 && row < seg_rows) {
+            if (tid - j * P == 0 && (LEAN || row < seg_rows)) {
                 float *o = out + row;
                 if constexpr (DUAL) {
                     *o = jl_swiglu_value(v0, v1);
@@ -768,7 +812,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     // tile later, no barrier behind the last tile.  For gate/up the rows are dealt gate 0, up 0,
     // gate 1, up 1, ... so that both halves of an output sit in the same wave (rows of 64 slices
     // fill a wave each, so gate/up keeps the LDS hand-over there).
-    const bool in_wave = p.Sp <= (DUAL ? 32 : 64);
+    const bool in_wave = Sp <= (DUAL ? 32 : 64);
     const int r_lds = (DUAL && in_wave) ? (r & 1) * half_rows + (r >> 1) : r;   // tile row this thread reads
     for (int it = 0; it < mine; it++) {
         const int tile = first + it * gridDim.x;
@@ -786,26 +830,35 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
 
         float v = 0.f;
         if (active) {
-            if constexpr (PACKED) v = slice_dot_lds_packed<TYPE>(ring0 + (it % kStages) * stage_bytes, r_lds, s, p.row_bytes, px);
-            else v = slice_dot_lds<TYPE>(ring0 + (it % kStages) * stage_bytes, r_lds, s, p.row_bytes, x, sx);
+            if constexpr (PACKED) v = slice_dot_lds_packed<TYPE>(ring0 + (it % kStages) * stage_bytes, r_lds, s, row_bytes, px);
+            else v = slice_dot_lds<TYPE>(ring0 + (it % kStages) * stage_bytes, r_lds, s, row_bytes, x, sx);
         }
         if (it == mine - 1) GSTAMP(6);
         if (in_wave) {
-            v = group_sum(v, p.Sp);
+            v = group_sum(v, Sp);
             float up = 0.f;
-            if constexpr (DUAL) up = __shfl(v, lane + p.Sp, JL_WAVE);   // the up row sits Sp lanes on
+            if constexpr (DUAL) up = __shfl(v, lane + Sp, JL_WAVE);   // the up row sits Sp lanes on
             const int j = DUAL ? r >> 1 : r;   // output row of the tile
-            if (s == 0 && r < p.R && (!DUAL || (r & 1) == 0)) {
+            if (s == 0 && (LEAN || r < R) && (!DUAL || (r & 1) == 0)) {
                 int local = tile, seg_rows = rows0;
                 float *out = out0;
                 if (nseg > 1) {
-                    const int seg = segment_of(tile);
-                    local = tile - (int)uniform_value((uint32_t)p.seg_tile_begin[seg]);
-                    seg_rows = (int)uniform_value((uint32_t)p.seg_rows[seg]);
-                    out = (float *)uniform_value((uintptr_t)p.out[seg]);
+                    if constexpr (LEAN) {
+#pragma unroll
+                        for (int i = 1; i < kMaxSeg; i++)
+                            if (i < nseg && tile >= seg_begin[i]) {
+                                out = seg_out[i];
+                                local = tile - seg_begin[i];
+                            }
+                    } else {
+                        const int seg = segment_of(tile);
+                        local = tile - (int)uniform_value((uint32_t)p.seg_tile_begin[seg]);
+                        seg_rows = (int)uniform_value((uint32_t)p.seg_rows[seg]);
+                        out = (float *)uniform_value((uintptr_t)p.out[seg]);
+                    }
                 }
                 const int row = local * half_rows + j;
-                if (row < seg_rows) {
+                if (LEAN || row < seg_rows) {
                     float *o = out + row;
                     if constexpr (DUAL) {
                         *o = jl_swiglu_value(v, up);
@@ -818,9 +871,9 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
             }
             continue;
         }
-        if (p.Sp >= 2) v += quad_xor1(v);
-        if (p.Sp >= 4) v += quad_xor2(v);
-        if (r < p.R && (p.Sp < 4 ? s == 0 : (s & 3) == 0)) {
+        if (Sp >= 2) v += quad_xor1(v);
+        if (Sp >= 4) v += quad_xor2(v);
+        if ((LEAN || r < R) && (Sp < 4 ? s == 0 : (s & 3) == 0)) {
             const int slot = r * P + (s >> 2);
             lds_write_b32(lds0 + (it & 1) * kParity + slot * 4, __float_as_uint(v));
         }
@@ -943,9 +996,9 @@ int blocks_per_cu(const void *fn, int device, int threads, int lds) {
     return nb;
 }
 
-template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256>
+template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false>
 int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) {
-    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED, THREADS>;
+    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED, THREADS, SPT, SEGS>;
     int per_cu = blocks_per_cu((const void *)fn, ctx->device, threads, lds);
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
@@ -955,12 +1008,45 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
     return JL_OK;
 }
 
+// `fixed`: the launch meets the fixed-geometry form's conditions (rows of exactly Sp slices, whole
+// tiles only); it has an instance for the row lengths 2048, 4096, 8192 (plain and
+// residual only) and, in the 1024-thread form, 16384.
 template <int TYPE, bool DUAL>
-int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds) {
+int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, bool fixed) {
     if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
-    if (p.rms_w) return launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds);
+    if (p.rms_w) {
+        // (the RMS-folding projections are q|k|v, gate/up and the vocabulary: rows of dim columns)
+        if (fixed && threads == 256 && (p.Sp == 32 || p.Sp == 64)) {
+            if constexpr (!DUAL) {
+                if (p.nseg > 1) {
+                    return p.Sp == 32 ? launch_tiles_of<TYPE, false, true, false, 256, 32, true>(ctx, p, threads, lds)
+                                      : launch_tiles_of<TYPE, false, true, false, 256, 64, true>(ctx, p, threads, lds);
+                }
+            }
+            return p.Sp == 32 ? launch_tiles_of<TYPE, DUAL, true, false, 256, 32>(ctx, p, threads, lds)
+                              : launch_tiles_of<TYPE, DUAL, true, false, 256, 64>(ctx, p, threads, lds);
+        }
+        return launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds);
+    }
     if constexpr (!DUAL) {
-        if (threads == kWideThreads) return launch_tiles_of<TYPE, false, false, false, kWideThreads>(ctx, p, threads, lds);
+        if (fixed && threads == 256 && p.nseg > 1) {
+            if (p.Sp == 32) return launch_tiles_of<TYPE, false, false, false, 256, 32, true>(ctx, p, threads, lds);
+            if (p.Sp == 64) return launch_tiles_of<TYPE, false, false, false, 256, 64, true>(ctx, p, threads, lds);
+            return launch_tiles_of<TYPE, false, false>(ctx, p, threads, lds);
+        }
+    }
+    if (fixed && threads == 256) {
+        if (p.Sp == 32) return launch_tiles_of<TYPE, DUAL, false, false, 256, 32>(ctx, p, threads, lds);
+        if (p.Sp == 64) return launch_tiles_of<TYPE, DUAL, false, false, 256, 64>(ctx, p, threads, lds);
+        if constexpr (!DUAL) {
+            if (p.Sp == 128) return launch_tiles_of<TYPE, false, false, false, 256, 128>(ctx, p, threads, lds);
+        }
+    }
+    if constexpr (!DUAL) {
+        if (threads == kWideThreads) {
+            if (fixed && p.Sp == 256 && p.nseg == 1) return launch_tiles_of<TYPE, false, false, false, kWideThreads, 256>(ctx, p, threads, lds);
+            return launch_tiles_of<TYPE, false, false, false, kWideThreads>(ctx, p, threads, lds);
+        }
     }
     return launch_tiles_of<TYPE, DUAL, false>(ctx, p, threads, lds);
 }
@@ -1088,17 +1174,19 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
 
     const int threads = (R * Sp + 63) / 64 * 64;
     const int lds = tile_lds_bytes(threads, slice, S);
+    bool fixed = S == Sp && R * Sp == threads;
+    for (int i = 0; i < nseg; i++) fixed = fixed && w[i]->rows % half_rows == 0;
 
     switch (type) {
         case JL_Q8_0:
-            return dual ? launch_tiles<JL_Q8_0, true>(ctx, p, threads, lds)
-                        : launch_tiles<JL_Q8_0, false>(ctx, p, threads, lds);
+            return dual ? launch_tiles<JL_Q8_0, true>(ctx, p, threads, lds, fixed)
+                        : launch_tiles<JL_Q8_0, false>(ctx, p, threads, lds, fixed);
         case JL_Q4_0:
-            return dual ? launch_tiles<JL_Q4_0, true>(ctx, p, threads, lds)
-                        : launch_tiles<JL_Q4_0, false>(ctx, p, threads, lds);
+            return dual ? launch_tiles<JL_Q4_0, true>(ctx, p, threads, lds, fixed)
+                        : launch_tiles<JL_Q4_0, false>(ctx, p, threads, lds, fixed);
         case JL_Q4_K:
-            return dual ? launch_tiles<JL_Q4_K, true>(ctx, p, threads, lds)
-                        : launch_tiles<JL_Q4_K, false>(ctx, p, threads, lds);
+            return dual ? launch_tiles<JL_Q4_K, true>(ctx, p, threads, lds, fixed)
+                        : launch_tiles<JL_Q4_K, false>(ctx, p, threads, lds, fixed);
         default:
             return jl_fail(JL_ERR_UNSUPPORTED,
                            "no single-token projection kernel for a ggml type %d weight", type);
