@@ -163,6 +163,38 @@ def test_gemv_over_activation_magnitudes(ctx, t, scale):
     assert rel_err(out.get(), ref, magnitude(t, raw, x, d, n)) < 2e-5
 
 
+@pytest.mark.parametrize("n", [2048, 4096, 8192, 16384])
+@pytest.mark.parametrize("t", [O.Q8_0, O.Q4_0, O.Q4_K])
+def test_fixed_geometry_and_general_kernels_give_the_same_bits(ctx, t, n):
+    """A weight of whole tiles runs the kernel compiled for its row length; the same weight less its
+    last row has a ragged last tile and runs the general one.  Same arithmetic in the same order:
+    the rows they share come out bit for bit equal (plain and gate/up)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    d = 272
+    say("fixed vs general", NAMES[t], d, n)
+    raw = synthetic.weight(t, d, n, seed=1900 + n)
+    raw_up = synthetic.weight(t, d, n, seed=1901 + n)
+    row_bytes = raw.size // d
+    x = ctx.from_numpy(synthetic.activations(n, seed=1902))
+    outs = []
+    for rows in (d, d - 1):
+        w = upload(ctx, t, raw[: rows * row_bytes], rows, n)
+        w_up = upload(ctx, t, raw_up[: rows * row_bytes], rows, n)
+        out = ctx.float_array(rows, fill=POISON)
+        hb = ctx.float_array(rows, fill=POISON)
+        ws = TornadoWorkspace(wrapXb=x, wrapHb=hb)
+        proj = QuantizedProjections(ctx, ws)
+        proj.floatMatvec(x, out, w, n, rows)
+        if n <= 8192:
+            proj.gateUp(w, w_up, n, rows)
+        ctx.sync()
+        outs.append((out.get(), hb.get()))
+    assert bits_equal(outs[0][0][: d - 1], outs[1][0])
+    if n <= 8192:
+        assert bits_equal(outs[0][1][: d - 1], outs[1][1])
+
+
 @pytest.mark.parametrize("t,d,n", [(O.Q8_0, 130, 14336), (O.Q4_0, 1022, 14336), (O.Q4_K, 67, 12288)])
 def test_residual_matvec_on_long_rows(ctx, t, d, n):
     """x += w . hb at the down projection's row lengths (the 1024-thread workgroups), ragged last tile."""
