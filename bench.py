@@ -738,6 +738,43 @@ def traffic_probe(ctx, proj, layers):
                                   "algorithmic_write_bytes": 4 * HIDDEN}}))
 
 
+def decode_probe(ctx, proj, layers, wcls, acts):
+    """What the kernel trace of the decode kernels is collected on: the 65 launches of a decode
+    step, kernel by kernel (no graph: a tracer serialises a replayed graph anyway), six steps over
+    the 16 layers' distinct weights; then one layer at 8B-model shapes for the other two weight
+    types (Q4_0: ffn 14336, Q4_K: ffn 12288), five device copies in turn, four rounds."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    for _ in range(6):
+        decode_step(proj, layers, wcls, acts)
+    ctx.sync()
+    dim, kv = 4096, 1024
+    for type_name, ffn in (("Q4_0", 14336), ("Q4_K", 12288)):
+        t = GGMLType[type_name]
+        shapes = {"wq": (dim, dim), "wk": (kv, dim), "wv": (kv, dim), "wo": (dim, dim),
+                  "w1": (ffn, dim), "w3": (ffn, dim), "w2": (dim, ffn)}
+        host = {k: synthetic.weight(t, r, c, 71 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
+        copies = [{k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes} for _ in range(5)]
+        x, xb = ctx.from_numpy(synthetic.activations(dim, 78)), ctx.from_numpy(synthetic.activations(dim, 79))
+        q, k_, v = ctx.float_array(dim), ctx.float_array(kv), ctx.float_array(kv)
+        hb = ctx.from_numpy(synthetic.activations(ffn, 80) * np.float32(0.1))
+        hb2 = ctx.float_array(ffn)
+        p8 = QuantizedProjections(ctx, TornadoWorkspace(wrapX=x, wrapXb=xb, wrapHb=hb2, wrapHb2=hb))
+        for _ in range(4):
+            for w in copies:
+                p8.fusedQKV(xb, q, k_, v, w["wq"], w["wk"], w["wv"])
+                p8.residualMatvec(xb, w["wo"], dim, dim)
+                p8.gateUp(w["w1"], w["w3"], dim, ffn)
+                p8.residualMatvec(hb, w["w2"], ffn, dim)
+        ctx.sync()
+        for w in copies:
+            for a in w.values():
+                a.free()
+    print(json.dumps({"decode_probe": {"steps": 6, "launches_per_step": 65,
+                                       "other_types": {"layers": 5, "rounds": 4}}}))
+
+
 def prefill_probe(ctx, t, T=2048):
     """What the matrix-pipe counters (`rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F16 SQ_VALU_MFMA_BUSY_CYCLES
     SQ_BUSY_CU_CYCLES GRBM_GUI_ACTIVE`) are collected on: one Llama-3.2-1B layer's four prefill calls at
@@ -833,6 +870,8 @@ def main():
                     help="only launch what the matrix-pipe counters are read on (see prefill_probe)")
     ap.add_argument("--batched-probe", action="store_true",
                     help="only launch the batched-decode calls, kernel by kernel (see batched_probe)")
+    ap.add_argument("--decode-probe", action="store_true",
+                    help="only launch the decode kernels, kernel by kernel (see decode_probe)")
     ap.add_argument("--int8-probe", action="store_true",
                     help="only launch the int8 prefill calls, kernel by kernel (see int8_probe)")
     args = ap.parse_args()
@@ -868,6 +907,9 @@ def main():
         proj = QuantizedProjections(ctx, ws)
         if args.traffic_probe:
             traffic_probe(ctx, proj, layers)
+            return
+        if args.decode_probe:
+            decode_probe(ctx, proj, layers, wcls, acts)
             return
         total_bytes = decode_bytes()
         assert total_bytes == 1316320256, total_bytes
