@@ -470,10 +470,15 @@ __device__ uint64_t *jl_gemv_stamp_buf = nullptr;
 // finishing a row are then constants and most of the loop's branches and scalar bookkeeping (226
 // scalar instructions per tile and wave in the general form, as many as the vector ones) are gone.
 // (SEGS: the fixed-geometry form of the fused q|k|v, up to three weights side by side.)
-template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false>
+// (PART: rows of fewer than SPT slices -- 11 008, 12 288, 14 336 columns under SPT = 256 -- whose
+// lanes past the row's end idle; everything but the row length is still a constant.)
+template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false,
+          bool PART = false>
 __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     static_assert(!(RMS && PACKED), "the packed activation is normalised before it is quantised");
     constexpr bool LEAN = SPT != 0;
+    constexpr bool FULL = LEAN && !PART;   // every lane has a slice, every load slot is real data
+    static_assert(!PART || (LEAN && !SEGS), "rows shorter than SPT slices: one weight, fixed tile shape");
     static_assert(!LEAN || !PACKED, "the packed form has no fixed-geometry instances");
 #ifdef JL_GEMV_STAMPS
     uint64_t stamp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -487,20 +492,20 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     const int tid = threadIdx.x;
     const int nthreads = LEAN ? THREADS : (int)blockDim.x;
     // geometry: constants in the fixed-geometry form, launch arguments otherwise
-    const int Sp = LEAN ? SPT : p.Sp, S = LEAN ? SPT : p.S, R = LEAN ? THREADS / (LEAN ? SPT : 1) : p.R;
-    const int row_bytes = LEAN ? SPT * SLICE : p.row_bytes;
+    const int Sp = LEAN ? SPT : p.Sp, S = FULL ? SPT : p.S, R = LEAN ? THREADS / (LEAN ? SPT : 1) : p.R;
+    const int row_bytes = FULL ? SPT * SLICE : p.row_bytes;
     const int wave = __builtin_amdgcn_readfirstlane(tid / JL_WAVE);   // uniform: LDS-DMA bases stay scalar
     const int lane = tid & (JL_WAVE - 1);
     const int r = tid / Sp;           // row of the tile this thread works on
     const int s = tid - r * Sp;       // its 64-column slice
-    const bool active = LEAN || ((s < S) && (r < R));
+    const bool active = FULL || ((s < S) && (LEAN || r < R));
     const int half_rows = DUAL ? R / 2 : R;       // output rows per tile
     const int half_bytes = half_rows * row_bytes;   // bytes of a tile that come from one weight
     const int nseg = (LEAN && !SEGS) ? 1 : p.nseg;
     const int total_tiles = (LEAN && !SEGS) ? p.seg_tile_begin[1] : p.seg_tile_begin[nseg];
     const int stage_bytes = nthreads * SLICE;
     // every thread of the workgroup owns a slice and every load slot is real data
-    const bool exact = LEAN || ((S == Sp) && (R * Sp == nthreads));
+    const bool exact = FULL || (!PART && (S == Sp) && (R * Sp == nthreads));
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
     const uint32_t ring0 = lds0 + kPartialBytes;
@@ -570,7 +575,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
         const uint8_t *base = wseg + offset;
         const uint8_t *base_up = DUAL ? p.w_up + offset : base;
         uint8_t *dst = ring + st * stage_bytes;
-        const bool whole = LEAN || (exact && bytes == half_bytes);  // uniform
+        const bool whole = FULL || (exact && bytes == half_bytes);  // uniform
         if (whole) {
             // the usual case (uniform): every slot is inside the tile, nothing to redirect
 #pragma unroll
@@ -996,9 +1001,10 @@ int blocks_per_cu(const void *fn, int device, int threads, int lds) {
     return nb;
 }
 
-template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false>
+template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false,
+          bool PART = false>
 int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) {
-    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED, THREADS, SPT, SEGS>;
+    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED, THREADS, SPT, SEGS, PART>;
     int per_cu = blocks_per_cu((const void *)fn, ctx->device, threads, lds);
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
@@ -1014,9 +1020,10 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
 template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, bool fixed) {
     if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
+    const bool full = fixed && p.S == p.Sp;
     if (p.rms_w) {
         // (the RMS-folding projections are q|k|v, gate/up and the vocabulary: rows of dim columns)
-        if (fixed && threads == 256 && (p.Sp == 32 || p.Sp == 64)) {
+        if (full && threads == 256 && (p.Sp == 32 || p.Sp == 64)) {
             if constexpr (!DUAL) {
                 if (p.nseg > 1) {
                     return p.Sp == 32 ? launch_tiles_of<TYPE, false, true, false, 256, 32, true>(ctx, p, threads, lds)
@@ -1029,13 +1036,13 @@ int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, boo
         return launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds);
     }
     if constexpr (!DUAL) {
-        if (fixed && threads == 256 && p.nseg > 1) {
+        if (full && threads == 256 && p.nseg > 1) {
             if (p.Sp == 32) return launch_tiles_of<TYPE, false, false, false, 256, 32, true>(ctx, p, threads, lds);
             if (p.Sp == 64) return launch_tiles_of<TYPE, false, false, false, 256, 64, true>(ctx, p, threads, lds);
             return launch_tiles_of<TYPE, false, false>(ctx, p, threads, lds);
         }
     }
-    if (fixed && threads == 256) {
+    if (full && threads == 256) {
         if (p.Sp == 32) return launch_tiles_of<TYPE, DUAL, false, false, 256, 32>(ctx, p, threads, lds);
         if (p.Sp == 64) return launch_tiles_of<TYPE, DUAL, false, false, 256, 64>(ctx, p, threads, lds);
         if constexpr (!DUAL) {
@@ -1044,7 +1051,10 @@ int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, boo
     }
     if constexpr (!DUAL) {
         if (threads == kWideThreads) {
-            if (fixed && p.Sp == 256 && p.nseg == 1) return launch_tiles_of<TYPE, false, false, false, kWideThreads, 256>(ctx, p, threads, lds);
+            if (fixed && p.Sp == 256 && p.nseg == 1) {
+                return p.S == p.Sp ? launch_tiles_of<TYPE, false, false, false, kWideThreads, 256>(ctx, p, threads, lds)
+                                   : launch_tiles_of<TYPE, false, false, false, kWideThreads, 256, false, true>(ctx, p, threads, lds);
+            }
             return launch_tiles_of<TYPE, false, false, false, kWideThreads>(ctx, p, threads, lds);
         }
     }
@@ -1174,7 +1184,8 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
 
     const int threads = (R * Sp + 63) / 64 * 64;
     const int lds = tile_lds_bytes(threads, slice, S);
-    bool fixed = S == Sp && R * Sp == threads;
+    // (whole tiles only; `full`: rows of exactly Sp slices as well)
+    bool fixed = R * Sp == threads;
     for (int i = 0; i < nseg; i++) fixed = fixed && w[i]->rows % half_rows == 0;
 
     switch (type) {

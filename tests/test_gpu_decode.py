@@ -163,7 +163,7 @@ def test_gemv_over_activation_magnitudes(ctx, t, scale):
     assert rel_err(out.get(), ref, magnitude(t, raw, x, d, n)) < 2e-5
 
 
-@pytest.mark.parametrize("n", [2048, 4096, 8192, 16384])
+@pytest.mark.parametrize("n", [2048, 4096, 8192, 11008, 14336, 16384])
 @pytest.mark.parametrize("t", [O.Q8_0, O.Q4_0, O.Q4_K])
 def test_fixed_geometry_and_general_kernels_give_the_same_bits(ctx, t, n):
     """A weight of whole tiles runs the kernel compiled for its row length; the same weight less its
