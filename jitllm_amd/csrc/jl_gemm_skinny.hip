@@ -731,13 +731,35 @@ __global__ void __launch_bounds__(256) jl_skinny_reduce(SkinnyParams p, int padd
     if (local >= seg_rows) return;
     const int64_t width = (int64_t)total_groups * 16;
     const float *pp = p.planes + (int64_t)m * width + v;
+    float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + seg_col + local;
+    const bool add = !DUAL && p.epilogue == JL_RESIDUAL;
+    const bool whole = local + 3 < seg_rows && (((uintptr_t)dst) & 15) == 0;
+    // Every load of the thread goes out before the first sum needs one -- the planes four at a
+    // time, the output's old value with them -- so the kernel waits for memory once, not once per
+    // plane; absent planes add +0, which changes nothing (a running sum that began at +0 is never -0).
+    float4 o = {0.f, 0.f, 0.f, 0.f};
+    if (add && whole) o = *(const float4 *)dst;
     float4 s = {0.f, 0.f, 0.f, 0.f}, u = {0.f, 0.f, 0.f, 0.f};
-    for (int zz = 0; zz < p.Z; zz++) {
-        const float4 a = *(const float4 *)(pp + (int64_t)zz * padded_rows * width);
-        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
-        if (DUAL) {
-            const float4 c = *(const float4 *)(pp + (int64_t)zz * padded_rows * width + 8);
-            u.x += c.x; u.y += c.y; u.z += c.z; u.w += c.w;
+    const int64_t plane = (int64_t)padded_rows * width;
+    for (int z0 = 0; z0 < p.Z; z0 += 4) {
+        float4 a[4], c[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const bool on = z0 + j < p.Z;
+            const float *q = pp + (on ? z0 + j : z0) * plane;
+            a[j] = *(const float4 *)q;
+            if (!on) a[j] = float4{0.f, 0.f, 0.f, 0.f};
+            if (DUAL) {
+                c[j] = *(const float4 *)(q + 8);
+                if (!on) c[j] = float4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            s.x += a[j].x; s.y += a[j].y; s.z += a[j].z; s.w += a[j].w;
+            if (DUAL) {
+                u.x += c[j].x; u.y += c[j].y; u.z += c[j].z; u.w += c[j].w;
+            }
         }
     }
     float out[4] = {s.x, s.y, s.z, s.w};
@@ -745,11 +767,8 @@ __global__ void __launch_bounds__(256) jl_skinny_reduce(SkinnyParams p, int padd
         out[0] = skinny_swiglu(s.x, u.x); out[1] = skinny_swiglu(s.y, u.y);
         out[2] = skinny_swiglu(s.z, u.z); out[3] = skinny_swiglu(s.w, u.w);
     }
-    float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + seg_col + local;
-    const bool add = !DUAL && p.epilogue == JL_RESIDUAL;
-    if (local + 3 < seg_rows && (((uintptr_t)dst) & 15) == 0) {
+    if (whole) {
         if (add) {
-            const float4 o = *(const float4 *)dst;
             *(float4 *)dst = float4{o.x + out[0], o.y + out[1], o.z + out[2], o.w + out[3]};
         } else {
             *(float4 *)dst = float4{out[0], out[1], out[2], out[3]};
