@@ -704,10 +704,10 @@ def bench_wq_shape(ctx, hip, t, steps, warmup, cpu):
 
 
 # HBM bytes one gate/up launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
-# `bench.py --traffic-probe` (profiles/gemv_q8_0_gate_up_hbm_traffic.md): 17 517 KiB x 2.0 read
+# `bench.py --traffic-probe` (profiles/gemv_q8_0_gate_up_hbm_traffic.md): 17 475 KiB x 2.0 read
 # (the counter books 64 bytes for each of this chip's 128-byte requests; a 256 MiB plain copy reads
-# 131 088 KiB on it) + 64 KiB x 1.0 written.  The algorithmic figure is 35 733 504 bytes.
-GATE_UP_HBM_TRAFFIC_BYTES = 17517 * 1024 * 2 + 64 * 1024
+# 131 087 KiB on it) + 64 KiB x 1.0 written.  The algorithmic figure is 35 733 504 bytes.
+GATE_UP_HBM_TRAFFIC_BYTES = 17475 * 1024 * 2 + 64 * 1024
 
 
 def traffic_probe(ctx, proj, layers):
