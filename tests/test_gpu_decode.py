@@ -195,6 +195,46 @@ def test_fixed_geometry_and_general_kernels_give_the_same_bits(ctx, t, n):
         assert bits_equal(outs[0][1][: d - 1], outs[1][1])
 
 
+def _random_shapes():
+    """Seeded row counts and row lengths across every dispatch of the tile kernel: the
+    fixed-geometry instances (whole tiles of 2048 / 4096 / 8192 / 16384-column rows), rows that
+    fill their slices only in part, ragged last tiles, the 1024-thread workgroups."""
+    rng = np.random.default_rng(20260917)
+    shapes = []
+    for t, step in ((O.Q8_0, 64), (O.Q4_0, 64), (O.Q4_K, 256)):
+        for _ in range(14):
+            n = int(rng.integers(1, 16384 // step + 1)) * step
+            d = int(rng.integers(1, 400))
+            shapes.append((t, d, n))
+        for n in (2048, 4096, 8192, 12288):
+            shapes.append((t, int(rng.integers(1, 40)) * 8, n))   # whole tiles
+    return shapes
+
+
+@pytest.mark.parametrize("t,d,n", _random_shapes())
+def test_gemv_and_residual_on_random_shapes(ctx, t, d, n):
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("gemv, random shape", NAMES[t], d, n)
+    raw = synthetic.weight(t, d, n, seed=3000 + d + n)
+    x = synthetic.activations(n, seed=3100 + n)
+    ref = O.matmul(t, raw, x, d, n, O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256)
+    mag = magnitude(t, raw, x, d, n)
+    w = upload(ctx, t, raw, d, n)
+    out = ctx.float_array(d, fill=POISON)
+    base = synthetic.activations(d, seed=3200)
+    acc = ctx.from_numpy(base)
+    proj = QuantizedProjections(ctx, TornadoWorkspace(wrapX=acc))
+    dx = ctx.from_numpy(x)
+    proj.floatMatvec(dx, out, w, n, d)
+    proj.residualMatvec(dx, w, n, d)
+    ctx.sync()
+    got = out.get()
+    assert np.all(got != POISON)
+    assert rel_err(got, ref, mag) < 2e-5
+    assert rel_err(acc.get(), ref.astype(np.float64) + base, mag + np.abs(base) * 6e-8) < 2e-5
+
+
 @pytest.mark.parametrize("t,d,n", [(O.Q8_0, 130, 14336), (O.Q4_0, 1022, 14336), (O.Q4_K, 67, 12288)])
 def test_residual_matvec_on_long_rows(ctx, t, d, n):
     """x += w . hb at the down projection's row lengths (the 1024-thread workgroups), ragged last tile."""
