@@ -59,10 +59,20 @@ struct GemvParams {
     const int32_t *xq_sums;
 };
 
+// Bytes of a tile a thread brings in: kX4 sixteen-byte loads and kTail four-byte ones.  For the
+// three main types that is exactly a thread's 64-column slice, so every load slot is real data; a
+// Q6_K slice is 52.5 bytes (210 per 256 columns), its threads bring in 64 each and the slots past
+// the tile's end re-read a dummy address.
 template <int TYPE> struct Traits;
-template <> struct Traits<JL_Q8_0> { static constexpr int kX4 = 4; };  // 68 B = 4 x 16 + 4
-template <> struct Traits<JL_Q4_0> { static constexpr int kX4 = 2; };  // 36 B = 2 x 16 + 4
-template <> struct Traits<JL_Q4_K> { static constexpr int kX4 = 2; };  // 144 B / 4 = 36 B
+template <> struct Traits<JL_Q8_0> { static constexpr int kX4 = 4, kTail = 1; };  // 68 B = 4 x 16 + 4
+template <> struct Traits<JL_Q4_0> { static constexpr int kX4 = 2, kTail = 1; };  // 36 B = 2 x 16 + 4
+template <> struct Traits<JL_Q4_K> { static constexpr int kX4 = 2, kTail = 1; };  // 144 B / 4 = 36 B
+template <> struct Traits<JL_Q6_K> { static constexpr int kX4 = 4, kTail = 0; };  // 64 B >= 210 B / 4
+// bytes of a row of `slices` 64-column slices
+template <int TYPE>
+__device__ __host__ constexpr int row_bytes_of(int slices) {
+    return TYPE == JL_Q8_0 ? slices * 68 : TYPE == JL_Q6_K ? slices / 4 * 210 : slices * 36;
+}
 
 __device__ __forceinline__ float ubyte(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
 __device__ __forceinline__ float sbyte(uint32_t v, int k) { return (float)(int)(int8_t)(v >> (8 * k)); }
@@ -129,7 +139,7 @@ constexpr float kTwo24 = 16777216.f, kTwoM24 = 1.f / 16777216.f;
 //   bytes 0..1 scale A | 2..17 nibbles A | 18..19 scale B | 20..35 nibbles B
 // element i < 16 of a block is the low nibble of its byte i, element 16 + i the high nibble.
 __device__ __forceinline__ float slice_dot_q4_0(const uint32_t (&dw)[9], const float (&x)[64],
-                                                const float (&sx)[2]) {
+                                                const float (&sx)[4]) {
     NibblePairs n[9];
 #pragma unroll
     for (int i = 0; i < 9; i++) n[i] = nibble_pairs(dw[i]);
@@ -158,7 +168,7 @@ __device__ __forceinline__ float slice_dot_q4_0(const uint32_t (&dw)[9], const f
 // sum(w x) = (d sc) sum(q x) - (dmin m) sum(x) per sub-block.
 __device__ __forceinline__ float slice_dot_q4_k(const uint4 &h, const uint4 &q0, const uint4 &q1,
                                                 int pair, const float (&x)[64],
-                                                const float (&sx)[2]) {
+                                                const float (&sx)[4]) {
     const uint32_t w[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
     const float d = jl_half_bits_to_float(h.x);
     const float dmin = jl_half_bits_to_float(h.x >> 16);
@@ -178,6 +188,44 @@ __device__ __forceinline__ float slice_dot_q4_k(const uint4 &h, const uint4 &q0,
     float lo_term = ((d * (float)sc0) * kTwo24) * (a0 + a1) - (dmin * (float)mn0) * sx[0];
     float hi_term = ((d * (float)sc1) * (kTwo24 * 0.0625f)) * (b0 + b1) - (dmin * (float)mn1) * sx[1];
     return lo_term + hi_term;
+}
+
+// acc += (the four bytes of v, values up to 255, as binary16 subnormals b * 2^-24) . x[0..3]
+__device__ __forceinline__ void mix_bytes4(float &acc, uint32_t v, float x0, float x1, float x2, float x3) {
+    const uint32_t even = v & 0x00FF00FFu, odd = (v >> 8) & 0x00FF00FFu;
+    mix_low(acc, even, x0);
+    mix_low(acc, odd, x1);
+    mix_high(acc, even, x2);
+    mix_high(acc, odd, x3);
+}
+
+// Dot of a quarter of a Q6_K super-block (ql[128] | qh[64] | 16 signed scales | fp16 d,
+// J/tensor/standard/Q6_KFloatTensor.java:66-122) with 64 activations.  Quarter (h, upper): the
+// 64 ql bytes and 32 qh bytes of half h; element l < 32 of the quarter is nibble `upper` of ql[l]
+// with bits 4 upper .. 4 upper + 1 of qh[l] on top, element 32 + l nibble `upper` of ql[32 + l]
+// with bits 4 upper + 2 .. + 3 of qh[l].  w = d * scale * (q - 32) with one scale per 16 elements;
+// sx are the sums of the activations facing each 16.
+__device__ __forceinline__ float slice_dot_q6_k(const uint32_t (&ql)[16], const uint32_t (&qh)[8], uint32_t scales,
+                                                uint32_t dbits, int upper, const float (&x)[64],
+                                                const float (&sx)[4]) {
+    const int shl = 4 * upper;
+    float a[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t h = qh[j] >> shl;
+        const uint32_t v0 = ((ql[j] >> shl) & 0x0F0F0F0Fu) | ((h & 0x03030303u) << 4);
+        const uint32_t v1 = ((ql[8 + j] >> shl) & 0x0F0F0F0Fu) | ((h & 0x0C0C0C0Cu) << 2);
+        mix_bytes4(a[j >> 2], v0, x[4 * j], x[4 * j + 1], x[4 * j + 2], x[4 * j + 3]);
+        mix_bytes4(a[2 + (j >> 2)], v1, x[32 + 4 * j], x[32 + 4 * j + 1], x[32 + 4 * j + 2], x[32 + 4 * j + 3]);
+    }
+    const float d = jl_half_bits_to_float(dbits) * kTwo24;
+    float acc = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const float sc = (float)(int)(int8_t)(scales >> (8 * g));
+        acc = fmaf(sc, fmaf(-32.f * kTwoM24, sx[g], a[g]), acc);
+    }
+    return acc * d;
 }
 
 // ---- packed-integer mode -----------------------------------------------------------------------
@@ -383,11 +431,33 @@ __device__ __forceinline__ void lds_read_q4k(uint32_t hdr, uint32_t qs, uint4 &h
         : "=&v"(h), "=&v"(q0), "=&v"(q1) : "v"(hdr), "v"(qs) : "memory");
 }
 
+// the 64 ql bytes, 32 qh bytes, four scales and d of a Q6_K quarter (super-blocks are 210 bytes
+// apart: the addresses are two-byte aligned, which the LDS serves)
+__device__ __forceinline__ void lds_read_q6k(uint32_t ql_at, uint32_t qh_at, uint32_t sc_at, uint32_t d_at,
+                                             uint32_t (&ql)[16], uint32_t (&qh)[8], uint32_t &scales, uint32_t &d) {
+    uint4 a, b, c, e, f, g;
+    asm volatile(
+        "ds_read_b128 %0, %8\n\tds_read_b128 %1, %8 offset:16\n\tds_read_b128 %2, %8 offset:32\n\t"
+        "ds_read_b128 %3, %8 offset:48\n\tds_read_b128 %4, %9\n\tds_read_b128 %5, %9 offset:16\n\t"
+        "ds_read_b32 %6, %10\n\tds_read_u16 %7, %11\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(e), "=&v"(f), "=&v"(g), "=&v"(scales), "=&v"(d)
+        : "v"(ql_at), "v"(qh_at), "v"(sc_at), "v"(d_at) : "memory");
+    ql[0] = a.x; ql[1] = a.y; ql[2] = a.z; ql[3] = a.w; ql[4] = b.x; ql[5] = b.y; ql[6] = b.z; ql[7] = b.w;
+    ql[8] = c.x; ql[9] = c.y; ql[10] = c.z; ql[11] = c.w; ql[12] = e.x; ql[13] = e.y; ql[14] = e.z; ql[15] = e.w;
+    qh[0] = f.x; qh[1] = f.y; qh[2] = f.z; qh[3] = f.w; qh[4] = g.x; qh[5] = g.y; qh[6] = g.z; qh[7] = g.w;
+}
+
 template <int TYPE>
 __device__ __forceinline__ float slice_dot_lds(uint32_t stage, int r, int s, int row_bytes,
-                                               const float (&x)[64], const float (&sx)[2]) {
+                                               const float (&x)[64], const float (&sx)[4]) {
     const uint32_t row = stage + (uint32_t)(r * row_bytes);
-    if constexpr (TYPE == JL_Q8_0) {
+    if constexpr (TYPE == JL_Q6_K) {
+        const uint32_t sb = row + (s >> 2) * 210;
+        const int h = (s >> 1) & 1;
+        uint32_t ql[16], qh[8], scales, d;
+        lds_read_q6k(sb + 64 * h, sb + 128 + 32 * h, sb + 192 + 4 * (s & 3), sb + 208, ql, qh, scales, d);
+        return slice_dot_q6_k(ql, qh, scales, d, s & 1, x, sx);
+    } else if constexpr (TYPE == JL_Q8_0) {
         uint32_t w[17];
         lds_read_17(row + s * 68, w);
         return slice_dot_q8_0(w, x);
@@ -486,14 +556,15 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     GSTAMP(0);
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
-    constexpr int L = X4 + 1;                     // plus one 4-byte load
-    constexpr int SLICE = X4 * 16 + 4;            // bytes of a tile one thread brings in
+    constexpr int L = X4 + Traits<TYPE>::kTail;   // plus (three main types) one 4-byte load
+    constexpr int SLICE = X4 * 16 + 4 * Traits<TYPE>::kTail;   // bytes of a tile one thread brings in
+    constexpr bool kExactDma = TYPE != JL_Q6_K;   // a thread's loads are exactly its slice
 
     const int tid = threadIdx.x;
     const int nthreads = LEAN ? THREADS : (int)blockDim.x;
     // geometry: constants in the fixed-geometry form, launch arguments otherwise
     const int Sp = LEAN ? SPT : p.Sp, S = FULL ? SPT : p.S, R = LEAN ? THREADS / (LEAN ? SPT : 1) : p.R;
-    const int row_bytes = FULL ? SPT * SLICE : p.row_bytes;
+    const int row_bytes = FULL ? row_bytes_of<TYPE>(SPT) : p.row_bytes;
     const int wave = __builtin_amdgcn_readfirstlane(tid / JL_WAVE);   // uniform: LDS-DMA bases stay scalar
     const int lane = tid & (JL_WAVE - 1);
     const int r = tid / Sp;           // row of the tile this thread works on
@@ -505,7 +576,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     const int total_tiles = (LEAN && !SEGS) ? p.seg_tile_begin[1] : p.seg_tile_begin[nseg];
     const int stage_bytes = nthreads * SLICE;
     // every thread of the workgroup owns a slice and every load slot is real data
-    const bool exact = FULL || (!PART && (S == Sp) && (R * Sp == nthreads));
+    const bool exact = kExactDma && (FULL || (!PART && (S == Sp) && (R * Sp == nthreads)));
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
     const uint32_t ring0 = lds0 + kPartialBytes;
@@ -575,7 +646,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
         const uint8_t *base = wseg + offset;
         const uint8_t *base_up = DUAL ? p.w_up + offset : base;
         uint8_t *dst = ring + st * stage_bytes;
-        const bool whole = FULL || (exact && bytes == half_bytes);  // uniform
+        const bool whole = exact && (FULL || bytes == half_bytes);  // uniform
         if (whole) {
             // the usual case (uniform): every slot is inside the tile, nothing to redirect
 #pragma unroll
@@ -723,7 +794,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     GSTAMP(4);
 
     float x[64];
-    float sx[2] = {0.f, 0.f};
+    float sx[4] = {0.f, 0.f, 0.f, 0.f};   // sums of the slice's activations by 32 (4-bit types) or 16 (Q6_K)
     PackedX px;
     if constexpr (PACKED) {
         // the slice's 64 bytes, two scales and two sums straight from global memory (a few KB that
@@ -751,7 +822,15 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
 #pragma unroll
             for (int k = 0; k < 4; k++) lds_read_16f(xs0 + s * 272 + k * 64, &x[k * 16]);
         }
-        if constexpr (TYPE != JL_Q8_0) {
+        if constexpr (TYPE == JL_Q6_K) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                sx[0] += x[k];
+                sx[1] += x[16 + k];
+                sx[2] += x[32 + k];
+                sx[3] += x[48 + k];
+            }
+        } else if constexpr (TYPE != JL_Q8_0) {
 #pragma unroll
             for (int k = 0; k < 32; k++) {
                 sx[0] += x[k];
@@ -1019,9 +1098,13 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
 // residual only) and, in the 1024-thread form, 16384.
 template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, bool fixed) {
-    if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
+    // (Q6_K: plain, residual and gate/up only -- the caller has refused the rest)
+    constexpr bool kMain = TYPE != JL_Q6_K;
+    if constexpr (kMain) {
+        if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
+    }
     const bool full = fixed && p.S == p.Sp;
-    if (p.rms_w) {
+    if constexpr (kMain) if (p.rms_w) {
         // (the RMS-folding projections are q|k|v, gate/up and the vocabulary: rows of dim columns)
         if (full && threads == 256 && (p.Sp == 32 || p.Sp == 64)) {
             if constexpr (!DUAL) {
@@ -1035,7 +1118,7 @@ int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, boo
         }
         return launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds);
     }
-    if constexpr (!DUAL) {
+    if constexpr (!DUAL && kMain) {
         if (full && threads == 256 && p.nseg > 1) {
             if (p.Sp == 32) return launch_tiles_of<TYPE, false, false, false, 256, 32, true>(ctx, p, threads, lds);
             if (p.Sp == 64) return launch_tiles_of<TYPE, false, false, false, 256, 64, true>(ctx, p, threads, lds);
@@ -1092,11 +1175,12 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
             return jl_fail(JL_ERR_UNSUPPORTED, "no fused q|k|v or RMS-folding single-token kernel for a %s weight "
                                                "(plain, residual and gate/up projections only)", jl_type_name(type));
         }
-        return jl_launch_gemv_direct(ctx, w[0], w_up, x, outs[0], epilogue);
+        // Q6_K goes on to the tile kernel when the shape allows, the rest have the one-wave-per-row kernels
+        if (type != JL_Q6_K) return jl_launch_gemv_direct(ctx, w[0], w_up, x, outs[0], epilogue);
     }
 
     const bool dual = w_up != nullptr;
-    const int slice = type == JL_Q8_0 ? 68 : 36;
+    const int slice = type == JL_Q8_0 ? 68 : type == JL_Q6_K ? 64 : 36;   // bytes a thread brings in per tile
     bool fast = (n % 64 == 0) && (n / 64 <= 256) &&
                 (xq ? (((uintptr_t)xq->quants & 15) == 0 && ((uintptr_t)xq->scales & 7) == 0 &&
                        ((uintptr_t)xq->sums & 7) == 0)
@@ -1135,6 +1219,13 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     }
     if (rms && ((uintptr_t)rms->weights & 15) != 0) {
         return jl_fail(JL_ERR_UNSUPPORTED, "the RMS weights must be 16-byte aligned");
+    }
+    if (type == JL_Q6_K) {
+        // measured: the tile kernel overtakes the one-wave-per-row kernel at about 32 MB of weights
+        // (vocabulary and 8B-model feed-forward projections); below that its fixed costs lose
+        constexpr int64_t kTileFromBytes = (int64_t)32 << 20;
+        if (!fast || w[0]->bytes * (dual ? 2 : 1) < kTileFromBytes)
+            return jl_launch_gemv_direct(ctx, w[0], w_up, x, outs[0], epilogue);
     }
     if (!fast) {
         for (int i = 0; i < nseg; i++) {
@@ -1198,6 +1289,9 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
         case JL_Q4_K:
             return dual ? launch_tiles<JL_Q4_K, true>(ctx, p, threads, lds, fixed)
                         : launch_tiles<JL_Q4_K, false>(ctx, p, threads, lds, fixed);
+        case JL_Q6_K:
+            return dual ? launch_tiles<JL_Q6_K, true>(ctx, p, threads, lds, fixed)
+                        : launch_tiles<JL_Q6_K, false>(ctx, p, threads, lds, fixed);
         default:
             return jl_fail(JL_ERR_UNSUPPORTED,
                            "no single-token projection kernel for a ggml type %d weight", type);

@@ -316,6 +316,51 @@ def test_k_quant_decode_bit_exact(ctx, t):
         assert bits_equal(w.dequantize(), O.dequant(t, raw))
 
 
+@pytest.mark.parametrize("d,n,dual", [(4096, 14336, False), (4099, 11008, False), (10001, 4096, False),
+                                      (21000, 2048, False), (4800, 8192, False), (6144, 4096, True),
+                                      (5001, 4096, True), (10000, 2048, True)])
+def test_q6_k_on_the_tile_kernel(ctx, d, n, dual):
+    """Q6_K weights of 32 MB and more leave the one-wave-per-row kernel for the tile kernel (LDS-DMA
+    ring, 52.5-byte slices read at two-byte alignment): whole and ragged tiles, rows that do not
+    fill their slices, 1024-thread workgroups, plain / residual / gate-up."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    t = O.Q6_K
+    say("q6_k tile kernel", d, n, dual)
+    raw = synthetic.weight(t, d, n, seed=4000 + d)
+    x = synthetic.activations(n, seed=4100 + n)
+    ref = O.matmul(t, raw, x, d, n)
+    mag = magnitude(t, raw, x, d, n)
+    w = upload(ctx, t, raw, d, n)
+    dx = ctx.from_numpy(x)
+    if not dual:
+        out = ctx.float_array(d, fill=POISON)
+        base = synthetic.activations(d, seed=4200)
+        acc = ctx.from_numpy(base)
+        proj = QuantizedProjections(ctx, TornadoWorkspace(wrapX=acc))
+        proj.floatMatvec(dx, out, w, n, d)
+        proj.residualMatvec(dx, w, n, d)
+        ctx.sync()
+        assert rel_err(out.get(), ref, mag) < 2e-5
+        assert rel_err(acc.get(), ref.astype(np.float64) + base, mag + np.abs(base) * 6e-8) < 2e-5
+        return
+    raw_up = synthetic.weight(t, d, n, seed=4300 + d)
+    up = O.matmul(t, raw_up, x, d, n)
+    w_up = upload(ctx, t, raw_up, d, n)
+    hb = ctx.float_array(d, fill=POISON)
+    # (the host mirror fuses gate/up only where the reference does; the library's entry point takes Q6_K)
+    from jitllm_amd import _lib as L
+    L.check(L.load().jl_gemv_gate_up(ctx.handle, w.handle, w_up.handle, dx.ptr, hb.ptr))
+    ctx.sync()
+    want = O.swiglu(ref, up)
+    got = hb.get()
+    assert np.all(got != POISON)
+    # SiLU(g) * u moves with both sums: each is held to 2e-5 of its own magnitude
+    mu = magnitude(t, raw_up, x, d, n)
+    bound = 2e-5 * (mag * np.abs(up) + mu * np.abs(ref) * 1.2 + 1e-6)
+    assert np.all(np.abs(got.astype(np.float64) - want) <= bound + 1e-6)
+
+
 @pytest.mark.parametrize("t", KQ)
 @pytest.mark.parametrize("d,n", [(2048, 2048), (32000, 2048), (2048, 8192), (37, 512), (1000, 256), (4, 4096),
                                  (64, 1024)])
