@@ -68,10 +68,11 @@ template <> struct Traits<JL_Q8_0> { static constexpr int kX4 = 4, kTail = 1; };
 template <> struct Traits<JL_Q4_0> { static constexpr int kX4 = 2, kTail = 1; };  // 36 B = 2 x 16 + 4
 template <> struct Traits<JL_Q4_K> { static constexpr int kX4 = 2, kTail = 1; };  // 144 B / 4 = 36 B
 template <> struct Traits<JL_Q6_K> { static constexpr int kX4 = 4, kTail = 0; };  // 64 B >= 210 B / 4
+template <> struct Traits<JL_Q5_K> { static constexpr int kX4 = 3, kTail = 0; };  // 48 B >= 176 B / 4
 // bytes of a row of `slices` 64-column slices
 template <int TYPE>
 __device__ __host__ constexpr int row_bytes_of(int slices) {
-    return TYPE == JL_Q8_0 ? slices * 68 : TYPE == JL_Q6_K ? slices / 4 * 210 : slices * 36;
+    return TYPE == JL_Q8_0 ? slices * 68 : TYPE == JL_Q6_K ? slices / 4 * 210 : TYPE == JL_Q5_K ? slices * 44 : slices * 36;
 }
 
 __device__ __forceinline__ float ubyte(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
@@ -226,6 +227,31 @@ __device__ __forceinline__ float slice_dot_q6_k(const uint32_t (&ql)[16], const 
         acc = fmaf(sc, fmaf(-32.f * kTwoM24, sx[g], a[g]), acc);
     }
     return acc * d;
+}
+
+// Dot of a quarter of a Q5_K super-block (fp16 d, dmin | 12 packed scale / min bytes | qh[32] |
+// qs[128], J/tensor/standard/Q5_KFloatTensor.java:78-122) with 64 activations: Q4_K's layout with a
+// fifth bit per weight -- bit 2 pair of qh[l] for the low-nibble sub-block, bit 2 pair + 1 for the
+// high-nibble one.  sum(w x) = (d sc) sum(q x) - (dmin m) sum(x) per sub-block.
+__device__ __forceinline__ float slice_dot_q5_k(const uint4 &h, const uint32_t (&qs)[8], const uint32_t (&qh)[8],
+                                                int pair, const float (&x)[64], const float (&sx)[4]) {
+    const float d = jl_half_bits_to_float(h.x);
+    const float dmin = jl_half_bits_to_float(h.x >> 16);
+    int sc0, mn0, sc1, mn1;
+    jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair, sc0, mn0);
+    jl_q4k_scale_min(h.y, h.z, h.w, 2 * pair + 1, sc1, mn1);
+    float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t hb = qh[j] >> (2 * pair);
+        const uint32_t v0 = (qs[j] & 0x0F0F0F0Fu) | ((hb & 0x01010101u) << 4);
+        const uint32_t v1 = ((qs[j] >> 4) & 0x0F0F0F0Fu) | ((hb & 0x02020202u) << 3);
+        mix_bytes4((j & 1) ? a1 : a0, v0, x[4 * j], x[4 * j + 1], x[4 * j + 2], x[4 * j + 3]);
+        mix_bytes4((j & 1) ? b1 : b0, v1, x[32 + 4 * j], x[32 + 4 * j + 1], x[32 + 4 * j + 2], x[32 + 4 * j + 3]);
+    }
+    float lo_term = ((d * (float)sc0) * kTwo24) * (a0 + a1) - (dmin * (float)mn0) * sx[0];
+    float hi_term = ((d * (float)sc1) * kTwo24) * (b0 + b1) - (dmin * (float)mn1) * sx[1];
+    return lo_term + hi_term;
 }
 
 // ---- packed-integer mode -----------------------------------------------------------------------
@@ -431,31 +457,42 @@ __device__ __forceinline__ void lds_read_q4k(uint32_t hdr, uint32_t qs, uint4 &h
         : "=&v"(h), "=&v"(q0), "=&v"(q1) : "v"(hdr), "v"(qs) : "memory");
 }
 
-// the 64 ql bytes, 32 qh bytes, four scales and d of a Q6_K quarter (super-blocks are 210 bytes
-// apart: the addresses are two-byte aligned, which the LDS serves)
-__device__ __forceinline__ void lds_read_q6k(uint32_t ql_at, uint32_t qh_at, uint32_t sc_at, uint32_t d_at,
-                                             uint32_t (&ql)[16], uint32_t (&qh)[8], uint32_t &scales, uint32_t &d) {
-    uint4 a, b, c, e, f, g;
-    asm volatile(
-        "ds_read_b128 %0, %8\n\tds_read_b128 %1, %8 offset:16\n\tds_read_b128 %2, %8 offset:32\n\t"
-        "ds_read_b128 %3, %8 offset:48\n\tds_read_b128 %4, %9\n\tds_read_b128 %5, %9 offset:16\n\t"
-        "ds_read_b32 %6, %10\n\tds_read_u16 %7, %11\n\ts_waitcnt lgkmcnt(0)"
-        : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(e), "=&v"(f), "=&v"(g), "=&v"(scales), "=&v"(d)
-        : "v"(ql_at), "v"(qh_at), "v"(sc_at), "v"(d_at) : "memory");
-    ql[0] = a.x; ql[1] = a.y; ql[2] = a.z; ql[3] = a.w; ql[4] = b.x; ql[5] = b.y; ql[6] = b.z; ql[7] = b.w;
-    ql[8] = c.x; ql[9] = c.y; ql[10] = c.z; ql[11] = c.w; ql[12] = e.x; ql[13] = e.y; ql[14] = e.z; ql[15] = e.w;
-    qh[0] = f.x; qh[1] = f.y; qh[2] = f.z; qh[3] = f.w; qh[4] = g.x; qh[5] = g.y; qh[6] = g.z; qh[7] = g.w;
-}
-
 template <int TYPE>
 __device__ __forceinline__ float slice_dot_lds(uint32_t stage, int r, int s, int row_bytes,
                                                const float (&x)[64], const float (&sx)[4]) {
     const uint32_t row = stage + (uint32_t)(r * row_bytes);
-    if constexpr (TYPE == JL_Q6_K) {
+    if constexpr (TYPE == JL_Q5_K) {
+        // header, the 32 fifth-bit bytes, the 32 nibble bytes of pair s & 3 (super-blocks are 176
+        // bytes apart: everything is 16-byte aligned)
+        const uint32_t sb = row + (s >> 2) * 176;
+        uint4 h, g0, g1, q0, q1;
+        asm volatile(
+            "ds_read_b128 %0, %5\n\tds_read_b128 %1, %5 offset:16\n\tds_read_b128 %2, %5 offset:32\n\t"
+            "ds_read_b128 %3, %6\n\tds_read_b128 %4, %6 offset:16\n\ts_waitcnt lgkmcnt(0)"
+            : "=&v"(h), "=&v"(g0), "=&v"(g1), "=&v"(q0), "=&v"(q1) : "v"(sb), "v"(sb + 48 + (s & 3) * 32) : "memory");
+        const uint32_t qs[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        const uint32_t qh[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+        return slice_dot_q5_k(h, qs, qh, s & 3, x, sx);
+    } else if constexpr (TYPE == JL_Q6_K) {
+        // Super-blocks are 210 bytes apart, so every other one starts two bytes off a dword.  The
+        // LDS serves such reads, but at a fraction of its rate (measured: 40 % of the kernel's
+        // time): the quarter is read as aligned dwords from two bytes before where that is needed
+        // and each dword put together from its two neighbours with a funnel shift of 0 or 16 bits.
         const uint32_t sb = row + (s >> 2) * 210;
         const int h = (s >> 1) & 1;
-        uint32_t ql[16], qh[8], scales, d;
-        lds_read_q6k(sb + 64 * h, sb + 128 + 32 * h, sb + 192 + 4 * (s & 3), sb + 208, ql, qh, scales, d);
+        const uint32_t off = sb & 2u, shift = off * 8;
+        uint32_t wl[17], wh[9], ql[16], qh[8];
+        lds_read_17(sb - off + 64 * h, wl);
+        lds_read_9(sb - off + 128 + 32 * h, wh);
+        uint2 sc2;
+        uint32_t d;
+        asm volatile("ds_read2_b32 %0, %2 offset0:0 offset1:1\n\tds_read_u16 %1, %3\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(sc2), "=&v"(d) : "v"(sb - off + 192 + 4 * (s & 3)), "v"(sb + 208) : "memory");
+#pragma unroll
+        for (int i = 0; i < 16; i++) ql[i] = __builtin_amdgcn_alignbit(wl[i + 1], wl[i], shift);
+#pragma unroll
+        for (int i = 0; i < 8; i++) qh[i] = __builtin_amdgcn_alignbit(wh[i + 1], wh[i], shift);
+        const uint32_t scales = __builtin_amdgcn_alignbit(sc2.y, sc2.x, shift);
         return slice_dot_q6_k(ql, qh, scales, d, s & 1, x, sx);
     } else if constexpr (TYPE == JL_Q8_0) {
         uint32_t w[17];
@@ -558,7 +595,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
     constexpr int L = X4 + Traits<TYPE>::kTail;   // plus (three main types) one 4-byte load
     constexpr int SLICE = X4 * 16 + 4 * Traits<TYPE>::kTail;   // bytes of a tile one thread brings in
-    constexpr bool kExactDma = TYPE != JL_Q6_K;   // a thread's loads are exactly its slice
+    constexpr bool kExactDma = TYPE != JL_Q6_K && TYPE != JL_Q5_K;   // a thread's loads are exactly its slice
 
     const int tid = threadIdx.x;
     const int nthreads = LEAN ? THREADS : (int)blockDim.x;
@@ -830,7 +867,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
                 sx[2] += x[32 + k];
                 sx[3] += x[48 + k];
             }
-        } else if constexpr (TYPE != JL_Q8_0) {
+        } else if constexpr (TYPE != JL_Q8_0) {   // Q4_0, Q4_K, Q5_K: by 32
 #pragma unroll
             for (int k = 0; k < 32; k++) {
                 sx[0] += x[k];
@@ -1099,7 +1136,7 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
 template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, bool fixed) {
     // (Q6_K: plain, residual and gate/up only -- the caller has refused the rest)
-    constexpr bool kMain = TYPE != JL_Q6_K;
+    constexpr bool kMain = TYPE != JL_Q6_K && TYPE != JL_Q5_K;
     if constexpr (kMain) {
         if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
     }
@@ -1175,12 +1212,14 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
             return jl_fail(JL_ERR_UNSUPPORTED, "no fused q|k|v or RMS-folding single-token kernel for a %s weight "
                                                "(plain, residual and gate/up projections only)", jl_type_name(type));
         }
-        // Q6_K goes on to the tile kernel when the shape allows, the rest have the one-wave-per-row kernels
-        if (type != JL_Q6_K) return jl_launch_gemv_direct(ctx, w[0], w_up, x, outs[0], epilogue);
+        // Q6_K and Q5_K go on to the tile kernel when the shape allows, the rest have the
+        // one-wave-per-row kernels
+        if (type != JL_Q6_K && type != JL_Q5_K) return jl_launch_gemv_direct(ctx, w[0], w_up, x, outs[0], epilogue);
     }
 
     const bool dual = w_up != nullptr;
-    const int slice = type == JL_Q8_0 ? 68 : type == JL_Q6_K ? 64 : 36;   // bytes a thread brings in per tile
+    // bytes a thread brings in per tile
+    const int slice = type == JL_Q8_0 ? 68 : type == JL_Q6_K ? 64 : type == JL_Q5_K ? 48 : 36;
     bool fast = (n % 64 == 0) && (n / 64 <= 256) &&
                 (xq ? (((uintptr_t)xq->quants & 15) == 0 && ((uintptr_t)xq->scales & 7) == 0 &&
                        ((uintptr_t)xq->sums & 7) == 0)
@@ -1220,11 +1259,11 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     if (rms && ((uintptr_t)rms->weights & 15) != 0) {
         return jl_fail(JL_ERR_UNSUPPORTED, "the RMS weights must be 16-byte aligned");
     }
-    if (type == JL_Q6_K) {
-        // measured: the tile kernel overtakes the one-wave-per-row kernel at about 32 MB of weights
-        // (vocabulary and 8B-model feed-forward projections); below that its fixed costs lose
-        constexpr int64_t kTileFromBytes = (int64_t)32 << 20;
-        if (!fast || w[0]->bytes * (dual ? 2 : 1) < kTileFromBytes)
+    if (type == JL_Q6_K || type == JL_Q5_K) {
+        // measured: the tile kernel is the faster one from rows of 2048 columns and 2 MB of weights
+        // (by up to 1.7 x on the vocabulary and feed-forward projections); below that the two are
+        // within a few tenths of a microsecond of each other and the one-wave-per-row kernel stays
+        if (!fast || n < 2048 || w[0]->bytes * (dual ? 2 : 1) < ((int64_t)2 << 20))
             return jl_launch_gemv_direct(ctx, w[0], w_up, x, outs[0], epilogue);
     }
     if (!fast) {
@@ -1292,6 +1331,9 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
         case JL_Q6_K:
             return dual ? launch_tiles<JL_Q6_K, true>(ctx, p, threads, lds, fixed)
                         : launch_tiles<JL_Q6_K, false>(ctx, p, threads, lds, fixed);
+        case JL_Q5_K:
+            return dual ? launch_tiles<JL_Q5_K, true>(ctx, p, threads, lds, fixed)
+                        : launch_tiles<JL_Q5_K, false>(ctx, p, threads, lds, fixed);
         default:
             return jl_fail(JL_ERR_UNSUPPORTED,
                            "no single-token projection kernel for a ggml type %d weight", type);
