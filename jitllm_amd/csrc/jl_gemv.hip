@@ -69,10 +69,20 @@ template <> struct Traits<JL_Q4_0> { static constexpr int kX4 = 2, kTail = 1; };
 template <> struct Traits<JL_Q4_K> { static constexpr int kX4 = 2, kTail = 1; };  // 144 B / 4 = 36 B
 template <> struct Traits<JL_Q6_K> { static constexpr int kX4 = 4, kTail = 0; };  // 64 B >= 210 B / 4
 template <> struct Traits<JL_Q5_K> { static constexpr int kX4 = 3, kTail = 0; };  // 48 B >= 176 B / 4
+template <> struct Traits<JL_Q4_1> { static constexpr int kX4 = 3, kTail = 0; };  // 48 B >= 2 x 20 B
+template <> struct Traits<JL_Q5_0> { static constexpr int kX4 = 3, kTail = 0; };  // 48 B >= 2 x 22 B
+template <> struct Traits<JL_IQ4_XS> { static constexpr int kX4 = 3, kTail = 0; };  // 48 B >= 136 B / 4
+// the three types every entry point exists for; the others have the plain, residual and gate/up forms
+constexpr bool is_main_type(int type) { return type == JL_Q8_0 || type == JL_Q4_0 || type == JL_Q4_K; }
+// the others the tile kernel takes
+constexpr bool is_side_type(int type) {
+    return type == JL_Q6_K || type == JL_Q5_K || type == JL_Q4_1 || type == JL_Q5_0 || type == JL_IQ4_XS;
+}
 // bytes of a row of `slices` 64-column slices
 template <int TYPE>
 __device__ __host__ constexpr int row_bytes_of(int slices) {
-    return TYPE == JL_Q8_0 ? slices * 68 : TYPE == JL_Q6_K ? slices / 4 * 210 : TYPE == JL_Q5_K ? slices * 44 : slices * 36;
+    return TYPE == JL_Q8_0 ? slices * 68 : TYPE == JL_Q6_K ? slices / 4 * 210 : TYPE == JL_Q5_K ? slices * 44
+           : TYPE == JL_Q4_1 ? slices * 40 : TYPE == JL_Q5_0 ? slices * 44 : TYPE == JL_IQ4_XS ? slices * 34 : slices * 36;
 }
 
 __device__ __forceinline__ float ubyte(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
@@ -227,6 +237,84 @@ __device__ __forceinline__ float slice_dot_q6_k(const uint32_t (&ql)[16], const 
         acc = fmaf(sc, fmaf(-32.f * kTwoM24, sx[g], a[g]), acc);
     }
     return acc * d;
+}
+
+// Dot of one Q4_1 block pair (40 bytes: fp16 d, m | 16 nibble bytes, twice;
+// J/tensor/standard/Q4_1FloatTensor.java:73-94) with 64 activations: w = d q + m, so
+// sum(w x) = d sum(q x) + m sum(x) per block.  Element i < 16 of a block is the low nibble of its
+// byte i, element 16 + i the high nibble.
+__device__ __forceinline__ float slice_dot_q4_1(const uint32_t (&dw)[10], const float (&x)[64],
+                                                const float (&sx)[4]) {
+    float acc = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+        const float d = jl_half_bits_to_float(dw[5 * blk]), m = jl_half_bits_to_float(dw[5 * blk] >> 16);
+        float lo = 0.f, hi = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const NibblePairs n = nibble_pairs(dw[5 * blk + 1 + j]);
+#pragma unroll
+            for (int b = 0; b < 4; b++) mix_byte(n, b, x[32 * blk + 4 * j + b], x[32 * blk + 16 + 4 * j + b], lo, hi);
+        }
+        acc = fmaf(d * kTwo24, fmaf(hi, 0.0625f, lo), fmaf(m, sx[blk], acc));
+    }
+    return acc;
+}
+
+// Dot of one Q5_0 block pair (44 bytes: fp16 d | 32 fifth bits | 16 nibble bytes, twice;
+// J/tensor/standard/Q5_0FloatTensor.java:61-85) with 64 activations: w = d (q - 16), q the nibble
+// with its fifth bit on top; bit i of the 32 belongs to element i.  `qh`, `qs`: the fifth bits and
+// the four nibble dwords of block A, then of block B.
+__device__ __forceinline__ float slice_dot_q5_0(uint32_t dA, uint32_t dB, const uint32_t (&qh)[2],
+                                                const uint32_t (&qs)[8], const float (&x)[64],
+                                                const float (&sx)[4]) {
+    float acc = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+        float lo = 0.f, hi = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t q = qs[4 * blk + j];
+            // elements 4 j .. 4 j + 3 (low nibbles, fifth bits 4 j ..) and 16 + 4 j .. (high nibbles)
+            const uint32_t v0 = (q & 0x0F0F0F0Fu) | (jl_spread4(qh[blk] >> (4 * j)) << 4);
+            const uint32_t v1 = ((q >> 4) & 0x0F0F0F0Fu) | (jl_spread4(qh[blk] >> (16 + 4 * j)) << 4);
+            mix_bytes4(lo, v0, x[32 * blk + 4 * j], x[32 * blk + 4 * j + 1], x[32 * blk + 4 * j + 2], x[32 * blk + 4 * j + 3]);
+            mix_bytes4(hi, v1, x[32 * blk + 16 + 4 * j], x[32 * blk + 16 + 4 * j + 1], x[32 * blk + 16 + 4 * j + 2],
+                       x[32 * blk + 16 + 4 * j + 3]);
+        }
+        const float d = jl_half_bits_to_float(blk ? dB : dA);
+        acc = fmaf(d * kTwo24, fmaf(-16.f * kTwoM24, sx[blk], lo + hi), acc);
+    }
+    return acc;
+}
+
+// Dot of a quarter of an IQ4_XS super-block (fp16 d | scales_h | scales_l[4] | qs[128];
+// J/tensor/standard/IQ4_XSFloatTensor.java:72-100) with 64 activations: sub-blocks 2 q and 2 q + 1,
+// w = d (ls - 32) kvalues_iq4nl[nibble] with a 6-bit ls per sub-block; the 16 nibble bytes of a
+// sub-block hold elements 0..15 in their low halves and 16..31 in their high halves.  The table is
+// used with 128 added (bytes 1..241), which comes off through the activations' sums.
+__device__ __forceinline__ float slice_dot_iq4_xs(uint2 hdr, const uint32_t (&qs)[8], int q, const float (&x)[64],
+                                                  const float (&sx)[4]) {
+    const float d = jl_half_bits_to_float(hdr.x);
+    const uint32_t scales_h = hdr.x >> 16, scales_l = hdr.y;
+    float acc = 0.f;
+#pragma unroll
+    for (int sub = 0; sub < 2; sub++) {
+        const int g = 2 * q + sub;
+        const int ls = (int)(((scales_l >> (4 * g)) & 0xFu) | (((scales_h >> (2 * g)) & 3u) << 4));
+        float lo = 0.f, hi = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t w = qs[4 * sub + j];
+            const uint32_t v0 = jl_iq4nl_lookup4(w & 0x0F0F0F0Fu) ^ 0x80808080u;
+            const uint32_t v1 = jl_iq4nl_lookup4((w >> 4) & 0x0F0F0F0Fu) ^ 0x80808080u;
+            mix_bytes4(lo, v0, x[32 * sub + 4 * j], x[32 * sub + 4 * j + 1], x[32 * sub + 4 * j + 2], x[32 * sub + 4 * j + 3]);
+            mix_bytes4(hi, v1, x[32 * sub + 16 + 4 * j], x[32 * sub + 16 + 4 * j + 1], x[32 * sub + 16 + 4 * j + 2],
+                       x[32 * sub + 16 + 4 * j + 3]);
+        }
+        acc = fmaf((d * (float)(ls - 32)) * kTwo24, fmaf(-128.f * kTwoM24, sx[sub], lo + hi), acc);
+    }
+    return acc;
 }
 
 // Dot of a quarter of a Q5_K super-block (fp16 d, dmin | 12 packed scale / min bytes | qh[32] |
@@ -384,6 +472,13 @@ __device__ __forceinline__ void wait_vm_tiles(int tiles) {
     }
 }
 
+// two consecutive dwords from a four-byte aligned address
+__device__ __forceinline__ uint2 lds_read_b64(uint32_t addr) {
+    uint2 v;
+    asm volatile("ds_read2_b32 %0, %1 offset0:0 offset1:1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+    return v;
+}
+
 __device__ __forceinline__ uint32_t lds_read_b32(uint32_t addr) {
     uint32_t v;
     asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
@@ -461,7 +556,44 @@ template <int TYPE>
 __device__ __forceinline__ float slice_dot_lds(uint32_t stage, int r, int s, int row_bytes,
                                                const float (&x)[64], const float (&sx)[4]) {
     const uint32_t row = stage + (uint32_t)(r * row_bytes);
-    if constexpr (TYPE == JL_Q5_K) {
+    if constexpr (TYPE == JL_IQ4_XS) {
+        // the 8-byte header and the 32 nibble bytes of quarter s & 3 (super-blocks are 136 bytes
+        // apart: everything is 8-byte aligned)
+        const uint32_t sb = row + (s >> 2) * 136;
+        uint2 hdr, a, b, c, e;
+        asm volatile(
+            "ds_read_b64 %0, %5\n\tds_read_b64 %1, %6\n\tds_read_b64 %2, %6 offset:8\n\t"
+            "ds_read_b64 %3, %6 offset:16\n\tds_read_b64 %4, %6 offset:24\n\ts_waitcnt lgkmcnt(0)"
+            : "=&v"(hdr), "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(e) : "v"(sb), "v"(sb + 8 + (s & 3) * 32) : "memory");
+        const uint32_t qs[8] = {a.x, a.y, b.x, b.y, c.x, c.y, e.x, e.y};
+        return slice_dot_iq4_xs(hdr, qs, s & 3, x, sx);
+    } else if constexpr (TYPE == JL_Q4_1) {
+        // ten dwords, four-byte aligned (blocks are 20 bytes)
+        uint32_t w9[9], w[10];
+        lds_read_9(row + s * 40, w9);
+        w[9] = lds_read_b32(row + s * 40 + 36);
+#pragma unroll
+        for (int i = 0; i < 9; i++) w[i] = w9[i];
+        return slice_dot_q4_1(w, x, sx);
+    } else if constexpr (TYPE == JL_Q5_0) {
+        // eleven dwords from a four-byte aligned start (a pair of 22-byte blocks is 44 bytes); block
+        // A's fields sit two bytes off the dwords: d | qh lo, qh hi | qs .., block B's on them
+        uint32_t w9[9], w[11];
+        lds_read_9(row + s * 44, w9);
+        const uint2 t = lds_read_b64(row + s * 44 + 36);
+#pragma unroll
+        for (int i = 0; i < 9; i++) w[i] = w9[i];
+        w[9] = t.x;
+        w[10] = t.y;
+        const uint32_t qh[2] = {__builtin_amdgcn_alignbit(w[1], w[0], 16), w[6]};
+        uint32_t qs[8];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            qs[j] = __builtin_amdgcn_alignbit(w[2 + j], w[1 + j], 16);
+            qs[4 + j] = w[7 + j];
+        }
+        return slice_dot_q5_0(w[0], w[5] >> 16, qh, qs, x, sx);
+    } else if constexpr (TYPE == JL_Q5_K) {
         // header, the 32 fifth-bit bytes, the 32 nibble bytes of pair s & 3 (super-blocks are 176
         // bytes apart: everything is 16-byte aligned)
         const uint32_t sb = row + (s >> 2) * 176;
@@ -595,7 +727,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
     constexpr int L = X4 + Traits<TYPE>::kTail;   // plus (three main types) one 4-byte load
     constexpr int SLICE = X4 * 16 + 4 * Traits<TYPE>::kTail;   // bytes of a tile one thread brings in
-    constexpr bool kExactDma = TYPE != JL_Q6_K && TYPE != JL_Q5_K;   // a thread's loads are exactly its slice
+    constexpr bool kExactDma = is_main_type(TYPE);   // a thread's loads are exactly its slice
 
     const int tid = threadIdx.x;
     const int nthreads = LEAN ? THREADS : (int)blockDim.x;
@@ -751,8 +883,11 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
             const int q = base / 16 + tid;
             const int sl = q / 17, k = q - sl * 17;
             const int off = (sl < S && k < 16) ? (sl * 64 + k * 4) * 4 : 0;
-            __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.x + off),
-                                             (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
+            // (the side types' vector region, where it is one of its own, ends with the vector's last
+            // slot -- their 1024-thread form fits the LDS only so -- and nothing is written past it)
+            if (kExactDma || x_in_ring || q < x_slots)
+                __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.x + off),
+                                                 (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
         }
     }
     GSTAMP(2);
@@ -1077,10 +1212,10 @@ jl_gemv_generic(const uint8_t *__restrict__ w, const uint8_t *__restrict__ w_up,
 
 // LDS of a workgroup of `threads`: partial sums, the tile ring, and the staged activation vector
 // where it is larger than a ring stage.
-int tile_lds_bytes(int threads, int slice, int S) {
+int tile_lds_bytes(int threads, int slice, int S, bool exact_vector_region = false) {
     const int stage_bytes = threads * slice;
     const int x_bytes = (S * 17 + threads - 1) / threads * threads * 16;  // 17 slots per slice
-    const int x_extra = x_bytes <= stage_bytes ? 0 : x_bytes;
+    const int x_extra = x_bytes <= stage_bytes ? 0 : exact_vector_region ? S * 17 * 16 : x_bytes;
     return kPartialBytes + kStages * stage_bytes + x_extra;
 }
 
@@ -1136,7 +1271,7 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
 template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, bool fixed) {
     // (Q6_K: plain, residual and gate/up only -- the caller has refused the rest)
-    constexpr bool kMain = TYPE != JL_Q6_K && TYPE != JL_Q5_K;
+    constexpr bool kMain = is_main_type(TYPE);
     if constexpr (kMain) {
         if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
     }
@@ -1214,12 +1349,12 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
         }
         // Q6_K and Q5_K go on to the tile kernel when the shape allows, the rest have the
         // one-wave-per-row kernels
-        if (type != JL_Q6_K && type != JL_Q5_K) return jl_launch_gemv_direct(ctx, w[0], w_up, x, outs[0], epilogue);
+        if (!is_side_type(type)) return jl_launch_gemv_direct(ctx, w[0], w_up, x, outs[0], epilogue);
     }
 
     const bool dual = w_up != nullptr;
     // bytes a thread brings in per tile
-    const int slice = type == JL_Q8_0 ? 68 : type == JL_Q6_K ? 64 : type == JL_Q5_K ? 48 : 36;
+    const int slice = type == JL_Q8_0 ? 68 : type == JL_Q6_K ? 64 : is_side_type(type) ? 48 : 36;
     bool fast = (n % 64 == 0) && (n / 64 <= 256) &&
                 (xq ? (((uintptr_t)xq->quants & 15) == 0 && ((uintptr_t)xq->scales & 7) == 0 &&
                        ((uintptr_t)xq->sums & 7) == 0)
@@ -1232,7 +1367,7 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
         // it, at one workgroup per compute unit for the LDS that takes.  Sixteen waves share the
         // staged vector instead (plain and residual projections; the other variants keep 256).
         // (when its LDS fits: Q8_0 rows of more than 15 360 columns do not)
-        const bool wide = Sp == 256 && !dual && !rms && !xq && tile_lds_bytes(kWideThreads, slice, S) <= 160 * 1024;
+        const bool wide = Sp == 256 && !dual && !rms && !xq && tile_lds_bytes(kWideThreads, slice, S, is_side_type(type)) <= 160 * 1024;
         R = (wide ? kWideThreads : 256) / Sp;
         half_rows = dual ? R / 2 : R;
         if (half_rows < 1) fast = false;
@@ -1259,7 +1394,7 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     if (rms && ((uintptr_t)rms->weights & 15) != 0) {
         return jl_fail(JL_ERR_UNSUPPORTED, "the RMS weights must be 16-byte aligned");
     }
-    if (type == JL_Q6_K || type == JL_Q5_K) {
+    if (is_side_type(type)) {
         // measured: the tile kernel is the faster one from rows of 2048 columns and 2 MB of weights
         // (by up to 1.7 x on the vocabulary and feed-forward projections); below that the two are
         // within a few tenths of a microsecond of each other and the one-wave-per-row kernel stays
@@ -1313,7 +1448,7 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     }
 
     const int threads = (R * Sp + 63) / 64 * 64;
-    const int lds = tile_lds_bytes(threads, slice, S);
+    const int lds = tile_lds_bytes(threads, slice, S, is_side_type(type));
     // (whole tiles only; `full`: rows of exactly Sp slices as well)
     bool fixed = R * Sp == threads;
     for (int i = 0; i < nseg; i++) fixed = fixed && w[i]->rows % half_rows == 0;
@@ -1334,6 +1469,15 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
         case JL_Q5_K:
             return dual ? launch_tiles<JL_Q5_K, true>(ctx, p, threads, lds, fixed)
                         : launch_tiles<JL_Q5_K, false>(ctx, p, threads, lds, fixed);
+        case JL_Q4_1:
+            return dual ? launch_tiles<JL_Q4_1, true>(ctx, p, threads, lds, fixed)
+                        : launch_tiles<JL_Q4_1, false>(ctx, p, threads, lds, fixed);
+        case JL_Q5_0:
+            return dual ? launch_tiles<JL_Q5_0, true>(ctx, p, threads, lds, fixed)
+                        : launch_tiles<JL_Q5_0, false>(ctx, p, threads, lds, fixed);
+        case JL_IQ4_XS:
+            return dual ? launch_tiles<JL_IQ4_XS, true>(ctx, p, threads, lds, fixed)
+                        : launch_tiles<JL_IQ4_XS, false>(ctx, p, threads, lds, fixed);
         default:
             return jl_fail(JL_ERR_UNSUPPORTED,
                            "no single-token projection kernel for a ggml type %d weight", type);

@@ -316,14 +316,15 @@ def test_k_quant_decode_bit_exact(ctx, t):
         assert bits_equal(w.dequantize(), O.dequant(t, raw))
 
 
-@pytest.mark.parametrize("t", [O.Q6_K, O.Q5_K])
+@pytest.mark.parametrize("t", [O.Q6_K, O.Q5_K, O.Q4_1, O.Q5_0, O.IQ4_XS])
 @pytest.mark.parametrize("d,n,dual", [(4096, 14336, False), (4099, 11008, False), (10001, 4096, False),
                                       (21000, 2048, False), (4800, 8192, False), (803, 3072, False),
                                       (6144, 4096, True), (5001, 4096, True), (10000, 2048, True)])
 def test_k_quants_on_the_tile_kernel(ctx, t, d, n, dual):
-    """Q6_K weights with rows of 2048 columns and more run the tile kernel (LDS-DMA ring, 52.5-byte
-    slices that start two bytes off a dword in every other super-block): whole and ragged tiles,
-    rows that do not fill their slices, 1024-thread workgroups, plain / residual / gate-up."""
+    """Q6_K, Q5_K, Q4_1 and Q5_0 weights with rows of 2048 columns and more run the tile kernel
+    (LDS-DMA ring; slices of 52.5, 44, 40 and 44 bytes read wherever they fall in the row): whole
+    and ragged tiles, rows that do not fill their slices, 1024-thread workgroups, plain / residual /
+    gate-up."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
     say("k-quant tile kernel", KQ_NAMES[t], d, n, dual)
