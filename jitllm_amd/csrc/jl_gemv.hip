@@ -890,31 +890,35 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
                                                  (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
         }
     }
+    // RMS normalisation folded into the activation load.  CpuOperations.rmsnorm
+    // (J/inference/op/CpuOperations.java:60-72): out = w * (ss * x) with
+    // ss = (float)(1 / sqrt(sum x^2 / n + eps)); the reference's fused kernels fold the same
+    // product into their activation reads (TransformerComputeKernelsLayered.java:2168-2171).
+    // The workgroup reads x and the weights with coalesced 16-byte loads and leaves the
+    // product in the LDS region the plain path fills with x, so everything after is shared
+    // and the LDS footprint (workgroups per compute unit) is that of the plain path.
+    const int nvec = rms ? p.n / 4 : 0;
+    const float4 *xv = (const float4 *)p.x, *wv = (const float4 *)p.rms_w;
+    // rows of up to 4 x 4 x nthreads columns are read once and held in registers from the
+    // sum of squares to the product; longer ones are read again for the product
+    const bool held = nvec <= nthreads * 4;
+    float4 v[4], w[4];
+    auto load = [&](int base) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = base + j * nthreads + tid;
+            v[j] = i < nvec ? xv[i] : float4{0.f, 0.f, 0.f, 0.f};
+            w[j] = i < nvec ? wv[i] : float4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    // (these loads go out before the first tile's: a wait for them then leaves the tile in flight
+    // while the sum of squares and the products are computed, instead of waiting for it as well)
+    if constexpr (rms) {
+        if (held) load(0);
+    }
     GSTAMP(2);
     for (; issued < kStages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
     if constexpr (rms) {
-        // RMS normalisation folded into the activation load.  CpuOperations.rmsnorm
-        // (J/inference/op/CpuOperations.java:60-72): out = w * (ss * x) with
-        // ss = (float)(1 / sqrt(sum x^2 / n + eps)); the reference's fused kernels fold the same
-        // product into their activation reads (TransformerComputeKernelsLayered.java:2168-2171).
-        // The workgroup reads x and the weights with coalesced 16-byte loads and leaves the
-        // product in the LDS region the plain path fills with x, so everything after is shared
-        // and the LDS footprint (workgroups per compute unit) is that of the plain path.
-        const int nvec = p.n / 4;
-        const float4 *xv = (const float4 *)p.x, *wv = (const float4 *)p.rms_w;
-        // rows of up to 4 x 4 x nthreads columns are read once and held in registers from the
-        // sum of squares to the product; longer ones are read again for the product
-        const bool held = nvec <= nthreads * 4;
-        float4 v[4], w[4];
-        auto load = [&](int base) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int i = base + j * nthreads + tid;
-                v[j] = i < nvec ? xv[i] : float4{0.f, 0.f, 0.f, 0.f};
-                w[j] = i < nvec ? wv[i] : float4{0.f, 0.f, 0.f, 0.f};
-            }
-        };
-        if (held) load(0);
         float scale;
         if (p.rms_scale) {
             scale = *p.rms_scale;
