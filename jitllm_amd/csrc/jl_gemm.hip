@@ -896,13 +896,14 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     // many rows and enough tiles: weights decoded to fp16 once per call, then the plain fp16 GEMM
     int virt = 0;
     for (int i = 0; i < count; i++) virt += (int)weights[i]->rows;
-    int dsplits = 1;
-    int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits);
+    int dsplits = 1, bm = 256;
+    int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm);
     // A type without a decode-in-the-loop kernel (Q6_K) takes the decode-once path whatever the
     // shape: correct for any row count, tuned for none but prefill.
     const bool dense_only = !jl_has_fused_kernels(type);
     if (dense_only && bn == 0) {
         bn = 128;
+        bm = 256;
         dsplits = 1;
     }
     const size_t copy_bytes = round_up(jl_dense_copy_bytes(k, virt), 256);
@@ -942,7 +943,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     }
     if (dense) {
         const int st = jl_launch_gemm_dense(ctx, weights, count, A, row_scale, C, rows, ldo, col_offset, epilogue,
-                                            kept ? (_Float16 *)resident->copy : (_Float16 *)planes, decode, bn,
+                                            kept ? (_Float16 *)resident->copy : (_Float16 *)planes, decode, bm, bn,
                                             dsplits, (float *)((uint8_t *)planes + in_workspace), c_f16,
                                             ride_along ? X : nullptr, ride_along ? row_scale : nullptr);
         if (st == JL_OK && kept) *resident->state = layout;

@@ -9,9 +9,9 @@
 //
 //   jl_decode_to_f16   raw blocks -> [virtual rows x K] fp16, the host decode rounded once to fp16
 //                      (bit for bit what the fused kernel multiplies with); one launch per call
-//   jl_gemm_hh<BN>     C = A16 . W16^T on v_mfma_f32_16x16x32_f16, 256 x BN tiles in steps of 64
-//                      columns; eight waves that each bring in their share of both operands by
-//                      LDS-DMA, the two waves of a SIMD half a step apart
+//   jl_gemm_hh<BM, BN> C = A16 . W16^T on v_mfma_f32_16x16x32_f16, BM x BN tiles (256 x 256, 256 x 128,
+//                      128 x 128) in steps of 64 columns; eight waves that each bring in their
+//                      share of both operands by LDS-DMA, the two waves of a SIMD half a step apart
 #include "jl_device.h"
 #include "jl_internal.h"
 
@@ -244,42 +244,51 @@ struct DenseParams {
     int epilogue;
     int ntiles, mtiles;
     int splits;              // K is cut into `splits` equal runs of steps, one work item each
-    float *partial;          // splits > 1: [splits][mtiles * 256][ntiles * BN] fp32 partial sums
+    float *partial;          // splits > 1: [splits][mtiles * BM][ntiles * BN] fp32 partial sums
 };
 
-__device__ __forceinline__ float dense_swiglu(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
+__device__ __forceinline__ float dense_swiglu(float g, float u) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u; }
 
-constexpr int DBM = 256, DBK = 64;
+constexpr int DBK = 64;
+constexpr int kRowPad = 256;   // activation rows are padded to whole tiles of the largest row tile
 
 // hands fragment registers whose reads are complete back to the compiler
 template <int N>
 __device__ __forceinline__ void lds_settle(half8 (&f)[N]) {
     if constexpr (N == 8)
         asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]));
-    else
+    else if constexpr (N == 4)
         asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
+    else
+        asm volatile("" : "+v"(f[0]), "+v"(f[1]));
 }
 
 // LDS stage: A rows then W rows, 128 bytes (eight 16-byte chunks) per row; chunk c of row r sits
 // at position c ^ ((r >> 1) & 7) -- measured, this pairing of rows lets a 128-bit fragment read of
 // 16 rows x 4 chunks run at the full 256 bytes per clock.  A step is 64 columns = two MFMA
 // k-blocks: the second block's fragments are read while the first block's MFMAs run, one barrier
-// per step.  BN = 256: two stages of 64 KB (the next step's loads are issued right after the
-// barrier and have the whole step to land); BN = 128: three stages of 48 KB.
-template <int BN>
+// per step.  256 x 256: two stages of 64 KB (the next step's loads are issued right after the
+// barrier and have the whole step to land); 256 x 128: three stages of 48 KB; 128 x 128: four of
+// 32 KB -- the tile of calls too narrow to give every compute unit a larger one, which would
+// otherwise have to cut K across workgroups and pay for a fold.
+template <int BM, int BN> constexpr int hh_stages() { return BM + BN == 512 ? 2 : BM + BN == 384 ? 3 : 4; }
+
+template <int BM, int BN>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 jl_gemm_hh(DenseParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int DBM = BM;
     constexpr int WM = BN == 256 ? 2 : 4;     // waves along M
     constexpr int WN = 8 / WM;
-    constexpr int TM = DBM / WM, TN = BN / WN;   // wave tile: 128 x 64 or 64 x 64
+    constexpr int TM = DBM / WM, TN = BN / WN;   // wave tile: 128 x 64, 64 x 64 or 32 x 64
     constexpr int MB = TM / 16, NB = TN / 16;
     constexpr int STAGE = (DBM + BN) * 128;
-    constexpr int NS = BN == 256 ? 2 : 3;
+    constexpr int NS = hh_stages<BM, BN>();
     constexpr int AHEAD = NS - 1;
     constexpr int LA = DBM * 8 / 512;          // 16-byte loads per thread and stage, A part
     constexpr int LW = BN * 8 / 512;
     static_assert(NB == 4, "four column blocks per wave");
+    static_assert(BM == 256 || (BM == 128 && BN == 128), "row tiles: 256, or 128 with 128 columns");
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -324,7 +333,7 @@ jl_gemm_hh(DenseParams p) {
         const int logical = xcd * per_xcd + (item - split * per_xcd);
         if (logical >= total) continue;
         const int64_t kbytes = (int64_t)split * ksteps * (DBK * 2);   // first column of this run, in bytes
-        constexpr int GM = 2;
+        constexpr int GM = 4;
         const int group = logical / (GM * p.ntiles);
         const int rest = logical - group * (GM * p.ntiles);
         const int rows_in_group = p.mtiles - group * GM < GM ? p.mtiles - group * GM : GM;
@@ -401,7 +410,10 @@ jl_gemm_hh(DenseParams p) {
         };
         // stage s landed (this thread's part); the AHEAD - 1 younger stages may be in flight
         auto stage_ready = [&](int s) {
-            if (AHEAD == 2 && s + 1 < ksteps) JL_WAIT_VM(LA + LW);
+            const int left = ksteps - 1 - s;
+            const int younger = left < AHEAD - 1 ? left : AHEAD - 1;
+            if (younger >= 2) JL_WAIT_VM(2 * (LA + LW));
+            else if (younger == 1) JL_WAIT_VM(LA + LW);
             else JL_WAIT_VM(0);
             __builtin_amdgcn_s_barrier();
         };
@@ -414,7 +426,8 @@ jl_gemm_hh(DenseParams p) {
                 // LDS reads return in order: the first k-block's MB + NB fragments are back when
                 // that many of the second's are still outstanding
                 if constexpr (MB == 8) asm volatile("s_waitcnt lgkmcnt(12)" ::: "memory");
-                else asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+                else if constexpr (MB == 4) asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+                else asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory");
                 lds_settle(fa[0]);
                 lds_settle(fb[0]);
                 mfma_block(0, more, s + AHEAD);
@@ -521,10 +534,10 @@ jl_gemm_hh(DenseParams p) {
     }
 }
 
-template <int BN>
+template <int BM, int BN>
 int launch_dense(jl_context *ctx, const DenseParams &p) {
-    auto fn = jl_gemm_hh<BN>;
-    constexpr int lds = (BN == 256 ? 2 : 3) * (DBM + BN) * 128;
+    auto fn = jl_gemm_hh<BM, BN>;
+    constexpr int lds = hh_stages<BM, BN>() * (BM + BN) * 128;
     static bool configured[16] = {};
     if (ctx->device < 16 && !configured[ctx->device]) {
         JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -549,34 +562,38 @@ int launch_decode(jl_context *ctx, const DecodeParams &d, int activation_rows) {
 
 }  // namespace
 
-// Column tile the dense path would use for a call, 0 when the call is not one for it: it takes
-// 512 rows or more and enough work items to give most compute units one.  Narrow projections
-// get there by cutting K into 2, 4 or 8 runs of at least four steps (plain store / residual only);
-// what is still too small keeps the decode-in-the-loop kernel, whose 128-row tiles fill the chip
-// better.
-int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits) {
+// Column tile the dense path would use for a call (and in *row_tile the row tile), 0 when the call
+// is not one for it: it takes 512 rows or more and enough work items to give most compute units
+// one.  The largest tile that does so wins: 256 x 256, 256 x 128, then 128 x 128; narrow
+// projections on few rows get there by cutting K into 2, 4 or 8 runs of at least four steps as well
+// (plain store / residual only); what is still too small keeps the decode-in-the-loop kernel.
+int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits,
+                         int *row_tile) {
     *splits = 1;
+    *row_tile = 256;
     if (rows < 512 || k % 64 != 0) return 0;
-    const int mtiles = (rows + DBM - 1) / DBM;
+    const int mtiles = (rows + 255) / 256;
     // 256-wide tiles when they still give every compute unit work, else 128-wide ones
     if ((int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units) return 256;
     const int64_t items = (int64_t)mtiles * ((out_cols_virtual + 127) / 128);
     if (items * 10 >= (int64_t)compute_units * 7) return 128;
-    if (epilogue != JL_SWIGLU) {
-        for (int s = 2; s <= 8; s *= 2) {
-            if ((k / DBK) % s != 0 || k / s < 4 * DBK) break;
-            if (items * s * 10 >= (int64_t)compute_units * 7) {
-                *splits = s;
-                return 128;
-            }
+    const int64_t small = (int64_t)((rows + 127) / 128) * ((out_cols_virtual + 127) / 128);
+    for (int s = 1; s <= 8; s *= 2) {
+        if (s > 1 && epilogue == JL_SWIGLU) break;
+        if ((k / DBK) % s != 0 || k / s < 4 * DBK) break;
+        if (small * s * 10 >= (int64_t)compute_units * 7) {
+            *splits = s;
+            *row_tile = 128;
+            return 128;
         }
     }
     return 0;
 }
 
-// Bytes of the partial-sum planes of a call that cuts K into `splits` runs.
+// Bytes of the partial-sum planes of a call that cuts K into `splits` runs (an upper bound: rows
+// padded to the largest row tile).
 size_t jl_dense_plane_bytes(int rows, int out_cols_virtual, int splits) {
-    return (size_t)splits * (size_t)((rows + DBM - 1) / DBM * DBM) * (size_t)((out_cols_virtual + 127) / 128 * 128) * sizeof(float);
+    return (size_t)splits * (size_t)((rows + kRowPad - 1) / kRowPad * kRowPad) * (size_t)((out_cols_virtual + 127) / 128 * 128) * sizeof(float);
 }
 
 // Bytes of the decoded copy for `out_cols_virtual` weight rows of `k` columns.
@@ -586,7 +603,7 @@ size_t jl_dense_copy_bytes(int k, int out_cols_virtual) {
 
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
-                         int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes,
+                         int epilogue, _Float16 *copy, bool decode, int bm, int bn, int splits, float *planes,
                          bool c_f16, const float *X32, float *row_scale_out) {
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
@@ -620,7 +637,7 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
         d.A = const_cast<_Float16 *>(A);
         d.row_scale = row_scale_out;
         d.rows = rows;
-        xr = (rows + DBM - 1) / DBM * DBM;
+        xr = (rows + kRowPad - 1) / kRowPad * kRowPad;
     }
     int dst = JL_OK;
     if (decode) {
@@ -651,11 +668,14 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
     p.col_offset = col_offset;
     p.epilogue = epilogue;
     p.ntiles = ntiles;
-    p.mtiles = (rows + DBM - 1) / DBM;
+    p.mtiles = (rows + bm - 1) / bm;
     p.splits = splits;
     p.partial = planes;
-    const int st = bn == 256 ? launch_dense<256>(ctx, p) : launch_dense<128>(ctx, p);
+    if (!(bm == 256 || (bm == 128 && bn == 128)) || (bn != 128 && bn != 256))
+        return jl_fail(JL_ERR_INVALID, "jl_gemm: no %d x %d tile", bm, bn);
+    const int st = bn == 256 ? launch_dense<256, 256>(ctx, p)
+                 : bm == 256 ? launch_dense<256, 128>(ctx, p) : launch_dense<128, 128>(ctx, p);
     if (st != JL_OK || splits == 1) return st;
     return jl_launch_gemm_reduce(ctx, planes, row_scale, C, rows, n_total, ntiles,
-                                 (int64_t)p.mtiles * DBM * ntiles * 128, splits, ldo, col_offset, epilogue);
+                                 (int64_t)p.mtiles * bm * ntiles * 128, splits, ldo, col_offset, epilogue);
 }

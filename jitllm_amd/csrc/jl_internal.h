@@ -145,12 +145,13 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
                           float *C, int rows, int64_t ldo, int64_t col_offset, int epilogue,
                           float *planes, size_t plane_bytes, bool *taken);
 // Many-row prefill: weights decoded to fp16 once per call into `copy`, then a plain fp16 GEMM.
-int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits);
+int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits,
+                         int *row_tile);
 size_t jl_dense_copy_bytes(int k, int out_cols_virtual);
 size_t jl_dense_plane_bytes(int rows, int out_cols_virtual, int splits);
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
                          const float *row_scale, float *C, int rows, int64_t ldo, int64_t col_offset,
-                         int epilogue, _Float16 *copy, bool decode, int bn, int splits, float *planes,
+                         int epilogue, _Float16 *copy, bool decode, int bm, int bn, int splits, float *planes,
                          bool c_f16 = false, const float *X32 = nullptr, float *row_scale_out = nullptr);
 // Adds split-K planes [splits][rows padded][ntiles * 128] in split order and applies the epilogue.
 int jl_launch_gemm_reduce(jl_context *ctx, const float *planes, const float *row_scale, float *C, int rows,
