@@ -775,29 +775,33 @@ def decode_probe(ctx, proj, layers, wcls, acts):
                                        "other_types": {"layers": 5, "rounds": 4}}}))
 
 
-def prefill_probe(ctx, t, T=2048):
+def prefill_probe(ctx, t, T=2048, mode="xf16"):
     """What the matrix-pipe counters (`rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F16 SQ_VALU_MFMA_BUSY_CYCLES
-    SQ_BUSY_CU_CYCLES GRBM_GUI_ACTIVE`) are collected on: one Llama-3.2-1B layer's four prefill calls at
-    T tokens with the resident fp16 copy and fp16 activations (every call is then one launch of the
-    fp16 GEMM, plus a fold for o and down), launched kernel by kernel -- no graph, so that every
-    dispatch has a counter row of its own -- three times after one call that decodes the copy."""
+    SQ_BUSY_CU_CYCLES GRBM_GUI_ACTIVE`) and the prefill kernel traces are collected on: one
+    Llama-3.2-1B layer's four prefill calls at T tokens, launched kernel by kernel -- no graph, so that
+    every dispatch has a row of its own -- four times.  Mode "xf16": resident fp16 copy and fp16
+    activations (every call is then one launch of the fp16 GEMM, plus a fold where K is cut; the first
+    pass decodes the copy); "resident": the copy with fp32 activations; "default": plain `jl_gemm`."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
     shapes = {"wq": (DIM, DIM), "wk": (KV_DIM, DIM), "wv": (KV_DIM, DIM), "wo": (DIM, DIM),
               "w1": (HIDDEN, DIM), "w3": (HIDDEN, DIM), "w2": (DIM, HIDDEN)}
     w = {k: ctx.load_weight(t, synthetic.weight(t, r, c, 41 + i), r, c) for i, (k, (r, c)) in enumerate(shapes.items())}
-    X16 = ctx.half_from_numpy(synthetic.activations((T, DIM), 48))
-    H16 = ctx.half_from_numpy(synthetic.activations((T, HIDDEN), 49) * np.float32(0.1))
+    x_host = synthetic.activations((T, DIM), 48)
+    h_host = synthetic.activations((T, HIDDEN), 49) * np.float32(0.1)
     qkv, res = ctx.float_array(T * (DIM + 2 * KV_DIM)), ctx.float_array(T * DIM, fill=0.0)
-    hb16 = ctx.half_array(T * HIDDEN)
-    proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=True)
+    if mode == "xf16":
+        x, h, hb = ctx.half_from_numpy(x_host), ctx.half_from_numpy(h_host), ctx.half_array(T * HIDDEN)
+    else:
+        x, h, hb = ctx.from_numpy(x_host), ctx.from_numpy(h_host), ctx.float_array(T * HIDDEN)
+    proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=mode != "default")
     for _ in range(4):
-        proj.fusedQKV(X16, qkv, w["wq"], w["wk"], w["wv"])
-        proj.projection(X16, res, w["wo"], DIM, DIM, True)
-        proj.gateUp(X16, hb16, w["w1"], w["w3"], DIM, HIDDEN)
-        proj.projection(H16, res, w["w2"], HIDDEN, DIM, True)
+        proj.fusedQKV(x, qkv, w["wq"], w["wk"], w["wv"])
+        proj.projection(x, res, w["wo"], DIM, DIM, True)
+        proj.gateUp(x, hb, w["w1"], w["w3"], DIM, HIDDEN)
+        proj.projection(h, res, w["w2"], HIDDEN, DIM, True)
         ctx.sync()
-    print(json.dumps({"tokens": T, "flops": {"q|k|v": 2.0 * T * DIM * (DIM + 2 * KV_DIM), "o": 2.0 * T * DIM * DIM,
+    print(json.dumps({"tokens": T, "mode": mode, "flops": {"q|k|v": 2.0 * T * DIM * (DIM + 2 * KV_DIM), "o": 2.0 * T * DIM * DIM,
                                              "gate/up": 2.0 * T * 2 * HIDDEN * DIM, "down": 2.0 * T * HIDDEN * DIM},
                       "mfma_f16_flops_per_instruction_16x16x32": 2 * 16 * 16 * 32}))
 
@@ -868,6 +872,9 @@ def main():
                     help="only launch what the HBM-traffic counters are read on (see traffic_probe)")
     ap.add_argument("--prefill-probe", action="store_true",
                     help="only launch what the matrix-pipe counters are read on (see prefill_probe)")
+    ap.add_argument("--probe-tokens", type=int, default=2048, help="--prefill-probe: tokens")
+    ap.add_argument("--probe-mode", default="xf16", choices=["xf16", "resident", "default"],
+                    help="--prefill-probe: operand types and residency (see prefill_probe)")
     ap.add_argument("--batched-probe", action="store_true",
                     help="only launch the batched-decode calls, kernel by kernel (see batched_probe)")
     ap.add_argument("--decode-probe", action="store_true",
@@ -894,7 +901,7 @@ def main():
         cu, name = ctx.device_info()
         clock_khz = hip.clock_khz(0)
         if args.prefill_probe:
-            prefill_probe(ctx, t)
+            prefill_probe(ctx, t, args.probe_tokens, args.probe_mode)
             return
         if args.batched_probe:
             batched_probe(ctx)
