@@ -310,8 +310,12 @@ template <int TYPE> struct Loads { static constexpr int kPerWave = TYPE == JL_Q8
 
 // ZIN: spans of a row that one workgroup walks itself, one tile after the other, adding their
 // results in registers (it then holds ZIN sets of activation fragments); p.Z spans of ZIN each.
-template <int TYPE, int NBB, bool DUAL, int ZIN>
+// HALF: at most 8 activation rows -- the prologue reads, scales and converts rows 0..7 only (rows
+// 8..15 of the row block are zeros either way).
+template <int TYPE, int NBB, bool DUAL, int ZIN, bool HALF = false>
 __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_skinny(SkinnyParams p) {
+    static_assert(!HALF || NBB == 1, "a row block of at most 8 rows is the only one");
+    constexpr int XR = HALF ? 8 : 16;   // activation rows of a row block the prologue reads
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int LD = Loads<TYPE>::kPerWave;
     const int tid = threadIdx.x;
@@ -555,14 +559,14 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         // region of the wave's own: the last ring stage and the partial sums behind it, neither of
         // which anybody touches before the first tile has been multiplied.
         uint8_t *scr = lds + (p.stages - 1) * stage_bytes + wave * kScratchPerWave;
-        float4 x[NBB * ZIN][16];
+        float4 x[NBB * ZIN][XR];
 #pragma unroll
         for (int b = 0; b < NBB; b++) {
 #pragma unroll
             for (int q = 0; q < ZIN; q++) {
                 const float4 *src = (const float4 *)(p.X + 64 * ((z * ZIN + q) * p.Ss + 4 * wave)) + lane;
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
+                for (int r = 0; r < XR; r++) {
                     const int m = row0 + 16 * b + r;   // (uniform: a scalar branch)
                     if (m < p.rows) x[b * ZIN + q][r] = *(const float4 *)((const float *)src + (int64_t)m * p.k);
                     else x[b * ZIN + q][r] = float4{0.f, 0.f, 0.f, 0.f};
@@ -573,7 +577,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         for (int b = 0; b < NBB; b++) {
 #pragma unroll
             for (int q = 0; q < ZIN; q++) {
-                const float4 (&xs)[16] = x[b * ZIN + q];
+                const float4 (&xs)[XR] = x[b * ZIN + q];
                 // The largest magnitude of each row's 256 columns.  Sixteen registers of per-lane
                 // maxima are folded over the lanes and halved twice on the way (a swap of lane
                 // halves puts row r and row r + 8 side by side, a swap of lane quarters rows r and
@@ -581,7 +585,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                 // whose results its lanes will hold.
                 float v16[16];
 #pragma unroll
-                for (int r = 0; r < 16; r++) v16[r] = max_abs4(xs[r]);
+                for (int r = 0; r < 16; r++) v16[r] = r < XR ? max_abs4(xs[r]) : 0.f;
                 float v8[8], v4[4];
 #pragma unroll
                 for (int r = 0; r < 8; r++) {
@@ -610,16 +614,21 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                     E = E < 12 ? 12 : E;
                     undo[b][q][e] = __uint_as_float((uint32_t)(E - 9) << 23);
                 }
-                float inv[16];
+                float inv[XR];
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
+                for (int r = 0; r < XR; r++) {
                     const uint32_t bits = __builtin_amdgcn_readlane(__float_as_uint(v4[r & 3]), 16 * (r >> 2));
                     int E = (int)((bits >> 23) & 0xFF);
                     E = E < 12 ? 12 : E;
                     inv[r] = __uint_as_float((uint32_t)(263 - E) << 23);
                 }
+                if constexpr (HALF) {
+                    const _Float16 z16 = (_Float16)0.f;
 #pragma unroll
-                for (int pass = 0; pass < 2; pass++) {
+                    for (int i = 0; i < 8; i++) af[b][q][i] = half8{z16, z16, z16, z16, z16, z16, z16, z16};
+                }
+#pragma unroll
+                for (int pass = 0; pass < XR / 8; pass++) {
 #pragma unroll
                     for (int rr = 0; rr < 8; rr++) {
                         const int r = 8 * pass + rr;
@@ -785,9 +794,9 @@ __global__ void __launch_bounds__(256) jl_skinny_reduce(SkinnyParams p, int padd
 #else
 #define JL_PROBE_LDS 0
 #endif
-template <int TYPE, int NBB, bool DUAL, int ZIN>
+template <int TYPE, int NBB, bool DUAL, int ZIN, bool HALF = false>
 int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int groups) {
-    auto fn = jl_gemm_skinny<TYPE, NBB, DUAL, ZIN>;
+    auto fn = jl_gemm_skinny<TYPE, NBB, DUAL, ZIN, HALF>;
     static bool configured[16] = {};
     if (ctx->device < 16 && !configured[ctx->device]) {
         JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
@@ -814,6 +823,10 @@ int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int gro
 
 template <int TYPE, bool DUAL>
 int launch_nbb(jl_context *ctx, const SkinnyParams &p, int nbb, int zin, int threads, int lds, int groups) {
+    if (nbb == 1 && p.rows <= 8) {
+        return zin == 2 ? launch<TYPE, 1, DUAL, 2, true>(ctx, p, threads, lds, groups)
+                        : launch<TYPE, 1, DUAL, 1, true>(ctx, p, threads, lds, groups);
+    }
     if (nbb == 1) {
         return zin == 2 ? launch<TYPE, 1, DUAL, 2>(ctx, p, threads, lds, groups)
                         : launch<TYPE, 1, DUAL, 1>(ctx, p, threads, lds, groups);

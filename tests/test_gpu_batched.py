@@ -68,6 +68,38 @@ def test_batched_projection_matches_oracle(ctx, t, d, n, B):
     assert err < 2e-4, err  # random rounding errors: far inside the worst-case bound
 
 
+@pytest.mark.parametrize("t", [O.Q8_0, O.Q4_0, O.Q4_K])
+@pytest.mark.parametrize("d,n,rows", [(512, 4096, 8), (200, 2304, 5), (96, 12288, 1)])
+def test_calls_of_at_most_eight_rows_match_the_same_rows_of_a_larger_call(ctx, t, d, n, rows):
+    """Calls of at most 8 rows run an instance of the weight-streaming kernel whose prologue skips
+    rows 8..15 of the row block.  A row's scale, fragments and sums do not depend on the other rows
+    (FloatTensor.java:127-140: row b is a dot of its own), so the results must equal the first rows
+    of a 12-row call over the same activations bit for bit -- plain, residual and gate/up -- and
+    meet the oracle."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("at most eight rows", NAMES[t], d, n, rows)
+    raw = synthetic.weight(t, d, n, seed=7300 + d)
+    raw_up = synthetic.weight(t, d, n, seed=7301 + d)
+    X = synthetic.activations((12, n), seed=7302 + rows)
+    w, w_up = ctx.load_weight(t, raw, d, n), ctx.load_weight(t, raw_up, d, n)
+    big = QuantizedBatchProjections(ctx, 12, n, 2 * d)
+    small = QuantizedBatchProjections(ctx, rows, n, 2 * d)
+    xd, xs = ctx.from_numpy(X), ctx.from_numpy(X[:rows])
+    results = []
+    for proj, x, b in ((big, xd, 12), (small, xs, rows)):
+        plain, res, hb = ctx.float_array(b * d), ctx.float_array(b * d, fill=1.5), ctx.float_array(b * d)
+        proj.projection(x, plain, w, n, d, False)
+        proj.projection(x, res, w, n, d, True)
+        proj.gateUp(x, hb, w, w_up, n, d)
+        ctx.sync()
+        results.append([a.get().reshape(b, d)[:rows] for a in (plain, res, hb)])
+    for a, b in zip(*results):
+        assert np.array_equal(a, b)
+    ref = O.matmul_batch(t, raw, X[:rows], d, n, O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256)
+    assert rel_err(results[1][0], ref, magnitude(t, raw, X[:rows], d, n)) < 2e-4
+
+
 def test_batched_row_is_the_single_vector_result(ctx):
     """FloatTensor.java:127-140: batched row b is the same dot as the single-vector call, so the
     batched kernel's rows must agree with each other when their activations are equal."""
