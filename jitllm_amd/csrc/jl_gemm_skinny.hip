@@ -24,9 +24,10 @@
 //
 // The activation fragments (read as fp32 and rounded to fp16 by the kernel itself) depend on the
 // slice only and stay in registers for the whole kernel.  A wave's result is a partial sum over its
-// 256 columns; a wave of its own folds the compute waves' partials through LDS one tile later and
-// applies the epilogue, rows wider than the workgroup's span are cut across workgroups and folded
-// by jl_skinny_reduce.  Calls of 33..64 rows run as two row blocks of up to 32 on the two halves of
+// 256 columns; two waves of their own fold the compute waves' partials through LDS two tiles later
+// and apply the epilogue (one row block each when there are two), rows wider than the workgroup's
+// span are cut across workgroups and folded by jl_skinny_reduce.  The two compute waves of a SIMD
+// run half a tile apart: one decodes while the other multiplies.  Calls of 33..64 rows run as two row blocks of up to 32 on the two halves of
 // the chip; the halves walk the same tiles at the same time, so the second reader of a tile finds
 // it in the L2 of its XCD.
 #include <stdlib.h>
@@ -297,8 +298,11 @@ __device__ __forceinline__ float skinny_swiglu(float g, float u) { return g * __
 // their own and the two kinds meet at one barrier per tile.
 constexpr int kDmaWaves = 2;
 // ... and so has the fold of the compute waves' partial sums with the epilogue: a chain of LDS
-// round trips, exponentials and stores that would otherwise stall the decode of the next tile.
-constexpr int kFoldWaves = 1;
+// round trips, exponentials and stores that would otherwise stall the decode of the next tile
+// (two waves: one per row block).
+constexpr int kFoldWaves = 2;
+// buffers of partial sums that a workgroup cycles through, one per group in flight
+constexpr int kParities = 3;
 constexpr int max_slices(int) { return 32; }
 // The prologue's staging area of a compute wave: 8 activation rows x 256 columns as fp16, rows 16
 // bytes apart from a multiple of 256 so that the fragment reads of 16 lanes hit all banks.
@@ -328,11 +332,11 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     const int slots_per_row = lds_row >> 4;
     const int n_loads = (kGroup * slots_per_row + 64 * kDmaWaves - 1) / (64 * kDmaWaves);
     const int stage_bytes = n_loads * 64 * kDmaWaves * 16;
-    const int partial_bytes = waves * NBB * 1024;  // one parity
+    const int partial_bytes = waves * NBB * 1024;  // one buffer of kParities
     const int total_groups = p.seg_group_begin[p.nseg];
     const int out_rows = DUAL ? kGroup / 2 : kGroup;   // outputs per group
 
-    // LDS: the tile ring, then the partial sums (two parities)
+    // LDS: the tile ring, then the partial sums (kParities buffers)
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lvoid *)lds;
     const uint32_t ring0 = lds0;
     uint8_t *ring = lds;
@@ -456,9 +460,11 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     }
 
     if (wave >= waves + kDmaWaves) {
-        // ---- fold wave.  After the barrier that opens group it + 1 the partial sums of group it
-        // (parity it & 1) are complete; they are overwritten two groups later, behind barriers this
-        // wave takes part in, so it has one group's time.  A partial is what one lane of one
+        // ---- fold waves.  The partial sums of group it (buffer it % kParities) are complete one
+        // tile after the group's last one -- the late compute waves multiply a tile behind -- and
+        // are overwritten three groups later, behind barriers these waves take part in.  With two
+        // row blocks each fold wave takes one (a fold of both took longer than a tile when the
+        // workgroup walks a single span), else the first does the work.  A partial is what one lane of one
         // compute wave held: weight row o % 16 of the group against activation rows
         // 16 b + 4 (o / 16) .. + 3, for lane o and row block b; in a gate/up group weight rows 8..15
         // are the up rows of outputs 0..7.  Lane o of this wave adds the waves' partials of its
@@ -466,6 +472,9 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         const int o = lane;
         const int n = o & 15;
         const int go = o >> 4;
+        // with two fold waves and two row blocks each takes one block (the fold of a group has one
+        // tile's time when the workgroup walks a single span)
+        const int fw = wave - waves - kDmaWaves;
         // its few instructions go ahead of the compute waves' on the SIMD they share: every
         // barrier between two folds waits for this wave
         __builtin_amdgcn_s_setprio(2);
@@ -476,6 +485,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             const int local = (group - sg.group_begin) * out_rows + n;   // output column inside the weight
 #pragma unroll
             for (int b = 0; b < NBB; b++) {
+                if (kFoldWaves > 1 && (NBB > 1 ? b != fw : fw != 0)) continue;
                 // all of the (at most eight) compute waves' partials in one round trip
                 floatx4 v[8], u[8];
 #pragma unroll
@@ -517,18 +527,23 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                 }
             }
         };
-        for (int it = 0; it < mine; it++) {
-#pragma unroll
-            for (int q = 0; q < ZIN; q++) {
-                __builtin_amdgcn_s_barrier();
-                STAMP(2 * it);
-                if (q == 0 && it > 0) fold(wg + (it - 1) * stride, (it - 1) & 1);
-                if (q == 0) STAMP(2 * it + 1);
+        // The late compute waves (below) finish group it during the tile after its last one, so
+        // its partial sums are complete at the barrier of tile (it + 1) ZIN + 1; they sit in buffer
+        // it % 3, which the early waves write again at the end of group it + 3.
+        const int tiles = mine * ZIN;
+        int folded = 0;
+        for (int t = 0; t < tiles; t++) {
+            __builtin_amdgcn_s_barrier();
+            STAMP(2 * t);
+            if (folded < mine && (folded + 1) * ZIN + 1 <= t) {
+                fold(wg + folded * stride, folded % kParities);
+                folded++;
             }
+            STAMP(2 * t + 1);
         }
         if (mine > 0) {
             __builtin_amdgcn_s_barrier();
-            fold(wg + (mine - 1) * stride, (mine - 1) & 1);
+            for (; folded < mine; folded++) fold(wg + folded * stride, folded % kParities);
         }
         return;
     }
@@ -662,46 +677,93 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     }
 
     STAMP(1);
-    for (int it = 0; it < mine; it++) {
+    // One tile: the slice's fragments against the activation fragments of span q, added to `total`.
+    auto multiply = [&](int q, const half8 (&wf)[8], const Q4KTail &tail, floatx4 (&total)[NBB]) {
+#pragma unroll
+        for (int b = 0; b < NBB; b++) {
+            floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) {
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[b][q][i], wf[i], acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[b][q][i + 1], wf[i + 1], acc1, 0, 0, 0);
+            }
+            if constexpr (TYPE == JL_Q4_K) {
+                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                const floatx4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[b][q], tail.mins, zero, 0, 0, 0);
+                total[b] += ((acc0 + acc1) * tail.d - accm * tail.dmin) * undo[b][q];
+            } else {
+                total[b] += (acc0 + acc1) * undo[b][q];
+            }
+        }
+    };
+    // plain arithmetic happened on the MFMA results: the compiler placed the wait states itself
+    auto publish = [&](int it, floatx4 (&total)[NBB]) {
+        asm volatile("" : "+v"(total[0]));
+        const uint32_t pw = part0 + (it % kParities) * partial_bytes + wave * (NBB * 1024) + lane * 16;
+#pragma unroll
+        for (int b = 0; b < NBB; b++) lds_write_f4(pw + b * 1024, total[b]);
+    };
+    const int tiles = mine * ZIN;
+    // The two compute waves of a SIMD (w and w + 4) run half a tile apart, so that one of them
+    // decodes (vector ALU) while the other multiplies (matrix pipe): after the barrier of tile t
+    // the early wave decodes tile t and multiplies it; the late wave first multiplies tile t - 1,
+    // whose fragments it holds, and then decodes tile t.  In lock step both decoded first and the
+    // second one's MFMAs, a chain of dependent accumulations, ended the tile alone.
+    if (wave < 4) {
+        for (int it = 0; it < mine; it++) {
+            floatx4 total[NBB];
+#pragma unroll
+            for (int b = 0; b < NBB; b++) total[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int q = 0; q < ZIN; q++) {
+                const int t = it * ZIN + q;
+                STAMP(2 + 4 * t);
+                __builtin_amdgcn_s_barrier();   // tile t has landed
+                STAMP(3 + 4 * t);
+                if (PROBE(1)) continue;   // copy only
+                half8 wf[8];
+                Q4KTail tail;
+                decode_slice<TYPE>(ring0 + (t % p.stages) * stage_bytes + c * lds_row, sl, wf, tail);
+                asm volatile("" : "+v"(wf[0]), "+v"(wf[7]));
+                STAMP(4 + 4 * t);
+                multiply(q, wf, tail, total);
+            }
+            STAMP(5 + 4 * (it * ZIN + ZIN - 1));
+            publish(it, total);
+        }
+    } else {
+        half8 wf[8];
+        Q4KTail tail;
         floatx4 total[NBB];
 #pragma unroll
         for (int b = 0; b < NBB; b++) total[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int it = 0; it < mine; it++) {
 #pragma unroll
-        for (int q = 0; q < ZIN; q++) {
-            const int t = it * ZIN + q;
-            STAMP(2 + 4 * t);
-            __builtin_amdgcn_s_barrier();   // tile t has landed; the fold wave takes the sums of group it - 1
-            STAMP(3 + 4 * t);
-
-            if (PROBE(1)) continue;   // copy only
-            half8 wf[8];
-            Q4KTail tail;
-            decode_slice<TYPE>(ring0 + (t % p.stages) * stage_bytes + c * lds_row, sl, wf, tail);
-            asm volatile("" : "+v"(wf[0]), "+v"(wf[7]));
-            STAMP(4 + 4 * t);
+            for (int q = 0; q < ZIN; q++) {
+                const int t = it * ZIN + q;
+                STAMP(2 + 4 * t);
+                __builtin_amdgcn_s_barrier();   // tile t has landed
+                STAMP(3 + 4 * t);
+                if (PROBE(1)) continue;   // copy only
+                if (t > 0) {
+                    // tile t - 1: span (q - 1) mod ZIN, the last of its group when q == 0
+                    multiply(q == 0 ? ZIN - 1 : q - 1, wf, tail, total);
+                    if (q == 0) {
+                        publish(it - 1, total);
 #pragma unroll
-            for (int b = 0; b < NBB; b++) {
-                floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int i = 0; i < 8; i += 2) {
-                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[b][q][i], wf[i], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[b][q][i + 1], wf[i + 1], acc1, 0, 0, 0);
+                        for (int b = 0; b < NBB; b++) total[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+                    }
                 }
-                if constexpr (TYPE == JL_Q4_K) {
-                    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-                    const floatx4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[b][q], tail.mins, zero, 0, 0, 0);
-                    total[b] += ((acc0 + acc1) * tail.d - accm * tail.dmin) * undo[b][q];
-                } else {
-                    total[b] += (acc0 + acc1) * undo[b][q];
-                }
+                STAMP(4 + 4 * t);
+                decode_slice<TYPE>(ring0 + (t % p.stages) * stage_bytes + c * lds_row, sl, wf, tail);
+                asm volatile("" : "+v"(wf[0]), "+v"(wf[7]));
+                STAMP(5 + 4 * t);
             }
         }
-        asm volatile("" : "+v"(total[0]));
-        STAMP(5 + 4 * (it * ZIN + ZIN - 1));
-        // plain arithmetic happened on the MFMA results: the compiler placed the wait states itself
-        const uint32_t pw = part0 + (it & 1) * partial_bytes + wave * (NBB * 1024) + lane * 16;
-#pragma unroll
-        for (int b = 0; b < NBB; b++) lds_write_f4(pw + b * 1024, total[b]);
+        if (mine > 0 && !PROBE(1)) {
+            multiply(ZIN - 1, wf, tail, total);
+            publish(mine - 1, total);
+        }
     }
     if (mine > 0) __builtin_amdgcn_s_barrier();
 #ifdef JL_SKINNY_PROBE
@@ -897,7 +959,7 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     const int n_loads = (kGroup * ((p.span_bytes + 16) / 16) + 64 * kDmaWaves - 1) / (64 * kDmaWaves);
     if (n_loads > per_wave) return JL_OK;
     const int stage_bytes = n_loads * 64 * kDmaWaves * 16;
-    const int partial = 2 * (threads / 64) * nbb * 1024;
+    const int partial = kParities * (threads / 64) * nbb * 1024;
     int stages = (160 * 1024 - partial) / stage_bytes;
     if (stages > 4) stages = 4;
     if (stages < 2) return JL_OK;
