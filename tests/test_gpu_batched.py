@@ -169,8 +169,8 @@ def test_batched_gate_up(ctx, t, d, n, T):
 def test_many_row_prefill_matches_oracle(ctx, t, d, n, T, residual):
     """A thousand rows or more: weights decoded to fp16 once per call, then the plain fp16 GEMM
     (dequantize*ToFP16 + gemmMMA, TransformerBatchPrefillKernels.java:917-1076,2325-2363).  Same
-    arithmetic as the fused kernel, so the same bound; the fourth shape takes the 256-wide tiles, the
-    fifth (few tiles, long rows) cuts K in two."""
+    arithmetic as the fused kernel, so the same bound; the shapes take different tiles (256 x 256,
+    256 x 128, 128 x 128)."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
     say("many-row prefill", NAMES[t], d, n, T, residual)
@@ -225,12 +225,13 @@ def test_many_row_prefill_qkv_and_gate_up(ctx):
 
 
 @pytest.mark.parametrize("t,d,n,T,residual", [
-    (O.Q8_0, 5800, 256, 1024, False),    # 128-wide tiles, last tile 40 columns
-    (O.Q4_K, 6016, 256, 1024, True),     # 128-wide tiles, residual
-    (O.Q4_0, 16500, 256, 1100, False),   # 256-wide tiles, ragged rows and columns
-    (O.Q8_0, 3000, 2048, 1024, True),    # K cut in two, last tile 56 columns
-    (O.Q4_K, 3000, 1024, 600, False),    # K cut in four runs of four steps, ragged rows
-    (O.Q8_0, 1500, 2048, 512, True),     # K cut in eight, last tile 92 columns
+    (O.Q8_0, 5800, 256, 1024, False),    # 256 x 128 tiles, last tile 40 columns
+    (O.Q4_K, 6016, 256, 1024, True),     # 256 x 128 tiles, residual
+    (O.Q4_0, 16500, 256, 1100, False),   # 256 x 256 tiles, ragged rows and columns
+    (O.Q8_0, 3000, 2048, 1024, True),    # 128 x 128 tiles, K whole, last tile 56 columns
+    (O.Q4_K, 3000, 1024, 600, False),    # 128 x 128 tiles, K cut in two, ragged rows
+    (O.Q8_0, 1500, 2048, 512, True),     # 128 x 128 tiles, K cut in four, last tile 92 columns
+    (O.Q4_0, 700, 2048, 520, False),     # 128 x 128 tiles, K cut in eight runs of four steps, ragged both ways
 ])
 def test_two_pass_prefill_tiles_and_edges(ctx, t, d, n, T, residual):
     """Shapes with enough tiles for the decode-once path on 256 compute units, one per tiling it
@@ -289,6 +290,25 @@ def test_two_pass_prefill_qkv_and_gate_up(ctx):
                                                 ctx.load_weight(t, r3, d, n), n, d)
     ctx.sync()
     got = hb.get().reshape(T, d)
+    mg, mu = magnitude(t, r1, X, d, n), magnitude(t, r3, X, d, n)
+    bound = 2e-4 * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
+    # gate/up on 128 x 128 tiles (9 x 20 of them: too few rows for the larger tiles), ragged rows,
+    # a last tile of 54 outputs
+    t, d, n, T = O.Q8_0, 1270, 512, 1100
+    r1 = synthetic.weight(t, d, n, seed=295)
+    r3 = synthetic.weight(t, d, n, seed=296)
+    X = synthetic.activations((T, n), seed=297)
+    g = O.matmul_batch(t, r1, X, d, n)
+    u = O.matmul_batch(t, r3, X, d, n)
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(T, d)
+    hb = ctx.float_array(T * d + 64, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, 2 * d).gateUp(ctx.from_numpy(X), hb, ctx.load_weight(t, r1, d, n),
+                                                ctx.load_weight(t, r3, d, n), n, d)
+    ctx.sync()
+    flat = hb.get()
+    assert np.all(flat[T * d:] == UNTOUCHED)
+    got = flat[:T * d].reshape(T, d)
     mg, mu = magnitude(t, r1, X, d, n), magnitude(t, r3, X, d, n)
     bound = 2e-4 * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
