@@ -100,6 +100,55 @@ def test_calls_of_at_most_eight_rows_match_the_same_rows_of_a_larger_call(ctx, t
     assert rel_err(results[1][0], ref, magnitude(t, raw, X[:rows], d, n)) < 2e-4
 
 
+def _random_batched_shapes():
+    """Seeded shapes across the weight-streaming kernel's launch geometries: one to eight compute
+    waves per workgroup (row lengths of 256 .. 2048 columns per span), one, two and several spans
+    per row, one or two row blocks per workgroup, two row blocks across the grid, partial batches."""
+    rng = np.random.default_rng(20261125)
+    shapes = []
+    for t in (O.Q8_0, O.Q4_0, O.Q4_K):
+        for n in (256, 768, 1280, 2048, 2304, 4096, 6144):
+            rows = int(rng.choice([1, 3, 8, 9, 16, 17, 31, 32, 33, 50, 64]))
+            d = int(rng.integers(1, 300))
+            active = rows if rng.integers(0, 2) else int(rng.integers(1, rows + 1))
+            shapes.append((t, d, n, rows, active))
+    return shapes
+
+
+@pytest.mark.parametrize("t,d,n,rows,active", _random_batched_shapes())
+def test_batched_decode_on_random_shapes(ctx, t, d, n, rows, active):
+    """Plain, residual and gate/up results of the weight-streaming kernel against the oracle; rows
+    past the active ones keep their contents (BatchProjectionTilingAccelTest.java:151-215)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("batched, random shape", NAMES[t], d, n, rows, active)
+    raw = synthetic.weight(t, d, n, seed=7500 + d)
+    raw_up = synthetic.weight(t, d, n, seed=7501 + d)
+    X = synthetic.activations((rows, n), seed=7502 + n)
+    dot = O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256
+    g = O.matmul_batch(t, raw, X[:active], d, n, dot)
+    u = O.matmul_batch(t, raw_up, X[:active], d, n, dot)
+    mg, mu = magnitude(t, raw, X[:active], d, n), magnitude(t, raw_up, X[:active], d, n)
+    w, w_up = ctx.load_weight(t, raw, d, n), ctx.load_weight(t, raw_up, d, n)
+    proj = QuantizedBatchProjections(ctx, rows, n, 2 * d)
+    xd = ctx.from_numpy(X)
+    plain = ctx.float_array(rows * d, fill=UNTOUCHED)
+    res = ctx.float_array(rows * d, fill=UNTOUCHED)
+    hb = ctx.float_array(rows * d, fill=UNTOUCHED)
+    proj.projection(xd, plain, w, n, d, False, activeRows=active)
+    proj.projection(xd, res, w, n, d, True, activeRows=active)
+    proj.gateUp(xd, hb, w, w_up, n, d, activeRows=active)
+    ctx.sync()
+    plain, res, hb = (a.get().reshape(rows, d) for a in (plain, res, hb))
+    for a in (plain, res, hb):
+        assert np.all(a[active:] == UNTOUCHED)
+    assert rel_err(plain[:active], g, mg) < F16_BOUND
+    assert rel_err(res[:active], g + UNTOUCHED, mg + 12345.5 * 6e-8) < F16_BOUND
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(active, d)
+    bound = F16_BOUND * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(hb[:active].astype(np.float64) - ref) <= bound)
+
+
 def test_batched_row_is_the_single_vector_result(ctx):
     """FloatTensor.java:127-140: batched row b is the same dot as the single-vector call, so the
     batched kernel's rows must agree with each other when their activations are equal."""
