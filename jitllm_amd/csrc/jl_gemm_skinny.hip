@@ -580,11 +580,14 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
 #pragma unroll
             for (int q = 0; q < ZIN; q++) {
                 const float4 *src = (const float4 *)(p.X + 64 * ((z * ZIN + q) * p.Ss + 4 * wave)) + lane;
+                // rows past the last active one re-read it (their results are never stored): no
+                // branch and no zero fill per row, and the address moves by one row length
+                const int first = row0 + 16 * b;
+                const float *rowp = (const float *)src + (int64_t)(first < p.rows ? first : p.rows - 1) * p.k;
 #pragma unroll
                 for (int r = 0; r < XR; r++) {
-                    const int m = row0 + 16 * b + r;   // (uniform: a scalar branch)
-                    if (m < p.rows) x[b * ZIN + q][r] = *(const float4 *)((const float *)src + (int64_t)m * p.k);
-                    else x[b * ZIN + q][r] = float4{0.f, 0.f, 0.f, 0.f};
+                    x[b * ZIN + q][r] = *(const float4 *)rowp;
+                    if (first + r + 1 < p.rows) rowp += p.k;
                 }
             }
         }
@@ -623,20 +626,18 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                 // amax = 1.f * 2^(E - 127): multiply by 2^(136 - E), undo with 2^(E - 136); the
                 // row's largest value lands in [2^9, 2^10), which keeps huge rows finite, tiny rows
                 // out of fp16's subnormals and a sub-block's sum of 32 inside fp16's range
+                uint32_t inv4[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     int E = (int)((__float_as_uint(v4[e]) >> 23) & 0xFF);
                     E = E < 12 ? 12 : E;
                     undo[b][q][e] = __uint_as_float((uint32_t)(E - 9) << 23);
+                    inv4[e] = (uint32_t)(263 - E) << 23;
                 }
+                // (the scale of row r, a scalar operand of its conversions: lane group r / 4 holds it)
                 float inv[XR];
 #pragma unroll
-                for (int r = 0; r < XR; r++) {
-                    const uint32_t bits = __builtin_amdgcn_readlane(__float_as_uint(v4[r & 3]), 16 * (r >> 2));
-                    int E = (int)((bits >> 23) & 0xFF);
-                    E = E < 12 ? 12 : E;
-                    inv[r] = __uint_as_float((uint32_t)(263 - E) << 23);
-                }
+                for (int r = 0; r < XR; r++) inv[r] = __uint_as_float(__builtin_amdgcn_readlane(inv4[r & 3], 16 * (r >> 2)));
                 if constexpr (HALF) {
                     const _Float16 z16 = (_Float16)0.f;
 #pragma unroll
