@@ -806,6 +806,27 @@ def prefill_probe(ctx, t, T=2048, mode="xf16"):
                       "mfma_f16_flops_per_instruction_16x16x32": 2 * 16 * 16 * 32}))
 
 
+def mfma_rate_probe(cu, reps=5, steps=20000):
+    """The rate at which the chip sustains fp16 matrix instructions out of registers, measured by
+    `jitllm_amd/lib/libjl_probes.so` (a measurement aid built beside the product library, not part
+    of it): loops of nothing but `v_mfma_f32_16x16x32_f16` / `32x32x16` on one 8-wave workgroup per
+    compute unit, with every operand 1.0 and with random operands.  The published 2.5 PFLOP/s is
+    reached only by the former; the latter is what a GEMM on real data can approach.  Medians over
+    `reps` launches of about 20 ms, the first left out (the clock settles during it)."""
+    lib = C.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)), "jitllm_amd", "lib", "libjl_probes.so"))
+    lib.jl_probe_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
+    lib.jl_probe_mfma_rate.restype = C.c_int
+    out = {"what": "register-only MFMA loops, 8 waves per compute unit, TFLOP/s (median of %d launches)" % reps}
+    for shape, name in ((0, "16x16x32"), (1, "32x32x16")):
+        for random, data in ((1, "random_operands"), (0, "constant_operands")):
+            buf = (C.c_double * (reps + 1))()
+            rc = lib.jl_probe_mfma_rate(0, shape, random, steps, reps + 1, cu, buf)
+            if rc != 0:
+                raise RuntimeError(f"jl_probe_mfma_rate: HIP error {rc}")
+            out[f"{name}_{data}"] = round(statistics.median(list(buf)[1:]), 1)
+    return out
+
+
 def batched_probe(ctx):
     """What the kernel trace of the batched-decode kernels is collected on: the four calls of one
     Q4_K Qwen3-8B-like layer (q|k|v, o +=, gate/up SwiGLU, down +=) at 8, 32 and 64 rows, launched
@@ -875,6 +896,8 @@ def main():
     ap.add_argument("--probe-tokens", type=int, default=2048, help="--prefill-probe: tokens")
     ap.add_argument("--probe-mode", default="xf16", choices=["xf16", "resident", "default"],
                     help="--prefill-probe: operand types and residency (see prefill_probe)")
+    ap.add_argument("--mfma-rate-probe", action="store_true",
+                    help="only measure the sustained rate of fp16 matrix instructions (see mfma_rate_probe)")
     ap.add_argument("--batched-probe", action="store_true",
                     help="only launch the batched-decode calls, kernel by kernel (see batched_probe)")
     ap.add_argument("--decode-probe", action="store_true",
@@ -900,6 +923,9 @@ def main():
     with Context(0) as ctx:
         cu, name = ctx.device_info()
         clock_khz = hip.clock_khz(0)
+        if args.mfma_rate_probe:
+            print(json.dumps(mfma_rate_probe(cu)))
+            return
         if args.prefill_probe:
             prefill_probe(ctx, t, args.probe_tokens, args.probe_mode)
             return
@@ -1063,6 +1089,12 @@ def main():
         if "prefill" in legs:
             out["prefill"] = [bench_gemm(ctx, hip, t, T, max(4, args.steps // 2), prefill_warmup, cpu and T == 512,
                                          clock_khz, cu) for T in (512, 2048)]
+            # what the matrix pipe sustains on this box, beside the published peak the fractions use
+            sustained = mfma_rate_probe(cu)
+            for leg in out["prefill"]:
+                leg["roofline"]["sustained_from_box"] = dict(
+                    sustained, frac_of_random_operand_rate=round(
+                        leg["roofline"]["achieved"] / sustained["16x16x32_random_operands"], 4))
         if "other_types" in legs:
             out["decode_other_types"] = [
                 bench_decode_layers(ctx, hip, "Q4_0", 4096, 1024, 14336, 4, args.steps, args.warmup, cpu),
