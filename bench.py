@@ -806,6 +806,29 @@ def prefill_probe(ctx, t, T=2048, mode="xf16"):
                       "mfma_f16_flops_per_instruction_16x16x32": 2 * 16 * 16 * 32}))
 
 
+def _probes_lib():
+    lib = C.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)), "jitllm_amd", "lib", "libjl_probes.so"))
+    lib.jl_probe_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
+    lib.jl_probe_mfma_rate.restype = C.c_int
+    lib.jl_probe_hbm_read_rate.argtypes = [C.c_int, C.c_size_t, C.c_int, C.c_int, C.POINTER(C.c_double)]
+    lib.jl_probe_hbm_read_rate.restype = C.c_int
+    return lib
+
+
+def hbm_rate_probe(cu, reps=5, gib=2):
+    """The rate at which the chip streams HBM with nothing else in the way, measured by
+    `jitllm_amd/lib/libjl_probes.so` (a measurement aid built beside the product library, not part
+    of it): plain 16-byte loads over `gib` GiB (far more than the 256 MB memory-side cache), eight
+    in flight per thread, 8 workgroups of 256 per compute unit.  Median of `reps` launches, the
+    first left out.  The decode kernels' fractions of the published 8 TB/s are to be read against it."""
+    buf = (C.c_double * (reps + 1))()
+    rc = _probes_lib().jl_probe_hbm_read_rate(0, gib << 30, reps + 1, cu, buf)
+    if rc != 0:
+        raise RuntimeError(f"jl_probe_hbm_read_rate: HIP error {rc}")
+    return {"what": f"plain streaming read of {gib} GiB, GB/s (median of {reps} launches)",
+            "hbm_read_GB_s": round(statistics.median(list(buf)[1:]), 1)}
+
+
 def mfma_rate_probe(cu, reps=5, steps=20000):
     """The rate at which the chip sustains fp16 matrix instructions out of registers, measured by
     `jitllm_amd/lib/libjl_probes.so` (a measurement aid built beside the product library, not part
@@ -813,9 +836,7 @@ def mfma_rate_probe(cu, reps=5, steps=20000):
     compute unit, with every operand 1.0 and with random operands.  The published 2.5 PFLOP/s is
     reached only by the former; the latter is what a GEMM on real data can approach.  Medians over
     `reps` launches of about 20 ms, the first left out (the clock settles during it)."""
-    lib = C.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)), "jitllm_amd", "lib", "libjl_probes.so"))
-    lib.jl_probe_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
-    lib.jl_probe_mfma_rate.restype = C.c_int
+    lib = _probes_lib()
     out = {"what": "register-only MFMA loops, 8 waves per compute unit, TFLOP/s (median of %d launches)" % reps}
     for shape, name in ((0, "16x16x32"), (1, "32x32x16")):
         for random, data in ((1, "random_operands"), (0, "constant_operands")):
@@ -896,6 +917,8 @@ def main():
     ap.add_argument("--probe-tokens", type=int, default=2048, help="--prefill-probe: tokens")
     ap.add_argument("--probe-mode", default="xf16", choices=["xf16", "resident", "default"],
                     help="--prefill-probe: operand types and residency (see prefill_probe)")
+    ap.add_argument("--hbm-rate-probe", action="store_true",
+                    help="only measure the rate of a plain streaming read of HBM (see hbm_rate_probe)")
     ap.add_argument("--mfma-rate-probe", action="store_true",
                     help="only measure the sustained rate of fp16 matrix instructions (see mfma_rate_probe)")
     ap.add_argument("--batched-probe", action="store_true",
@@ -925,6 +948,9 @@ def main():
         clock_khz = hip.clock_khz(0)
         if args.mfma_rate_probe:
             print(json.dumps(mfma_rate_probe(cu)))
+            return
+        if args.hbm_rate_probe:
+            print(json.dumps(hbm_rate_probe(cu)))
             return
         if args.prefill_probe:
             prefill_probe(ctx, t, args.probe_tokens, args.probe_mode)
@@ -1080,6 +1106,11 @@ def main():
                              "frac": round(single_bytes / (single_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}},
             "decode_kernels": kernels,
         }
+        # what a plain read loop streams from HBM on this box, beside the published peak
+        hbm = hbm_rate_probe(cu)
+        out["roofline"]["sustained_from_box"] = dict(
+            hbm, frac_of_sustained=round(achieved / hbm["hbm_read_GB_s"], 4),
+            step_frac_of_sustained=round(gbs / hbm["hbm_read_GB_s"], 4))
         legs = set() if args.no_extra else set(args.extra.split(","))
         if "wq_shape" in legs:
             out["wq_shape"] = bench_wq_shape(ctx, hip, t, args.steps, args.warmup, cpu)

@@ -1,5 +1,6 @@
-// Measurement aid, not part of libjitllm_hip.so: the rate at which this chip sustains fp16 matrix
-// instructions out of registers, with constant and with random operands.
+// Measurement aids, not part of libjitllm_hip.so: the rates this chip sustains with nothing else in
+// the way -- fp16 matrix instructions out of registers (constant and random operands), and a plain
+// streaming read of HBM.  bench.py prints them beside the published peaks its fractions use.
 //
 // The published dense fp16 figure (2.5 PFLOP/s) is 256 compute units x 4096 flops per clock at
 // 2.4 GHz.  A loop of nothing but v_mfma_f32_16x16x32_f16 reaches it when every operand is 1.0; with
@@ -14,6 +15,7 @@ namespace {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
 
 // SHAPE 0: 16x16x32 over a 128 x 64 wave tile (8 x 4 blocks, as the prefill GEMM's widest tile);
 // SHAPE 1: 32x32x16 over the same wave tile (4 x 2 blocks).  64 (32) instructions per step and wave.
@@ -83,7 +85,56 @@ __global__ void probe_fill(uint16_t *dst, size_t n, int random) {
     }
 }
 
+// Streams `n16` 16-byte pieces once: every thread has eight loads in flight, workgroups take
+// interleaved 32 KB runs.  What it reads is folded into one word per thread so that no load is dropped.
+__global__ void __launch_bounds__(256) probe_read(const uintx4 *src, size_t n16, uint32_t *out) {
+    const size_t stride = (size_t)gridDim.x * 256 * 8;
+    uint32_t acc = 0;
+    for (size_t i = (size_t)blockIdx.x * 256 * 8 + threadIdx.x; i + 7 * 256 < n16; i += stride) {
+        uintx4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = __builtin_nontemporal_load(src + i + j * 256);
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc ^= v[j][0] ^ v[j][1] ^ v[j][2] ^ v[j][3];
+    }
+    out[blockIdx.x * 256 + threadIdx.x] = acc;
+}
+
 }  // namespace
+
+// The rate at which the chip streams `bytes` (far more than its 256 MB memory-side cache) from HBM
+// with plain 16-byte loads: `reps` launches, GB/s of each into gbps[0 .. reps).  The decode
+// kernels' fractions of the published 8 TB/s are to be read against this.
+extern "C" int jl_probe_hbm_read_rate(int device, size_t bytes, int reps, int compute_units, double *gbps) {
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return (int)e;
+    uintx4 *src = nullptr;
+    uint32_t *out = nullptr;
+    const int blocks = compute_units * 8;
+    if ((e = hipMalloc(&src, bytes)) != hipSuccess) return (int)e;
+    if ((e = hipMalloc(&out, (size_t)blocks * 256 * 4)) != hipSuccess) return (int)e;
+    (void)hipMemset(src, 1, bytes);
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    const size_t n16 = bytes / 16;
+    const size_t per_pass = (size_t)blocks * 256 * 8;
+    const size_t read16 = n16 / per_pass * per_pass;   // what the loop covers
+    for (int r = 0; r < reps; r++) {
+        (void)hipEventRecord(e0, 0);
+        hipLaunchKernelGGL(probe_read, dim3(blocks), dim3(256), 0, 0, src, n16, out);
+        (void)hipEventRecord(e1, 0);
+        if ((e = hipEventSynchronize(e1)) != hipSuccess) break;
+        float ms = 0;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        gbps[r] = (double)read16 * 16.0 / (ms * 1e-3) / 1e9;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(src);
+    (void)hipFree(out);
+    return (int)e;
+}
 
 // Runs `reps` launches of `steps` loop steps on one workgroup of 8 waves per compute unit and
 // writes each launch's TFLOP/s into tflops[0 .. reps).  Returns 0, or the HIP error code.
