@@ -713,7 +713,13 @@ __device__ uint64_t *jl_gemv_stamp_buf = nullptr;
 // lanes past the row's end idle; everything but the row length is still a constant.)
 template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false,
           bool PART = false>
-__global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
+__global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first, const uint8_t *w_up_first, const float *x_first, int tiles_first,
+              int rows_first, int grid_first, GemvParams p) {
+    // The leading arguments repeat what the kernel needs before its first tile's loads can go out
+    // (first weight, up weight, the activation vector, tile count, first weight's rows, grid width):
+    // the build preloads them into scalar registers at dispatch (-amdgpu-kernarg-preload-count),
+    // where a read of the argument buffer is a round trip to memory at the head of every launch.
+    // (Preloading the q|k|v form's other two weights and first tiles as well changed nothing.)
     static_assert(!(RMS && PACKED), "the packed activation is normalised before it is quantised");
     constexpr bool LEAN = SPT != 0;
     constexpr bool FULL = LEAN && !PART;   // every lane has a slice, every load slot is real data
@@ -742,7 +748,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     const int half_rows = DUAL ? R / 2 : R;       // output rows per tile
     const int half_bytes = half_rows * row_bytes;   // bytes of a tile that come from one weight
     const int nseg = (LEAN && !SEGS) ? 1 : p.nseg;
-    const int total_tiles = (LEAN && !SEGS) ? p.seg_tile_begin[1] : p.seg_tile_begin[nseg];
+    const int total_tiles = tiles_first;
     const int stage_bytes = nthreads * SLICE;
     // every thread of the workgroup owns a slice and every load slot is real data
     const bool exact = kExactDma && (FULL || (!PART && (S == Sp) && (R * Sp == nthreads)));
@@ -767,8 +773,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     // each wave's outstanding-load count is a compile-time constant per tile.
     // (a launch with one segment -- every one but the fused q|k|v -- never indexes the argument
     // arrays with a run-time segment: that is a scalar memory load, and a wait, per tile)
-    const uint8_t *const w0 = p.w[0];
-    const int rows0 = p.seg_rows[0];
+    const uint8_t *const w0 = w_first;
+    const int rows0 = rows_first;
     float *const out0 = p.out[0];
     auto segment_of = [&](int tile) {
         int seg = 0;
@@ -813,7 +819,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
         const int64_t remain = (int64_t)seg_rows * row_bytes - offset;
         const int bytes = remain < half_bytes ? (int)remain : half_bytes;
         const uint8_t *base = wseg + offset;
-        const uint8_t *base_up = DUAL ? p.w_up + offset : base;
+        const uint8_t *base_up = DUAL ? w_up_first + offset : base;
         uint8_t *dst = ring + st * stage_bytes;
         const bool whole = exact && (FULL || bytes == half_bytes);  // uniform
         if (whole) {
@@ -848,9 +854,10 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     asm volatile("" :: "v"(slot_off[0]), "s"(total_tiles), "s"(half_bytes));   // the arguments have arrived
 #endif
     GSTAMP(1);
-    // my tiles: blockIdx.x, blockIdx.x + gridDim.x, ...
+    // my tiles: blockIdx.x, blockIdx.x + grid, ...
+    const int grid = grid_first;
     const int first = blockIdx.x;
-    const int mine = first < total_tiles ? (total_tiles - first + gridDim.x - 1) / gridDim.x : 0;
+    const int mine = first < total_tiles ? (total_tiles - first + grid - 1) / grid : 0;
 
     // Segmented sum over aligned groups of `width` lanes (a power of two): row-local DPP moves up
     // to 16 lanes, cross-row permutes beyond.
@@ -886,7 +893,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
             // (the side types' vector region, where it is one of its own, ends with the vector's last
             // slot -- their 1024-thread form fits the LDS only so -- and nothing is written past it)
             if (kExactDma || x_in_ring || q < x_slots)
-                __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)p.x + off),
+                __builtin_amdgcn_global_load_lds((gvoid *)((const uint8_t *)x_first + off),
                                                  (lvoid *)(xs + base + wave * JL_WAVE * 16), 16, 0, 0);
         }
     }
@@ -917,7 +924,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
         if (held) load(0);
     }
     GSTAMP(2);
-    for (; issued < kStages - 1 && issued < mine; issued++) issue(first + issued * gridDim.x, issued);
+    for (; issued < kStages - 1 && issued < mine; issued++) issue(first + issued * grid, issued);
     if constexpr (rms) {
         float scale;
         if (p.rms_scale) {
@@ -1075,7 +1082,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     const bool in_wave = Sp <= (DUAL ? 32 : 64);
     const int r_lds = (DUAL && in_wave) ? (r & 1) * half_rows + (r >> 1) : r;   // tile row this thread reads
     for (int it = 0; it < mine; it++) {
-        const int tile = first + it * gridDim.x;
+        const int tile = first + it * grid;
         // with two stages nothing was issued after tile `it`: its loads are the youngest
         JL_WAIT_VM(0);
         __builtin_amdgcn_s_barrier();
@@ -1083,10 +1090,10 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
         // the stage that tile it - 1 (or, the first time round, the activation vector) occupied
         // is free now: every wave is past its reads
         if (issued < mine) {
-            issue(first + issued * gridDim.x, issued % kStages);
+            issue(first + issued * grid, issued % kStages);
             issued++;
         }
-        if (!in_wave && it > 0) finish(tile - gridDim.x, (it - 1) & 1);
+        if (!in_wave && it > 0) finish(tile - grid, (it - 1) & 1);
 
         float v = 0.f;
         if (active) {
@@ -1140,7 +1147,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(GemvParams p) {
     }
     if (mine > 0 && !in_wave) {
         __builtin_amdgcn_s_barrier();
-        finish(first + (mine - 1) * gridDim.x, (mine - 1) & 1);
+        finish(first + (mine - 1) * grid, (mine - 1) & 1);
     }
     GSTAMP(7);
 #ifdef JL_GEMV_STAMPS
@@ -1264,7 +1271,7 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
     if (grid > total) grid = total;
-    hipLaunchKernelGGL(fn, dim3(grid), dim3(threads), lds, ctx->stream, p);
+    hipLaunchKernelGGL(fn, dim3(grid), dim3(threads), lds, ctx->stream, p.w[0], p.w_up, p.x, total, p.seg_rows[0], grid, p);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
