@@ -714,9 +714,11 @@ __device__ uint64_t *jl_gemv_stamp_buf = nullptr;
 template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false,
           bool PART = false>
 __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first, const uint8_t *w_up_first, const float *x_first, int tiles_first,
-              int rows_first, int grid_first, GemvParams p) {
+              int rows_first, int grid_first, int S_first, int row_bytes_first, const float *rms_w_first,
+              GemvParams p) {
     // The leading arguments repeat what the kernel needs before its first tile's loads can go out
-    // (first weight, up weight, the activation vector, tile count, first weight's rows, grid width):
+    // (first weight, up weight, the activation vector, tile count, first weight's rows, grid width,
+    // slices and bytes of a row, the RMS weights):
     // the build preloads them into scalar registers at dispatch (-amdgpu-kernarg-preload-count),
     // where a read of the argument buffer is a round trip to memory at the head of every launch.
     // (Preloading the q|k|v form's other two weights and first tiles as well changed nothing.)
@@ -738,8 +740,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     const int tid = threadIdx.x;
     const int nthreads = LEAN ? THREADS : (int)blockDim.x;
     // geometry: constants in the fixed-geometry form, launch arguments otherwise
-    const int Sp = LEAN ? SPT : p.Sp, S = FULL ? SPT : p.S, R = LEAN ? THREADS / (LEAN ? SPT : 1) : p.R;
-    const int row_bytes = FULL ? row_bytes_of<TYPE>(SPT) : p.row_bytes;
+    const int Sp = LEAN ? SPT : p.Sp, S = FULL ? SPT : S_first, R = LEAN ? THREADS / (LEAN ? SPT : 1) : p.R;
+    const int row_bytes = FULL ? row_bytes_of<TYPE>(SPT) : row_bytes_first;
     const int wave = __builtin_amdgcn_readfirstlane(tid / JL_WAVE);   // uniform: LDS-DMA bases stay scalar
     const int lane = tid & (JL_WAVE - 1);
     const int r = tid / Sp;           // row of the tile this thread works on
@@ -905,7 +907,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     // product in the LDS region the plain path fills with x, so everything after is shared
     // and the LDS footprint (workgroups per compute unit) is that of the plain path.
     const int nvec = rms ? p.n / 4 : 0;
-    const float4 *xv = (const float4 *)p.x, *wv = (const float4 *)p.rms_w;
+    const float4 *xv = (const float4 *)x_first, *wv = (const float4 *)rms_w_first;
     // rows of up to 4 x 4 x nthreads columns are read once and held in registers from the
     // sum of squares to the product; longer ones are read again for the product
     const bool held = nvec <= nthreads * 4;
@@ -1271,7 +1273,8 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
     if (grid > total) grid = total;
-    hipLaunchKernelGGL(fn, dim3(grid), dim3(threads), lds, ctx->stream, p.w[0], p.w_up, p.x, total, p.seg_rows[0], grid, p);
+    hipLaunchKernelGGL(fn, dim3(grid), dim3(threads), lds, ctx->stream, p.w[0], p.w_up, p.x, total, p.seg_rows[0], grid, p.S, p.row_bytes,
+                       p.rms_w, p);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
