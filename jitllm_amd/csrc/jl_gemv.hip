@@ -725,7 +725,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     static_assert(!(RMS && PACKED), "the packed activation is normalised before it is quantised");
     constexpr bool LEAN = SPT != 0;
     constexpr bool FULL = LEAN && !PART;   // every lane has a slice, every load slot is real data
-    static_assert(!PART || (LEAN && !SEGS), "rows shorter than SPT slices: one weight, fixed tile shape");
+    static_assert(!PART || LEAN, "rows shorter than SPT slices: a fixed tile shape");
     static_assert(!LEAN || !PACKED, "the packed form has no fixed-geometry instances");
 #ifdef JL_GEMV_STAMPS
     uint64_t stamp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -1310,12 +1310,24 @@ int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, boo
             if (p.Sp == 64) return launch_tiles_of<TYPE, false, false, false, 256, 64, true>(ctx, p, threads, lds);
             return launch_tiles_of<TYPE, false, false>(ctx, p, threads, lds);
         }
+        // (q|k|v over rows that fill their slices only in part)
+        if (fixed && !full && threads == 256 && p.nseg > 1) {
+            if (p.Sp == 64) return launch_tiles_of<TYPE, false, false, false, 256, 64, true, true>(ctx, p, threads, lds);
+            if (p.Sp == 128) return launch_tiles_of<TYPE, false, false, false, 256, 128, true, true>(ctx, p, threads, lds);
+        }
     }
     if (full && threads == 256) {
         if (p.Sp == 32) return launch_tiles_of<TYPE, DUAL, false, false, 256, 32>(ctx, p, threads, lds);
         if (p.Sp == 64) return launch_tiles_of<TYPE, DUAL, false, false, 256, 64>(ctx, p, threads, lds);
-        if constexpr (!DUAL) {
-            if (p.Sp == 128) return launch_tiles_of<TYPE, false, false, false, 256, 128>(ctx, p, threads, lds);
+        if constexpr (!DUAL || kMain) {
+            if (p.Sp == 128) return launch_tiles_of<TYPE, DUAL, false, false, 256, 128>(ctx, p, threads, lds);
+        }
+    }
+    // rows that fill their slices only in part (3072 columns: 48 of 64 slices; 5120: 80 of 128)
+    if constexpr (kMain) {
+        if (fixed && !full && threads == 256 && p.nseg == 1) {
+            if (p.Sp == 64) return launch_tiles_of<TYPE, DUAL, false, false, 256, 64, false, true>(ctx, p, threads, lds);
+            if (p.Sp == 128) return launch_tiles_of<TYPE, DUAL, false, false, 256, 128, false, true>(ctx, p, threads, lds);
         }
     }
     if constexpr (!DUAL) {

@@ -163,11 +163,12 @@ def test_gemv_over_activation_magnitudes(ctx, t, scale):
     assert rel_err(out.get(), ref, magnitude(t, raw, x, d, n)) < 2e-5
 
 
-@pytest.mark.parametrize("n", [2048, 4096, 8192, 11008, 14336, 16384])
+@pytest.mark.parametrize("n", [2048, 2560, 3072, 4096, 5120, 7168, 8192, 11008, 14336, 16384])
 @pytest.mark.parametrize("t", [O.Q8_0, O.Q4_0, O.Q4_K])
 def test_fixed_geometry_and_general_kernels_give_the_same_bits(ctx, t, n):
-    """A weight of whole tiles runs the kernel compiled for its row length; the same weight less its
-    last row has a ragged last tile and runs the general one.  Same arithmetic in the same order:
+    """A weight of whole tiles runs the kernel compiled for its row length (or, for rows that fill
+    their slices only in part -- 2560, 3072, 5120, 7168, 11008, 14336 columns -- for its slice count);
+    the same weight less its last row has a ragged last tile and runs the general one.  Same arithmetic in the same order:
     the rows they share come out bit for bit equal (plain and gate/up)."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
@@ -188,11 +189,20 @@ def test_fixed_geometry_and_general_kernels_give_the_same_bits(ctx, t, n):
         proj.floatMatvec(x, out, w, n, rows)
         if n <= 8192:
             proj.gateUp(w, w_up, n, rows)
+        # fused q|k|v: the weight as q, its first 64 rows as k and as v (whole tiles both times; the
+        # second pass, with a ragged q, runs the general kernel)
+        q, k, v = ctx.float_array(rows, fill=POISON), ctx.float_array(64, fill=POISON), ctx.float_array(64, fill=POISON)
+        wk = upload(ctx, t, raw[: 64 * row_bytes], 64, n)
+        wv = upload(ctx, t, raw_up[: 64 * row_bytes], 64, n)
+        proj.fusedQKV(x, q, k, v, w, wk, wv)
         ctx.sync()
-        outs.append((out.get(), hb.get()))
+        outs.append((out.get(), hb.get(), q.get(), k.get(), v.get()))
     assert bits_equal(outs[0][0][: d - 1], outs[1][0])
     if n <= 8192:
         assert bits_equal(outs[0][1][: d - 1], outs[1][1])
+        assert bits_equal(outs[0][2][: d - 1], outs[1][2])
+        assert bits_equal(outs[0][3], outs[1][3]) and bits_equal(outs[0][4], outs[1][4])
+        assert bits_equal(outs[0][2], outs[0][0])   # q of the fused call = the plain projection
 
 
 def _random_shapes():
