@@ -714,11 +714,12 @@ __device__ uint64_t *jl_gemv_stamp_buf = nullptr;
 template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false,
           bool PART = false>
 __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first, const uint8_t *w_up_first, const float *x_first, int tiles_first,
-              int rows_first, int grid_first, int S_first, int row_bytes_first, const float *rms_w_first,
-              GemvParams p) {
+              int rows_first, int grid_first, int S_first, int row_bytes_first, int shape_first,
+              const float *rms_w_first, GemvParams p) {
     // The leading arguments repeat what the kernel needs before its first tile's loads can go out
     // (first weight, up weight, the activation vector, tile count, first weight's rows, grid width,
-    // slices and bytes of a row, the RMS weights):
+    // slices and bytes of a row, padded slices | rows per tile << 10 | weights << 20 for the general
+    // form, the RMS weights):
     // the build preloads them into scalar registers at dispatch (-amdgpu-kernarg-preload-count),
     // where a read of the argument buffer is a round trip to memory at the head of every launch.
     // (Preloading the q|k|v form's other two weights and first tiles as well changed nothing.)
@@ -740,7 +741,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     const int tid = threadIdx.x;
     const int nthreads = LEAN ? THREADS : (int)blockDim.x;
     // geometry: constants in the fixed-geometry form, launch arguments otherwise
-    const int Sp = LEAN ? SPT : p.Sp, S = FULL ? SPT : S_first, R = LEAN ? THREADS / (LEAN ? SPT : 1) : p.R;
+    const int Sp = LEAN ? SPT : (shape_first & 0x3FF), S = FULL ? SPT : S_first;
+    const int R = LEAN ? THREADS / (LEAN ? SPT : 1) : ((shape_first >> 10) & 0x3FF);
     const int row_bytes = FULL ? row_bytes_of<TYPE>(SPT) : row_bytes_first;
     const int wave = __builtin_amdgcn_readfirstlane(tid / JL_WAVE);   // uniform: LDS-DMA bases stay scalar
     const int lane = tid & (JL_WAVE - 1);
@@ -749,7 +751,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     const bool active = FULL || ((s < S) && (LEAN || r < R));
     const int half_rows = DUAL ? R / 2 : R;       // output rows per tile
     const int half_bytes = half_rows * row_bytes;   // bytes of a tile that come from one weight
-    const int nseg = (LEAN && !SEGS) ? 1 : p.nseg;
+    const int nseg = (LEAN && !SEGS) ? 1 : ((shape_first >> 20) & 0xF);
     const int total_tiles = tiles_first;
     const int stage_bytes = nthreads * SLICE;
     // every thread of the workgroup owns a slice and every load slot is real data
@@ -1274,7 +1276,7 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
     int grid = ctx->compute_units * per_cu;
     if (grid > total) grid = total;
     hipLaunchKernelGGL(fn, dim3(grid), dim3(threads), lds, ctx->stream, p.w[0], p.w_up, p.x, total, p.seg_rows[0], grid, p.S, p.row_bytes,
-                       p.rms_w, p);
+                       p.Sp | (p.R << 10) | (p.nseg << 20), p.rms_w, p);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }
