@@ -910,13 +910,15 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     // and the LDS footprint (workgroups per compute unit) is that of the plain path.
     const int nvec = rms ? p.n / 4 : 0;
     const float4 *xv = (const float4 *)x_first, *wv = (const float4 *)rms_w_first;
-    // rows of up to 4 x 4 x nthreads columns are read once and held in registers from the
-    // sum of squares to the product; longer ones are read again for the product
-    const bool held = nvec <= nthreads * 4;
-    float4 v[4], w[4];
+    // rows of up to kHold x 4 x nthreads columns are read once and held in registers from the
+    // sum of squares to the product; longer ones are read again for the product (the
+    // fixed-geometry form's rows always fit: SPT slices of 64 columns)
+    constexpr int kHold = LEAN ? (SPT * 16 / THREADS > 1 ? SPT * 16 / THREADS : 1) : 4;
+    const bool held = LEAN || nvec <= nthreads * kHold;
+    float4 v[kHold], w[kHold];
     auto load = [&](int base) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < kHold; j++) {
             const int i = base + j * nthreads + tid;
             v[j] = i < nvec ? xv[i] : float4{0.f, 0.f, 0.f, 0.f};
             w[j] = i < nvec ? wv[i] : float4{0.f, 0.f, 0.f, 0.f};
@@ -937,7 +939,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
             float ss = 0.f;
             if (held) {
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
+                for (int j = 0; j < kHold; j++) {
                     ss = fmaf(v[j].x, v[j].x, ss);
                     ss = fmaf(v[j].y, v[j].y, ss);
                     ss = fmaf(v[j].z, v[j].z, ss);
@@ -962,10 +964,10 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
             for (int i = 0; i < nthreads / JL_WAVE; i++) ss += __uint_as_float(lds_read_b32(cell + i * 4));
             scale = (float)(1.0 / sqrt((double)(ss / (float)p.n + p.rms_eps)));
         }
-        for (int base = 0; base < nvec; base += nthreads * 4) {
+        for (int base = 0; base < nvec; base += nthreads * kHold) {
             if (!held) load(base);
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < kHold; j++) {
                 const int i = base + j * nthreads + tid;
                 if (i < nvec) {
                     const floatx4 o = {w[j].x * (scale * v[j].x), w[j].y * (scale * v[j].y),
@@ -1303,6 +1305,18 @@ int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, boo
             }
             return p.Sp == 32 ? launch_tiles_of<TYPE, DUAL, true, false, 256, 32>(ctx, p, threads, lds)
                               : launch_tiles_of<TYPE, DUAL, true, false, 256, 64>(ctx, p, threads, lds);
+        }
+        // (rows of 3072 / 3584 / 5120 columns: 48 / 56 of 64 slices, 80 of 128)
+        if (fixed && !full && threads == 256 && (p.Sp == 64 || p.Sp == 128)) {
+            if constexpr (!DUAL) {
+                if (p.nseg > 1) {
+                    return p.Sp == 64
+                               ? launch_tiles_of<TYPE, false, true, false, 256, 64, true, true>(ctx, p, threads, lds)
+                               : launch_tiles_of<TYPE, false, true, false, 256, 128, true, true>(ctx, p, threads, lds);
+                }
+            }
+            return p.Sp == 64 ? launch_tiles_of<TYPE, DUAL, true, false, 256, 64, false, true>(ctx, p, threads, lds)
+                              : launch_tiles_of<TYPE, DUAL, true, false, 256, 128, false, true>(ctx, p, threads, lds);
         }
         return launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds);
     }

@@ -463,7 +463,10 @@ def test_rms_scale_on_device(ctx, n):
 
 
 @pytest.mark.parametrize("t,dq,dkv,n", [(O.Q8_0, 2048, 512, 2048), (O.Q4_0, 4096, 1024, 4096),
-                                         (O.Q4_K, 4096, 1024, 4096), (O.Q8_0, 96, 32, 8192)])
+                                         (O.Q4_K, 4096, 1024, 4096), (O.Q8_0, 96, 32, 8192),
+                                         # rows that fill their slices only in part
+                                         (O.Q8_0, 3072, 1024, 3072), (O.Q4_0, 3584, 512, 3584),
+                                         (O.Q4_K, 5120, 1024, 5120), (O.Q8_0, 5120, 1024, 5120)])
 def test_fused_rms_qkv(ctx, t, dq, dkv, n):
     """q | k | v of rmsnorm(x), held against the host's rmsnorm followed by three matVecs
     (InferenceCore.java:86-91)."""
@@ -495,7 +498,10 @@ def test_fused_rms_qkv(ctx, t, dq, dkv, n):
 
 
 @pytest.mark.parametrize("t,d,n", [(O.Q8_0, 8192, 2048), (O.Q4_0, 14336, 4096),
-                                    (O.Q4_K, 12288, 4096), (O.Q8_0, 40, 8192), (O.Q4_K, 37, 512)])
+                                    (O.Q4_K, 12288, 4096), (O.Q8_0, 40, 8192), (O.Q4_K, 37, 512),
+                                    # rows that fill their slices only in part
+                                    (O.Q8_0, 8192, 3072), (O.Q4_0, 4736, 3584), (O.Q4_K, 3456, 5120),
+                                    (O.Q8_0, 3456, 5120)])
 def test_fully_fused_rms_gate_up(ctx, t, d, n):
     """hb = SiLU(w1 . xn) * (w3 . xn) with xn = rmsnorm(x), the scale computed inside the kernel:
     against the host's rmsnorm, matVec, matVec, swiGLU (InferenceCore.java:124-129)."""
@@ -522,12 +528,12 @@ def test_fully_fused_rms_gate_up(ctx, t, d, n):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + 1e-6)
 
 
-def test_rms_vocabulary_projection_and_argmax(ctx):
+@pytest.mark.parametrize("t,d,n", [(O.Q8_0, 32000, 2048), (O.Q8_0, 9000, 3072), (O.Q4_K, 7000, 5120)])
+def test_rms_vocabulary_projection_and_argmax(ctx, t, d, n):
     """Final norm folded into the vocabulary projection, then the greedy token on the device
     (LogitsQ8_0Layer.java:85-110) against rmsnorm, matVec and FloatTensor.argmax on the host."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
-    t, d, n = O.Q8_0, 32000, 2048
     say("rms vocabulary + argmax", d, n)
     raw = synthetic.weight(t, d, n, seed=661)
     x = synthetic.activations(n, seed=662)
