@@ -1283,67 +1283,61 @@ int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) 
     return JL_OK;
 }
 
-// `fixed`: the launch meets the fixed-geometry form's conditions (rows of exactly Sp slices, whole
-// tiles only); it has an instance for the row lengths 2048, 4096, 8192 (plain and
-// residual only) and, in the 1024-thread form, 16384.
+// The 256-thread fixed-geometry instance of the three main types for rows padded to Sp slices of
+// 64 columns, `full`: every slice is one of the row's (else the row is shorter: 3072 columns are 48
+// of 64 slices, 5120 are 80 of 128).  -1: no instance for this Sp.
+template <int TYPE, bool DUAL, bool RMS, bool SEGS, int SP>
+int launch_fixed_sp(jl_context *ctx, const GemvParams &p, int lds, bool full) {
+    return full ? launch_tiles_of<TYPE, DUAL, RMS, false, 256, SP, SEGS, false>(ctx, p, 256, lds)
+                : launch_tiles_of<TYPE, DUAL, RMS, false, 256, SP, SEGS, true>(ctx, p, 256, lds);
+}
+template <int TYPE, bool DUAL, bool RMS, bool SEGS>
+int launch_fixed(jl_context *ctx, const GemvParams &p, int lds, bool full) {
+    switch (p.Sp) {
+        case 16: return launch_fixed_sp<TYPE, DUAL, RMS, SEGS, 16>(ctx, p, lds, full);
+        case 32: return launch_fixed_sp<TYPE, DUAL, RMS, SEGS, 32>(ctx, p, lds, full);
+        case 64: return launch_fixed_sp<TYPE, DUAL, RMS, SEGS, 64>(ctx, p, lds, full);
+        case 128: return launch_fixed_sp<TYPE, DUAL, RMS, SEGS, 128>(ctx, p, lds, full);
+        default: return -1;
+    }
+}
+
+// `fixed`: the launch meets the fixed-geometry form's conditions (whole tiles only in every
+// weight).  The three main types have an instance for every variant at row lengths of 513 ... 8192
+// columns and, in the 1024-thread form (plain and residual), up to 16384; the side types for
+// whole rows of 2048, 4096 and (plain and residual) 8192 columns.
 template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, bool fixed) {
-    // (Q6_K: plain, residual and gate/up only -- the caller has refused the rest)
+    // (side types: plain, residual and gate/up only -- the caller has refused the rest)
     constexpr bool kMain = is_main_type(TYPE);
     if constexpr (kMain) {
         if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
     }
     const bool full = fixed && p.S == p.Sp;
-    if constexpr (kMain) if (p.rms_w) {
-        // (the RMS-folding projections are q|k|v, gate/up and the vocabulary: rows of dim columns)
-        if (full && threads == 256 && (p.Sp == 32 || p.Sp == 64)) {
-            if constexpr (!DUAL) {
-                if (p.nseg > 1) {
-                    return p.Sp == 32 ? launch_tiles_of<TYPE, false, true, false, 256, 32, true>(ctx, p, threads, lds)
-                                      : launch_tiles_of<TYPE, false, true, false, 256, 64, true>(ctx, p, threads, lds);
-                }
-            }
-            return p.Sp == 32 ? launch_tiles_of<TYPE, DUAL, true, false, 256, 32>(ctx, p, threads, lds)
-                              : launch_tiles_of<TYPE, DUAL, true, false, 256, 64>(ctx, p, threads, lds);
-        }
-        // (rows of 3072 / 3584 / 5120 columns: 48 / 56 of 64 slices, 80 of 128)
-        if (fixed && !full && threads == 256 && (p.Sp == 64 || p.Sp == 128)) {
-            if constexpr (!DUAL) {
-                if (p.nseg > 1) {
-                    return p.Sp == 64
-                               ? launch_tiles_of<TYPE, false, true, false, 256, 64, true, true>(ctx, p, threads, lds)
-                               : launch_tiles_of<TYPE, false, true, false, 256, 128, true, true>(ctx, p, threads, lds);
-                }
-            }
-            return p.Sp == 64 ? launch_tiles_of<TYPE, DUAL, true, false, 256, 64, false, true>(ctx, p, threads, lds)
-                              : launch_tiles_of<TYPE, DUAL, true, false, 256, 128, false, true>(ctx, p, threads, lds);
-        }
-        return launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds);
-    }
-    if constexpr (!DUAL && kMain) {
-        if (full && threads == 256 && p.nseg > 1) {
-            if (p.Sp == 32) return launch_tiles_of<TYPE, false, false, false, 256, 32, true>(ctx, p, threads, lds);
-            if (p.Sp == 64) return launch_tiles_of<TYPE, false, false, false, 256, 64, true>(ctx, p, threads, lds);
-            return launch_tiles_of<TYPE, false, false>(ctx, p, threads, lds);
-        }
-        // (q|k|v over rows that fill their slices only in part)
-        if (fixed && !full && threads == 256 && p.nseg > 1) {
-            if (p.Sp == 64) return launch_tiles_of<TYPE, false, false, false, 256, 64, true, true>(ctx, p, threads, lds);
-            if (p.Sp == 128) return launch_tiles_of<TYPE, false, false, false, 256, 128, true, true>(ctx, p, threads, lds);
-        }
-    }
-    if (full && threads == 256) {
-        if (p.Sp == 32) return launch_tiles_of<TYPE, DUAL, false, false, 256, 32>(ctx, p, threads, lds);
-        if (p.Sp == 64) return launch_tiles_of<TYPE, DUAL, false, false, 256, 64>(ctx, p, threads, lds);
-        if constexpr (!DUAL || kMain) {
-            if (p.Sp == 128) return launch_tiles_of<TYPE, DUAL, false, false, 256, 128>(ctx, p, threads, lds);
-        }
-    }
-    // rows that fill their slices only in part (3072 columns: 48 of 64 slices; 5120: 80 of 128)
     if constexpr (kMain) {
-        if (fixed && !full && threads == 256 && p.nseg == 1) {
-            if (p.Sp == 64) return launch_tiles_of<TYPE, DUAL, false, false, 256, 64, false, true>(ctx, p, threads, lds);
-            if (p.Sp == 128) return launch_tiles_of<TYPE, DUAL, false, false, 256, 128, false, true>(ctx, p, threads, lds);
+        if (fixed && threads == 256) {
+            int st;
+            // (the RMS-folding projections are q|k|v, gate/up and the vocabulary: rows of dim columns)
+            if constexpr (DUAL) {
+                st = p.rms_w ? launch_fixed<TYPE, true, true, false>(ctx, p, lds, full)
+                             : launch_fixed<TYPE, true, false, false>(ctx, p, lds, full);
+            } else if (p.nseg > 1) {
+                st = p.rms_w ? launch_fixed<TYPE, false, true, true>(ctx, p, lds, full)
+                             : launch_fixed<TYPE, false, false, true>(ctx, p, lds, full);
+            } else {
+                st = p.rms_w ? launch_fixed<TYPE, false, true, false>(ctx, p, lds, full)
+                             : launch_fixed<TYPE, false, false, false>(ctx, p, lds, full);
+            }
+            if (st != -1) return st;
+        }
+        if (p.rms_w) return launch_tiles_of<TYPE, DUAL, true>(ctx, p, threads, lds);
+    } else {
+        if (full && threads == 256) {
+            if (p.Sp == 32) return launch_tiles_of<TYPE, DUAL, false, false, 256, 32>(ctx, p, threads, lds);
+            if (p.Sp == 64) return launch_tiles_of<TYPE, DUAL, false, false, 256, 64>(ctx, p, threads, lds);
+            if constexpr (!DUAL) {
+                if (p.Sp == 128) return launch_tiles_of<TYPE, false, false, false, 256, 128>(ctx, p, threads, lds);
+            }
         }
     }
     if constexpr (!DUAL) {

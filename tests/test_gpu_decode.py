@@ -163,13 +163,15 @@ def test_gemv_over_activation_magnitudes(ctx, t, scale):
     assert rel_err(out.get(), ref, magnitude(t, raw, x, d, n)) < 2e-5
 
 
-@pytest.mark.parametrize("n", [2048, 2560, 3072, 4096, 5120, 7168, 8192, 11008, 14336, 16384])
+@pytest.mark.parametrize("n", [768, 1024, 1536, 2048, 2560, 3072, 3584, 4096, 5120, 7168, 8192, 11008, 14336,
+                               16384])
 @pytest.mark.parametrize("t", [O.Q8_0, O.Q4_0, O.Q4_K])
 def test_fixed_geometry_and_general_kernels_give_the_same_bits(ctx, t, n):
     """A weight of whole tiles runs the kernel compiled for its row length (or, for rows that fill
-    their slices only in part -- 2560, 3072, 5120, 7168, 11008, 14336 columns -- for its slice count);
-    the same weight less its last row has a ragged last tile and runs the general one.  Same arithmetic in the same order:
-    the rows they share come out bit for bit equal (plain and gate/up)."""
+    their slices only in part -- 768, 1536, 2560, 3072, 3584, 5120, 7168, 11008, 14336 columns -- for
+    its slice count); the same weight less its last row has a ragged last tile and runs the general
+    one.  Same arithmetic in the same order: the rows they share come out bit for bit equal (plain,
+    gate/up, fused q|k|v and their RMS-folding forms)."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
     d = 272
@@ -178,6 +180,7 @@ def test_fixed_geometry_and_general_kernels_give_the_same_bits(ctx, t, n):
     raw_up = synthetic.weight(t, d, n, seed=1901 + n)
     row_bytes = raw.size // d
     x = ctx.from_numpy(synthetic.activations(n, seed=1902))
+    rms = ctx.from_numpy(np.random.default_rng(1903).uniform(0.5, 1.5, n).astype(np.float32))
     outs = []
     for rows in (d, d - 1):
         w = upload(ctx, t, raw[: rows * row_bytes], rows, n)
@@ -196,13 +199,26 @@ def test_fixed_geometry_and_general_kernels_give_the_same_bits(ctx, t, n):
         wv = upload(ctx, t, raw_up[: 64 * row_bytes], 64, n)
         proj.fusedQKV(x, q, k, v, w, wk, wv)
         ctx.sync()
-        outs.append((out.get(), hb.get(), q.get(), k.get(), v.get()))
+        got = [out.get(), hb.get(), q.get(), k.get(), v.get()]
+        if n <= 8192:
+            proj.rmsMatvec(x, rms, None, out, w, n, rows, eps=1e-5)
+            proj.fullyFusedRmsNormGateUp(x, rms, 1e-5, w, w_up, n, rows)
+            proj.fusedRmsNormQKV(x, q, k, v, rms, None, w, wk, wv, eps=1e-5)
+            ctx.sync()
+            got += [out.get(), hb.get(), q.get(), k.get(), v.get()]
+        outs.append(got)
     assert bits_equal(outs[0][0][: d - 1], outs[1][0])
     if n <= 8192:
         assert bits_equal(outs[0][1][: d - 1], outs[1][1])
         assert bits_equal(outs[0][2][: d - 1], outs[1][2])
         assert bits_equal(outs[0][3], outs[1][3]) and bits_equal(outs[0][4], outs[1][4])
         assert bits_equal(outs[0][2], outs[0][0])   # q of the fused call = the plain projection
+        # the RMS-folding forms
+        assert bits_equal(outs[0][5][: d - 1], outs[1][5])
+        assert bits_equal(outs[0][6][: d - 1], outs[1][6])
+        assert bits_equal(outs[0][7][: d - 1], outs[1][7])
+        assert bits_equal(outs[0][8], outs[1][8]) and bits_equal(outs[0][9], outs[1][9])
+        assert bits_equal(outs[0][7], outs[0][5])
 
 
 def _random_shapes():
