@@ -287,6 +287,16 @@ jl_gemm_hh(DenseParams p) {
     constexpr int AHEAD = NS - 1;
     constexpr int LA = DBM * 8 / 512;          // 16-byte loads per thread and stage, A part
     constexpr int LW = BN * 8 / 512;
+    // Cache prefetch of the weight operand, 256 x 256 tiles: their two-stage ring looks ahead by one
+    // step, about a microsecond -- enough for operands that come from the caches, just short for
+    // weights that come from HBM, as a model's successive layers' do.  Wave 0 therefore touches 64
+    // cache lines (a tile row's 128 bytes of a step each, one 4-byte LDS-DMA load into a spare KB
+    // behind the ring) of the step PFD steps past every stage it brings in; the workgroups that
+    // share a weight tile take a quarter of its rows each.  Measured on weights from HBM: gate/up
+    // at 2048 tokens 126 -> 122 us; with the weights in the memory-side cache it costs 1-2 us, and
+    // the smaller tiles (deeper rings, shorter steps) lose more than they gain and go without.
+    constexpr int PFW = NS == 2 ? 1 : 0;
+    constexpr int PFD = 2;
     static_assert(NB == 4, "four column blocks per wave");
     static_assert(BM == 256 || (BM == 128 && BN == 128), "row tiles: 256, or 128 with 128 columns");
 
@@ -328,6 +338,7 @@ jl_gemm_hh(DenseParams p) {
     }
 
     const uint32_t toff = (uint32_t)(tid >> 3) * (uint32_t)(p.k * 2) + (uint32_t)(((tid & 7) ^ ((tid >> 4) & 7)) << 4);
+
     for (int item = slot; item < per_xcd * p.splits; item += slots) {
         const int split = item / per_xcd;
         const int logical = xcd * per_xcd + (item - split * per_xcd);
@@ -357,9 +368,21 @@ jl_gemm_hh(DenseParams p) {
                 __builtin_amdgcn_global_load_lds((gvoid *)(w_item + (n - LA) * slot_stride + (int64_t)s * 128 + toff),
                                                  (lvoid *)(dst + DBM * 128 + ((n - LA) * 512 + wave * 64) * 16), 16, 0, 0);
         };
+        // after stage s's last load (past the last step: its own line again, so that the count of
+        // loads per stage does not change)
+        // (the GM workgroups that share this weight tile touch a GM-th of its rows each)
+        const uint32_t pf_off = (uint32_t)((mt - group * GM) * (BN / GM) + (lane & (BN / GM - 1))) * (uint32_t)(p.k * 2);
+        auto prefetch = [&](int s) {
+            if (wave < PFW) {
+                const int ps = s + PFD < ksteps ? s + PFD : ksteps - 1;
+                __builtin_amdgcn_global_load_lds((gvoid *)(w_item + (int64_t)ps * 128 + pf_off),
+                                                 (lvoid *)(lds + NS * STAGE + wave * 256), 4, 0, 0);
+            }
+        };
         auto issue = [&](int s) {
 #pragma unroll
             for (int n = 0; n < LA + LW; n++) issue_one(s, n);
+            prefetch(s);
         };
 
         floatx4 acc[MB][NB];
@@ -405,16 +428,24 @@ jl_gemm_hh(DenseParams p) {
                 if (loads) {
 #pragma unroll
                     for (int n = i * PER; n < (i + 1) * PER && n < LA + LW; n++) issue_one(next, n);
+                    if (i == MB - 1) prefetch(next);
                 }
             }
         };
-        // stage s landed (this thread's part); the AHEAD - 1 younger stages may be in flight
+        // stage s landed (this thread's part); the AHEAD - 1 younger stages may be in flight, and in
+        // a prefetching wave the line touched after each stage, that of stage s included
         auto stage_ready = [&](int s) {
             const int left = ksteps - 1 - s;
             const int younger = left < AHEAD - 1 ? left : AHEAD - 1;
-            if (younger >= 2) JL_WAIT_VM(2 * (LA + LW));
-            else if (younger == 1) JL_WAIT_VM(LA + LW);
-            else JL_WAIT_VM(0);
+            if (wave < PFW) {
+                if (younger >= 2) JL_WAIT_VM(2 * (LA + LW + 1) + 1);
+                else if (younger == 1) JL_WAIT_VM(LA + LW + 2);
+                else JL_WAIT_VM(1);
+            } else {
+                if (younger >= 2) JL_WAIT_VM(2 * (LA + LW));
+                else if (younger == 1) JL_WAIT_VM(LA + LW);
+                else JL_WAIT_VM(0);
+            }
             __builtin_amdgcn_s_barrier();
         };
         // (the slot that stage s + AHEAD goes to held stage s - 1, last read before barrier s)
@@ -537,7 +568,7 @@ jl_gemm_hh(DenseParams p) {
 template <int BM, int BN>
 int launch_dense(jl_context *ctx, const DenseParams &p) {
     auto fn = jl_gemm_hh<BM, BN>;
-    constexpr int lds = hh_stages<BM, BN>() * (BM + BN) * 128;
+    constexpr int lds = hh_stages<BM, BN>() * (BM + BN) * 128 + 1024;   // the ring and the prefetch's landing KB
     static bool configured[16] = {};
     if (ctx->device < 16 && !configured[ctx->device]) {
         JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
