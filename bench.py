@@ -794,15 +794,17 @@ def decode_probe(ctx, proj, layers, wcls, acts):
 def prefill_probe(ctx, t, T=2048, mode="xf16"):
     """What the matrix-pipe counters (`rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F16 SQ_VALU_MFMA_BUSY_CYCLES
     SQ_BUSY_CU_CYCLES GRBM_GUI_ACTIVE`) and the prefill kernel traces are collected on: one
-    Llama-3.2-1B layer's four prefill calls at T tokens, launched kernel by kernel -- no graph, so that
-    every dispatch has a row of its own -- four times.  Mode "xf16": resident fp16 copy and fp16
+    Llama-3.2-1B layer's four prefill calls at T tokens over PREFILL_LAYERS distinct sets of weights
+    in turn (so that they are read from HBM), launched kernel by kernel -- no graph, so that every
+    dispatch has a row of its own -- four passes.  Mode "xf16": resident fp16 copy and fp16
     activations (every call is then one launch of the fp16 GEMM, plus a fold where K is cut; the first
     pass decodes the copy); "resident": the copy with fp32 activations; "default": plain `jl_gemm`."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
     shapes = {"wq": (DIM, DIM), "wk": (KV_DIM, DIM), "wv": (KV_DIM, DIM), "wo": (DIM, DIM),
               "w1": (HIDDEN, DIM), "w3": (HIDDEN, DIM), "w2": (DIM, HIDDEN)}
-    w = {k: ctx.load_weight(t, synthetic.weight(t, r, c, 41 + i), r, c) for i, (k, (r, c)) in enumerate(shapes.items())}
+    host = {k: synthetic.weight(t, r, c, 41 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
+    layers = [{k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes} for _ in range(PREFILL_LAYERS)]
     x_host = synthetic.activations((T, DIM), 48)
     h_host = synthetic.activations((T, HIDDEN), 49) * np.float32(0.1)
     qkv, res = ctx.float_array(T * (DIM + 2 * KV_DIM)), ctx.float_array(T * DIM, fill=0.0)
@@ -812,12 +814,13 @@ def prefill_probe(ctx, t, T=2048, mode="xf16"):
         x, h, hb = ctx.from_numpy(x_host), ctx.from_numpy(h_host), ctx.float_array(T * HIDDEN)
     proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=mode != "default")
     for _ in range(4):
-        proj.fusedQKV(x, qkv, w["wq"], w["wk"], w["wv"])
-        proj.projection(x, res, w["wo"], DIM, DIM, True)
-        proj.gateUp(x, hb, w["w1"], w["w3"], DIM, HIDDEN)
-        proj.projection(h, res, w["w2"], HIDDEN, DIM, True)
+        for w in layers:
+            proj.fusedQKV(x, qkv, w["wq"], w["wk"], w["wv"])
+            proj.projection(x, res, w["wo"], DIM, DIM, True)
+            proj.gateUp(x, hb, w["w1"], w["w3"], DIM, HIDDEN)
+            proj.projection(h, res, w["w2"], HIDDEN, DIM, True)
         ctx.sync()
-    print(json.dumps({"tokens": T, "mode": mode, "flops": {"q|k|v": 2.0 * T * DIM * (DIM + 2 * KV_DIM), "o": 2.0 * T * DIM * DIM,
+    print(json.dumps({"tokens": T, "mode": mode, "layers_swept": PREFILL_LAYERS, "passes": 4, "flops": {"q|k|v": 2.0 * T * DIM * (DIM + 2 * KV_DIM), "o": 2.0 * T * DIM * DIM,
                                              "gate/up": 2.0 * T * 2 * HIDDEN * DIM, "down": 2.0 * T * HIDDEN * DIM},
                       "mfma_f16_flops_per_instruction_16x16x32": 2 * 16 * 16 * 32}))
 
