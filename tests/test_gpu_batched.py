@@ -306,6 +306,44 @@ def test_two_pass_prefill_tiles_and_edges(ctx, t, d, n, T, residual):
     assert np.all(excess <= 5e-4 * magnitude(t, raw, X, d, n)), float(excess.max())
 
 
+def _random_prefill_shapes():
+    """Seeded many-row shapes across both prefill kernels and every tiling: 65 .. 1400 rows, row
+    lengths of 256 .. 4096 columns, output widths from a fraction of a tile to dozens of tiles,
+    partial batches, both epilogues (sizes kept to what the oracle multiplies in seconds)."""
+    rng = np.random.default_rng(20261126)
+    shapes = []
+    for t in (O.Q8_0, O.Q4_0, O.Q4_K):
+        for n in (256, 1024, 2048, 4096):
+            T = int(rng.integers(65, 1401))
+            d = int(rng.integers(40, max(41, min(5000, int(1.6e9 // (T * n))))))
+            active = T if rng.integers(0, 2) else int(rng.integers(T // 2, T + 1))
+            shapes.append((t, d, n, T, active, bool(rng.integers(0, 2))))
+    return shapes
+
+
+@pytest.mark.parametrize("t,d,n,T,active,residual", _random_prefill_shapes())
+def test_prefill_on_random_shapes(ctx, t, d, n, T, active, residual):
+    """Many-row projections of random shape against the oracle; rows past the active ones and
+    whatever lies behind the output keep their contents."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("prefill, random shape", NAMES[t], d, n, T, active, residual)
+    raw = synthetic.weight(t, d, n, seed=8600 + d)
+    X = synthetic.activations((T, n), seed=8700 + T)
+    ref = O.matmul_batch(t, raw, X[:active], d, n)
+    out = ctx.float_array(T * d + 64, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, d).projection(ctx.from_numpy(X), out, ctx.load_weight(t, raw, d, n),
+                                                       n, d, residual, activeRows=active)
+    ctx.sync()
+    flat = out.get()
+    assert np.all(flat[active * d:] == UNTOUCHED)
+    got = flat[:active * d].reshape(active, d)
+    want = ref.astype(np.float64) + (float(UNTOUCHED) if residual else 0.0)
+    slack = abs(np.spacing(np.float32(UNTOUCHED))) / 2 if residual else 0.0
+    excess = np.abs(got.astype(np.float64) - want) - slack
+    assert np.all(excess <= F16_BOUND * magnitude(t, raw, X[:active], d, n)), float(excess.max())
+
+
 def test_two_pass_prefill_qkv_and_gate_up(ctx):
     """The decode-once path with several weights in one call: q|k|v of unequal widths side by side,
     and gate/up interleaved by half tiles with a last tile of 8 outputs."""
