@@ -234,6 +234,9 @@ def _random_shapes():
             shapes.append((t, d, n))
         for n in (2048, 4096, 8192, 12288):
             shapes.append((t, int(rng.integers(1, 40)) * 8, n))   # whole tiles
+    for t in (O.Q8_0, O.Q4_0, O.Q4_K):   # (appended: the shapes above keep their seeds)
+        for n in (768, 1024, 1536, 3072, 3584, 5120):
+            shapes.append((t, int(rng.integers(1, 20)) * 16, n))  # whole tiles of the other row lengths
     return shapes
 
 
