@@ -487,7 +487,10 @@ def bench_gemm(ctx, hip, t, T, steps, warmup, cpu, clock_khz, cu):
             rms_proj.rmsApplyFP16(X, rms_w, 1e-5, X16, DIM)
     rms_us = statistics.median(timed_graph(ctx, hip, rms_apply, steps, 3)) / 8 * 1e3
     half["rms_apply_to_fp16_us"] = round(rms_us, 2)
-    out = {"tokens": T, "layers_swept": PREFILL_LAYERS, "ms_per_layer": default["ms_per_layer"],
+    out = {"tokens": T, "layers_swept": PREFILL_LAYERS,
+           "weights_from": f"HBM: {PREFILL_LAYERS} layers' distinct weights in turn (their fp16 copies, "
+                           f"{PREFILL_LAYERS} x 121 MB, exceed the 256 MB memory-side cache)",
+           "ms_per_layer": default["ms_per_layer"],
            "ms_stats": default["ms_stats"],
            "tok_s_16_layers": round(T / (default["ms_per_layer"] * 1e-3 * LAYERS), 1),
            "tflops": default["tflops"], "frac_f16_mfma_peak": default["frac_f16_mfma_peak"],
