@@ -45,6 +45,12 @@ UNSTABLE_SPREAD = 0.10
 # Llama-3.2-1B geometry: the decode projection set the headline metric is quoted on
 DIM, KV_DIM, HIDDEN, VOCAB, LAYERS = 2048, 512, 8192, 128256, 16
 PREFILL_LAYERS = 4                   # distinct weight sets a prefill leg sweeps (fp16 copies: 4 x 121 MB)
+# Layer copies the batched-decode and the Q4_0 / Q4_K decode legs sweep in one replayed graph: far
+# more than the 256 MB memory-side cache holds (8 x 109 MB, 10 x 123 MB), and enough layers to a
+# replay that the pause between two replays (a model runs 32 or more layers per replay) is a small
+# part of what a layer is charged: with 3 and 4 copies the same kernels read 3-4 % slower.
+BATCHED_COPIES = 8
+OTHER_TYPE_COPIES = 10
 
 
 class Hip:
@@ -519,8 +525,9 @@ def bench_batched_q4k(ctx, hip, B, steps, warmup, cpu):
     shapes = {"wq": (dim, dim), "wk": (kv, dim), "wv": (kv, dim), "wo": (dim, dim),
               "w1": (ffn, dim), "w3": (ffn, dim), "w2": (dim, ffn)}
     host = {k: synthetic.weight(t, r, c, 61 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
-    # enough copies of the layer that a replay cannot be served from the 256 MB memory-side cache
-    copies = 3
+    # enough copies of the layer (109 MB each) that a replay cannot be served from the 256 MB
+    # memory-side cache, whatever it keeps of what it has seen
+    copies = BATCHED_COPIES
     layers = [{k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes} for _ in range(copies)]
     Xh = synthetic.activations((B, dim), 68)
     Hh = synthetic.activations((B, ffn), 69) * np.float32(0.1)
@@ -1150,8 +1157,8 @@ def main():
                         leg["roofline"]["achieved"] / sustained["16x16x32_random_operands"], 4))
         if "other_types" in legs:
             out["decode_other_types"] = [
-                bench_decode_layers(ctx, hip, "Q4_0", 4096, 1024, 14336, 4, args.steps, args.warmup, cpu),
-                bench_decode_layers(ctx, hip, "Q4_K", 4096, 1024, 12288, 4, args.steps, args.warmup, cpu)]
+                bench_decode_layers(ctx, hip, "Q4_0", 4096, 1024, 14336, OTHER_TYPE_COPIES, args.steps, args.warmup, cpu),
+                bench_decode_layers(ctx, hip, "Q4_K", 4096, 1024, 12288, OTHER_TYPE_COPIES, args.steps, args.warmup, cpu)]
         if "batched" in legs:
             out["batched_q4k"] = [bench_batched_q4k(ctx, hip, B, max(5, args.steps // 5), 3, cpu)
                                   for B in (8, 32, 64)]
