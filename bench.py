@@ -764,6 +764,24 @@ def traffic_probe(ctx, proj, layers):
                                   "algorithmic_write_bytes": 4 * HIDDEN}}))
 
 
+def roofline_probe(ctx, hip, proj, layers, replays=12):
+    """What the kernel trace behind `roofline.avg_launch_us` is collected on: the fused gate/up GEMV
+    launched the way the benchmark's roofline leg launches it -- one HIP graph of four sweeps over
+    the 16 layers' distinct weights, 64 launches back to back, replayed `replays` times -- so that
+    the tracer's per-dispatch durations are of launches that follow one another as in the timed
+    leg, not of launches enqueued one by one from Python.  Prints the HIP-event figure of the same
+    replays (what the benchmark itself reports) beside the launch count the trace must hold."""
+    def sweeps():
+        for _ in range(4):
+            for w in layers:
+                proj.gateUp(w["w1"], w["w3"], DIM, HIDDEN)
+    us = [m / (4 * LAYERS) * 1e3 for m in timed_graph(ctx, hip, sweeps, replays, 2, reps=3)]
+    print(json.dumps({"roofline_probe": {"kernel": "gate/up GEMV 2 x [8192 x 2048]", "launches_per_replay": 4 * LAYERS,
+                                         "replays": 2 + 3 * replays, "launches_outside_graph": 4 * LAYERS,
+                                         "bytes_per_launch": 2 * gemv_bytes(HIDDEN, DIM),
+                                         "hip_event_us_per_launch": spread_stats(us, 1.0, 3)}}))
+
+
 def decode_probe(ctx, proj, layers, wcls, acts):
     """What the kernel trace of the decode kernels is collected on: the 65 launches of a decode
     step, kernel by kernel (no graph: a tracer serialises a replayed graph anyway), six steps over
@@ -954,6 +972,8 @@ def main():
                     help="only launch the batched-decode calls, kernel by kernel (see batched_probe)")
     ap.add_argument("--decode-probe", action="store_true",
                     help="only launch the decode kernels, kernel by kernel (see decode_probe)")
+    ap.add_argument("--roofline-probe", action="store_true",
+                    help="only replay the roofline leg's graph of gate/up launches (see roofline_probe)")
     ap.add_argument("--int8-probe", action="store_true",
                     help="only launch the int8 prefill calls, kernel by kernel (see int8_probe)")
     args = ap.parse_args()
@@ -998,6 +1018,9 @@ def main():
             return
         if args.decode_probe:
             decode_probe(ctx, proj, layers, wcls, acts)
+            return
+        if args.roofline_probe:
+            roofline_probe(ctx, hip, proj, layers)
             return
         total_bytes = decode_bytes()
         assert total_bytes == 1316320256, total_bytes

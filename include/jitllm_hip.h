@@ -98,7 +98,9 @@ int jl_device_info(jl_context *ctx, int *compute_units, char *name, size_t name_
 
 int jl_malloc(jl_context *ctx, size_t bytes, void **device_ptr);
 int jl_free(jl_context *ctx, void *device_ptr);
-/* Stream-ordered copies; the host side has returned only after the copy completed. */
+/* Stream-ordered copies; the host side has returned only after the copy completed.  The host
+ * pointer may be pageable (a heap segment, a mapped file): it is copied through pinned staging
+ * memory the context owns, 8 MiB at a time, so neither call is legal inside a stream capture. */
 int jl_upload(jl_context *ctx, void *device_dst, const void *host_src, size_t bytes);
 int jl_download(jl_context *ctx, void *host_dst, const void *device_src, size_t bytes);
 /* Fills `count` floats with `value` (FloatArray.init). */

@@ -23,6 +23,15 @@ int jl_abi_version(void) { return JL_ABI_VERSION; }
 
 const char *jl_last_error(void) { return g_error; }
 
+static void context_release(jl_context *ctx) {
+    for (int i = 0; i < 2; i++)
+        if (ctx->bounce_done[i]) (void)hipEventDestroy(ctx->bounce_done[i]);
+    if (ctx->bounce) (void)hipHostFree(ctx->bounce);
+    if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
 static int context_create(int device, hipStream_t borrowed, bool borrow, jl_context **out) {
     JL_REQUIRE(out != nullptr, "jl_context_create: out is null");
     *out = nullptr;
@@ -57,11 +66,12 @@ static int context_create(int device, hipStream_t borrowed, bool borrow, jl_cont
         }
         ctx->owns_stream = true;
     }
-    const hipError_t e = hipMalloc(&ctx->scratch, JL_CONTEXT_SCRATCH_BYTES);   // written before it is read
+    hipError_t e = hipMalloc(&ctx->scratch, JL_CONTEXT_SCRATCH_BYTES);   // written before it is read
+    if (e == hipSuccess) e = hipHostMalloc((void **)&ctx->bounce, 2 * (size_t)JL_BOUNCE_HALF_BYTES, hipHostMallocDefault);
+    for (int i = 0; i < 2 && e == hipSuccess; i++) e = hipEventCreateWithFlags(&ctx->bounce_done[i], hipEventDisableTiming);
     if (e != hipSuccess) {
-        if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
-        delete ctx;
-        return jl_fail(JL_ERR_OOM, "jl_context_create: scratch allocation failed: %s", hipGetErrorString(e));
+        context_release(ctx);
+        return jl_fail(JL_ERR_OOM, "jl_context_create: scratch / staging allocation failed: %s", hipGetErrorString(e));
     }
     *out = ctx;
     return JL_OK;
@@ -79,9 +89,7 @@ int jl_context_destroy(jl_context *ctx) {
     if (!ctx) return JL_OK;
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
-    if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
-    (void)hipFree(ctx->scratch);
-    delete ctx;
+    context_release(ctx);
     return JL_OK;
 }
 
@@ -120,10 +128,28 @@ int jl_free(jl_context *ctx, void *device_ptr) {
     return JL_OK;
 }
 
+// Host memory handed to these two is the caller's, pageable as a rule (a Java heap segment, a numpy
+// array, a mapped file).  It is copied through the context's pinned staging halves in turn, so the
+// device only ever runs DMA transfers against pinned memory and the runtime's own handling of
+// pageable pointers (staging of its own, or host writes straight into device memory) is not used.
 int jl_upload(jl_context *ctx, void *device_dst, const void *host_src, size_t bytes) {
     JL_REQUIRE(ctx && (bytes == 0 || (device_dst && host_src)), "jl_upload: null argument");
     if (!bytes) return JL_OK;
-    JL_HIP(hipMemcpyAsync(device_dst, host_src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    JL_HIP(hipSetDevice(ctx->device));
+    const uint8_t *src = (const uint8_t *)host_src;
+    uint8_t *dst = (uint8_t *)device_dst;
+    int half = 0;
+    bool used[2] = {false, false};
+    for (size_t done = 0; done < bytes; half ^= 1) {
+        const size_t n = bytes - done < JL_BOUNCE_HALF_BYTES ? bytes - done : (size_t)JL_BOUNCE_HALF_BYTES;
+        uint8_t *stage = ctx->bounce + (size_t)half * JL_BOUNCE_HALF_BYTES;
+        if (used[half]) JL_HIP(hipEventSynchronize(ctx->bounce_done[half]));   // its last transfer has left it
+        memcpy(stage, src + done, n);
+        JL_HIP(hipMemcpyAsync(dst + done, stage, n, hipMemcpyHostToDevice, ctx->stream));
+        JL_HIP(hipEventRecord(ctx->bounce_done[half], ctx->stream));
+        used[half] = true;
+        done += n;
+    }
     JL_HIP(hipStreamSynchronize(ctx->stream));
     return JL_OK;
 }
@@ -131,8 +157,29 @@ int jl_upload(jl_context *ctx, void *device_dst, const void *host_src, size_t by
 int jl_download(jl_context *ctx, void *host_dst, const void *device_src, size_t bytes) {
     JL_REQUIRE(ctx && (bytes == 0 || (host_dst && device_src)), "jl_download: null argument");
     if (!bytes) return JL_OK;
-    JL_HIP(hipMemcpyAsync(host_dst, device_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
-    JL_HIP(hipStreamSynchronize(ctx->stream));
+    JL_HIP(hipSetDevice(ctx->device));
+    uint8_t *dst = (uint8_t *)host_dst;
+    const uint8_t *src = (const uint8_t *)device_src;
+    // chunk i + 1 is on its way into the other half while chunk i is copied out to the caller
+    size_t issued = 0, copied = 0;
+    size_t len[2] = {0, 0};
+    int half = 0;
+    auto issue = [&](int h) -> hipError_t {
+        len[h] = bytes - issued < JL_BOUNCE_HALF_BYTES ? bytes - issued : (size_t)JL_BOUNCE_HALF_BYTES;
+        hipError_t e = hipMemcpyAsync(ctx->bounce + (size_t)h * JL_BOUNCE_HALF_BYTES, src + issued, len[h],
+                                      hipMemcpyDeviceToHost, ctx->stream);
+        if (e == hipSuccess) e = hipEventRecord(ctx->bounce_done[h], ctx->stream);
+        issued += len[h];
+        return e;
+    };
+    JL_HIP(issue(0));
+    while (copied < bytes) {
+        if (issued < bytes) JL_HIP(issue(half ^ 1));
+        JL_HIP(hipEventSynchronize(ctx->bounce_done[half]));
+        memcpy(dst + copied, ctx->bounce + (size_t)half * JL_BOUNCE_HALF_BYTES, len[half]);
+        copied += len[half];
+        half ^= 1;
+    }
     return JL_OK;
 }
 

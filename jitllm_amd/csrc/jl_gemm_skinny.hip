@@ -66,20 +66,7 @@ struct SkinnyParams {
     int span_bytes;           // bytes of a weight row inside one span
     int stages;               // depth of the tile ring
     int row_blocks;           // gridDim.y: blocks of 16 NBB activation rows, each on its own workgroups
-#ifdef JL_SKINNY_PROBE
-    int probe;                // timing experiments: parts of the kernel switched off
-    uint32_t *stamps;         // cycle stamps of workgroup 8: [wave][96]
-    int lds_total;
-#endif
 };
-#ifdef JL_SKINNY_PROBE
-#define PROBE(x) (p.probe == (x))
-#define STAMP(slot) do { if (p.stamps && blockIdx.x == 8 && blockIdx.y == 0) { const uint32_t t_ = (uint32_t)__builtin_readcyclecounter(); \
-    if (lane == 0 && (slot) < 96) asm volatile("ds_write_b32 %0, %1" :: "v"(lds0 + p.lds_total + 4 * (wave * 96 + (slot))), "v"(t_) : "memory"); } } while (0)
-#else
-#define PROBE(x) false
-#define STAMP(slot) do { } while (0)
-#endif
 
 #define JL_WAIT_VM(N) \
     __builtin_amdgcn_s_waitcnt(((N)&0xF) | (((N) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
@@ -367,8 +354,6 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     const int wg = blockIdx.x / p.Z;
     const int stride = gridDim.x / p.Z;
     int mine = wg < total_groups ? (total_groups - wg + stride - 1) / stride : 0;
-    if (PROBE(4)) return;          // launch only
-    if (PROBE(3)) mine = 0;        // launch + activation prologue
 
     if (wave >= waves && wave < waves + kDmaWaves) {
         // ---- copy waves.  Slot s of a tile is 16 bytes at LDS offset 16 s: row s / slots_per_row,
@@ -419,7 +404,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                 // every row of the group exists (uniform; all groups but a weight's last)
 #pragma unroll
                 for (int j = 0; j < LD; j++) {
-                    if (j >= n_loads || PROBE(2)) break;
+                    if (j >= n_loads) break;
                     __builtin_amdgcn_global_load_lds((gvoid *)(w_gate + slot_off[j]),
                                                      (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, 0);
                 }
@@ -440,20 +425,16 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             issue(issued, next_stage);
             next_stage = next_stage + 1 == p.stages ? 0 : next_stage + 1;
         }
-        STAMP(0);
         for (int t = 0; t < tiles; t++) {
             // tiles issued after tile t may stay in flight
             wait_vm((issued - t - 1) * n_loads);
-            STAMP(1 + 3 * t);
             __builtin_amdgcn_s_barrier();
-            STAMP(2 + 3 * t);
             // the stage of tile t - 1 is free now: every compute wave is past its reads
             if (issued < tiles) {
                 issue(issued, next_stage);
                 next_stage = next_stage + 1 == p.stages ? 0 : next_stage + 1;
                 issued++;
             }
-            STAMP(3 + 3 * t);
         }
         if (mine > 0) __builtin_amdgcn_s_barrier();
         return;
@@ -534,12 +515,10 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         int folded = 0;
         for (int t = 0; t < tiles; t++) {
             __builtin_amdgcn_s_barrier();
-            STAMP(2 * t);
             if (folded < mine && (folded + 1) * ZIN + 1 <= t) {
                 fold(wg + folded * stride, folded % kParities);
                 folded++;
             }
-            STAMP(2 * t + 1);
         }
         if (mine > 0) {
             __builtin_amdgcn_s_barrier();
@@ -560,7 +539,6 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     // fp16's subnormals and the sum of a sub-block's 32 activations inside fp16's range.  The
     // results of activation row r sit in lane group r / 4 of every weight row's lanes, so each lane
     // fetches the four scales it has to undo from the lanes that computed them.
-    STAMP(0);
     half8 af[NBB][ZIN][8];
     half8 sums[NBB][ZIN];     // Q4_K: the two sub-blocks' activation sums, each as hi + lo, as k slots
     floatx4 undo[NBB][ZIN];
@@ -676,8 +654,6 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             }
         }
     }
-
-    STAMP(1);
     // One tile: the slice's fragments against the activation fragments of span q, added to `total`.
     auto multiply = [&](int q, const half8 (&wf)[8], const Q4KTail &tail, floatx4 (&total)[NBB]) {
 #pragma unroll
@@ -718,18 +694,13 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
 #pragma unroll
             for (int q = 0; q < ZIN; q++) {
                 const int t = it * ZIN + q;
-                STAMP(2 + 4 * t);
                 __builtin_amdgcn_s_barrier();   // tile t has landed
-                STAMP(3 + 4 * t);
-                if (PROBE(1)) continue;   // copy only
                 half8 wf[8];
                 Q4KTail tail;
                 decode_slice<TYPE>(ring0 + (t % p.stages) * stage_bytes + c * lds_row, sl, wf, tail);
                 asm volatile("" : "+v"(wf[0]), "+v"(wf[7]));
-                STAMP(4 + 4 * t);
                 multiply(q, wf, tail, total);
             }
-            STAMP(5 + 4 * (it * ZIN + ZIN - 1));
             publish(it, total);
         }
     } else {
@@ -742,10 +713,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
 #pragma unroll
             for (int q = 0; q < ZIN; q++) {
                 const int t = it * ZIN + q;
-                STAMP(2 + 4 * t);
                 __builtin_amdgcn_s_barrier();   // tile t has landed
-                STAMP(3 + 4 * t);
-                if (PROBE(1)) continue;   // copy only
                 if (t > 0) {
                     // tile t - 1: span (q - 1) mod ZIN, the last of its group when q == 0
                     multiply(q == 0 ? ZIN - 1 : q - 1, wf, tail, total);
@@ -755,28 +723,16 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                         for (int b = 0; b < NBB; b++) total[b] = floatx4{0.f, 0.f, 0.f, 0.f};
                     }
                 }
-                STAMP(4 + 4 * t);
                 decode_slice<TYPE>(ring0 + (t % p.stages) * stage_bytes + c * lds_row, sl, wf, tail);
                 asm volatile("" : "+v"(wf[0]), "+v"(wf[7]));
-                STAMP(5 + 4 * t);
             }
         }
-        if (mine > 0 && !PROBE(1)) {
+        if (mine > 0) {
             multiply(ZIN - 1, wf, tail, total);
             publish(mine - 1, total);
         }
     }
     if (mine > 0) __builtin_amdgcn_s_barrier();
-#ifdef JL_SKINNY_PROBE
-    if (p.stamps && blockIdx.x == 8 && blockIdx.y == 0 && wave == 0) {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        for (int i = lane; i < 16 * 96; i += 64) {
-            uint32_t v;
-            asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds0 + p.lds_total + 4 * i) : "memory");
-            p.stamps[i] = v;
-        }
-    }
-#endif
 }
 
 // Adds the spans' partial sums in span order and applies the epilogue; one thread per activation
@@ -852,11 +808,6 @@ __global__ void __launch_bounds__(256) jl_skinny_reduce(SkinnyParams p, int padd
     }
 }
 
-#ifdef JL_SKINNY_PROBE
-#define JL_PROBE_LDS 6144
-#else
-#define JL_PROBE_LDS 0
-#endif
 template <int TYPE, int NBB, bool DUAL, int ZIN, bool HALF = false>
 int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int groups) {
     auto fn = jl_gemm_skinny<TYPE, NBB, DUAL, ZIN, HALF>;
@@ -873,7 +824,7 @@ int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int gro
     if (p.row_blocks > 1) per_span = per_span / 8 * 8;
     if (per_span < 1) per_span = 1;
     if (per_span > groups) per_span = groups;
-    hipLaunchKernelGGL(fn, dim3(per_span * p.Z, p.row_blocks), dim3(threads + 64 * (kDmaWaves + kFoldWaves)), lds + JL_PROBE_LDS,
+    hipLaunchKernelGGL(fn, dim3(per_span * p.Z, p.row_blocks), dim3(threads + 64 * (kDmaWaves + kFoldWaves)), lds,
                        ctx->stream, p);
     JL_HIP(hipGetLastError());
     if (p.Z > 1) {
@@ -949,9 +900,6 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     p.Ss = Ss;
     p.Z = Z;
     p.row_blocks = row_blocks;
-#ifdef JL_SKINNY_PROBE
-    p.probe = getenv("JL_SKINNY_PROBE") ? atoi(getenv("JL_SKINNY_PROBE")) : 0;
-#endif
     p.span_bytes = Ss * (type == JL_Q8_0 ? 68 : 36);
     if (Z > 1 && (size_t)Z * (16 * nbb * row_blocks) * groups * 16 * sizeof(float) > plane_bytes) return JL_OK;
 
@@ -969,21 +917,6 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     p.stages = stages;
     const int lds = partial + stages * stage_bytes;
     *taken = true;
-#ifdef JL_SKINNY_PROBE
-    p.lds_total = lds;
-    {
-        static uint32_t *stamp_buf = nullptr;
-        if (!stamp_buf && getenv("JL_SKINNY_STAMPS")) (void)hipMalloc(&stamp_buf, 16 * 96 * 4);
-        p.stamps = stamp_buf;
-        if (stamp_buf && getenv("JL_SKINNY_STAMPS_DUMP")) {
-            static uint32_t host[16 * 96];
-            (void)hipDeviceSynchronize();
-            (void)hipMemcpy(host, stamp_buf, sizeof host, hipMemcpyDeviceToHost);
-            FILE *f = fopen(getenv("JL_SKINNY_STAMPS_DUMP"), "wb");
-            if (f) { fwrite(host, 1, sizeof host, f); fclose(f); }
-        }
-    }
-#endif
 
     switch (type) {
         case JL_Q8_0:

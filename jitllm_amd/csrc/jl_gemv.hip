@@ -693,14 +693,6 @@ __device__ __forceinline__ uintptr_t uniform_value(uintptr_t v) {
     return v;
 }
 
-#ifdef JL_GEMV_STAMPS
-// Timing experiments only: the 100 MHz real-time counter at eight points of every workgroup's
-// life, kept in scalar registers and written out when the workgroup is done.
-__device__ uint64_t *jl_gemv_stamp_buf = nullptr;
-#define GSTAMP(k) do { stamp[k] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define GSTAMP(k) do { } while (0)
-#endif
 
 // SPT != 0 is the kernel for the usual launch, with its geometry known to the compiler: rows of
 // exactly SPT slices (a power of two), THREADS / SPT rows per tile and, in every segment, a row
@@ -728,10 +720,6 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     constexpr bool FULL = LEAN && !PART;   // every lane has a slice, every load slot is real data
     static_assert(!PART || LEAN, "rows shorter than SPT slices: a fixed tile shape");
     static_assert(!LEAN || !PACKED, "the packed form has no fixed-geometry instances");
-#ifdef JL_GEMV_STAMPS
-    uint64_t stamp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#endif
-    GSTAMP(0);
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
     constexpr int L = X4 + Traits<TYPE>::kTail;   // plus (three main types) one 4-byte load
@@ -853,11 +841,6 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
             }
         }
     };
-
-#ifdef JL_GEMV_STAMPS
-    asm volatile("" :: "v"(slot_off[0]), "s"(total_tiles), "s"(half_bytes));   // the arguments have arrived
-#endif
-    GSTAMP(1);
     // my tiles: blockIdx.x, blockIdx.x + grid, ...
     const int grid = grid_first;
     const int first = blockIdx.x;
@@ -929,7 +912,6 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     if constexpr (rms) {
         if (held) load(0);
     }
-    GSTAMP(2);
     for (; issued < kStages - 1 && issued < mine; issued++) issue(first + issued * grid, issued);
     if constexpr (rms) {
         float scale;
@@ -977,10 +959,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
             }
         }
     }
-    GSTAMP(3);
     wait_vm_tiles<L>(issued);
     __builtin_amdgcn_s_barrier();
-    GSTAMP(4);
 
     float x[64];
     float sx[4] = {0.f, 0.f, 0.f, 0.f};   // sums of the slice's activations by 32 (4-bit types) or 16 (Q6_K)
@@ -1092,7 +1072,6 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
         // with two stages nothing was issued after tile `it`: its loads are the youngest
         JL_WAIT_VM(0);
         __builtin_amdgcn_s_barrier();
-        if (it == mine - 1) GSTAMP(5);
         // the stage that tile it - 1 (or, the first time round, the activation vector) occupied
         // is free now: every wave is past its reads
         if (issued < mine) {
@@ -1106,7 +1085,6 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
             if constexpr (PACKED) v = slice_dot_lds_packed<TYPE>(ring0 + (it % kStages) * stage_bytes, r_lds, s, row_bytes, px);
             else v = slice_dot_lds<TYPE>(ring0 + (it % kStages) * stage_bytes, r_lds, s, row_bytes, x, sx);
         }
-        if (it == mine - 1) GSTAMP(6);
         if (in_wave) {
             v = group_sum(v, Sp);
             float up = 0.f;
@@ -1155,12 +1133,6 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
         __builtin_amdgcn_s_barrier();
         finish(first + (mine - 1) * grid, (mine - 1) & 1);
     }
-    GSTAMP(7);
-#ifdef JL_GEMV_STAMPS
-    if (jl_gemv_stamp_buf && tid == 0) {
-        for (int k = 0; k < 8; k++) jl_gemv_stamp_buf[(size_t)blockIdx.x * 8 + k] = stamp[k];
-    }
-#endif
 }
 
 // Catch-all for shapes the tile kernel does not take (row length not a multiple of 64, rows wider
@@ -1364,11 +1336,6 @@ int launch_generic(jl_context *ctx, const jl_weight *w, const jl_weight *w_up, c
 
 }  // namespace
 
-#ifdef JL_GEMV_STAMPS
-extern "C" int jl_probe_gemv_stamps(uint64_t *device_buffer) {
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(jl_gemv_stamp_buf), &device_buffer, sizeof(device_buffer));
-}
-#endif
 
 int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *const *outs,
                    const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms, const jl_q8x *xq) {

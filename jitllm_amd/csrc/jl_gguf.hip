@@ -401,14 +401,14 @@ int jl_gguf_upload(jl_context *ctx, const jl_gguf *g, const char *name, jl_weigh
     // compared as unsigned quantities against what is left of the file: a sum of offsets near
     // 2^63 would wrap and pass
     const uint64_t room = g->data_offset <= g->size ? (uint64_t)(g->size - g->data_offset) : 0;
-    const int64_t begin = g->data_offset + t.offset;
     if (t.offset < 0 || t.bytes < 0 || (uint64_t)t.offset > room || (uint64_t)t.bytes > room - (uint64_t)t.offset) {
         return jl_fail(JL_ERR_INVALID, "tensor %s (%s, %lld bytes) runs past the end of the file", name,
                        jl_type_name(t.type), (long long)t.bytes);
     }
     // (the file's own faults are reported before a missing context is)
     JL_REQUIRE(ctx != nullptr, "jl_gguf_upload: null context");
-    // GGUF dimensions are in ne order: dims[0] is the row length
+    // GGUF dimensions are in ne order: dims[0] is the row length (the sum below is in range: checked above)
+    const int64_t begin = g->data_offset + t.offset;
     return jl_weight_upload(ctx, t.type, g->base + begin, t.dims[1], t.dims[0], out);
 }
 

@@ -15,8 +15,14 @@ struct jl_context {
     char name[128];
     void *scratch;   // JL_CONTEXT_SCRATCH_BYTES of device memory for results handed from one launch of
                      // a call to the next (calls on a context are ordered on its stream)
+    // Pinned host memory that jl_upload / jl_download stage the caller's pageable memory through, two
+    // halves in turn: every transfer the device sees is then a DMA from / to pinned memory, and the
+    // caller's pointer is only ever touched by a host memcpy.
+    uint8_t *bounce;
+    hipEvent_t bounce_done[2];
 };
 #define JL_CONTEXT_SCRATCH_BYTES 4096
+#define JL_BOUNCE_HALF_BYTES (8u << 20)
 
 struct jl_weight {
     jl_context *ctx;

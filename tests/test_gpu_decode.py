@@ -299,8 +299,14 @@ def test_fused_qkv(ctx, t, dq, dkv, n):
         assert rel_err(out.get(), ref, magnitude(t, raw, x, d, n)) < 2e-5
 
 
+# Rows of 128 slices (5120, 7168, 8192 columns) put one gate row and one up row in a tile, so 272 rows
+# and 271 rows are both whole tiles and both run the fixed-geometry instance: the bit comparison of
+# fixed and general kernels cannot reach those instances, and they are held to the oracle here.
+WIDE_GATE_UP = [(t, d, n) for t in (O.Q8_0, O.Q4_0, O.Q4_K) for n in (5120, 7168, 8192) for d in (272, 271)]
+
+
 @pytest.mark.parametrize("t,d,n", [(O.Q8_0, 8192, 2048), (O.Q4_0, 14336, 4096),
-                                    (O.Q4_K, 12288, 4096), (O.Q4_K, 37, 512)])
+                                    (O.Q4_K, 12288, 4096), (O.Q4_K, 37, 512)] + WIDE_GATE_UP)
 def test_fused_gate_up(ctx, t, d, n):
     """hb = SiLU(w1 . x) * (w3 . x), held against the host's matVec, matVec, swiGLU sequence
     (InferenceCore.java:127-129)."""
@@ -520,7 +526,7 @@ def test_fused_rms_qkv(ctx, t, dq, dkv, n):
                                     (O.Q4_K, 12288, 4096), (O.Q8_0, 40, 8192), (O.Q4_K, 37, 512),
                                     # rows that fill their slices only in part
                                     (O.Q8_0, 8192, 3072), (O.Q4_0, 4736, 3584), (O.Q4_K, 3456, 5120),
-                                    (O.Q8_0, 3456, 5120)])
+                                    (O.Q8_0, 3456, 5120)] + WIDE_GATE_UP)
 def test_fully_fused_rms_gate_up(ctx, t, d, n):
     """hb = SiLU(w1 . xn) * (w3 . xn) with xn = rmsnorm(x), the scale computed inside the kernel:
     against the host's rmsnorm, matVec, matVec, swiGLU (InferenceCore.java:124-129)."""

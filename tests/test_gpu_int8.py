@@ -158,6 +158,84 @@ def test_int8_prefill_shapes_on_a_sample(ctx, t, d, n, T):
     w.free()
 
 
+def _sample(count, total, seed):
+    rng = np.random.default_rng(seed)
+    return np.unique(np.concatenate([np.arange(min(16, total)), np.arange(max(0, total - 16), total),
+                                     rng.choice(total, size=min(count, total), replace=False)]))
+
+
+def test_int8_big_tile_gate_up_q8_0_with_ragged_rows(ctx):
+    """Q8_0 gate/up on the 128 x 128 tile (4100 weight rows: the last tile of each weight is ragged,
+    1000 of 1024 activation rows active)."""
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    t, d, n, T, active = O.Q8_0, 4100, 1024, 1024, 1000
+    say("int8 big-tile gate/up", d, n, T)
+    r1, r3 = synthetic.weight(t, d, n, seed=2150), synthetic.weight(t, d, n, seed=2151)
+    w1, w3 = ctx.load_weight(t, r1, d, n), ctx.load_weight(t, r3, d, n)
+    X = synthetic.activations((T, n), seed=2152)
+    hb = ctx.float_array(T * d, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, 2 * d, math=L.JL_MATH_INT8).gateUp(ctx.from_numpy(X), hb, w1, w3, n, d,
+                                                                            activeRows=active)
+    ctx.sync()
+    got = hb.get().reshape(T, d)
+    assert np.all(got[:active] != UNTOUCHED) and np.all(got[active:] == UNTOUCHED)
+    rows, arows = _sample(64, d, 2153), _sample(32, active, 2154)
+    g = int8_reference(t, r1, X[arows], d, n, rows).astype(np.float64)
+    u = int8_reference(t, r3, X[arows], d, n, rows).astype(np.float64)
+    want = g / (1.0 + np.exp(-g)) * u
+    assert np.max(np.abs(got[np.ix_(arows, rows)] - want) / (np.abs(want) + 1e-6 * np.abs(u) + 1e-30)) < 1e-5
+    w1.free()
+    w3.free()
+
+
+def test_int8_big_tile_residual_with_ragged_rows(ctx):
+    """JL_RESIDUAL through the 128 x 128 tile: 3100 weight rows (a ragged last tile), 2048 tokens."""
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    t, d, n, T = O.Q8_0, 3100, 1024, 2048
+    say("int8 big-tile residual", d, n, T)
+    raw = synthetic.weight(t, d, n, seed=2160)
+    w = ctx.load_weight(t, raw, d, n)
+    X = synthetic.activations((T, n), seed=2161)
+    start = synthetic.activations((T, d), seed=2162)
+    out = ctx.from_numpy(start)
+    QuantizedBatchProjections(ctx, T, n, d, math=L.JL_MATH_INT8).projection(ctx.from_numpy(X), out, w, n, d, True)
+    ctx.sync()
+    got = out.get().reshape(T, d)
+    rows, arows = _sample(96, d, 2163), _sample(48, T, 2164)
+    ref = int8_reference(t, raw, X[arows], d, n, rows)
+    assert np.array_equal(bits(got[np.ix_(arows, rows)]), bits(start[np.ix_(arows, rows)] + ref))
+    w.free()
+
+
+@pytest.mark.parametrize("t", [O.Q8_0, O.Q4_0])
+def test_int8_big_tile_three_weights_side_by_side(ctx, t):
+    """q|k|v of 2048, 520 and 520 rows at 2048 tokens: three weights, each with a ragged last tile,
+    on the 128 x 128 tile (where a weight's first tile and first output column are looked up)."""
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    n, T, ds = 1024, 2048, (2048, 520, 520)
+    say("int8 big-tile q|k|v", t)
+    raws = [synthetic.weight(t, d, n, seed=2170 + i) for i, d in enumerate(ds)]
+    ws = [ctx.load_weight(t, r, d, n) for r, d in zip(raws, ds)]
+    X = synthetic.activations((T, n), seed=2173)
+    out = ctx.float_array(T * sum(ds), fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, sum(ds), math=L.JL_MATH_INT8).fusedQKV(ctx.from_numpy(X), out, *ws)
+    ctx.sync()
+    got = out.get().reshape(T, sum(ds))
+    assert np.all(got != UNTOUCHED)
+    arows = _sample(32, T, 2174)
+    col = 0
+    for raw, d in zip(raws, ds):
+        rows = _sample(48, d, 2175 + d)
+        ref = int8_reference(t, raw, X[arows], d, n, rows)
+        assert np.array_equal(bits(got[np.ix_(arows, col + rows)]), bits(ref))
+        col += d
+    for w in ws:
+        w.free()
+
+
 def test_int8_refusals(ctx):
     import ctypes as C
     from jitllm_amd import _lib as L, synthetic

@@ -76,3 +76,65 @@ def test_static_argmax_refuses_more_than_its_maximum(ctx):
     assert st == L.JL_ERR_INVALID
     assert b"at most" in lib.jl_last_error()
     assert lib.jl_argmax_static(ctx.handle, dv.ptr, 0, out.ptr) == L.JL_ERR_INVALID
+
+
+def _hip():
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    return hip
+
+
+def _free_bytes(hip) -> int:
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return int(free.value)
+
+
+def test_static_argmax_allocates_nothing_and_can_be_captured(ctx):
+    """What the entry point is for: a burst of calls leaves the device's free memory where it was,
+    and the call is legal inside a stream capture (launches only), whose replays -- with the
+    program's own eager work and synchronisations between them -- give the eager index."""
+    from jitllm_amd import _lib as L
+    lib, hip = ctx._lib, _hip()
+    say("static argmax: no allocation, capture")
+    rng = np.random.default_rng(99)
+    values = rng.standard_normal(50_000).astype(np.float32)
+    values[31_337] = 40.0
+    dv = ctx.from_numpy(values)
+    other = ctx.from_numpy(rng.standard_normal(4097).astype(np.float32))
+    out = ctx.raw_buffer(8)
+    out.upload(np.array([-7, -7], dtype=np.int32))
+    L.check(lib.jl_argmax_static(ctx.handle, dv.ptr, values.size, out.ptr.value))   # first call on the device done
+    ctx.sync()
+    before = _free_bytes(hip)
+    for _ in range(200):
+        L.check(lib.jl_argmax_static(ctx.handle, dv.ptr, values.size, out.ptr.value))
+    ctx.sync()
+    assert _free_bytes(hip) == before
+    assert int(out.download(np.int32, 2)[0]) == 31_337
+    stream = lib.jl_context_stream(ctx.handle)
+    assert hip.hipStreamBeginCapture(stream, 0) == 0
+    st = lib.jl_argmax_static(ctx.handle, dv.ptr, values.size, out.ptr.value)
+    graph, exe = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+    L.check(st)
+    assert hip.hipGraphInstantiate(C.byref(exe), graph, None, None, 0) == 0
+    hip.hipGraphDestroy(graph)
+    for replay in range(4):
+        out.upload(np.array([-7, -7], dtype=np.int32))
+        # eager work between the replays: another input through the same static cells
+        L.check(lib.jl_argmax_static(ctx.handle, other.ptr, 4097, out.ptr.value + 4))
+        ctx.sync()
+        assert hip.hipGraphLaunch(exe, stream) == 0
+        ctx.sync()
+        got = out.download(np.int32, 2)
+        assert int(got[0]) == 31_337, replay
+        assert int(got[1]) == O.argmax(other.get()), replay
+    assert hip.hipGraphExecDestroy(exe) == 0
+    assert _free_bytes(hip) == before
