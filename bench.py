@@ -360,10 +360,13 @@ def check_swiglu(name, got, g, u, mag_g, mag_u, bound):
     return check(name, got, ref, mag, bound)
 
 
-def bench_gemm(ctx, hip, t, T, steps, warmup, cpu, clock_khz, cu):
-    """Batched prefill of one Llama-3.2-1B layer (q|k|v, o, gate/up SwiGLU, down) over T tokens."""
+def bench_gemm(ctx, hip, t, T, steps, warmup, cpu, clock_khz, cu, dims=None, int8=True, model="Llama-3.2-1B"):
+    """Batched prefill of one layer (q|k|v, o, gate/up SwiGLU, down) over T tokens: Llama-3.2-1B
+    geometry unless `dims` = (dim, kv, ffn) names another; `int8` adds the block-scaled int8 mode
+    (Q8_0 / Q4_0 only)."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
+    DIM, KV_DIM, HIDDEN = dims or (globals()["DIM"], globals()["KV_DIM"], globals()["HIDDEN"])
     shapes = {"wq": (DIM, DIM), "wk": (KV_DIM, DIM), "wv": (KV_DIM, DIM), "wo": (DIM, DIM),
               "w1": (HIDDEN, DIM), "w3": (HIDDEN, DIM), "w2": (DIM, HIDDEN)}
     host = {k: synthetic.weight(t, r, c, 41 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
@@ -440,33 +443,35 @@ def bench_gemm(ctx, hip, t, T, steps, warmup, cpu, clock_khz, cu):
     # results are fixed bit for bit, so the check is equality with the oracle's int8 statement
     from jitllm_amd import _lib as L
     from oracle import pyoracle as O
-    i8_proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, math=L.JL_MATH_INT8)
+    int8_leg = None
+    if int8:
+        i8_proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, math=L.JL_MATH_INT8)
 
-    def i8_layer(w=w):
-        i8_proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
-        i8_proj.projection(X, res, w["wo"], DIM, DIM, True)
-        i8_proj.gateUp(X, hb, w["w1"], w["w3"], DIM, HIDDEN)
-        i8_proj.projection(H, res, w["w2"], HIDDEN, DIM, True)
+        def i8_layer(w=w):
+            i8_proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
+            i8_proj.projection(X, res, w["wo"], DIM, DIM, True)
+            i8_proj.gateUp(X, hb, w["w1"], w["w3"], DIM, HIDDEN)
+            i8_proj.projection(H, res, w["w2"], HIDDEN, DIM, True)
 
-    def i8_sweep():
-        for lw in layers:
-            i8_layer(lw)
-    res.init(0.0)
-    i8_layer()
-    ctx.sync()
-    xq, xs = O.quantize_q8(Xh[arows])
-    hq, hs = O.quantize_q8(Hh[arows])
-    ro = sample_rows(DIM, 48, 56)
-    ref_o = O.gemm_int8_block_scaled(int(t), xq, xs, gather_rows(host["wo"], t, DIM, ro), ro.size)
-    ref_d = O.gemm_int8_block_scaled(int(t), hq, hs, gather_rows(host["w2"], t, HIDDEN, ro), ro.size)
-    got = res.get().reshape(T, DIM)[arows][:, ro]
-    if not np.array_equal(got.view(np.uint32), (ref_o + ref_d).astype(np.float32).view(np.uint32)):
-        raise SystemExit(f"bench.py: the int8 prefill path at T={T} differs from the oracle's int8 arithmetic")
-    int8 = mode([m / PREFILL_LAYERS for m in timed_graph(ctx, hip, i8_sweep, steps, warmup)],
-                {"o+down": "bit-equal to the oracle's int8 statement"})
-    int8["frac_int8_mfma_peak"] = round(int8["tflops"] / INT8_MFMA_PEAK_TOPS, 4)
-    int8["math"] = ("int8 MFMA over the raw blocks, fp32 (float) dot * dA fused-multiplied by dW per 32-block in k order; "
-                    "bound by the three vector-ALU operations per int32 result at one sixth of the int8 MFMA peak")
+        def i8_sweep():
+            for lw in layers:
+                i8_layer(lw)
+        res.init(0.0)
+        i8_layer()
+        ctx.sync()
+        xq, xs = O.quantize_q8(Xh[arows])
+        hq, hs = O.quantize_q8(Hh[arows])
+        ro = sample_rows(DIM, 48, 56)
+        ref_o = O.gemm_int8_block_scaled(int(t), xq, xs, gather_rows(host["wo"], t, DIM, ro), ro.size)
+        ref_d = O.gemm_int8_block_scaled(int(t), hq, hs, gather_rows(host["w2"], t, HIDDEN, ro), ro.size)
+        got = res.get().reshape(T, DIM)[arows][:, ro]
+        if not np.array_equal(got.view(np.uint32), (ref_o + ref_d).astype(np.float32).view(np.uint32)):
+            raise SystemExit(f"bench.py: the int8 prefill path at T={T} differs from the oracle's int8 arithmetic")
+        int8_leg = mode([m / PREFILL_LAYERS for m in timed_graph(ctx, hip, i8_sweep, steps, warmup)],
+                        {"o+down": "bit-equal to the oracle's int8 statement"})
+        int8_leg["frac_int8_mfma_peak"] = round(int8_leg["tflops"] / INT8_MFMA_PEAK_TOPS, 4)
+        int8_leg["math"] = ("int8 MFMA over the raw blocks, fp32 (float) dot * dA fused-multiplied by dW per 32-block in k order; "
+                            "bound by the three vector-ALU operations per int32 result at one sixth of the int8 MFMA peak")
     # the dominant kernel on its own: the gate/up call of that last mode is one launch of the fp16
     # GEMM and nothing else (one per layer to a graph)
     def gate_ups():
@@ -493,17 +498,23 @@ def bench_gemm(ctx, hip, t, T, steps, warmup, cpu, clock_khz, cu):
             rms_proj.rmsApplyFP16(X, rms_w, 1e-5, X16, DIM)
     rms_us = statistics.median(timed_graph(ctx, hip, rms_apply, steps, 3)) / 8 * 1e3
     half["rms_apply_to_fp16_us"] = round(rms_us, 2)
-    out = {"tokens": T, "layers_swept": PREFILL_LAYERS,
+    copy_mb = round(2e-6 * sum(r * c for r, c in shapes.values()))
+    out = {"tokens": T, "type": t.name, "layer": f"{model} (dim {DIM}, kv {KV_DIM}, ffn {HIDDEN})",
+           "layers_swept": PREFILL_LAYERS,
            "weights_from": f"HBM: {PREFILL_LAYERS} layers' distinct weights in turn (their fp16 copies, "
-                           f"{PREFILL_LAYERS} x 121 MB, exceed the 256 MB memory-side cache)",
+                           f"{PREFILL_LAYERS} x {copy_mb} MB, exceed the 256 MB memory-side cache)",
            "ms_per_layer": default["ms_per_layer"],
            "ms_stats": default["ms_stats"],
-           "tok_s_16_layers": round(T / (default["ms_per_layer"] * 1e-3 * LAYERS), 1),
+           "tok_s_per_layer": round(T / (default["ms_per_layer"] * 1e-3), 1),
            "tflops": default["tflops"], "frac_f16_mfma_peak": default["frac_f16_mfma_peak"],
            "check_rel_err": default["check_rel_err"],
            "math": "f16 MFMA, fp32 accumulate; weights decoded to fp16 inside the call (in LDS, or once per call into the workspace)",
            "with_resident_fp16_copy": kept, "with_resident_copy_and_fp16_activations": half,
-           "int8_block_scaled": int8, "roofline": roofline}
+           "roofline": roofline}
+    if dims is None:
+        out["tok_s_16_layers"] = round(T / (default["ms_per_layer"] * 1e-3 * LAYERS), 1)
+    if int8_leg is not None:
+        out["int8_block_scaled"] = int8_leg
     if cpu:
         rows = sample_rows(HIDDEN, 224, 55)
         out["cpu_baseline"] = cpu_baseline_rows(t, host["w1"], DIM, rows, Xh, HIDDEN, 2.0, f"gate projection at T={T}")
@@ -515,19 +526,21 @@ def bench_gemm(ctx, hip, t, T, steps, warmup, cpu, clock_khz, cu):
     return out
 
 
-def bench_batched_q4k(ctx, hip, B, steps, warmup, cpu):
-    """Q4_K batched decode, Qwen3-8B-like shapes (dim 4096, ffn 12288, kv 1024), B sequences."""
+def bench_batched(ctx, hip, B, steps, warmup, cpu, type_name="Q4_K", dims=(4096, 1024, 12288),
+                  model="Qwen3-8B-like", copies=None):
+    """Batched decode of one layer's projections for B sequences: Q4_K at Qwen3-8B-like shapes (dim
+    4096, ffn 12288, kv 1024) unless another type and geometry are named."""
     from jitllm_amd import synthetic
     from jitllm_amd.ggml import GGMLType
     from jitllm_amd.projections import QuantizedBatchProjections
-    t = GGMLType.Q4_K
-    dim, kv, ffn = 4096, 1024, 12288
+    t = GGMLType[type_name]
+    dim, kv, ffn = dims
     shapes = {"wq": (dim, dim), "wk": (kv, dim), "wv": (kv, dim), "wo": (dim, dim),
               "w1": (ffn, dim), "w3": (ffn, dim), "w2": (dim, ffn)}
     host = {k: synthetic.weight(t, r, c, 61 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
     # enough copies of the layer (109 MB each) that a replay cannot be served from the 256 MB
     # memory-side cache, whatever it keeps of what it has seen
-    copies = BATCHED_COPIES
+    copies = copies or BATCHED_COPIES
     layers = [{k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes} for _ in range(copies)]
     Xh = synthetic.activations((B, dim), 68)
     Hh = synthetic.activations((B, ffn), 69) * np.float32(0.1)
@@ -572,7 +585,8 @@ def bench_batched_q4k(ctx, hip, B, steps, warmup, cpu):
     io = 4 * B * (dim + dim + 2 * kv + dim + dim + dim + ffn + ffn + dim)
     flops = 2.0 * B * (dim * (dim + 2 * kv) + dim * dim + 2 * dim * ffn + ffn * dim)
     gbs = (wbytes + io) / (ms * 1e-3) / 1e9
-    out = {"B": B, "ms_per_layer": round(ms, 4), "ms_stats": spread_stats(ms_list), "layers_swept": copies,
+    out = {"B": B, "type": type_name, "layer": f"{model} (dim {dim}, kv {kv}, ffn {ffn})",
+           "ms_per_layer": round(ms, 4), "ms_stats": spread_stats(ms_list), "layers_swept": copies,
            "GB_s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
            "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "bytes": wbytes + io, "check_rel_err": errs}
     # which roof applies at this batch: the call's flop per byte against the chip's ridge
@@ -582,7 +596,7 @@ def bench_batched_q4k(ctx, hip, B, steps, warmup, cpu):
     out["bound"] = "hbm" if intensity < ridge else "mfma"
     out["frac_f16_mfma_peak"] = round(out["tflops"] / F16_MFMA_PEAK_TFLOPS, 4)
     if cpu and B == 8:
-        rows = sample_rows(ffn, 480, 75)
+        rows = sample_rows(ffn, 480 if t == GGMLType.Q4_K else 2048, 75)
         out["cpu_baseline"] = cpu_baseline_rows(t, host["w1"], dim, rows, Xh, ffn, 2.0, "gate projection at B=8")
         out["cpu_baseline"]["ms_per_layer_equiv"] = round(flops / (out["cpu_baseline"]["gflops"] * 1e9) * 1e3, 1)
     for w in layers:
@@ -953,7 +967,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-extra", action="store_true", help="skip the legs beside the decode set")
-    ap.add_argument("--extra", default="wq_shape,fused_rms,prefill,other_types,batched",
+    ap.add_argument("--extra", default="wq_shape,fused_rms,prefill,other_types,batched,prefill_other_types,batched_other_types",
                     help="comma-separated legs beside the decode set (a profiler run takes a few at a time)")
     ap.add_argument("--prefill-warmup", type=int, default=-1,
                     help="untimed replays before the prefill legs (default 100; 10 under a profiler)")
@@ -1188,8 +1202,25 @@ def main():
                 bench_decode_layers(ctx, hip, "Q4_0", 4096, 1024, 14336, OTHER_TYPE_COPIES, args.steps, args.warmup, cpu),
                 bench_decode_layers(ctx, hip, "Q4_K", 4096, 1024, 12288, OTHER_TYPE_COPIES, args.steps, args.warmup, cpu)]
         if "batched" in legs:
-            out["batched_q4k"] = [bench_batched_q4k(ctx, hip, B, max(5, args.steps // 5), 3, cpu)
+            out["batched_q4k"] = [bench_batched(ctx, hip, B, max(5, args.steps // 5), 3, cpu)
                                   for B in (8, 32, 64)]
+        if "prefill_other_types" in legs:
+            # the prefill GEMM of the other two weight types at 8B-model shapes: Q4_K is decoded to
+            # fp16 (in LDS or once per call) and multiplied on the fp16 MFMA, Q4_0 likewise by default
+            out["prefill_other_types"] = [
+                bench_gemm(ctx, hip, GGMLType[name], T, max(4, args.steps // 4), prefill_warmup // 2, cpu and T == 512,
+                           clock_khz, cu, dims=dims, int8=False, model=model)
+                for name, dims, model in (("Q4_K", (4096, 1024, 12288), "Qwen3-8B-like"),
+                                          ("Q4_0", (4096, 1024, 14336), "Llama-3-8B"))
+                for T in (512, 2048)]
+        if "batched_other_types" in legs:
+            # batched decode of the other two weight types: Q8_0 at Llama-3.2-1B shapes (32 layer
+            # copies of 65 MB to a replay), Q4_0 at Llama-3-8B shapes
+            out["batched_other_types"] = [
+                bench_batched(ctx, hip, B, max(5, args.steps // 5), 3, cpu, name, dims, model, copies)
+                for name, dims, model, copies in (("Q8_0", (DIM, KV_DIM, HIDDEN), "Llama-3.2-1B", 32),
+                                                  ("Q4_0", (4096, 1024, 14336), "Llama-3-8B", 8))
+                for B in (8, 32, 64)]
         out["cpu_baseline"] = cpu_baseline(host, shapes, t) if cpu else None
     print(json.dumps(out))
 

@@ -885,7 +885,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const size_t plane_bytes = workspace_bytes > head ? workspace_bytes - head : 0;
 
 
-    if (rows <= 64 && jl_has_fused_kernels(type) && !X16) {
+    if (rows <= 64 && !X16) {
         // batched decode of up to 64 rows: the weight-streaming kernel reads X itself
         bool taken = false;
         int st = jl_launch_gemm_skinny(ctx, weights, count, X, C, rows, ldo, col_offset, epilogue, planes,

@@ -40,6 +40,7 @@ namespace {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) const void gvoid;
 typedef __attribute__((address_space(3))) void lvoid;
 
@@ -124,6 +125,30 @@ __device__ __forceinline__ void lds_read_q4k(uint32_t hdr, uint32_t qs, uint4 &h
         : "=&v"(h), "=&v"(q0), "=&v"(q1) : "v"(hdr), "v"(qs) : "memory");
 }
 
+// N 16-byte reads at consecutive 16-byte offsets from `addr` (16-byte aligned), one wait.
+template <int N>
+__device__ __forceinline__ void lds_read_x4(uint32_t addr, u32x4 (&v)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; i++) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v[i]) : "v"(addr), "n"(16 * i) : "memory");
+}
+// N dword reads at consecutive offsets from `addr` (4-byte aligned)
+template <int N>
+__device__ __forceinline__ void lds_read_x1(uint32_t addr, uint32_t (&v)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; i++) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=&v"(v[i]) : "v"(addr), "n"(4 * i) : "memory");
+}
+// The wait behind reads issued without one; the values pass through it so that no use moves ahead.
+template <typename T, int N>
+__device__ __forceinline__ void lds_landed(T (&v)[N]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        T t = v[i];
+        asm volatile("" : "+v"(t));
+        v[i] = t;
+    }
+}
+
 // Never hand an MFMA result straight to this: the matrix pipe does not interlock with an LDS store
 // that reads its destination registers, and the compiler's hazard pass cannot see inside inline
 // assembly.  Callers pass values that went through ordinary vector arithmetic first.
@@ -174,6 +199,46 @@ struct Q4KTail {
     half8 mins;   // {m0, m0, m1, m1, 0, 0, 0, 0}: each minimum meets its sub-block's activation sum as hi + lo
 };
 
+// Bytes of 256 columns of a row (four slices): every type's blocks tile 256 columns exactly.
+constexpr int quad_bytes(int type) {
+    return type == JL_Q8_0 ? 272 : type == JL_Q4_0 ? 144 : type == JL_Q4_K ? 144 : type == JL_Q6_K ? 210
+           : type == JL_Q5_K ? 176 : type == JL_Q4_1 ? 160 : type == JL_Q5_0 ? 176 : type == JL_IQ4_XS ? 136 : 0;
+}
+// Types whose 256-column block has one scale for everything a wave's MFMAs add up: the fragments
+// hold small integers (sub-block scale x quant) and the block's d multiplies the MFMA result.
+template <int TYPE> constexpr bool kPostScale = TYPE == JL_Q4_K || TYPE == JL_Q5_K || TYPE == JL_Q6_K || TYPE == JL_IQ4_XS;
+// Types with an additive term per 32 columns (a minimum), folded in by one more MFMA against the
+// activations' sums over those 32 columns.
+template <int TYPE> constexpr bool kHasMins = TYPE == JL_Q4_K || TYPE == JL_Q5_K || TYPE == JL_Q4_1;
+
+// The scales and minimums of sub-blocks 2 pair and 2 pair + 1 of a Q4_K / Q5_K header (d, dmin, 12
+// packed bytes: h.y, h.z, h.w), each scale as a pair of equal fp16 values, the minimums as the k
+// slots of the minimum MFMA.  Sub-blocks 0..3 keep them in the low six bits of bytes j and j + 4,
+// sub-blocks 4..7 in the nibbles of byte j + 4 with bits 4..5 in the top bits of bytes j - 4 and j
+// (Q4_KFloatTensor.getScaleK4 / getMinK4, J/tensor/standard/Q4_KFloatTensor.java:68-85).
+__device__ __forceinline__ void k_scales(const uint4 &h, int pair, h2 &s0, h2 &s1, Q4KTail &tail) {
+    tail.d = jl_half_bits_to_float(h.x);
+    tail.dmin = jl_half_bits_to_float(h.x >> 16);
+    const int sh = 16 * (pair & 1);
+    const uint32_t a = h.y >> sh, b = h.z >> sh, c = h.w >> sh;
+    const uint32_t sc2 = pair < 2 ? (a & 0x3F3Fu) : ((c & 0x0F0Fu) | ((a >> 2) & 0x3030u));
+    const uint32_t mn2 = pair < 2 ? (b & 0x3F3Fu) : (((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u));
+    // small integers as fp16: bits 0x6400 | v are 1024 + v
+    const h2 k1024 = {(_Float16)1024.f, (_Float16)1024.f};
+    s0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(sc2, 0x64646464u, 0x00040004u)) - k1024;
+    s1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(sc2, 0x64646464u, 0x00050005u)) - k1024;
+    const h2 m01 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(mn2, 0x64646464u, 0x00040004u)) - k1024;
+    const h2 m11 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(mn2, 0x64646464u, 0x00050005u)) - k1024;
+    const _Float16 z = (_Float16)0.f;
+    tail.mins = half8{m01[0], m01[1], m11[0], m11[1], z, z, z, z};
+}
+
+// a signed byte of `v` as a pair of equal fp16 values
+__device__ __forceinline__ h2 sbyte_h2(uint32_t v, int byte) {
+    const _Float16 f = (_Float16)(float)(int)(int8_t)(v >> (8 * byte));
+    return h2{f, f};
+}
+
 // Decodes the 64-column slice `sl` of the tile row at LDS address `row`.
 template <int TYPE>
 __device__ __forceinline__ void decode_slice(uint32_t row, int sl, half8 (&f)[8], Q4KTail &tail) {
@@ -214,31 +279,178 @@ __device__ __forceinline__ void decode_slice(uint32_t row, int sl, half8 (&f)[8]
             f[4 + i] = frag_scaled(qb[2 * i] & 0x0F0F0F0Fu, qb[2 * i + 1] & 0x0F0F0F0Fu, bias, b2);
             f[6 + i] = frag_scaled((qb[2 * i] >> 4) & 0x0F0F0F0Fu, (qb[2 * i + 1] >> 4) & 0x0F0F0F0Fu, bias, b2);
         }
+    } else if constexpr (TYPE == JL_Q5_K) {
+        // Q4_K's layout with a fifth bit per weight (fp16 d, dmin | 12 scale bytes | qh[32] |
+        // qs[128], J/tensor/standard/Q5_KFloatTensor.java:78-122): bit 2 pair of qh[l] tops the low
+        // nibble of qs[32 pair + l], bit 2 pair + 1 the high one.  sc q is at most 63 x 31: exact.
+        const uint32_t sb = row + (sl >> 2) * 176;
+        const int pair = sl & 3;
+        u32x4 r[3], q[2];
+        lds_read_x4(sb, r);                       // header, the 32 fifth-bit bytes
+        lds_read_x4(sb + 48 + pair * 32, q);
+        lds_landed(r);
+        lds_landed(q);
+        h2 s0, s1;
+        k_scales(uint4{r[0].x, r[0].y, r[0].z, r[0].w}, pair, s0, s1, tail);
+        const h2 o0 = s0 * h2{(_Float16)-1024.f, (_Float16)-1024.f};
+        const h2 o1 = s1 * h2{(_Float16)-1024.f, (_Float16)-1024.f};
+        const uint32_t qs[8] = {q[0].x, q[0].y, q[0].z, q[0].w, q[1].x, q[1].y, q[1].z, q[1].w};
+        const uint32_t qh[8] = {r[1].x, r[1].y, r[1].z, r[1].w, r[2].x, r[2].y, r[2].z, r[2].w};
+        uint32_t lo[8], hi[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t hb = qh[j] >> (2 * pair);
+            lo[j] = (qs[j] & 0x0F0F0F0Fu) | ((hb & 0x01010101u) << 4);
+            hi[j] = ((qs[j] >> 4) & 0x0F0F0F0Fu) | ((hb & 0x02020202u) << 3);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            f[i] = frag_times(lo[2 * i], lo[2 * i + 1], s0, o0);
+            f[4 + i] = frag_times(hi[2 * i], hi[2 * i + 1], s1, o1);
+        }
+    } else if constexpr (TYPE == JL_Q6_K) {
+        // A quarter (h, upper) of a super-block (ql[128] | qh[64] | 16 signed scales | fp16 d,
+        // J/tensor/standard/Q6_KFloatTensor.java:66-122): element l < 32 is nibble `upper` of
+        // ql[64 h + l] under bits 4 upper .. + 1 of qh[32 h + l], element 32 + l nibble `upper` of
+        // ql[64 h + 32 + l] under bits 4 upper + 2 .. + 3 of the same qh byte; one scale per 16
+        // elements; w = d sc (q - 32).  A fragment holds sc (q - 32), an integer of at most 4096 in
+        // magnitude (rounded to fp16 only beyond 2048), and d multiplies the MFMA result.
+        // Super-blocks are 210 bytes apart, so every other one starts two bytes off a dword: the
+        // quarter is read as aligned dwords from two bytes before where that is needed and each
+        // dword put together from its two neighbours with a funnel shift of 0 or 16 bits.
+        const uint32_t sb = row + (sl >> 2) * 210;
+        const int h = (sl >> 1) & 1, upper = sl & 1;
+        const uint32_t off = sb & 2u, shift = off * 8;
+        uint32_t wl[17], wh[9], sc2[2], d16[1];
+        lds_read_x1(sb - off + 64 * h, wl);
+        lds_read_x1(sb - off + 128 + 32 * h, wh);
+        lds_read_x1(sb - off + 192 + 4 * (sl & 3), sc2);
+        asm volatile("ds_read_u16 %0, %1" : "=&v"(d16[0]) : "v"(sb + 208) : "memory");
+        lds_landed(wl);
+        lds_landed(wh);
+        lds_landed(sc2);
+        lds_landed(d16);
+        tail.d = jl_half_bits_to_float(d16[0]);
+        tail.dmin = 0.f;
+        const uint32_t scales = __builtin_amdgcn_alignbit(sc2[1], sc2[0], shift);
+        const h2 bias = {(_Float16)1056.f, (_Float16)1056.f};
+        const int shl = 4 * upper;
+        uint32_t v0[8], v1[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t ql0 = __builtin_amdgcn_alignbit(wl[j + 1], wl[j], shift);
+            const uint32_t ql1 = __builtin_amdgcn_alignbit(wl[9 + j], wl[8 + j], shift);
+            const uint32_t hb = __builtin_amdgcn_alignbit(wh[j + 1], wh[j], shift) >> shl;
+            v0[j] = ((ql0 >> shl) & 0x0F0F0F0Fu) | ((hb & 0x03030303u) << 4);
+            v1[j] = ((ql1 >> shl) & 0x0F0F0F0Fu) | ((hb & 0x0C0C0C0Cu) << 2);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            f[i] = frag_scaled(v0[2 * i], v0[2 * i + 1], bias, sbyte_h2(scales, i >> 1));
+            f[4 + i] = frag_scaled(v1[2 * i], v1[2 * i + 1], bias, sbyte_h2(scales, 2 + (i >> 1)));
+        }
+    } else if constexpr (TYPE == JL_Q4_1) {
+        // 40 bytes: d, m | 16 nibble bytes, twice (J/tensor/standard/Q4_1FloatTensor.java:73-94);
+        // w = d q + m.  The fragments hold d q rounded once; the minimums go through the extra MFMA
+        // with the opposite sign of a K-quant's (dmin = -1).
+        uint32_t w[10];
+        lds_read_x1(row + sl * 40, w);
+        lds_landed(w);
+        const _Float16 dA = __builtin_bit_cast(_Float16, (unsigned short)(w[0] & 0xFFFF));
+        const _Float16 mA = __builtin_bit_cast(_Float16, (unsigned short)(w[0] >> 16));
+        const _Float16 dB = __builtin_bit_cast(_Float16, (unsigned short)(w[5] & 0xFFFF));
+        const _Float16 mB = __builtin_bit_cast(_Float16, (unsigned short)(w[5] >> 16));
+        const _Float16 z = (_Float16)0.f;
+        tail.d = 1.f;
+        tail.dmin = -1.f;
+        tail.mins = half8{mA, mA, mB, mB, z, z, z, z};
+        const h2 bias = {(_Float16)1024.f, (_Float16)1024.f};
+        const h2 a2 = {dA, dA}, b2 = {dB, dB};
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            f[i] = frag_scaled(w[1 + 2 * i] & 0x0F0F0F0Fu, w[2 + 2 * i] & 0x0F0F0F0Fu, bias, a2);
+            f[2 + i] = frag_scaled((w[1 + 2 * i] >> 4) & 0x0F0F0F0Fu, (w[2 + 2 * i] >> 4) & 0x0F0F0F0Fu, bias, a2);
+            f[4 + i] = frag_scaled(w[6 + 2 * i] & 0x0F0F0F0Fu, w[7 + 2 * i] & 0x0F0F0F0Fu, bias, b2);
+            f[6 + i] = frag_scaled((w[6 + 2 * i] >> 4) & 0x0F0F0F0Fu, (w[7 + 2 * i] >> 4) & 0x0F0F0F0Fu, bias, b2);
+        }
+    } else if constexpr (TYPE == JL_Q5_0) {
+        // 44 bytes: d | 32 fifth bits | 16 nibble bytes, twice (J/tensor/standard/Q5_0FloatTensor.java:
+        // 61-85); w = d (q - 16), bit i of the 32 tops element i.  Block A's fields sit two bytes off
+        // the dwords (d | qh lo, qh hi | qs ..), block B's on them.
+        uint32_t w[11];
+        lds_read_x1(row + sl * 44, w);
+        lds_landed(w);
+        const _Float16 dA = __builtin_bit_cast(_Float16, (unsigned short)(w[0] & 0xFFFF));
+        const _Float16 dB = __builtin_bit_cast(_Float16, (unsigned short)(w[5] >> 16));
+        const h2 bias = {(_Float16)1040.f, (_Float16)1040.f};
+        const h2 d2[2] = {h2{dA, dA}, h2{dB, dB}};
+        const uint32_t qh[2] = {__builtin_amdgcn_alignbit(w[1], w[0], 16), w[6]};
+        uint32_t qs[8];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            qs[j] = __builtin_amdgcn_alignbit(w[2 + j], w[1 + j], 16);
+            qs[4 + j] = w[7 + j];
+        }
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) {
+            uint32_t lo[4], hi[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t q = qs[4 * blk + j];
+                lo[j] = (q & 0x0F0F0F0Fu) | (jl_spread4(qh[blk] >> (4 * j)) << 4);
+                hi[j] = ((q >> 4) & 0x0F0F0F0Fu) | (jl_spread4(qh[blk] >> (16 + 4 * j)) << 4);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                f[4 * blk + i] = frag_scaled(lo[2 * i], lo[2 * i + 1], bias, d2[blk]);
+                f[4 * blk + 2 + i] = frag_scaled(hi[2 * i], hi[2 * i + 1], bias, d2[blk]);
+            }
+        }
+    } else if constexpr (TYPE == JL_IQ4_XS) {
+        // A quarter of a super-block (fp16 d | scales_h | scales_l[4] | qs[128],
+        // J/tensor/standard/IQ4_XSFloatTensor.java:72-100): sub-blocks 2 q and 2 q + 1,
+        // w = d (ls - 32) kvalues_iq4nl[nibble]; a sub-block's 16 bytes hold elements 0..15 in their
+        // low halves and 16..31 in their high halves.  A fragment holds (ls - 32) kvalue, at most
+        // 4064 in magnitude (rounded to fp16 only beyond 2048); d multiplies the MFMA result.
+        const uint32_t sb = row + (sl >> 2) * 136;
+        const int q = sl & 3;
+        uint32_t hdr[2], qs[8];
+        lds_read_x1(sb, hdr);
+        lds_read_x1(sb + 8 + q * 32, qs);
+        lds_landed(hdr);
+        lds_landed(qs);
+        tail.d = jl_half_bits_to_float(hdr[0]);
+        tail.dmin = 0.f;
+        const uint32_t scales_h = hdr[0] >> 16, scales_l = hdr[1];
+        const h2 bias = {(_Float16)1152.f, (_Float16)1152.f};   // the table bytes with 128 added, under 1024
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+            const int g = 2 * q + sub;
+            const int ls = (int)(((scales_l >> (4 * g)) & 0xFu) | (((scales_h >> (2 * g)) & 3u) << 4)) - 32;
+            const _Float16 lsf = (_Float16)(float)ls;
+            const h2 ls2 = {lsf, lsf};
+            uint32_t lo[4], hi[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                lo[j] = jl_iq4nl_lookup4(qs[4 * sub + j] & 0x0F0F0F0Fu) ^ 0x80808080u;
+                hi[j] = jl_iq4nl_lookup4((qs[4 * sub + j] >> 4) & 0x0F0F0F0Fu) ^ 0x80808080u;
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                f[4 * sub + i] = frag_scaled(lo[2 * i], lo[2 * i + 1], bias, ls2);
+                f[4 * sub + 2 + i] = frag_scaled(hi[2 * i], hi[2 * i + 1], bias, ls2);
+            }
+        }
     } else {
+        static_assert(TYPE == JL_Q4_K, "no slice decoder for this type");
         // a quarter of a super-block: 32 nibble bytes; low nibbles are sub-block 2 pair (columns
         // 0..31 of the slice), high nibbles sub-block 2 pair + 1; w = d (sc q) - dmin m
         uint4 h, q0, q1;
         const uint32_t sb = row + (sl >> 2) * 144;
         const int pair = sl & 3;
         lds_read_q4k(sb, sb + 16 + pair * 32, h, q0, q1);
-        tail.d = jl_half_bits_to_float(h.x);
-        tail.dmin = jl_half_bits_to_float(h.x >> 16);
-        // the scales / minimums of sub-blocks 2 pair and 2 pair + 1, two to a register (bytes 0 and
-        // 1): sub-blocks 0..3 keep them in the low six bits of bytes j and j + 4, sub-blocks 4..7
-        // in the nibbles of byte j + 4 with bits 4..5 in the top bits of bytes j - 4 and j
-        // (Q4_KFloatTensor.getScaleK4 / getMinK4, J/tensor/standard/Q4_KFloatTensor.java:68-85)
-        const int sh = 16 * (pair & 1);
-        const uint32_t a = h.y >> sh, b = h.z >> sh, c = h.w >> sh;
-        const uint32_t sc2 = pair < 2 ? (a & 0x3F3Fu) : ((c & 0x0F0Fu) | ((a >> 2) & 0x3030u));
-        const uint32_t mn2 = pair < 2 ? (b & 0x3F3Fu) : (((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u));
-        // small integers as fp16: bits 0x6400 | v are 1024 + v
-        const h2 k1024 = {(_Float16)1024.f, (_Float16)1024.f};
-        const h2 s0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(sc2, 0x64646464u, 0x00040004u)) - k1024;
-        const h2 s1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(sc2, 0x64646464u, 0x00050005u)) - k1024;
-        const h2 m01 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(mn2, 0x64646464u, 0x00040004u)) - k1024;
-        const h2 m11 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(mn2, 0x64646464u, 0x00050005u)) - k1024;
-        const _Float16 z = (_Float16)0.f;
-        tail.mins = half8{m01[0], m01[1], m11[0], m11[1], z, z, z, z};
+        h2 s0, s1;
+        k_scales(h, pair, s0, s1, tail);
         const h2 o0 = s0 * h2{(_Float16)-1024.f, (_Float16)-1024.f};   // exact: at most 63 * 1024
         // the high nibbles stay where they are: a byte 16 q is 1024 + 16 q, times sc / 16 (exact)
         const h2 s1x = s1 * h2{(_Float16)0.0625f, (_Float16)0.0625f};
@@ -297,7 +509,9 @@ constexpr int kScratchRow = 528, kScratchPerWave = 8 * kScratchRow;
 
 // 16-byte loads per DMA wave and tile (upper bound): a tile row takes span_bytes + 16 bytes of LDS
 // (the padding spreads the 16 rows a wave reads at once over all banks), 16 rows, 128 lanes.
-template <int TYPE> struct Loads { static constexpr int kPerWave = TYPE == JL_Q8_0 ? 18 : 10; };
+constexpr int loads_per_wave(int type) { return (kGroup * (8 * quad_bytes(type) / 16 + 1) + 64 * kDmaWaves - 1) / (64 * kDmaWaves); }
+template <int TYPE> struct Loads { static constexpr int kPerWave = loads_per_wave(TYPE); };
+static_assert(Loads<JL_Q8_0>::kPerWave == 18 && Loads<JL_Q4_K>::kPerWave == 10 && Loads<JL_Q6_K>::kPerWave == 14, "");
 
 // ZIN: spans of a row that one workgroup walks itself, one tile after the other, adding their
 // results in registers (it then holds ZIN sets of activation fragments); p.Z spans of ZIN each.
@@ -636,7 +850,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                     }
                     __builtin_amdgcn_wave_barrier();
                 }
-                if constexpr (TYPE == JL_Q4_K) {
+                if constexpr (kHasMins<TYPE>) {
                     // sums of the values the MFMAs will see: at most 32 x 2^10, exact in fp32
                     float part[2] = {0.f, 0.f};
                     const h2 ones = {(_Float16)1.f, (_Float16)1.f};
@@ -664,10 +878,12 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                 acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[b][q][i], wf[i], acc0, 0, 0, 0);
                 acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[b][q][i + 1], wf[i + 1], acc1, 0, 0, 0);
             }
-            if constexpr (TYPE == JL_Q4_K) {
+            if constexpr (kHasMins<TYPE>) {
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                 const floatx4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(sums[b][q], tail.mins, zero, 0, 0, 0);
                 total[b] += ((acc0 + acc1) * tail.d - accm * tail.dmin) * undo[b][q];
+            } else if constexpr (kPostScale<TYPE>) {
+                total[b] += (acc0 + acc1) * (tail.d * undo[b][q]);
             } else {
                 total[b] += (acc0 + acc1) * undo[b][q];
             }
@@ -866,9 +1082,15 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     const int S = k / 64;
     const int row_blocks = rows > 32 ? 2 : 1;
     const int nbb = jl_skinny_padded_rows(rows) / 16;
+    const int quad = quad_bytes(type);
+    if (quad == 0) return JL_OK;
+    for (int i = 0; i < count; i++)
+        if (weights[i]->type != type) return JL_OK;
+    // a span is a whole number of 256-column blocks and of 16-byte pieces (Q6_K: 8 blocks of 210
+    // bytes, IQ4_XS: 2 of 136), and so is a row
     int Ss = max_slices(nbb);
-    while (Ss > 4 && S % Ss) Ss -= 4;
-    if (S % Ss) return JL_OK;
+    while (Ss > 4 && (S % Ss || (Ss / 4 * quad) % 16)) Ss -= 4;
+    if (S % Ss || (Ss / 4 * quad) % 16 || (S / 4 * quad) % 16) return JL_OK;
     // up to 16 rows: a workgroup walks two spans itself (no partial sums to fold for rows of up to
     // 4096 columns); more rows leave no registers for a second set of activation fragments
     const int zin = (nbb == 1 && (S / Ss) % 2 == 0) ? 2 : 1;
@@ -900,11 +1122,11 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     p.Ss = Ss;
     p.Z = Z;
     p.row_blocks = row_blocks;
-    p.span_bytes = Ss * (type == JL_Q8_0 ? 68 : 36);
+    p.span_bytes = Ss / 4 * quad;
     if (Z > 1 && (size_t)Z * (16 * nbb * row_blocks) * groups * 16 * sizeof(float) > plane_bytes) return JL_OK;
 
     const int threads = 16 * Ss;   // compute threads; the copy and fold waves come on top
-    const int per_wave = type == JL_Q8_0 ? 18 : 10;
+    const int per_wave = loads_per_wave(type);
     const int n_loads = (kGroup * ((p.span_bytes + 16) / 16) + 64 * kDmaWaves - 1) / (64 * kDmaWaves);
     if (n_loads > per_wave) return JL_OK;
     const int stage_bytes = n_loads * 64 * kDmaWaves * 16;
@@ -928,6 +1150,21 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
         case JL_Q4_K:
             return dual ? launch_nbb<JL_Q4_K, true>(ctx, p, nbb, zin, threads, lds, groups)
                         : launch_nbb<JL_Q4_K, false>(ctx, p, nbb, zin, threads, lds, groups);
+        case JL_Q6_K:
+            return dual ? launch_nbb<JL_Q6_K, true>(ctx, p, nbb, zin, threads, lds, groups)
+                        : launch_nbb<JL_Q6_K, false>(ctx, p, nbb, zin, threads, lds, groups);
+        case JL_Q5_K:
+            return dual ? launch_nbb<JL_Q5_K, true>(ctx, p, nbb, zin, threads, lds, groups)
+                        : launch_nbb<JL_Q5_K, false>(ctx, p, nbb, zin, threads, lds, groups);
+        case JL_Q4_1:
+            return dual ? launch_nbb<JL_Q4_1, true>(ctx, p, nbb, zin, threads, lds, groups)
+                        : launch_nbb<JL_Q4_1, false>(ctx, p, nbb, zin, threads, lds, groups);
+        case JL_Q5_0:
+            return dual ? launch_nbb<JL_Q5_0, true>(ctx, p, nbb, zin, threads, lds, groups)
+                        : launch_nbb<JL_Q5_0, false>(ctx, p, nbb, zin, threads, lds, groups);
+        case JL_IQ4_XS:
+            return dual ? launch_nbb<JL_IQ4_XS, true>(ctx, p, nbb, zin, threads, lds, groups)
+                        : launch_nbb<JL_IQ4_XS, false>(ctx, p, nbb, zin, threads, lds, groups);
         default:
             *taken = false;
             return JL_OK;

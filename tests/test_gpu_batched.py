@@ -401,11 +401,95 @@ def test_two_pass_prefill_qkv_and_gate_up(ctx):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
 
 
-@pytest.mark.parametrize("t", [O.Q5_K, O.Q6_K, O.Q4_1, O.Q5_0, O.IQ4_XS])
+MINOR = [O.Q5_K, O.Q6_K, O.Q4_1, O.Q5_0, O.IQ4_XS]
+
+
+@pytest.mark.parametrize("t", MINOR)
+@pytest.mark.parametrize("d,n,rows,active", [(1000, 2048, 8, 8), (1100, 4096, 32, 29), (1030, 6144, 64, 64),
+                                             (1000, 14336, 17, 17), (1500, 2048, 1, 1)])
+def test_minor_types_stream_their_weights_at_up_to_64_rows(ctx, t, d, n, rows, active):
+    """Q6_K / Q5_K / Q4_1 / Q5_0 / IQ4_XS at up to 64 rows run the weight-streaming kernel like the
+    three main types (the reference has tiled batch kernels for each: QuantizedBatchProjections.java:
+    168-281): plain, residual and gate/up against the oracle, rows past the active ones untouched.
+    The workspace is sized for 16 output columns -- room for partial sums, far too small for an fp16
+    copy of these weights -- so a call that fell back to decoding the weights would be refused."""
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("minor type, streaming", t, d, n, rows, active)
+    raw = synthetic.weight(t, d, n, seed=9700 + d)
+    raw_up = synthetic.weight(t, d, n, seed=9701 + d)
+    X = synthetic.activations((rows, n), seed=9702 + rows)
+    g = O.matmul_batch(t, raw, X[:active], d, n)
+    u = O.matmul_batch(t, raw_up, X[:active], d, n)
+    mg, mu = magnitude(t, raw, X[:active], d, n), magnitude(t, raw_up, X[:active], d, n)
+    w, w_up = ctx.load_weight(t, raw, d, n), ctx.load_weight(t, raw_up, d, n)
+    proj = QuantizedBatchProjections(ctx, rows, n, 16)
+    assert proj.workspace_bytes() < 2 * d * n      # no room for 2 bytes per weight
+    xd = ctx.from_numpy(X)
+    start = synthetic.activations((rows, d), seed=9703)
+    plain = ctx.float_array(rows * d, fill=UNTOUCHED)
+    res = ctx.from_numpy(start)
+    hb = ctx.float_array(rows * d, fill=UNTOUCHED)
+    proj.projection(xd, plain, w, n, d, False, activeRows=active)
+    proj.projection(xd, res, w, n, d, True, activeRows=active)
+    proj._gemm([w, w_up], xd, hb, active, d, 0, L.JL_SWIGLU)
+    ctx.sync()
+    got, got_res, got_hb = (a.get().reshape(rows, d) for a in (plain, res, hb))
+    assert np.all(got[active:] == UNTOUCHED) and np.all(got_hb[active:] == UNTOUCHED)
+    assert np.array_equal(got_res[active:], start[active:])
+    err = rel_err(got[:active], g, mg)
+    assert err < F16_BOUND, err
+    assert err < 3e-4, err
+    assert rel_err(got_res[:active], g.astype(np.float64) + start[:active], mg + np.abs(start[:active]) * 1e-6) < 3e-4
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(active, d)
+    bound = 3e-4 * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(got_hb[:active].astype(np.float64) - ref) <= bound)
+    w.free()
+    w_up.free()
+
+
+@pytest.mark.parametrize("t", MINOR)
+def test_minor_type_super_blocks_with_extreme_scales(ctx, t):
+    """Scales at their extremes: every sub-block scale / minimum field at its largest, the signed
+    Q6_K scales at -128 (where scale x quant passes 2048 and a fragment is rounded), quants at both
+    ends -- against the oracle at 9 rows."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("minor type, extreme scales", t)
+    d, n, rows = 48, 2048, 9
+    raw = synthetic.weight(t, d, n, seed=9800).copy()
+    bb, be = O.block_bytes(t), O.block_elems(t)
+    blocks = raw.reshape(-1, bb)
+    rng = np.random.default_rng(9801)
+    pick = rng.random(blocks.shape[0]) < 0.5
+    if t == O.Q6_K:
+        blocks[pick, 192:208] = np.where(rng.random((int(pick.sum()), 16)) < 0.5, 0x80, 0x7F).astype(np.uint8)
+        blocks[pick, :192] = np.where(rng.random((int(pick.sum()), 192)) < 0.5, 0x00, 0xFF).astype(np.uint8)
+    elif t == O.Q5_K:
+        blocks[pick, 4:16] = 0xFF
+        blocks[pick, 16:] = np.where(rng.random((int(pick.sum()), bb - 16)) < 0.5, 0x00, 0xFF).astype(np.uint8)
+    elif t == O.IQ4_XS:
+        blocks[pick, 2:8] = np.where(rng.random((int(pick.sum()), 6)) < 0.5, 0x00, 0xFF).astype(np.uint8)
+        blocks[pick, 8:] = np.where(rng.random((int(pick.sum()), bb - 8)) < 0.5, 0x00, 0x77).astype(np.uint8)
+    else:   # Q4_1 (d, m | 16 B), Q5_0 (d | 4 B | 16 B): quants and fifth bits at both ends
+        head = 4 if t == O.Q4_1 else 2
+        blocks[pick, head:] = np.where(rng.random((int(pick.sum()), bb - head)) < 0.5, 0x00, 0xFF).astype(np.uint8)
+    raw = blocks.reshape(-1)
+    X = synthetic.activations((rows, n), seed=9802)
+    ref = O.matmul_batch(t, raw, X, d, n)
+    out = ctx.float_array(rows * d, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, rows, n, 16).projection(ctx.from_numpy(X), out, ctx.load_weight(t, raw, d, n), n, d, False)
+    ctx.sync()
+    err = rel_err(out.get().reshape(rows, d), ref, magnitude(t, raw, X, d, n))
+    assert err < 5e-4, err
+
+
+@pytest.mark.parametrize("t", MINOR)
 @pytest.mark.parametrize("d,n,T,residual", [(300, 512, 8, False), (1000, 2048, 100, True), (4096, 256, 600, False)])
 def test_k_quant_batched_rows_take_the_decode_once_path(ctx, t, d, n, T, residual):
-    """A Q6_K / Q5_K / Q4_1 / Q5_0 / IQ4_XS weight has no decode-in-the-loop kernel: every batched call decodes it to fp16 into
-    the workspace and runs the fp16 GEMM, few rows or many; partial batches leave the rest alone."""
+    """A Q6_K / Q5_K / Q4_1 / Q5_0 / IQ4_XS weight has no decode-in-the-loop GEMM: batched calls of
+    more than 64 rows (and shapes the weight-streaming kernel does not take) decode it to fp16 into
+    the workspace and run the fp16 GEMM; partial batches leave the rest alone."""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
     say("k-quant batched", t, d, n, T, residual)
