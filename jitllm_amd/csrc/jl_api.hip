@@ -28,6 +28,7 @@ static void context_release(jl_context *ctx) {
         if (ctx->bounce_done[i]) (void)hipEventDestroy(ctx->bounce_done[i]);
     if (ctx->bounce) (void)hipHostFree(ctx->bounce);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->arrivals) (void)hipFree(ctx->arrivals);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -67,6 +68,10 @@ static int context_create(int device, hipStream_t borrowed, bool borrow, jl_cont
         ctx->owns_stream = true;
     }
     hipError_t e = hipMalloc(&ctx->scratch, JL_CONTEXT_SCRATCH_BYTES);   // written before it is read
+    if (e == hipSuccess) e = hipMalloc((void **)&ctx->arrivals, JL_CONTEXT_ARRIVALS * sizeof(uint32_t));
+    // (on the context's own stream, which does not wait for the default stream, and waited for)
+    if (e == hipSuccess) e = hipMemsetAsync(ctx->arrivals, 0, JL_CONTEXT_ARRIVALS * sizeof(uint32_t), ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e == hipSuccess) e = hipHostMalloc((void **)&ctx->bounce, 2 * (size_t)JL_BOUNCE_HALF_BYTES, hipHostMallocDefault);
     for (int i = 0; i < 2 && e == hipSuccess; i++) e = hipEventCreateWithFlags(&ctx->bounce_done[i], hipEventDisableTiming);
     if (e != hipSuccess) {

@@ -56,7 +56,8 @@ struct SkinnyParams {
     const uint8_t *w_up;      // JL_SWIGLU: the up weight (a group is 8 gate rows + 8 up rows)
     const float *X;           // [rows x k] fp32 activations
     float *C;
-    float *planes;            // Z > 1: [Z][16 * NBB][groups * 16] partial sums
+    float *planes;            // Z > 1: [Z][row blocks][groups][64 lanes] x 4 partial sums, as the fold's lanes hold them
+    uint32_t *arrivals;       // Z > 1: one counter per (set of workgroups that share their groups, row block); all 0 between calls
     int rows;                 // active activation rows
     int k;
     int64_t ldo, col_offset;
@@ -148,6 +149,23 @@ __device__ __forceinline__ void lds_landed(T (&v)[N]) {
         v[i] = t;
     }
 }
+
+// Partial sums that travel from one workgroup to another inside a launch: stores written through to
+// device scope and loads that are served from there (the sc1 cache policy; what the compiler emits
+// for relaxed atomic accesses at agent scope), 16 bytes per lane.  The eight XCDs' L2 caches are
+// not kept coherent by hardware, and the by-the-book alternative -- plain accesses between a
+// release fence and an acquire fence at agent scope -- writes back and invalidates a whole L2 on
+// every fence (measured here: 10-20 us a call).  The load does not wait for its data: agent_landed.
+__device__ __forceinline__ void agent_store_f4(floatx4 *p, floatx4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ floatx4 agent_load_f4(const floatx4 *p) {
+    floatx4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void vm_drained() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void agent_landed(floatx4 &v) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(v) : : "memory"); }
 
 // Never hand an MFMA result straight to this: the matrix pipe does not interlock with an LDS store
 // that reads its destination registers, and the compiler's hazard pass cannot see inside inline
@@ -569,6 +587,30 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     const int stride = gridDim.x / p.Z;
     int mine = wg < total_groups ? (total_groups - wg + stride - 1) / stride : 0;
 
+    // Where lane `o` of a fold keeps the four partial sums of (span run zz, row block b, group).
+    auto plane_at = [&](int zz, int b, int group, int o) {
+        const int64_t slot = (((int64_t)zz * p.row_blocks + blockIdx.y) * NBB + b) * total_groups + group;
+        return (floatx4 *)p.planes + slot * 64 + o;
+    };
+    // The epilogue of one group and row block, by the 64 lanes that hold its sums: lane o has weight
+    // row o % 16 of the group against activation rows 16 b + 4 (o / 16) .. + 3 (in a gate/up group
+    // the lanes of weight rows 8..15 hold the up rows of outputs 0..7 and store nothing).
+    auto finish = [&](int group, int b, int o, const floatx4 &sum, const floatx4 &sum_up) {
+        const int n = o & 15, go = o >> 4;
+        const Segment sg = segment_of(group);
+        const int local = (group - sg.group_begin) * out_rows + n;   // output column inside the weight
+        const int m0 = row0 + 16 * b + 4 * go;                       // first of this lane's four activation rows
+        if ((DUAL && n >= 8) || local >= sg.rows) return;
+        float *dst = p.C + (int64_t)m0 * p.ldo + p.col_offset + sg.col_begin + local;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (m0 + e >= p.rows) break;
+            const float r = DUAL ? skinny_swiglu(sum[e], sum_up[e]) : sum[e];
+            if (p.epilogue == JL_RESIDUAL) unsafeAtomicAdd(dst + e * p.ldo, r);   // one add per element, no load to wait for
+            else dst[e * p.ldo] = r;
+        }
+    };
+
     if (wave >= waves && wave < waves + kDmaWaves) {
         // ---- copy waves.  Slot s of a tile is 16 bytes at LDS offset 16 s: row s / slots_per_row,
         // byte 16 (s % slots_per_row) of the row's span.  A slot past the data (the padding behind
@@ -651,10 +693,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             }
         }
         if (mine > 0) __builtin_amdgcn_s_barrier();
-        return;
-    }
-
-    if (wave >= waves + kDmaWaves) {
+    } else if (wave >= waves + kDmaWaves) {
         // ---- fold waves.  The partial sums of group it (buffer it % kParities) are complete one
         // tile after the group's last one -- the late compute waves multiply a tile behind -- and
         // are overwritten three groups later, behind barriers these waves take part in.  With two
@@ -665,19 +704,14 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         // are the up rows of outputs 0..7.  Lane o of this wave adds the waves' partials of its
         // (b, o) in wave order and applies the epilogue.
         const int o = lane;
-        const int n = o & 15;
-        const int go = o >> 4;
         // with two fold waves and two row blocks each takes one block (the fold of a group has one
         // tile's time when the workgroup walks a single span)
         const int fw = wave - waves - kDmaWaves;
         // its few instructions go ahead of the compute waves' on the SIMD they share: every
         // barrier between two folds waits for this wave
         __builtin_amdgcn_s_setprio(2);
-        float *const c_lane = p.C + (int64_t)(row0 + 4 * go) * p.ldo + p.col_offset + n;
         auto fold = [&](int group, int par) {
-            const Segment sg = segment_of(group);
             const uint32_t pbase = part0 + par * partial_bytes + o * 16;
-            const int local = (group - sg.group_begin) * out_rows + n;   // output column inside the weight
 #pragma unroll
             for (int b = 0; b < NBB; b++) {
                 if (kFoldWaves > 1 && (NBB > 1 ? b != fw : fw != 0)) continue;
@@ -703,23 +737,14 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                         if constexpr (DUAL) sum_up += u[j];
                     }
                 }
-                const int m0 = row0 + 16 * b + 4 * go;   // first of this lane's four activation rows
                 if (p.Z > 1) {
-                    // partial sums of this span: [z][row][group * 16 + weight row of the group]
-                    float *pp = p.planes + ((int64_t)z * (16 * NBB * p.row_blocks) + m0) * ((int64_t)total_groups * 16) + group * 16 + n;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) pp[(int64_t)e * total_groups * 16] = sum[e];
+                    // this span's partial sums, 16 bytes per lane: the workgroup that arrives last
+                    // adds the spans' in span order (the tail of the kernel)
+                    asm volatile("" : "+v"(sum));   // (plain vector arithmetic has run on it: no matrix-pipe hazard)
+                    agent_store_f4(plane_at(z, b, group, o), sum);
                     continue;
                 }
-                if ((DUAL && n >= 8) || local >= sg.rows) continue;
-                float *dst = c_lane + (int64_t)(16 * b) * p.ldo + sg.col_begin + (local - n);
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    if (m0 + e >= p.rows) break;
-                    const float r = DUAL ? skinny_swiglu(sum[e], sum_up[e]) : sum[e];
-                    if (p.epilogue == JL_RESIDUAL) unsafeAtomicAdd(dst + e * p.ldo, r);   // one add per element, no load to wait for
-                    else dst[e * p.ldo] = r;
-                }
+                finish(group, b, o, sum, sum_up);
             }
         };
         // The late compute waves (below) finish group it during the tile after its last one, so
@@ -738,9 +763,8 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             __builtin_amdgcn_s_barrier();
             for (; folded < mine; folded++) fold(wg + folded * stride, folded % kParities);
         }
-        return;
-    }
-
+        __builtin_amdgcn_s_setprio(0);
+    } else {
     // ---- compute waves
     const int c = lane & 15;                   // weight row of the group; activation row of a row block
     const int g = lane >> 4;                   // which of the wave's four slices
@@ -949,78 +973,75 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
         }
     }
     if (mine > 0) __builtin_amdgcn_s_barrier();
-}
+    }
 
-// Adds the spans' partial sums in span order and applies the epilogue; one thread per activation
-// row and four consecutive weight rows of a group (16-byte loads from the planes).
-template <bool DUAL>
-__global__ void __launch_bounds__(256) jl_skinny_reduce(SkinnyParams p, int padded_rows) {
-    const int total_groups = p.seg_group_begin[p.nseg];
-    const int v = (blockIdx.x * blockDim.x + threadIdx.x) * 4;  // group * 16 + first row of the group
-    const int m = blockIdx.y;
-    if (v >= total_groups * 16 || m >= p.rows) return;
-    const int group = v >> 4, r = v & 15;
-    if (DUAL && r >= 8) return;
-    int seg_rows = p.seg_rows[0], seg_begin = 0, seg_col = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxSeg; i++) {
-        if (i < p.nseg && group >= p.seg_group_begin[i]) {
-            seg_rows = p.seg_rows[i];
-            seg_begin = p.seg_group_begin[i];
-            seg_col = p.seg_col_begin[i];
+    // ---- rows cut across workgroups (Z > 1): the workgroup of a set that finishes last adds the
+    // set's partial sums in span order and applies the epilogue -- no launch behind this one.  The
+    // Z workgroups of a set (same groups, one span run each) count themselves in on the set's
+    // counter once their partial sums have been written through to device scope; the one that draws
+    // the last number reads every span's planes from there (its own included: one order of addition
+    // whoever is last) and finishes the set's groups with all twelve waves.  Nobody waits for
+    // anybody: a workgroup that is not last is done.  The counter is back at zero for the next call.
+    if (p.Z > 1 && mine > 0) {
+        vm_drained();   // the fold waves' plane stores have completed
+        __builtin_amdgcn_s_barrier();
+        uint32_t *flag = (uint32_t *)lds;      // the ring is no longer in use
+        if (wave == waves + kDmaWaves && lane == 0) {
+            uint32_t *counter = p.arrivals + blockIdx.y * stride + wg;
+            const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (before == (uint32_t)(p.Z - 1)) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *flag = before;
         }
-    }
-    const int out_rows = DUAL ? 8 : 16;
-    const int local = (group - seg_begin) * out_rows + r;
-    if (local >= seg_rows) return;
-    const int64_t width = (int64_t)total_groups * 16;
-    const float *pp = p.planes + (int64_t)m * width + v;
-    float *dst = p.C + (int64_t)m * p.ldo + p.col_offset + seg_col + local;
-    const bool add = !DUAL && p.epilogue == JL_RESIDUAL;
-    const bool whole = local + 3 < seg_rows && (((uintptr_t)dst) & 15) == 0;
-    // Every load of the thread goes out before the first sum needs one -- the planes four at a
-    // time, the output's old value with them -- so the kernel waits for memory once, not once per
-    // plane; absent planes add +0, which changes nothing (a running sum that began at +0 is never -0).
-    float4 o = {0.f, 0.f, 0.f, 0.f};
-    if (add && whole) o = *(const float4 *)dst;
-    float4 s = {0.f, 0.f, 0.f, 0.f}, u = {0.f, 0.f, 0.f, 0.f};
-    const int64_t plane = (int64_t)padded_rows * width;
-    for (int z0 = 0; z0 < p.Z; z0 += 4) {
-        float4 a[4], c[4];
+        __builtin_amdgcn_s_barrier();
+        if (*flag != (uint32_t)(p.Z - 1)) return;
+        // This wave's (group, row block) pairs are wave, wave + 12, ...; a pair has Z planes.  The
+        // loads of up to kChunk planes are in flight at a time (one round trip to memory per chunk)
+        // and are added in span order; a pair is finished when its last plane has been added.
+        const int all_waves = blockDim.x >> 6;
+        const int pairs = mine * NBB;
+        const int my_pairs = wave < pairs ? (pairs - wave + all_waves - 1) / all_waves : 0;
+        const int items = my_pairs * p.Z;
+        constexpr int kChunk = DUAL ? 8 : 16;
+        floatx4 sum = {0.f, 0.f, 0.f, 0.f}, sum_up = {0.f, 0.f, 0.f, 0.f};
+        // (two walks over the same list of (pair, span run): one issues loads, one adds; counters
+        // instead of a division per item)
+        int lq = wave, lz = 0, aq = wave, az = 0;
+        for (int base = 0; base < items; base += kChunk) {
+            floatx4 v[kChunk], u[kChunk];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const bool on = z0 + j < p.Z;
-            const float *q = pp + (on ? z0 + j : z0) * plane;
-            a[j] = *(const float4 *)q;
-            if (!on) a[j] = float4{0.f, 0.f, 0.f, 0.f};
-            if (DUAL) {
-                c[j] = *(const float4 *)(q + 8);
-                if (!on) c[j] = float4{0.f, 0.f, 0.f, 0.f};
+            for (int j = 0; j < kChunk; j++) {
+                if (base + j < items) {
+                    const int group = wg + (lq / NBB) * stride, b = lq % NBB;
+                    v[j] = agent_load_f4(plane_at(lz, b, group, lane));
+                    // (a gate/up group keeps the up rows' sums eight lanes on; lanes that have no
+                    // such neighbour read their own group's first lanes and drop the result)
+                    if constexpr (DUAL) u[j] = agent_load_f4(plane_at(lz, b, group, (lane + 8) & 63));
+                    if (++lz == p.Z) {
+                        lz = 0;
+                        lq += all_waves;
+                    }
+                }
+            }
+            vm_drained();
+#pragma unroll
+            for (int j = 0; j < kChunk; j++) {
+                if (base + j < items) {
+                    asm volatile("" : "+v"(v[j]));
+                    sum += v[j];
+                    if constexpr (DUAL) {
+                        asm volatile("" : "+v"(u[j]));
+                        sum_up += u[j];
+                    }
+                    if (++az == p.Z) {
+                        finish(wg + (aq / NBB) * stride, aq % NBB, lane, sum, sum_up);
+                        sum = floatx4{0.f, 0.f, 0.f, 0.f};
+                        sum_up = floatx4{0.f, 0.f, 0.f, 0.f};
+                        az = 0;
+                        aq += all_waves;
+                    }
+                }
             }
         }
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            s.x += a[j].x; s.y += a[j].y; s.z += a[j].z; s.w += a[j].w;
-            if (DUAL) {
-                u.x += c[j].x; u.y += c[j].y; u.z += c[j].z; u.w += c[j].w;
-            }
-        }
-    }
-    float out[4] = {s.x, s.y, s.z, s.w};
-    if (DUAL) {
-        out[0] = skinny_swiglu(s.x, u.x); out[1] = skinny_swiglu(s.y, u.y);
-        out[2] = skinny_swiglu(s.z, u.z); out[3] = skinny_swiglu(s.w, u.w);
-    }
-    if (whole) {
-        if (add) {
-            *(float4 *)dst = float4{o.x + out[0], o.y + out[1], o.z + out[2], o.w + out[3]};
-        } else {
-            *(float4 *)dst = float4{out[0], out[1], out[2], out[3]};
-        }
-    } else {
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-            if (local + e < seg_rows) dst[e] = add ? dst[e] + out[e] : out[e];
     }
 }
 
@@ -1040,14 +1061,13 @@ int launch(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int gro
     if (p.row_blocks > 1) per_span = per_span / 8 * 8;
     if (per_span < 1) per_span = 1;
     if (per_span > groups) per_span = groups;
+    if (p.Z > 1 && per_span * p.row_blocks > JL_CONTEXT_ARRIVALS) {
+        return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: %d workgroup sets exceed the context's %d arrival counters",
+                       per_span * p.row_blocks, JL_CONTEXT_ARRIVALS);
+    }
     hipLaunchKernelGGL(fn, dim3(per_span * p.Z, p.row_blocks), dim3(threads + 64 * (kDmaWaves + kFoldWaves)), lds,
                        ctx->stream, p);
     JL_HIP(hipGetLastError());
-    if (p.Z > 1) {
-        hipLaunchKernelGGL(jl_skinny_reduce<DUAL>, dim3((groups * 4 + 255) / 256, p.rows), dim3(256), 0,
-                           ctx->stream, p, 16 * NBB * p.row_blocks);
-        JL_HIP(hipGetLastError());
-    }
     return JL_OK;
 }
 
@@ -1113,6 +1133,7 @@ int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int 
     p.X = X;
     p.C = C;
     p.planes = planes;
+    p.arrivals = ctx->arrivals;
     p.rows = rows;
     p.k = k;
     p.ldo = ldo;

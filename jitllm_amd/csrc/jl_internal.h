@@ -15,6 +15,10 @@ struct jl_context {
     char name[128];
     void *scratch;   // JL_CONTEXT_SCRATCH_BYTES of device memory for results handed from one launch of
                      // a call to the next (calls on a context are ordered on its stream)
+    // JL_CONTEXT_ARRIVALS counters, all zero between calls: the workgroups of a batched-decode launch
+    // that share a set of output rows count themselves in here, and the last one to arrive folds
+    // their partial sums (and puts the counter back to zero).
+    uint32_t *arrivals;
     // Pinned host memory that jl_upload / jl_download stage the caller's pageable memory through, two
     // halves in turn: every transfer the device sees is then a DMA from / to pinned memory, and the
     // caller's pointer is only ever touched by a host memcpy.
@@ -22,6 +26,7 @@ struct jl_context {
     hipEvent_t bounce_done[2];
 };
 #define JL_CONTEXT_SCRATCH_BYTES 4096
+#define JL_CONTEXT_ARRIVALS 1024
 #define JL_BOUNCE_HALF_BYTES (8u << 20)
 
 struct jl_weight {

@@ -401,6 +401,37 @@ def test_two_pass_prefill_qkv_and_gate_up(ctx):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= bound)
 
 
+@pytest.mark.parametrize("t,d,n,rows", [(O.Q4_K, 1024, 12288, 32), (O.Q8_0, 520, 4096, 64), (O.Q4_0, 4096, 6144, 9)])
+def test_rows_cut_across_workgroups_are_folded_afresh_on_every_call(ctx, t, d, n, rows):
+    """Rows longer than one workgroup's span are cut across workgroups; the one that finishes last
+    adds the others' partial sums, which travel through the workspace.  Calls that follow one
+    another without a pause, with two different inputs in turn and the same workspace, must each
+    see their own partial sums -- never what an earlier call left in a cache -- and must give the
+    same bits every time (the order of addition does not depend on who is last)."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("folded afresh", NAMES[t], d, n, rows)
+    raw = synthetic.weight(t, d, n, seed=9900 + d)
+    w = ctx.load_weight(t, raw, d, n)
+    Xs = [synthetic.activations((rows, n), seed=9901), synthetic.activations((rows, n), seed=9902) * np.float32(3.0)]
+    xd = [ctx.from_numpy(X) for X in Xs]
+    proj = QuantizedBatchProjections(ctx, rows, n, d)
+    rounds = 12
+    outs = [[ctx.float_array(rows * d, fill=UNTOUCHED) for _ in range(rounds)] for _ in Xs]
+    for r in range(rounds):
+        for i in range(2):
+            proj.projection(xd[i], outs[i][r], w, n, d, False)
+    ctx.sync()
+    dot = O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256
+    for i, X in enumerate(Xs):
+        first = outs[i][0].get().reshape(rows, d)
+        err = rel_err(first, O.matmul_batch(t, raw, X, d, n, dot), magnitude(t, raw, X, d, n))
+        assert err < 2e-4, err
+        for r in range(1, rounds):
+            assert np.array_equal(outs[i][r].get().reshape(rows, d).view(np.uint32), first.view(np.uint32)), (i, r)
+    w.free()
+
+
 MINOR = [O.Q5_K, O.Q6_K, O.Q4_1, O.Q5_0, O.IQ4_XS]
 
 
