@@ -1136,6 +1136,15 @@ def main():
             "o [2048 x 2048] +=": per_kernel(os_, LAYERS, gemv_bytes(DIM, DIM)),
             "down [2048 x 8192] +=": per_kernel(downs, LAYERS, gemv_bytes(DIM, HIDDEN)),
         }
+        # the vocabulary projection over two device copies of its weight in turn (2 x 280 MB: what
+        # one launch reads, the memory-side cache has lost by the time the launch comes round again)
+        wcls_b = ctx.load_weight(t, host["wcls"], VOCAB, DIM)
+
+        def vocabs():
+            for w in (wcls, wcls_b):
+                proj.floatMatvec(acts["xb"], acts["logits"], w, DIM, VOCAB)
+        kernels["vocabulary [128256 x 2048]"] = per_kernel(vocabs, 2, gemv_bytes(VOCAB, DIM))
+        wcls_b.free()
         # the single-weight instances of the tile kernel (q|k|v, o, down, vocabulary) together:
         # everything in the step that is not a gate/up launch
         single_bytes = total_bytes - LAYERS * gate_up_bytes
