@@ -157,7 +157,9 @@ __device__ __forceinline__ void lds_landed(T (&v)[N]) {
 // release fence and an acquire fence at agent scope -- writes back and invalidates a whole L2 on
 // every fence (measured here: 10-20 us a call).  The load does not wait for its data: agent_landed.
 __device__ __forceinline__ void agent_store_f4(floatx4 *p, floatx4 v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+    // (a store of more than 8 bytes reads its data registers for two more cycles: the wait states
+    // the compiler would place before a write of those registers, had it emitted the store itself)
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ floatx4 agent_load_f4(const floatx4 *p) {
     floatx4 v;
