@@ -1,5 +1,8 @@
-"""Committed golden vectors (tests/golden/): the oracle must keep reproducing them bit for bit on the
-CPU, and the HIP library must match them on the GPU without the oracle recomputing anything."""
+"""Committed vectors (tests/golden/).  projection_golden.npz is a freeze of the oracle -- inputs from
+the reference's test recipes, outputs written by oracle/ itself (make_golden.py) -- not a vector
+the reference holds: the oracle must keep reproducing it bit for bit on the CPU, and the HIP library
+must match it on the GPU without the oracle recomputing anything.  reference_known_answers.json is
+the one file of answers the reference itself states (Q4_0DecodeTest.java:95-126)."""
 import json
 import os
 
