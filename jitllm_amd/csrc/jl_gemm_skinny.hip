@@ -155,7 +155,8 @@ __device__ __forceinline__ void lds_landed(T (&v)[N]) {
 // for relaxed atomic accesses at agent scope), 16 bytes per lane.  The eight XCDs' L2 caches are
 // not kept coherent by hardware, and the by-the-book alternative -- plain accesses between a
 // release fence and an acquire fence at agent scope -- writes back and invalidates a whole L2 on
-// every fence (measured here: 10-20 us a call).  The load does not wait for its data: agent_landed.
+// every fence (measured here: 10-20 us a call).  The load does not wait for its data: the caller
+// waits (s_waitcnt vmcnt) in a statement that every destination register passes through.
 __device__ __forceinline__ void agent_store_f4(floatx4 *p, floatx4 v) {
     // (a store of more than 8 bytes reads its data registers for two more cycles: the wait states
     // the compiler would place before a write of those registers, had it emitted the store itself)
@@ -163,11 +164,10 @@ __device__ __forceinline__ void agent_store_f4(floatx4 *p, floatx4 v) {
 }
 __device__ __forceinline__ floatx4 agent_load_f4(const floatx4 *p) {
     floatx4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(v) : "v"(p) : "memory");
     return v;
 }
 __device__ __forceinline__ void vm_drained() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ void agent_landed(floatx4 &v) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(v) : : "memory"); }
 
 // Never hand an MFMA result straight to this: the matrix pipe does not interlock with an LDS store
 // that reads its destination registers, and the compiler's hazard pass cannot see inside inline
@@ -1012,6 +1012,10 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             floatx4 v[kChunk], u[kChunk];
 #pragma unroll
             for (int j = 0; j < kChunk; j++) {
+                // (slots past the list hold zeros: every register of the chunk is defined when the
+                // one wait below takes them all)
+                v[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+                u[j] = floatx4{0.f, 0.f, 0.f, 0.f};
                 if (base + j < items) {
                     const int group = wg + (lq / NBB) * stride, b = lq % NBB;
                     v[j] = agent_load_f4(plane_at(lz, b, group, lane));
@@ -1024,16 +1028,24 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                     }
                 }
             }
-            vm_drained();
+            // one wait for the chunk; every destination passes through it, so that no use of one
+            // can move ahead of it
+            if constexpr (DUAL) {
+                asm volatile("s_waitcnt vmcnt(0)"
+                             : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]),
+                               "+v"(u[0]), "+v"(u[1]), "+v"(u[2]), "+v"(u[3]), "+v"(u[4]), "+v"(u[5]), "+v"(u[6]), "+v"(u[7])
+                             : : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)"
+                             : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]),
+                               "+v"(v[8]), "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15])
+                             : : "memory");
+            }
 #pragma unroll
             for (int j = 0; j < kChunk; j++) {
                 if (base + j < items) {
-                    asm volatile("" : "+v"(v[j]));
                     sum += v[j];
-                    if constexpr (DUAL) {
-                        asm volatile("" : "+v"(u[j]));
-                        sum_up += u[j];
-                    }
+                    if constexpr (DUAL) sum_up += u[j];
                     if (++az == p.Z) {
                         finish(wg + (aq / NBB) * stride, aq % NBB, lane, sum, sum_up);
                         sum = floatx4{0.f, 0.f, 0.f, 0.f};
