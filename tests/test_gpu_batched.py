@@ -479,6 +479,55 @@ def test_minor_types_stream_their_weights_at_up_to_64_rows(ctx, t, d, n, rows, a
     w_up.free()
 
 
+def _random_minor_shapes():
+    """Seeded shapes for the five minor types across the streaming kernel's geometries: row lengths
+    it takes for each type (a span must be a whole number of 16-byte pieces: Q6_K rows of a multiple
+    of 2048 columns, IQ4_XS of 512, the others of 256) and some it does not (those fall back to the
+    decode-once path, which the ordinary workspace holds), 1 .. 64 rows, partial batches."""
+    rng = np.random.default_rng(20261127)
+    shapes = []
+    for t in MINOR:
+        for n in (256, 512, 1280, 2048, 2304, 4096, 6144, 8192):
+            rows = int(rng.choice([1, 2, 7, 8, 9, 16, 17, 31, 32, 33, 48, 64]))
+            d = int(rng.integers(1, 260))
+            active = rows if rng.integers(0, 2) else int(rng.integers(1, rows + 1))
+            shapes.append((t, d, n, rows, active))
+    return shapes
+
+
+@pytest.mark.parametrize("t,d,n,rows,active", _random_minor_shapes())
+def test_minor_types_on_random_shapes(ctx, t, d, n, rows, active):
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("minor type, random shape", t, d, n, rows, active)
+    raw = synthetic.weight(t, d, n, seed=9850 + d)
+    raw_up = synthetic.weight(t, d, n, seed=9851 + d)
+    X = synthetic.activations((rows, n), seed=9852 + n)
+    g = O.matmul_batch(t, raw, X[:active], d, n)
+    u = O.matmul_batch(t, raw_up, X[:active], d, n)
+    mg, mu = magnitude(t, raw, X[:active], d, n), magnitude(t, raw_up, X[:active], d, n)
+    w, w_up = ctx.load_weight(t, raw, d, n), ctx.load_weight(t, raw_up, d, n)
+    proj = QuantizedBatchProjections(ctx, rows, n, 2 * d)
+    xd = ctx.from_numpy(X)
+    plain = ctx.float_array(rows * d, fill=UNTOUCHED)
+    res = ctx.float_array(rows * d, fill=UNTOUCHED)
+    hb = ctx.float_array(rows * d, fill=UNTOUCHED)
+    proj.projection(xd, plain, w, n, d, False, activeRows=active)
+    proj.projection(xd, res, w, n, d, True, activeRows=active)
+    proj._gemm([w, w_up], xd, hb, active, d, 0, L.JL_SWIGLU)
+    ctx.sync()
+    got, got_res, got_hb = (a.get().reshape(rows, d) for a in (plain, res, hb))
+    for a in (got, got_res, got_hb):
+        assert np.all(a[active:] == UNTOUCHED)
+    assert rel_err(got[:active], g, mg) < 5e-4
+    assert rel_err(got_res[:active], g.astype(np.float64) + float(UNTOUCHED), mg + 12345.5 * 6e-8) < 5e-4
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(active, d)
+    bound = 5e-4 * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(got_hb[:active].astype(np.float64) - ref) <= bound)
+    w.free()
+    w_up.free()
+
+
 @pytest.mark.parametrize("t", MINOR)
 def test_minor_type_super_blocks_with_extreme_scales(ctx, t):
     """Scales at their extremes: every sub-block scale / minimum field at its largest, the signed
