@@ -242,7 +242,7 @@ def decode_step(proj, layers, wcls, acts):
     proj.floatMatvec(acts["xb"], acts["logits"], wcls, DIM, VOCAB)
 
 
-def decode_step_fused_rms(proj, layers, wcls, acts):
+def decode_step_fused_rms(proj, layers, wcls, acts, one_call=True):
     """The same token with the reference's fused decode kernels: the attention norm folded into
     q|k|v behind its own scale (fusedRmsNormQKVMatmulQ8), the FFN norm computed and folded inside
     gate/up (fullyFusedRmsNormFFNGateUpQ8), the final norm folded into the vocabulary projection,
@@ -253,8 +253,12 @@ def decode_step_fused_rms(proj, layers, wcls, acts):
         proj.residualMatvec(acts["xb"], w["wo"], DIM, DIM)
         proj.fullyFusedRmsNormGateUp(acts["x"], acts["rms_ffn"], 1e-5, w["w1"], w["w3"], DIM, HIDDEN)
         proj.residualMatvec(acts["hb"], w["w2"], HIDDEN, DIM)
-    proj.rmsMatvec(acts["x"], acts["rms_final"], None, acts["logits"], wcls, DIM, VOCAB, eps=1e-5)
-    proj.argmax(acts["logits"], VOCAB, acts["token"])
+    if one_call:   # the projection's workgroups keep their best logits: one launch fewer
+        proj.matvecArgmax(acts["x"], acts["logits"], wcls, DIM, VOCAB, acts["token"],
+                          rmsWeights=acts["rms_final"], eps=1e-5)
+    else:
+        proj.rmsMatvec(acts["x"], acts["rms_final"], None, acts["logits"], wcls, DIM, VOCAB, eps=1e-5)
+        proj.argmax(acts["logits"], VOCAB, acts["token"])
 
 
 def bench_fused_rms(ctx, hip, proj, layers, wcls, acts, host, steps, warmup):
@@ -268,8 +272,8 @@ def bench_fused_rms(ctx, hip, proj, layers, wcls, acts, host, steps, warmup):
     acts["token"] = ctx.raw_buffer(4)
     # check: the vocabulary projection of the normalised vector, and the token picked from it
     x0 = acts["x"].get()
-    proj.rmsMatvec(acts["x"], acts["rms_final"], None, acts["logits"], wcls, DIM, VOCAB, eps=1e-5)
-    proj.argmax(acts["logits"], VOCAB, acts["token"])
+    proj.matvecArgmax(acts["x"], acts["logits"], wcls, DIM, VOCAB, acts["token"], rmsWeights=acts["rms_final"],
+                      eps=1e-5)
     ctx.sync()
     logits = acts["logits"].get()
     rows = sample_rows(VOCAB, 128, 7)
@@ -279,11 +283,17 @@ def bench_fused_rms(ctx, hip, proj, layers, wcls, acts, host, steps, warmup):
         raise SystemExit("bench.py: the device's greedy token is not the first maximum of its logits")
     ms = timed_graph(ctx, hip, lambda: decode_step_fused_rms(proj, layers, wcls, acts), steps, warmup)
     st = spread_stats(ms)
+    apart = timed_graph(ctx, hip, lambda: decode_step_fused_rms(proj, layers, wcls, acts, one_call=False), steps,
+                        warmup)
     return {"ms_per_step": st["median"], "ms_stats": st, "tok_s": round(1e3 / statistics.median(ms), 1),
             "launches": 4 * LAYERS + 2, "check_rel_err": err,
+            "ms_per_step_with_argmax_as_its_own_scan": spread_stats(apart)["median"],
             "what": "decode set with the 33 RMS normalisations folded into q|k|v, gate/up and the "
                     "vocabulary projection (scale computed inside each kernel, no normalised vector "
-                    "written) and the greedy token chosen on the device"}
+                    "written) and the greedy token chosen on the device: the vocabulary projection's "
+                    "workgroups keep their best logits and one small launch folds those "
+                    "(ms_per_step_with_argmax_as_its_own_scan: a scan over the logits and that fold, 67 "
+                    "launches)"}
 
 
 def decode_bytes():

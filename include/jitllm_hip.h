@@ -204,6 +204,21 @@ int jl_gemv_gate_up_rms(jl_context *ctx, const jl_weight *w1, const jl_weight *w
 int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
 
 /*
+ * The tail of a greedy decode step in one call: out = w . x, the vocabulary projection -- with the
+ * final RMS normalisation folded in as in jl_gemv_rms when rms_weights is set (rms_scale and eps as
+ * there), x used as it is when rms_weights is null -- and index[0] = jl_argmax(out) (the
+ * vocabulary projection followed by "argmax_sample", LogitsQ8_0Layer.java:92-110,
+ * LogitsFP16Layer.java:217).  out and index[0] are bit for bit what jl_gemv / jl_gemv_rms followed
+ * by jl_argmax leave.  A Q8_0, Q4_0 or Q4_K weight of 2048 or 4096 columns and a multiple of eight
+ * (four) rows takes two launches instead of three: the projection's workgroups keep the largest
+ * logit they store and its row, and the second launch folds those thousand candidates instead of
+ * reading the logits back.  Any other weight the single-token kernels take is the two calls, made
+ * here.
+ */
+int jl_gemv_argmax(jl_context *ctx, const jl_weight *w, const float *x, const float *rms_weights,
+                   const float *rms_scale, float eps, float *out, int32_t *index);
+
+/*
  * jl_argmax for callers that cannot allocate device memory: code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The
  * candidates that the first launch hands to the second -- one (value, index) cell per scanning

@@ -416,6 +416,14 @@ int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
     return jl_launch_argmax(ctx, values, n, index);
 }
 
+int jl_gemv_argmax(jl_context *ctx, const jl_weight *w, const float *x, const float *rms_weights,
+                   const float *rms_scale, float eps, float *out, int32_t *index) {
+    JL_REQUIRE(ctx && w && x && out && index, "jl_gemv_argmax: null argument");
+    JL_REQUIRE(w->rows <= INT32_MAX, "jl_gemv_argmax: %lld rows", (long long)w->rows);
+    const jl_rms rms{rms_weights, rms_scale, eps};
+    return jl_launch_gemv_argmax(ctx, w, x, rms_weights ? &rms : nullptr, out, index);
+}
+
 int jl_argmax_static(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
     JL_REQUIRE(ctx && values && index, "jl_argmax_static: null argument");
     JL_REQUIRE(n > 0, "jl_argmax_static: %lld values", (long long)n);

@@ -57,6 +57,9 @@ struct GemvParams {
     const int8_t *xq;
     const float *xq_scales;
     const int32_t *xq_sums;
+    // The ARGMAX instances leave every workgroup's largest output, and its row, in cell blockIdx.x.
+    float *best_value;
+    int *best_index;
 };
 
 // Bytes of a tile a thread brings in: kX4 sixteen-byte loads and kTail four-byte ones.  For the
@@ -710,8 +713,11 @@ __device__ __forceinline__ uintptr_t uniform_value(uintptr_t v) {
 // (SEGS: the fixed-geometry form of the fused q|k|v, up to three weights side by side.)
 // (PART: rows of fewer than SPT slices -- 11 008, 12 288, 14 336 columns under SPT = 256 -- whose
 // lanes past the row's end idle; everything but the row length is still a constant.)
+// (ARGMAX: a plain projection whose rows lie inside a wave also keeps, per workgroup, the largest
+// value it stored and that value's row -- greedy sampling then folds a thousand cells instead of
+// reading the logits back.)
 template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false,
-          bool PART = false>
+          bool PART = false, bool ARGMAX = false>
 __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first, const uint8_t *w_up_first, const float *x_first, int tiles_first,
               int rows_first, int grid_first, int S_first, int row_bytes_first, int shape_first,
               const float *rms_w_first, GemvParams p) {
@@ -727,6 +733,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     constexpr bool FULL = LEAN && !PART;   // every lane has a slice, every load slot is real data
     static_assert(!PART || LEAN, "rows shorter than SPT slices: a fixed tile shape");
     static_assert(!LEAN || !PACKED, "the packed form has no fixed-geometry instances");
+    static_assert(!ARGMAX || (FULL && !DUAL && !SEGS && SPT <= 64), "the argmax form: whole in-wave rows of one weight");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
     constexpr int L = X4 + Traits<TYPE>::kTail;   // plus (three main types) one 4-byte load
@@ -1074,6 +1081,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     // fill a wave each, so gate/up keeps the LDS hand-over there).
     const bool in_wave = Sp <= (DUAL ? 32 : 64);
     const int r_lds = (DUAL && in_wave) ? (r & 1) * half_rows + (r >> 1) : r;   // tile row this thread reads
+    float best = -INFINITY;   // ARGMAX: the largest value this lane has stored, and its row
+    int best_at = INT_MAX;
     for (int it = 0; it < mine; it++) {
         const int tile = first + it * grid;
         // with two stages nothing was issued after tile `it`: its loads are the youngest
@@ -1124,6 +1133,13 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
                         // no read-modify-write through a load: a load's wait would drain the prefetch ring
                         if (p.epilogue == JL_RESIDUAL) unsafeAtomicAdd(o, v);
                         else *o = v;
+                        if constexpr (ARGMAX) {
+                            // a lane's rows ascend: the strict comparison keeps the first of equals
+                            if (v > best) {
+                                best = v;
+                                best_at = row;
+                            }
+                        }
                     }
                 }
             }
@@ -1139,6 +1155,33 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     if (mine > 0 && !in_wave) {
         __builtin_amdgcn_s_barrier();
         finish(first + (mine - 1) * grid, (mine - 1) & 1);
+    }
+    if constexpr (ARGMAX) {
+        // larger value wins, equal values: the lower row.  Lanes, then waves through the (unused,
+        // rows being in-wave) partial-sum region, then one cell per workgroup.
+        auto keep_better = [](float &v, int &i, float ov, int oi) {
+            if (ov > v || (ov == v && oi < i)) {
+                v = ov;
+                i = oi;
+            }
+        };
+#pragma unroll
+        for (int o = JL_WAVE / 2; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o, JL_WAVE);
+            const int oi = __shfl_xor(best_at, o, JL_WAVE);
+            keep_better(best, best_at, ov, oi);
+        }
+        if (lane == 0) {
+            lds_write_b32(lds0 + wave * 8, __float_as_uint(best));
+            lds_write_b32(lds0 + wave * 8 + 4, (uint32_t)best_at);
+        }
+        __builtin_amdgcn_s_barrier();
+        if (tid == 0) {
+            for (int i = 1; i < THREADS / JL_WAVE; i++)
+                keep_better(best, best_at, __uint_as_float(lds_read_b32(lds0 + i * 8)), (int)lds_read_b32(lds0 + i * 8 + 4));
+            p.best_value[blockIdx.x] = best;
+            p.best_index[blockIdx.x] = best_at;
+        }
     }
 }
 
@@ -1249,13 +1292,17 @@ int blocks_per_cu(const void *fn, int device, int threads, int lds) {
 }
 
 template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false,
-          bool PART = false>
-int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds) {
-    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED, THREADS, SPT, SEGS, PART>;
+          bool PART = false, bool ARGMAX = false>
+int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds, int *cells = nullptr) {
+    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED, THREADS, SPT, SEGS, PART, ARGMAX>;
     int per_cu = blocks_per_cu((const void *)fn, ctx->device, threads, lds);
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
     if (grid > total) grid = total;
+    if (cells) {
+        if (grid > *cells) return JL_NO_CELLS_FORM;   // more workgroups than the caller has cells for
+        *cells = grid;
+    }
     hipLaunchKernelGGL(fn, dim3(grid), dim3(threads), lds, ctx->stream, p.w[0], p.w_up, p.x, total, p.seg_rows[0], grid, p.S, p.row_bytes,
                        p.Sp | (p.R << 10) | (p.nseg << 20), p.rms_w, p);
     JL_HIP(hipGetLastError());
@@ -1286,9 +1333,24 @@ int launch_fixed(jl_context *ctx, const GemvParams &p, int lds, bool full) {
 // columns and, in the 1024-thread form (plain and residual), up to 16384; the side types for
 // whole rows of 2048, 4096 and (plain and residual) 8192 columns.
 template <int TYPE, bool DUAL>
-int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, bool fixed) {
+int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, bool fixed, int *cells = nullptr) {
     // (side types: plain, residual and gate/up only -- the caller has refused the rest)
     constexpr bool kMain = is_main_type(TYPE);
+    if (cells) {
+        // the argmax form: one main-type weight, whole tiles of whole in-wave rows of 2048 or 4096
+        // columns, stored (not accumulated) outputs
+        if constexpr (kMain && !DUAL) {
+            if (fixed && threads == 256 && p.S == p.Sp && p.nseg == 1 && !p.xq && p.epilogue == JL_STORE) {
+                if (p.Sp == 32)
+                    return p.rms_w ? launch_tiles_of<TYPE, false, true, false, 256, 32, false, false, true>(ctx, p, 256, lds, cells)
+                                   : launch_tiles_of<TYPE, false, false, false, 256, 32, false, false, true>(ctx, p, 256, lds, cells);
+                if (p.Sp == 64)
+                    return p.rms_w ? launch_tiles_of<TYPE, false, true, false, 256, 64, false, false, true>(ctx, p, 256, lds, cells)
+                                   : launch_tiles_of<TYPE, false, false, false, 256, 64, false, false, true>(ctx, p, 256, lds, cells);
+            }
+        }
+        return JL_NO_CELLS_FORM;
+    }
     if constexpr (kMain) {
         if (p.xq) return launch_tiles_of<TYPE, DUAL, false, true>(ctx, p, threads, lds);
     }
@@ -1345,10 +1407,12 @@ int launch_generic(jl_context *ctx, const jl_weight *w, const jl_weight *w_up, c
 
 
 int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *const *outs,
-                   const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms, const jl_q8x *xq) {
+                   const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms, const jl_q8x *xq,
+                   jl_best_cells *cells) {
     const int type = w[0]->type;
     const int n = (int)w[0]->cols;
     const int row_bytes = n / jl_block_elems(type) * jl_block_bytes(type);
+    if (cells && !is_main_type(type)) return JL_NO_CELLS_FORM;
     if (xq && !jl_has_fused_kernels(type)) {
         return jl_fail(JL_ERR_UNSUPPORTED, "no packed-activation kernel for a %s weight", jl_type_name(type));
     }
@@ -1391,6 +1455,7 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     }
     if (w_up && ((uintptr_t)w_up->blocks & 15) != 0) fast = false;
 
+    if (cells && !fast) return JL_NO_CELLS_FORM;
     if (!fast && xq) {
         return jl_fail(JL_ERR_UNSUPPORTED,
                        "no packed-activation kernel for a row length of %d (a multiple of 64 up to %d "
@@ -1456,6 +1521,10 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
         p.rms_scale = rms->scale;
         p.rms_eps = rms->eps;
     }
+    if (cells) {
+        p.best_value = cells->value;
+        p.best_index = cells->index;
+    }
 
     const int threads = (R * Sp + 63) / 64 * 64;
     const int lds = tile_lds_bytes(threads, slice, S, is_side_type(type));
@@ -1463,6 +1532,15 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     bool fixed = R * Sp == threads;
     for (int i = 0; i < nseg; i++) fixed = fixed && w[i]->rows % half_rows == 0;
 
+    if (cells) {
+        if (dual) return JL_NO_CELLS_FORM;
+        switch (type) {
+            case JL_Q8_0: return launch_tiles<JL_Q8_0, false>(ctx, p, threads, lds, fixed, &cells->count);
+            case JL_Q4_0: return launch_tiles<JL_Q4_0, false>(ctx, p, threads, lds, fixed, &cells->count);
+            case JL_Q4_K: return launch_tiles<JL_Q4_K, false>(ctx, p, threads, lds, fixed, &cells->count);
+            default: return JL_NO_CELLS_FORM;
+        }
+    }
     switch (type) {
         case JL_Q8_0:
             return dual ? launch_tiles<JL_Q8_0, true>(ctx, p, threads, lds, fixed)

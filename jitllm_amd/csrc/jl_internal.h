@@ -25,7 +25,7 @@ struct jl_context {
     uint8_t *bounce;
     hipEvent_t bounce_done[2];
 };
-#define JL_CONTEXT_SCRATCH_BYTES 4096
+#define JL_CONTEXT_SCRATCH_BYTES 8192
 #define JL_CONTEXT_ARRIVALS 1024
 #define JL_BOUNCE_HALF_BYTES (8u << 20)
 
@@ -110,10 +110,19 @@ struct jl_q8x {
     const float *scales;
     const int32_t *sums;
 };
-// `xq` set: the packed-integer kernels read it instead of `x`.
+// Per-workgroup (largest stored output, its row) cells of a projection, for greedy sampling:
+// `count` is the room going in and the cells written coming out.
+struct jl_best_cells {
+    float *value;
+    int *index;
+    int count;
+};
+#define JL_NO_CELLS_FORM 1   // jl_launch_gemv with `cells`: this launch has no such form, nothing was launched
+// `xq` set: the packed-integer kernels read it instead of `x`.  `cells` set (one weight, JL_STORE):
+// the kernel also leaves them, or the call returns JL_NO_CELLS_FORM.
 int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *const *outs,
                    const jl_weight *w_up, const float *x, int epilogue, const jl_rms *rms,
-                   const jl_q8x *xq = nullptr);
+                   const jl_q8x *xq = nullptr, jl_best_cells *cells = nullptr);
 // `rms_w` set: xb = rms_w * (rms_scale[0] * x) is written and quantised instead of x.
 int jl_launch_quantize_q8(jl_context *ctx, const float *x, const float *rms_w, const float *rms_scale, float *xb,
                           int64_t n, int8_t *quants, float *scales, int32_t *sums);
@@ -125,6 +134,9 @@ int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const jl_weight *
 int jl_launch_dequant_direct(jl_context *ctx, const jl_weight *w, float *out);
 int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale);
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
+// out = w . x (rms set: the normalisation folded in) and index[0] = the first maximum of out.
+int jl_launch_gemv_argmax(jl_context *ctx, const jl_weight *w, const float *x, const jl_rms *rms, float *out,
+                          int32_t *index);
 // jl_argmax with its (value, index) cells in a device array that is part of the library's code
 // object instead of the context's allocation.  jl_static_scratch_init looks that array's address
 // up on the current device (once per device; jl_context_create calls it).

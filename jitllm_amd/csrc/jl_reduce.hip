@@ -126,6 +126,24 @@ __global__ void __launch_bounds__(kArgmaxGroups) jl_argmax_fold(const float *val
     }
 }
 
+// The fold for cells a projection kernel left (one per workgroup, up to a thousand, rows in no
+// particular order from cell to cell): the same rule, a strided walk first.
+constexpr int kProjectionCells = JL_CONTEXT_SCRATCH_BYTES / 8;
+__global__ void __launch_bounds__(kArgmaxThreads) jl_argmax_fold_cells(const float *values, const float *cell_value,
+                                                                       const int *cell_index, int cells, int32_t *index) {
+    __shared__ float pv[kArgmaxThreads / JL_WAVE];
+    __shared__ int pi[kArgmaxThreads / JL_WAVE];
+    const int tid = threadIdx.x;
+    float best = -INFINITY;
+    int at = INT_MAX;
+    for (int i = tid; i < cells; i += kArgmaxThreads) keep_better(best, at, cell_value[i], cell_index[i]);
+    fold_waves(best, at, pv, pi, tid, kArgmaxThreads / JL_WAVE);
+    if (tid == 0) {
+        if (at == INT_MAX || values[0] != values[0]) at = 0;   // as in jl_argmax_fold
+        index[0] = at;
+    }
+}
+
 // One lane per activation, 32 lanes per block: inverse = 127 / max|x| (0 for a block of zeros),
 // q = (int)(x * inverse +- 0.5) clamped to +-127, scale = max|x| / 127, sum = sum of q.  With RMS
 // the lane first computes its element of the normalised vector, rms_w[i] * (rms_scale * x[i]) with
@@ -186,6 +204,24 @@ static int argmax_launches(jl_context *ctx, const float *values, int64_t n, int3
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
     static_assert(sizeof(ArgmaxCells) <= JL_CONTEXT_SCRATCH_BYTES, "argmax cells exceed the context scratch");
     return argmax_launches(ctx, values, n, index, (ArgmaxCells *)ctx->scratch);
+}
+
+int jl_launch_gemv_argmax(jl_context *ctx, const jl_weight *w, const float *x, const jl_rms *rms, float *out,
+                          int32_t *index) {
+    float *cell_value = (float *)ctx->scratch;
+    jl_best_cells cells{cell_value, (int *)(cell_value + kProjectionCells), kProjectionCells};
+    int st = jl_launch_gemv(ctx, &w, 1, &out, nullptr, x, JL_STORE, rms, nullptr, &cells);
+    if (st == JL_NO_CELLS_FORM) {
+        // a shape or type whose kernel keeps no cells: the projection, then the scan over its output
+        st = jl_launch_gemv(ctx, &w, 1, &out, nullptr, x, JL_STORE, rms);
+        if (st != JL_OK) return st;
+        return jl_launch_argmax(ctx, out, w->rows, index);
+    }
+    if (st != JL_OK) return st;
+    hipLaunchKernelGGL(jl_argmax_fold_cells, dim3(1), dim3(kArgmaxThreads), 0, ctx->stream, out, cells.value, cells.index,
+                       cells.count, index);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
 }
 
 // ---- jl_argmax_static: the same two launches with the cells in a device array of the library ----

@@ -202,6 +202,21 @@ class QuantizedProjections:
         L.check(self._lib.jl_argmax(self.context.handle, logits.ptr, n, token.ptr))
 
 
+    def matvecArgmax(self, x: FloatArray, logits: FloatArray, w: TornadoTensor, n: int, d: int,
+                     token: DeviceBuffer, rmsWeights: FloatArray | None = None,
+                     rmsScale: FloatArray | None = None, eps: float = 0.0) -> None:
+        """The tail of a greedy decode step in one call: ``logits = w . x`` -- with ``rmsWeights`` set,
+        of the RMS-normalised ``x`` as in ``rmsMatvec`` -- and ``token[0]`` = ``argmax(logits)``
+        (the vocabulary projection followed by "argmax_sample", LogitsQ8_0Layer.java:92-110).  Bit for
+        bit what ``matvec`` / ``rmsMatvec`` followed by ``argmax`` leave; where the projection kernel
+        can keep its workgroups' best logits, one launch fewer."""
+        _check_shape(w, n, d)
+        L.check(self._lib.jl_gemv_argmax(self.context.handle, w.handle, x.ptr,
+                                         rmsWeights.ptr if rmsWeights is not None else None,
+                                         rmsScale.ptr if rmsScale is not None else None, float(eps),
+                                         logits.ptr, token.ptr))
+
+
 class QuantizedBatchProjections:
     """Projections of ``batchSize`` activation rows at once (batched decode, batched prefill)."""
 

@@ -582,6 +582,95 @@ def test_rms_vocabulary_projection_and_argmax(ctx, t, d, n):
     assert rel_err(logits.get(), ref, magnitude(t, raw, xn, d, n)) < 2e-5
 
 
+# (type, rows, columns): the first four take the projection kernel that keeps its workgroups' best
+# logits; then a row count that is not whole tiles, rows shorter than their padded slices, rows in
+# several waves, a type with no such form -- those run the projection and the scan, inside the call
+PROJECTION_ARGMAX = [(O.Q8_0, 32000, 2048), (O.Q4_0, 20008, 4096), (O.Q4_K, 16384, 2048), (O.Q4_K, 4100, 4096),
+                     (O.Q8_0, 1001, 2048), (O.Q8_0, 9000, 3072), (O.Q4_0, 3000, 8192), (O.Q6_K, 5000, 2048)]
+
+
+@pytest.mark.parametrize("t,d,n", PROJECTION_ARGMAX)
+@pytest.mark.parametrize("rms", ["plain", "scale given", "scale in kernel"])
+def test_projection_and_argmax_in_one_call(ctx, t, d, n, rms):
+    """matvecArgmax against the calls it stands for -- matvec / rmsMatvec, then argmax: the same
+    logits bit for bit, the same token, and that token the host's FloatTensor.argmax of the
+    logits.  The weight's best row is repeated further down (other tiles, other workgroups), so the
+    first of equal maxima has to win across lanes, waves and workgroups."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("projection + argmax", t, d, n, rms)
+    if rms != "plain" and t == O.Q6_K:
+        pytest.skip("the RMS-folding projections take the three main types only")
+    raw = synthetic.weight(t, d, n, seed=671).reshape(d, -1).copy()
+    x = synthetic.activations(n, seed=672)
+    rw = (1.0 + 0.25 * synthetic.activations(n, seed=673)).astype(np.float32)
+    proj = QuantizedProjections(ctx, TornadoWorkspace())
+    dx, drw, scale = ctx.from_numpy(x), ctx.from_numpy(rw), ctx.float_array(1, fill=POISON)
+    proj.rmsScale(dx, n, 1e-5, scale)
+    token = ctx.raw_buffer(8)
+
+    def two_calls(w, logits):
+        if rms == "plain":
+            proj.floatMatvec(dx, logits, w, n, d)
+        else:
+            proj.rmsMatvec(dx, drw, scale if rms == "scale given" else None, logits, w, n, d, eps=1e-5)
+        proj.argmax(logits, d, token)
+        ctx.sync()
+        return logits.get(), int(token.download(np.int32, 1)[0])
+
+    def one_call(w, logits):
+        token.upload(np.array([-7, -7], dtype=np.int32))
+        proj.matvecArgmax(dx, logits, w, n, d, token, rmsWeights=None if rms == "plain" else drw,
+                          rmsScale=scale if rms == "scale given" else None, eps=1e-5)
+        ctx.sync()
+        return logits.get(), int(token.download(np.int32, 1)[0])
+
+    first, _ = two_calls(upload(ctx, t, raw.reshape(-1), d, n), ctx.float_array(d, fill=POISON))
+    best = O.argmax(first)
+    rng = np.random.default_rng(d + n)
+    for at in sorted(set(int(i) for i in rng.integers(0, d, 6)) | {d - 1}):
+        raw[at] = raw[best]
+    w = upload(ctx, t, raw.reshape(-1), d, n)
+    want, want_token = two_calls(w, ctx.float_array(d, fill=POISON))
+    got, got_token = one_call(w, ctx.float_array(d, fill=POISON))
+    assert bits_equal(got, want)
+    assert got_token == want_token == O.argmax(want)
+    assert np.count_nonzero(want == want[want_token]) >= 2 and want_token == int(np.flatnonzero(want == want.max())[0])
+
+
+@pytest.mark.parametrize("t,d,n", [(O.Q8_0, 32000, 2048), (O.Q4_K, 4100, 4096)])
+def test_projection_argmax_when_no_logit_is_a_number_or_all_are_equal(ctx, t, d, n):
+    """FloatTensor.argmax's corners through the one-call form: an activation vector of zeros (every
+    logit 0: token 0), one with a NaN (every logit NaN: token 0), and a second call on the same
+    context with a smaller weight, which must not see the first call's candidates."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("projection + argmax corners", t, d, n)
+    raw = synthetic.weight(t, d, n, seed=681)
+    w = upload(ctx, t, raw, d, n)
+    proj = QuantizedProjections(ctx, TornadoWorkspace())
+    token = ctx.raw_buffer(4)
+    logits = ctx.float_array(d, fill=POISON)
+    x = synthetic.activations(n, seed=682)
+    nan = x.copy()
+    nan[n // 3] = np.nan
+    for v in (np.zeros(n, dtype=np.float32), nan):
+        token.upload(np.array([-7], dtype=np.int32))
+        proj.matvecArgmax(ctx.from_numpy(v), logits, w, n, d, token)
+        ctx.sync()
+        assert int(token.download(np.int32, 1)[0]) == O.argmax(logits.get()) == 0
+    proj.matvecArgmax(ctx.from_numpy(x), logits, w, n, d, token)
+    ctx.sync()
+    assert int(token.download(np.int32, 1)[0]) == O.argmax(logits.get())
+    small = 264
+    ws = upload(ctx, t, raw[: small * (raw.size // d)], small, n)
+    few = ctx.float_array(small, fill=POISON)
+    proj.matvecArgmax(ctx.from_numpy(x), few, ws, n, small, token)
+    ctx.sync()
+    assert bits_equal(few.get(), logits.get()[:small])
+    assert int(token.download(np.int32, 1)[0]) == O.argmax(few.get())
+
+
 @pytest.mark.parametrize("n", [1, 5, 1023, 4097, 128256])
 def test_argmax_ties_and_edges(ctx, n):
     from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
