@@ -9,8 +9,8 @@
 //
 //   jl_decode_to_f16   raw blocks -> [virtual rows x K] fp16, the host decode rounded once to fp16
 //                      (bit for bit what the fused kernel multiplies with); one launch per call
-//   jl_gemm_hh<BM, BN> C = A16 . W16^T on v_mfma_f32_16x16x32_f16, BM x BN tiles (256 x 256, 256 x 128,
-//                      128 x 128) in steps of 64 columns; eight waves that each bring in their
+//   jl_gemm_hh<BM, BN> C = A16 . W16^T on v_mfma_f32_16x16x32_f16, BM x BN tiles (256 x 256, 256 x 192,
+//                      256 x 128, 128 x 192, 128 x 128) in steps of 64 columns; eight waves that each bring in their
 //                      share of both operands by LDS-DMA, the two waves of a SIMD half a step apart
 #include "jl_device.h"
 #include "jl_internal.h"
@@ -257,6 +257,8 @@ template <int N>
 __device__ __forceinline__ void lds_settle(half8 (&f)[N]) {
     if constexpr (N == 8)
         asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]));
+    else if constexpr (N == 6)
+        asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]));
     else if constexpr (N == 4)
         asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
     else
@@ -271,7 +273,9 @@ __device__ __forceinline__ void lds_settle(half8 (&f)[N]) {
 // barrier and have the whole step to land); 256 x 128: three stages of 48 KB; 128 x 128: four of
 // 32 KB -- the tile of calls too narrow to give every compute unit a larger one, which would
 // otherwise have to cut K across workgroups and pay for a fold.
-template <int BM, int BN> constexpr int hh_stages() { return BM + BN == 512 ? 2 : BM + BN == 384 ? 3 : 4; }
+// (192-column tiles, for projections whose width is a multiple of 192 and not of 256 -- a fused
+// q|k|v of 3072 or 6144 columns: 256 x 192 in two stages of 56 KB, 128 x 192 in three of 40 KB)
+template <int BM, int BN> constexpr int hh_stages() { return BM + BN >= 448 ? 2 : BM + BN >= 320 ? 3 : 4; }
 
 template <int BM, int BN>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -280,7 +284,7 @@ jl_gemm_hh(DenseParams p) {
     constexpr int DBM = BM;
     constexpr int WM = BN == 256 ? 2 : 4;     // waves along M
     constexpr int WN = 8 / WM;
-    constexpr int TM = DBM / WM, TN = BN / WN;   // wave tile: 128 x 64, 64 x 64 or 32 x 64
+    constexpr int TM = DBM / WM, TN = BN / WN;   // wave tile: 128 x 64, 64 x 64, 32 x 64; 64 x 96, 32 x 96
     constexpr int MB = TM / 16, NB = TN / 16;
     constexpr int STAGE = (DBM + BN) * 128;
     constexpr int NS = hh_stages<BM, BN>();
@@ -297,8 +301,8 @@ jl_gemm_hh(DenseParams p) {
     // the smaller tiles (deeper rings, shorter steps) lose more than they gain and go without.
     constexpr int PFW = NS == 2 ? 1 : 0;
     constexpr int PFD = 2;
-    static_assert(NB == 4, "four column blocks per wave");
-    static_assert(BM == 256 || (BM == 128 && BN == 128), "row tiles: 256, or 128 with 128 columns");
+    static_assert(NB == 4 || NB == 6, "four or six column blocks per wave");
+    static_assert(BM == 256 || (BM == 128 && BN <= 192), "row tiles: 256, or 128 with 128 or 192 columns");
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -371,7 +375,7 @@ jl_gemm_hh(DenseParams p) {
         // after stage s's last load (past the last step: its own line again, so that the count of
         // loads per stage does not change)
         // (the GM workgroups that share this weight tile touch a GM-th of its rows each)
-        const uint32_t pf_off = (uint32_t)((mt - group * GM) * (BN / GM) + (lane & (BN / GM - 1))) * (uint32_t)(p.k * 2);
+        const uint32_t pf_off = (uint32_t)((mt - group * GM) * (BN / GM) + lane % (BN / GM)) * (uint32_t)(p.k * 2);
         auto prefetch = [&](int s) {
             if (wave < PFW) {
                 const int ps = s + PFD < ksteps ? s + PFD : ksteps - 1;
@@ -456,9 +460,11 @@ jl_gemm_hh(DenseParams p) {
                 read_frags(lds0 + (s % NS) * STAGE);
                 // LDS reads return in order: the first k-block's MB + NB fragments are back when
                 // that many of the second's are still outstanding
-                if constexpr (MB == 8) asm volatile("s_waitcnt lgkmcnt(12)" ::: "memory");
-                else if constexpr (MB == 4) asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+                if constexpr (MB + NB == 12) asm volatile("s_waitcnt lgkmcnt(12)" ::: "memory");
+                else if constexpr (MB + NB == 10) asm volatile("s_waitcnt lgkmcnt(10)" ::: "memory");
+                else if constexpr (MB + NB == 8) asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
                 else asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory");
+                static_assert(MB + NB == 12 || MB + NB == 10 || MB + NB == 8 || MB + NB == 6, "fragments per k-block");
                 lds_settle(fa[0]);
                 lds_settle(fb[0]);
                 mfma_block(0, more, s + AHEAD);
@@ -595,7 +601,8 @@ int launch_decode(jl_context *ctx, const DecodeParams &d, int activation_rows) {
 
 // Column tile the dense path would use for a call (and in *row_tile the row tile), 0 when the call
 // is not one for it: it takes 512 rows or more and enough work items to give most compute units
-// one.  The largest tile that does so wins: 256 x 256, 256 x 128, then 128 x 128; narrow
+// one.  The largest tile that does so wins: 256 x 256, 256 x 128, then 128 x 128 (a width of whole
+// 192-column tiles can also get 256 x 192 or 128 x 192, returned as 192); narrow
 // projections on few rows get there by cutting K into 2, 4 or 8 runs of at least four steps as well
 // (plain store / residual only); what is still too small keeps the decode-in-the-loop kernel.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits,
@@ -604,9 +611,30 @@ int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, in
     *row_tile = 256;
     if (rows < 512 || k % 64 != 0) return 0;
     const int mtiles = (rows + 255) / 256;
-    // 256-wide tiles when they still give every compute unit work, else 128-wide ones
-    if ((int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units) return 256;
+    const bool wide_fills = (int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units;
     const int64_t items = (int64_t)mtiles * ((out_cols_virtual + 127) / 128);
+    // A width of whole 192-column tiles (a fused q|k|v of 3072 or 6144 columns) has two more tiles
+    // to choose from.  Each candidate is priced as rounds of work items over the compute units x
+    // outputs per item x what an output costs in that tile (measured, K = 2048: 256 x 256 runs at
+    // ~1180 TFLOP/s when every compute unit has an item, 256 x 192 at ~980, 256 x 128 at ~960,
+    // 128 x 192 at ~790, 128 x 128 at ~650), against the choice the rules below would make.
+    if (epilogue != JL_SWIGLU && out_cols_virtual % 192 == 0) {
+        auto cost = [&](int bm, int bn, int per_output) {
+            const int64_t n = (int64_t)((rows + bm - 1) / bm) * ((out_cols_virtual + bn - 1) / bn);
+            return (n + compute_units - 1) / compute_units * bm * bn * per_output;
+        };
+        const int64_t other = wide_fills                                    ? cost(256, 256, 85)
+                              : items * 10 >= (int64_t)compute_units * 7 ? cost(256, 128, 105)
+                                                                          : cost(128, 128, 150);
+        const int64_t wide = cost(256, 192, 100), tall = cost(128, 192, 125);
+        if (wide <= tall && wide < other) return 192;
+        if (tall < other) {
+            *row_tile = 128;
+            return 192;
+        }
+    }
+    // 256-wide tiles when they still give every compute unit work, else 128-wide ones
+    if (wide_fills) return 256;
     if (items * 10 >= (int64_t)compute_units * 7) return 128;
     const int64_t small = (int64_t)((rows + 127) / 128) * ((out_cols_virtual + 127) / 128);
     for (int s = 1; s <= 8; s *= 2) {
@@ -702,10 +730,13 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
     p.mtiles = (rows + bm - 1) / bm;
     p.splits = splits;
     p.partial = planes;
-    if (!(bm == 256 || (bm == 128 && bn == 128)) || (bn != 128 && bn != 256))
+    if (!(bm == 256 || (bm == 128 && bn != 256)) || (bn != 128 && bn != 192 && bn != 256) ||
+        (bn == 192 && (swiglu || splits != 1 || n_total % 192 != 0)))
         return jl_fail(JL_ERR_INVALID, "jl_gemm: no %d x %d tile", bm, bn);
-    const int st = bn == 256 ? launch_dense<256, 256>(ctx, p)
-                 : bm == 256 ? launch_dense<256, 128>(ctx, p) : launch_dense<128, 128>(ctx, p);
+    const int st = bn == 256   ? launch_dense<256, 256>(ctx, p)
+                   : bn == 192 ? (bm == 256 ? launch_dense<256, 192>(ctx, p) : launch_dense<128, 192>(ctx, p))
+                   : bm == 256 ? launch_dense<256, 128>(ctx, p)
+                               : launch_dense<128, 128>(ctx, p);
     if (st != JL_OK || splits == 1) return st;
     return jl_launch_gemm_reduce(ctx, planes, row_scale, C, rows, n_total, ntiles,
                                  (int64_t)p.mtiles * bm * ntiles * 128, splits, ldo, col_offset, epilogue);

@@ -281,6 +281,9 @@ def test_many_row_prefill_qkv_and_gate_up(ctx):
     (O.Q4_K, 3000, 1024, 600, False),    # 128 x 128 tiles, K cut in two, ragged rows
     (O.Q8_0, 1500, 2048, 512, True),     # 128 x 128 tiles, K cut in four, last tile 92 columns
     (O.Q4_0, 700, 2048, 520, False),     # 128 x 128 tiles, K cut in eight runs of four steps, ragged both ways
+    (O.Q8_0, 3072, 256, 2000, False),    # 128 x 192 tiles (16 x 16 of them), ragged rows
+    (O.Q4_K, 6144, 256, 2000, True),     # 256 x 192 tiles (8 x 32), ragged rows, residual
+    (O.Q4_0, 3072, 512, 4096, True),     # 256 x 192 tiles (16 x 16), whole rows
 ])
 def test_two_pass_prefill_tiles_and_edges(ctx, t, d, n, T, residual):
     """Shapes with enough tiles for the decode-once path on 256 compute units, one per tiling it

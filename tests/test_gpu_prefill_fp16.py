@@ -69,7 +69,10 @@ def test_fp16_activations_give_the_fp32_entry_points_bits(ctx, t, d, n, batch, r
     assert rel_err(got16[:rows], ref, mag) < F16_BOUND
 
 
-@pytest.mark.parametrize("t,dq,dkv,n,T,resident", [(O.Q8_0, 2048, 512, 2048, 512, True), (O.Q4_K, 256, 128, 1024, 70, False)])
+# (the last two: 3072 and 6144 columns on 128 x 192 and 256 x 192 tiles, whose column tiles straddle
+# the three weights' boundaries; ragged rows in the second)
+@pytest.mark.parametrize("t,dq,dkv,n,T,resident", [(O.Q8_0, 2048, 512, 2048, 512, True), (O.Q4_K, 256, 128, 1024, 70, False),
+                                                   (O.Q8_0, 2048, 512, 256, 2048, True), (O.Q4_0, 4096, 1024, 256, 2000, False)])
 def test_fp16_activations_fused_qkv(ctx, t, dq, dkv, n, T, resident):
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
