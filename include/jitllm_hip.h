@@ -50,8 +50,8 @@ typedef enum jl_status {
  * of "Q4_K_M" files are Q6_K, "Q5_K_M" files are Q5_K with Q6_K), and the types quantisers mix
  * into other files -- Q4_1 (20 B / 32, GGMLType.java:8), Q5_0 (22 B / 32, :11) and IQ4_XS
  * (136 B / 256, :39-41) -- have
- * jl_dequant_f32, jl_gemv, jl_gemv_gate_up and jl_gemm -- the latter always by decoding the weights
- * to fp16 into the workspace first, whatever the row count.  (Of these the reference fuses gate/up
+ * jl_dequant_f32, jl_gemv, jl_gemv_gate_up and jl_gemm -- the latter on the weight-streaming kernel
+ * at up to 64 rows and by decoding the weights to fp16 into the workspace first above that.  (Of these the reference fuses gate/up
  * for Q5_K only, QuantizedProjections.java:386-393; the one-launch form is there for all five.)  The
  * fused q|k|v, RMS-folding and packed-activation single-token entry points return
  * JL_ERR_UNSUPPORTED for them; a caller that gets JL_ERR_UNSUPPORTED runs the unfused steps. */
@@ -352,7 +352,10 @@ int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count
  *        first rescales every fp32 row by a power of two; there is nothing to rescale here, so a
  *        row whose products leave fp16's range is the producer's to avoid, as in the reference).
  *        Calls that read whole 256-row tiles take X in place when `batch` covers the last tile,
- *        otherwise the active rows are copied into the workspace first.
+ *        otherwise the active rows are copied into the workspace first.  Calls of at most 64 active
+ *        rows -- a short prompt, the tail of a chunked one -- run jl_gemm's weight-streaming kernel,
+ *        which reads X where it lies and brings every row into range by a power of two as it does
+ *        for fp32 rows (exact, undone on the results).
  *   C    fp32 as in jl_gemm; with c_fp16 != 0 -- JL_SWIGLU only, the feed-forward hidden vector
  *        batchedFFNSwiGLUFP16Packed writes -- binary16, `ldo` and `col_offset` counting fp16 values
  *        and every result rounded once from its fp32 value.

@@ -163,10 +163,20 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
                    int epilogue, int math, void *workspace, size_t workspace_bytes,
                    const jl_resident *resident, const jl_half_io *half = nullptr);
 // Batched decode (at most 64 rows): the weight-streaming kernel.  `taken` says whether the shape
-// was one it handles; when not, nothing was launched and the tiled GEMM must run instead.
+// was one it handles; when not, nothing was launched and the tiled GEMM must run instead.  `X16`
+// set: the activations as binary16 (X is then ignored); `c_f16` (JL_SWIGLU): C holds binary16.
 int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
-                          float *C, int rows, int64_t ldo, int64_t col_offset, int epilogue,
-                          float *planes, size_t plane_bytes, bool *taken);
+                          const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
+                          int epilogue, float *planes, size_t plane_bytes, bool *taken);
+// Activation rows one of its workgroups multiplies: 16 or 32; calls of more rows run as two row blocks.
+int jl_skinny_padded_rows(int rows);
+// (its two halves, one translation unit each: fp32 activations, binary16 activations)
+int jl_launch_gemm_skinny_x32(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
+                              const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
+                              int epilogue, float *planes, size_t plane_bytes, bool *taken);
+int jl_launch_gemm_skinny_x16(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
+                              const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
+                              int epilogue, float *planes, size_t plane_bytes, bool *taken);
 // Many-row prefill: weights decoded to fp16 once per call into `copy`, then a plain fp16 GEMM.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits,
                          int *row_tile);

@@ -42,6 +42,9 @@ CASES = [
     (O.Q8_0, 300, 256, 64, 40, True),
     (O.Q8_0, 300, 256, 96, 70, True),
     (O.Q6_K, 640, 512, 96, 90, False),
+    (O.Q4_K, 4100, 4096, 32, 32, True),      # up to 64 rows: the weight-streaming kernel, rows cut across workgroups
+    (O.Q4_0, 1000, 2048, 64, 50, False),
+    (O.IQ4_XS, 520, 1024, 16, 16, True),
 ]
 
 
@@ -61,8 +64,7 @@ def test_fp16_activations_give_the_fp32_entry_points_bits(ctx, t, d, n, batch, r
     p.projection(ctx.half_from_numpy(X16), b, w, n, d, residual, activeRows=rows)
     ctx.sync()
     got32, got16 = a.get().reshape(batch, d), b.get().reshape(batch, d)
-    if rows > 64:       # up to 64 rows the fp32 entry point reads X itself, in another kernel
-        assert np.array_equal(got16.view(np.uint32), got32.view(np.uint32))
+    assert np.array_equal(got16.view(np.uint32), got32.view(np.uint32))
     assert np.array_equal(got16[rows:], start[rows:])
     ref = O.matmul_batch(t, raw, X32[:rows], d, n).astype(np.float64) + (start[:rows] if residual else 0.0)
     mag = magnitude(t, raw, X32[:rows], d, n) + (np.abs(start[:rows]) * 1e-6 if residual else 0.0)
@@ -97,13 +99,15 @@ def test_fp16_activations_fused_qkv(ctx, t, dq, dkv, n, T, resident):
 
 
 @pytest.mark.parametrize("t,ffn,n,batch,rows", [(O.Q8_0, 8192, 2048, 512, 512), (O.Q4_K, 1002, 512, 768, 700),
-                                                (O.Q4_0, 1002, 1024, 96, 96), (O.Q5_K, 520, 256, 96, 70)])
+                                                (O.Q4_0, 1002, 1024, 96, 96), (O.Q5_K, 520, 256, 96, 70),
+                                                (O.Q4_K, 1002, 4096, 40, 33), (O.Q8_0, 520, 2048, 64, 64),
+                                                (O.Q6_K, 300, 2048, 8, 5)])
 def test_fp16_hidden_vector_is_the_fp32_one_rounded_once(ctx, t, ffn, n, batch, rows):
     """gate/up + SwiGLU with the result stored as fp16 (batchedFFNSwiGLUFP16Packed): every value is
     the fp32 result of the same call rounded to nearest even, rows past the active ones untouched;
-    the fp32 result itself equals the fp32 entry point's and meets the oracle.  (More than 64 active
-    rows throughout: at up to 64 rows fp32 activations take the weight-streaming kernel, whose
-    arithmetic is its own.)"""
+    the fp32 result itself equals the fp32 entry point's and meets the oracle.  (The last three:
+    at most 64 rows, where both kinds of activations take the weight-streaming kernel -- a short
+    prompt's prefill.)"""
     from jitllm_amd import synthetic
     from jitllm_amd.projections import QuantizedBatchProjections
     say("xf16 gate/up", t, ffn, n, batch, rows)
