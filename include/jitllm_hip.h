@@ -51,7 +51,8 @@ typedef enum jl_status {
  * into other files -- Q4_1 (20 B / 32, GGMLType.java:8), Q5_0 (22 B / 32, :11) and IQ4_XS
  * (136 B / 256, :39-41) -- have
  * jl_dequant_f32, jl_gemv, jl_gemv_gate_up and jl_gemm -- the latter on the weight-streaming kernel
- * at up to 64 rows and by decoding the weights to fp16 into the workspace first above that.  (Of these the reference fuses gate/up
+ * at up to 64 rows -- and up to 511 where that is the faster way -- and by decoding the weights to fp16 into the workspace
+ * first above that.  (Of these the reference fuses gate/up
  * for Q5_K only, QuantizedProjections.java:386-393; the one-launch form is there for all five.)  The
  * fused q|k|v, RMS-folding and packed-activation single-token entry points return
  * JL_ERR_UNSUPPORTED for them; a caller that gets JL_ERR_UNSUPPORTED runs the unfused steps. */
@@ -290,7 +291,8 @@ int jl_gemv_gate_up_q8(jl_context *ctx, const jl_weight *w1, const jl_weight *w3
  * more, the reference's dequantize-then-gemmMMA prefill shape -- an fp16 copy of the call's
  * weights, decoded afresh by every such call and dead after it.  A smaller workspace that still
  * holds the first two is accepted; such calls simply keep to one pass and do not cut K.  Calls of
- * at most 64 rows read X directly and use only the partial sums.
+ * at most 64 rows -- and calls of up to 511 rows whose weights are small enough that streaming
+ * them once per 32 rows beats the tiled kernels -- read X directly and use only the partial sums.
  */
 size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols, int math);
 

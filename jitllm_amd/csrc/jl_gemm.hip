@@ -885,8 +885,9 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const size_t plane_bytes = workspace_bytes > head ? workspace_bytes - head : 0;
 
 
-    if (rows <= 64) {
-        // batched decode of up to 64 rows: the weight-streaming kernel reads X itself, fp32 or fp16
+    if (rows < 512) {
+        // batched decode of up to 64 rows, and calls of up to 511 where it is the faster one: the
+        // weight-streaming kernel reads X itself, fp32 or fp16
         bool taken = false;
         int st = jl_launch_gemm_skinny(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, epilogue,
                                        planes, plane_bytes, &taken);

@@ -1103,6 +1103,19 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
     }
 }
 
+// Workgroups per span: one workgroup per compute unit and span (the ring takes most of the LDS),
+// fewer for less work.  The row blocks of a call share the chip: workgroup (x, y) runs beside
+// (x, y + 1), and with a grid width that is a multiple of 8 both land on the same XCD, whose L2
+// then serves the later readers of every tile -- unless rounding down to that multiple would idle
+// more than a fifth of the chip (Q4_K down projection of 12288 columns at 96 rows: 8 instead of 14
+// workgroups per span took 46 us instead of 34).
+int workgroups_per_span(int compute_units, int row_blocks, int Z, int groups) {
+    int per_span = compute_units / row_blocks / Z;
+    if (row_blocks > 1 && per_span / 8 * 8 * 5 >= per_span * 4) per_span = per_span / 8 * 8;
+    if (per_span < 1) per_span = 1;
+    return per_span > groups ? groups : per_span;
+}
+
 template <int TYPE, int NBB, bool DUAL, int ZIN, bool HALF, bool XH>
 int launch_of(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int groups) {
     auto fn = jl_gemm_skinny<TYPE, NBB, DUAL, ZIN, HALF, XH>;
@@ -1111,14 +1124,7 @@ int launch_of(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int 
         JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         configured[ctx->device] = true;
     }
-    // one workgroup per compute unit and span (the ring takes most of the LDS), fewer for less work
-    // The row blocks of a call share the chip: workgroup (x, y) runs beside (x, y + 1), and with a
-    // grid width that is a multiple of 8 both land on the same XCD, whose L2 then serves the second
-    // reader of every tile.
-    int per_span = ctx->compute_units / p.row_blocks / p.Z;
-    if (p.row_blocks > 1) per_span = per_span / 8 * 8;
-    if (per_span < 1) per_span = 1;
-    if (per_span > groups) per_span = groups;
+    const int per_span = workgroups_per_span(ctx->compute_units, p.row_blocks, p.Z, groups);
     if (p.Z > 1 && per_span * p.row_blocks > JL_CONTEXT_ARRIVALS) {
         return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: %d workgroup sets exceed the context's %d arrival counters",
                        per_span * p.row_blocks, JL_CONTEXT_ARRIVALS);
@@ -1158,9 +1164,9 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     const bool dual = epilogue == JL_SWIGLU;
-    if (rows > 64 || k % 256 != 0 || count > kMaxSeg) return JL_OK;
+    if (rows >= 512 || k % 256 != 0 || count > kMaxSeg) return JL_OK;
     const int S = k / 64;
-    const int row_blocks = rows > 32 ? 2 : 1;
+    const int row_blocks = (rows + 31) / 32;
     const int nbb = jl_skinny_padded_rows(rows) / 16;
     const int quad = quad_bytes(type);
     if (quad == 0) return JL_OK;
@@ -1175,6 +1181,28 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
     // 4096 columns); more rows leave no registers for a second set of activation fragments
     const int zin = (nbb == 1 && (S / Ss) % 2 == 0) ? 2 : 1;
     const int Z = S / Ss / zin;
+
+    if (rows > 64) {
+        // 65 .. 511 rows run as three to sixteen row blocks, each streaming the whole weight over its
+        // share of the chip: what this costs grows with blocks x weights, and it is taken when that
+        // is less than what the tiled GEMMs cost.  Microseconds, fitted to graph replays of the calls
+        // of a Llama-3.2-1B layer (Q8_0) and of 8B-shaped layers (Q4_K, Q6_K, Q5_K) at 65 .. 384 rows:
+        //   here                    10 + 0.155 x row blocks x million weights / share of the chip in use
+        //   decode in the loop      22 + (Q8_0: 0.30, 4-bit: 0.37) x 128-row tiles x million weights
+        //   decode once (the types with no decode-in-the-loop kernel)   30 + 2.8 x million weights
+        double millions = 0.0;
+        int all_groups = 0;
+        for (int i = 0; i < count; i++) millions += (double)weights[i]->rows * k * 1e-6;
+        for (int i = 0; i < (dual ? 1 : count); i++) all_groups += ((int)weights[i]->rows + (dual ? 8 : 16) - 1) / (dual ? 8 : 16);
+        const int per_span = workgroups_per_span(ctx->compute_units, row_blocks, Z, all_groups);
+        double share = (double)per_span * Z * row_blocks / ctx->compute_units;
+        if (share > 1.0) share = 1.0;
+        const double here = 10.0 + 0.155 * row_blocks * millions / share;
+        const double tiled = jl_has_fused_kernels(type)
+                                 ? 22.0 + (type == JL_Q8_0 ? 0.30 : 0.37) * ((rows + 127) / 128) * millions
+                                 : 30.0 + 2.8 * millions;
+        if (here >= tiled) return JL_OK;
+    }
 
     SkinnyParams p{};
     p.nseg = dual ? 1 : count;
