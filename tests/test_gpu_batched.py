@@ -435,6 +435,91 @@ def test_rows_cut_across_workgroups_are_folded_afresh_on_every_call(ctx, t, d, n
     w.free()
 
 
+# (type, weight rows, row length, batch, active rows, residual): 65 .. 511 rows on the
+# weight-streaming kernel as 3 .. 16 row blocks -- a last block of one row, partial batches, rows cut
+# across workgroups (more than 2048 columns) with up to eight blocks' partial sums in the workspace,
+# the types whose other way decodes the whole weight first
+MID_ROWS = [
+    (O.Q8_0, 520, 2048, 65, 65, False),
+    (O.Q8_0, 520, 2048, 160, 131, True),
+    (O.Q4_K, 1000, 4096, 96, 96, True),
+    (O.Q4_K, 264, 8192, 250, 250, False),
+    (O.Q4_0, 300, 6144, 129, 100, False),
+    (O.Q4_0, 2048, 256, 511, 511, True),
+    (O.Q6_K, 300, 2048, 200, 170, False),
+    (O.Q5_K, 520, 4096, 384, 384, True),
+    (O.IQ4_XS, 264, 1024, 97, 97, False),
+]
+
+
+@pytest.mark.parametrize("t,d,n,batch,rows,residual", MID_ROWS)
+def test_mid_row_counts_stream_their_weights(ctx, t, d, n, batch, rows, residual):
+    """Calls between batched decode and prefill against the oracle; rows past the active ones and
+    whatever lies behind the output keep their contents, and a second call gives the same bits."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("mid row counts", t, d, n, batch, rows, residual)
+    raw = synthetic.weight(t, d, n, seed=9950 + d)
+    X = synthetic.activations((batch, n), seed=9951 + rows)
+    ref = O.matmul_batch(t, raw, X[:rows], d, n)
+    w = ctx.load_weight(t, raw, d, n)
+    proj = QuantizedBatchProjections(ctx, batch, n, d)
+    outs = [ctx.float_array(batch * d + 64, fill=UNTOUCHED) for _ in range(2)]
+    for out in outs:
+        proj.projection(ctx.from_numpy(X), out, w, n, d, residual, activeRows=rows)
+    ctx.sync()
+    flat = outs[0].get()
+    assert np.all(flat[rows * d:] == UNTOUCHED)
+    assert np.array_equal(flat.view(np.uint32), outs[1].get().view(np.uint32))
+    got = flat[:rows * d].reshape(rows, d)
+    want = ref.astype(np.float64) + (float(UNTOUCHED) if residual else 0.0)
+    slack = abs(np.spacing(np.float32(UNTOUCHED))) / 2 if residual else 0.0
+    excess = np.abs(got.astype(np.float64) - want) - slack
+    assert np.all(excess <= F16_BOUND * magnitude(t, raw, X[:rows], d, n)), float(excess.max())
+    w.free()
+
+
+def test_mid_row_counts_gate_up_and_side_by_side_weights(ctx):
+    """The other two call forms at 65 .. 511 rows: q|k|v of unequal widths side by side (five row
+    blocks) and gate/up + SwiGLU (four row blocks, the last one partial), fp32 and binary16
+    activations giving the same bits."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("mid row counts, qkv / gate_up")
+    t, n, T = O.Q8_0, 2048, 150
+    dims = (1024, 256, 264)
+    raws = [synthetic.weight(t, d, n, seed=9960 + i) for i, d in enumerate(dims)]
+    X16 = synthetic.activations((T, n), seed=9963).astype(np.float16)
+    X = X16.astype(np.float32)
+    ws = [ctx.load_weight(t, r, d, n) for r, d in zip(raws, dims)]
+    ld = sum(dims)
+    a, b = ctx.float_array(T * ld, fill=UNTOUCHED), ctx.float_array(T * ld, fill=UNTOUCHED)
+    p = QuantizedBatchProjections(ctx, T, n, ld)
+    p.fusedQKV(ctx.from_numpy(X), a, *ws)
+    p.fusedQKV(ctx.half_from_numpy(X16), b, *ws)
+    ctx.sync()
+    got = a.get().reshape(T, ld)
+    assert np.array_equal(got.view(np.uint32), b.get().reshape(T, ld).view(np.uint32))
+    col = 0
+    for raw, d in zip(raws, dims):
+        assert rel_err(got[:, col:col + d], O.matmul_batch(t, raw, X, d, n), magnitude(t, raw, X, d, n)) < F16_BOUND
+        col += d
+    t, d, n, T = O.Q4_K, 1000, 2048, 100
+    r1, r3 = synthetic.weight(t, d, n, seed=9970), synthetic.weight(t, d, n, seed=9971)
+    X = synthetic.activations((T, n), seed=9972)
+    g, u = O.matmul_batch(t, r1, X, d, n), O.matmul_batch(t, r3, X, d, n)
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(T, d)
+    hb = ctx.float_array(T * d + 64, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, T, n, 2 * d).gateUp(ctx.from_numpy(X), hb, ctx.load_weight(t, r1, d, n),
+                                                ctx.load_weight(t, r3, d, n), n, d)
+    ctx.sync()
+    flat = hb.get()
+    assert np.all(flat[T * d:] == UNTOUCHED)
+    mg, mu = magnitude(t, r1, X, d, n), magnitude(t, r3, X, d, n)
+    bound = F16_BOUND * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(flat[:T * d].reshape(T, d).astype(np.float64) - ref) <= bound)
+
+
 MINOR = [O.Q5_K, O.Q6_K, O.Q4_1, O.Q5_0, O.IQ4_XS]
 
 
