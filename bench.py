@@ -296,6 +296,56 @@ def bench_fused_rms(ctx, hip, proj, layers, wcls, acts, host, steps, warmup):
                     "launches)"}
 
 
+def bench_short_prompt(ctx, hip, tokens, steps, warmup):
+    """One Llama-3.2-1B Q8_0 layer's four batched calls between batched decode and prefill -- a
+    short prompt, or the tail of a chunked one: 65 .. 511 rows, fp32 activations and the binary16
+    ones the reference's prefill plan hands over, eight layers' weights swept per replay.  Checked
+    against the oracle on sampled rows and columns first."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.projections import QuantizedBatchProjections
+    t, copies, bound = GGMLType.Q8_0, 8, 2e-3
+    shapes = {"wq": (DIM, DIM), "wk": (KV_DIM, DIM), "wv": (KV_DIM, DIM), "wo": (DIM, DIM),
+              "w1": (HIDDEN, DIM), "w3": (HIDDEN, DIM), "w2": (DIM, HIDDEN)}
+    host = {k: synthetic.weight(t, r, c, 141 + i) for i, (k, (r, c)) in enumerate(shapes.items())}
+    layers = [{k: ctx.load_weight(t, host[k], *shapes[k]) for k in shapes} for _ in range(copies)]
+    legs = []
+    for T in tokens:
+        Xh = synthetic.activations((T, DIM), 148).astype(np.float16).astype(np.float32)
+        Hh = (synthetic.activations((T, HIDDEN), 149) * np.float32(0.1)).astype(np.float16).astype(np.float32)
+        qkv, res, hb = ctx.float_array(T * (DIM + 2 * KV_DIM)), ctx.float_array(T * DIM, fill=0.0), ctx.float_array(T * HIDDEN)
+        proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN)
+        leg = {"tokens": T, "type": "Q8_0", "layer": "Llama-3.2-1B (dim 2048, kv 512, ffn 8192)", "layers_swept": copies}
+        for name, X, H in (("fp32_activations", ctx.from_numpy(Xh), ctx.from_numpy(Hh)),
+                           ("fp16_activations", ctx.half_from_numpy(Xh), ctx.half_from_numpy(Hh))):
+            def layer(w, X=X, H=H):
+                proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
+                proj.projection(X, res, w["wo"], DIM, DIM, True)
+                proj.gateUp(X, hb, w["w1"], w["w3"], DIM, HIDDEN)
+                proj.projection(H, res, w["w2"], HIDDEN, DIM, True)
+            res.init(0.0)
+            layer(layers[0])
+            ctx.sync()
+            arows, ro, rh = sample_rows(T, 8, 150), sample_rows(DIM, 48, 151), sample_rows(HIDDEN, 48, 152)
+            ref_o, mag_o = oracle_rows(t, host["wo"], DIM, ro, Xh[arows])
+            ref_d, mag_d = oracle_rows(t, host["w2"], HIDDEN, ro, Hh[arows])
+            errs = {"o+down": check(f"short prompt T={T} o + down", res.get().reshape(T, DIM)[arows][:, ro], ref_o + ref_d,
+                                    mag_o + mag_d, bound)}
+            g, mg = oracle_rows(t, host["w1"], DIM, rh, Xh[arows])
+            u, mu = oracle_rows(t, host["w3"], DIM, rh, Xh[arows])
+            errs["gate/up"] = check_swiglu(f"short prompt T={T} gate/up", hb.get().reshape(T, HIDDEN)[arows][:, rh], g, u, mg, mu, bound)
+            ms = [m / copies for m in timed_graph(ctx, hip, lambda: [layer(w) for w in layers], steps, warmup)]
+            med = statistics.median(ms)
+            flops = 2.0 * T * (DIM * (DIM + 2 * KV_DIM) + DIM * DIM + 3 * DIM * HIDDEN)
+            leg[name] = {"ms_per_layer": round(med, 4), "ms_stats": spread_stats(ms), "tok_s_per_layer": round(T / (med * 1e-3), 1),
+                         "tflops": round(flops / (med * 1e-3) / 1e12, 1), "check_rel_err": errs}
+        legs.append(leg)
+    for w in layers:
+        for tensor in w.values():
+            tensor.free()
+    return legs
+
+
 def decode_bytes():
     """Algorithmic bytes of a step: every one of the 7 projections of a layer counted on its own
     (weight blocks + fp32 input + fp32 output), as the benchmark's definition does, even where one
@@ -977,7 +1027,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-extra", action="store_true", help="skip the legs beside the decode set")
-    ap.add_argument("--extra", default="wq_shape,fused_rms,prefill,other_types,batched,prefill_other_types,batched_other_types",
+    ap.add_argument("--extra", default="wq_shape,fused_rms,prefill,other_types,batched,prefill_other_types,batched_other_types,short_prompt",
                     help="comma-separated legs beside the decode set (a profiler run takes a few at a time)")
     ap.add_argument("--prefill-warmup", type=int, default=-1,
                     help="untimed replays before the prefill legs (default 100; 10 under a profiler)")
@@ -1240,6 +1290,9 @@ def main():
                 for name, dims, model, copies in (("Q8_0", (DIM, KV_DIM, HIDDEN), "Llama-3.2-1B", 32),
                                                   ("Q4_0", (4096, 1024, 14336), "Llama-3-8B", 8))
                 for B in (8, 32, 64)]
+        if "short_prompt" in legs:
+            # between batched decode and prefill: 96, 192 and 384 rows (most prompts are this long)
+            out["short_prompt"] = bench_short_prompt(ctx, hip, (96, 192, 384), max(5, args.steps // 5), 3)
         out["cpu_baseline"] = cpu_baseline(host, shapes, t) if cpu else None
     print(json.dumps(out))
 
