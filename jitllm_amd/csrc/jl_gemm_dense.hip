@@ -599,54 +599,50 @@ int launch_decode(jl_context *ctx, const DecodeParams &d, int activation_rows) {
 
 }  // namespace
 
-// Column tile the dense path would use for a call (and in *row_tile the row tile), 0 when the call
-// is not one for it: it takes 512 rows or more and enough work items to give most compute units
-// one.  The largest tile that does so wins: 256 x 256, 256 x 128, then 128 x 128 (a width of whole
-// 192-column tiles can also get 256 x 192 or 128 x 192, returned as 192); narrow
-// projections on few rows get there by cutting K into 2, 4 or 8 runs of at least four steps as well
-// (plain store / residual only); what is still too small keeps the decode-in-the-loop kernel.
+// Column tile the dense path would use for a call (and in *row_tile the row tile, in *splits the
+// runs K is cut into), 0 when the call is not one for it: it takes 512 rows or more and enough
+// work to give most compute units a 128 x 128 tile of an eighth of K.  Every tiling the kernel has
+// is priced -- rounds of work items over the compute units x outputs per item x what an output costs
+// in that tile, measured with every compute unit busy at K = 2048: 256 x 256 runs at ~1180 TFLOP/s,
+// 256 x 192 at ~980, 256 x 128 at ~960, 128 x 192 at ~790, 128 x 128 at ~650 -- and the cheapest
+// wins, larger tiles and fewer runs first among equals.  192-column tiles are for widths that are
+// whole multiples of them (a fused q|k|v of 3072 or 6144 columns; plain store / residual only).
+// 128 x 128 tiles may also cut K into 2, 4 or 8 runs of at least four steps (plain store / residual
+// only), which costs the fold's launch and the partial sums' trip through memory.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits,
                          int *row_tile) {
     *splits = 1;
     *row_tile = 256;
     if (rows < 512 || k % 64 != 0) return 0;
-    const int mtiles = (rows + 255) / 256;
-    const bool wide_fills = (int64_t)mtiles * ((out_cols_virtual + 255) / 256) >= compute_units;
-    const int64_t items = (int64_t)mtiles * ((out_cols_virtual + 127) / 128);
-    // A width of whole 192-column tiles (a fused q|k|v of 3072 or 6144 columns) has two more tiles
-    // to choose from.  Each candidate is priced as rounds of work items over the compute units x
-    // outputs per item x what an output costs in that tile (measured, K = 2048: 256 x 256 runs at
-    // ~1180 TFLOP/s when every compute unit has an item, 256 x 192 at ~980, 256 x 128 at ~960,
-    // 128 x 192 at ~790, 128 x 128 at ~650), against the choice the rules below would make.
-    if (epilogue != JL_SWIGLU && out_cols_virtual % 192 == 0) {
-        auto cost = [&](int bm, int bn, int per_output) {
-            const int64_t n = (int64_t)((rows + bm - 1) / bm) * ((out_cols_virtual + bn - 1) / bn);
-            return (n + compute_units - 1) / compute_units * bm * bn * per_output;
-        };
-        const int64_t other = wide_fills                                    ? cost(256, 256, 85)
-                              : items * 10 >= (int64_t)compute_units * 7 ? cost(256, 128, 105)
-                                                                          : cost(128, 128, 150);
-        const int64_t wide = cost(256, 192, 100), tall = cost(128, 192, 125);
-        if (wide <= tall && wide < other) return 192;
-        if (tall < other) {
-            *row_tile = 128;
-            return 192;
-        }
-    }
-    // 256-wide tiles when they still give every compute unit work, else 128-wide ones
-    if (wide_fills) return 256;
-    if (items * 10 >= (int64_t)compute_units * 7) return 128;
+    const bool swiglu = epilogue == JL_SWIGLU;
     const int64_t small = (int64_t)((rows + 127) / 128) * ((out_cols_virtual + 127) / 128);
-    for (int s = 1; s <= 8; s *= 2) {
-        if (s > 1 && epilogue == JL_SWIGLU) break;
-        if ((k / DBK) % s != 0 || k / s < 4 * DBK) break;
-        if (small * s * 10 >= (int64_t)compute_units * 7) {
-            *splits = s;
-            *row_tile = 128;
-            return 128;
+    if (small * 8 * 10 < (int64_t)compute_units * 7) return 0;
+    // one microsecond in the units below: a 256 x 256 item of 2048 columns takes ~61 us
+    const double per_us = 256.0 * 256.0 * 85.0 / 61.0 * 2048.0 / k;
+    static const struct { int bm, bn, per_output; } tilings[] = {
+        {256, 256, 85}, {256, 192, 100}, {256, 128, 105}, {128, 192, 125}, {128, 128, 150}};
+    double best = 0.0;
+    int best_bn = 0;
+    for (const auto &t : tilings) {
+        if (t.bn == 192 && (swiglu || out_cols_virtual % 192 != 0)) continue;
+        const int64_t items = (int64_t)((rows + t.bm - 1) / t.bm) * ((out_cols_virtual + t.bn - 1) / t.bn);
+        for (int s = 1; s <= 8; s *= 2) {
+            if (s > 1 && (swiglu || t.bm != 128 || t.bn != 128)) break;
+            if ((k / DBK) % s != 0 || k / s < 4 * DBK) break;
+            if (s > 1 && items * s > 2 * (int64_t)compute_units) break;   // (bounds the planes: the workspace counts on it)
+            const int64_t rounds = (items * s + compute_units - 1) / compute_units;
+            double cost = (double)rounds * t.bm * t.bn * t.per_output / s;
+            // the fold: a launch, and s planes of partial sums written and read back
+            if (s > 1) cost += (2.0 + (double)s * rows * out_cols_virtual * 4.0 / 4e6) * per_us;
+            if (best_bn == 0 || cost < best * 0.999) {
+                best = cost;
+                best_bn = t.bn;
+                *row_tile = t.bm;
+                *splits = s;
+            }
         }
     }
-    return 0;
+    return best_bn;
 }
 
 // Bytes of the partial-sum planes of a call that cuts K into `splits` runs (an upper bound: rows

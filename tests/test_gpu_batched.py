@@ -276,7 +276,8 @@ def test_many_row_prefill_qkv_and_gate_up(ctx):
 @pytest.mark.parametrize("t,d,n,T,residual", [
     (O.Q8_0, 5800, 256, 1024, False),    # 256 x 128 tiles, last tile 40 columns
     (O.Q4_K, 6016, 256, 1024, True),     # 256 x 128 tiles, residual
-    (O.Q4_0, 16500, 256, 1100, False),   # 256 x 256 tiles, ragged rows and columns
+    (O.Q4_0, 12700, 256, 1100, False),   # 256 x 256 tiles (5 x 50: one round), ragged rows and columns
+    (O.Q4_0, 16500, 256, 1100, False),   # 256 x 128 tiles in three rounds (5 x 65 of 256 x 256 would be two)
     (O.Q8_0, 3000, 2048, 1024, True),    # 128 x 128 tiles, K whole, last tile 56 columns
     (O.Q4_K, 3000, 1024, 600, False),    # 128 x 128 tiles, K cut in two, ragged rows
     (O.Q8_0, 1500, 2048, 512, True),     # 128 x 128 tiles, K cut in four, last tile 92 columns
@@ -368,7 +369,7 @@ def test_two_pass_prefill_qkv_and_gate_up(ctx):
         ref = O.matmul_batch(t, raw, X, d, n)
         assert rel_err(got[:, col:col + d], ref, magnitude(t, raw, X, d, n)) < 2e-4
         col += d
-    t, d, n, T = O.Q4_0, 8200, 256, 1024
+    t, d, n, T = O.Q4_0, 7944, 256, 1024   # 256 x 256 tiles, 4 x 63 of them, the last with 8 outputs
     r1 = synthetic.weight(t, d, n, seed=291)
     r3 = synthetic.weight(t, d, n, seed=292)
     X = synthetic.activations((T, n), seed=293)
