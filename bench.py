@@ -314,11 +314,14 @@ def bench_short_prompt(ctx, hip, tokens, steps, warmup):
         Xh = synthetic.activations((T, DIM), 148).astype(np.float16).astype(np.float32)
         Hh = (synthetic.activations((T, HIDDEN), 149) * np.float32(0.1)).astype(np.float16).astype(np.float32)
         qkv, res, hb = ctx.float_array(T * (DIM + 2 * KV_DIM)), ctx.float_array(T * DIM, fill=0.0), ctx.float_array(T * HIDDEN)
-        proj = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN)
+        plain = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN)
+        # (the reference's residency choice: an fp16 copy per projection kept across calls)
+        keeping = QuantizedBatchProjections(ctx, T, HIDDEN, 2 * HIDDEN, resident=True)
         leg = {"tokens": T, "type": "Q8_0", "layer": "Llama-3.2-1B (dim 2048, kv 512, ffn 8192)", "layers_swept": copies}
-        for name, X, H in (("fp32_activations", ctx.from_numpy(Xh), ctx.from_numpy(Hh)),
-                           ("fp16_activations", ctx.half_from_numpy(Xh), ctx.half_from_numpy(Hh))):
-            def layer(w, X=X, H=H):
+        for name, proj, X, H in (("fp32_activations", plain, ctx.from_numpy(Xh), ctx.from_numpy(Hh)),
+                                 ("fp16_activations", plain, ctx.half_from_numpy(Xh), ctx.half_from_numpy(Hh)),
+                                 ("fp16_activations_resident_fp16_copy", keeping, ctx.half_from_numpy(Xh), ctx.half_from_numpy(Hh))):
+            def layer(w, X=X, H=H, proj=proj):
                 proj.fusedQKV(X, qkv, w["wq"], w["wk"], w["wv"])
                 proj.projection(X, res, w["wo"], DIM, DIM, True)
                 proj.gateUp(X, hb, w["w1"], w["w3"], DIM, HIDDEN)

@@ -885,33 +885,53 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const size_t plane_bytes = workspace_bytes > head ? workspace_bytes - head : 0;
 
 
-    if (rows < 512) {
-        // batched decode of up to 64 rows, and calls of up to 511 where it is the faster one: the
-        // weight-streaming kernel reads X itself, fp32 or fp16
-        bool taken = false;
-        int st = jl_launch_gemm_skinny(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, epilogue,
-                                       planes, plane_bytes, &taken);
-        if (st != JL_OK || taken) return st;
-    }
-
     // many rows and enough tiles: weights decoded to fp16 once per call, then the plain fp16 GEMM
     int virt = 0;
     for (int i = 0; i < count; i++) virt += (int)weights[i]->rows;
-    int dsplits = 1, bm = 256;
-    int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm);
     // A type without a decode-in-the-loop kernel (Q6_K) takes the decode-once path whatever the
     // shape: correct for any row count, tuned for none but prefill.
     const bool dense_only = !jl_has_fused_kernels(type);
-    if (dense_only && bn == 0) {
-        bn = 128;
-        bm = 256;
-        dsplits = 1;
-    }
     const size_t copy_bytes = round_up(jl_dense_copy_bytes(k, virt), 256);
     // the decoded copy goes to the caller's resident buffer when there is one that holds it,
     // otherwise to the head of the workspace's third region
     const bool kept = resident && resident->copy && resident->state && resident->bytes >= copy_bytes &&
                       ((uintptr_t)resident->copy & 255) == 0;
+
+    // Calls of 65 .. 511 rows have up to three ways to go, priced per call in microseconds (fitted to
+    // graph replays of the calls of a Llama-3.2-1B layer and of 8B-shaped layers at 65 .. 511 rows):
+    //   the weight-streaming kernel    its own estimate, which grows with rows x weights
+    //   decode in the loop             22 + (Q8_0: 0.30, 4-bit: 0.37) x 128-row tiles x million weights
+    //                                  (its cost moves in steps this does not follow beyond 256 rows;
+    //                                  with a kept copy it loses to the next way from 192 rows on,
+    //                                  every call measured, and is not considered there)
+    //   the plain fp16 GEMM            24 + 0.45 x 256-row tiles x million weights over a copy that is
+    //                                  kept across calls (from 128 rows); 30 + 2.8 x million weights
+    //                                  when the call has to decode first and has no other kernel
+    double millions = 0.0;
+    for (int i = 0; i < count; i++) millions += (double)weights[i]->rows * k * 1e-6;
+    const double in_loop_us = dense_only || (kept && rows >= 192)
+                                  ? 1e30
+                                  : 22.0 + (type == JL_Q8_0 ? 0.30 : 0.37) * ((rows + 127) / 128) * millions;
+    const double copy_us = kept && rows >= 128 ? 24.0 + 0.45 * ((rows + 255) / 256) * millions
+                           : dense_only       ? 30.0 + 2.8 * millions
+                                              : 1e30;
+    if (rows < 512) {
+        // batched decode of up to 64 rows, and calls of up to 511 where it is the cheapest: the
+        // weight-streaming kernel reads X itself, fp32 or fp16
+        bool taken = false;
+        int st = jl_launch_gemm_skinny(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, epilogue,
+                                       planes, plane_bytes, in_loop_us < copy_us ? in_loop_us : copy_us, &taken);
+        if (st != JL_OK || taken) return st;
+    }
+
+    int dsplits = 1, bm = 256;
+    int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm,
+                                  kept && copy_us < in_loop_us ? 128 : 512);
+    if (dense_only && bn == 0) {
+        bn = 128;
+        bm = 256;
+        dsplits = 1;
+    }
     const size_t in_workspace = kept ? 0 : copy_bytes;
     const bool dense = bn != 0 && in_workspace + (dsplits > 1 ? jl_dense_plane_bytes(rows, virt, dsplits) : 0) <= plane_bytes;
     const int padded_rows = dense ? (int)round_up((size_t)rows, 256) : padded;

@@ -600,7 +600,8 @@ int launch_decode(jl_context *ctx, const DecodeParams &d, int activation_rows) {
 }  // namespace
 
 // Column tile the dense path would use for a call (and in *row_tile the row tile, in *splits the
-// runs K is cut into), 0 when the call is not one for it: it takes 512 rows or more and enough
+// runs K is cut into), 0 when the call is not one for it: it takes `min_rows` rows or more (512
+// where the call has to decode its weights first) and enough
 // work to give most compute units a 128 x 128 tile of an eighth of K.  Every tiling the kernel has
 // is priced -- rounds of work items over the compute units x outputs per item x what an output costs
 // in that tile, measured with every compute unit busy at K = 2048: 256 x 256 runs at ~1180 TFLOP/s,
@@ -610,10 +611,10 @@ int launch_decode(jl_context *ctx, const DecodeParams &d, int activation_rows) {
 // 128 x 128 tiles may also cut K into 2, 4 or 8 runs of at least four steps (plain store / residual
 // only), which costs the fold's launch and the partial sums' trip through memory.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits,
-                         int *row_tile) {
+                         int *row_tile, int min_rows) {
     *splits = 1;
     *row_tile = 256;
-    if (rows < 512 || k % 64 != 0) return 0;
+    if (rows < min_rows || k % 64 != 0) return 0;
     const bool swiglu = epilogue == JL_SWIGLU;
     const int64_t small = (int64_t)((rows + 127) / 128) * ((out_cols_virtual + 127) / 128);
     if (small * 8 * 10 < (int64_t)compute_units * 7) return 0;

@@ -10,9 +10,9 @@ int jl_skinny_padded_rows(int rows) { return rows <= 16 ? 16 : 32; }
 
 int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                           const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
-                          int epilogue, float *planes, size_t plane_bytes, bool *taken) {
+                          int epilogue, float *planes, size_t plane_bytes, double other_us, bool *taken) {
     return X16 ? jl_launch_gemm_skinny_x16(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, epilogue,
-                                           planes, plane_bytes, taken)
+                                           planes, plane_bytes, other_us, taken)
                : jl_launch_gemm_skinny_x32(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, epilogue,
-                                           planes, plane_bytes, taken);
+                                           planes, plane_bytes, other_us, taken);
 }

@@ -1159,7 +1159,7 @@ int launch_nbb(jl_context *ctx, const SkinnyParams &p, int nbb, int zin, int thr
 // then uses the tiled GEMM.  (JL_SKINNY_XH: X16 is read, else X.)
 int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                     const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
-                    int epilogue, float *planes, size_t plane_bytes, bool *taken) {
+                    int epilogue, float *planes, size_t plane_bytes, double other_us, bool *taken) {
     *taken = false;
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
@@ -1184,12 +1184,10 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
 
     if (rows > 64) {
         // 65 .. 511 rows run as three to sixteen row blocks, each streaming the whole weight over its
-        // share of the chip: what this costs grows with blocks x weights, and it is taken when that
-        // is less than what the tiled GEMMs cost.  Microseconds, fitted to graph replays of the calls
-        // of a Llama-3.2-1B layer (Q8_0) and of 8B-shaped layers (Q4_K, Q6_K, Q5_K) at 65 .. 384 rows:
-        //   here                    10 + 0.155 x row blocks x million weights / share of the chip in use
-        //   decode in the loop      22 + (Q8_0: 0.30, 4-bit: 0.37) x 128-row tiles x million weights
-        //   decode once (the types with no decode-in-the-loop kernel)   30 + 2.8 x million weights
+        // share of the chip: what this costs grows with blocks x weights, and the call is taken when
+        // that is less than the caller's estimate for its other way.  Microseconds, fitted to graph
+        // replays of the calls of a Llama-3.2-1B layer (Q8_0) and of 8B-shaped layers (Q4_K, Q6_K,
+        // Q5_K) at 65 .. 384 rows: 10 + 0.155 x row blocks x million weights / share of the chip in use.
         double millions = 0.0;
         int all_groups = 0;
         for (int i = 0; i < count; i++) millions += (double)weights[i]->rows * k * 1e-6;
@@ -1197,11 +1195,7 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
         const int per_span = workgroups_per_span(ctx->compute_units, row_blocks, Z, all_groups);
         double share = (double)per_span * Z * row_blocks / ctx->compute_units;
         if (share > 1.0) share = 1.0;
-        const double here = 10.0 + 0.155 * row_blocks * millions / share;
-        const double tiled = jl_has_fused_kernels(type)
-                                 ? 22.0 + (type == JL_Q8_0 ? 0.30 : 0.37) * ((rows + 127) / 128) * millions
-                                 : 30.0 + 2.8 * millions;
-        if (here >= tiled) return JL_OK;
+        if (10.0 + 0.155 * row_blocks * millions / share >= other_us) return JL_OK;
     }
 
     SkinnyParams p{};

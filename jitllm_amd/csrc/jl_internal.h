@@ -165,21 +165,23 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
 // Batched decode (at most 64 rows): the weight-streaming kernel.  `taken` says whether the shape
 // was one it handles; when not, nothing was launched and the tiled GEMM must run instead.  `X16`
 // set: the activations as binary16 (X is then ignored); `c_f16` (JL_SWIGLU): C holds binary16.
+// `other_us`: what the caller's other way of running a call of 65 .. 511 rows is estimated to take,
+// in microseconds; such a call is taken only when streaming is estimated cheaper.
 int jl_launch_gemm_skinny(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                           const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
-                          int epilogue, float *planes, size_t plane_bytes, bool *taken);
+                          int epilogue, float *planes, size_t plane_bytes, double other_us, bool *taken);
 // Activation rows one of its workgroups multiplies: 16 or 32; calls of more rows run as two row blocks.
 int jl_skinny_padded_rows(int rows);
 // (its two halves, one translation unit each: fp32 activations, binary16 activations)
 int jl_launch_gemm_skinny_x32(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                               const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
-                              int epilogue, float *planes, size_t plane_bytes, bool *taken);
+                              int epilogue, float *planes, size_t plane_bytes, double other_us, bool *taken);
 int jl_launch_gemm_skinny_x16(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
                               const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
-                              int epilogue, float *planes, size_t plane_bytes, bool *taken);
+                              int epilogue, float *planes, size_t plane_bytes, double other_us, bool *taken);
 // Many-row prefill: weights decoded to fp16 once per call into `copy`, then a plain fp16 GEMM.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits,
-                         int *row_tile);
+                         int *row_tile, int min_rows = 512);
 size_t jl_dense_copy_bytes(int k, int out_cols_virtual);
 size_t jl_dense_plane_bytes(int rows, int out_cols_virtual, int splits);
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,
