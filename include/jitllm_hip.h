@@ -335,7 +335,9 @@ int jl_gemm(jl_context *ctx, const jl_weight *const *weights, int count, const f
  * whose weights it holds: reset *resident_state to 0 whenever the set of weights behind the buffer
  * changes -- also when a weight is freed and another one is uploaded in its place, even if the new
  * jl_weight comes back at the old address.  Calls that do not decode ignore both.  Results are the
- * same as jl_gemm's, bit for bit.
+ * same as jl_gemm's, bit for bit -- except that calls of 128 .. 511 rows may run the plain fp16 GEMM
+ * over a kept copy where jl_gemm, which would have to decode first, runs a kernel that decodes as it
+ * goes: the same products of the same fp16 operands, added in fp32 in another order.
  */
 size_t jl_gemm_resident_bytes(const jl_weight *const *weights, int count);
 int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count, const float *X, float *C,
@@ -364,7 +366,8 @@ int jl_gemm_resident(jl_context *ctx, const jl_weight *const *weights, int count
  *   resident / resident_state: as in jl_gemm_resident, or both null for jl_gemm's behaviour.
  * The workspace is sized by jl_gemm_workspace_bytes as for jl_gemm.  On inputs that fp16 holds
  * exactly and whose rows jl_gemm's rescaling does not push below fp16's normal range the fp32
- * results equal jl_gemm's bit for bit.
+ * results equal, bit for bit, those of jl_gemm (resident null) or jl_gemm_resident (the same
+ * resident buffer) on the widened inputs.
  */
 int jl_gemm_xf16(jl_context *ctx, const jl_weight *const *weights, int count, const uint16_t *X, void *C,
                  int c_fp16, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset, int epilogue,

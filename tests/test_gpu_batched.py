@@ -734,6 +734,39 @@ def test_resident_fp16_copy_gives_the_same_bits(ctx):
     assert len(kept._copies) == 2
 
 
+@pytest.mark.parametrize("t,d,n,rows,residual", [(O.Q8_0, 16384, 2048, 300, False), (O.Q4_K, 12288, 4096, 200, True)])
+def test_kept_copy_at_mid_row_counts(ctx, t, d, n, rows, residual):
+    """128 .. 511 rows over a kept fp16 copy run the plain fp16 GEMM where the call without one
+    decodes in its loop: the same fp16 products in another order of addition.  Both against the
+    oracle on the weight's first and last rows, and against each other; the second call (no decode)
+    gives the first one's bits."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("kept copy, mid rows", t, d, n, rows, residual)
+    raw = synthetic.weight(t, d, n, seed=9650)
+    w = ctx.load_weight(t, raw, d, n)
+    X = synthetic.activations((rows, n), seed=9651)
+    start = synthetic.activations((rows, d), seed=9652) if residual else np.full((rows, d), UNTOUCHED, np.float32)
+    plain = QuantizedBatchProjections(ctx, rows, n, d)
+    kept = QuantizedBatchProjections(ctx, rows, n, d, resident=True)
+    outs = [ctx.from_numpy(start) for _ in range(3)]
+    plain.projection(ctx.from_numpy(X), outs[0], w, n, d, residual)
+    kept.projection(ctx.from_numpy(X), outs[1], w, n, d, residual)
+    kept.projection(ctx.from_numpy(X), outs[2], w, n, d, residual)
+    ctx.sync()
+    a, b, c = (o.get().reshape(rows, d) for o in outs)
+    assert np.array_equal(b.view(np.uint32), c.view(np.uint32))
+    row_bytes = raw.size // d
+    edge = 96
+    for cols, part in ((slice(0, edge), raw[:edge * row_bytes]), (slice(d - edge, d), raw[(d - edge) * row_bytes:])):
+        ref = O.matmul_batch(t, part, X, edge, n).astype(np.float64) + (start[:, cols] if residual else 0.0)
+        mag = magnitude(t, part, X, edge, n) + (np.abs(start[:, cols]) * 1e-6 if residual else 0.0)
+        assert rel_err(a[:, cols], ref, mag) < F16_BOUND
+        assert rel_err(b[:, cols], ref, mag) < F16_BOUND
+        assert rel_err(b[:, cols], a[:, cols].astype(np.float64), mag) < 1e-5
+    w.free()
+
+
 def test_huge_activation_rows_stay_finite(ctx):
     """Rows far outside fp16's range are rescaled by a power of two, not turned into infinities."""
     from jitllm_amd import synthetic
