@@ -767,6 +767,44 @@ def test_kept_copy_at_mid_row_counts(ctx, t, d, n, rows, residual):
     w.free()
 
 
+def test_kept_copy_gate_up_at_mid_row_counts(ctx):
+    """gate/up + SwiGLU at 300 rows over a kept copy (the plain fp16 GEMM on interleaved half tiles),
+    fp32 result and binary16 result, against the oracle on the first and last outputs; then 40 rows
+    with the same projections, which stream the weights and leave the kept copy alone."""
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("kept copy, mid rows, gate/up")
+    t, d, n, rows = O.Q8_0, 8192, 2048, 300
+    r1, r3 = synthetic.weight(t, d, n, seed=9660), synthetic.weight(t, d, n, seed=9661)
+    w1, w3 = ctx.load_weight(t, r1, d, n), ctx.load_weight(t, r3, d, n)
+    X16 = synthetic.activations((rows, n), seed=9662).astype(np.float16)
+    X = X16.astype(np.float32)
+    kept = QuantizedBatchProjections(ctx, rows, n, 2 * d, resident=True)
+    edge, row_bytes = 64, r1.size // d
+
+    def check(got, active):
+        for cols in (slice(0, edge), slice(d - edge, d)):
+            lo = cols.start * row_bytes
+            g = O.matmul_batch(t, r1[lo:lo + edge * row_bytes], X[:active], edge, n)
+            u = O.matmul_batch(t, r3[lo:lo + edge * row_bytes], X[:active], edge, n)
+            want = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(active, edge)
+            mg = magnitude(t, r1[lo:lo + edge * row_bytes], X[:active], edge, n)
+            mu = magnitude(t, r3[lo:lo + edge * row_bytes], X[:active], edge, n)
+            bound = F16_BOUND * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+            assert np.all(np.abs(got[:active, cols].astype(np.float64) - want) <= bound)
+
+    for active in (rows, 40):
+        h32 = ctx.float_array(rows * d, fill=UNTOUCHED)
+        h16 = ctx.half_from_numpy(np.full(rows * d, 7.5, dtype=np.float16))
+        kept._gemm([w1, w3], ctx.half_from_numpy(X16), h32, active, d, 0, L.JL_SWIGLU)
+        kept._gemm([w1, w3], ctx.half_from_numpy(X16), h16, active, d, 0, L.JL_SWIGLU)
+        ctx.sync()
+        a, b = h32.get().reshape(rows, d), h16.get().reshape(rows, d)
+        check(a, active)
+        assert np.array_equal(b[:active].view(np.uint16), a[:active].astype(np.float16).view(np.uint16))
+        assert np.all(a[active:] == UNTOUCHED) and np.all(b[active:] == np.float16(7.5))
+
+
 def test_huge_activation_rows_stay_finite(ctx):
     """Rows far outside fp16's range are rescaled by a power of two, not turned into infinities."""
     from jitllm_amd import synthetic
