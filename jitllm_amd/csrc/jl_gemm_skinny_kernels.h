@@ -678,13 +678,22 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
             const uint8_t *w_gate = sg.w + base_off;
             asm volatile("" : "+s"(w_gate));   // in scalar registers before any per-lane arithmetic
             uint8_t *dst = ring + st * stage_bytes;
-            if (first_row + out_rows <= sg.rows) {
-                // every row of the group exists (uniform; all groups but a weight's last)
+            if (first_row + out_rows <= sg.rows && p.row_blocks == 1) {
+                // every row of the group exists (uniform; all groups but a weight's last), and
+                // nobody else reads this tile: read once, marked so
 #pragma unroll
                 for (int j = 0; j < LD; j++) {
                     if (j >= n_loads) break;
                     __builtin_amdgcn_global_load_lds((gvoid *)(w_gate + slot_off[j]),
                                                      (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, kStreamNonTemporal);
+                }
+            } else if (first_row + out_rows <= sg.rows) {
+                // the other row blocks' workgroups read the same tile from the same L2: default policy
+#pragma unroll
+                for (int j = 0; j < LD; j++) {
+                    if (j >= n_loads) break;
+                    __builtin_amdgcn_global_load_lds((gvoid *)(w_gate + slot_off[j]),
+                                                     (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, 0);
                 }
             } else {
 #pragma unroll
@@ -693,7 +702,7 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
                     // past the weight's last row: re-read the group's first row
                     const int wrow = first_row + slot_wrow[j] >= sg.rows ? 0 : slot_wrow[j];
                     __builtin_amdgcn_global_load_lds((gvoid *)(w_gate + slot_off_row0[j] + (int64_t)wrow * p.row_bytes),
-                                                     (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, kStreamNonTemporal);
+                                                     (lvoid *)(dst + (j * kDmaWaves + dw) * 1024), 16, 0, 0);
                 }
             }
         };
