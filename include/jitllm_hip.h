@@ -289,7 +289,9 @@ int jl_gemv_gate_up_q8(jl_context *ctx, const jl_weight *w1, const jl_weight *w3
  * call that a call uses for one of two things: the partial sums of calls that cut K across
  * workgroups (calls whose tile grid would leave compute units idle), or -- calls of 512 rows and
  * more, the reference's dequantize-then-gemmMMA prefill shape -- an fp16 copy of the call's
- * weights, decoded afresh by every such call and dead after it.  A smaller workspace that still
+ * weights, decoded afresh by every such call and dead after it (beside it the partial sums of
+ * narrow projections, which also calls of 128 rows and more over a kept copy use: the size counts
+ * them from max_rows = 128).  A smaller workspace that still
  * holds the first two is accepted; such calls simply keep to one pass and do not cut K.  Calls of
  * at most 64 rows -- and calls of up to 511 rows whose weights are small enough that streaming
  * them once per 32 rows beats the tiled kernels -- read X directly and use only the partial sums.

@@ -781,13 +781,14 @@ size_t jl_gemm_workspace_bytes_impl(int64_t max_rows, int64_t cols, int64_t out_
     // (256: the fp16 copy of a call's weights, which calls of a type without a decode-in-the-loop
     // kernel always make, is padded to whole 256-row column tiles)
     size_t planes = round_up(round_up((size_t)out_cols, 256) * (size_t)cols * 17 / 8 + 128 * 128 * 4, 256);
-    // calls of 512 rows or more may decode the weights to fp16 once, into the same region
-    // (and, for narrow projections, up to eight planes of partial sums; such calls have fewer
-    // 256 x 128 tiles than 0.7 x 256 compute units and are cut no further than twice that many
-    // work items, which bounds the planes)
-    if (max_rows >= 512) {
+    // calls of 512 rows or more may decode the weights to fp16 once, into the same region (and,
+    // for narrow projections, up to eight planes of partial sums: K is cut for 128 x 128 tiles only
+    // and into no more work items than twice 256 compute units, which bounds the planes -- their
+    // rows are padded to 256, at most twice the tiles' rows); calls of 128 rows or more over a copy
+    // the caller keeps cut K the same way.  A call whose workspace is smaller than this keeps K whole.
+    if (max_rows >= 128) {
         size_t two = jl_dense_plane_bytes((int)max_rows, (int)out_cols, 8);
-        const size_t cap = 2 * (size_t)180 * 256 * 128 * sizeof(float);
+        const size_t cap = 2 * (size_t)2 * 256 * 128 * 128 * sizeof(float);
         if (two > cap) two = cap;
         const size_t need = round_up(jl_dense_copy_bytes((int)cols, (int)out_cols), 256) + two;
         if (need > planes) planes = need;
@@ -924,15 +925,19 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
         if (st != JL_OK || taken) return st;
     }
 
+    const size_t in_workspace = kept ? 0 : copy_bytes;
+    const int dense_from = kept && copy_us < in_loop_us ? 128 : 512;
     int dsplits = 1, bm = 256;
-    int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm,
-                                  kept && copy_us < in_loop_us ? 128 : 512);
+    int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm, dense_from);
+    if (bn != 0 && dsplits > 1 && in_workspace + jl_dense_plane_bytes(rows, virt, dsplits) > plane_bytes) {
+        // no room for the partial sums of a cut K: the cheapest tiling that keeps K whole
+        bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm, dense_from, false);
+    }
     if (dense_only && bn == 0) {
         bn = 128;
         bm = 256;
         dsplits = 1;
     }
-    const size_t in_workspace = kept ? 0 : copy_bytes;
     const bool dense = bn != 0 && in_workspace + (dsplits > 1 ? jl_dense_plane_bytes(rows, virt, dsplits) : 0) <= plane_bytes;
     const int padded_rows = dense ? (int)round_up((size_t)rows, 256) : padded;
 

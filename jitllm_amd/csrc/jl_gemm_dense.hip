@@ -609,9 +609,10 @@ int launch_decode(jl_context *ctx, const DecodeParams &d, int activation_rows) {
 // wins, larger tiles and fewer runs first among equals.  192-column tiles are for widths that are
 // whole multiples of them (a fused q|k|v of 3072 or 6144 columns; plain store / residual only).
 // 128 x 128 tiles may also cut K into 2, 4 or 8 runs of at least four steps (plain store / residual
-// only), which costs the fold's launch and the partial sums' trip through memory.
+// only; not with `may_cut_k` false), which costs the fold's launch and the partial sums' trip
+// through memory.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits,
-                         int *row_tile, int min_rows) {
+                         int *row_tile, int min_rows, bool may_cut_k) {
     *splits = 1;
     *row_tile = 256;
     if (rows < min_rows || k % 64 != 0) return 0;
@@ -628,7 +629,7 @@ int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, in
         if (t.bn == 192 && (swiglu || out_cols_virtual % 192 != 0)) continue;
         const int64_t items = (int64_t)((rows + t.bm - 1) / t.bm) * ((out_cols_virtual + t.bn - 1) / t.bn);
         for (int s = 1; s <= 8; s *= 2) {
-            if (s > 1 && (swiglu || t.bm != 128 || t.bn != 128)) break;
+            if (s > 1 && (!may_cut_k || swiglu || t.bm != 128 || t.bn != 128)) break;
             if ((k / DBK) % s != 0 || k / s < 4 * DBK) break;
             if (s > 1 && items * s > 2 * (int64_t)compute_units) break;   // (bounds the planes: the workspace counts on it)
             const int64_t rounds = (items * s + compute_units - 1) / compute_units;

@@ -181,7 +181,7 @@ int jl_launch_gemm_skinny_x16(jl_context *ctx, const jl_weight *const *weights, 
                               int epilogue, float *planes, size_t plane_bytes, double other_us, bool *taken);
 // Many-row prefill: weights decoded to fp16 once per call into `copy`, then a plain fp16 GEMM.
 int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, int compute_units, int *splits,
-                         int *row_tile, int min_rows = 512);
+                         int *row_tile, int min_rows = 512, bool may_cut_k = true);
 size_t jl_dense_copy_bytes(int k, int out_cols_virtual);
 size_t jl_dense_plane_bytes(int rows, int out_cols_virtual, int splits);
 int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int count, const _Float16 *A,

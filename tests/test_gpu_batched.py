@@ -767,6 +767,36 @@ def test_kept_copy_at_mid_row_counts(ctx, t, d, n, rows, residual):
     w.free()
 
 
+@pytest.mark.parametrize("t,d,n,batch,rows,tight", [(O.Q6_K, 5870, 768, 243, 243, False), (O.Q6_K, 3554, 1024, 345, 155, False),
+                                                    (O.Q6_K, 5870, 768, 243, 243, True), (O.Q8_0, 4000, 1024, 130, 130, True),
+                                                    (O.Q4_K, 1500, 2048, 600, 600, True)])
+def test_kept_copy_of_a_narrow_projection_cuts_k_only_where_the_workspace_has_room(ctx, t, d, n, batch, rows, tight):
+    """A narrow projection over a kept copy would cut K and fold partial sums from the workspace:
+    with the workspace the size query gives it does, with the least workspace a call may bring
+    (``tight``: the activations' region only) it keeps K whole -- and a type that has no kernel but
+    the decode-once one is served either way instead of refused."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("kept copy, narrow projection", t, d, n, batch, rows, tight)
+    raw = synthetic.weight(t, d, n, seed=9670 + d)
+    w = ctx.load_weight(t, raw, d, n)
+    X = synthetic.activations((batch, n), seed=9671)
+    kept = QuantizedBatchProjections(ctx, batch, n, 0 if tight else d, resident=True)
+    outs = [ctx.float_array(batch * d, fill=UNTOUCHED) for _ in range(2)]
+    for out in outs:
+        kept.projection(ctx.from_numpy(X), out, w, n, d, False, activeRows=rows)
+    ctx.sync()
+    a, b = (o.get().reshape(batch, d) for o in outs)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.all(a[rows:] == UNTOUCHED)
+    row_bytes = raw.size // d
+    edge = 96
+    for cols, part in ((slice(0, edge), raw[:edge * row_bytes]), (slice(d - edge, d), raw[(d - edge) * row_bytes:])):
+        ref = O.matmul_batch(t, part, X[:rows], edge, n)
+        assert rel_err(a[:rows, cols], ref, magnitude(t, part, X[:rows], edge, n)) < F16_BOUND
+    w.free()
+
+
 def test_kept_copy_gate_up_at_mid_row_counts(ctx):
     """gate/up + SwiGLU at 300 rows over a kept copy (the plain fp16 GEMM on interleaved half tiles),
     fp32 result and binary16 result, against the oracle on the first and last outputs; then 40 rows
