@@ -823,7 +823,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
         }
         const int64_t offset = (int64_t)local * half_bytes;
         const int64_t remain = (int64_t)seg_rows * row_bytes - offset;
-        const int bytes = remain < half_bytes ? (int)remain : half_bytes;
+        // (the fixed-geometry form is launched over whole tiles only, and tracks no segment's rows)
+        const int bytes = LEAN || remain >= half_bytes ? half_bytes : (int)remain;
         const uint8_t *base = wseg + offset;
         const uint8_t *base_up = DUAL ? w_up_first + offset : base;
         uint8_t *dst = ring + st * stage_bytes;

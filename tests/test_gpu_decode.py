@@ -299,6 +299,33 @@ def test_fused_qkv(ctx, t, dq, dkv, n):
         assert rel_err(out.get(), ref, magnitude(t, raw, x, d, n)) < 2e-5
 
 
+@pytest.mark.parametrize("t,dims,n", [(O.Q8_0, (276, 1024, 1024), 3008), (O.Q4_0, (198, 242, 242), 6144),
+                                       (O.Q4_K, (64, 512, 256), 5120), (O.Q8_0, (8, 1024, 512), 2048),
+                                       (O.Q4_K, (12, 40, 2000), 1536)])
+def test_fused_qkv_whose_first_weight_is_the_shortest(ctx, t, dims, n):
+    """q | k | v with fewer rows in the first weight than in the others, on rows that fill their
+    slices only in part (and on ones that fill them): every weight's tiles are read to their own
+    end, whatever the first weight's row count; plain and RMS-folding."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("qkv, short first weight", NAMES[t], dims, n)
+    raws = [synthetic.weight(t, d, n, seed=3300 + i) for i, d in enumerate(dims)]
+    x = synthetic.activations(n, seed=3310)
+    rw = (1.0 + 0.25 * synthetic.activations(n, seed=3311)).astype(np.float32)
+    xn = O.rmsnorm(x, rw, 1e-5)
+    ws = [upload(ctx, t, r, d, n) for r, d in zip(raws, dims)]
+    plain = [ctx.float_array(d, fill=POISON) for d in dims]
+    folded = [ctx.float_array(d, fill=POISON) for d in dims]
+    proj = QuantizedProjections(ctx, TornadoWorkspace())
+    dx = ctx.from_numpy(x)
+    proj.fusedQKV(dx, *plain, *ws)
+    proj.fusedRmsNormQKV(dx, *folded, ctx.from_numpy(rw), None, *ws, eps=1e-5)
+    ctx.sync()
+    for raw, d, a, b in zip(raws, dims, plain, folded):
+        assert rel_err(a.get(), O.matmul(t, raw, x, d, n), magnitude(t, raw, x, d, n)) < 2e-5
+        assert rel_err(b.get(), O.matmul(t, raw, xn, d, n), magnitude(t, raw, xn, d, n)) < 2e-5
+
+
 # Rows of 128 slices (5120, 7168, 8192 columns) put one gate row and one up row in a tile, so 272 rows
 # and 271 rows are both whole tiles and both run the fixed-geometry instance: the bit comparison of
 # fixed and general kernels cannot reach those instances, and they are held to the oracle here.
