@@ -178,3 +178,67 @@ def test_hostile_header_fields_are_refused_not_followed(tmp_path):
     for count in (1 << 40, 400):
         with pytest.raises(JitllmHipError, match="impossible counts|malformed|end early"):
             GGUF(_crafted(tmp_path, "count.gguf", tensor_count=count))
+
+
+def test_mutated_files_get_a_status_from_every_call(tmp_path):
+    """1 500 seeded mutations of a valid file -- flipped bytes, truncations, inserted bytes, length
+    and type fields overwritten with boundary values: opening either fails with a message or gives a
+    file every accessor answers with a status; a tensor is never uploaded without a context, and
+    never before the file's own faults are reported."""
+    import ctypes as C
+    import struct
+
+    from jitllm_amd import _lib as L
+    lib = L.load()
+    rng = np.random.default_rng(20261124)
+    base = tmp_path / "base.gguf"
+    W.write_gguf(base, META, tensors())
+    blob = bytearray(base.read_bytes())
+    keys = [k.encode() for k, _, _ in META] + [b"general.alignment", b"no.such.key"]
+    big = [2 ** 64 - 1, 2 ** 63, 2 ** 62, 2 ** 32, 2 ** 31, len(blob), len(blob) + 1, 0]
+    small = [2 ** 32 - 1, 2 ** 31, 13, 12, 9, 8, 5, 0]
+    opened = 0
+    path = tmp_path / "mutated.gguf"
+    for case in range(1500):
+        b = bytearray(blob)
+        kind = int(rng.integers(0, 5))
+        if kind == 0:
+            for _ in range(int(rng.integers(1, 4))):
+                b[int(rng.integers(0, len(b)))] = int(rng.integers(0, 256))
+        elif kind == 1:
+            b = b[:int(rng.integers(0, len(b)))]
+        elif kind == 2:
+            at = int(rng.integers(0, len(b) - 8))
+            b[at:at + 8] = struct.pack("<Q", big[int(rng.integers(0, 8))])
+        elif kind == 3:
+            at = int(rng.integers(0, len(b) - 4))
+            b[at:at + 4] = struct.pack("<I", small[int(rng.integers(0, 8))])
+        else:
+            at = int(rng.integers(0, len(b)))
+            b[at:at] = bytes(rng.integers(0, 256, int(rng.integers(1, 40)), dtype=np.uint8))
+        path.write_bytes(b)
+        h = C.c_void_p()
+        if lib.jl_gguf_open(str(path).encode(), C.byref(h)) != 0:
+            assert lib.jl_last_error() and not h.value
+            continue
+        opened += 1
+        count = lib.jl_gguf_tensor_count(h)
+        assert count >= 0 and lib.jl_gguf_metadata_count(h) >= 0 and lib.jl_gguf_data_offset(h) >= 0
+        for i in range(-1, count + 1):
+            name, typ, nd = C.c_char_p(), C.c_int(), C.c_int()
+            dims, off, nbytes = (C.c_int64 * 4)(), C.c_int64(), C.c_int64()
+            st = lib.jl_gguf_tensor_info(h, i, C.byref(name), C.byref(typ), C.byref(nd), dims, C.byref(off), C.byref(nbytes))
+            assert (st == 0) == (0 <= i < count)
+            if st == 0:
+                w = C.c_void_p()
+                assert lib.jl_gguf_upload(None, h, name.value, C.byref(w)) != 0 and not w.value
+        for key in keys:
+            v, d, s, ln, et, cnt = C.c_int64(), C.c_double(), C.c_char_p(), C.c_int64(), C.c_int(), C.c_int64()
+            lib.jl_gguf_metadata_int(h, key, C.byref(v))
+            lib.jl_gguf_metadata_float(h, key, C.byref(d))
+            if lib.jl_gguf_metadata_string(h, key, C.byref(s), C.byref(ln)) == 0:
+                assert len(s.value) <= ln.value <= len(b)
+            if lib.jl_gguf_metadata_array(h, key, C.byref(et), C.byref(cnt)) == 0:
+                assert 0 <= cnt.value or et.value >= 0
+        assert lib.jl_gguf_close(h) == 0
+    assert 100 < opened < 1500
