@@ -102,3 +102,40 @@ def test_synthetic_weights_follow_the_stated_distributions():
     assert np.array_equal(raw.reshape(-1), synthetic.weight(GGMLType.Q8_0, 8, 2048, seed=3))
     k = synthetic.weight(GGMLType.Q4_K, 4, 1024, seed=4)
     assert k.size == 4 * 4 * 144
+
+
+def test_header_is_plain_c_and_the_library_links_from_c(lib, tmp_path):
+    """The boundary is a C ABI: the header compiles as strict C99 with no other include than the
+    standard ones, and a C program that knows nothing but the header links against the library and
+    gets answers from the calls that need no device."""
+    import shutil
+    import subprocess
+    from jitllm_amd import _lib as L
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "consumer.c"
+    src.write_text(
+        '#include "jitllm_hip.h"\n'
+        '#include <stdio.h>\n'
+        '#include <string.h>\n'
+        'int main(void) {\n'
+        '    jl_context *ctx = (jl_context *)0;\n'
+        '    jl_weight *w = (jl_weight *)0;\n'
+        '    unsigned char block[34] = {0};\n'
+        '    int st = jl_weight_upload(ctx, JL_Q8_0, block, 1, 32, &w);\n'
+        '    if (st != JL_ERR_INVALID || w != (jl_weight *)0) return 2;\n'
+        '    if (strlen(jl_last_error()) == 0) return 3;\n'
+        '    if (jl_gemm_workspace_bytes(64, 4096, 4096, JL_MATH_DEFAULT) == 0) return 4;\n'
+        '    printf("%d\\n", jl_abi_version());\n'
+        '    return 0;\n'
+        '}\n')
+    include = os.path.join(ROOT, "include")
+    subprocess.run([gcc, "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", include, str(src)],
+                   check=True)
+    exe = tmp_path / "consumer"
+    libdir = os.path.dirname(L.LIB)
+    subprocess.run([gcc, "-std=c99", "-I", include, str(src), "-o", str(exe), "-L", libdir, "-ljitllm_hip",
+                    "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert int(out) == lib.jl_abi_version()
