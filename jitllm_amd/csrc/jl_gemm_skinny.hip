@@ -1,4 +1,5 @@
-// Batched decode of at most 64 rows on the weight-streaming kernel: the instances for fp32
+// Batched decode (at most 64 rows, and calls of up to 511 rows where streaming the weights once per
+// 32 rows is priced cheaper than the tiled kernels) on the weight-streaming kernel: the instances for fp32
 // activations (QuantizedBatchProjections.java:76-309 hands FloatArrays) and the choice between them
 // and the binary16 ones.  The kernel itself is jl_gemm_skinny_kernels.h.
 #define JL_SKINNY_XH false

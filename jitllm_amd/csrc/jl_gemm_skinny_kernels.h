@@ -1,4 +1,5 @@
-// Batched decode (at most 64 activation rows): C = X . [W0 | W1 | ...]^T streamed at HBM speed.
+// Batched decode (at most 64 activation rows; up to 511 as row blocks of 32 where the launcher
+// prices that cheaper than the tiled kernels): C = X . [W0 | W1 | ...]^T streamed at HBM speed.
 //
 // Replaces the reference's tiled batched-row kernels (matrixVectorTiledBatchQ4_0 / Q4_K,
 // J/backend/tornado/kernels/TransformerComputeKernelsQ4_0.java:1205-1292,
@@ -28,9 +29,9 @@
 // and apply the epilogue (one row block each when there are two), rows wider than the workgroup's
 // span are cut across workgroups and folded, inside the launch, by the workgroup that arrives
 // last.  The two compute waves of a SIMD run half a tile apart: one decodes while the other
-// multiplies.  Calls of 33..64 rows run as two row blocks of up to 32 on the two halves of the
-// chip; the halves walk the same tiles at the same time, so the second reader of a tile finds it in
-// the L2 of its XCD.
+// multiplies.  Calls of more than 32 rows run as row blocks of up to 32 that share the chip (two
+// halves at 33..64 rows); the blocks walk the same tiles at about the same time, so the later
+// readers of a tile may find it in the L2 of their XCD.
 //
 // This file is compiled twice: jl_gemm_skinny.hip includes it for fp32 activations, and
 // jl_gemm_skinny_x16.hip for binary16 ones (JL_SKINNY_XH; the entry point's name is

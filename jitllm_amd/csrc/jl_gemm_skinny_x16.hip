@@ -1,4 +1,5 @@
-// Batched decode of at most 64 rows on the weight-streaming kernel: the instances for binary16
+// The weight-streaming kernel (batched decode, and calls of up to 511 rows where it is priced
+// cheaper than the tiled kernels): the instances for binary16
 // activations, as the reference's prefill plan hands them (DecodedMatMul.project,
 // J/backend/tornado/ops/DecodedMatMul.java:100-109) -- a short prompt, or the tail of a chunked one.
 #define JL_SKINNY_XH true

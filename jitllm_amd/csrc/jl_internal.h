@@ -162,7 +162,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
                    float *C, int64_t batch, int64_t active_rows, int64_t ldo, int64_t col_offset,
                    int epilogue, int math, void *workspace, size_t workspace_bytes,
                    const jl_resident *resident, const jl_half_io *half = nullptr);
-// Batched decode (at most 64 rows): the weight-streaming kernel.  `taken` says whether the shape
+// Batched decode (at most 64 rows; up to 511 where priced cheaper, see `other_us`): the weight-streaming kernel.  `taken` says whether the shape
 // was one it handles; when not, nothing was launched and the tiled GEMM must run instead.  `X16`
 // set: the activations as binary16 (X is then ignored); `c_f16` (JL_SWIGLU): C holds binary16.
 // `other_us`: what the caller's other way of running a call of 65 .. 511 rows is estimated to take,
