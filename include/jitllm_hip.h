@@ -316,7 +316,14 @@ size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols,
  *            are multiples of 64.  An opt-in mode: an activation carries 7 bits, so against the
  *            fp32 CPU path it is looser than JL_MATH_F16 (every output within sum over the blocks
  *            of (dA / 2) * sum |w|).
- * JL_MATH_F16: the row length must be a multiple of 256 columns, else JL_ERR_UNSUPPORTED.
+ * JL_MATH_F16: the row length must be a multiple of 256 columns, else JL_ERR_UNSUPPORTED.  The
+ * weights of a call may differ in type (a "Q4_K_M" file's q | k | v with v in Q6_K; a gate and an up
+ * weight of different types): each is then decoded to fp16 by its own type and one fp16 GEMM
+ * multiplies them, as the reference's prefill projections do (FP16Projections.project,
+ * J/backend/tornado/layers/FP16Projections.java:250-330: one decode task per weight, chosen by its
+ * dataType()); such a call needs the workspace jl_gemm_workspace_bytes gives for its `out_cols` (or
+ * a resident buffer) whatever its row count.  JL_MATH_INT8 multiplies the raw blocks and refuses
+ * mixed types.
  * This is Int8GemmKernels.gemmInt8Q8_0's contract (:651-676: epilogue, rowsHolder, ldo,
  * colOffset) and gemmMMAQ8's, behind one call.
  */

@@ -458,8 +458,10 @@ static int gemm_checked(jl_context *ctx, const jl_weight *const *weights, int co
     int64_t total = 0;
     for (int i = 0; i < count; i++) {
         JL_REQUIRE(weights[i] != nullptr, "jl_gemm: weight %d is null", i);
-        if (weights[i]->type != weights[0]->type) {
-            return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: mixed weight types %s and %s in one call",
+        // (weights of different types run the decode-once path, each decoded by its own type; the
+        // int8 mode multiplies the raw blocks and has no such path)
+        if (weights[i]->type != weights[0]->type && math == JL_MATH_INT8) {
+            return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: mixed weight types %s and %s in one int8 call",
                            jl_type_name(weights[0]->type), jl_type_name(weights[i]->type));
         }
         JL_REQUIRE(weights[i]->cols == weights[0]->cols, "jl_gemm: weight %d row length %lld != %lld",

@@ -890,8 +890,13 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     int virt = 0;
     for (int i = 0; i < count; i++) virt += (int)weights[i]->rows;
     // A type without a decode-in-the-loop kernel (Q6_K) takes the decode-once path whatever the
-    // shape: correct for any row count, tuned for none but prefill.
-    const bool dense_only = !jl_has_fused_kernels(type);
+    // shape: correct for any row count, tuned for none but prefill.  So do weights of different
+    // types in one call (a "Q4_K_M" file's q | k | v with v in Q6_K): each is decoded by its own
+    // type, as the reference's prefill projections do (FP16Projections.java:250-330), and the
+    // fp16 GEMM does not know the difference.
+    bool mixed = false;
+    for (int i = 1; i < count; i++) mixed = mixed || weights[i]->type != type;
+    const bool dense_only = mixed || !jl_has_fused_kernels(type);
     const size_t copy_bytes = round_up(jl_dense_copy_bytes(k, virt), 256);
     // the decoded copy goes to the caller's resident buffer when there is one that holds it,
     // otherwise to the head of the workspace's third region
@@ -942,6 +947,10 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const int padded_rows = dense ? (int)round_up((size_t)rows, 256) : padded;
 
     if (dense_only && !dense) {
+        if (mixed) {
+            return jl_fail(JL_ERR_WORKSPACE, "jl_gemm: weights of mixed types need room for their fp16 copy (%zu bytes) "
+                                             "in the workspace", copy_bytes);
+        }
         return jl_fail(JL_ERR_WORKSPACE, "jl_gemm: a %s weight needs room for its fp16 copy (%zu bytes) in the workspace",
                        jl_type_name(type), copy_bytes);
     }

@@ -47,6 +47,8 @@ struct DecodeParams {
     int n_total;           // SWIGLU: rows of one weight
     int half;              // SWIGLU: BN / 2 of the GEMM that will read the copy, else 0; virtual row
                            // t * BN + sel * half + i is row t * half + i of weight sel (0 gate, 1 up)
+    int only_own;          // a later pass over weights of mixed types: rows of a weight whose
+                           // pointer is null here (another type's, or padding) are left as they are
     // the call's activations, when they ride along (else virtual_rows = the grid's width):
     // workgroups blockIdx.x >= virtual_rows convert activation row blockIdx.x - virtual_rows
     int virtual_rows;
@@ -108,7 +110,7 @@ __global__ void __launch_bounds__(256) jl_decode_to_f16(DecodeParams p) {
             }
     }
     if (w == nullptr) {
-        *dst = uint4{0, 0, 0, 0};
+        if (!p.only_own) *dst = uint4{0, 0, 0, 0};
         return;
     }
     const uint8_t *row = w + (int64_t)r * p.row_bytes;
@@ -696,21 +698,38 @@ int jl_launch_gemm_dense(jl_context *ctx, const jl_weight *const *weights, int c
         d.rows = rows;
         xr = (rows + kRowPad - 1) / kRowPad * kRowPad;
     }
-    int dst = JL_OK;
-    if (decode) {
-        switch (type) {
-            case JL_Q8_0: dst = launch_decode<JL_Q8_0>(ctx, d, xr); break;
-            case JL_Q4_0: dst = launch_decode<JL_Q4_0>(ctx, d, xr); break;
-            case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, d, xr); break;
-            case JL_Q5_K: dst = launch_decode<JL_Q5_K>(ctx, d, xr); break;
-            case JL_Q6_K: dst = launch_decode<JL_Q6_K>(ctx, d, xr); break;
-            case JL_Q4_1: dst = launch_decode<JL_Q4_1>(ctx, d, xr); break;
-            case JL_Q5_0: dst = launch_decode<JL_Q5_0>(ctx, d, xr); break;
-            case JL_IQ4_XS: dst = launch_decode<JL_IQ4_XS>(ctx, d, xr); break;
-            default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", type);
+    // Each weight is decoded by its own type, as the reference's prefill projections decode theirs
+    // (FP16Projections.project, J/backend/tornado/layers/FP16Projections.java:250-330: one decode
+    // task per weight, chosen by its dataType()): one pass per type that occurs.  The first pass
+    // sees the other types' weights as absent and fills their rows, like the padding, with zeros;
+    // the later ones write their own weights' rows only.  The activations ride along once.
+    bool first_pass = true;
+    for (int i0 = 0; decode && i0 < count; i0++) {
+        const int pass_type = weights[i0]->type;
+        bool earlier = false;   // decoded by the pass that began at the type's first weight
+        for (int j = 0; j < i0; j++) earlier = earlier || weights[j]->type == pass_type;
+        if (earlier) continue;
+        DecodeParams pass = d;
+        for (int j = 0; j < count; j++)
+            if (weights[j]->type != pass_type) pass.w[j] = nullptr;
+        pass.row_bytes = k / jl_block_elems(pass_type) * jl_block_bytes(pass_type);
+        pass.only_own = first_pass ? 0 : 1;
+        const int ride = first_pass ? xr : 0;
+        first_pass = false;
+        int dst;
+        switch (pass_type) {
+            case JL_Q8_0: dst = launch_decode<JL_Q8_0>(ctx, pass, ride); break;
+            case JL_Q4_0: dst = launch_decode<JL_Q4_0>(ctx, pass, ride); break;
+            case JL_Q4_K: dst = launch_decode<JL_Q4_K>(ctx, pass, ride); break;
+            case JL_Q5_K: dst = launch_decode<JL_Q5_K>(ctx, pass, ride); break;
+            case JL_Q6_K: dst = launch_decode<JL_Q6_K>(ctx, pass, ride); break;
+            case JL_Q4_1: dst = launch_decode<JL_Q4_1>(ctx, pass, ride); break;
+            case JL_Q5_0: dst = launch_decode<JL_Q5_0>(ctx, pass, ride); break;
+            case JL_IQ4_XS: dst = launch_decode<JL_IQ4_XS>(ctx, pass, ride); break;
+            default: return jl_fail(JL_ERR_UNSUPPORTED, "jl_gemm: no kernel for a ggml type %d weight", pass_type);
         }
+        if (dst != JL_OK) return dst;
     }
-    if (dst != JL_OK) return dst;
 
     DenseParams p{};
     p.A = A;

@@ -279,8 +279,11 @@ class HipImplementation(Implementation):
             return False
         if any(m.dataType not in SUPPORTED for m in mm):
             return False
-        if len({m.dataType for m in mm}) != 1 or len({m.columns for m in mm}) != 1:
-            return False      # one call multiplies weights of one type and one row length
+        # one call multiplies weights of one row length; their types may differ -- each is decoded
+        # by its own, as tensorCoresOverDecoded asks only that every type be decodable
+        # (DequantizingMatMul.java:53-63)
+        if len({m.columns for m in mm}) != 1:
+            return False
         if mm[0].columns % 256:
             return False
         if step.fusion.name == GATE_UP_SWIGLU.name and mm[0].rows != mm[1].rows:

@@ -835,6 +835,54 @@ def test_kept_copy_gate_up_at_mid_row_counts(ctx):
         assert np.all(a[active:] == UNTOUCHED) and np.all(b[active:] == np.float16(7.5))
 
 
+@pytest.mark.parametrize("rows", [7, 40, 200, 700])
+@pytest.mark.parametrize("resident", [False, True])
+def test_weights_of_different_types_side_by_side(ctx, rows, resident):
+    """q | k | v as a "Q4_K_M" file holds them -- q and k in Q4_K, v in Q6_K -- in one call, and a
+    Q5_0 gate with an IQ4_XS up weight: each weight is decoded by its own type (the reference's
+    prefill projections pick the decode task per weight, FP16Projections.java:250-330), at every
+    row count, with and without a kept copy, fp32 and binary16 activations giving the same bits."""
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("mixed types side by side", rows, resident)
+    n = 2048
+    types, dims = (O.Q4_K, O.Q4_K, O.Q6_K), (1000, 264, 250)
+    raws = [synthetic.weight(t, d, n, seed=9700 + i) for i, (t, d) in enumerate(zip(types, dims))]
+    ws = [ctx.load_weight(t, r, d, n) for t, r, d in zip(types, raws, dims)]
+    X16 = synthetic.activations((rows, n), seed=9703).astype(np.float16)
+    X = X16.astype(np.float32)
+    ld = sum(dims) + 9
+    proj = QuantizedBatchProjections(ctx, rows, n, sum(dims), resident=resident)
+    outs = [ctx.float_array(rows * ld, fill=UNTOUCHED) for _ in range(3)]
+    proj._gemm(ws, ctx.from_numpy(X), outs[0], rows, ld, 5, L.JL_STORE)
+    proj._gemm(ws, ctx.half_from_numpy(X16), outs[1], rows, ld, 5, L.JL_STORE)
+    proj._gemm(ws, ctx.from_numpy(X), outs[2], rows, ld, 5, L.JL_STORE)     # (a kept copy: no decode this time)
+    ctx.sync()
+    got = outs[0].get().reshape(rows, ld)
+    for other in outs[1:]:
+        assert np.array_equal(got.view(np.uint32), other.get().reshape(rows, ld).view(np.uint32))
+    assert np.all(got[:, :5] == UNTOUCHED) and np.all(got[:, 5 + sum(dims):] == UNTOUCHED)
+    col = 5
+    for t, raw, d in zip(types, raws, dims):
+        assert rel_err(got[:, col:col + d], O.matmul_batch(t, raw, X, d, n), magnitude(t, raw, X, d, n)) < F16_BOUND
+        col += d
+    # gate / up of different types
+    d = 520
+    r1, r3 = synthetic.weight(O.Q5_0, d, n, seed=9710), synthetic.weight(O.IQ4_XS, d, n, seed=9711)
+    g, u = O.matmul_batch(O.Q5_0, r1, X, d, n), O.matmul_batch(O.IQ4_XS, r3, X, d, n)
+    ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(rows, d)
+    hb = ctx.float_array(rows * d + 64, fill=UNTOUCHED)
+    QuantizedBatchProjections(ctx, rows, n, 2 * d, resident=resident)._gemm(
+        [ctx.load_weight(O.Q5_0, r1, d, n), ctx.load_weight(O.IQ4_XS, r3, d, n)], ctx.from_numpy(X), hb, rows, d, 0,
+        L.JL_SWIGLU)
+    ctx.sync()
+    flat = hb.get()
+    assert np.all(flat[rows * d:] == UNTOUCHED)
+    mg, mu = magnitude(O.Q5_0, r1, X, d, n), magnitude(O.IQ4_XS, r3, X, d, n)
+    bound = F16_BOUND * (mg * np.abs(u) + 1.2 * mu * np.abs(g)) + 1e-6
+    assert np.all(np.abs(flat[:rows * d].reshape(rows, d).astype(np.float64) - ref) <= bound)
+
+
 def test_huge_activation_rows_stay_finite(ctx):
     """Rows far outside fp16's range are rescaled by a power of two, not turned into infinities."""
     from jitllm_amd import synthetic
@@ -873,3 +921,10 @@ def test_batched_errors(ctx):
     assert st == L.JL_ERR_INVALID
     st = lib.jl_gemm(ctx.handle, arr, 1, x.ptr, o.ptr, 4, 4, 32, 0, L.JL_STORE, L.JL_MATH_F16, ws.ptr, ws.nbytes)
     assert st == L.JL_ERR_INVALID and b"ldo" in lib.jl_last_error()
+    # the int8 mode multiplies the raw blocks: no mixed types there
+    w8 = ctx.load_weight(O.Q8_0, synthetic.weight(O.Q8_0, 64, 256, 2), 64, 256)
+    w4 = ctx.load_weight(O.Q4_0, synthetic.weight(O.Q4_0, 64, 256, 3), 64, 256)
+    two = (C.c_void_p * 2)(w8.handle, w4.handle)
+    o2 = ctx.float_array(4 * 128, 0.0)
+    st = lib.jl_gemm(ctx.handle, two, 2, x.ptr, o2.ptr, 4, 4, 128, 0, L.JL_STORE, L.JL_MATH_INT8, ws.ptr, ws.nbytes)
+    assert st == L.JL_ERR_UNSUPPORTED and b"mixed weight types Q8_0 and Q4_0" in lib.jl_last_error()

@@ -16,31 +16,39 @@ def ctx():
     c.close()
 
 
+# "Q4_K_M": a layer as such a file holds it -- Q4_K except the value and down projections in Q6_K, so
+# that q|k|v is one step over two types; "odd pair": a gate and an up weight of different types
 @pytest.mark.parametrize("t,T,residency", [(O.Q8_0, 40, False), (O.Q4_K, 600, False), (O.Q4_K, 600, True),
-                                           (O.Q6_K, 40, True)])
+                                           (O.Q6_K, 40, True), ("Q4_K_M", 40, False), ("Q4_K_M", 600, True),
+                                           ("odd pair", 130, False)])
 def test_instance_emits_a_layer(ctx, t, T, residency):
     from jitllm_amd import ops, synthetic
     from jitllm_amd.ggml import GGMLType
     from jitllm_amd.ops import HipImplementation, MatMul, ResidualAdd, SwiGLU, Target, TensorRole as R
     say("ops layer", t, T, residency)
     dim, kv, ffn = 512, 256, 4352
-    g = GGMLType(t)
+    mixed = {"Q4_K_M": {R.ATTENTION_VALUE: O.Q6_K, R.FFN_DOWN: O.Q6_K}, "odd pair": {R.FFN_UP: O.Q5_0}}.get(t, {})
+    base = O.Q4_K if isinstance(t, str) else t
     shapes = {R.ATTENTION_QUERY: (dim, dim), R.ATTENTION_KEY: (kv, dim), R.ATTENTION_VALUE: (kv, dim),
               R.ATTENTION_OUTPUT: (dim, dim), R.FFN_GATE: (ffn, dim), R.FFN_UP: (ffn, dim), R.FFN_DOWN: (dim, ffn)}
-    raws = {r: synthetic.weight(g, d, n, seed=1000 + i) for i, (r, (d, n)) in enumerate(shapes.items())}
-    tensors = {r: ctx.load_weight(g, raws[r], *shapes[r]) for r in shapes}
+    tt = {r: mixed.get(r, base) for r in shapes}          # the type of each role's weight
+    g = {r: GGMLType(tt[r]) for r in shapes}
+    raws = {r: synthetic.weight(g[r], d, n, seed=1000 + i) for i, (r, (d, n)) in enumerate(shapes.items())}
+    tensors = {r: ctx.load_weight(g[r], raws[r], *shapes[r]) for r in shapes}
     program = [
-        MatMul(R.ATTENTION_QUERY, "xb", "qkv", dim, dim, T, g), MatMul(R.ATTENTION_KEY, "xb", "k", kv, dim, T, g),
-        MatMul(R.ATTENTION_VALUE, "xb", "v", kv, dim, T, g),
-        MatMul(R.ATTENTION_OUTPUT, "att", "xb2", dim, dim, T, g),
-        MatMul(R.FFN_GATE, "xb", "hb", ffn, dim, T, g), MatMul(R.FFN_UP, "xb", "hb2", ffn, dim, T, g),
+        MatMul(R.ATTENTION_QUERY, "xb", "qkv", dim, dim, T, g[R.ATTENTION_QUERY]),
+        MatMul(R.ATTENTION_KEY, "xb", "k", kv, dim, T, g[R.ATTENTION_KEY]),
+        MatMul(R.ATTENTION_VALUE, "xb", "v", kv, dim, T, g[R.ATTENTION_VALUE]),
+        MatMul(R.ATTENTION_OUTPUT, "att", "xb2", dim, dim, T, g[R.ATTENTION_OUTPUT]),
+        MatMul(R.FFN_GATE, "xb", "hb", ffn, dim, T, g[R.FFN_GATE]), MatMul(R.FFN_UP, "xb", "hb2", ffn, dim, T, g[R.FFN_UP]),
         SwiGLU("hb", "hb2", "hb"),
-        MatMul(R.FFN_DOWN, "hb_in", "xb2", dim, ffn, T, g), ResidualAdd("x", "xb2"),
+        MatMul(R.FFN_DOWN, "hb_in", "xb2", dim, ffn, T, g[R.FFN_DOWN]), ResidualAdd("x", "xb2"),
     ]
     impl = HipImplementation(residency=residency)
     chosen = ops.split(program, 0, T, [impl], Target())
-    if t == O.Q6_K:
-        # no fused gate|up + SwiGLU restriction applies to jl_gemm: the step is claimed whole
+    if t == O.Q6_K or isinstance(t, str):
+        # no fused gate|up + SwiGLU restriction applies to jl_gemm, and the weights of a step may
+        # differ in type: the steps are claimed whole
         assert [c.step.fusion.name for c in chosen] == ["q|k|v", "projection", "gate|up + SwiGLU", "down + residual add"]
     steps = [c.step for c in chosen]
     host = {"xb": synthetic.activations((T, dim), 1101), "att": synthetic.activations((T, dim), 1102),
@@ -64,19 +72,21 @@ def test_instance_emits_a_layer(ctx, t, T, residency):
         col = 0
         for r in (R.ATTENTION_QUERY, R.ATTENTION_KEY, R.ATTENTION_VALUE):
             d, n = shapes[r]
-            ref = O.matmul_batch(t, raws[r], host["xb"], d, n)
-            assert rel_err(got[:, col:col + d], ref, magnitude(t, raws[r], host["xb"], d, n)) < tol
+            ref = O.matmul_batch(tt[r], raws[r], host["xb"], d, n)
+            assert rel_err(got[:, col:col + d], ref, magnitude(tt[r], raws[r], host["xb"], d, n)) < tol
             col += d
-        ref = O.matmul_batch(t, raws[R.ATTENTION_OUTPUT], host["att"], dim, dim)
-        assert rel_err(acts["xb2"].get().reshape(T, dim), ref, magnitude(t, raws[R.ATTENTION_OUTPUT], host["att"], dim, dim)) < tol
-        gt = O.matmul_batch(t, raws[R.FFN_GATE], host["xb"], ffn, dim)
-        up = O.matmul_batch(t, raws[R.FFN_UP], host["xb"], ffn, dim)
+        ref = O.matmul_batch(tt[R.ATTENTION_OUTPUT], raws[R.ATTENTION_OUTPUT], host["att"], dim, dim)
+        assert rel_err(acts["xb2"].get().reshape(T, dim), ref,
+                       magnitude(tt[R.ATTENTION_OUTPUT], raws[R.ATTENTION_OUTPUT], host["att"], dim, dim)) < tol
+        gt = O.matmul_batch(tt[R.FFN_GATE], raws[R.FFN_GATE], host["xb"], ffn, dim)
+        up = O.matmul_batch(tt[R.FFN_UP], raws[R.FFN_UP], host["xb"], ffn, dim)
         want = O.swiglu(gt.reshape(-1), up.reshape(-1)).reshape(T, ffn)
-        mg, mu = magnitude(t, raws[R.FFN_GATE], host["xb"], ffn, dim), magnitude(t, raws[R.FFN_UP], host["xb"], ffn, dim)
+        mg = magnitude(tt[R.FFN_GATE], raws[R.FFN_GATE], host["xb"], ffn, dim)
+        mu = magnitude(tt[R.FFN_UP], raws[R.FFN_UP], host["xb"], ffn, dim)
         bound = tol * (mg * np.abs(up) + 1.2 * mu * np.abs(gt)) + 1e-6
         assert np.all(np.abs(acts["hb"].get().reshape(T, ffn).astype(np.float64) - want) <= bound)
-        ref = O.matmul_batch(t, raws[R.FFN_DOWN], host["hb_in"], dim, ffn).astype(np.float64) + host["x"]
-        mag = magnitude(t, raws[R.FFN_DOWN], host["hb_in"], dim, ffn) + np.abs(host["x"]) * 1e-6
+        ref = O.matmul_batch(tt[R.FFN_DOWN], raws[R.FFN_DOWN], host["hb_in"], dim, ffn).astype(np.float64) + host["x"]
+        mag = magnitude(tt[R.FFN_DOWN], raws[R.FFN_DOWN], host["hb_in"], dim, ffn) + np.abs(host["x"]) * 1e-6
         assert rel_err(acts["x"].get().reshape(T, dim), ref, mag) < tol
     if residency:
         assert len(inst.copies) == len(steps) and narrow.copies is inst.copies

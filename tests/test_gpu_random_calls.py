@@ -5,7 +5,7 @@ the least size a call accepts.  The reference is a float64 product of the weight
 models decode them (the int8 mode: the oracle's statement of its arithmetic, bit for bit); a call
 the library refuses must leave its outputs alone.  Two bugs of shape dispatch were found this way
 (a fused q|k|v whose first weight was the shortest, a kept copy whose partial sums had no room in
-the workspace): both sit here as ordinary cases of the seeds below."""
+the workspace): both are kept below as cases of their own."""
 import numpy as np
 import pytest
 
@@ -98,7 +98,11 @@ def batched_case(rng):
     resident = rng.random() < 0.4
     tight = bool(resident and rng.random() < 0.3)
     shift = int(rng.choice([0, 0, 0, 1, 2, 3]))
-    return dict(t=t, n=n, batch=batch, active=active, dims=dims, swiglu=swiglu, residual=residual, col_offset=col_offset,
+    # one call in six with more than one weight mixes types (each weight is then decoded by its own)
+    types = [t] * len(dims)
+    if len(dims) > 1 and rng.random() < 0.35:
+        types = [int(rng.choice(MAIN + MINOR)) for _ in dims]
+    return dict(t=t, types=types, n=n, batch=batch, active=active, dims=dims, swiglu=swiglu, residual=residual, col_offset=col_offset,
                 ldo=ldo, xf16=xf16, c_f16=c_f16, resident=resident, tight=tight, shift=shift)
 
 
@@ -108,8 +112,9 @@ def run_batched_case(ctx, c, seed):
     t, n, batch, active, dims, ldo, col_offset = c["t"], c["n"], c["batch"], c["active"], c["dims"], c["ldo"], c["col_offset"]
     swiglu, residual, c_f16 = c["swiglu"], c["residual"], c["c_f16"]
     total = dims[0] if swiglu else sum(dims)
-    raws = [synthetic.weight(t, d, n, seed=seed + i) for i, d in enumerate(dims)]
-    ws = [ctx.load_weight(t, r, d, n) for r, d in zip(raws, dims)]
+    types = c.get("types", [t] * len(dims))
+    raws = [synthetic.weight(ti, d, n, seed=seed + i) for i, (ti, d) in enumerate(zip(types, dims))]
+    ws = [ctx.load_weight(ti, r, d, n) for ti, r, d in zip(types, raws, dims)]
     X = synthetic.activations((batch, n), seed=seed + 7)
     if c["xf16"]:
         X16 = X.astype(np.float16)
@@ -137,7 +142,7 @@ def run_batched_case(ctx, c, seed):
     outside[:active, col_offset:col_offset + total] = False
     assert np.array_equal(a.view(bits)[outside], start.view(bits)[outside]), "wrote outside its rows and columns"
     Xa = X[:active].astype(np.float64)
-    W = [decoded(t, r, d, n) for r, d in zip(raws, dims)]
+    W = [decoded(ti, r, d, n) for ti, r, d in zip(types, raws, dims)]
     prods = [Xa @ w.T for w in W]
     mags = [np.abs(Xa) @ np.abs(w).T for w in W]
     got = a[:active, col_offset:col_offset + total].astype(np.float64)

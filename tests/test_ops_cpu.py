@@ -69,11 +69,15 @@ def test_what_the_library_cannot_run_falls_to_the_next_candidate_or_is_named():
              MatMul(R.ATTENTION_KEY, "b", "k", 256, 256, T, GGMLType.Q4_K),
              MatMul(R.ATTENTION_VALUE, "b", "v", 256, 256, T, GGMLType.Q4_K)]
     assert [c.step.fusion.name for c in ops.split(three, 0, T, [HipImplementation()], Target())] == [PROJECTION.name] * 3
-    # mixed representations in one fused step: refused as a step, taken one projection at a time
+    # mixed representations in one fused step are one call (each weight decoded by its own type,
+    # DequantizingMatMul.java:53-63); weights of different row lengths are not
     mixed = [MatMul(R.FFN_GATE, "xb", "hb", 512, 256, T, GGMLType.Q4_K),
              MatMul(R.FFN_UP, "xb", "hb2", 512, 256, T, GGMLType.Q6_K), SwiGLU("hb", "hb2", "hb")]
+    assert [c.step.fusion.name for c in ops.split(mixed, 0, T, [HipImplementation()], Target())] == [GATE_UP_SWIGLU.name]
+    uneven = [MatMul(R.FFN_GATE, "xb", "hb", 512, 256, T, GGMLType.Q4_K),
+              MatMul(R.FFN_UP, "xb", "hb2", 512, 512, T, GGMLType.Q4_K), SwiGLU("hb", "hb2", "hb")]
     with pytest.raises(RuntimeError, match="no implementation runs SWIGLU"):
-        ops.split(mixed, 0, T, [HipImplementation()], Target())
+        ops.split(uneven, 0, T, [HipImplementation()], Target())
 
 
 def test_needs_is_the_workspace_query_and_counts_residency():
