@@ -163,6 +163,13 @@ int jl_gemv_gate_up(jl_context *ctx, const jl_weight *w1, const jl_weight *w3, c
 
 /* gate[i] = SiLU(gate[i]) * up[i] (siluAndMultiply; the unfused tail of gateUp). */
 int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
+/*
+ * residual[i] += delta[i]: batchedResidualAddFP32 (TransformerBatchPrefillKernels.java:1078-1084), the
+ * prefill plan's "residual add" step where a family runs a task of its own between the down
+ * projection and the add (TensorCoreSteps.java:70-75); a down projection that is followed by its add
+ * directly is one jl_gemm call with JL_RESIDUAL instead.
+ */
+int jl_residual_add(jl_context *ctx, float *residual, const float *delta, int64_t count);
 
 /* ---- the steps on either side of a decode projection ------------------------------------------ */
 

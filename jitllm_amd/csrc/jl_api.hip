@@ -438,6 +438,13 @@ int jl_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count) {
     return jl_launch_swiglu(ctx, gate, up, count);
 }
 
+int jl_residual_add(jl_context *ctx, float *residual, const float *delta, int64_t count) {
+    JL_REQUIRE(ctx && residual && delta && count >= 0 && count <= (int64_t)UINT32_MAX * 256,
+               "jl_residual_add: bad argument");
+    if (!count) return JL_OK;
+    return jl_launch_residual_add(ctx, residual, delta, count);
+}
+
 size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols, int math) {
     if (max_rows <= 0 || cols <= 0 || out_cols < 0) return 0;
     return jl_gemm_workspace_bytes_impl(max_rows, cols, out_cols, math == JL_MATH_DEFAULT ? JL_MATH_F16 : math);

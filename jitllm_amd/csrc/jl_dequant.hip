@@ -68,6 +68,14 @@ jl_swiglu_kernel(float *__restrict__ gate, const float *__restrict__ up, int64_t
     if (i < count) gate[i] = jl_swiglu_value(gate[i], up[i]);
 }
 
+// batchedResidualAddFP32 (J/backend/tornado/kernels/TransformerBatchPrefillKernels.java:1078-1084):
+// residual[i] = residual[i] + delta[i].
+__global__ void __launch_bounds__(256)
+jl_residual_add_kernel(float *__restrict__ residual, const float *__restrict__ delta, int64_t count) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) residual[i] = __fadd_rn(residual[i], delta[i]);
+}
+
 int jl_launch_dequant(jl_context *ctx, const jl_weight *w, float *out) {
     int64_t total = w->rows * w->cols;
     unsigned grid = (unsigned)((total + 255) / 256);
@@ -108,6 +116,13 @@ int jl_launch_fill(jl_context *ctx, float *dst, float value, size_t count) {
 int jl_launch_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count) {
     unsigned grid = (unsigned)((count + 255) / 256);
     hipLaunchKernelGGL(jl_swiglu_kernel, dim3(grid), dim3(256), 0, ctx->stream, gate, up, count);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
+}
+
+int jl_launch_residual_add(jl_context *ctx, float *residual, const float *delta, int64_t count) {
+    unsigned grid = (unsigned)((count + 255) / 256);
+    hipLaunchKernelGGL(jl_residual_add_kernel, dim3(grid), dim3(256), 0, ctx->stream, residual, delta, count);
     JL_HIP(hipGetLastError());
     return JL_OK;
 }

@@ -144,6 +144,7 @@ int jl_launch_gemv_argmax(jl_context *ctx, const jl_weight *w, const float *x, c
 int jl_static_scratch_init(int device);
 int jl_launch_argmax_static(jl_context *ctx, const float *values, int64_t n, int32_t *index);
 int jl_launch_swiglu(jl_context *ctx, float *gate, const float *up, int64_t count);
+int jl_launch_residual_add(jl_context *ctx, float *residual, const float *delta, int64_t count);
 int jl_launch_fill(jl_context *ctx, float *dst, float value, size_t count);
 // A caller-owned fp16 copy of one projection's weights that outlives the call: decoded when
 // *state does not name the layout the call needs (0 = empty), reused otherwise.

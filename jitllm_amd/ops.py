@@ -39,6 +39,8 @@ class TensorRole(enum.Enum):
     FFN_GATE = "FFN_GATE"
     FFN_UP = "FFN_UP"
     FFN_DOWN = "FFN_DOWN"
+    ATTENTION_NORM = "ATTENTION_NORM"
+    FFN_NORM = "FFN_NORM"
 
 
 @dataclass(frozen=True)
@@ -80,9 +82,22 @@ class ResidualAdd:
 
 @dataclass(frozen=True)
 class RmsNorm:
+    """``output = input / rms(input) * weight`` over rows of ``groupLength`` values
+    (J/program/op/RmsNorm.java:44-60).  ``weight`` is the role of the learned scale, None for the
+    unweighted form; ``groups`` above 1 is the per-head form."""
     input: str
     output: str
+    weight: Optional[TensorRole] = None
+    epsilon: float = 1e-5
+    groupLength: int = 0
+    groups: int = 1
     kind = OperationKind.RMS_NORM
+
+    def __post_init__(self):
+        if self.groups < 1:
+            raise ValueError(f"groups must be at least 1: {self.groups}")
+        if self.groups > 1 and self.groupLength < 1:
+            raise ValueError(f"a norm over {self.groups} groups must state the group length")
 
 
 @dataclass(frozen=True)
@@ -121,8 +136,7 @@ class Fusion:
         return len(inputs) <= 1
 
 
-# The tensor-core fusion table (J/backend/tornado/ops/TensorCoreSteps.java:44-78), the entries this
-# library has kernels for.  The norms and the bare residual add stay with the next candidate.
+# The tensor-core fusion table (J/backend/tornado/ops/TensorCoreSteps.java:44-78), longest first.
 QKV = Fusion.of("q|k|v", OperationKind.MAT_MUL, OperationKind.MAT_MUL, OperationKind.MAT_MUL).when(Fusion.sameInput)
 GATE_UP_SWIGLU = Fusion.of("gate|up + SwiGLU", OperationKind.MAT_MUL, OperationKind.MAT_MUL,
                            OperationKind.SWIGLU).when(Fusion.sameInput)
@@ -131,7 +145,15 @@ DOWN_ADD = Fusion.of("down + residual add", OperationKind.MAT_MUL, OperationKind
 GATE_UP = Fusion.of("gate|up", OperationKind.MAT_MUL, OperationKind.MAT_MUL).when(Fusion.sameInput).when(
     lambda ops: ops[0].weight == TensorRole.FFN_GATE and ops[1].weight == TensorRole.FFN_UP)
 PROJECTION = Fusion.of("projection", OperationKind.MAT_MUL)
-FUSIONS = [QKV, GATE_UP_SWIGLU, DOWN_ADD, GATE_UP, PROJECTION]
+ADD_NORM = Fusion.of("residual add + RMS norm", OperationKind.RESIDUAL_ADD, OperationKind.RMS_NORM)
+NORM = Fusion.of("RMS norm", OperationKind.RMS_NORM)
+RESIDUAL = Fusion.of("residual add", OperationKind.RESIDUAL_ADD)
+FUSIONS = [QKV, GATE_UP_SWIGLU, ADD_NORM, DOWN_ADD, GATE_UP, PROJECTION, NORM, RESIDUAL]
+
+
+def scaleOf(norm: RmsNorm) -> str:
+    """The name of a norm's row-scale buffer: its output's name and ".scale" (TensorCoreSteps.java:291-294)."""
+    return norm.output + ".scale"
 
 
 @dataclass(frozen=True)
@@ -275,6 +297,15 @@ class HipImplementation(Implementation):
         if not target.hip():
             return False
         mm = step.matMuls()
+        name = step.fusion.name
+        if name in (NORM.name, ADD_NORM.name):
+            # the norm that feeds a GEMM its fp16 rows: one group over the row, a learned scale
+            norm = step.first(RmsNorm)
+            if norm.weight is None or norm.groups != 1 or norm.groupLength <= 0:
+                return False
+            return name == NORM.name or step.first(ResidualAdd).residual == norm.input
+        if name == RESIDUAL.name:
+            return True
         if not mm or len(mm) > 8:
             return False
         if any(m.dataType not in SUPPORTED for m in mm):
@@ -291,6 +322,7 @@ class HipImplementation(Implementation):
         return True
 
     def needs(self, steps: Sequence[Step], target: Target) -> BatchPrefillWorkspace:
+        steps = [s for s in steps if s.matMuls()]      # the norms and adds need no scratch
         if not steps:
             return BatchPrefillWorkspace.withoutResidencyChoice(0)
         rows, cols, widest = _sizes(steps)
@@ -306,6 +338,8 @@ class HipImplementation(Implementation):
         if prepacking is not None:
             raise RuntimeError("the hip implementation reads the file's blocks, not prepacked tiles")
         need = self.needs(steps, target)
+        if not steps:
+            raise ValueError("an instance runs at least one step")
         return HipInstance(context, max(s.tokens for s in steps), DeviceBuffer(context, max(need.bytes, 256)),
                            self.residency, ResidentCopies(context))
 
@@ -324,6 +358,7 @@ class HipInstance(Instance):
         self.residency = residency
         self.copies = copies
         self._lib = context._lib
+        self._producers: Dict[str, MatMul] = {}     # output name -> the projection that wrote it
 
     def buffers(self) -> list:
         return [self.workspace] + self.copies.buffers()
@@ -333,17 +368,42 @@ class HipInstance(Instance):
         array (the reference's packed rows, DecodedMatMul.java:93-109), gate|up + SwiGLU writes the
         SwiGLU's output, down + residual add accumulates into the residual."""
         mm = step.matMuls()
+        name = step.fusion.name
+        if step.tokens > self.batchSize:
+            raise ValueError(f"a step of {step.tokens} tokens in an instance built for {self.batchSize}")
+        if name in (NORM.name, ADD_NORM.name):
+            # RMS norm into the fp16 input of the next GEMM, the row scales kept beside it; with a
+            # residual add in front, the add runs inside the same launch (TensorCoreSteps.norm,
+            # TensorCoreSteps.java:209-277: batchedRmsReduceParallel / batchedRmsReduceFusedResidual,
+            # then batchedRmsApplyFP16 / batchedFFNRmsApplyFP16)
+            norm = step.first(RmsNorm)
+            delta = operands.activation(step.first(ResidualAdd).input) if name == ADD_NORM.name else None
+            out = operands.activation(norm.output)
+            if not isinstance(out, HalfFloatArray):
+                raise ValueError(f"the norm's output {norm.output} is the next GEMM's fp16 input")
+            L.check(self._lib.jl_rms_apply_xf16(
+                self.context.handle, operands.activation(norm.input).ptr, delta.ptr if delta is not None else None,
+                operands.weight(norm.weight, step.layer).ptr, norm.epsilon, step.tokens, norm.groupLength,
+                operands.activation(scaleOf(norm)).ptr, out.ptr))
+            return
+        if name == RESIDUAL.name:
+            # x += down on its own: it follows the down projection (TensorCoreSteps.java:145-153)
+            add = step.first(ResidualAdd)
+            down = self._producers.get(add.input)
+            if down is None or down.weight != TensorRole.FFN_DOWN:
+                raise ValueError(f"a residual add on its own follows the down projection, not {add.input}")
+            L.check(self._lib.jl_residual_add(self.context.handle, operands.activation(add.residual).ptr,
+                                              operands.activation(add.input).ptr, step.tokens * down.rows))
+            return
         weights = [operands.weight(m.weight, step.layer) for m in mm]
         x = operands.activation(mm[0].input)
-        name = step.fusion.name
+        self._producers[mm[0].output] = mm[0]
         if name == GATE_UP_SWIGLU.name:
             out, epilogue, ldo = operands.activation(step.first(SwiGLU).output), L.JL_SWIGLU, mm[0].rows
         elif name == DOWN_ADD.name:
             out, epilogue, ldo = operands.activation(step.first(ResidualAdd).residual), L.JL_RESIDUAL, mm[0].rows
         else:
             out, epilogue, ldo = operands.activation(mm[0].output), L.JL_STORE, step.outputWidth()
-        if step.tokens > self.batchSize:
-            raise ValueError(f"a step of {step.tokens} tokens in an instance built for {self.batchSize}")
         arr = (C.c_void_p * len(weights))(*[w.handle for w in weights])
         copy, state = None, None
         if self.residency:

@@ -213,6 +213,110 @@ def test_plugin_instance_takes_the_references_operand_types(ctx):
     assert rel_err(acts["x"].get().reshape(T, dim), ref, mag) < F16_BOUND
 
 
+def test_plugin_instance_runs_the_whole_layer_plan(ctx):
+    """Every step of the reference's tensor-core table through the plugin mirror, in a Llama layer's
+    order: RMS norm -> q|k|v, o projection, residual add + RMS norm -> gate|up + SwiGLU, down +
+    residual add (TensorCoreSteps.java:44-78, 133-169), and the bare residual add behind a down
+    projection.  The norms are held to the oracle bit for bit (fp16 rows and row scales), the
+    projections to the oracle on exactly the fp16 rows the device holds."""
+    from jitllm_amd import ops, synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.ops import (ADD_NORM, DOWN_ADD, GATE_UP_SWIGLU, NORM, PROJECTION, QKV, RESIDUAL, HipImplementation,
+                                MatMul, ResidualAdd, RmsNorm, Step, SwiGLU, Target, TensorRole as R)
+    say("whole layer plan")
+    t, T, dim, kv, ffn, eps = O.Q4_K, 200, 512, 256, 1536, 1e-5
+    g = GGMLType(t)
+    shapes = {R.ATTENTION_QUERY: (dim, dim), R.ATTENTION_KEY: (kv, dim), R.ATTENTION_VALUE: (kv, dim),
+              R.ATTENTION_OUTPUT: (dim, dim), R.FFN_GATE: (ffn, dim), R.FFN_UP: (ffn, dim), R.FFN_DOWN: (dim, ffn)}
+    raws = {r: synthetic.weight(g, d, n, seed=1770 + i) for i, (r, (d, n)) in enumerate(shapes.items())}
+    tensors = {r: ctx.load_weight(g, raws[r], *shapes[r]) for r in shapes}
+    norm_w = {R.ATTENTION_NORM: np.random.default_rng(1780).uniform(0.5, 1.5, dim).astype(np.float32),
+              R.FFN_NORM: np.random.default_rng(1781).uniform(0.5, 1.5, dim).astype(np.float32)}
+    tensors.update({r: ctx.from_numpy(w) for r, w in norm_w.items()})
+    down = MatMul(R.FFN_DOWN, "hb", "xb2", dim, ffn, T, g)
+    program = [
+        RmsNorm("x", "xb", R.ATTENTION_NORM, eps, dim),
+        MatMul(R.ATTENTION_QUERY, "xb", "qkv", dim, dim, T, g), MatMul(R.ATTENTION_KEY, "xb", "k", kv, dim, T, g),
+        MatMul(R.ATTENTION_VALUE, "xb", "v", kv, dim, T, g),
+        MatMul(R.ATTENTION_OUTPUT, "att", "xb2", dim, dim, T, g),
+        ResidualAdd("x", "xb2"), RmsNorm("x", "xb", R.FFN_NORM, eps, dim),
+        MatMul(R.FFN_GATE, "xb", "hb", ffn, dim, T, g), MatMul(R.FFN_UP, "xb", "hb2", ffn, dim, T, g),
+        SwiGLU("hb", "hb2", "hb"),
+        down, ResidualAdd("x", "xb2"),
+    ]
+    impl = HipImplementation()
+    chosen = ops.split(program, 0, T, [impl], Target())
+    assert [c.step.fusion.name for c in chosen] == [NORM.name, QKV.name, PROJECTION.name, ADD_NORM.name,
+                                                    GATE_UP_SWIGLU.name, DOWN_ADD.name]
+    steps = [c.step for c in chosen]
+    x0 = synthetic.activations((T, dim), 1790) * np.float32(1.7)
+    att = half_activations((T, dim), 1791)
+    acts = {"x": ctx.from_numpy(x0), "xb": ctx.half_array(T * dim), "xb.scale": ctx.float_array(T, fill=UNTOUCHED),
+            "att": ctx.half_from_numpy(att), "xb2": ctx.float_array(T * dim), "qkv": ctx.float_array(T * (dim + 2 * kv)),
+            "hb": ctx.half_array(T * ffn)}
+    operands = ops.Operands(acts, lambda role, layer: tensors[role])
+    inst = impl.create(steps, Target(), ctx)
+
+    def held_to(name, got, raw_role, X32):
+        d, n = shapes[raw_role]
+        assert rel_err(got, O.matmul_batch(t, raws[raw_role], X32, d, n), magnitude(t, raws[raw_role], X32, d, n)) < F16_BOUND, name
+
+    # RMS norm -> q|k|v
+    inst.emit(steps[0], operands)
+    inst.emit(steps[1], operands)
+    ctx.sync()
+    want_scale, want_xb = O.batched_rms_apply_f16(x0, norm_w[R.ATTENTION_NORM], eps)
+    xb = acts["xb"].get().reshape(T, dim)
+    assert np.array_equal(xb.view(np.uint16), want_xb.view(np.uint16))
+    assert np.array_equal(acts["xb.scale"].get().view(np.uint32), want_scale.view(np.uint32))
+    assert np.array_equal(acts["x"].get().reshape(T, dim), x0)          # a norm on its own only reads x
+    qkv = acts["qkv"].get().reshape(T, dim + 2 * kv)
+    col = 0
+    for r in (R.ATTENTION_QUERY, R.ATTENTION_KEY, R.ATTENTION_VALUE):
+        held_to(r, qkv[:, col:col + shapes[r][0]], r, xb.astype(np.float32))
+        col += shapes[r][0]
+    # o projection, then the residual add inside the next norm
+    inst.emit(steps[2], operands)
+    ctx.sync()
+    xb2 = acts["xb2"].get().reshape(T, dim)
+    held_to("o", xb2, R.ATTENTION_OUTPUT, att.astype(np.float32))
+    inst.emit(steps[3], operands)
+    ctx.sync()
+    x1 = x0 + xb2
+    assert np.array_equal(acts["x"].get().reshape(T, dim).view(np.uint32), x1.view(np.uint32))
+    want_scale, want_xb = O.batched_rms_apply_f16(x1, norm_w[R.FFN_NORM], eps)
+    xb = acts["xb"].get().reshape(T, dim)
+    assert np.array_equal(xb.view(np.uint16), want_xb.view(np.uint16))
+    assert np.array_equal(acts["xb.scale"].get().view(np.uint32), want_scale.view(np.uint32))
+    # gate|up + SwiGLU into the fp16 hidden rows, down + residual add
+    inst.emit(steps[4], operands)
+    inst.emit(steps[5], operands)
+    ctx.sync()
+    xb32 = xb.astype(np.float32)
+    hb = acts["hb"].get().reshape(T, ffn)
+    gt, up = O.matmul_batch(t, raws[R.FFN_GATE], xb32, ffn, dim), O.matmul_batch(t, raws[R.FFN_UP], xb32, ffn, dim)
+    want = O.swiglu(gt.reshape(-1), up.reshape(-1)).reshape(T, ffn)
+    mg, mu = magnitude(t, raws[R.FFN_GATE], xb32, ffn, dim), magnitude(t, raws[R.FFN_UP], xb32, ffn, dim)
+    assert np.all(np.abs(hb.astype(np.float64) - want) <= F16_BOUND * (mg * np.abs(up) + 1.2 * mu * np.abs(gt))
+                  + np.abs(want) * 2.0 ** -11 + 1e-6)
+    hb32 = hb.astype(np.float32)
+    ref = O.matmul_batch(t, raws[R.FFN_DOWN], hb32, dim, ffn).astype(np.float64) + x1
+    mag = magnitude(t, raws[R.FFN_DOWN], hb32, dim, ffn) + np.abs(x1) * 1e-6
+    x2 = acts["x"].get().reshape(T, dim)
+    assert rel_err(x2, ref, mag) < F16_BOUND
+    # the down projection and its residual add as two steps (a family with a task of its own between them)
+    inst.emit(Step(0, T, PROJECTION, (down,)), operands)
+    inst.emit(Step(0, T, RESIDUAL, (ResidualAdd("x", "xb2"),)), operands)
+    ctx.sync()
+    assert np.array_equal(acts["x"].get().reshape(T, dim).view(np.uint32),
+                          (x2 + acts["xb2"].get().reshape(T, dim)).view(np.uint32))
+    # ... and a bare add that follows anything else is refused by name
+    inst.emit(Step(0, T, PROJECTION, (MatMul(R.ATTENTION_OUTPUT, "att", "xb2", dim, dim, T, g),)), operands)
+    with pytest.raises(ValueError, match="follows the down projection, not xb2"):
+        inst.emit(Step(0, T, RESIDUAL, (ResidualAdd("x", "xb2"),)), operands)
+    ctx.sync()
+
+
 def test_xf16_refusals(ctx):
     from jitllm_amd import _lib as L, synthetic
     from jitllm_amd.projections import QuantizedBatchProjections

@@ -5,23 +5,25 @@ import pytest
 from jitllm_amd import _lib as L
 from jitllm_amd import ops
 from jitllm_amd.ggml import GGMLType
-from jitllm_amd.ops import (DOWN_ADD, GATE_UP_SWIGLU, PROJECTION, QKV, HipImplementation, MatMul, OperationKind,
-                            ResidualAdd, RmsNorm, Step, SwiGLU, Target, TensorRole)
+from jitllm_amd.ops import (ADD_NORM, DOWN_ADD, GATE_UP_SWIGLU, NORM, PROJECTION, QKV, RESIDUAL, HipImplementation, MatMul,
+                            OperationKind, ResidualAdd, RmsNorm, Step, SwiGLU, Target, TensorRole)
 
 DIM, KV, FFN, T = 2048, 512, 8192, 512
 
 
-def llama_layer(t=GGMLType.Q8_0, dim=DIM):
-    """The operations of one Llama layer around attention, in program order."""
+def llama_layer(t=GGMLType.Q8_0, dim=DIM, weighted=True):
+    """The operations of one Llama layer around attention, in program order (``weighted`` false: the
+    norms without a learned scale, which the library has no kernel for)."""
     R = TensorRole
+    att, ffn = (R.ATTENTION_NORM, R.FFN_NORM) if weighted else (None, None)
     return [
-        RmsNorm("x", "xb"),
+        RmsNorm("x", "xb", att, 1e-5, dim),
         MatMul(R.ATTENTION_QUERY, "xb", "q", dim, dim, T, t),
         MatMul(R.ATTENTION_KEY, "xb", "k", KV, dim, T, t),
         MatMul(R.ATTENTION_VALUE, "xb", "v", KV, dim, T, t),
         MatMul(R.ATTENTION_OUTPUT, "att", "xb2", dim, dim, T, t),
         ResidualAdd("x", "xb2"),
-        RmsNorm("x", "xb"),
+        RmsNorm("x", "xb", ffn, 1e-5, dim),
         MatMul(R.FFN_GATE, "xb", "hb", FFN, dim, T, t),
         MatMul(R.FFN_UP, "xb", "hb2", FFN, dim, T, t),
         SwiGLU("hb", "hb2", "hb"),
@@ -44,8 +46,16 @@ class JitNorms(ops.Implementation):
 def test_the_first_accepting_candidate_takes_each_step():
     chosen = ops.split(llama_layer(), 3, T, [HipImplementation(), JitNorms()], Target())
     got = [(c.implementation.library(), c.step.fusion.name) for c in chosen]
-    assert got == [("none", "RMS norm"), ("hip", QKV.name), ("hip", PROJECTION.name), ("none", "residual add"),
+    # the reference's own split of a Llama layer: the residual add after attention is merged into
+    # the next RMS norm (DecodedMatMul.java:31-35)
+    assert got == [("hip", NORM.name), ("hip", QKV.name), ("hip", PROJECTION.name), ("hip", ADD_NORM.name),
+                   ("hip", GATE_UP_SWIGLU.name), ("hip", DOWN_ADD.name)]
+    # norms without a learned scale stay with the next candidate; the bare add is the library's
+    chosen = ops.split(llama_layer(weighted=False), 3, T, [HipImplementation(), JitNorms()], Target())
+    got = [(c.implementation.library(), c.step.fusion.name) for c in chosen]
+    assert got == [("none", "RMS norm"), ("hip", QKV.name), ("hip", PROJECTION.name), ("hip", RESIDUAL.name),
                    ("none", "RMS norm"), ("hip", GATE_UP_SWIGLU.name), ("hip", DOWN_ADD.name)]
+    chosen = ops.split(llama_layer(), 3, T, [HipImplementation(), JitNorms()], Target())
     qkv = chosen[1].step
     assert qkv.outputWidth() == DIM + 2 * KV and qkv.weights() == DIM * (DIM + 2 * KV)
     assert [m.weight for m in qkv.matMuls()] == [TensorRole.ATTENTION_QUERY, TensorRole.ATTENTION_KEY,
@@ -58,7 +68,14 @@ def test_what_the_library_cannot_run_falls_to_the_next_candidate_or_is_named():
     assert all(c.implementation.library() == "none" for c in chosen if c.step.matMuls()
                and c.step.matMuls()[0].columns == 2080)
     with pytest.raises(RuntimeError, match=r"no implementation runs RMS_NORM in layer 7 \(ffn\)"):
-        ops.split(llama_layer(), 7, T, [HipImplementation()], Target(), region="ffn")
+        ops.split(llama_layer(weighted=False), 7, T, [HipImplementation()], Target(), region="ffn")
+    # a per-head norm (Qwen3's query / key norms) is not the row norm the library runs
+    per_head = [RmsNorm("q", "q", TensorRole.ATTENTION_NORM, 1e-6, 128, groups=16)]
+    with pytest.raises(RuntimeError, match="no implementation runs RMS_NORM"):
+        ops.split(per_head, 0, T, [HipImplementation()], Target())
+    # an add in front of a norm of some other array is two steps, not the fused one
+    apart = [ResidualAdd("y", "xb2"), RmsNorm("x", "xb", TensorRole.FFN_NORM, 1e-5, DIM)]
+    assert [c.step.fusion.name for c in ops.split(apart, 0, T, [HipImplementation()], Target())] == [RESIDUAL.name, NORM.name]
     # native libraries switched off (--no-native-libraries), or no matrix cores: never claimed
     for target in (Target(nativeLibraries=False), Target(capabilities=frozenset())):
         chosen = ops.split(llama_layer(), 0, T, [HipImplementation(), JitNorms()], target)
