@@ -181,6 +181,16 @@ int jl_residual_add(jl_context *ctx, float *residual, const float *delta, int64_
  * so its last bits may differ from the host's sequential sum.
  */
 int jl_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale);
+/*
+ * xb[i] = rms_weights[i] * (rms_scale[0] * x[i]), both products rounded to fp32: the second phase of
+ * the unfused normalisation, reductionOneBlock2WithLayer
+ * (J/backend/tornado/kernels/TransformerComputeKernelsLayered.java:570-580), which
+ * QuantizedProjections.rmsApply dispatches where the projections are not packed
+ * (QuantizedProjections.java:117-130).  For the steps that have no RMS-folding launch -- projections
+ * over Q6_K, Q5_K, Q4_1, Q5_0 and IQ4_XS weights, row lengths the folding kernels refuse.  xb may be x.
+ */
+int jl_rms_apply(jl_context *ctx, const float *x, const float *rms_weights, const float *rms_scale, int64_t n,
+                 float *xb);
 
 /*
  * The projections above with the RMS normalisation of x folded into the activation load:

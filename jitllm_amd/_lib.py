@@ -48,6 +48,7 @@ SYMBOLS = {
     "jl_swiglu": (C.c_int, [vp, vp, vp, i64]),
     "jl_residual_add": (C.c_int, [vp, vp, vp, i64]),
     "jl_rms_scale": (C.c_int, [vp, vp, i64, C.c_float, vp]),
+    "jl_rms_apply": (C.c_int, [vp, vp, vp, vp, i64, vp]),
     "jl_gemv_rms": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp, C.c_int]),
     "jl_gemv_qkv_rms": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_float, vp, vp, vp]),
     "jl_gemv_gate_up_rms": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp]),

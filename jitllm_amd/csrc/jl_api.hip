@@ -315,6 +315,13 @@ int jl_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *s
     return jl_launch_rms_scale(ctx, x, n, eps, scale);
 }
 
+int jl_rms_apply(jl_context *ctx, const float *x, const float *rms_weights, const float *rms_scale, int64_t n,
+                 float *xb) {
+    JL_REQUIRE(ctx && x && rms_weights && rms_scale && xb && n > 0 && n <= (int64_t)UINT32_MAX * 256,
+               "jl_rms_apply: bad argument");
+    return jl_launch_rms_apply(ctx, x, rms_weights, rms_scale, n, xb);
+}
+
 int jl_gemv_rms(jl_context *ctx, const jl_weight *w, const float *x, const float *rms_weights,
                 const float *rms_scale, float eps, float *out, int epilogue) {
     JL_REQUIRE(ctx && w && x && rms_weights && out, "jl_gemv_rms: null argument");

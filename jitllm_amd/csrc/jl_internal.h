@@ -133,6 +133,8 @@ int jl_launch_gemv_direct(jl_context *ctx, const jl_weight *w, const jl_weight *
                           int epilogue);
 int jl_launch_dequant_direct(jl_context *ctx, const jl_weight *w, float *out);
 int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale);
+int jl_launch_rms_apply(jl_context *ctx, const float *x, const float *rms_w, const float *rms_scale, int64_t n,
+                        float *xb);
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
 // out = w . x (rms set: the normalisation folded in) and index[0] = the first maximum of out.
 int jl_launch_gemv_argmax(jl_context *ctx, const jl_weight *w, const float *x, const jl_rms *rms, float *out,

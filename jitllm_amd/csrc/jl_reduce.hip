@@ -181,7 +181,25 @@ jl_quantize_q8_kernel(const float *__restrict__ x, const float *__restrict__ rms
     }
 }
 
+// reductionOneBlock2WithLayer (J/backend/tornado/kernels/TransformerComputeKernelsLayered.java:570-580),
+// the second phase of the unfused normalisation: output[i] = weights[i] * (ss * x[i]), both products
+// rounded to fp32.
+__global__ void __launch_bounds__(256)
+jl_rms_apply_kernel(const float *__restrict__ x, const float *__restrict__ rms_w, const float *__restrict__ rms_scale,
+                    float *__restrict__ xb, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) xb[i] = jl_mul_rn(rms_w[i], jl_mul_rn(rms_scale[0], x[i]));
+}
+
 }  // namespace
+
+int jl_launch_rms_apply(jl_context *ctx, const float *x, const float *rms_w, const float *rms_scale, int64_t n,
+                        float *xb) {
+    hipLaunchKernelGGL(jl_rms_apply_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, x, rms_w,
+                       rms_scale, xb, n);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
+}
 
 int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, float *scale) {
     hipLaunchKernelGGL(jl_rms_scale_kernel, dim3(1), dim3(kThreads), 0, ctx->stream, x, n, eps, scale);

@@ -83,6 +83,16 @@ class QuantizedProjections:
             raise RuntimeError("the packed path needs ws.packedX bound to a PackedActivation of the row length")
         L.check(self._lib.jl_quantize_q8(self.context.handle, x.ptr, n, px.quants.ptr, px.scales.ptr, px.sums.ptr))
 
+    def rmsApply(self, rmsWeights: FloatArray, temp: FloatArray, n: int) -> None:
+        """``wrapXb = rmsWeights * (temp[0] * wrapX)``, quantised as well where the projections are
+        packed (QuantizedProjections.rmsApply, QuantizedProjections.java:117-130: reductionOneBlock2WithLayer,
+        or PackedActivationTasks.rmsApplyAndQuantize).  ``temp`` is the scalar ``rmsScale`` leaves."""
+        if self.packed():
+            self.rmsApplyAndQuantize(self.ws.wrapX, rmsWeights, temp, n)
+            return
+        L.check(self._lib.jl_rms_apply(self.context.handle, self.ws.wrapX.ptr, rmsWeights.ptr, temp.ptr, n,
+                                       self.ws.wrapXb.ptr))
+
     def rmsApplyAndQuantize(self, x: FloatArray, rmsWeights: FloatArray, rmsScale: FloatArray, n: int) -> None:
         """``wrapXb = rmsWeights * (rmsScale[0] * x)`` and ``packedX`` = its Q8 blocks, in one launch
         (QuantizedProjections.rmsApply, QuantizedProjections.java:117-121 ->

@@ -719,6 +719,36 @@ def test_argmax_ties_and_edges(ctx, n):
         assert int(token.download(np.int32, 1)[0]) == O.argmax(v)
 
 
+@pytest.mark.parametrize("t,d,n", [(O.Q6_K, 1000, 4096), (O.Q5_K, 264, 2048), (O.IQ4_XS, 96, 256), (O.Q8_0, 16, 96)])
+def test_unfused_normalisation_in_front_of_a_projection(ctx, t, d, n):
+    """Where there is no RMS-folding launch -- the minor types, a row length the folding kernels
+    refuse -- the layer runs the reference's unfused steps: rmsScale (reductionOneBlockWithLayer),
+    rmsApply (reductionOneBlock2WithLayer: wrapXb = w * (ss * wrapX), two fp32 roundings) and matvec.
+    The apply step is held bit for bit to that formula on the device's own scale, the projection to
+    the host's rmsnorm + matVec."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("unfused rms", KQ_NAMES.get(t, t), d, n)
+    raw = synthetic.weight(t, d, n, seed=3400 + d)
+    x = synthetic.activations(n, seed=3401) * np.float32(2.0)
+    rw = (1.0 + 0.25 * synthetic.activations(n, seed=3402)).astype(np.float32)
+    w = upload(ctx, t, raw, d, n)
+    ws = TornadoWorkspace(wrapX=ctx.from_numpy(x), wrapXb=ctx.float_array(n + 8, fill=POISON))
+    proj = QuantizedProjections(ctx, ws)
+    scale, out = ctx.float_array(1, fill=POISON), ctx.float_array(d, fill=POISON)
+    proj.rmsScale(ws.wrapX, n, 1e-5, scale)
+    proj.rmsApply(ctx.from_numpy(rw), scale, n)
+    proj.matvec(out, w, n, d)
+    ctx.sync()
+    ss = scale.get()[0]
+    xb = ws.wrapXb.get()
+    assert np.all(xb[n:] == POISON)
+    assert bits_equal(xb[:n], rw * (ss * x))
+    assert np.array_equal(ws.wrapX.get(), x)
+    xn = O.rmsnorm(x, rw, 1e-5)
+    assert rel_err(out.get(), O.matmul(t, raw, xn, d, n), magnitude(t, raw, xn, d, n)) < 2e-5
+
+
 def test_rms_folding_refuses_what_it_has_no_kernel_for(ctx):
     """A row length the tile kernel does not take is refused by name, never normalised some other
     way (the caller then runs the unfused sequence, as the reference does)."""
