@@ -297,3 +297,46 @@ def test_q8_0_prefill_qkv_and_o(ctx, T):
         col += d
     for w in ws:
         w.free()
+
+
+# ---- a weight past 2 GiB ---------------------------------------------------------------------------
+
+def test_a_weight_of_more_than_two_gib(ctx):
+    """Q8_0 140000 x 16384 is 2.44e9 bytes: byte offsets into it do not fit 32 bits.  The single-token
+    projection, batched decode (8 and 40 rows), a mid row count (200) and prefill (600 rows, a 4.9 GB
+    fp16 copy in the workspace) over it, held to the oracle on the first and last rows, a random
+    sample and the rows on either side of the 2^31-byte mark; every output is written."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections, QuantizedProjections, TornadoWorkspace
+    t, d, n = O.Q8_0, 140000, 16384
+    say("a weight past 2 GiB", d, n)
+    part = synthetic.weight(t, 20000, n, seed=31)
+    rb = row_bytes(t, n)
+    raw = np.concatenate([np.roll(part.reshape(20000, rb), i, axis=0).reshape(-1) for i in range(7)])
+    assert raw.size > 2 ** 31
+    mark = 2 ** 31 // rb
+    rows = np.unique(np.concatenate([sample_rows(d, 64, 32), np.arange(mark - 4, mark + 4)]))
+    sub = gather(raw, t, n, rows)
+    w = ctx.load_weight(t, raw, d, n)
+    del raw
+    x = synthetic.activations(n, seed=33)
+    out = ctx.float_array(d, fill=POISON)
+    QuantizedProjections(ctx, TornadoWorkspace()).floatMatvec(ctx.from_numpy(x), out, w, n, d)
+    ctx.sync()
+    got = out.get()
+    assert np.all(got != POISON)
+    assert rel_err(got[rows], O.matmul(t, sub, x, rows.size, n), magnitude(t, sub, x, rows.size, n)) < 2e-5
+    out.free()
+    for B in (8, 40, 200, 600):
+        say("a weight past 2 GiB, rows", B)
+        X = synthetic.activations((B, n), seed=34 + B)
+        proj = QuantizedBatchProjections(ctx, B, n, d)
+        o = ctx.float_array(B * d, fill=POISON)
+        proj.projection(ctx.from_numpy(X), o, w, n, d, False)
+        ctx.sync()
+        g = o.get().reshape(B, d)
+        assert np.all(g != POISON)
+        assert rel_err(g[:, rows], O.matmul_batch(t, sub, X, rows.size, n), magnitude(t, sub, X, rows.size, n)) < 2e-3
+        o.free()
+        proj.workspace.free()
+    w.free()
