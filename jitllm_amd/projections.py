@@ -314,15 +314,14 @@ class QuantizedBatchProjections:
 
     def gateUp(self, x: FloatArray, hb: FloatArray, w1: TornadoTensor, w3: TornadoTensor, dim: int,
                hidDim: int, activeRows: int | None = None) -> None:
-        """``hb = SiLU(w1 . x) * (w3 . x)`` over the batch (QuantizedBatchProjections.java:329-458;
+        """``hb = SiLU(w1 . x) * (w3 . x)`` over the batch, for every pair of weight types
+        (QuantizedBatchProjections.java:329-458;
         the RMS norm the reference folds in front is not part of this path: ``x`` is already
         normalised)."""
         _check_shape(w1, dim, hidDim)
         _check_shape(w3, dim, hidDim)
-        if not self.fusedGateUp(w1, w3):
-            raise L.UnsupportedProjection(
-                L.JL_ERR_UNSUPPORTED,
-                f"no fused batched gate/up kernel for a {w1.data_type().name} gate and a "
-                f"{w3.data_type().name} up weight")
+        # Where fusedGateUp does not hold the reference runs gate into wrapHbBatch, up into
+        # ffnUpResult and siluAndMultiply (:446-457); jl_gemm takes any pair of types the library
+        # decodes -- equal or not -- with the SwiGLU as its epilogue, so it is one call either way.
         rows = self.batchSize if activeRows is None else activeRows
         self._gemm([w1, w3], x, hb, rows, hidDim, 0, L.JL_SWIGLU)

@@ -866,15 +866,16 @@ def test_weights_of_different_types_side_by_side(ctx, rows, resident):
     for t, raw, d in zip(types, raws, dims):
         assert rel_err(got[:, col:col + d], O.matmul_batch(t, raw, X, d, n), magnitude(t, raw, X, d, n)) < F16_BOUND
         col += d
-    # gate / up of different types
+    # gate / up of different types: not a pair the reference fuses, one call here all the same
     d = 520
     r1, r3 = synthetic.weight(O.Q5_0, d, n, seed=9710), synthetic.weight(O.IQ4_XS, d, n, seed=9711)
     g, u = O.matmul_batch(O.Q5_0, r1, X, d, n), O.matmul_batch(O.IQ4_XS, r3, X, d, n)
     ref = O.swiglu(g.reshape(-1), u.reshape(-1)).reshape(rows, d)
     hb = ctx.float_array(rows * d + 64, fill=UNTOUCHED)
-    QuantizedBatchProjections(ctx, rows, n, 2 * d, resident=resident)._gemm(
-        [ctx.load_weight(O.Q5_0, r1, d, n), ctx.load_weight(O.IQ4_XS, r3, d, n)], ctx.from_numpy(X), hb, rows, d, 0,
-        L.JL_SWIGLU)
+    pair = QuantizedBatchProjections(ctx, rows, n, 2 * d, resident=resident)
+    w1, w3 = ctx.load_weight(O.Q5_0, r1, d, n), ctx.load_weight(O.IQ4_XS, r3, d, n)
+    assert not pair.fusedGateUp(w1, w3)
+    pair.gateUp(ctx.from_numpy(X), hb, w1, w3, n, d)
     ctx.sync()
     flat = hb.get()
     assert np.all(flat[rows * d:] == UNTOUCHED)
