@@ -668,6 +668,45 @@ def bench_batched(ctx, hip, B, steps, warmup, cpu, type_name="Q4_K", dims=(4096,
     return out
 
 
+def bench_batched_vocabulary(ctx, hip, type_name, vocab, dim, model, rows_list, steps, warmup):
+    """The vocabulary projection of a batched decode step -- logits for B sequences -- over two copies
+    of the weight in turn (each larger than the 256 MB memory-side cache): the weight-streaming kernel
+    on a launch large enough that its fixed costs are a small part."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.projections import QuantizedBatchProjections
+    t = GGMLType[type_name]
+    host = synthetic.weight(t, vocab, dim, 91)
+    ws = [ctx.load_weight(t, host, vocab, dim) for _ in range(2)]
+    legs = []
+    for B in rows_list:
+        Xh = synthetic.activations((B, dim), 92 + B)
+        X, out = ctx.from_numpy(Xh), ctx.float_array(B * vocab)
+        proj = QuantizedBatchProjections(ctx, B, dim, vocab)
+        proj.projection(X, out, ws[0], dim, vocab, False)
+        ctx.sync()
+        rows = sample_rows(vocab, 64, 93)
+        ref, mag = oracle_rows(t, host, dim, rows, Xh)
+        err = check(f"batched vocabulary projection B={B}", out.get().reshape(B, vocab)[:, rows], ref, mag, 2e-3)
+
+        def sweep():      # (sixteen calls to a replay: the pause between replays is shared)
+            for _ in range(8):
+                for w in ws:
+                    proj.projection(X, out, w, dim, vocab, False)
+        us_list = [m / (8 * len(ws)) * 1e3 for m in timed_graph(ctx, hip, sweep, steps, warmup)]
+        us = statistics.median(us_list)
+        nbytes = host.size + 4 * B * (dim + vocab)
+        legs.append({"B": B, "us_per_call": round(us, 2), "us_stats": spread_stats(us_list), "bytes": nbytes,
+                     "GB_s": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                     "check_rel_err": err})
+        for b in (X, out, proj.workspace):
+            b.free()
+    for w in ws:
+        w.free()
+    return {"type": type_name, "weight": f"{model} vocabulary projection [{vocab} x {dim}]", "weight_bytes": int(host.size),
+            "copies_swept": len(ws), "rows": legs}
+
+
 def bench_decode_layers(ctx, hip, type_name, dim, kv, ffn, copies, steps, warmup, cpu):
     """Single-token decode projections of one layer -- q|k|v, o (+=), gate/up SwiGLU, down (+=) --
     over `copies` distinct layers' weights (more bytes than the 256 MB last-level cache holds),
@@ -1030,7 +1069,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-extra", action="store_true", help="skip the legs beside the decode set")
-    ap.add_argument("--extra", default="wq_shape,fused_rms,prefill,other_types,batched,prefill_other_types,batched_other_types,short_prompt",
+    ap.add_argument("--extra", default="wq_shape,fused_rms,prefill,other_types,batched,prefill_other_types,batched_other_types,batched_vocabulary,short_prompt",
                     help="comma-separated legs beside the decode set (a profiler run takes a few at a time)")
     ap.add_argument("--prefill-warmup", type=int, default=-1,
                     help="untimed replays before the prefill legs (default 100; 10 under a profiler)")
@@ -1293,6 +1332,11 @@ def main():
                 for name, dims, model, copies in (("Q8_0", (DIM, KV_DIM, HIDDEN), "Llama-3.2-1B", 32),
                                                   ("Q4_0", (4096, 1024, 14336), "Llama-3-8B", 8))
                 for B in (8, 32, 64)]
+        if "batched_vocabulary" in legs:
+            # the other launch of a batched decode step: logits for B sequences
+            out["batched_vocabulary"] = [
+                bench_batched_vocabulary(ctx, hip, name, vocab, dim, model, (8, 32, 64), max(10, args.steps // 2), 3)
+                for name, vocab, dim, model in (("Q4_K", 151936, 4096, "Qwen3-8B-like"), ("Q8_0", VOCAB, DIM, "Llama-3.2-1B"))]
         if "short_prompt" in legs:
             # between batched decode and prefill: 96, 192 and 384 rows (most prompts are this long)
             out["short_prompt"] = bench_short_prompt(ctx, hip, (96, 192, 384), max(5, args.steps // 5), 3)
