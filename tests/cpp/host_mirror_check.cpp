@@ -4,8 +4,11 @@
 //
 //   host_mirror_check --no-device    argument checks and exception types only (no GPU needed)
 //   host_mirror_check                the parity checks on device 0; prints one line per case
+#include <unistd.h>
+
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -312,6 +315,51 @@ int main(int argc, char **argv) {
             mag.insert(mag.end(), m.begin(), m.end());
         }
         held(("projection over fp16 rows," + tag).c_str(), out.get().data(), ref.data(), mag.data(), ref.size(), 2e-3);
+    }
+    {
+        // ---- a weight straight from a GGUF file ----------------------------------------------
+        // version 3, one key (general.alignment = 32, u32), one Q8_0 tensor of ne = [256, 24]
+        const int d = 24, n = 256;
+        const auto raw = weight(JO_Q8_0, d, n, 501);
+        std::string blob;
+        auto put = [&](const void *p, std::size_t bytes) { blob.append(static_cast<const char *>(p), bytes); };
+        auto put_u32 = [&](std::uint32_t v) { put(&v, 4); };
+        auto put_u64 = [&](std::uint64_t v) { put(&v, 8); };
+        auto put_str = [&](const std::string &t) { put_u64(t.size()); put(t.data(), t.size()); };
+        put("GGUF", 4); put_u32(3); put_u64(1); put_u64(1);
+        put_str("general.alignment"); put_u32(4 /* u32 */); put_u32(32);
+        put_str("blk.0.attn_q.weight"); put_u32(2); put_u64((std::uint64_t)n); put_u64((std::uint64_t)d); put_u32(JO_Q8_0); put_u64(0);
+        blob.append((32 - blob.size() % 32) % 32, '\0');
+        put(raw.data(), raw.size());
+        char path[] = "/tmp/jitllm_cpp_host_XXXXXX";
+        const int fd = mkstemp(path);
+        bool written = fd >= 0 && write(fd, blob.data(), blob.size()) == (ssize_t)blob.size();
+        if (fd >= 0) close(fd);
+        expect("a GGUF file written", written);
+        if (written) {
+            GGUF file(path);
+            expect("GGUF: one tensor, found by name, alignment read",
+                   file.tensorCount() == 1 && file.has("blk.0.attn_q.weight") && !file.has("nope") &&
+                       file.metadataInt("general.alignment") == 32);
+            TornadoTensor w = file.load(ctx, "blk.0.attn_q.weight");
+            expect("GGUF: the tensor's type and ne order", w.dataType() == JO_Q8_0 && w.rows() == d && w.cols() == n);
+            const auto x = activations((std::size_t)n, 502);
+            FloatArray dx(ctx, x), out(ctx, (std::size_t)d);
+            QuantizedProjections(ctx, TornadoWorkspace{}).floatMatvec(dx, out, w, n, d);
+            ctx.sync();
+            std::vector<float> ref((std::size_t)d);
+            jo_matmul(JO_Q8_0, JO_DOT_VEC256, raw.data(), x.data(), ref.data(), d, n, threads);
+            held("floatMatvec over a weight loaded from GGUF", out.get().data(), ref.data(),
+                 magnitude(JO_Q8_0, raw, x.data(), d, n).data(), (std::size_t)d, 2e-5);
+            bool missing = false;
+            try {
+                file.load(ctx, "blk.9.nope");
+            } catch (const Error &e) {
+                missing = std::strstr(e.what(), "no tensor") != nullptr;
+            }
+            expect("GGUF: a missing tensor is named", missing);
+            std::remove(path);
+        }
     }
     std::printf("[cpp-host] %s\n", failures ? "FAILED" : "all ok");
     return failures ? 1 : 0;
