@@ -696,10 +696,21 @@ def bench_batched_vocabulary(ctx, hip, type_name, vocab, dim, model, rows_list, 
         us_list = [m / (8 * len(ws)) * 1e3 for m in timed_graph(ctx, hip, sweep, steps, warmup)]
         us = statistics.median(us_list)
         nbytes = host.size + 4 * B * (dim + vocab)
+        # ... and the greedy token of every row (batchedArgmaxLogits), one launch over the B x vocab logits
+        tokens = ctx.raw_buffer(4 * B)
+        proj.argmaxLogits(out, vocab, tokens)
+        ctx.sync()
+        if not np.array_equal(tokens.download(np.int32, B), np.argmax(out.get().reshape(B, vocab), axis=1)):
+            raise SystemExit("bench.py: the device's per-row greedy tokens are not the first maxima of its logits")
+
+        def picks():
+            for _ in range(16):
+                proj.argmaxLogits(out, vocab, tokens)
+        argmax_us = statistics.median(m / 16 * 1e3 for m in timed_graph(ctx, hip, picks, steps, warmup))
         legs.append({"B": B, "us_per_call": round(us, 2), "us_stats": spread_stats(us_list), "bytes": nbytes,
                      "GB_s": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-                     "check_rel_err": err})
-        for b in (X, out, proj.workspace):
+                     "check_rel_err": err, "argmax_rows_us": round(argmax_us, 2)})
+        for b in (X, out, proj.workspace, tokens):
             b.free()
     for w in ws:
         w.free()

@@ -220,6 +220,16 @@ int jl_gemv_gate_up_rms(jl_context *ctx, const jl_weight *w1, const jl_weight *w
  * first of equals, 0 when element 0 is NaN -- this follows).
  */
 int jl_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
+/*
+ * The same for the logits of a batch: indices[b] = position of the first maximum of
+ * values[b * row_stride .. + n), b < rows, in one launch -- batchedArgmaxLogits
+ * (J/backend/tornado/kernels/TransformerBatchPrefillKernels.java:2118-2159), the last task of the
+ * batched logits graph (J/backend/tornado/batch/TornadoBatchExecutor.java:226-232), so that only
+ * `rows` integers cross to the host.  Ties and NaN as jl_argmax (the reference kernel's tree keeps
+ * whichever of two equal maxima its lower thread held; the host's scan, followed here, the first).
+ */
+int jl_argmax_rows(jl_context *ctx, const float *values, int64_t rows, int64_t n, int64_t row_stride,
+                   int32_t *indices);
 
 /*
  * The tail of a greedy decode step in one call: out = w . x, the vocabulary projection -- with the

@@ -343,6 +343,13 @@ public:
     int batchSize() const { return batch_; }
     std::size_t workspaceBytes() const { return workspace_.bytes(); }
 
+    // tokens[b] = first maximum of row b of the batched logits, int32 on the device
+    // (batchedArgmaxLogits, TransformerBatchPrefillKernels.java:2118-2159)
+    void argmaxLogits(const FloatArray &logits, std::int64_t vocab, const DeviceBuffer &tokens, int activeRows = -1,
+                      std::int64_t rowStride = -1) const {
+        check(jl_argmax_rows(ctx_, logits.data(), activeRows < 0 ? batch_ : activeRows, vocab, rowStride < 0 ? vocab : rowStride,
+                             static_cast<std::int32_t *>(tokens.ptr())));
+    }
     // out = w . x over the batch, or out += w . x with `residual` (QuantizedBatchProjections.java:76-309);
     // rows past activeRows are left untouched
     void projection(const FloatArray &x, const FloatArray &out, const TornadoTensor &w, int n, int d, bool residual,

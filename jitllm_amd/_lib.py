@@ -53,6 +53,7 @@ SYMBOLS = {
     "jl_gemv_qkv_rms": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_float, vp, vp, vp]),
     "jl_gemv_gate_up_rms": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp]),
     "jl_argmax": (C.c_int, [vp, vp, i64, vp]),
+    "jl_argmax_rows": (C.c_int, [vp, vp, i64, i64, i64, vp]),
     "jl_gemv_argmax": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, vp, vp]),
     "jl_argmax_static": (C.c_int, [vp, vp, i64, vp]),
     "jl_quantize_q8": (C.c_int, [vp, vp, i64, vp, vp, vp]),

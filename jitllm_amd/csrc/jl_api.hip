@@ -431,6 +431,16 @@ int jl_gemv_argmax(jl_context *ctx, const jl_weight *w, const float *x, const fl
     return jl_launch_gemv_argmax(ctx, w, x, rms_weights ? &rms : nullptr, out, index);
 }
 
+int jl_argmax_rows(jl_context *ctx, const float *values, int64_t rows, int64_t n, int64_t row_stride,
+                   int32_t *indices) {
+    JL_REQUIRE(ctx && values && indices, "jl_argmax_rows: null argument");
+    JL_REQUIRE(rows >= 0 && rows <= INT32_MAX && n > 0 && n <= INT32_MAX && row_stride >= n,
+               "jl_argmax_rows: %lld rows of %lld values, %lld apart", (long long)rows, (long long)n,
+               (long long)row_stride);
+    if (rows == 0) return JL_OK;
+    return jl_launch_argmax_rows(ctx, values, rows, n, row_stride, indices);
+}
+
 int jl_argmax_static(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
     JL_REQUIRE(ctx && values && index, "jl_argmax_static: null argument");
     JL_REQUIRE(n > 0, "jl_argmax_static: %lld values", (long long)n);

@@ -136,6 +136,8 @@ int jl_launch_rms_scale(jl_context *ctx, const float *x, int64_t n, float eps, f
 int jl_launch_rms_apply(jl_context *ctx, const float *x, const float *rms_w, const float *rms_scale, int64_t n,
                         float *xb);
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index);
+int jl_launch_argmax_rows(jl_context *ctx, const float *values, int64_t rows, int64_t n, int64_t row_stride,
+                          int32_t *indices);
 // out = w . x (rms set: the normalisation folded in) and index[0] = the first maximum of out.
 int jl_launch_gemv_argmax(jl_context *ctx, const jl_weight *w, const float *x, const jl_rms *rms, float *out,
                           int32_t *index);

@@ -126,6 +126,89 @@ __global__ void __launch_bounds__(kArgmaxGroups) jl_argmax_fold(const float *val
     }
 }
 
+// Per-row argmax over batched logits, one workgroup per row: batchedArgmaxLogits
+// (J/backend/tornado/kernels/TransformerBatchPrefillKernels.java:2118-2159), the last task of the
+// reference's batched logits graph (J/backend/tornado/batch/TornadoBatchExecutor.java:226-232), with
+// the host scan's rule for equal maxima -- the first one, FloatTensor.argmax -- where the reference
+// kernel's tree keeps whichever its lower thread held.
+__global__ void __launch_bounds__(kThreads) jl_argmax_rows_kernel(const float *values, int n, int64_t row_stride,
+                                                                  int32_t *indices) {
+    __shared__ float pv[kThreads / JL_WAVE];
+    __shared__ int pi[kThreads / JL_WAVE];
+    const int tid = threadIdx.x;
+    const float *row = values + (int64_t)blockIdx.x * row_stride;
+    float best = -INFINITY;
+    int at = INT_MAX;
+    const int n4 = ((uintptr_t)row & 15) == 0 ? n / 4 : 0;
+    for (int i = tid; i < n4; i += kThreads) {
+        const float4 v = ((const float4 *)row)[i];
+        if (v.x > best) { best = v.x; at = 4 * i; }
+        if (v.y > best) { best = v.y; at = 4 * i + 1; }
+        if (v.z > best) { best = v.z; at = 4 * i + 2; }
+        if (v.w > best) { best = v.w; at = 4 * i + 3; }
+    }
+    for (int i = n4 * 4 + tid; i < n; i += kThreads)
+        if (row[i] > best) { best = row[i]; at = i; }
+    fold_waves(best, at, pv, pi, tid, kThreads / JL_WAVE);
+    if (tid == 0) {
+        if (at == INT_MAX || row[0] != row[0]) at = 0;   // as in jl_argmax_fold
+        indices[blockIdx.x] = at;
+    }
+}
+
+// The same with each row cut into `chunks` runs, one workgroup per (run, row), for batches too small
+// to fill the chip with a workgroup per row: the runs' best (value, index) go to cells
+// [row * chunks + run] and jl_argmax_rows_fold, one wave per row, folds them.
+__global__ void __launch_bounds__(kArgmaxThreads) jl_argmax_rows_scan(const float *values, int n, int64_t row_stride, int chunks,
+                                                                      float *cell_value, int *cell_index) {
+    __shared__ float pv[kArgmaxThreads / JL_WAVE];
+    __shared__ int pi[kArgmaxThreads / JL_WAVE];
+    const int tid = threadIdx.x, run = blockIdx.x;
+    const float *row = values + (int64_t)blockIdx.y * row_stride;
+    float best = -INFINITY;
+    int at = INT_MAX;
+    const int n4 = ((uintptr_t)row & 15) == 0 ? n / 4 : 0;
+    const int per4 = (n4 + chunks - 1) / chunks;
+    const int end4 = (run + 1) * per4 < n4 ? (run + 1) * per4 : n4;
+    for (int i = run * per4 + tid; i < end4; i += kArgmaxThreads) {
+        const float4 v = ((const float4 *)row)[i];
+        if (v.x > best) { best = v.x; at = 4 * i; }
+        if (v.y > best) { best = v.y; at = 4 * i + 1; }
+        if (v.z > best) { best = v.z; at = 4 * i + 2; }
+        if (v.w > best) { best = v.w; at = 4 * i + 3; }
+    }
+    // what the 16-byte loads do not cover (the last values of a row, or all of a row that starts off
+    // a 16-byte boundary), shared out over the runs the same way
+    const int rest = n - 4 * n4, per = (rest + chunks - 1) / chunks;
+    const int end = (run + 1) * per < rest ? (run + 1) * per : rest;
+    for (int i = run * per + tid; i < end; i += kArgmaxThreads)
+        if (row[4 * n4 + i] > best) { best = row[4 * n4 + i]; at = 4 * n4 + i; }
+    fold_waves(best, at, pv, pi, tid, kArgmaxThreads / JL_WAVE);
+    if (tid == 0) {
+        cell_value[blockIdx.y * chunks + run] = best;
+        cell_index[blockIdx.y * chunks + run] = at;
+    }
+}
+
+__global__ void __launch_bounds__(JL_WAVE) jl_argmax_rows_fold(const float *values, int64_t row_stride, int chunks,
+                                                               const float *cell_value, const int *cell_index,
+                                                               int32_t *indices) {
+    const int lane = threadIdx.x, row = blockIdx.x;
+    float best = lane < chunks ? cell_value[row * chunks + lane] : -INFINITY;
+    int at = lane < chunks ? cell_index[row * chunks + lane] : INT_MAX;
+#pragma unroll
+    for (int o = JL_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, JL_WAVE);
+        const int oi = __shfl_xor(at, o, JL_WAVE);
+        keep_better(best, at, ov, oi);
+    }
+    if (lane == 0) {
+        const float first = values[(int64_t)row * row_stride];
+        if (at == INT_MAX || first != first) at = 0;   // as in jl_argmax_fold
+        indices[row] = at;
+    }
+}
+
 // The fold for cells a projection kernel left (one per workgroup, up to a thousand, rows in no
 // particular order from cell to cell): the same rule, a strided walk first.
 constexpr int kProjectionCells = JL_CONTEXT_SCRATCH_BYTES / 8;
@@ -222,6 +305,31 @@ static int argmax_launches(jl_context *ctx, const float *values, int64_t n, int3
 int jl_launch_argmax(jl_context *ctx, const float *values, int64_t n, int32_t *index) {
     static_assert(sizeof(ArgmaxCells) <= JL_CONTEXT_SCRATCH_BYTES, "argmax cells exceed the context scratch");
     return argmax_launches(ctx, values, n, index, (ArgmaxCells *)ctx->scratch);
+}
+
+int jl_launch_argmax_rows(jl_context *ctx, const float *values, int64_t rows, int64_t n, int64_t row_stride,
+                          int32_t *indices) {
+    // a workgroup per row fills the chip from a few hundred rows on; smaller batches cut their rows
+    // into runs (at most a wave's worth, and no more (run, row) cells than the context's scratch holds)
+    int chunks = (int)(2 * ctx->compute_units / rows);
+    if (chunks > JL_WAVE) chunks = JL_WAVE;
+    if ((int64_t)chunks * rows > kProjectionCells) chunks = (int)(kProjectionCells / rows);
+    if ((int64_t)chunks * 4096 > n) chunks = (int)(n / 4096);   // (runs of at least 4096 values)
+    if (chunks < 2) {
+        hipLaunchKernelGGL(jl_argmax_rows_kernel, dim3((unsigned)rows), dim3(kThreads), 0, ctx->stream, values, (int)n,
+                           row_stride, indices);
+        JL_HIP(hipGetLastError());
+        return JL_OK;
+    }
+    float *cell_value = (float *)ctx->scratch;
+    int *cell_index = (int *)(cell_value + kProjectionCells);
+    hipLaunchKernelGGL(jl_argmax_rows_scan, dim3((unsigned)chunks, (unsigned)rows), dim3(kArgmaxThreads), 0, ctx->stream,
+                       values, (int)n, row_stride, chunks, cell_value, cell_index);
+    JL_HIP(hipGetLastError());
+    hipLaunchKernelGGL(jl_argmax_rows_fold, dim3((unsigned)rows), dim3(JL_WAVE), 0, ctx->stream, values, row_stride, chunks,
+                       cell_value, cell_index, indices);
+    JL_HIP(hipGetLastError());
+    return JL_OK;
 }
 
 int jl_launch_gemv_argmax(jl_context *ctx, const jl_weight *w, const float *x, const jl_rms *rms, float *out,

@@ -292,6 +292,15 @@ class QuantizedBatchProjections:
                                             rmsWeights.ptr, eps, rows, dim,
                                             scales.ptr if scales is not None else None, out.ptr))
 
+    def argmaxLogits(self, logits: FloatArray, vocab: int, tokens: DeviceBuffer, activeRows: int | None = None,
+                     rowStride: int | None = None) -> None:
+        """``tokens[b]`` = first maximum of row ``b`` of the batched logits, int32 on the device
+        (batchedArgmaxLogits, TransformerBatchPrefillKernels.java:2118-2159; the "argmax" task of
+        TornadoBatchExecutor's logits graph, :226-232): only the batch's token ids go to the host."""
+        rows = self.batchSize if activeRows is None else activeRows
+        L.check(self._lib.jl_argmax_rows(self.context.handle, logits.ptr, rows, vocab,
+                                         vocab if rowStride is None else rowStride, tokens.ptr))
+
     def projection(self, x: FloatArray, out: FloatArray, w: TornadoTensor, n: int, d: int,
                    residual: bool, activeRows: int | None = None) -> None:
         """``out = w . x`` over the batch, or ``out += w . x`` with ``residual``

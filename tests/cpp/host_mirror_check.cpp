@@ -315,6 +315,16 @@ int main(int argc, char **argv) {
             mag.insert(mag.end(), m.begin(), m.end());
         }
         held(("projection over fp16 rows," + tag).c_str(), out.get().data(), ref.data(), mag.data(), ref.size(), 2e-3);
+        // one token per row of those outputs, as the batched logits graph ends
+        DeviceBuffer tokens(ctx, (std::size_t)B * 4);
+        batch.argmaxLogits(out, dq, tokens);
+        ctx.sync();
+        std::vector<std::int32_t> tok((std::size_t)B);
+        tokens.download(tok.data(), tok.size() * 4);
+        const auto rows = out.get();
+        bool first_maxima = true;
+        for (int b = 0; b < B; b++) first_maxima = first_maxima && tok[(std::size_t)b] == (std::int32_t)jo_argmax(rows.data() + (std::size_t)b * dq, dq);
+        expect(("argmaxLogits: every row's first maximum," + tag).c_str(), first_maxima);
     }
     {
         // ---- a weight straight from a GGUF file ----------------------------------------------

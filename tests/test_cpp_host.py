@@ -34,8 +34,7 @@ def test_the_header_is_strict_cxx17_on_its_own(tmp_path):
 
 
 def test_errors_arrive_as_exceptions_without_a_device():
-    import torch
-    if torch.cuda.is_available():
+    if os.path.exists("/dev/kfd"):
         pytest.skip("a GPU is present: the parity run covers the binary")
     out = subprocess.run([built(), "--no-device"], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stdout + out.stderr

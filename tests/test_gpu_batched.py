@@ -884,6 +884,34 @@ def test_weights_of_different_types_side_by_side(ctx, rows, resident):
     assert np.all(np.abs(flat[:rows * d].reshape(rows, d).astype(np.float64) - ref) <= bound)
 
 
+@pytest.mark.parametrize("rows,n,stride", [(1, 1000, 1000), (8, 128256, 128256), (64, 32000, 32003), (40, 5, 9),
+                                           (300, 4097, 4100)])
+def test_argmax_of_every_row_of_batched_logits(ctx, rows, n, stride):
+    """batchedArgmaxLogits: one token per row in one launch, the host scan's rule on ties and NaN
+    (first maximum; a NaN at element 0 wins, elsewhere never; all -inf gives 0); row strides that
+    leave the rows off a 16-byte boundary; rows past the active ones keep their token."""
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("argmax rows", rows, n, stride)
+    rng = np.random.default_rng(9800 + rows)
+    v = rng.standard_normal((rows + 2, stride)).astype(np.float32)
+    v[:, n:] = 1e30                                        # what lies between the rows is not looked at
+    for b in range(rows):
+        v[b, rng.integers(0, n, size=3)] = 7.0             # the maximum three times: the first one counts
+    if rows > 3 and n > 4:
+        v[1, :n] = -np.inf
+        v[2, 0] = np.nan
+        v[3, n // 2] = np.nan
+    logits = ctx.from_numpy(v.reshape(-1))
+    tokens = ctx.raw_buffer(4 * (rows + 2))
+    tokens.upload(np.full(rows + 2, -5, dtype=np.int32))
+    QuantizedBatchProjections(ctx, rows + 2, 256, 256).argmaxLogits(logits, n, tokens, activeRows=rows, rowStride=stride)
+    ctx.sync()
+    got = tokens.download(np.int32, rows + 2)
+    assert np.all(got[rows:] == -5)
+    for b in range(rows):
+        assert int(got[b]) == O.argmax(v[b, :n]), b
+
+
 def test_huge_activation_rows_stay_finite(ctx):
     """Rows far outside fp16's range are rescaled by a power of two, not turned into infinities."""
     from jitllm_amd import synthetic
