@@ -1051,6 +1051,28 @@ def batched_probe(ctx):
     print(json.dumps({"weight_bytes": {k: int(v.size) for k, v in host.items()}}))
 
 
+def vocabulary_probe(ctx):
+    """What the kernel trace of the batched vocabulary projection is collected on: the Q8_0
+    [128256 x 2048] projection and the per-row greedy token at 8, 32 and 64 rows, kernel by kernel
+    over two device copies of the weight in turn, six rounds each."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.projections import QuantizedBatchProjections
+    t = GGMLType.Q8_0
+    host = synthetic.weight(t, VOCAB, DIM, 91)
+    ws = [ctx.load_weight(t, host, VOCAB, DIM) for _ in range(2)]
+    for B in (8, 32, 64):
+        X, out = ctx.from_numpy(synthetic.activations((B, DIM), 92 + B)), ctx.float_array(B * VOCAB)
+        tokens = ctx.raw_buffer(4 * B)
+        proj = QuantizedBatchProjections(ctx, B, DIM, VOCAB)
+        for _ in range(6):
+            for w in ws:
+                proj.projection(X, out, w, DIM, VOCAB, False)
+                proj.argmaxLogits(out, VOCAB, tokens)
+            ctx.sync()
+    print(json.dumps({"weight_bytes": int(host.size)}))
+
+
 def int8_probe(ctx, t, T=2048):
     """What the counters and the kernel trace of the int8 prefill path are collected on: one
     Llama-3.2-1B layer's four calls at T tokens with JL_MATH_INT8, kernel by kernel, four times."""
@@ -1095,6 +1117,8 @@ def main():
                     help="only measure the rate of a plain streaming read of HBM (see hbm_rate_probe)")
     ap.add_argument("--mfma-rate-probe", action="store_true",
                     help="only measure the sustained rate of fp16 matrix instructions (see mfma_rate_probe)")
+    ap.add_argument("--vocabulary-probe", action="store_true",
+                    help="only launch the batched vocabulary projection and its per-row argmax (see vocabulary_probe)")
     ap.add_argument("--batched-probe", action="store_true",
                     help="only launch the batched-decode calls, kernel by kernel (see batched_probe)")
     ap.add_argument("--decode-probe", action="store_true",
@@ -1130,6 +1154,9 @@ def main():
             return
         if args.prefill_probe:
             prefill_probe(ctx, t, args.probe_tokens, args.probe_mode)
+            return
+        if args.vocabulary_probe:
+            vocabulary_probe(ctx)
             return
         if args.batched_probe:
             batched_probe(ctx)
