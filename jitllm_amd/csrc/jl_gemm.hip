@@ -913,11 +913,16 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     //   the plain fp16 GEMM            24 + 0.45 x 256-row tiles x million weights over a copy that is
     //                                  kept across calls (from 128 rows); 30 + 2.8 x million weights
     //                                  when the call has to decode first and has no other kernel
-    double millions = 0.0;
-    for (int i = 0; i < count; i++) millions += (double)weights[i]->rows * k * 1e-6;
-    const double in_loop_us = dense_only || (kept && rows >= 192)
-                                  ? 1e30
-                                  : 22.0 + (type == JL_Q8_0 ? 0.30 : 0.37) * ((rows + 127) / 128) * millions;
+    double millions = 0.0, weight_bytes = 0.0;
+    for (int i = 0; i < count; i++) {
+        millions += (double)weights[i]->rows * k * 1e-6;
+        weight_bytes += (double)weights[i]->bytes;
+    }
+    // (the kernel that decodes in its loop streams no faster than ~1.9 TB/s: the floor of a call over
+    // hundreds of MB of Q8_0 at up to 128 rows, a vocabulary projection -- 147 us for 279 MB)
+    double in_loop_us = 22.0 + (type == JL_Q8_0 ? 0.30 : 0.37) * ((rows + 127) / 128) * millions;
+    if (in_loop_us < weight_bytes / 1.9e6) in_loop_us = weight_bytes / 1.9e6;
+    if (dense_only || (kept && rows >= 192)) in_loop_us = 1e30;
     const double copy_us = kept && rows >= 128 ? 24.0 + 0.45 * ((rows + 255) / 256) * millions
                            : dense_only       ? 30.0 + 2.8 * millions
                                               : 1e30;
