@@ -87,6 +87,34 @@ def test_vocabulary_projection_128256(ctx):
     w.free()
 
 
+@pytest.mark.parametrize("B", [64, 96, 128])
+def test_vocabulary_projection_for_many_sequences(ctx, B):
+    """The same 128256 x 2048 weight for B rows of activations: two and three row blocks of the
+    weight-streaming kernel and, at 128 rows, the tiled kernel that decodes in its loop -- a call
+    of 279 MB, where the streaming kernel is still the cheaper at 96 rows."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    t, d, n = O.Q8_0, 128256, 2048
+    say("vocabulary projection, rows", B)
+    raw = synthetic.weight(t, d, n, seed=18)
+    rows = sample_rows(d, 96, 905)
+    sub = gather(raw, t, n, rows)
+    w = ctx.load_weight(t, raw, d, n)
+    del raw
+    X = synthetic.activations((B, n), seed=906 + B)
+    proj = QuantizedBatchProjections(ctx, B, n, d)
+    out = ctx.float_array(B * d, fill=POISON)
+    proj.projection(ctx.from_numpy(X), out, w, n, d, False)
+    ctx.sync()
+    got = out.get().reshape(B, d)
+    assert np.all(got != POISON)
+    ref = O.matmul_batch(t, sub, X, rows.size, n)
+    assert rel_err(got[:, rows], ref, magnitude(t, sub, X, rows.size, n)) < 2e-3
+    out.free()
+    proj.workspace.free()
+    w.free()
+
+
 @pytest.mark.parametrize("d,n", [(4096, 14336), (14336, 4096)])
 def test_q4_0_llama3_8b_feed_forward_shapes(ctx, d, n):
     """Q4_0 w2 4096 x 14336 (rows of 14336 columns) and w1 / w3 14336 x 4096, plain and residual."""
