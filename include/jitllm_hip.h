@@ -94,6 +94,16 @@ int jl_sync(jl_context *ctx);
 void *jl_context_stream(jl_context *ctx);
 /* Compute units of the device and its name (DeviceCapability of the reference's backend SPI). */
 int jl_device_info(jl_context *ctx, int *compute_units, char *name, size_t name_bytes);
+/*
+ * enabled == 0: no jl_gemm* call on this context cuts K across work items; every GEMM stays whole,
+ * as under the reference's -Djitllm.prefill.splitK=false (SplitKGemm.java:40-42,
+ * J/backend/tornado/layers/).  A narrow output at few rows (a 2048-wide projection of a 512-token
+ * chunk) is otherwise computed as 2, 4 or 8 runs of K whose partial sums are added afterwards: faster,
+ * and a different order of addition than the same rows get in a larger chunk.  With the switch off
+ * a prefill row's result does not depend on how many rows (>= 512) share its call.  Default: on.
+ * Batched decode (calls of up to 64 rows) is not affected.
+ */
+int jl_context_set_split_k(jl_context *ctx, int enabled);
 
 /* ---- device buffers for fp32 activations (TornadoVM FloatArray of the reference) ----------- */
 

@@ -65,6 +65,8 @@ public:
     jl_context *handle() const { return handle_; }
     void *stream() const { return jl_context_stream(handle_); }
     void sync() const { check(jl_sync(handle_)); }
+    // false: every GEMM whole (-Djitllm.prefill.splitK=false, SplitKGemm.java:40-42)
+    void setSplitK(bool enabled) const { check(jl_context_set_split_k(handle_, enabled ? 1 : 0)); }
 
 private:
     jl_context *handle_ = nullptr;

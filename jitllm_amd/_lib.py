@@ -30,6 +30,7 @@ SYMBOLS = {
     "jl_sync": (C.c_int, [vp]),
     "jl_context_stream": (vp, [vp]),
     "jl_device_info": (C.c_int, [vp, C.POINTER(C.c_int), C.c_char_p, C.c_size_t]),
+    "jl_context_set_split_k": (C.c_int, [vp, C.c_int]),
     "jl_malloc": (C.c_int, [vp, C.c_size_t, C.POINTER(vp)]),
     "jl_free": (C.c_int, [vp, vp]),
     "jl_upload": (C.c_int, [vp, vp, vp, C.c_size_t]),

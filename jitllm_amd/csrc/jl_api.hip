@@ -106,6 +106,12 @@ int jl_sync(jl_context *ctx) {
 
 void *jl_context_stream(jl_context *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
 
+int jl_context_set_split_k(jl_context *ctx, int enabled) {
+    JL_REQUIRE(ctx != nullptr, "jl_context_set_split_k: context is null");
+    ctx->split_k = enabled != 0;
+    return JL_OK;
+}
+
 int jl_device_info(jl_context *ctx, int *compute_units, char *name, size_t name_bytes) {
     JL_REQUIRE(ctx != nullptr, "jl_device_info: context is null");
     if (compute_units) *compute_units = ctx->compute_units;

@@ -308,7 +308,7 @@ constexpr int W16_BYTES = BN * W16_STRIDE;     // 16384
 template <int TYPE> struct Raw;
 template <> struct Raw<JL_Q8_0> { static constexpr int kRowBytes = 272, kStepBytes = 68; };
 template <> struct Raw<JL_Q4_0> { static constexpr int kRowBytes = 144, kStepBytes = 36; };
-template <> struct Raw<JL_Q4_K> { static constexpr int kRowBytes = 144, kStepBytes = 32; };
+template <> struct Raw<JL_Q4_K> { static constexpr int kRowBytes = 144; };
 
 // Threads that do nothing but issue the LDS-DMA loads of both operands (two waves).
 constexpr int kCopyThreads = 128;
@@ -819,7 +819,7 @@ int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows, float *planes, si
     p.ntiles = (p.n_total + cols_per_tile - 1) / cols_per_tile;
     const int bm = rows <= 32 ? 32 : rows <= 64 ? 64 : 128;
     p.mtiles = (rows + bm - 1) / bm;
-    p.splits = choose_splits(rows, bm, p.k, p.ntiles * p.mtiles, p.row_bytes, ctx->compute_units);
+    p.splits = ctx->split_k ? choose_splits(rows, bm, p.k, p.ntiles * p.mtiles, p.row_bytes, ctx->compute_units) : 1;
     const int64_t plane = (int64_t)p.mtiles * bm * p.ntiles * BN;
     if (p.splits > 1 && (size_t)p.splits * plane * 4 > plane_bytes) p.splits = 1;
     p.partial = planes;
@@ -938,7 +938,7 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     const size_t in_workspace = kept ? 0 : copy_bytes;
     const int dense_from = kept && copy_us < in_loop_us ? 128 : 512;
     int dsplits = 1, bm = 256;
-    int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm, dense_from);
+    int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm, dense_from, ctx->split_k);
     if (bn != 0 && dsplits > 1 && in_workspace + jl_dense_plane_bytes(rows, virt, dsplits) > plane_bytes) {
         // no room for the partial sums of a cut K: the cheapest tiling that keeps K whole
         bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm, dense_from, false);

@@ -976,7 +976,6 @@ __global__ void __launch_bounds__(512 + 64 * (kDmaWaves + kFoldWaves)) jl_gemm_s
 #pragma unroll
         for (int b = 0; b < NBB; b++) lds_write_f4(pw + b * 1024, total[b]);
     };
-    const int tiles = mine * ZIN;
     // The two compute waves of a SIMD (w and w + 4) run half a tile apart, so that one of them
     // decodes (vector ALU) while the other multiplies (matrix pipe): after the barrier of tile t
     // the early wave decodes tile t and multiplies it; the late wave first multiplies tile t - 1,

@@ -24,6 +24,9 @@ struct jl_context {
     // caller's pointer is only ever touched by a host memcpy.
     uint8_t *bounce;
     hipEvent_t bounce_done[2];
+    // false: no GEMM of this context cuts K across work items (jl_context_set_split_k), so that a
+    // row's sums are added in one order whatever the call's row count
+    bool split_k = true;
 };
 #define JL_CONTEXT_SCRATCH_BYTES 8192
 #define JL_CONTEXT_ARRIVALS 1024

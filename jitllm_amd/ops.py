@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import ctypes as C
 import enum
+import os
 from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional, Sequence
 
@@ -284,8 +285,13 @@ class HipImplementation(Implementation):
     """The batched prefill through libjitllm_hip.so.  Listed ahead of the JIT candidates it claims
     the projection steps whose weights it has kernels for; everything else falls through."""
 
-    def __init__(self, residency: bool = False):
+    def __init__(self, residency: bool = False, splitK: Optional[bool] = None):
         self.residency = bool(residency)
+        # -Djitllm.prefill.splitK=false keeps every GEMM whole (SplitKGemm.java:40-42); here the
+        # environment variable JITLLM_PREFILL_SPLITK=false, unless the caller says
+        if splitK is None:
+            splitK = os.environ.get("JITLLM_PREFILL_SPLITK", "true").lower() != "false"
+        self.splitK = bool(splitK)
 
     def library(self) -> str:
         return "hip"
@@ -340,6 +346,7 @@ class HipImplementation(Implementation):
         need = self.needs(steps, target)
         if not steps:
             raise ValueError("an instance runs at least one step")
+        context.set_split_k(self.splitK)
         return HipInstance(context, max(s.tokens for s in steps), DeviceBuffer(context, max(need.bytes, 256)),
                            self.residency, ResidentCopies(context))
 

@@ -48,6 +48,12 @@ class Context:
         L.check(self._lib.jl_device_info(self.handle, C.byref(cu), name, 128))
         return cu.value, name.value.decode()
 
+    def set_split_k(self, enabled: bool) -> None:
+        """False keeps every GEMM of this context whole, as -Djitllm.prefill.splitK=false does in the
+        reference (SplitKGemm.java:40-42): a prefill row's sums are then added in one order whatever
+        the chunk size."""
+        L.check(self._lib.jl_context_set_split_k(self.handle, 1 if enabled else 0))
+
     # -- arrays --
     def float_array(self, size: int, fill: float | None = None) -> "FloatArray":
         a = FloatArray(self, size)

@@ -118,6 +118,7 @@ int no_device() {
         threw = e.status() == JL_ERR_INVALID;
     }
     expect("no device: a null argument is JL_ERR_INVALID", threw);
+    expect("no device: the split-K switch wants a context", jl_context_set_split_k(nullptr, 0) == JL_ERR_INVALID);
     return failures ? 1 : 0;
 }
 
@@ -241,6 +242,8 @@ int main(int argc, char **argv) {
 
     // ---- batched rows -------------------------------------------------------------------------
     for (int B : {8, 40, 200}) {
+        // (the largest batch with every GEMM kept whole, as under -Djitllm.prefill.splitK=false)
+        ctx.setSplitK(B != 200);
         const int n = 1024, dq = 520, dkv = 136, dff = 600;
         const std::string tag = " B " + std::to_string(B);
         const auto rq = weight(JO_Q4_K, dq, n, 401), rk = weight(JO_Q4_K, dkv, n, 402), rv = weight(JO_Q6_K, dkv, n, 403);

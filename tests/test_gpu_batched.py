@@ -957,3 +957,46 @@ def test_batched_errors(ctx):
     o2 = ctx.float_array(4 * 128, 0.0)
     st = lib.jl_gemm(ctx.handle, two, 2, x.ptr, o2.ptr, 4, 4, 128, 0, L.JL_STORE, L.JL_MATH_INT8, ws.ptr, ws.nbytes)
     assert st == L.JL_ERR_UNSUPPORTED and b"mixed weight types Q8_0 and Q4_0" in lib.jl_last_error()
+
+
+@pytest.mark.parametrize("t,residual", [(O.Q8_0, False), (O.Q4_K, True)])
+def test_with_k_kept_whole_a_row_does_not_depend_on_the_chunk(ctx, t, residual):
+    """jl_context_set_split_k(0) is the reference's -Djitllm.prefill.splitK=false (SplitKGemm.java:40-42):
+    a 2048-wide projection of a 512-row chunk, which otherwise cuts K into runs and adds their partial
+    sums afterwards, then gives each of its rows bit for bit what the same row gets in a 2048-row
+    chunk, whose K is whole anyway; with the switch on the two differ in their last bits.  The oracle
+    holds either way."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    d, n, small, large = 2048, 2048, 512, 2048
+    say("K kept whole", t, residual)
+    raw = synthetic.weight(t, d, n, seed=9680)
+    w = ctx.load_weight(t, raw, d, n)
+    X = synthetic.activations((large, n), seed=9681)
+    base = synthetic.activations((large, d), seed=9682) if residual else None
+
+    def run(rows):
+        proj = QuantizedBatchProjections(ctx, rows, n, d)
+        out = ctx.from_numpy(base[:rows].reshape(-1).copy()) if residual else ctx.float_array(rows * d, fill=UNTOUCHED)
+        proj.projection(ctx.from_numpy(X[:rows]), out, w, n, d, residual)
+        ctx.sync()
+        got = out.get().reshape(rows, d)
+        out.free()
+        proj.workspace.free()
+        return got
+
+    try:
+        ctx.set_split_k(False)
+        whole_small, whole_large = run(small), run(large)
+        ctx.set_split_k(True)
+        cut_small = run(small)
+    finally:
+        ctx.set_split_k(True)
+    assert np.array_equal(whole_small.view(np.uint32), whole_large[:small].view(np.uint32))
+    assert not np.array_equal(cut_small.view(np.uint32), whole_small.view(np.uint32))
+    edge, row_bytes = 64, raw.size // d
+    for got in (whole_small, cut_small):
+        ref = O.matmul_batch(t, raw[:edge * row_bytes], X[:small], edge, n)
+        delta = got[:, :edge] - (base[:small, :edge] if residual else 0.0)
+        assert rel_err(delta, ref, magnitude(t, raw[:edge * row_bytes], X[:small], edge, n)) < F16_BOUND
+    w.free()
