@@ -23,6 +23,13 @@
  *                              QuantizedDeviceDecodeParityTest q5_0 / iq4_XS ReadsGgmlsLayout), second
  *                              wordings, numpy statements of ggml's dequantize_row_*; dots: Q4_1 lane
  *                              model as above, Q5_0 / IQ4_XS block sums bit-equal to a numpy loop.
+ *   Q8_0 quantized-activation dot (JO_DOT_Q8ACT)  activations on their own int8 grid with power-of-two
+ *                              scales make every step exact: the result is the integer dot product
+ *                              times the scales, computed with Python integers; halves round away
+ *                              from zero; the integer values come from the fp32 scale and the sum
+ *                              is multiplied by the binary16-rounded one (a block whose scale is
+ *                              not a binary16 number shows the difference); a zero block adds
+ *                              nothing; an independent numpy float32 statement on random input.
  *   packed path                quantiser: known answers (the maximum maps to +-127, halves round away
  *                              from zero, a zero block gives zero scale and quants, sums = sum q);
  *                              projections: an activation that lies on its own int8 grid makes the
@@ -763,6 +770,52 @@ static float block_sum_dot(int type, const uint8_t *w, int64_t this_offset, cons
 }
 
 /*
+ * Q8_0FloatTensor.dotQ8Activation (J/tensor/standard/Q8_0FloatTensor.java:107-140), the branch
+ * Q8_0FloatTensor.dot takes under -Djitllm.quantizeActivation=true (:86-93; off by default).  Per
+ * block of 32: the activations' largest magnitude over 127 is the quantization scale; the int8
+ * values are derived with that fp32 scale (x * (1 / scale), rounded half away from zero through
+ * `(int)(s + copySign(0.5f, s))`), the scale that multiplies the integer sum is the same number
+ * rounded to binary16 and back; `result += isum * (wScale * aScale)` block after block.  Offsets
+ * and sizes are multiples of 32 for every caller; a remainder is dropped, as there.
+ */
+/* Java's (int) of a float: NaN gives 0 and the range saturates; C leaves both undefined. */
+static int32_t java_float_to_int(float v) {
+    if (v != v) return 0;
+    if (v >= 2147483648.0f) return INT32_MAX;
+    if (v <= -2147483648.0f) return INT32_MIN;
+    return (int32_t)v;
+}
+
+static float q8_activation_dot(const uint8_t *w, int64_t this_offset, const float *x, int64_t that_offset,
+                               int64_t size) {
+    float result = 0.0f;
+    const int64_t nblocks = size / 32;
+    for (int64_t b = 0; b < nblocks; b++) {
+        const int64_t elem_base = b * 32;
+        const uint8_t *blk = w + (this_offset + elem_base) / 32 * 34;
+        const float w_scale = jo_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        float amax = 0.0f;
+        for (int i = 0; i < 32; i++) {
+            const float av = fabsf(x[that_offset + elem_base + i]);
+            if (av > amax) amax = av;
+        }
+        const float quantization_scale = amax / 127.0f;
+        const float a_scale = jo_f16_to_f32(jo_f32_to_f16(quantization_scale));
+        const float a_inv = quantization_scale != 0.0f ? 1.0f / quantization_scale : 0.0f;
+        int32_t isum = 0;
+        for (int i = 0; i < 32; i++) {
+            const float s = x[that_offset + elem_base + i] * a_inv;
+            const float shifted = s + copysignf(0.5f, s);
+            const int32_t aq = java_float_to_int(shifted);
+            isum += aq * (int32_t)(int8_t)blk[2 + i];
+        }
+        const float scales = w_scale * a_scale;
+        result += (float)isum * scales;
+    }
+    return result;
+}
+
+/*
  * Q8_0FloatTensor.dot (J/tensor/standard/Q8_0FloatTensor.java:89-99), Q4_0FloatTensor.dot
  * (Q4_0FloatTensor.java:82-88), Q4_KFloatTensor.dot (Q4_KFloatTensor.java:124-127).  The flavour
  * is the branch a JVM would take: vector kernels exist for 128- and 256-bit species only
@@ -772,6 +825,8 @@ float jo_dot(int type, int flavour, const uint8_t *w, int64_t this_offset, const
              int64_t that_offset, int64_t size) {
     /* Q5_0 and IQ4_XS have one dot for every JVM (the flavour only matters to the vector kernels) */
     if (type == JO_Q5_0 || type == JO_IQ4_XS) return block_sum_dot(type, w, this_offset, x, that_offset, size);
+    /* the quantized-activation branch exists in Q8_0FloatTensor only and comes before the others */
+    if (type == JO_Q8_0 && flavour == JO_DOT_Q8ACT) return q8_activation_dot(w, this_offset, x, that_offset, size);
     if ((type == JO_Q8_0 || type == JO_Q4_0 || type == JO_Q4_1) && (flavour == JO_DOT_VEC128 || flavour == JO_DOT_VEC256)) {
         return vector_dot(type, flavour, w, this_offset, x, that_offset, size);
     }

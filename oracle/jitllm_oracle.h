@@ -20,8 +20,10 @@ extern "C" {
 /* ggml type ids, the numbering GGUF files carry (J/format/GGMLType.java:7,13,18 by ordinal). */
 enum { JO_Q4_0 = 2, JO_Q4_1 = 3, JO_Q5_0 = 6, JO_Q8_0 = 8, JO_Q4_K = 12, JO_Q5_K = 13, JO_Q6_K = 14, JO_IQ4_XS = 23 };
 
-/* dot flavours: which branch of Q8_0FloatTensor.dot / Q4_0FloatTensor.dot runs. */
-enum { JO_DOT_SCALAR = 0, JO_DOT_VEC128 = 128, JO_DOT_VEC256 = 256 };
+/* dot flavours: which branch of Q8_0FloatTensor.dot / Q4_0FloatTensor.dot runs.  JO_DOT_Q8ACT is
+ * Q8_0FloatTensor's -Djitllm.quantizeActivation=true branch (activations quantized per block of 32,
+ * integer sums); the other types have no such branch and read it as JO_DOT_SCALAR. */
+enum { JO_DOT_SCALAR = 0, JO_DOT_Q8ACT = 8, JO_DOT_VEC128 = 128, JO_DOT_VEC256 = 256 };
 
 int jo_block_elems(int type);  /* 32 / 32 / 256 / 256 */
 int jo_block_bytes(int type);  /* 18 / 34 / 144 / 210 */

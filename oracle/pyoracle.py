@@ -15,6 +15,7 @@ import numpy as np
 Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
 Q4_1, Q5_0, IQ4_XS = 3, 6, 23
 DOT_SCALAR, DOT_VEC128, DOT_VEC256 = 0, 128, 256
+DOT_Q8ACT = 8   # Q8_0FloatTensor.dotQ8Activation (-Djitllm.quantizeActivation=true), Q8_0 only
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "_build", "libjitllm_oracle.so")

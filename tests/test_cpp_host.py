@@ -38,7 +38,7 @@ def test_errors_arrive_as_exceptions_without_a_device():
         pytest.skip("a GPU is present: the parity run covers the binary")
     out = subprocess.run([built(), "--no-device"], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stdout + out.stderr
-    assert out.stdout.count(" ok") == 3 and "FAILED" not in out.stdout
+    assert out.stdout.count(" ok") == 4 and "FAILED" not in out.stdout
 
 
 @pytest.mark.gpu

@@ -164,6 +164,35 @@ def test_packed_path_inside_the_references_envelope(ctx, t):
     assert rel_l2 > 1e-4
 
 
+@pytest.mark.parametrize("d,n", [(2048, 2048), (1000, 4096), (512, 8192)])
+def test_packed_q8_0_against_the_cpu_paths_own_quantized_activation_dot(ctx, d, n):
+    """The reference's CPU path has the same idea behind a switch: Q8_0FloatTensor.dotQ8Activation
+    (-Djitllm.quantizeActivation=true, Q8_0FloatTensor.java:86-140) quantizes the activation per block
+    of 32 with the same rounding and multiplies integer sums.  It differs from the device path in one
+    step -- the activation scale that multiplies the sum is rounded to binary16 there and kept fp32
+    here -- so the two agree to 2^-11 of a row's magnitude, an order closer than either is to the fp32
+    path."""
+    from jitllm_amd import synthetic
+    say("packed gemv against the CPU quantized-activation dot", d, n)
+    raw = synthetic.weight(O.Q8_0, d, n, seed=1600 + d % 7)
+    x = synthetic.activations(n, seed=1601) * np.float32(1.5)
+    out = ctx.float_array(d, fill=POISON)
+    proj, ws = packed_projections(ctx, n)
+    proj.quantize(ctx.from_numpy(x), n)
+    w = ctx.load_weight(O.Q8_0, raw, d, n)
+    proj.packedMatvec(out, w, n, d)
+    ctx.sync()
+    got = out.get()
+    assert np.all(got != POISON)
+    ref = O.matmul(O.Q8_0, raw, x, d, n, O.DOT_Q8ACT)
+    mag = magnitude(O.Q8_0, raw, x, d, n)
+    close = rel_err(got, ref, mag)
+    far = rel_err(got, O.matmul(O.Q8_0, raw, x, d, n, O.DOT_VEC256), mag)
+    assert close < 6e-4, close
+    assert far > 4 * close, (close, far)
+    w.free()
+
+
 def test_packed_path_refusals(ctx):
     from jitllm_amd import synthetic
     from jitllm_amd._lib import JitllmHipError, UnsupportedProjection

@@ -781,3 +781,92 @@ def test_packed_projection_numpy_model(t):
         mag = (np.abs(dd[:, :, None]) * sc * sb * (nib * np.abs(qb)).sum(axis=3)
                + np.abs(dmin[:, :, None]) * mn * sb * np.abs(mb)).sum(axis=(1, 2))
     assert np.max(np.abs(got - want) / mag) < 2e-6
+
+
+# ---- Q8_0FloatTensor.dotQ8Activation (-Djitllm.quantizeActivation=true) --------------------------
+
+def _q8_0_row(quants, scales_f16):
+    """Q8_0 blocks from int8 values [blocks][32] and binary16 scales [blocks]."""
+    blocks = np.zeros((len(scales_f16), 34), dtype=np.uint8)
+    blocks[:, 0:2] = np.asarray(scales_f16, dtype=np.float16).view(np.uint8).reshape(-1, 2)
+    blocks[:, 2:] = np.asarray(quants, dtype=np.int8).view(np.uint8)
+    return blocks.reshape(-1)
+
+
+def test_quantized_activation_dot_is_exact_on_the_grid():
+    """Activations that lie on their own int8 grid with a power-of-two step, weights with power-of-two
+    scales: every step of dotQ8Activation (Q8_0FloatTensor.java:107-140) is exact, and the result is
+    the integer dot product times the scales -- evaluated here with Python integers and fractions."""
+    from fractions import Fraction
+    rng = np.random.default_rng(71)
+    blocks = 6
+    wq = rng.integers(-127, 128, size=(blocks, 32))
+    w_exp = rng.integers(-8, -2, size=blocks)
+    aq = rng.integers(-127, 128, size=(blocks, 32))
+    aq[:, 5] = 127 * rng.choice([-1, 1], size=blocks)       # the block maximum fixes the step
+    a_exp = rng.integers(-6, 4, size=blocks)
+    x = (aq * np.ldexp(1.0, a_exp)[:, None]).astype(np.float32).reshape(-1)
+    raw = _q8_0_row(wq, np.ldexp(1.0, w_exp))
+    want = sum(Fraction(int((wq[b] * aq[b]).sum())) * Fraction(2) ** int(w_exp[b] + a_exp[b]) for b in range(blocks))
+    got = O.dot(O.Q8_0, O.DOT_Q8ACT, raw, 0, x, 0, blocks * 32)
+    assert Fraction(float(got)) == want       # (the six terms and their running sums fit 24 bits)
+    # an offset into both operands, as matmul passes them: the last four blocks only
+    got = O.dot(O.Q8_0, O.DOT_Q8ACT, raw, 64, x, 64, (blocks - 2) * 32)
+    want = sum(Fraction(int((wq[b] * aq[b]).sum())) * Fraction(2) ** int(w_exp[b] + a_exp[b]) for b in range(2, blocks))
+    assert Fraction(float(got)) == want
+
+
+def test_quantized_activation_dot_rounding_and_scale():
+    """Halves round away from zero; the integers come from the fp32 scale while the sum is multiplied
+    by that scale rounded to binary16 (ggml's order, :123-127); a zero block adds nothing."""
+    ones = np.ones((1, 32), dtype=np.int64)
+    raw = _q8_0_row(ones, [1.0])
+    x = np.zeros(32, dtype=np.float32)
+    x[0] = 127.0                       # step 1: s = x
+    x[1:6] = [2.5, -2.5, 0.49999997, -0.49999997, 126.5]
+    # 127 + 3 - 3 + 0 - 0 + 127
+    assert O.dot(O.Q8_0, O.DOT_Q8ACT, raw, 0, x, 0, 32) == 254.0
+    # a step that is no binary16 number: 1 + 2^-12 rounds to 1, the integers still use 1 + 2^-12
+    step = np.float32(1.0) + np.float32(2.0 ** -12)
+    x = np.zeros(32, dtype=np.float32)
+    x[0] = np.float32(127.0) * step
+    x[1] = np.float32(100.4)
+    a_inv = np.float32(1.0) / (x[0] / np.float32(127.0))
+    q1 = int(np.float32(x[1] * a_inv) + np.float32(0.5))
+    assert O.dot(O.Q8_0, O.DOT_Q8ACT, raw, 0, x, 0, 32) == float(127 + q1)      # not (127 + q1) * step
+    assert O.dot(O.Q8_0, O.DOT_Q8ACT, raw, 0, np.zeros(32, np.float32), 0, 32) == 0.0
+    # a NaN among the activations quantizes to 0 (Java's (int) of NaN) and is no maximum
+    x = np.zeros(32, dtype=np.float32)
+    x[0], x[1] = 127.0, np.nan
+    assert O.dot(O.Q8_0, O.DOT_Q8ACT, raw, 0, x, 0, 32) == 127.0
+
+
+def test_quantized_activation_matmul_numpy_model():
+    """An independent numpy float32 statement on ordinary input, row by row, bit for bit; the result
+    is the true product to within the quantization step; the other types read the flavour as scalar."""
+    from jitllm_amd import synthetic
+    d, n = 9, 1024
+    raw = synthetic.weight(O.Q8_0, d, n, seed=72)
+    x = synthetic.activations(n, seed=73) * np.float32(2.3)
+    got = O.matmul(O.Q8_0, raw, x, d, n, O.DOT_Q8ACT)
+    b = raw.reshape(d, n // 32, 34)
+    dw = NP.half_bits_to_f32(b[:, :, 0:2].copy().view(np.uint16)[:, :, 0])
+    wq = b[:, :, 2:].view(np.int8).astype(np.int64)
+    xb = x.reshape(n // 32, 32)
+    amax = np.abs(xb).max(axis=1)
+    qs = (amax / np.float32(127.0)).astype(np.float32)
+    a_scale = qs.astype(np.float16).astype(np.float32)
+    a_inv = (np.float32(1.0) / qs).astype(np.float32)
+    s = (xb * a_inv[:, None]).astype(np.float32)
+    aq = (s + np.copysign(np.float32(0.5), s)).astype(np.float32).astype(np.int64)    # truncation toward zero
+    isum = (wq * aq[None, :, :]).sum(axis=2)
+    want = np.zeros(d, dtype=np.float32)
+    for blk in range(n // 32):
+        want = (want + isum[:, blk].astype(np.float32) * (dw[:, blk] * a_scale[blk]).astype(np.float32)).astype(np.float32)
+    assert_bit_equal(got, want)
+    w = NP.DEQUANT[O.Q8_0](raw).reshape(d, n).astype(np.float64)
+    exact, mag = w @ x.astype(np.float64), np.abs(w) @ np.abs(x.astype(np.float64))
+    assert np.max(np.abs(got - exact) / mag) < 5e-3
+    assert np.max(np.abs(got - exact) / mag) > 1e-6          # it is not the unquantized product
+    raw4 = synthetic.weight(O.Q4_0, d, n, seed=74)
+    assert_bit_equal(O.matmul(O.Q4_0, raw4, x, d, n, O.DOT_Q8ACT), O.matmul(O.Q4_0, raw4, x, d, n, O.DOT_SCALAR))
