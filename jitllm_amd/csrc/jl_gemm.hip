@@ -803,10 +803,10 @@ int launch_gemm(jl_context *ctx, const GemmParams &p, dim3 grid) {
     auto fn = jl_gemm_f16<TYPE, BM>;
     constexpr int lds = gemm_lds_bytes<TYPE, BM>();
     static_assert(lds <= 160 * 1024, "operand rings exceed the 160 KB of LDS");
-    static bool configured[16] = {};
-    if (ctx->device < 16 && !configured[ctx->device]) {
-        JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        configured[ctx->device] = true;
+    static jl_lds_limit_flags configured;
+    {
+        const int st = jl_raise_lds_limit(configured, ctx->device, (const void *)fn, lds);
+        if (st != JL_OK) return st;
     }
     hipLaunchKernelGGL(fn, grid, dim3(640), lds, ctx->stream, p);
     JL_HIP(hipGetLastError());

@@ -577,10 +577,10 @@ template <int BM, int BN>
 int launch_dense(jl_context *ctx, const DenseParams &p) {
     auto fn = jl_gemm_hh<BM, BN>;
     constexpr int lds = hh_stages<BM, BN>() * (BM + BN) * 128 + 1024;   // the ring and the prefetch's landing KB
-    static bool configured[16] = {};
-    if (ctx->device < 16 && !configured[ctx->device]) {
-        JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        configured[ctx->device] = true;
+    static jl_lds_limit_flags configured;
+    {
+        const int st = jl_raise_lds_limit(configured, ctx->device, (const void *)fn, lds);
+        if (st != JL_OK) return st;
     }
     const int items = p.ntiles * p.mtiles * p.splits;
     int wgs = items < ctx->compute_units ? items : ctx->compute_units;

@@ -437,10 +437,10 @@ int launch_i8(jl_context *ctx, const I8Params &p) {
     constexpr int region = 8 * BM < 1024 ? 1024 : 8 * BM;
     constexpr int stage = BM * 64 + Raw<TYPE>::kPlanes * BN * 16 + BN * 4 + region * (TYPE == JL_Q4_0 ? 2 : 1);
     constexpr int lds = 3 * stage;
-    static bool configured[16] = {};
-    if (ctx->device < 16 && !configured[ctx->device]) {
-        JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        configured[ctx->device] = true;
+    static jl_lds_limit_flags configured;
+    {
+        const int st = jl_raise_lds_limit(configured, ctx->device, (const void *)fn, lds);
+        if (st != JL_OK) return st;
     }
     const int total = p.ntiles * p.mtiles;
     const int grid = (total + 7) / 8 * 8;

@@ -1128,10 +1128,10 @@ int workgroups_per_span(int compute_units, int row_blocks, int Z, int groups) {
 template <int TYPE, int NBB, bool DUAL, int ZIN, bool HALF, bool XH>
 int launch_of(jl_context *ctx, const SkinnyParams &p, int threads, int lds, int groups) {
     auto fn = jl_gemm_skinny<TYPE, NBB, DUAL, ZIN, HALF, XH>;
-    static bool configured[16] = {};
-    if (ctx->device < 16 && !configured[ctx->device]) {
-        JL_HIP(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        configured[ctx->device] = true;
+    static jl_lds_limit_flags configured;
+    {
+        const int st = jl_raise_lds_limit(configured, ctx->device, (const void *)fn, 160 * 1024);
+        if (st != JL_OK) return st;
     }
     const int per_span = workgroups_per_span(ctx->compute_units, p.row_blocks, p.Z, groups);
     if (p.Z > 1 && per_span * p.row_blocks > JL_CONTEXT_ARRIVALS) {

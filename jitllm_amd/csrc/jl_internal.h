@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdint.h>
 #include <stdio.h>
 
@@ -92,6 +93,20 @@ int jl_fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3
             return jl_fail(e_ == hipErrorOutOfMemory ? JL_ERR_OOM : JL_ERR_HIP,           \
                            "%s failed: %s", #call, hipGetErrorString(e_));                \
     } while (0)
+
+// Raises a kernel's limit of dynamic LDS, once per kernel and device: `done` is the launcher's own
+// static array of flags, one per device index (contexts on several host threads may come through
+// here at once; an index past the array is configured on every call).
+struct jl_lds_limit_flags {
+    std::atomic<bool> done[16];
+};
+inline int jl_raise_lds_limit(jl_lds_limit_flags &flags, int device, const void *kernel, int bytes) {
+    const bool tracked = device >= 0 && device < 16;
+    if (tracked && flags.done[device].load(std::memory_order_acquire)) return JL_OK;
+    JL_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    if (tracked) flags.done[device].store(true, std::memory_order_release);
+    return JL_OK;
+}
 
 #define JL_REQUIRE(cond, ...)                                  \
     do {                                                       \

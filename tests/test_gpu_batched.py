@@ -1000,3 +1000,59 @@ def test_with_k_kept_whole_a_row_does_not_depend_on_the_chunk(ctx, t, residual):
         delta = got[:, :edge] - (base[:small, :edge] if residual else 0.0)
         assert rel_err(delta, ref, magnitude(t, raw[:edge * row_bytes], X[:small], edge, n)) < F16_BOUND
     w.free()
+
+
+def test_two_contexts_on_two_host_threads():
+    """Two host threads, a context (and stream) each, on the one device at the same time -- a second
+    session beside the first.  Every call's result is bit for bit what the same thread got the first
+    time, and the first meets the oracle: contexts share nothing that a call writes (their scratch,
+    arrival counters and workspaces are their own; the once-per-kernel set-up is guarded)."""
+    import threading
+
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections, QuantizedProjections, TornadoWorkspace
+    from jitllm_amd.runtime import Context
+    say("two contexts, two threads")
+    t, d, n = O.Q4_K, 1536, 2048
+    raws = [synthetic.weight(t, d, n, seed=9700 + i) for i in range(2)]
+    X = synthetic.activations((600, n), seed=9702)
+    failures = []
+
+    def session(index):
+        try:
+            with Context(0) as c:
+                w = c.load_weight(t, raws[index], d, n)
+                single = QuantizedProjections(c, TornadoWorkspace())
+                dx = c.from_numpy(X[0])
+                first = {}
+                for it in range(40):
+                    for rows in (1, 40, 200, 600):
+                        if rows == 1:
+                            out = c.float_array(d, fill=UNTOUCHED)
+                            single.floatMatvec(dx, out, w, n, d)
+                        else:
+                            proj = QuantizedBatchProjections(c, rows, n, d)
+                            out = c.float_array(rows * d, fill=UNTOUCHED)
+                            proj.projection(c.from_numpy(X[:rows]), out, w, n, d, False)
+                        c.sync()
+                        got = out.get().reshape(rows, d)
+                        out.free()
+                        if rows != 1:
+                            proj.workspace.free()
+                        if it == 0:
+                            first[rows] = got
+                            ref = O.matmul_batch(t, raws[index][:64 * (raws[index].size // d)], X[:rows], 64, n)
+                            mag = magnitude(t, raws[index][:64 * (raws[index].size // d)], X[:rows], 64, n)
+                            assert rel_err(got[:, :64], ref, mag) < F16_BOUND, (index, rows)
+                        else:
+                            assert np.array_equal(got.view(np.uint32), first[rows].view(np.uint32)), (index, it, rows)
+                w.free()
+        except BaseException as e:   # noqa: BLE001 -- handed to the main thread
+            failures.append((index, repr(e)))
+
+    threads = [threading.Thread(target=session, args=(i,)) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not failures, failures
