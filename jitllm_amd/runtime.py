@@ -17,10 +17,16 @@ from .ggml import GGMLType
 class Context:
     """One device and one stream (jl_context)."""
 
-    def __init__(self, device: int = 0):
+    def __init__(self, device: int = 0, stream: int | None = None):
+        """``stream``: a hipStream_t the caller owns (an integer handle, e.g. a
+        ``torch.cuda.Stream().cuda_stream``); the context then enqueues on it and never destroys it.
+        Without one the context makes a stream of its own."""
         self._lib = L.load()
         h = C.c_void_p()
-        L.check(self._lib.jl_context_create(device, C.byref(h)))
+        if stream is None:
+            L.check(self._lib.jl_context_create(device, C.byref(h)))
+        else:
+            L.check(self._lib.jl_context_create_on_stream(device, C.c_void_p(stream), C.byref(h)))
         self.handle = h
         self.device = device
 

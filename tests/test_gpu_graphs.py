@@ -154,3 +154,44 @@ def test_prefill_calls_replayed(ctx, hip, mode):
     for w in (wo, w1, w3, w2):
         w.free()
     proj.workspace.free()
+
+
+# ---- streams and device memory that belong to the caller -------------------------------------------
+
+def test_context_on_a_stream_the_caller_owns():
+    """jl_context_create_on_stream: the calls are enqueued on the caller's stream (an event the caller
+    records there after the call covers them), jl_context_stream hands the same handle back, and
+    destroying the context leaves the stream alive."""
+    import ctypes as C
+
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    from jitllm_amd.runtime import Context
+    say("a context on the caller's stream")
+    rt = C.CDLL("libamdhip64.so")
+    rt.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+    rt.hipStreamSynchronize.argtypes = [C.c_void_p]
+    rt.hipStreamDestroy.argtypes = [C.c_void_p]
+    rt.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+    rt.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+    rt.hipEventSynchronize.argtypes = [C.c_void_p]
+    rt.hipEventDestroy.argtypes = [C.c_void_p]
+    stream, done = C.c_void_p(), C.c_void_p()
+    assert rt.hipStreamCreate(C.byref(stream)) == 0 and rt.hipEventCreate(C.byref(done)) == 0
+    t, d, n = O.Q8_0, 4096, 2048
+    raw = synthetic.weight(t, d, n, seed=9870)
+    x = synthetic.activations(n, seed=9871)
+    c = Context(0, stream=stream.value)
+    assert c.stream == stream.value
+    w = c.load_weight(t, raw, d, n)
+    out = c.float_array(d, fill=UNTOUCHED)
+    QuantizedProjections(c, TornadoWorkspace()).floatMatvec(c.from_numpy(x), out, w, n, d)
+    assert rt.hipEventRecord(done, stream) == 0 and rt.hipEventSynchronize(done) == 0
+    got = out.get()
+    ref = O.matmul(t, raw, x, d, n, O.DOT_VEC256)
+    assert np.max(np.abs(got - ref)) <= 2e-5 * np.max(np.abs(ref)) * 50
+    assert np.all(got != UNTOUCHED)
+    w.free()
+    c.close()
+    assert rt.hipStreamSynchronize(stream) == 0      # still the caller's to use
+    assert rt.hipEventDestroy(done) == 0 and rt.hipStreamDestroy(stream) == 0
