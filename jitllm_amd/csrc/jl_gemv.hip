@@ -716,8 +716,15 @@ __device__ __forceinline__ uintptr_t uniform_value(uintptr_t v) {
 // (ARGMAX: a plain projection whose rows lie inside a wave also keeps, per workgroup, the largest
 // value it stored and that value's row -- greedy sampling then folds a thousand cells instead of
 // reading the logits back.)
+// (HALVES: rows of more than 256 slices, up to 512 -- 16 448 to 32 768 columns, the down projections of
+// the largest models.  A row of 2 m columns is, byte for byte, two consecutive rows of m columns, so
+// the launch describes the weight as [2 d x m]: even rows meet the first half of the activation
+// vector, odd rows the second.  A tile holds four such half rows, so a thread always serves the same
+// half and keeps its 64 activations in registers as ever; they come straight from global memory, as
+// the vector is longer than a ring stage.  The thread that finishes a row adds its two halves'
+// partial sums.)
 template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false,
-          bool PART = false, bool ARGMAX = false>
+          bool PART = false, bool ARGMAX = false, bool HALVES = false>
 __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first, const uint8_t *w_up_first, const float *x_first, int tiles_first,
               int rows_first, int grid_first, int S_first, int row_bytes_first, int shape_first,
               const float *rms_w_first, GemvParams p) {
@@ -734,6 +741,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     static_assert(!PART || LEAN, "rows shorter than SPT slices: a fixed tile shape");
     static_assert(!LEAN || !PACKED, "the packed form has no fixed-geometry instances");
     static_assert(!ARGMAX || (FULL && !DUAL && !SEGS && SPT <= 64), "the argmax form: whole in-wave rows of one weight");
+    static_assert(!HALVES || (PART && !DUAL && !RMS && !PACKED && !SEGS && !ARGMAX && THREADS == 1024 && SPT == 256),
+                  "rows in two halves: the plain 1024-thread form");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int X4 = Traits<TYPE>::kX4;        // 16-byte loads per thread and tile
     constexpr int L = X4 + Traits<TYPE>::kTail;   // plus (three main types) one 4-byte load
@@ -887,7 +896,7 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
     uint8_t *xs = x_in_ring ? ring + (kStages - 1) * stage_bytes : ring + kStages * stage_bytes;
     const uint32_t xs0 = x_in_ring ? ring0 + (kStages - 1) * stage_bytes : ring0 + kStages * stage_bytes;
     int issued = 0;
-    if constexpr (!rms && !PACKED) {
+    if constexpr (!rms && !PACKED && !HALVES) {
         for (int base = 0; base < x_bytes; base += nthreads * 16) {
             const int q = base / 16 + tid;
             const int sl = q / 17, k = q - sl * 17;
@@ -1002,7 +1011,16 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
         pack_x<TYPE>(raw, px);
     } else {
         // (threads with no slice never use theirs: the dot product below is skipped for them)
-        if (active) {
+        if constexpr (HALVES) {
+            if (active) {
+                const float4 *src = (const float4 *)(x_first + ((r & 1) * S + s) * 64);
+#pragma unroll
+                for (int k = 0; k < 16; k++) {
+                    const float4 v4 = src[k];
+                    x[4 * k] = v4.x; x[4 * k + 1] = v4.y; x[4 * k + 2] = v4.z; x[4 * k + 3] = v4.w;
+                }
+            }
+        } else if (active) {
 #pragma unroll
             for (int k = 0; k < 4; k++) lds_read_16f(xs0 + s * 272 + k * 64, &x[k * 16]);
         }
@@ -1038,6 +1056,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
             float v0 = __uint_as_float(lds_read_b32(pb + tid * 4));
             float v1 = 0.f;
             if constexpr (DUAL) v1 = __uint_as_float(lds_read_b32(pb + (slots + tid) * 4));
+            // (the row's other half lies P partials further on, or back)
+            if constexpr (HALVES) v0 += __uint_as_float(lds_read_b32(pb + (tid ^ P) * 4));
             if (P > 1) {
                 const int width = P < JL_WAVE ? P : JL_WAVE;
                 v0 = group_sum(v0, width);
@@ -1062,8 +1082,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
                 }
             }
             const int row = local * half_rows + j;
-            if (tid - j * P == 0 && (LEAN || row < seg_rows)) {
-                float *o = out + row;
+            if (tid - j * P == 0 && (LEAN || row < seg_rows) && (!HALVES || (j & 1) == 0)) {
+                float *o = out + (HALVES ? row >> 1 : row);
                 if constexpr (DUAL) {
                     *o = jl_swiglu_value(v0, v1);
                 } else {
@@ -1293,9 +1313,9 @@ int blocks_per_cu(const void *fn, int device, int threads, int lds) {
 }
 
 template <int TYPE, bool DUAL, bool RMS, bool PACKED = false, int THREADS = 256, int SPT = 0, bool SEGS = false,
-          bool PART = false, bool ARGMAX = false>
+          bool PART = false, bool ARGMAX = false, bool HALVES = false>
 int launch_tiles_of(jl_context *ctx, const GemvParams &p, int threads, int lds, int *cells = nullptr) {
-    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED, THREADS, SPT, SEGS, PART, ARGMAX>;
+    auto fn = jl_gemv_tiles<TYPE, DUAL, RMS, PACKED, THREADS, SPT, SEGS, PART, ARGMAX, HALVES>;
     int per_cu = blocks_per_cu((const void *)fn, ctx->device, threads, lds);
     int total = p.seg_tile_begin[p.nseg];
     int grid = ctx->compute_units * per_cu;
@@ -1430,6 +1450,32 @@ int jl_launch_gemv(jl_context *ctx, const jl_weight *const *w, int nseg, float *
     const bool dual = w_up != nullptr;
     // bytes a thread brings in per tile
     const int slice = type == JL_Q8_0 ? 68 : type == JL_Q6_K ? 64 : is_side_type(type) ? 48 : 36;
+    // Rows of 16 448 .. 32 768 columns, plain and residual projections of the three main types: the
+    // weight seen as [2 rows x n / 2] (the kernel's HALVES form); a half row is whole blocks, a tile
+    // -- four half rows, two rows -- whole 16-byte pieces.
+    if (is_main_type(type) && !dual && !rms && !xq && !cells && nseg == 1 && n > 16384 && n <= 32768 &&
+        n % 128 == 0 && (n / 2) % jl_block_elems(type) == 0 && w[0]->rows % 2 == 0 && ((uintptr_t)x & 15) == 0 &&
+        ((uintptr_t)w[0]->blocks & 15) == 0 && ((int64_t)2 * row_bytes) % 16 == 0) {
+        GemvParams h{};
+        h.nseg = 1;
+        h.w[0] = w[0]->blocks;
+        h.out[0] = outs[0];
+        h.seg_rows[0] = 2 * (int)w[0]->rows;
+        h.seg_tile_begin[1] = (int)w[0]->rows / 2;
+        h.x = x;
+        h.n = n;
+        h.S = n / 128;
+        h.Sp = 256;
+        h.R = 4;
+        h.row_bytes = row_bytes / 2;
+        h.epilogue = epilogue;
+        const int lds = kPartialBytes + kStages * kWideThreads * slice;
+        switch (type) {
+            case JL_Q8_0: return launch_tiles_of<JL_Q8_0, false, false, false, kWideThreads, 256, false, true, false, true>(ctx, h, kWideThreads, lds);
+            case JL_Q4_0: return launch_tiles_of<JL_Q4_0, false, false, false, kWideThreads, 256, false, true, false, true>(ctx, h, kWideThreads, lds);
+            default: return launch_tiles_of<JL_Q4_K, false, false, false, kWideThreads, 256, false, true, false, true>(ctx, h, kWideThreads, lds);
+        }
+    }
     bool fast = (n % 64 == 0) && (n / 64 <= 256) &&
                 (xq ? (((uintptr_t)xq->quants & 15) == 0 && ((uintptr_t)xq->scales & 7) == 0 &&
                        ((uintptr_t)xq->sums & 7) == 0)

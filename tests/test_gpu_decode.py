@@ -849,3 +849,41 @@ def test_results_do_not_change_from_run_to_run(ctx, t):
     first, second = run(), run()
     for a, b in zip(first, second):
         assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("t,d,n", [(O.Q8_0, 512, 17408), (O.Q4_K, 256, 27648), (O.Q4_0, 64, 28672), (O.Q4_K, 6, 32768),
+                                   (O.Q8_0, 10, 16512), (O.Q4_0, 1026, 25600), (O.Q4_K, 2048, 25600),
+                                   (O.Q8_0, 7, 17408), (O.Q4_0, 4, 16416)])
+def test_rows_of_more_than_16384_columns(ctx, t, d, n):
+    """The down projections of the largest models (17 408, 25 600, 27 648, 28 672 columns): a thread of
+    the tile kernel owns 64 columns and a workgroup has 1 024 threads, so such a row is taken as two
+    half rows whose sums meet in the thread that finishes the row.  Plain and residual, against the
+    oracle on every output, twice with the same bits; an odd row count and a row length that does not
+    halve into whole 64-column slices (the last two cases) go to the catch-all kernel and hold too."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedProjections, TornadoWorkspace
+    say("long rows", t, d, n)
+    raw = synthetic.weight(t, d, n, seed=9900 + d)
+    x = synthetic.activations(n, seed=9901)
+    base = synthetic.activations(d, seed=9902)
+    w = ctx.load_weight(t, raw, d, n)
+    dx = ctx.from_numpy(x)
+    ref = O.matmul(t, raw, x, d, n, O.DOT_SCALAR if t == O.Q4_K else O.DOT_VEC256)
+    mag = magnitude(t, raw, x, d, n)
+    runs = []
+    for _ in range(2):
+        out = ctx.float_array(d, fill=POISON)
+        acc = ctx.from_numpy(base.copy())
+        proj = QuantizedProjections(ctx, TornadoWorkspace(wrapX=acc))
+        proj.floatMatvec(dx, out, w, n, d)
+        proj.residualMatvec(dx, w, n, d)
+        ctx.sync()
+        runs.append((out.get(), acc.get()))
+        out.free()
+        acc.free()
+    got, added = runs[0]
+    assert np.all(got != POISON)
+    assert rel_err(got, ref, mag) < 2e-5
+    assert rel_err(added - base, ref, mag + np.abs(base) * 1e-6) < 2e-5
+    assert bits_equal(got, runs[1][0]) and bits_equal(added, runs[1][1])
+    w.free()
