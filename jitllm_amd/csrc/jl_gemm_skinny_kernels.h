@@ -1164,17 +1164,20 @@ int launch_nbb(jl_context *ctx, const SkinnyParams &p, int nbb, int zin, int thr
 
 }  // namespace
 
-// Sets *taken to false, launching nothing, when the shape is not one this kernel takes; the caller
-// then uses the tiled GEMM.  (JL_SKINNY_XH: X16 is read, else X.)
-int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
-                    const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
-                    int epilogue, float *planes, size_t plane_bytes, double other_us, bool *taken) {
+// One launch over a window of the weights' columns: `window_slices` 64-column slices from slice
+// `first_slice` on (0 slices: the whole row).  The kernel needs nothing for it but bases that start at
+// the window -- a weight row's stride and an activation row's stride stay those of the whole row.
+// `probe`: says in *taken whether the launch would be made, and makes none.
+static int skinny_window(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
+                         const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
+                         int epilogue, float *planes, size_t plane_bytes, double other_us, bool *taken,
+                         int first_slice, int window_slices, bool probe) {
     *taken = false;
     const int type = weights[0]->type;
     const int k = (int)weights[0]->cols;
     const bool dual = epilogue == JL_SWIGLU;
     if (rows >= 512 || k % 256 != 0 || count > kMaxSeg) return JL_OK;
-    const int S = k / 64;
+    const int S = window_slices ? window_slices : k / 64;
     const int row_blocks = (rows + 31) / 32;
     const int nbb = jl_skinny_padded_rows(rows) / 16;
     const int quad = quad_bytes(type);
@@ -1185,7 +1188,7 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
     // bytes, IQ4_XS: 2 of 136), and so is a row
     int Ss = max_slices(nbb);
     while (Ss > 4 && (S % Ss || (Ss / 4 * quad) % 16)) Ss -= 4;
-    if (S % Ss || (Ss / 4 * quad) % 16 || (S / 4 * quad) % 16) return JL_OK;
+    if (S % Ss || (Ss / 4 * quad) % 16 || (k / 256 * quad) % 16 || (first_slice / 4 * quad) % 16) return JL_OK;
     // up to 16 rows: a workgroup walks two spans itself (no partial sums to fold for rows of up to
     // 4096 columns); more rows leave no registers for a second set of activation fragments
     const int zin = (nbb == 1 && (S / Ss) % 2 == 0) ? 2 : 1;
@@ -1212,7 +1215,7 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
     int groups = 0, col = 0;
     const int per_group = dual ? 8 : 16;
     for (int i = 0; i < p.nseg; i++) {
-        p.w[i] = weights[i]->blocks;
+        p.w[i] = weights[i]->blocks + (int64_t)(first_slice / 4) * quad;
         p.seg_rows[i] = (int)weights[i]->rows;
         p.seg_group_begin[i] = groups;
         p.seg_col_begin[i] = col;
@@ -1221,7 +1224,7 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
     }
     p.seg_group_begin[p.nseg] = groups;
     p.w_up = dual ? weights[1]->blocks : nullptr;
-    p.X = JL_SKINNY_XH ? (const float *)X16 : X;
+    p.X = JL_SKINNY_XH ? (const float *)(X16 + (int64_t)first_slice * 64) : X + (int64_t)first_slice * 64;
     p.C = C;
     p.c_f16 = c_f16 ? 1 : 0;
     p.planes = planes;
@@ -1252,6 +1255,7 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
     p.stages = stages;
     const int lds = partial + stages * stage_bytes;
     *taken = true;
+    if (probe) return JL_OK;
 
     switch (type) {
         case JL_Q8_0:
@@ -1282,4 +1286,40 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
             *taken = false;
             return JL_OK;
     }
+}
+
+// Sets *taken to false, launching nothing, when the shape is not one this kernel takes; the caller
+// then uses the tiled GEMM.  (JL_SKINNY_XH: X16 is read, else X.)
+int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count, const float *X,
+                    const _Float16 *X16, float *C, bool c_f16, int rows, int64_t ldo, int64_t col_offset,
+                    int epilogue, float *planes, size_t plane_bytes, double other_us, bool *taken) {
+    // A row is cut into equal spans of whole 256-column blocks, at most eight blocks each, one compute
+    // wave per block: a row of 43 blocks (11 008 columns, the feed-forward width of many 7B models) or
+    // of 74 (18 944) has no such cut but spans of one or two blocks, on one or two compute waves.  Up
+    // to 64 rows, a plain or residual projection over such a row is two launches instead: the whole
+    // eights of its blocks, then the rest as one span that adds to what the first left.
+    *taken = false;
+    const int k = (int)weights[0]->cols;
+    const int blocks = k / 256;
+    int widest = 8;
+    while (widest > 1 && blocks % widest) widest--;
+    if (epilogue != JL_SWIGLU && rows <= 64 && k % 256 == 0 && blocks > 8 && widest < 5 && blocks % 8 != 0) {
+        const int head = blocks / 8 * 8, tail = blocks - head;
+        bool head_ok = false, tail_ok = false;
+        int st = skinny_window(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, epilogue, planes, plane_bytes,
+                               other_us, &head_ok, 0, head * 4, true);
+        if (st == JL_OK)
+            st = skinny_window(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, JL_RESIDUAL, planes,
+                               plane_bytes, other_us, &tail_ok, head * 4, tail * 4, true);
+        if (st != JL_OK) return st;
+        if (head_ok && tail_ok) {
+            st = skinny_window(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, epilogue, planes, plane_bytes,
+                               other_us, taken, 0, head * 4, false);
+            if (st != JL_OK) return st;
+            return skinny_window(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, JL_RESIDUAL, planes,
+                                 plane_bytes, other_us, taken, head * 4, tail * 4, false);
+        }
+    }
+    return skinny_window(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, epilogue, planes, plane_bytes,
+                         other_us, taken, 0, 0, false);
 }
