@@ -755,7 +755,7 @@ namespace {
 // work items to cover the chip, at least 2 raw stages (512 columns) per split, and partial-sum
 // traffic (written once, read once) bounded by the weight bytes: splits * padded_rows <=
 // row_bytes / 2.  A divisor of the stage count.
-int choose_splits(int rows, int bm, int k, int tiles, int row_bytes, int compute_units) {
+int choose_splits(int rows, int bm, int k, int tiles, int row_bytes, int compute_units, int *unconstrained = nullptr) {
     const int ksteps = k / (BK * SUPER);  // raw stages of 256 columns
     const int padded = (rows + bm - 1) / bm * bm;
     int want = rows <= 64 ? (2 * compute_units + tiles - 1) / tiles : compute_units / tiles;
@@ -764,6 +764,7 @@ int choose_splits(int rows, int bm, int k, int tiles, int row_bytes, int compute
     int s = want < by_steps ? want : by_steps;
     if (by_traffic < s) s = by_traffic;
     if (s < 1) s = 1;
+    if (unconstrained) *unconstrained = s;
     while (ksteps % s) s--;
     return s;
 }
@@ -922,6 +923,18 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     // hundreds of MB of Q8_0 at up to 128 rows, a vocabulary projection -- 147 us for 279 MB)
     double in_loop_us = 22.0 + (type == JL_Q8_0 ? 0.30 : 0.37) * ((rows + 127) / 128) * millions;
     if (in_loop_us < weight_bytes / 1.9e6) in_loop_us = weight_bytes / 1.9e6;
+    // (that kernel cuts K into equal runs of whole 256-column stages: a stage count with no divisor
+    // near the cut it wants -- 43 stages, 11 008 columns: prime -- leaves it a few dozen work items
+    // that each walk most of K, and the call takes as many times longer as the runs are too long:
+    // measured 137 us where the fit says 39)
+    if (rows > 64 && k % 256 == 0) {
+        const int tiles = ((virt + 127) / 128) * (((int)rows + 127) / 128);
+        int wanted = 1;
+        const int got = ctx->split_k ? choose_splits((int)rows, 128, k, tiles, k / jl_block_elems(type) * jl_block_bytes(type),
+                                                     ctx->compute_units, &wanted)
+                                     : 1;
+        if (ctx->split_k && wanted >= 2 * got) in_loop_us = 22.0 + (in_loop_us - 22.0) * wanted / got;
+    }
     if (dense_only || (kept && rows >= 192)) in_loop_us = 1e30;
     const double copy_us = kept && rows >= 128 ? 24.0 + 0.45 * ((rows + 255) / 256) * millions
                            : dense_only       ? 30.0 + 2.8 * millions

@@ -1202,7 +1202,7 @@ static int skinny_window(jl_context *ctx, const jl_weight *const *weights, int c
         // Q5_K) at 65 .. 384 rows: 10 + 0.155 x row blocks x million weights / share of the chip in use.
         double millions = 0.0;
         int all_groups = 0;
-        for (int i = 0; i < count; i++) millions += (double)weights[i]->rows * k * 1e-6;
+        for (int i = 0; i < count; i++) millions += (double)weights[i]->rows * (S * 64) * 1e-6;   // (of the window)
         for (int i = 0; i < (dual ? 1 : count); i++) all_groups += ((int)weights[i]->rows + (dual ? 8 : 16) - 1) / (dual ? 8 : 16);
         const int per_span = workgroups_per_span(ctx->compute_units, row_blocks, Z, all_groups);
         double share = (double)per_span * Z * row_blocks / ctx->compute_units;
@@ -1296,7 +1296,7 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
     // A row is cut into equal spans of whole 256-column blocks, at most eight blocks each, one compute
     // wave per block: a row of 43 blocks (11 008 columns, the feed-forward width of many 7B models) or
     // of 74 (18 944) has no such cut but spans of one or two blocks, on one or two compute waves (100
-    // blocks, 25 600 columns: five).  Up to 64 rows, a plain or residual projection over a row whose
+    // blocks, 25 600 columns: five).  A plain or residual projection over a row whose
     // widest equal span is under six blocks is two launches instead: the whole eights of its blocks,
     // then the rest as one span that adds to what the first left (measured: 4-14 x at 11 008 columns,
     // 3-5 x at 18 944, 1.4 x at 64 rows of 25 600).
@@ -1305,7 +1305,7 @@ int JL_SKINNY_ENTRY(jl_context *ctx, const jl_weight *const *weights, int count,
     const int blocks = k / 256;
     int widest = 8;
     while (widest > 1 && blocks % widest) widest--;
-    if (epilogue != JL_SWIGLU && rows <= 64 && k % 256 == 0 && blocks > 8 && widest < 6 && blocks % 8 != 0) {
+    if (epilogue != JL_SWIGLU && rows < 512 && k % 256 == 0 && blocks > 8 && widest < 6 && blocks % 8 != 0) {
         const int head = blocks / 8 * 8, tail = blocks - head;
         bool head_ok = false, tail_ok = false;
         int st = skinny_window(ctx, weights, count, X, X16, C, c_f16, rows, ldo, col_offset, epilogue, planes, plane_bytes,
