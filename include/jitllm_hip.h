@@ -353,7 +353,9 @@ size_t jl_gemm_workspace_bytes(int64_t max_rows, int64_t cols, int64_t out_cols,
  *            are multiples of 64.  An opt-in mode: an activation carries 7 bits, so against the
  *            fp32 CPU path it is looser than JL_MATH_F16 (every output within sum over the blocks
  *            of (dA / 2) * sum |w|).
- * JL_MATH_F16: the row length must be a multiple of 256 columns, else JL_ERR_UNSUPPORTED.  The
+ * JL_MATH_F16: the row length must be a multiple of 64 columns, else JL_ERR_UNSUPPORTED (rows of
+ * whole 256-column blocks have kernels for every row count; others -- 896 columns -- are decoded to
+ * fp16 in the workspace on every call, as the types without a fused kernel are).  The
  * weights of a call may differ in type (a "Q4_K_M" file's q | k | v with v in Q6_K; a gate and an up
  * weight of different types): each is then decoded to fp16 by its own type and one fp16 GEMM
  * multiplies them, as the reference's prefill projections do (FP16Projections.project,

@@ -866,9 +866,9 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
         return jl_launch_gemm_i8(ctx, weights, count, X, C, batch, (int)active_rows, ldo, col_offset, epilogue,
                                  workspace, workspace_bytes);
     }
-    if (k % 256 != 0) {
+    if (k % 64 != 0) {
         return jl_fail(JL_ERR_UNSUPPORTED,
-                       "jl_gemm: no batched kernel for a row length of %d (a multiple of 256 is needed)", k);
+                       "jl_gemm: no batched kernel for a row length of %d (a multiple of 64 is needed)", k);
     }
     const _Float16 *X16 = half ? half->x16 : nullptr;
     const bool c_f16 = half && half->c_f16;
@@ -897,7 +897,9 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     // fp16 GEMM does not know the difference.
     bool mixed = false;
     for (int i = 1; i < count; i++) mixed = mixed || weights[i]->type != type;
-    const bool dense_only = mixed || !jl_has_fused_kernels(type);
+    // (and so do rows that are whole 64-column steps but not whole 256-column blocks -- 896 columns,
+    // the width of the smallest Qwen2.5 -- which the other two kernels' spans and stages cannot cut)
+    const bool dense_only = mixed || !jl_has_fused_kernels(type) || k % 256 != 0;
     const size_t copy_bytes = round_up(jl_dense_copy_bytes(k, virt), 256);
     // the decoded copy goes to the caller's resident buffer when there is one that holds it,
     // otherwise to the head of the workspace's third region

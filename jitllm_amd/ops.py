@@ -321,7 +321,7 @@ class HipImplementation(Implementation):
         # (DequantizingMatMul.java:53-63)
         if len({m.columns for m in mm}) != 1:
             return False
-        if mm[0].columns % 256:
+        if mm[0].columns % 64:
             return False
         if step.fusion.name == GATE_UP_SWIGLU.name and mm[0].rows != mm[1].rows:
             return False

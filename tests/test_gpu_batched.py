@@ -1100,3 +1100,42 @@ def test_row_lengths_with_no_equal_spans(ctx, t, d, n, rows, active, residual, h
     assert rel_err(delta, ref, magnitude(t, part, X[:active], cols, n) + (np.abs(base[:active, :cols]) * 1e-6 if residual else 0.0)) < F16_BOUND
     proj.workspace.free()
     w.free()
+
+
+@pytest.mark.parametrize("t,n", [(O.Q8_0, 896), (O.Q4_0, 896), (O.Q8_0, 1600), (O.Q5_0, 2112)])
+@pytest.mark.parametrize("rows", [3, 64, 200, 640])
+def test_row_lengths_that_are_not_whole_256_column_blocks(ctx, t, n, rows):
+    """896 columns (the width of the smallest Qwen2.5) are whole 64-column steps but three and a half
+    256-column blocks: such rows take the decode-once path at every row count -- a projection, q | k
+    side by side and gate/up + SwiGLU against the oracle."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("rows that are no whole 256-column blocks", t, n, rows)
+    d, dk = 328, 136
+    r1, r3 = synthetic.weight(t, d, n, seed=9920), synthetic.weight(t, d, n, seed=9921)
+    rk = synthetic.weight(t, dk, n, seed=9922)
+    w1, w3, wk = ctx.load_weight(t, r1, d, n), ctx.load_weight(t, r3, d, n), ctx.load_weight(t, rk, dk, n)
+    X = synthetic.activations((rows, n), seed=9923)
+    proj = QuantizedBatchProjections(ctx, rows, n, 2 * d)
+    dx = ctx.from_numpy(X)
+    out, hb = ctx.float_array(rows * d, fill=UNTOUCHED), ctx.float_array(rows * d, fill=UNTOUCHED)
+    side = ctx.float_array(rows * (d + 2 * dk), fill=UNTOUCHED)
+    proj.projection(dx, out, w1, n, d, False)
+    proj.fusedQKV(dx, side, w1, wk, wk)
+    proj.gateUp(dx, hb, w1, w3, n, d)
+    ctx.sync()
+    g, u = O.matmul_batch(t, r1, X, d, n), O.matmul_batch(t, r3, X, d, n)
+    mg, mu = magnitude(t, r1, X, d, n), magnitude(t, r3, X, d, n)
+    assert rel_err(out.get().reshape(rows, d), g, mg) < F16_BOUND
+    s = side.get().reshape(rows, d + 2 * dk)
+    assert rel_err(s[:, :d], g, mg) < F16_BOUND
+    kref, mk = O.matmul_batch(t, rk, X, dk, n), magnitude(t, rk, X, dk, n)
+    assert rel_err(s[:, d:d + dk], kref, mk) < F16_BOUND and rel_err(s[:, d + dk:], kref, mk) < F16_BOUND
+    got = hb.get().reshape(rows, d).astype(np.float64)
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    want = g64 / (1.0 + np.exp(-g64)) * u64
+    bound = F16_BOUND * (mg * (np.abs(u64) + mu) + mu * np.abs(g64)) + 1e-6
+    assert np.all(np.abs(got - want) <= bound)
+    for w in (w1, w3, wk):
+        w.free()
+    proj.workspace.free()

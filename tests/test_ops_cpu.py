@@ -63,7 +63,7 @@ def test_the_first_accepting_candidate_takes_each_step():
 
 
 def test_what_the_library_cannot_run_falls_to_the_next_candidate_or_is_named():
-    odd = llama_layer(dim=2080)                      # row length not a multiple of 256
+    odd = llama_layer(dim=2080)                      # row length not a multiple of 64
     chosen = ops.split(odd, 0, T, [HipImplementation(), JitNorms()], Target())
     assert all(c.implementation.library() == "none" for c in chosen if c.step.matMuls()
                and c.step.matMuls()[0].columns == 2080)
