@@ -401,3 +401,31 @@ def test_random_int8_calls(ctx, chunk):
             w.free()
         out.free()
         proj.workspace.free()
+
+
+# ---- the same generators over row lengths that leave the usual kernels ----------------------------
+
+AWKWARD_BATCHED = [2816, 4864, 5632, 6912, 11008, 13824, 18944, 25600]     # 11, 19, 22, 27, 43, 54, 74, 100 blocks of 256
+LONG_SINGLE = [16640, 17408, 18944, 22016, 25600, 27648, 28672, 32768]     # past the 16 384 columns a workgroup spans
+
+
+@pytest.mark.parametrize("chunk", range(3))
+def test_random_calls_over_awkward_row_lengths(ctx, chunk, monkeypatch):
+    """Batched calls over rows whose blocks have no cut into equal spans (served as two column windows,
+    or by the in-loop kernel, or decoded once), and single-token calls over rows longer than a
+    workgroup spans (the two-halves form of the tile kernel, or the catch-all kernel)."""
+    import sys
+    me = sys.modules[__name__]
+    rng = np.random.default_rng(20261300 + chunk)
+    monkeypatch.setattr(me, "ROW_LENGTHS", AWKWARD_BATCHED)
+    for i in range(20):
+        c = batched_case(rng)
+        if c["batch"] * c["ldo"] > 30_000_000:
+            continue
+        say("random batched call, awkward row length", chunk, i, c)
+        run_batched_case(ctx, c, seed=(chunk * 100 + i) * 16 + 13000)
+    monkeypatch.setattr(me, "ROW_LENGTHS", LONG_SINGLE)
+    for i in range(30):
+        c = single_case(rng)
+        say("random single-token call, long rows", chunk, i, c)
+        run_single_case(ctx, c, seed=(chunk * 100 + i) * 16 + 14000)
