@@ -1207,7 +1207,8 @@ __global__ void __launch_bounds__(THREADS) jl_gemv_tiles(const uint8_t *w_first,
 }
 
 // Catch-all for shapes the tile kernel does not take (row length not a multiple of 64, rows wider
-// than 16384 columns, unaligned buffers): one wave per row, lanes stride over blocks, byte loads.
+// than 16384 columns that the two-halves form does not take either, unaligned buffers): one wave per
+// row, lanes stride over blocks, byte loads.
 template <int TYPE>
 __device__ float block_dot_generic(const uint8_t *blk, const float *x) {
     float acc = 0.f;
@@ -1351,8 +1352,9 @@ int launch_fixed(jl_context *ctx, const GemvParams &p, int lds, bool full) {
 
 // `fixed`: the launch meets the fixed-geometry form's conditions (whole tiles only in every
 // weight).  The three main types have an instance for every variant at row lengths of 513 ... 8192
-// columns and, in the 1024-thread form (plain and residual), up to 16384; the side types for
-// whole rows of 2048, 4096 and (plain and residual) 8192 columns.
+// columns and, in the 1024-thread form (plain and residual), up to 16384 -- and, a row taken as two
+// half rows, up to 32768 (launched from jl_launch_gemv itself); the side types for whole rows of
+// 2048, 4096 and (plain and residual) 8192 columns.
 template <int TYPE, bool DUAL>
 int launch_tiles(jl_context *ctx, const GemvParams &p, int threads, int lds, bool fixed, int *cells = nullptr) {
     // (side types: plain, residual and gate/up only -- the caller has refused the rest)
