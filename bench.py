@@ -1073,6 +1073,46 @@ def vocabulary_probe(ctx):
     print(json.dumps({"weight_bytes": int(host.size)}))
 
 
+def shapes_probe(ctx):
+    """What the kernel trace of the shapes beside the benchmark's is collected on: single-token
+    projections over rows longer than 16 384 columns (the two-halves form of the tile kernel) and batched
+    decode over rows whose blocks have no cut into equal spans (two column windows), each beside a
+    well-shaped neighbour, kernel by kernel over three device copies in turn, four rounds each."""
+    from jitllm_amd import synthetic
+    from jitllm_amd.ggml import GGMLType
+    from jitllm_amd.projections import QuantizedBatchProjections, QuantizedProjections, TornadoWorkspace
+    shapes = {}
+    for name, d, n in (("Q8_0", 5120, 16384), ("Q8_0", 5120, 17408), ("Q4_K", 5120, 27648), ("Q4_0", 8192, 28672)):
+        t = GGMLType[name]
+        host = synthetic.weight(t, d, n, 95)
+        ws = [ctx.load_weight(t, host, d, n) for _ in range(3)]
+        proj = QuantizedProjections(ctx, TornadoWorkspace())
+        x, out = ctx.from_numpy(synthetic.activations(n, 96)), ctx.float_array(d)
+        for _ in range(4):
+            for w in ws:
+                proj.floatMatvec(x, out, w, n, d)
+            ctx.sync()
+        shapes["gemv %s %d x %d" % (name, d, n)] = int(host.size)
+        for w in ws:
+            w.free()
+    for name, d, n in (("Q4_K", 4096, 12288), ("Q4_K", 4096, 11008), ("Q8_0", 4096, 11008), ("Q4_K", 3584, 18944)):
+        t = GGMLType[name]
+        host = synthetic.weight(t, d, n, 97)
+        ws = [ctx.load_weight(t, host, d, n) for _ in range(3)]
+        for B in (8, 64, 96):
+            X, out = ctx.from_numpy(synthetic.activations((B, n), 98 + B)), ctx.float_array(B * d)
+            proj = QuantizedBatchProjections(ctx, B, n, d)
+            for _ in range(4):
+                for w in ws:
+                    proj.projection(X, out, w, n, d, True)
+                ctx.sync()
+            proj.workspace.free()
+        shapes["batched %s %d x %d" % (name, d, n)] = int(host.size)
+        for w in ws:
+            w.free()
+    print(json.dumps({"weight_bytes": shapes}))
+
+
 def int8_probe(ctx, t, T=2048):
     """What the counters and the kernel trace of the int8 prefill path are collected on: one
     Llama-3.2-1B layer's four calls at T tokens with JL_MATH_INT8, kernel by kernel, four times."""
@@ -1119,6 +1159,8 @@ def main():
                     help="only measure the sustained rate of fp16 matrix instructions (see mfma_rate_probe)")
     ap.add_argument("--vocabulary-probe", action="store_true",
                     help="only launch the batched vocabulary projection and its per-row argmax (see vocabulary_probe)")
+    ap.add_argument("--shapes-probe", action="store_true",
+                    help="long single-token rows and awkward batched row lengths, kernel by kernel (for rocprofv3)")
     ap.add_argument("--batched-probe", action="store_true",
                     help="only launch the batched-decode calls, kernel by kernel (see batched_probe)")
     ap.add_argument("--decode-probe", action="store_true",
@@ -1160,6 +1202,9 @@ def main():
             return
         if args.batched_probe:
             batched_probe(ctx)
+            return
+        if args.shapes_probe:
+            shapes_probe(ctx)
             return
         if args.int8_probe:
             int8_probe(ctx, t)
