@@ -951,7 +951,9 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
     }
 
     const size_t in_workspace = kept ? 0 : copy_bytes;
-    const int dense_from = kept && copy_us < in_loop_us ? 128 : 512;
+    // (a call that has no other kernel takes the priced tiling at any row count: a few rows over a
+    // narrow weight are a few dozen 128 x 128 tiles, and K cut into runs is what fills the chip)
+    const int dense_from = dense_only ? 1 : kept && copy_us < in_loop_us ? 128 : 512;
     int dsplits = 1, bm = 256;
     int bn = jl_dense_column_tile(rows, k, virt, epilogue, ctx->compute_units, &dsplits, &bm, dense_from, ctx->split_k);
     if (bn != 0 && dsplits > 1 && in_workspace + jl_dense_plane_bytes(rows, virt, dsplits) > plane_bytes) {
