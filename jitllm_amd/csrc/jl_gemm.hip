@@ -876,6 +876,29 @@ int jl_launch_gemm(jl_context *ctx, const jl_weight *const *weights, int count, 
                "jl_gemm: X must be 16-byte and the workspace 256-byte aligned");
     for (int i = 0; i < count; i++)
         JL_REQUIRE(((uintptr_t)weights[i]->blocks & 15) == 0, "jl_gemm: weight %d is not 16-byte aligned", i);
+    // Weights of different types side by side at fewer than 512 rows -- batched decode or a short
+    // prompt over a "Q4_K_M" layer's q | k | v, whose v is Q6_K: decoding all of them to fp16 on every
+    // call is what a long prompt amortises and a few rows do not.  Without a kept copy such a call is
+    // made one run of equal types at a time, each through the kernels its type has, the runs' outputs
+    // side by side as one call would leave them.
+    if (count > 1 && epilogue != JL_SWIGLU && active_rows < 512 && k % 256 == 0 && !(resident && resident->copy)) {
+        bool differ = false;
+        for (int i = 1; i < count; i++) differ = differ || weights[i]->type != type;
+        if (differ) {
+            int64_t at = col_offset;
+            for (int i = 0; i < count;) {
+                int j = i;
+                int64_t width = 0;
+                while (j < count && weights[j]->type == weights[i]->type) width += weights[j++]->rows;
+                const int st = jl_launch_gemm(ctx, weights + i, j - i, X, C, batch, active_rows, ldo, at, epilogue, math,
+                                              workspace, workspace_bytes, nullptr, half);
+                if (st != JL_OK) return st;
+                at += width;
+                i = j;
+            }
+            return JL_OK;
+        }
+    }
     const int rows = (int)active_rows;
     // rows are padded to the row tile the kernel will use, never beyond what the workspace holds
     const int padded = (int)round_up((size_t)rows, rows <= 32 ? 32 : rows <= 64 ? 64 : 128);
