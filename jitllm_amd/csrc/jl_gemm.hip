@@ -758,7 +758,10 @@ namespace {
 int choose_splits(int rows, int bm, int k, int tiles, int row_bytes, int compute_units, int *unconstrained = nullptr) {
     const int ksteps = k / (BK * SUPER);  // raw stages of 256 columns
     const int padded = (rows + bm - 1) / bm * bm;
-    int want = rows <= 64 ? (2 * compute_units + tiles - 1) / tiles : compute_units / tiles;
+    // (the kernel deals each XCD a contiguous eighth of the tiles, rounded up, times the runs: 84
+    // tiles are 11 to an XCD, and three runs of each would be 33 work items for its 32 workgroups --
+    // two rounds.  Many rows want one round.)
+    int want = rows <= 64 ? (2 * compute_units + tiles - 1) / tiles : (compute_units / 8) / ((tiles + 7) / 8);
     int by_steps = ksteps / 2;
     int by_traffic = row_bytes / (2 * padded);
     int s = want < by_steps ? want : by_steps;
@@ -826,9 +829,10 @@ int launch_gemm_type(jl_context *ctx, GemmParams &p, int rows, float *planes, si
     p.partial = planes;
     // persistent workgroups, one per compute unit (fewer when there is less work), a multiple of 8
     // so that every XCD runs the same number of them
-    const int items = p.ntiles * p.mtiles * p.splits;
-    int wgs = items < ctx->compute_units ? items : ctx->compute_units;
-    wgs = (wgs + 7) / 8 * 8;
+    // (an XCD's share is an eighth of the tiles rounded up, times the runs: 84 tiles in two runs are
+    // 22 work items to an XCD, and a grid of 168 would give it 21 workgroups)
+    const int items = (p.ntiles * p.mtiles + 7) / 8 * 8 * p.splits;
+    const int wgs = items < ctx->compute_units ? items : ctx->compute_units / 8 * 8;
     const dim3 grid(wgs);
     int st;
     if (bm == 32) st = launch_gemm<TYPE, 32>(ctx, p, grid);

@@ -582,9 +582,9 @@ int launch_dense(jl_context *ctx, const DenseParams &p) {
         const int st = jl_raise_lds_limit(configured, ctx->device, (const void *)fn, lds);
         if (st != JL_OK) return st;
     }
-    const int items = p.ntiles * p.mtiles * p.splits;
-    int wgs = items < ctx->compute_units ? items : ctx->compute_units;
-    wgs = (wgs + 7) / 8 * 8;
+    // (an XCD's share is an eighth of the tiles rounded up, times the runs of K)
+    const int items = (p.ntiles * p.mtiles + 7) / 8 * 8 * p.splits;
+    const int wgs = items < ctx->compute_units ? items : ctx->compute_units / 8 * 8;
     hipLaunchKernelGGL(fn, dim3(wgs), dim3(512), lds, ctx->stream, p);
     JL_HIP(hipGetLastError());
     return JL_OK;
@@ -634,7 +634,8 @@ int jl_dense_column_tile(int rows, int k, int out_cols_virtual, int epilogue, in
             if (s > 1 && (!may_cut_k || swiglu || t.bm != 128 || t.bn != 128)) break;
             if ((k / DBK) % s != 0 || k / s < 4 * DBK) break;
             if (s > 1 && items * s > 2 * (int64_t)compute_units) break;   // (bounds the planes: the workspace counts on it)
-            const int64_t rounds = (items * s + compute_units - 1) / compute_units;
+            // (per XCD: an eighth of the items rounded up, times the runs, over an eighth of the chip)
+            const int64_t rounds = ((items + 7) / 8 * s + compute_units / 8 - 1) / (compute_units / 8);
             double cost = (double)rounds * t.bm * t.bn * t.per_output / s;
             // the fold: a launch, and s planes of partial sums written and read back
             if (s > 1) cost += (2.0 + (double)s * rows * out_cols_virtual * 4.0 / 4e6) * per_us;
