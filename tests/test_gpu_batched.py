@@ -1139,3 +1139,34 @@ def test_row_lengths_that_are_not_whole_256_column_blocks(ctx, t, n, rows):
     for w in (w1, w3, wk):
         w.free()
     proj.workspace.free()
+
+
+@pytest.mark.parametrize("rows", [8, 64, 200])
+def test_mixed_types_side_by_side_below_512_rows_are_their_runs(ctx, rows):
+    """A "Q4_K_M" q | k | v (q and k in Q4_K, v in Q6_K) at a few rows is made one run of equal types at a
+    time, each through the kernels its type has: the result is bit for bit what the two calls -- q | k,
+    then v beside them -- leave, and meets the oracle."""
+    from jitllm_amd import _lib as L, synthetic
+    from jitllm_amd.projections import QuantizedBatchProjections
+    say("mixed types, their runs", rows)
+    n, dq, dkv = 2048, 1024, 256
+    rq, rk = synthetic.weight(O.Q4_K, dq, n, seed=9930), synthetic.weight(O.Q4_K, dkv, n, seed=9931)
+    rv = synthetic.weight(O.Q6_K, dkv, n, seed=9932)
+    wq, wk, wv = ctx.load_weight(O.Q4_K, rq, dq, n), ctx.load_weight(O.Q4_K, rk, dkv, n), ctx.load_weight(O.Q6_K, rv, dkv, n)
+    X = synthetic.activations((rows, n), seed=9933)
+    dx = ctx.from_numpy(X)
+    width = dq + 2 * dkv
+    proj = QuantizedBatchProjections(ctx, rows, n, width)
+    one, two = ctx.float_array(rows * width, fill=UNTOUCHED), ctx.float_array(rows * width, fill=UNTOUCHED)
+    proj.fusedQKV(dx, one, wq, wk, wv)
+    proj._gemm([wq, wk], dx, two, rows, width, 0, L.JL_STORE)
+    proj._gemm([wv], dx, two, rows, width, dq + dkv, L.JL_STORE)
+    ctx.sync()
+    a, b = one.get().reshape(rows, width), two.get().reshape(rows, width)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    for cols, t, raw, d in ((slice(0, dq), O.Q4_K, rq, dq), (slice(dq, dq + dkv), O.Q4_K, rk, dkv),
+                            (slice(dq + dkv, width), O.Q6_K, rv, dkv)):
+        assert rel_err(a[:, cols], O.matmul_batch(t, raw, X, d, n), magnitude(t, raw, X, d, n)) < F16_BOUND
+    for w in (wq, wk, wv):
+        w.free()
+    proj.workspace.free()
